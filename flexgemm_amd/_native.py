@@ -1,0 +1,98 @@
+"""ctypes binding of libflexgemm_hip.so (the C ABI declared in include/flexgemm_hip.h).
+
+The library is mandatory: nothing in this package falls back to another implementation when
+it is missing.  Device pointers, sizes and the current HIP stream are taken from torch tensors;
+torch itself is only the allocator and the stream owner.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "libflexgemm_hip.so")
+_lib: Optional[C.CDLL] = None
+
+FGX_F16, FGX_BF16, FGX_F32 = 0, 1, 2
+DTYPE_CODE = {torch.float16: FGX_F16, torch.bfloat16: FGX_BF16, torch.float32: FGX_F32}
+PASS_FWD, PASS_DGRAD, PASS_WGRAD = 0, 1, 2
+
+# every symbol the header declares; the CPU-side test checks that the library exports each of them
+EXPORTS = [
+    "fgx_abi_version", "fgx_last_error",
+    "fgx_hash_init", "fgx_hash_insert_3d_idx_as_val", "fgx_hash_insert", "fgx_hash_lookup",
+    "fgx_hash_insert_3d", "fgx_hash_lookup_3d",
+    "fgx_subm_neighbor_map", "fgx_mask_codes",
+    "fgx_sort_workspace_bytes", "fgx_sort_by_code",
+    "fgx_pair_workspace_bytes", "fgx_pair_count", "fgx_pair_fill",
+    "fgx_tile_workspace_bytes", "fgx_tile_codes", "fgx_tile_fill",
+    "fgx_table_lookup", "fgx_weight_panel_bytes", "fgx_pack_weight",
+    "fgx_conv_scratch_bytes", "fgx_conv_gather_gemm",
+    "fgx_wgrad_scratch_bytes", "fgx_conv_wgrad",
+    "fgx_colsum_scratch_bytes", "fgx_colsum",
+]
+
+
+class Schedule(C.Structure):
+    _fields_ = [("tile_rows", C.c_int), ("tile_cols", C.c_int), ("splitk", C.c_int), ("chunk_pairs", C.c_int)]
+
+
+class NativeError(RuntimeError):
+    pass
+
+
+def lib_path() -> str:
+    return _LIB_PATH
+
+
+def lib() -> C.CDLL:
+    """Load the shared library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise NativeError(
+                f"{_LIB_PATH} is missing: build it with `python -m flexgemm_amd.build` "
+                "(hipcc --offload-arch=gfx950).  There is no fallback implementation.")
+        L = C.CDLL(_LIB_PATH)
+        L.fgx_last_error.restype = C.c_char_p
+        for name in ("fgx_sort_workspace_bytes", "fgx_pair_workspace_bytes", "fgx_tile_workspace_bytes",
+                     "fgx_weight_panel_bytes", "fgx_conv_scratch_bytes", "fgx_wgrad_scratch_bytes",
+                     "fgx_colsum_scratch_bytes"):
+            getattr(L, name).restype = C.c_size_t
+        _lib = L
+    return _lib
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        msg = lib().fgx_last_error().decode("utf-8", "replace")
+        if rc == -1:
+            raise ValueError(msg)
+        if rc == -3:
+            raise NotImplementedError(msg)
+        raise NativeError(msg)
+
+
+def ptr(t: Optional[torch.Tensor]) -> C.c_void_p:
+    return C.c_void_p(0 if t is None else t.data_ptr())
+
+
+def stream() -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def sz(x: int) -> C.c_size_t:
+    return C.c_size_t(int(x))
+
+
+def workspace(nbytes: int, device) -> torch.Tensor:
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def table_lookup(pass_kind: int, dtype: torch.dtype, n: int, ci: int, co: int, v: int) -> Schedule:
+    s = Schedule()
+    check(lib().fgx_table_lookup(C.c_int(pass_kind), C.c_int(DTYPE_CODE[dtype]), sz(n), C.c_int(ci), C.c_int(co),
+                                 C.c_int(v), C.byref(s)))
+    return s

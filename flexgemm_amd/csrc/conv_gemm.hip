@@ -1,0 +1,452 @@
+// Masked implicit GEMM (forward and dgrad) for submanifold sparse conv on gfx950.
+//
+//   out[sorted[r], :] = sum over offsets v present for row r of src[map[sorted[r], v], :] x panel_v (+ bias)
+//
+// One workgroup owns a tile of BM consecutive rows of the mask-sorted voxel order and BN output
+// channels.  Offsets whose bit is clear in the tile's OR-mask are skipped altogether.  For every
+// remaining (offset, K-slab) step the gathered source rows (A, BM x 128 bytes) and the matching
+// panel slice (B, BN x 128 bytes) are staged in LDS with an XOR swizzle on 16-byte chunks, and each
+// of the WAVES_M x WAVES_N wavefronts multiplies its (BM/WAVES_M) x (BN/WAVES_N) sub-tile with
+// 32x32 MFMA instructions, accumulating in fp32.  Global loads of step s+1 are issued before the
+// MFMAs of step s (register-staged double buffering, one barrier per step).
+//
+// Both operands are K-contiguous per row, and A and B fragments are read from LDS with the same
+// (chunk, lane-group) -> k assignment, so the contraction is independent of how the hardware
+// numbers k inside a fragment.
+//
+// dgrad is the same kernel: src = grad_output and a panel packed with the mirrored, transposed
+// weight (fgx_pack_weight mode 1).
+#include "fgx_common.h"
+
+namespace fgx {
+namespace {
+
+using f16x8 = _Float16 __attribute__((ext_vector_type(8)));
+using bf16x8 = __bf16 __attribute__((ext_vector_type(8)));
+using f32x4 = float __attribute__((ext_vector_type(4)));
+using f32x16 = float __attribute__((ext_vector_type(16)));
+using u32x4 = uint32_t __attribute__((ext_vector_type(4)));
+
+constexpr int kSlabBytes = 128;   // bytes of K per row and step
+constexpr int kChunks = 8;        // 16-byte chunks per slab row
+constexpr int kXcds = 8;
+
+struct F16 { using type = _Float16; };
+struct BF16 { using type = __bf16; };
+struct F32 { using type = float; };
+
+template <typename Tag> __device__ __forceinline__ void mma(f32x16& acc, const u32x4& a, const u32x4& b);
+template <> __device__ __forceinline__ void mma<F16>(f32x16& acc, const u32x4& a, const u32x4& b) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), acc, 0, 0, 0);
+}
+template <> __device__ __forceinline__ void mma<BF16>(f32x16& acc, const u32x4& a, const u32x4& b) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
+}
+template <> __device__ __forceinline__ void mma<F32>(f32x16& acc, const u32x4& a, const u32x4& b) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, a[i]), __builtin_bit_cast(float, b[i]), acc, 0, 0, 0);
+}
+
+template <typename T> __device__ __forceinline__ T from_float(float x);
+template <> __device__ __forceinline__ _Float16 from_float<_Float16>(float x) { return (_Float16)x; }
+template <> __device__ __forceinline__ float from_float<float>(float x) { return x; }
+template <> __device__ __forceinline__ __bf16 from_float<__bf16>(float x) {
+    // round to nearest even; NaN stays NaN
+    uint32_t u = __builtin_bit_cast(uint32_t, x);
+    uint16_t h;
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) h = (uint16_t)((u >> 16) | 0x0040u);
+    else h = (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+    return __builtin_bit_cast(__bf16, h);
+}
+template <typename T> __device__ __forceinline__ float to_float(T x) { return (float)x; }
+template <> __device__ __forceinline__ float to_float<__bf16>(__bf16 x) {
+    return __builtin_bit_cast(float, (uint32_t)__builtin_bit_cast(uint16_t, x) << 16);
+}
+
+__device__ __forceinline__ int swz(int row, int chunk) { return row * kSlabBytes + ((chunk ^ (row & 7)) << 4); }
+
+// ------------------------------------------------------------------------------------------------
+// Weight panels
+// ------------------------------------------------------------------------------------------------
+// panel[v][slab][col][k] with k in [0, SK); mode 0: w[col][v][slab*SK+k]; mode 1: w[slab*SK+k][V-1-v][col].
+template <typename T>
+__global__ void __launch_bounds__(256) pack_weight_kernel(const T* __restrict__ w, int Ci, int Co, int V, int mode,
+                                                          int slabs, int cols_pad, T* __restrict__ panel) {
+    constexpr int SK = kSlabBytes / (int)sizeof(T);
+    const int K = mode == 0 ? Ci : Co;
+    const int cols = mode == 0 ? Co : Ci;
+    const size_t total = (size_t)V * slabs * cols_pad * SK;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        int k = (int)(i % SK);
+        size_t t = i / SK;
+        int col = (int)(t % cols_pad);
+        t /= cols_pad;
+        int slab = (int)(t % slabs);
+        int v = (int)(t / slabs);
+        int kk = slab * SK + k;
+        T val = (T)0;
+        if (kk < K && col < cols) {
+            if (mode == 0) val = w[((size_t)col * V + v) * Ci + kk];
+            else val = w[((size_t)kk * V + (V - 1 - v)) * Ci + col];
+        }
+        panel[i] = val;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Gather GEMM
+// ------------------------------------------------------------------------------------------------
+template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N>
+struct GemmCfg {
+    using T = typename Tag::type;
+    static constexpr int NT = 64 * WAVES_M * WAVES_N;
+    static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    static constexpr int TM = WM / 32, TN = WN / 32;
+    static constexpr int SK = kSlabBytes / (int)sizeof(T);
+    static constexpr int A_CHUNKS = BM * kChunks, B_CHUNKS = BN * kChunks;
+    static constexpr int A_PER = (A_CHUNKS + NT - 1) / NT, B_PER = (B_CHUNKS + NT - 1) / NT;
+    static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
+    static_assert(A_CHUNKS % NT == 0 && B_CHUNKS % NT == 0, "tile must split evenly over the workgroup");
+    static constexpr size_t lds_bytes(int V) {
+        return (size_t)2 * (BM + BN) * kSlabBytes + (size_t)BM * V * 4 + (size_t)BM * 4 + 32 * 4;
+    }
+};
+
+template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ void __launch_bounds__(64 * WAVES_M * WAVES_N)
+gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Tag::type* __restrict__ panel,
+                   const typename Tag::type* __restrict__ bias, const uint32_t* __restrict__ map,
+                   const int64_t* __restrict__ sorted_idx, const int32_t* __restrict__ tile_code, uint32_t n, int K,
+                   int cols, int cols_pad, int V, int splitk, unsigned row_tiles, unsigned col_tiles,
+                   float* __restrict__ partial, typename Tag::type* __restrict__ out) {
+    using C = GemmCfg<Tag, BM, BN, WAVES_M, WAVES_N>;
+    using T = typename Tag::type;
+    constexpr int NT = C::NT;
+
+    // XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs, so give each XCD a
+    // contiguous run of tiles (neighbouring tiles gather overlapping rows -> same L2).
+    const unsigned total_tiles = row_tiles * col_tiles;
+    const unsigned per_xcd = (total_tiles + kXcds - 1) / kXcds;
+    const unsigned logical = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
+    if (logical >= total_tiles) return;
+    const unsigned row_tile = logical / col_tiles;
+    const unsigned col_tile = logical % col_tiles;
+    const int kid = blockIdx.y;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    unsigned char* a_lds = lds_raw;                                   // [2][BM * 128]
+    unsigned char* b_lds = a_lds + 2 * BM * kSlabBytes;               // [2][BN * 128]
+    uint32_t* nbr_lds = (uint32_t*)(b_lds + 2 * BN * kSlabBytes);     // [V][BM]
+    uint32_t* row_lds = nbr_lds + (size_t)BM * V;                     // [BM] output row or EMPTY
+    int* v_lds = (int*)(row_lds + BM);                                // [32] offsets present in this tile
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+    const uint32_t code = (uint32_t)tile_code[row_tile];
+    const int nv = __popc(code);
+    const int slabs = (K + C::SK - 1) / C::SK;
+    const int steps_total = nv * slabs;
+    const int step_lo = (int)(((long long)steps_total * kid + splitk - 1) / splitk);
+    const int step_hi = (int)(((long long)steps_total * (kid + 1) + splitk - 1) / splitk);
+
+    // ---- stage the tile's output rows, present offsets and neighbor indices ----
+    for (int r = tid; r < BM; r += NT) {
+        size_t g = (size_t)row_tile * BM + r;
+        row_lds[r] = g < n ? (uint32_t)sorted_idx[g] : FGX_EMPTY32;
+    }
+    if (tid == 0) {
+        uint32_t c = code;
+        int i = 0;
+        while (c) {
+            v_lds[i++] = __ffs((int)c) - 1;
+            c &= c - 1;
+        }
+    }
+    __syncthreads();
+    for (int i = tid; i < BM * V; i += NT) {
+        int r = i / V, v = i - r * V;
+        uint32_t row = row_lds[r];
+        uint32_t m = FGX_EMPTY32;
+        if (row != FGX_EMPTY32 && ((code >> v) & 1u)) m = map[(size_t)row * V + v];
+        nbr_lds[v * BM + r] = m;
+    }
+    __syncthreads();
+
+    f32x16 acc[C::TM][C::TN];
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    u32x4 a_reg[C::A_PER], b_reg[C::B_PER];
+    const size_t row_bytes = (size_t)K * sizeof(T);
+    const unsigned char* src_b = (const unsigned char*)src;
+    const unsigned char* panel_b = (const unsigned char*)panel;
+
+    auto load_step = [&](int step) {
+        const int v = v_lds[step / slabs];
+        const int slab = step - (step / slabs) * slabs;
+#pragma unroll
+        for (int i = 0; i < C::A_PER; ++i) {
+            int c = tid + i * NT;
+            int row = c >> 3, ch = c & 7;
+            uint32_t m = nbr_lds[v * BM + row];
+            int kbyte = slab * kSlabBytes + ch * 16;
+            u32x4 val = {0u, 0u, 0u, 0u};
+            if (m != FGX_EMPTY32 && (size_t)kbyte < row_bytes) val = *(const u32x4*)(src_b + (size_t)m * row_bytes + kbyte);
+            a_reg[i] = val;
+        }
+        const unsigned char* pb = panel_b + (((size_t)v * slabs + slab) * cols_pad + (size_t)col_tile * BN) * kSlabBytes;
+#pragma unroll
+        for (int i = 0; i < C::B_PER; ++i) {
+            int c = tid + i * NT;
+            b_reg[i] = *(const u32x4*)(pb + (size_t)c * 16);
+        }
+    };
+    auto store_step = [&](int buf) {
+        unsigned char* a_dst = a_lds + buf * BM * kSlabBytes;
+        unsigned char* b_dst = b_lds + buf * BN * kSlabBytes;
+#pragma unroll
+        for (int i = 0; i < C::A_PER; ++i) {
+            int c = tid + i * NT;
+            *(u32x4*)(a_dst + swz(c >> 3, c & 7)) = a_reg[i];
+        }
+#pragma unroll
+        for (int i = 0; i < C::B_PER; ++i) {
+            int c = tid + i * NT;
+            *(u32x4*)(b_dst + swz(c >> 3, c & 7)) = b_reg[i];
+        }
+    };
+
+    if (step_lo < step_hi) {
+        load_step(step_lo);
+        store_step(0);
+    }
+    __syncthreads();
+    const int g = lane >> 5;        // lane group inside the MFMA fragment
+    const int l32 = lane & 31;
+    for (int step = step_lo; step < step_hi; ++step) {
+        const int buf = (step - step_lo) & 1;
+        if (step + 1 < step_hi) load_step(step + 1);
+        const unsigned char* a_cur = a_lds + buf * BM * kSlabBytes;
+        const unsigned char* b_cur = b_lds + buf * BN * kSlabBytes;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            const int chunk = kk * 2 + g;
+            u32x4 af[C::TM], bf[C::TN];
+#pragma unroll
+            for (int i = 0; i < C::TM; ++i) af[i] = *(const u32x4*)(a_cur + swz(wave_m * C::WM + i * 32 + l32, chunk));
+#pragma unroll
+            for (int j = 0; j < C::TN; ++j) bf[j] = *(const u32x4*)(b_cur + swz(wave_n * C::WN + j * 32 + l32, chunk));
+#pragma unroll
+            for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+                for (int j = 0; j < C::TN; ++j) mma<Tag>(acc[i][j], af[i], bf[j]);
+        }
+        if (step + 1 < step_hi) store_step(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: 32x32 accumulator tile, element e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32 ----
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) {
+        const int col = (int)col_tile * BN + wave_n * C::WN + j * 32 + l32;
+        if (col >= cols) continue;
+        float bv = 0.f;
+        if (bias != nullptr && kid == 0) bv = to_float<T>(bias[col]);
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                int r = wave_m * C::WM + i * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
+                uint32_t orow = row_lds[r];
+                if (orow == FGX_EMPTY32) continue;
+                float val = acc[i][j][e] + bv;
+                if (splitk > 1) partial[((size_t)kid * n + orow) * cols + col] = val;
+                else out[(size_t)orow * cols + col] = from_float<T>(val);
+            }
+        }
+    }
+}
+
+// out[i] = sum_s partial[s][i]
+template <typename T>
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restrict__ partial, int splitk, size_t numel,
+                                                            T* __restrict__ out) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < numel; i += (size_t)gridDim.x * 256) {
+        float s = 0.f;
+        for (int k = 0; k < splitk; ++k) s += partial[(size_t)k * numel + i];
+        out[i] = from_float<T>(s);
+    }
+}
+
+// Column sums with fp32 accumulation: stage 1 sums a slice of rows per block, stage 2 adds the slices.
+constexpr int kColsumRows = 1024;
+template <typename T>
+__global__ void __launch_bounds__(256) colsum_partial_kernel(const T* __restrict__ x, size_t n, int cols,
+                                                             float* __restrict__ partial) {
+    const size_t r0 = (size_t)blockIdx.x * kColsumRows;
+    const size_t r1 = r0 + kColsumRows < n ? r0 + kColsumRows : n;
+    for (int c = threadIdx.x; c < cols; c += 256) {
+        float s = 0.f;
+        for (size_t r = r0; r < r1; ++r) s += to_float<T>(x[r * cols + c]);
+        partial[(size_t)blockIdx.x * cols + c] = s;
+    }
+}
+template <typename T>
+__global__ void __launch_bounds__(256) colsum_final_kernel(const float* __restrict__ partial, unsigned slices, int cols,
+                                                           T* __restrict__ out) {
+    int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= cols) return;
+    float s = 0.f;
+    for (unsigned b = 0; b < slices; ++b) s += partial[(size_t)b * cols + c];
+    out[c] = from_float<T>(s);
+}
+
+int elem_size(int dtype) { return dtype == FGX_F32 ? 4 : 2; }
+bool dtype_ok(int dtype) { return dtype == FGX_F16 || dtype == FGX_BF16 || dtype == FGX_F32; }
+
+template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N>
+int launch_gemm(const void* src, const void* panel, const void* bias, const uint32_t* map, const int64_t* sorted_idx,
+                const int32_t* tile_code, size_t n, int K, int cols, int cols_pad, int V, int splitk, void* scratch,
+                void* out, hipStream_t s) {
+    using C = GemmCfg<Tag, BM, BN, WAVES_M, WAVES_N>;
+    using T = typename Tag::type;
+    auto kern = gather_gemm_kernel<Tag, BM, BN, WAVES_M, WAVES_N>;
+    const size_t lds = C::lds_bytes(V);
+    FGX_CHECK_ARG(lds <= 160 * 1024, "fgx_conv_gather_gemm: tile needs %zu bytes of LDS", lds);
+    static thread_local size_t lds_set = 0;   // raise the dynamic LDS limit once per thread and size
+    if (lds > 64 * 1024 && lds > lds_set) {
+        FGX_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        lds_set = lds;
+    }
+    const unsigned row_tiles = cdiv(n, BM), col_tiles = cdiv(cols, BN);
+    const unsigned total = row_tiles * col_tiles;
+    const unsigned grid_x = cdiv(total, kXcds) * kXcds;
+    dim3 grid(grid_x, splitk, 1);
+    kern<<<grid, C::NT, lds, s>>>((const T*)src, (const T*)panel, (const T*)bias, map, sorted_idx, tile_code, (uint32_t)n, K,
+                                  cols, cols_pad, V, splitk, row_tiles, col_tiles, (float*)scratch, (T*)out);
+    FGX_CHECK_LAUNCH("fgx_conv_gather_gemm");
+    if (splitk > 1) {
+        size_t numel = n * (size_t)cols;
+        unsigned g = cdiv(numel, 256);
+        if (g > 65536u) g = 65536u;
+        splitk_reduce_kernel<T><<<g, 256, 0, s>>>((const float*)scratch, splitk, numel, (T*)out);
+        FGX_CHECK_LAUNCH("fgx_conv_gather_gemm(reduce)");
+    }
+    return FGX_OK;
+}
+
+template <typename Tag>
+int dispatch_tile(int tile_rows, int tile_cols, const void* src, const void* panel, const void* bias,
+                  const uint32_t* map, const int64_t* sorted_idx, const int32_t* tile_code, size_t n, int K, int cols,
+                  int cols_pad, int V, int splitk, void* scratch, void* out, hipStream_t s) {
+#define FGX_TILE(BM, BN, WMv, WNv)                                                                                    \
+    if (tile_rows == BM && tile_cols == BN)                                                                           \
+        return launch_gemm<Tag, BM, BN, WMv, WNv>(src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, \
+                                                  V, splitk, scratch, out, s);
+    FGX_TILE(128, 128, 2, 2)
+    FGX_TILE(128, 64, 2, 2)
+    FGX_TILE(128, 32, 4, 1)
+    FGX_TILE(64, 64, 2, 2)
+    FGX_TILE(64, 32, 2, 1)
+    FGX_TILE(32, 32, 1, 1)
+#undef FGX_TILE
+    set_error("fgx_conv_gather_gemm: no kernel for tile %dx%d", tile_rows, tile_cols);
+    return FGX_ERR_UNSUPPORTED;
+}
+
+}  // namespace
+}  // namespace fgx
+
+using namespace fgx;
+
+extern "C" {
+
+size_t fgx_weight_panel_bytes(int dtype, int mode, int Ci, int Co, int V, int col_pad) {
+    if (!dtype_ok(dtype) || Ci <= 0 || Co <= 0 || V <= 0 || col_pad <= 0) return 0;
+    const int K = mode == 0 ? Ci : Co, cols = mode == 0 ? Co : Ci;
+    const int es = elem_size(dtype), SK = kSlabBytes / es;
+    const size_t slabs = (size_t)(K + SK - 1) / SK;
+    const size_t cols_pad = align_up((size_t)cols, (size_t)col_pad);
+    return (size_t)V * slabs * cols_pad * kSlabBytes;
+}
+
+int fgx_pack_weight(int dtype, int mode, const void* weight, int Ci, int Co, int V, int col_pad, void* panel,
+                    fgx_stream_t stream) {
+    FGX_CHECK_ARG(dtype_ok(dtype), "fgx_pack_weight: unknown dtype %d", dtype);
+    FGX_CHECK_ARG(mode == 0 || mode == 1, "fgx_pack_weight: mode must be 0 (forward) or 1 (dgrad)");
+    FGX_CHECK_ARG(Ci > 0 && Co > 0 && V > 0, "fgx_pack_weight: bad shape Ci=%d Co=%d V=%d", Ci, Co, V);
+    FGX_CHECK_ARG(col_pad > 0 && col_pad % 32 == 0, "fgx_pack_weight: col_pad must be a positive multiple of 32");
+    FGX_CHECK_ARG(weight && panel, "fgx_pack_weight: null buffer");
+    const int K = mode == 0 ? Ci : Co, cols = mode == 0 ? Co : Ci;
+    const int es = elem_size(dtype), SK = kSlabBytes / es;
+    const int slabs = (K + SK - 1) / SK;
+    const int cols_pad = (int)align_up((size_t)cols, (size_t)col_pad);
+    const size_t total = (size_t)V * slabs * cols_pad * SK;
+    unsigned grid = cdiv(total, 256);
+    if (grid > 32768u) grid = 32768u;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == FGX_F32) pack_weight_kernel<float><<<grid, 256, 0, s>>>((const float*)weight, Ci, Co, V, mode, slabs, cols_pad, (float*)panel);
+    else pack_weight_kernel<uint16_t><<<grid, 256, 0, s>>>((const uint16_t*)weight, Ci, Co, V, mode, slabs, cols_pad, (uint16_t*)panel);
+    FGX_CHECK_LAUNCH("fgx_pack_weight");
+    return FGX_OK;
+}
+
+size_t fgx_conv_scratch_bytes(size_t n, int cols, int splitk) {
+    return splitk > 1 ? (size_t)splitk * n * (size_t)cols * sizeof(float) : 0;
+}
+
+int fgx_conv_gather_gemm(int dtype, const void* src, const void* panel, const void* bias, const uint32_t* map,
+                         const int64_t* sorted_idx, const int32_t* tile_code, size_t n, int K, int cols, int V,
+                         int tile_rows, int tile_cols, int splitk, void* scratch, void* out, fgx_stream_t stream) {
+    FGX_CHECK_ARG(dtype_ok(dtype), "fgx_conv_gather_gemm: unknown dtype %d", dtype);
+    FGX_CHECK_ARG(K > 0 && cols > 0 && V >= 1 && V <= 32, "fgx_conv_gather_gemm: bad shape K=%d cols=%d V=%d", K, cols, V);
+    FGX_CHECK_ARG(splitk >= 1 && splitk <= 1024, "fgx_conv_gather_gemm: splitk %d out of range", splitk);
+    FGX_CHECK_ARG(n < 0xFFFFFFFFull, "fgx_conv_gather_gemm: too many rows");
+    if (n == 0) return FGX_OK;
+    const int es = elem_size(dtype);
+    FGX_CHECK_ARG(((size_t)K * es) % 16 == 0, "fgx_conv_gather_gemm: source row of %d elements is not a multiple of 16 bytes", K);
+    FGX_CHECK_ARG(src && panel && map && sorted_idx && tile_code && out, "fgx_conv_gather_gemm: null buffer");
+    FGX_CHECK_ARG((((uintptr_t)src | (uintptr_t)panel) & 15) == 0, "fgx_conv_gather_gemm: src and panel must be 16-byte aligned");
+    FGX_CHECK_ARG(splitk == 1 || scratch != nullptr, "fgx_conv_gather_gemm: split-K needs a scratch buffer");
+    FGX_CHECK_ARG(cdiv(n, tile_rows) <= 0x7FFFFFu, "fgx_conv_gather_gemm: too many row tiles");
+    const int cols_pad = (int)align_up((size_t)cols, (size_t)tile_cols);
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case FGX_F16: return dispatch_tile<F16>(tile_rows, tile_cols, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, out, s);
+        case FGX_BF16: return dispatch_tile<BF16>(tile_rows, tile_cols, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, out, s);
+        default: return dispatch_tile<F32>(tile_rows, tile_cols, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, out, s);
+    }
+}
+
+size_t fgx_colsum_scratch_bytes(size_t n, int cols) {
+    return (size_t)cdiv(n ? n : 1, kColsumRows) * (size_t)(cols > 0 ? cols : 1) * sizeof(float);
+}
+
+int fgx_colsum(int dtype, const void* x, size_t n, int cols, void* scratch, void* out, fgx_stream_t stream) {
+    FGX_CHECK_ARG(dtype_ok(dtype), "fgx_colsum: unknown dtype %d", dtype);
+    FGX_CHECK_ARG(cols > 0 && out != nullptr, "fgx_colsum: bad shape or null output");
+    FGX_CHECK_ARG(scratch != nullptr && (n == 0 || x != nullptr), "fgx_colsum: null buffer");
+    hipStream_t s = (hipStream_t)stream;
+    const unsigned slices = n ? cdiv(n, kColsumRows) : 0u;
+    const unsigned gfin = cdiv(cols, 256);
+#define FGX_COLSUM(T)                                                                                     \
+    do {                                                                                                  \
+        if (slices) colsum_partial_kernel<T><<<slices, 256, 0, s>>>((const T*)x, n, cols, (float*)scratch); \
+        colsum_final_kernel<T><<<gfin, 256, 0, s>>>((const float*)scratch, slices, cols, (T*)out);        \
+    } while (0)
+    if (dtype == FGX_F16) FGX_COLSUM(_Float16);
+    else if (dtype == FGX_BF16) FGX_COLSUM(__bf16);
+    else FGX_COLSUM(float);
+#undef FGX_COLSUM
+    FGX_CHECK_LAUNCH("fgx_colsum");
+    return FGX_OK;
+}
+
+}  // extern "C"

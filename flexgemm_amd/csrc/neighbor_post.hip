@@ -1,0 +1,309 @@
+// Post-processing of the neighbor map for the masked implicit GEMM on gfx950:
+// mask-sorted voxel order, (v, n)-ordered pair lists for wgrad, per-tile offset masks.
+//
+// Departures from the reference's data flow (flex_gemm/kernels/cuda/spconv/migemm_neighmap_pp.cu):
+//   * pair lists are built from the 4-byte validity masks with a per-block count, one device scan
+//     over [V, blocks] and a rank-and-write pass, instead of materialising a transposed map, a
+//     transposed 0/1 mask and their N*V-long prefix sum (:85-154, :224-225);
+//   * the sort is a stable LSD radix sort restricted to the V mask bits;
+//   * tile masks are OR-reduced one wavefront per tile with cross-lane shuffles and accept any
+//     tile size, not only powers of two.
+#include <cstring>
+#include <string.h>
+
+#include <rocprim/rocprim.hpp>
+
+#include "fgx_common.h"
+
+namespace fgx {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kPairRows = 256;   // voxels per block in the pair-list passes
+
+__global__ void __launch_bounds__(kBlock) iota_u32_kernel(uint32_t* out, size_t n) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) out[i] = (uint32_t)i;
+}
+
+__global__ void __launch_bounds__(kBlock) widen_u32_i64_kernel(const uint32_t* in, int64_t* out, size_t n) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) out[i] = (int64_t)in[i];
+}
+
+struct SortLayout {
+    size_t keys_out, vals_in, vals_out, temp, temp_bytes, total;
+};
+
+SortLayout sort_layout(size_t n) {
+    SortLayout L{};
+    size_t nn = n ? n : 1;
+    size_t temp_bytes = 0;
+    // size query only: no work is enqueued
+    (void)rocprim::radix_sort_pairs(nullptr, temp_bytes, (const int32_t*)nullptr, (int32_t*)nullptr,
+                                    (const uint32_t*)nullptr, (uint32_t*)nullptr, nn, 0u, 32u, (hipStream_t)0);
+    size_t off = 0;
+    L.keys_out = off; off = align_up(off + nn * 4, 256);
+    L.vals_in = off;  off = align_up(off + nn * 4, 256);
+    L.vals_out = off; off = align_up(off + nn * 4, 256);
+    L.temp = off;     off = align_up(off + temp_bytes, 256);
+    L.temp_bytes = temp_bytes;
+    L.total = off;
+    return L;
+}
+
+// counts[v * nblk + blk] = number of voxels of block blk whose mask has bit v set
+__global__ void __launch_bounds__(kPairRows) pair_count_kernel(const int32_t* __restrict__ gray, size_t n, int V,
+                                                               unsigned nblk, uint32_t* __restrict__ counts) {
+    __shared__ uint32_t wave_cnt[kPairRows / 64][32];
+    const size_t row = (size_t)blockIdx.x * kPairRows + threadIdx.x;
+    const uint32_t g = row < n ? (uint32_t)gray[row] : 0u;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int v = 0; v < V; ++v) {
+        unsigned long long b = __ballot((g >> v) & 1u);
+        if (lane == 0) wave_cnt[wave][v] = (uint32_t)__popcll(b);
+    }
+    __syncthreads();
+    if (threadIdx.x < V) {
+        uint32_t c = 0;
+        for (int w = 0; w < kPairRows / 64; ++w) c += wave_cnt[w][threadIdx.x];
+        counts[(size_t)threadIdx.x * nblk + blockIdx.x] = c;
+    }
+}
+
+// seg[v] = offsets[v * nblk] for v < V, seg[V] = total (last offset + last count)
+__global__ void pair_seg_kernel(const uint32_t* __restrict__ offsets, const uint32_t* __restrict__ counts, int V,
+                                unsigned nblk, uint32_t* __restrict__ seg) {
+    int v = threadIdx.x;
+    if (v < V) seg[v] = nblk ? offsets[(size_t)v * nblk] : 0u;
+    if (v == V) seg[V] = nblk ? offsets[(size_t)V * nblk - 1] + counts[(size_t)V * nblk - 1] : 0u;
+}
+
+// Stage the block's map rows in LDS with coalesced loads, then for every offset rank the present
+// voxels (wave ballot + prefix of the wave totals) and write (n, map[n, v]) at offsets[v, blk] + rank.
+__global__ void __launch_bounds__(kPairRows) pair_fill_kernel(const uint32_t* __restrict__ map,
+                                                              const int32_t* __restrict__ gray, size_t n, int V,
+                                                              unsigned nblk, const uint32_t* __restrict__ offsets,
+                                                              uint32_t* __restrict__ sig_i, uint32_t* __restrict__ sig_o) {
+    extern __shared__ uint32_t lds[];
+    uint32_t* rows = lds;                                 // [kPairRows * V]
+    uint32_t* wave_cnt = lds + (size_t)kPairRows * V;     // [4][32]
+    const size_t base = (size_t)blockIdx.x * kPairRows;
+    const size_t len = (n - base < (size_t)kPairRows ? n - base : (size_t)kPairRows) * V;
+    for (size_t i = threadIdx.x; i < len; i += kPairRows) rows[i] = map[base * V + i];
+    const size_t row = base + threadIdx.x;
+    const uint32_t g = row < n ? (uint32_t)gray[row] : 0u;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    for (int v = 0; v < V; ++v) {
+        unsigned long long b = __ballot((g >> v) & 1u);
+        if (lane == 0) wave_cnt[wave * 32 + v] = (uint32_t)__popcll(b);
+    }
+    __syncthreads();
+    for (int v = 0; v < V; ++v) {
+        unsigned long long b = __ballot((g >> v) & 1u);
+        if ((g >> v) & 1u) {
+            uint32_t r = (uint32_t)__popcll(b & below);
+            for (int w = 0; w < wave; ++w) r += wave_cnt[w * 32 + v];
+            size_t to = (size_t)offsets[(size_t)v * nblk + blockIdx.x] + r;
+            sig_o[to] = (uint32_t)row;
+            sig_i[to] = rows[(size_t)threadIdx.x * V + v];
+        }
+    }
+}
+
+// One wavefront per tile: OR of gray[sorted_idx[r]] over the tile's rows.
+__global__ void __launch_bounds__(kBlock) tile_or_kernel(const int32_t* __restrict__ gray,
+                                                         const int64_t* __restrict__ sorted_idx, size_t n, int block,
+                                                         size_t num_tiles, int32_t* __restrict__ tile_code,
+                                                         uint32_t* __restrict__ popc) {
+    const size_t tile = ((size_t)blockIdx.x * kBlock + threadIdx.x) >> 6;
+    const int lane = threadIdx.x & 63;
+    if (tile >= num_tiles) return;   // whole wavefronts leave together
+    const size_t lo = tile * (size_t)block;
+    const size_t hi = lo + (size_t)block < n ? lo + (size_t)block : n;
+    uint32_t code = 0;
+    for (size_t r = lo + lane; r < hi; r += 64) code |= (uint32_t)gray[sorted_idx[r]];
+    for (int off = 32; off > 0; off >>= 1) code |= (uint32_t)__shfl_xor((int)code, off, 64);
+    if (lane == 0) {
+        tile_code[tile] = (int32_t)code;
+        popc[tile] = (uint32_t)__popc(code);
+    }
+}
+
+// seg[0..nb) = exclusive offsets (already there from the scan), seg[nb] = total
+__global__ void tile_seg_tail_kernel(const uint32_t* __restrict__ popc, int32_t* __restrict__ seg, size_t num_tiles) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) seg[num_tiles] = seg[num_tiles - 1] + (int32_t)popc[num_tiles - 1];
+}
+
+__global__ void set_i32_kernel(int32_t* dst, int32_t value) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) *dst = value;
+}
+
+__global__ void __launch_bounds__(kBlock) tile_fill_kernel(const int32_t* __restrict__ tile_code,
+                                                           const int32_t* __restrict__ seg, size_t num_tiles,
+                                                           int32_t* __restrict__ valid_kernel) {
+    size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= num_tiles) return;
+    uint32_t code = (uint32_t)tile_code[t];
+    int32_t* dst = valid_kernel + seg[t];
+    while (code) {
+        *dst++ = __ffs((int)code) - 1;
+        code &= code - 1;
+    }
+}
+
+size_t scan_temp_bytes(size_t count) {
+    size_t bytes = 0;
+    (void)rocprim::exclusive_scan(nullptr, bytes, (const uint32_t*)nullptr, (uint32_t*)nullptr, 0u, count ? count : 1,
+                                  rocprim::plus<uint32_t>(), (hipStream_t)0);
+    return bytes;
+}
+
+struct PairLayout {
+    unsigned nblk;
+    size_t counts, offsets, temp, temp_bytes, total;
+};
+
+PairLayout pair_layout(size_t n, int V) {
+    PairLayout L{};
+    L.nblk = cdiv(n, kPairRows);
+    size_t cnt = (size_t)L.nblk * V;
+    size_t off = 0;
+    L.counts = off;  off = align_up(off + (cnt ? cnt : 1) * 4, 256);
+    L.offsets = off; off = align_up(off + (cnt ? cnt : 1) * 4, 256);
+    L.temp_bytes = scan_temp_bytes(cnt);
+    L.temp = off;    off = align_up(off + L.temp_bytes, 256);
+    L.total = off;
+    return L;
+}
+
+struct TileLayout {
+    size_t num_tiles, popc, temp, temp_bytes, total;
+};
+
+TileLayout tile_layout(size_t n, int block) {
+    TileLayout L{};
+    L.num_tiles = (n + block - 1) / block;
+    size_t off = 0;
+    L.popc = off; off = align_up(off + (L.num_tiles ? L.num_tiles : 1) * 4, 256);
+    L.temp_bytes = scan_temp_bytes(L.num_tiles);
+    L.temp = off; off = align_up(off + L.temp_bytes, 256);
+    L.total = off;
+    return L;
+}
+
+}  // namespace
+}  // namespace fgx
+
+using namespace fgx;
+
+extern "C" {
+
+size_t fgx_sort_workspace_bytes(size_t n) { return sort_layout(n).total; }
+
+int fgx_sort_by_code(const int32_t* binary, size_t n, int V, int64_t* sorted_idx, void* workspace,
+                     size_t workspace_bytes, fgx_stream_t stream) {
+    FGX_CHECK_ARG(V >= 1 && V <= 32, "fgx_sort_by_code: kernel volume must be in [1, 32], got %d", V);
+    FGX_CHECK_ARG(n < 0xFFFFFFFFull, "fgx_sort_by_code: too many rows");
+    if (n == 0) return FGX_OK;
+    SortLayout L = sort_layout(n);
+    FGX_CHECK_ARG(binary && sorted_idx && workspace, "fgx_sort_by_code: null buffer");
+    FGX_CHECK_ARG(workspace_bytes >= L.total, "fgx_sort_by_code: workspace of %zu bytes, need %zu", workspace_bytes, L.total);
+    FGX_CHECK_ARG(((uintptr_t)workspace & 255) == 0, "fgx_sort_by_code: workspace must be 256-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    char* ws = (char*)workspace;
+    int32_t* keys_out = (int32_t*)(ws + L.keys_out);
+    uint32_t* vals_in = (uint32_t*)(ws + L.vals_in);
+    uint32_t* vals_out = (uint32_t*)(ws + L.vals_out);
+    iota_u32_kernel<<<cdiv(n, kBlock), kBlock, 0, s>>>(vals_in, n);
+    FGX_CHECK_LAUNCH("fgx_sort_by_code(iota)");
+    size_t temp_bytes = L.temp_bytes;
+    // With V < 32 every key is non-negative and only bits [0, V) can differ.
+    unsigned end_bit = V < 32 ? (unsigned)V : 32u;
+    FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp_bytes, binary, keys_out, vals_in, vals_out, n, 0u, end_bit, s));
+    widen_u32_i64_kernel<<<cdiv(n, kBlock), kBlock, 0, s>>>(vals_out, sorted_idx, n);
+    FGX_CHECK_LAUNCH("fgx_sort_by_code(widen)");
+    return FGX_OK;
+}
+
+size_t fgx_pair_workspace_bytes(size_t n, int V) { return pair_layout(n, V > 0 ? V : 1).total; }
+
+int fgx_pair_count(const int32_t* gray, size_t n, int V, uint32_t* seg, void* workspace, size_t workspace_bytes,
+                   fgx_stream_t stream) {
+    FGX_CHECK_ARG(V >= 1 && V <= 32, "fgx_pair_count: kernel volume must be in [1, 32], got %d", V);
+    FGX_CHECK_ARG(seg != nullptr, "fgx_pair_count: null segment table");
+    FGX_CHECK_ARG(n * (size_t)V < 0xFFFFFFFFull, "fgx_pair_count: pair offsets must fit in 32 bits");
+    hipStream_t s = (hipStream_t)stream;
+    PairLayout L = pair_layout(n, V);
+    if (n > 0) {
+        FGX_CHECK_ARG(gray && workspace, "fgx_pair_count: null buffer");
+        FGX_CHECK_ARG(workspace_bytes >= L.total, "fgx_pair_count: workspace of %zu bytes, need %zu", workspace_bytes, L.total);
+        FGX_CHECK_ARG(((uintptr_t)workspace & 255) == 0, "fgx_pair_count: workspace must be 256-byte aligned");
+    }
+    char* ws = (char*)workspace;
+    uint32_t* counts = n ? (uint32_t*)(ws + L.counts) : nullptr;
+    uint32_t* offsets = n ? (uint32_t*)(ws + L.offsets) : nullptr;
+    if (n > 0) {
+        pair_count_kernel<<<L.nblk, kPairRows, 0, s>>>(gray, n, V, L.nblk, counts);
+        FGX_CHECK_LAUNCH("fgx_pair_count(count)");
+        size_t temp_bytes = L.temp_bytes;
+        FGX_CHECK_HIP(rocprim::exclusive_scan(ws + L.temp, temp_bytes, counts, offsets, 0u, (size_t)L.nblk * V,
+                                              rocprim::plus<uint32_t>(), s));
+    }
+    pair_seg_kernel<<<1, 64, 0, s>>>(offsets, counts, V, n ? L.nblk : 0u, seg);
+    FGX_CHECK_LAUNCH("fgx_pair_count(seg)");
+    return FGX_OK;
+}
+
+int fgx_pair_fill(const uint32_t* map, const int32_t* gray, size_t n, int V, const void* workspace, uint32_t* sig_i,
+                  uint32_t* sig_o, fgx_stream_t stream) {
+    FGX_CHECK_ARG(V >= 1 && V <= 32, "fgx_pair_fill: kernel volume must be in [1, 32], got %d", V);
+    if (n == 0) return FGX_OK;
+    FGX_CHECK_ARG(map && gray && workspace && sig_i && sig_o, "fgx_pair_fill: null buffer");
+    PairLayout L = pair_layout(n, V);
+    const uint32_t* offsets = (const uint32_t*)((const char*)workspace + L.offsets);
+    size_t lds = ((size_t)kPairRows * V + 4 * 32) * sizeof(uint32_t);
+    pair_fill_kernel<<<L.nblk, kPairRows, lds, (hipStream_t)stream>>>(map, gray, n, V, L.nblk, offsets, sig_i, sig_o);
+    FGX_CHECK_LAUNCH("fgx_pair_fill");
+    return FGX_OK;
+}
+
+size_t fgx_tile_workspace_bytes(size_t n, int block) { return tile_layout(n, block > 0 ? block : 1).total; }
+
+int fgx_tile_codes(const int32_t* gray, const int64_t* sorted_idx, size_t n, int block, int32_t* tile_code,
+                   int32_t* seg, void* workspace, size_t workspace_bytes, fgx_stream_t stream) {
+    FGX_CHECK_ARG(block >= 1, "fgx_tile_codes: tile size must be >= 1, got %d", block);
+    FGX_CHECK_ARG(seg != nullptr, "fgx_tile_codes: null segment table");
+    hipStream_t s = (hipStream_t)stream;
+    TileLayout L = tile_layout(n, block);
+    if (L.num_tiles == 0) {
+        set_i32_kernel<<<1, 64, 0, s>>>(seg, 0);
+        FGX_CHECK_LAUNCH("fgx_tile_codes(empty)");
+        return FGX_OK;
+    }
+    FGX_CHECK_ARG(gray && sorted_idx && tile_code && workspace, "fgx_tile_codes: null buffer");
+    FGX_CHECK_ARG(workspace_bytes >= L.total, "fgx_tile_codes: workspace of %zu bytes, need %zu", workspace_bytes, L.total);
+    FGX_CHECK_ARG(((uintptr_t)workspace & 255) == 0, "fgx_tile_codes: workspace must be 256-byte aligned");
+    char* ws = (char*)workspace;
+    uint32_t* popc = (uint32_t*)(ws + L.popc);
+    tile_or_kernel<<<cdiv(L.num_tiles * 64, kBlock), kBlock, 0, s>>>(gray, sorted_idx, n, block, L.num_tiles, tile_code, popc);
+    FGX_CHECK_LAUNCH("fgx_tile_codes(or)");
+    size_t temp_bytes = L.temp_bytes;
+    FGX_CHECK_HIP(rocprim::exclusive_scan(ws + L.temp, temp_bytes, popc, (uint32_t*)seg, 0u, L.num_tiles,
+                                          rocprim::plus<uint32_t>(), s));
+    tile_seg_tail_kernel<<<1, 64, 0, s>>>(popc, seg, L.num_tiles);
+    FGX_CHECK_LAUNCH("fgx_tile_codes(tail)");
+    return FGX_OK;
+}
+
+int fgx_tile_fill(const int32_t* tile_code, const int32_t* seg, size_t num_tiles, int32_t* valid_kernel,
+                  fgx_stream_t stream) {
+    if (num_tiles == 0) return FGX_OK;
+    FGX_CHECK_ARG(tile_code && seg && valid_kernel, "fgx_tile_fill: null buffer");
+    tile_fill_kernel<<<cdiv(num_tiles, kBlock), kBlock, 0, (hipStream_t)stream>>>(tile_code, seg, num_tiles, valid_kernel);
+    FGX_CHECK_LAUNCH("fgx_tile_fill");
+    return FGX_OK;
+}
+
+}  // extern "C"

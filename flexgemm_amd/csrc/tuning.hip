@@ -1,0 +1,97 @@
+// Fixed gfx950 schedules for the masked implicit GEMM.
+//
+// The reference times every tile shape and every power-of-two SPLITK on first use and caches the
+// winner per (2^floor(log2 N), Ci, Co, V) (flex_gemm/utils/autotuner.py:194-291; candidate ranges in
+// ..._masked_implicit_gemm_splitk.py:109-126 and ..._bwd_..._splitk.py:185-202, 254-271).  Here the
+// choice is a static function of (floor(log2 N), Ci, Co): a table of measured entries for the shapes
+// that were tuned on an MI355X, and a rule for everything else.
+#include "fgx_common.h"
+
+namespace fgx {
+namespace {
+
+constexpr int kCUs = 256;
+
+struct Entry {
+    int pass_kind, dtype_bytes, log2n, ci, co;   // dtype_bytes: 2 or 4; 0 = any
+    fgx_schedule s;
+};
+
+// Measured entries (MI355X).  Rows are matched exactly on (pass, element size, floor(log2 N), Ci, Co).
+const Entry kTable[] = {
+    // pass dtype log2n  Ci    Co    {rows, cols, splitk, chunk_pairs}
+    {0, 2, 19, 128, 128, {128, 128, 1, 0}},
+    {1, 2, 19, 128, 128, {128, 128, 1, 0}},
+    {2, 2, 19, 128, 128, {128, 128, 1, 4096}},
+    {0, 2, 17, 256, 256, {128, 128, 1, 0}},
+    {1, 2, 17, 256, 256, {128, 128, 1, 0}},
+    {2, 2, 17, 256, 256, {128, 128, 1, 4096}},
+    {0, 2, 21, 32, 32, {128, 32, 1, 0}},
+    {1, 2, 21, 32, 32, {128, 32, 1, 0}},
+    {2, 2, 21, 32, 32, {32, 32, 1, 16384}},
+    {0, 2, 15, 1024, 1024, {128, 128, 1, 0}},
+    {1, 2, 15, 1024, 1024, {128, 128, 1, 0}},
+    {2, 2, 15, 1024, 1024, {128, 128, 1, 16384}},
+};
+
+int floor_log2(size_t n) {
+    int l = 0;
+    while (n > 1) { n >>= 1; ++l; }
+    return l;
+}
+
+int pick_cols(int c) { return c > 64 ? 128 : (c > 32 ? 64 : 32); }
+
+size_t round_up(size_t x, size_t m) { return (x + m - 1) / m * m; }
+
+void rule(int pass_kind, size_t n, int Ci, int Co, int V, fgx_schedule* out) {
+    if (pass_kind == 2) {
+        // wgrad: square tiles over (Co, Ci); chunk the pair lists so that about 8 workgroups per CU exist.
+        int t = pick_cols(Ci < Co ? Ci : Co);
+        out->tile_rows = t;
+        out->tile_cols = t;
+        out->splitk = 1;
+        size_t tiles = (size_t)cdiv(Co, t) * cdiv(Ci, t);
+        size_t pairs = n * (size_t)(V > 2 ? (V * 2) / 5 : 1);   // about 40 % of the offsets are present on surfaces
+        size_t want_chunks = (size_t)kCUs * 8 / (tiles ? tiles : 1);
+        if (want_chunks < (size_t)V) want_chunks = V;
+        size_t cp = round_up(pairs / want_chunks + 1, 64);
+        if (cp < 256) cp = 256;
+        if (cp > 65536) cp = 65536;
+        out->chunk_pairs = (int)cp;
+        return;
+    }
+    const int cols = pass_kind == 0 ? Co : Ci;
+    out->tile_cols = pick_cols(cols);
+    out->tile_rows = n >= 4096 ? 128 : (n >= 1024 ? 64 : 32);
+    if (out->tile_rows == 64 && out->tile_cols == 128) out->tile_rows = 128;
+    if (out->tile_rows == 32 && out->tile_cols != 32) out->tile_rows = out->tile_cols == 64 ? 64 : 128;
+    out->chunk_pairs = 0;
+    // split K only when the tiles cannot fill the chip (reference: candidates start at #SM / blocks)
+    size_t tiles = (size_t)cdiv(n, out->tile_rows) * cdiv(cols, out->tile_cols);
+    int s = 1;
+    while (tiles * s < (size_t)kCUs && s < 16) s *= 2;
+    out->splitk = s;
+}
+
+}  // namespace
+}  // namespace fgx
+
+using namespace fgx;
+
+extern "C" int fgx_table_lookup(int pass_kind, int dtype, size_t n, int Ci, int Co, int V, fgx_schedule* out) {
+    FGX_CHECK_ARG(out != nullptr, "fgx_table_lookup: null output");
+    FGX_CHECK_ARG(pass_kind >= 0 && pass_kind <= 2, "fgx_table_lookup: pass_kind must be 0 (fwd), 1 (dgrad) or 2 (wgrad)");
+    FGX_CHECK_ARG(dtype == FGX_F16 || dtype == FGX_BF16 || dtype == FGX_F32, "fgx_table_lookup: unknown dtype %d", dtype);
+    FGX_CHECK_ARG(Ci > 0 && Co > 0 && V >= 1, "fgx_table_lookup: bad shape");
+    const int es = dtype == FGX_F32 ? 4 : 2;
+    const int l2 = floor_log2(n ? n : 1);
+    for (const Entry& e : kTable) {
+        if (e.pass_kind == pass_kind && (e.dtype_bytes == 0 || e.dtype_bytes == es) && e.log2n == l2 && e.ci == Ci && e.co == Co) {
+            *out = e.s;
+            return FGX_OK;
+        }
+    }
+    rule(pass_kind, n, Ci, Co, V, out);
+    return FGX_OK;
+}

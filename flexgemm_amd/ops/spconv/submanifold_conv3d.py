@@ -1,0 +1,478 @@
+"""Submanifold sparse 3-D convolution on MI355X: host side of the operator.
+
+Public surface and argument meaning follow the reference operator
+(flex_gemm/ops/spconv/submanifold_conv3d.py): `sparse_submanifold_conv3d`, `SubMConv3dFunction`
+with its four static helpers, and the attribute-bag `SubMConv3dNeighborCache`.  All device work
+of the implicit-GEMM algorithms is done by hand-written gfx950 kernels behind the C ABI in
+include/flexgemm_hip.h; torch only allocates tensors and owns the stream.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Tuple
+
+import torch
+from torch.autograd import Function
+
+from ... import _native as nat
+from .. import spconv, utils
+from . import Algorithm
+
+EMPTY = 0xFFFFFFFF
+
+_IMPLICIT = (Algorithm.IMPLICIT_GEMM, Algorithm.IMPLICIT_GEMM_SPLITK,
+             Algorithm.MASKED_IMPLICIT_GEMM, Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
+_NO_SPLITK = (Algorithm.IMPLICIT_GEMM, Algorithm.MASKED_IMPLICIT_GEMM)
+
+
+def _require_cuda(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise NotImplementedError(f"{what}: the implicit-GEMM algorithms run on the GPU only (got a {t.device} tensor)")
+
+
+class SubMConv3dNeighborCache:
+    """Neighbor tables of one coordinate set, reusable across layers and calls.
+
+    Fields (reference: submanifold_conv3d.py:86-104): `neighbor_map` uint32 [N, V]; for the
+    implicit-GEMM algorithms also `gray_code` int32 [N] (validity mask), `sorted_idx` int64 [N];
+    when gradients are needed `valid_signal_i`, `valid_signal_o` uint32 [L] and `valid_signal_seg`
+    uint32 [V+1].  `valid_kernel_{B}` / `valid_kernel_seg_{B}` are computed on demand per tile
+    size B.  Names starting with an underscore are private schedules of the gfx950 kernels.
+    """
+
+    def __init__(self, **kwargs):
+        for k, v in kwargs.items():
+            setattr(self, k, v)
+
+    def __getitem__(self, key):
+        return getattr(self, key)
+
+    def __setitem__(self, key, value):
+        setattr(self, key, value)
+
+    def __contains__(self, key):
+        return hasattr(self, key)
+
+    # -- per-tile offset lists -------------------------------------------------------------------
+    def _tile_tables(self, block_size: int):
+        """(tile_code int32 [nb], seg int32 [nb+1]) for tiles of `block_size` sorted rows; no host sync."""
+        key = f"_tile_code_{block_size}"
+        if not hasattr(self, key):
+            gray, order = self["gray_code"], self["sorted_idx"]
+            n = gray.shape[0]
+            nb = (n + block_size - 1) // block_size
+            code = torch.empty((nb,), dtype=torch.int32, device=gray.device)
+            seg = torch.empty((nb + 1,), dtype=torch.int32, device=gray.device)
+            with torch.cuda.device(gray.device):
+                L = nat.lib()
+                ws_bytes = L.fgx_tile_workspace_bytes(nat.sz(n), C.c_int(block_size))
+                ws = nat.workspace(ws_bytes, gray.device)
+                nat.check(L.fgx_tile_codes(nat.ptr(gray), nat.ptr(order), nat.sz(n), C.c_int(block_size),
+                                           nat.ptr(code), nat.ptr(seg), nat.ptr(ws), nat.sz(ws.numel()), nat.stream()))
+            setattr(self, key, code)
+            setattr(self, f"valid_kernel_seg_{block_size}", seg)
+        return getattr(self, key), getattr(self, f"valid_kernel_seg_{block_size}")
+
+    def compute_kernel_idx(self, block_size: int):
+        """Fill `valid_kernel_{B}` / `valid_kernel_seg_{B}` (reference: submanifold_conv3d.py:20-23,
+        native side migemm_neighmap_pp.cu:330-368).  One 4-byte read-back sizes the list."""
+        block_size = int(block_size)
+        if block_size < 1:
+            raise ValueError(f"block_size must be positive, got {block_size}")
+        code, seg = self._tile_tables(block_size)
+        nb = code.shape[0]
+        total = int(seg[-1].item())
+        vk = torch.empty((total,), dtype=torch.int32, device=code.device)
+        if total:
+            with torch.cuda.device(code.device):
+                nat.check(nat.lib().fgx_tile_fill(nat.ptr(code), nat.ptr(seg), nat.sz(nb), nat.ptr(vk), nat.stream()))
+        self[f"valid_kernel_{block_size}"] = vk
+
+    def valid_kernel_callback(self, block_size: int) -> torch.Tensor:
+        if not hasattr(self, f"valid_kernel_{block_size}"):
+            self.compute_kernel_idx(block_size)
+        return self[f"valid_kernel_{block_size}"]
+
+    def valid_kernel_seg_callback(self, block_size: int) -> torch.Tensor:
+        if not hasattr(self, f"valid_kernel_{block_size}"):
+            self.compute_kernel_idx(block_size)
+        return self[f"valid_kernel_seg_{block_size}"]
+
+    # -- lazily completed fields -----------------------------------------------------------------
+    def _ensure_sorted(self):
+        """gray_code / sorted_idx for a cache that only carries `neighbor_map`."""
+        if hasattr(self, "gray_code") and hasattr(self, "sorted_idx"):
+            return
+        nmap = self["neighbor_map"]
+        gray, order = _codes_and_order(nmap, None, None)
+        self["gray_code"], self["sorted_idx"] = gray, order
+
+    def _ensure_pairs(self):
+        """valid_signal_* for a cache that was built without gradients."""
+        if hasattr(self, "valid_signal_i") and hasattr(self, "valid_signal_o") and hasattr(self, "valid_signal_seg"):
+            return
+        self._ensure_sorted()
+        sig_i, sig_o, seg, seg_host = _pair_lists(self["neighbor_map"], self["gray_code"])
+        self["valid_signal_i"], self["valid_signal_o"], self["valid_signal_seg"] = sig_i, sig_o, seg
+        self["_valid_signal_seg_host"] = seg_host
+
+    def _seg_host(self):
+        if not hasattr(self, "_valid_signal_seg_host"):
+            seg = self["valid_signal_seg"]
+            self["_valid_signal_seg_host"] = [int(x) & 0xFFFFFFFF for x in seg.view(torch.int32).cpu().tolist()]
+        return self["_valid_signal_seg_host"]
+
+
+# ------------------------------------------------------------------------------------------------
+# native helpers
+# ------------------------------------------------------------------------------------------------
+def _codes_and_order(nmap: torch.Tensor, gray: Optional[torch.Tensor], binary: Optional[torch.Tensor]):
+    """(gray_code, sorted_idx) from a neighbor map; gray/binary may come precomputed from the fused builder."""
+    n, v = nmap.shape
+    dev = nmap.device
+    L = nat.lib()
+    with torch.cuda.device(dev):
+        if gray is None:
+            gray = torch.empty((n,), dtype=torch.int32, device=dev)
+            binary = torch.empty((n,), dtype=torch.int32, device=dev)
+            nat.check(L.fgx_mask_codes(nat.ptr(nmap), nat.sz(n), C.c_int(v), nat.ptr(gray), nat.ptr(binary), nat.stream()))
+        order = torch.empty((n,), dtype=torch.int64, device=dev)
+        ws = nat.workspace(L.fgx_sort_workspace_bytes(nat.sz(n)), dev)
+        nat.check(L.fgx_sort_by_code(nat.ptr(binary), nat.sz(n), C.c_int(v), nat.ptr(order), nat.ptr(ws),
+                                     nat.sz(ws.numel()), nat.stream()))
+    return gray, order
+
+
+def _pair_lists(nmap: torch.Tensor, gray: torch.Tensor):
+    n, v = nmap.shape
+    dev = nmap.device
+    L = nat.lib()
+    with torch.cuda.device(dev):
+        seg = torch.empty((v + 1,), dtype=torch.uint32, device=dev)
+        ws = nat.workspace(L.fgx_pair_workspace_bytes(nat.sz(n), C.c_int(v)), dev)
+        nat.check(L.fgx_pair_count(nat.ptr(gray), nat.sz(n), C.c_int(v), nat.ptr(seg), nat.ptr(ws), nat.sz(ws.numel()),
+                                   nat.stream()))
+        seg_host = [x & 0xFFFFFFFF for x in seg.view(torch.int32).cpu().tolist()]   # the one host sync: sizes L
+        total = seg_host[-1]
+        sig_i = torch.empty((total,), dtype=torch.uint32, device=dev)
+        sig_o = torch.empty((total,), dtype=torch.uint32, device=dev)
+        if total:
+            nat.check(L.fgx_pair_fill(nat.ptr(nmap), nat.ptr(gray), nat.sz(n), C.c_int(v), nat.ptr(ws), nat.ptr(sig_i),
+                                      nat.ptr(sig_o), nat.stream()))
+    return sig_i, sig_o, seg, seg_host
+
+
+def _build_neighbor_map(coords: torch.Tensor, shape, kernel_size, dilation, with_codes: bool):
+    n = coords.shape[0]
+    _, _, W, H, D = [int(s) for s in shape]
+    kw, kh, kd = [int(k) for k in kernel_size]
+    v = kw * kh * kd
+    dev = coords.device
+    table = int(spconv.HASHMAP_RATIO * n)
+    if n > 0 and table < n:
+        raise ValueError(f"hashmap ratio {spconv.HASHMAP_RATIO} gives a table smaller than the input")
+    keys, vals = utils.init_hashmap(shape, table, dev)
+    nmap = torch.empty((n, v), dtype=torch.uint32, device=dev)
+    gray = binary = None
+    if with_codes:
+        gray = torch.empty((n,), dtype=torch.int32, device=dev)
+        binary = torch.empty((n,), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        nat.check(nat.lib().fgx_subm_neighbor_map(
+            nat.ptr(keys), C.c_int(32 if keys.dtype == torch.uint32 else 64), nat.ptr(vals), nat.sz(table),
+            nat.ptr(coords), nat.sz(n), C.c_int(W), C.c_int(H), C.c_int(D), C.c_int(kw), C.c_int(kh), C.c_int(kd),
+            C.c_int(int(dilation[0])), C.c_int(int(dilation[1])), C.c_int(int(dilation[2])),
+            nat.ptr(nmap), nat.ptr(gray), nat.ptr(binary), nat.stream()))
+    return nmap, gray, binary
+
+
+def _pad_cols(t: torch.Tensor, mult: int) -> torch.Tensor:
+    c = t.shape[-1]
+    pad = (-c) % mult
+    return t if pad == 0 else torch.nn.functional.pad(t, (0, pad))
+
+
+def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[torch.Tensor], cache, mode: int,
+                 allow_splitk: bool) -> torch.Tensor:
+    """mode 0: out = conv(src) with weight [Co, V, Ci] (+bias); mode 1: grad_input from src = grad_output."""
+    co, v, ci = weight_cvk.shape
+    n = src.shape[0]
+    dt = src.dtype
+    if dt not in nat.DTYPE_CODE:
+        raise TypeError(f"unsupported feature dtype {dt}; expected float16, bfloat16 or float32")
+    if weight_cvk.dtype != dt or (bias is not None and bias.dtype != dt):
+        raise TypeError("features, weight and bias must share one dtype")
+    k_true, cols = (ci, co) if mode == 0 else (co, ci)
+    dev = src.device
+    # rows must be whole 16-byte chunks: zero-pad the contraction dimension when they are not
+    align = 16 // src.element_size()
+    if k_true % align:
+        src = _pad_cols(src, align)
+        if mode == 0:
+            weight_cvk = _pad_cols(weight_cvk, align)
+        else:
+            weight_cvk = torch.nn.functional.pad(weight_cvk, (0, 0, 0, 0, 0, (-co) % align))
+        co, v, ci = weight_cvk.shape
+    k = ci if mode == 0 else co
+    src = src.contiguous()
+    weight_cvk = weight_cvk.contiguous()
+    sched = nat.table_lookup(nat.PASS_FWD if mode == 0 else nat.PASS_DGRAD, dt, n, ci, co, v)
+    splitk = sched.splitk if allow_splitk else 1
+    cache._ensure_sorted()
+    tile_code, _ = cache._tile_tables(sched.tile_rows)
+    out = torch.empty((n, cols), dtype=dt, device=dev)
+    if n == 0:
+        return out
+    L = nat.lib()
+    code = nat.DTYPE_CODE[dt]
+    with torch.cuda.device(dev):
+        panel = nat.workspace(L.fgx_weight_panel_bytes(C.c_int(code), C.c_int(mode), C.c_int(ci), C.c_int(co), C.c_int(v),
+                                                       C.c_int(sched.tile_cols)), dev)
+        nat.check(L.fgx_pack_weight(C.c_int(code), C.c_int(mode), nat.ptr(weight_cvk), C.c_int(ci), C.c_int(co), C.c_int(v),
+                                    C.c_int(sched.tile_cols), nat.ptr(panel), nat.stream()))
+        scratch = None
+        if splitk > 1:
+            scratch = nat.workspace(L.fgx_conv_scratch_bytes(nat.sz(n), C.c_int(cols), C.c_int(splitk)), dev)
+        nat.check(L.fgx_conv_gather_gemm(
+            C.c_int(code), nat.ptr(src), nat.ptr(panel), nat.ptr(bias), nat.ptr(cache["neighbor_map"]),
+            nat.ptr(cache["sorted_idx"]), nat.ptr(tile_code), nat.sz(n), C.c_int(k), C.c_int(cols), C.c_int(v),
+            C.c_int(sched.tile_rows), C.c_int(sched.tile_cols), C.c_int(splitk), nat.ptr(scratch), nat.ptr(out),
+            nat.stream()))
+    return out
+
+
+def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int) -> torch.Tensor:
+    n, ci = feats.shape
+    co = grad_output.shape[1]
+    dt = feats.dtype
+    dev = feats.device
+    align = 16 // feats.element_size()
+    f = _pad_cols(feats, align).contiguous()
+    g = _pad_cols(grad_output, align).contiguous()
+    cip, cop = f.shape[1], g.shape[1]
+    cache._ensure_pairs()
+    seg_host = cache._seg_host()
+    seg_arr = (C.c_uint32 * (v + 1))(*seg_host)
+    sched = nat.table_lookup(nat.PASS_WGRAD, dt, n, cip, cop, v)
+    gw = torch.empty((cop, v, cip), dtype=dt, device=dev)
+    L = nat.lib()
+    code = nat.DTYPE_CODE[dt]
+    with torch.cuda.device(dev):
+        scratch = nat.workspace(L.fgx_wgrad_scratch_bytes(seg_arr, C.c_int(v), C.c_int(cip), C.c_int(cop),
+                                                          C.c_int(sched.chunk_pairs)), dev)
+        nat.check(L.fgx_conv_wgrad(
+            C.c_int(code), nat.ptr(g), nat.ptr(f), nat.ptr(cache["valid_signal_i"]), nat.ptr(cache["valid_signal_o"]),
+            seg_arr, nat.sz(n), C.c_int(cip), C.c_int(cop), C.c_int(v), C.c_int(sched.tile_rows), C.c_int(sched.tile_cols),
+            C.c_int(sched.chunk_pairs), nat.ptr(scratch), nat.ptr(gw), nat.stream()))
+    if cip != ci or cop != co:
+        gw = gw[:co, :, :ci].contiguous()
+    return gw
+
+
+def _colsum(grad_output: torch.Tensor) -> torch.Tensor:
+    n, co = grad_output.shape
+    out = torch.empty((co,), dtype=grad_output.dtype, device=grad_output.device)
+    L = nat.lib()
+    with torch.cuda.device(grad_output.device):
+        scratch = nat.workspace(L.fgx_colsum_scratch_bytes(nat.sz(n), C.c_int(co)), grad_output.device)
+        nat.check(L.fgx_colsum(C.c_int(nat.DTYPE_CODE[grad_output.dtype]), nat.ptr(grad_output), nat.sz(n), C.c_int(co),
+                               nat.ptr(scratch), nat.ptr(out), nat.stream()))
+    return out
+
+
+def _gathered_rows(src: torch.Tensor, nmap: torch.Tensor) -> torch.Tensor:
+    """[N, V*C] matrix whose (n, v) block is src[map[n, v]] or zeros (the explicit formulation's im2col)."""
+    n, v = nmap.shape
+    idx = nmap.view(torch.int32).to(torch.int64)
+    idx = torch.where(idx < 0, torch.full_like(idx, src.shape[0]), idx)
+    padded = torch.cat([src, src.new_zeros((1, src.shape[1]))], dim=0)
+    return padded.index_select(0, idx.reshape(-1)).view(n, v * src.shape[1])
+
+
+class SubMConv3dFunction(Function):
+    @staticmethod
+    def _compute_neighbor_cache(
+        coords: torch.Tensor,
+        shape: torch.Size,
+        kernel_size: Tuple[int, int, int],
+        dilation: Tuple[int, int, int],
+        needs_grad: bool,
+    ) -> SubMConv3dNeighborCache:
+        """Build the neighbor tables for `coords` under the current algorithm
+        (reference: submanifold_conv3d.py:46-107)."""
+        assert coords.is_contiguous(), "Coords should be contiguous"
+        assert coords.dtype in [torch.int32], "Unsupported coords dtype. Expect int32"
+        algo = spconv.ALGORITHM
+        if algo != Algorithm.EXPLICIT_GEMM and algo not in _IMPLICIT:
+            raise ValueError(f"Unsupported algorithm {algo}")
+        if not coords.is_cuda:
+            raise NotImplementedError("CPU version of hashmap is not implemented")
+        v = int(kernel_size[0]) * int(kernel_size[1]) * int(kernel_size[2])
+        if algo == Algorithm.EXPLICIT_GEMM:
+            nmap, _, _ = _build_neighbor_map(coords, shape, kernel_size, dilation, with_codes=False)
+            return SubMConv3dNeighborCache(neighbor_map=nmap)
+        assert v <= 32, "Currently, the max kernel volume is 32 because kernel mask is encoded as uint32"
+        nmap, gray, binary = _build_neighbor_map(coords, shape, kernel_size, dilation, with_codes=True)
+        gray, order = _codes_and_order(nmap, gray, binary)
+        cache = SubMConv3dNeighborCache(neighbor_map=nmap, gray_code=gray, sorted_idx=order)
+        if needs_grad:
+            sig_i, sig_o, seg, seg_host = _pair_lists(nmap, gray)
+            cache["valid_signal_seg"] = seg
+            cache["valid_signal_i"] = sig_i
+            cache["valid_signal_o"] = sig_o
+            cache["_valid_signal_seg_host"] = seg_host
+        return cache
+
+    @staticmethod
+    def _compute_neighbor_cache_torch(
+        coords: torch.Tensor,
+        shape: torch.Size,
+        kernel_size: Tuple[int, int, int],
+        dilation: Tuple[int, int, int],
+    ) -> SubMConv3dNeighborCache:
+        """Hash-free builder in torch ops (any device): sort the flattened coordinates once and
+        binary-search every shifted coordinate (reference: submanifold_conv3d.py:109-144; keys are
+        int64 here, so the grid may exceed 2^31 cells)."""
+        assert spconv.ALGORITHM == Algorithm.EXPLICIT_GEMM, "Only explicit_gemm is supported for torch implementation"
+        _, _, W, H, D = [int(s) for s in shape]
+        n = coords.shape[0]
+        kw, kh, kd = [int(k) for k in kernel_size]
+        c = coords.to(torch.int64)
+        dev = coords.device
+        keys = ((c[:, 0] * W + c[:, 1]) * H + c[:, 2]) * D + c[:, 3]
+        skeys, order = torch.sort(keys)
+        cols = []
+        for i in range(kw):
+            for j in range(kh):
+                for k in range(kd):
+                    x = c[:, 1] + (i - kw // 2) * int(dilation[0])
+                    y = c[:, 2] + (j - kh // 2) * int(dilation[1])
+                    z = c[:, 3] + (k - kd // 2) * int(dilation[2])
+                    inside = (x >= 0) & (x < W) & (y >= 0) & (y < H) & (z >= 0) & (z < D)
+                    q = ((c[:, 0] * W + x) * H + y) * D + z
+                    col = torch.full((n,), EMPTY, dtype=torch.int64, device=dev)
+                    if n:
+                        pos = torch.searchsorted(skeys, q).clamp_(max=n - 1)
+                        hit = inside & (skeys[pos] == q)
+                        col[hit] = order[pos[hit]]
+                    cols.append(col)
+        nmap = torch.stack(cols, dim=1).to(torch.uint32) if cols else torch.empty((n, 0), dtype=torch.uint32, device=dev)
+        return SubMConv3dNeighborCache(neighbor_map=nmap)
+
+    @staticmethod
+    def _sparse_submanifold_conv_forward(
+        feats: torch.Tensor,
+        neighbor_cache: SubMConv3dNeighborCache,
+        weight: torch.Tensor,
+        bias: Optional[torch.Tensor] = None,
+    ) -> torch.Tensor:
+        assert feats.is_contiguous(), "Input features should be contiguous"
+        co, kw, kh, kd, ci = weight.shape
+        v = kw * kh * kd
+        algo = spconv.ALGORITHM
+        if algo == Algorithm.EXPLICIT_GEMM:
+            col = _gathered_rows(feats, neighbor_cache["neighbor_map"])
+            w = weight.reshape(co, v * ci).t()
+            return torch.addmm(bias, col, w) if bias is not None else torch.mm(col, w)
+        if algo in _IMPLICIT:
+            _require_cuda(feats, "sparse_submanifold_conv3d")
+            return _gather_gemm(feats, weight.reshape(co, v, ci), bias, neighbor_cache, 0, algo not in _NO_SPLITK)
+        raise ValueError(f"Unsupported algorithm {algo}")
+
+    @staticmethod
+    def _sparse_submanifold_conv_backward(
+        grad_output: torch.Tensor,
+        feats: torch.Tensor,
+        neighbor_cache: SubMConv3dNeighborCache,
+        weight: torch.Tensor,
+        bias: Optional[torch.Tensor] = None,
+    ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], Optional[torch.Tensor]]:
+        co, kw, kh, kd, ci = weight.shape
+        v = kw * kh * kd
+        algo = spconv.ALGORITHM
+        grad_input = grad_weight = grad_bias = None
+        if algo == Algorithm.EXPLICIT_GEMM:
+            nmap = neighbor_cache["neighbor_map"]
+            if feats.requires_grad:
+                col = _gathered_rows(grad_output, torch.flip(nmap.view(torch.int32), [1]).view(torch.uint32))
+                grad_input = torch.mm(col, weight.reshape(co, v, ci).transpose(0, 1).reshape(v * co, ci))
+            if weight.requires_grad:
+                col = _gathered_rows(feats.detach(), nmap)
+                grad_weight = torch.mm(col.t(), grad_output).view(v, ci, co).permute(2, 0, 1).contiguous() \
+                    .view(co, kw, kh, kd, ci)
+            if bias is not None and bias.requires_grad:
+                grad_bias = grad_output.sum(dim=0)
+            return grad_input, grad_weight, grad_bias
+        if algo in _IMPLICIT:
+            _require_cuda(feats, "sparse_submanifold_conv3d backward")
+            grad_output = grad_output.contiguous()
+            if feats.requires_grad:
+                grad_input = _gather_gemm(grad_output, weight.detach().reshape(co, v, ci), None, neighbor_cache, 1,
+                                          algo not in _NO_SPLITK)
+            if weight.requires_grad:
+                grad_weight = _wgrad(grad_output, feats.detach(), neighbor_cache, v).reshape(co, kw, kh, kd, ci)
+            if bias is not None and bias.requires_grad:
+                grad_bias = _colsum(grad_output)
+            return grad_input, grad_weight, grad_bias
+        raise ValueError(f"Unsupported algorithm {algo}")
+
+    @staticmethod
+    def forward(
+        ctx,
+        feats: torch.Tensor,
+        coords: torch.Tensor,
+        shape: torch.Size,
+        neighbor_cache: Optional[SubMConv3dNeighborCache],
+        weight: torch.Tensor,
+        bias: Optional[torch.Tensor] = None,
+        dilation: Tuple[int, int, int] = (1, 1, 1),
+    ) -> Tuple[torch.Tensor, SubMConv3dNeighborCache]:
+        co, kw, kh, kd, ci = weight.shape
+        assert feats.shape[-1] == ci, f"Input channels ({feats.shape[-1]}) should match weight channels ({ci})"
+        need_grad = any(ctx.needs_input_grad)
+        if neighbor_cache is None:
+            neighbor_cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (kw, kh, kd), dilation, need_grad)
+        output = SubMConv3dFunction._sparse_submanifold_conv_forward(feats, neighbor_cache, weight, bias)
+        ctx.save_for_backward(feats, weight, bias)
+        ctx.neighbor_cache = neighbor_cache
+        return output, neighbor_cache
+
+    @staticmethod
+    def backward(ctx, grad_output: torch.Tensor, _):
+        feats, weight, bias = ctx.saved_tensors
+        need_f, need_w, need_b = ctx.needs_input_grad[0], ctx.needs_input_grad[4], ctx.needs_input_grad[5]
+        # the helper decides what to compute from requires_grad, as the reference does
+        f = feats.detach().requires_grad_(need_f)
+        w = weight.detach().requires_grad_(need_w)
+        b = None if bias is None else bias.detach().requires_grad_(need_b)
+        grad_input, grad_weight, grad_bias = SubMConv3dFunction._sparse_submanifold_conv_backward(
+            grad_output, f, ctx.neighbor_cache, w, b)
+        return grad_input, None, None, None, grad_weight, grad_bias, None
+
+
+def sparse_submanifold_conv3d(
+    feats: torch.Tensor,
+    coords: torch.Tensor,
+    shape: torch.Size,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    neighbor_cache: Optional[SubMConv3dNeighborCache] = None,
+    dilation: Tuple[int, int, int] = (1, 1, 1),
+) -> Tuple[torch.Tensor, SubMConv3dNeighborCache]:
+    """
+    Sparse submanifold convolution for 3D input.
+
+    Args:
+        feats (torch.Tensor): [N, C] tensor of input features.
+        coords (torch.Tensor): [N, 4] int32 tensor of input coordinates (batch, x, y, z).
+        shape (torch.Size): shape of the input tensor in NCWHD order.
+        weight (torch.Tensor): [Co, Kw, Kh, Kd, Ci] tensor of weights.
+        bias (Optional[torch.Tensor]): [Co] tensor of biases.
+        neighbor_cache (Optional[SubMConv3dNeighborCache]): neighbor cache for this operation.
+            Can be reused for multiple runs using the same coordinates; computed on the fly if None.
+        dilation (Tuple[int, int, int]): dilation rate.
+
+    Returns:
+        (output [N, Co], neighbor_cache)
+    """
+    return SubMConv3dFunction.apply(feats, coords, shape, neighbor_cache, weight, bias, dilation)

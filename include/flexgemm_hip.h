@@ -1,0 +1,188 @@
+/*
+ * flexgemm_hip.h -- C ABI of libflexgemm_hip.so (gfx950 / MI355X).
+ *
+ * One shared library replaces the native side of FlexGEMM's submanifold sparse-conv path:
+ * the hash-map neighbor-map builder, its post-processing for the masked implicit GEMM, and
+ * the masked implicit GEMM forward / dgrad / wgrad with split-K.  Each entry point cites the
+ * reference interface it stands in for (paths relative to the reference checkout).
+ *
+ * Conventions
+ *   - every function returns 0 on success or a negative FGX_ERR_* code; fgx_last_error() gives
+ *     the message of the calling thread's last failure;
+ *   - all pointers are DEVICE pointers unless the name ends in _host; the library never
+ *     allocates or frees device memory: the caller owns every buffer, and data-dependent sizes
+ *     are obtained through a "count" call, a 4-byte read-back by the caller, then a "fill" call;
+ *   - `stream` is a hipStream_t (passed as void*); all work is enqueued on it and nothing
+ *     synchronises the host;
+ *   - neighbor tables use 0xFFFFFFFF for "no neighbor".
+ */
+#ifndef FLEXGEMM_HIP_H
+#define FLEXGEMM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FGX_OK 0
+#define FGX_ERR_ARG (-1)      /* bad argument (shape, dtype, alignment, workspace too small) */
+#define FGX_ERR_HIP (-2)      /* a HIP runtime call or kernel launch failed */
+#define FGX_ERR_UNSUPPORTED (-3)
+
+/* element types of feature / weight tensors */
+#define FGX_F16 0
+#define FGX_BF16 1
+#define FGX_F32 2
+
+typedef void* fgx_stream_t;
+
+/* Library identity and error text. */
+int fgx_abi_version(void);
+const char* fgx_last_error(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * Hash table (open addressing, linear probing, Murmur3 finaliser, all-ones key = empty slot).
+ * key_bits / val_bits are 32 or 64.
+ * ------------------------------------------------------------------------------------------- */
+
+/* Fill the key table with the empty sentinel.
+ * Replaces: init_hashmap's torch.full, flex_gemm/ops/utils.py:4-19. */
+int fgx_hash_init(void* keys, int key_bits, size_t table_size, fgx_stream_t stream);
+
+/* keys[] <- flattened (b,x,y,z), vals[] <- row index.
+ * Replaces: hashmap_insert_3d_idx_as_val, flex_gemm/kernels/cuda/hash/hash.cu:425-449. */
+int fgx_hash_insert_3d_idx_as_val(void* keys, int key_bits, void* vals, int val_bits, size_t table_size,
+                                  const int32_t* coords, size_t n, int W, int H, int D, fgx_stream_t stream);
+
+/* Generic key -> value insert / lookup on pre-serialised keys.
+ * Replaces: hashmap_insert / hashmap_lookup, flex_gemm/kernels/cuda/hash/hash.cu:60-89, 139-172. */
+int fgx_hash_insert(void* keys, int key_bits, void* vals, int val_bits, size_t table_size,
+                    const void* in_keys, const void* in_vals, size_t m, fgx_stream_t stream);
+int fgx_hash_lookup(const void* keys, int key_bits, const void* vals, int val_bits, size_t table_size,
+                    const void* in_keys, void* out_vals, size_t m, fgx_stream_t stream);
+
+/* (b,x,y,z) -> user value insert / lookup; a query outside [0,W)x[0,H)x[0,D) yields all ones.
+ * Replaces: hashmap_insert_3d / hashmap_lookup_3d, flex_gemm/kernels/cuda/hash/hash.cu:237-266, 336-365. */
+int fgx_hash_insert_3d(void* keys, int key_bits, void* vals, int val_bits, size_t table_size,
+                       const int32_t* coords, const void* in_vals, size_t m, int W, int H, int D,
+                       fgx_stream_t stream);
+int fgx_hash_lookup_3d(const void* keys, int key_bits, const void* vals, int val_bits, size_t table_size,
+                       const int32_t* coords, void* out_vals, size_t m, int W, int H, int D,
+                       fgx_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Neighbor map and its post-processing.
+ * ------------------------------------------------------------------------------------------- */
+
+/* Insert all voxels (value = row index) into the caller-initialised table, then write the
+ * [n, V] uint32 neighbor table, V = Kw*Kh*Kd (odd kernel sizes).  If gray / binary are non-NULL
+ * (requires V <= 32) the per-voxel validity mask and its Gray-decoded sort key are written in the
+ * same pass (int32 [n] each).
+ * Replaces: hashmap_build_submanifold_conv_neighbour_map,
+ *           flex_gemm/kernels/cuda/spconv/subm_neighbor_map.h:40-47 (.cu:104-162); the fused codes
+ *           replace neighbor_map_to_gray_binary_code_kernel, migemm_neighmap_pp.cu:19-44. */
+int fgx_subm_neighbor_map(void* keys, int key_bits, uint32_t* vals, size_t table_size,
+                          const int32_t* coords, size_t n, int W, int H, int D,
+                          int Kw, int Kh, int Kd, int Dw, int Dh, int Dd,
+                          uint32_t* out_map, int32_t* gray, int32_t* binary, fgx_stream_t stream);
+
+/* Validity mask (bit v <=> map[n, v] present) and Gray-decoded key from an existing map.
+ * Replaces: neighbor_map_to_gray_binary_code_kernel, migemm_neighmap_pp.cu:19-44. */
+int fgx_mask_codes(const uint32_t* map, size_t n, int V, int32_t* gray, int32_t* binary, fgx_stream_t stream);
+
+/* Stable ascending sort of voxels by key (signed int32 compare) -> int64 permutation.
+ * Replaces: torch::argsort(binary_code), migemm_neighmap_pp.cu:79,221 (whose tie order is unspecified;
+ *           this one keeps equal keys in ascending row order).
+ * Workspace: fgx_sort_workspace_bytes(n) bytes, 256-byte aligned. */
+size_t fgx_sort_workspace_bytes(size_t n);
+int fgx_sort_by_code(const int32_t* binary, size_t n, int V, int64_t* sorted_idx,
+                     void* workspace, size_t workspace_bytes, fgx_stream_t stream);
+
+/* Pair lists for wgrad: all (v, n) with map[n, v] present, ordered by v then n.
+ *   count: seg[V+1] <- exclusive offsets per v (seg[V] = L); caller reads seg[V] back, allocates
+ *          sig_i / sig_o of L uint32 each, then calls fill with the same workspace.
+ * Replaces: neighbor_map_post_process_for_masked_implicit_gemm_1's transposed map + cumsum +
+ *           gather_idx_val_seg_from_prefix_sum_kernel, migemm_neighmap_pp.cu:157-178, 207-240. */
+size_t fgx_pair_workspace_bytes(size_t n, int V);
+int fgx_pair_count(const int32_t* gray, size_t n, int V, uint32_t* seg,
+                   void* workspace, size_t workspace_bytes, fgx_stream_t stream);
+int fgx_pair_fill(const uint32_t* map, const int32_t* gray, size_t n, int V,
+                  const void* workspace, uint32_t* sig_i, uint32_t* sig_o, fgx_stream_t stream);
+
+/* Per row-tile (block consecutive rows of the sorted order) OR of the masks.
+ *   codes: tile_code[nb] <- OR mask, seg[nb+1] <- exclusive offsets of popcounts (seg[nb] = total);
+ *   fill : valid_kernel[total] <- set-bit positions, ascending per tile.
+ * Replaces: neighbor_map_post_process_for_masked_implicit_gemm_2 (reduce_code_kernel, cumsum,
+ *           scatter_reduced_code_kernel), migemm_neighmap_pp.cu:246-368.  Any block >= 1 is accepted. */
+size_t fgx_tile_workspace_bytes(size_t n, int block);
+int fgx_tile_codes(const int32_t* gray, const int64_t* sorted_idx, size_t n, int block,
+                   int32_t* tile_code, int32_t* seg, void* workspace, size_t workspace_bytes,
+                   fgx_stream_t stream);
+int fgx_tile_fill(const int32_t* tile_code, const int32_t* seg, size_t num_tiles, int32_t* valid_kernel,
+                  fgx_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Masked implicit GEMM.
+ * ------------------------------------------------------------------------------------------- */
+
+/* Fixed gfx950 schedule for a problem (replaces the Triton autotuner and autotune_cache.json:
+ * flex_gemm/utils/autotuner.py:18-291, flex_gemm/kernels/triton/spconv/config.py:10-83 and the
+ * SPLITK searches in ..._masked_implicit_gemm_splitk.py).  `pass_kind`: 0 fwd, 1 dgrad, 2 wgrad. */
+typedef struct fgx_schedule {
+    int tile_rows;      /* fwd/dgrad: sorted voxel rows per tile (B1); wgrad: Co rows per tile */
+    int tile_cols;      /* fwd/dgrad: output channels per tile (B2);   wgrad: Ci columns per tile */
+    int splitk;         /* fwd/dgrad: number of K splits (1 = none) */
+    int chunk_pairs;    /* wgrad: pairs per partial-sum chunk */
+} fgx_schedule;
+int fgx_table_lookup(int pass_kind, int dtype, size_t n, int Ci, int Co, int V, fgx_schedule* out);
+
+/* Re-layout the [Co, V, Ci] weight into K-slab-major panels consumed by fgx_conv_gather_gemm.
+ *   mode 0 (forward): panel[v][slab][co][k]  = w[co][v][slab*SK + k]          (K = Ci, cols = Co)
+ *   mode 1 (dgrad)  : panel[v][slab][ci][k]  = w[slab*SK + k][V-1-v][ci]      (K = Co, cols = Ci)
+ * SK = 128 bytes / element size; K is zero-padded to a whole slab and cols to a multiple of col_pad
+ * (a multiple of 32; pass the tile_cols the GEMM will run with).
+ * Replaces: the strided weight-tile loads of the Triton kernels
+ *           (..._fwd_masked_implicit_gemm.py:79, ..._bwd_masked_implicit_gemm.py:74). */
+size_t fgx_weight_panel_bytes(int dtype, int mode, int Ci, int Co, int V, int col_pad);
+int fgx_pack_weight(int dtype, int mode, const void* weight, int Ci, int Co, int V, int col_pad, void* panel,
+                    fgx_stream_t stream);
+
+/* out[sorted[r], :] = sum over offsets v present in row r of src[map[sorted[r], v], :] . panel_v  (+ bias)
+ * for K = src channels, cols = out channels.  Forward: src = feats, panel mode 0, bias optional.
+ * dgrad: src = grad_output, panel mode 1, bias = NULL.  Tiles of `tile_rows` sorted rows skip every
+ * offset whose bit is clear in tile_code[tile].  splitk > 1 needs `scratch` of
+ * fgx_conv_scratch_bytes() bytes (fp32 partial sums, reduced in a second kernel).
+ * Replaces: sparse_submanifold_conv_fwd_masked_implicit_gemm[_splitk] (kernels
+ *           ..._fwd_masked_implicit_gemm.py:20-100, ..._splitk.py:22-106, wrapper :133-172) and
+ *           sparse_submanifold_conv_bwd_input_masked_implicit_gemm[_splitk]
+ *           (..._bwd_masked_implicit_gemm.py:19-91, ..._splitk.py:24-100, 209-251). */
+size_t fgx_conv_scratch_bytes(size_t n, int cols, int splitk);
+int fgx_conv_gather_gemm(int dtype, const void* src, const void* panel, const void* bias,
+                         const uint32_t* map, const int64_t* sorted_idx, const int32_t* tile_code,
+                         size_t n, int K, int cols, int V, int tile_rows, int tile_cols, int splitk,
+                         void* scratch, void* out, fgx_stream_t stream);
+
+/* grad_weight[co, v, ci] = sum over pairs k in [seg[v], seg[v+1]) of grad_out[sig_o[k], co] * feats[sig_i[k], ci].
+ * seg_host is the HOST copy of valid_signal_seg (V+1 entries).  Partial sums of `chunk_pairs` pairs go to
+ * `scratch` (fgx_wgrad_scratch_bytes bytes, fp32) and are reduced per offset in a second kernel.
+ * Replaces: sparse_submanifold_conv_bwd_weight_masked_implicit_gemm[_splitk]
+ *           (..._bwd_masked_implicit_gemm.py:99-170, ..._splitk.py:108-182, 278-317). */
+size_t fgx_wgrad_scratch_bytes(const uint32_t* seg_host, int V, int Ci, int Co, int chunk_pairs);
+int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats,
+                   const uint32_t* sig_i, const uint32_t* sig_o, const uint32_t* seg_host,
+                   size_t n, int Ci, int Co, int V, int tile_rows, int tile_cols, int chunk_pairs,
+                   void* scratch, void* grad_weight, fgx_stream_t stream);
+
+/* grad_bias[co] = sum over rows of grad_out[:, co], accumulated in fp32.
+ * `scratch`: fgx_colsum_scratch_bytes bytes of fp32 partial sums.
+ * Replaces: grad_output.sum(0), ..._bwd_masked_implicit_gemm_splitk.py:365-366. */
+size_t fgx_colsum_scratch_bytes(size_t n, int cols);
+int fgx_colsum(int dtype, const void* grad_out, size_t n, int cols, void* scratch, void* out,
+               fgx_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLEXGEMM_HIP_H */

@@ -1,0 +1,126 @@
+"""The C-ABI library builds, loads and exports every symbol include/flexgemm_hip.h declares (CPU only:
+no compute call is made)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from flexgemm_amd import _native as nat
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "flexgemm_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fgx_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def library():
+    if not os.path.exists(nat.lib_path()):
+        from flexgemm_amd import build
+        build.build(verbose=False)
+    return ctypes.CDLL(nat.lib_path())
+
+
+def test_header_and_binding_agree():
+    assert _declared_symbols() == sorted(nat.EXPORTS)
+
+
+def test_every_declared_symbol_is_exported(library):
+    for name in _declared_symbols():
+        assert hasattr(library, name), name
+
+
+def test_host_only_entry_points(library):
+    # these touch no device: identity, sizing and the schedule table
+    assert library.fgx_abi_version() == 1
+    L = nat.lib()
+    import torch
+    s = nat.table_lookup(nat.PASS_FWD, torch.float16, 669288, 128, 128, 27)
+    assert (s.tile_rows, s.tile_cols, s.splitk) == (128, 128, 1)
+    s = nat.table_lookup(nat.PASS_WGRAD, torch.float16, 669288, 128, 128, 27)
+    assert s.chunk_pairs % 64 == 0 and s.chunk_pairs > 0
+    s = nat.table_lookup(nat.PASS_FWD, torch.float32, 100, 16, 16, 27)
+    assert s.tile_rows in (32, 64, 128) and s.tile_cols == 32 and s.splitk >= 1
+    assert L.fgx_weight_panel_bytes(0, 0, 128, 128, 27, 128) == 27 * 2 * 128 * 128
+    assert L.fgx_weight_panel_bytes(2, 1, 40, 24, 27, 32) == 27 * 1 * 64 * 128      # K=24 -> 1 slab, cols 40 -> 64
+    assert L.fgx_conv_scratch_bytes(ctypes.c_size_t(1000), 64, 1) == 0
+    assert L.fgx_conv_scratch_bytes(ctypes.c_size_t(1000), 64, 4) == 4 * 1000 * 64 * 4
+    seg = (ctypes.c_uint32 * 4)(0, 100, 100, 300)
+    assert L.fgx_wgrad_scratch_bytes(seg, 3, 8, 16, 64) == (2 + 0 + 4) * 8 * 16 * 4
+
+
+def test_argument_errors_map_to_exceptions(library):
+    L = nat.lib()
+    with pytest.raises(ValueError):
+        nat.check(L.fgx_hash_init(None, 16, ctypes.c_size_t(8), None))
+    assert b"key_bits" in L.fgx_last_error()
+    with pytest.raises(ValueError):
+        nat.check(L.fgx_subm_neighbor_map(None, 32, None, ctypes.c_size_t(0), None, ctypes.c_size_t(0), 4, 4, 4,
+                                          2, 3, 3, 1, 1, 1, None, None, None, None))
+    with pytest.raises(ValueError):
+        nat.check(L.fgx_conv_wgrad(0, None, None, None, None, None, ctypes.c_size_t(0), 8, 8, 27, 128, 128, 100,
+                                   None, None, None))
+
+
+def test_host_logic_without_gpu():
+    import torch
+    import flex_gemm
+    from flex_gemm.ops.spconv import Algorithm, SubMConv3dFunction, SubMConv3dNeighborCache
+    coords = torch.zeros((1, 4), dtype=torch.int32)
+    flex_gemm.ops.spconv.set_algorithm(Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
+    with pytest.raises(NotImplementedError):
+        SubMConv3dFunction._compute_neighbor_cache(coords, torch.Size([1, 1, 4, 4, 4]), (3, 3, 3), (1, 1, 1), False)
+    with pytest.raises(AssertionError):
+        SubMConv3dFunction._compute_neighbor_cache(coords.long(), torch.Size([1, 1, 4, 4, 4]), (3, 3, 3), (1, 1, 1), False)
+    flex_gemm.ops.spconv.set_algorithm("nonsense")
+    with pytest.raises(ValueError):
+        SubMConv3dFunction._compute_neighbor_cache(coords, torch.Size([1, 1, 4, 4, 4]), (3, 3, 3), (1, 1, 1), False)
+    flex_gemm.ops.spconv.set_algorithm(Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
+    c = SubMConv3dNeighborCache(a=1)
+    c["b"] = 2
+    assert c["a"] == 1 and c.b == 2
+    with pytest.raises(AttributeError):
+        c["missing"]
+    # masked algorithms never fall back to the CPU
+    with pytest.raises(NotImplementedError):
+        SubMConv3dFunction._sparse_submanifold_conv_forward(
+            torch.zeros(1, 8), SubMConv3dNeighborCache(neighbor_map=torch.zeros((1, 27), dtype=torch.int32)),
+            torch.zeros(8, 3, 3, 3, 8), None)
+
+
+def test_explicit_algorithm_matches_oracle_on_cpu():
+    """The EXPLICIT_GEMM algorithm is plain torch ops and runs on any device, like the reference's."""
+    import numpy as np
+    import torch
+    import flex_gemm
+    from flex_gemm.ops.spconv import Algorithm, SubMConv3dFunction, sparse_submanifold_conv3d
+    from flexgemm_amd.workloads import reference_test_shell
+    from oracle import explicit_gemm as eg
+    from oracle import neighbor as nb
+    flex_gemm.ops.spconv.set_algorithm(Algorithm.EXPLICIT_GEMM)
+    try:
+        res, ci, co = 8, 6, 5
+        coords = torch.from_numpy(reference_test_shell(res))
+        shape = torch.Size([1, ci, res, res, res])
+        cache = SubMConv3dFunction._compute_neighbor_cache_torch(coords, shape, (3, 3, 3), (1, 1, 1))
+        ref_map = nb.neighbor_map(coords.numpy(), tuple(shape))
+        assert cache.neighbor_map.dtype == torch.uint32
+        assert np.array_equal(cache.neighbor_map.numpy(), ref_map)
+        g = torch.Generator().manual_seed(0)
+        feats = torch.randn(len(coords), ci, generator=g, dtype=torch.float64, requires_grad=True)
+        weight = torch.randn(co, 3, 3, 3, ci, generator=g, dtype=torch.float64, requires_grad=True)
+        bias = torch.randn(co, generator=g, dtype=torch.float64, requires_grad=True)
+        out, cache2 = sparse_submanifold_conv3d(feats, coords, shape, weight, bias, neighbor_cache=cache)
+        assert cache2 is cache
+        grad = torch.randn(len(coords), co, generator=g, dtype=torch.float64)
+        out.backward(grad)
+        nm = torch.from_numpy(ref_map.view(np.int32))
+        assert torch.allclose(out.detach(), eg.forward(feats.detach(), nm, weight.detach(), bias.detach()))
+        gi, gw, gb = eg.backward(grad, feats.detach(), nm, weight.detach())
+        assert torch.allclose(feats.grad, gi) and torch.allclose(weight.grad, gw) and torch.allclose(bias.grad, gb)
+    finally:
+        flex_gemm.ops.spconv.set_algorithm(Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)

@@ -1,0 +1,202 @@
+"""GPU parity of the masked implicit GEMM (forward, dgrad, wgrad, dbias) against the explicit gather-GEMM oracle.
+
+Tolerances (stated by the build's north star): max relative error <= 1e-2 for fp16 / bf16 and <= 1e-4 for fp32.
+Two readings of "relative error" are asserted, both against the oracle evaluated in float64 on the same
+(already rounded) inputs: the reference's own metric max(min(|d|, |d|/|ref|)) (tests/utils.py:28-32) and
+max|d| / max|ref|.
+"""
+import math
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import flex_gemm
+from flex_gemm.ops.spconv import Algorithm, SubMConv3dFunction, sparse_submanifold_conv3d
+from flexgemm_amd.workloads import make_workload, reference_test_shell
+from oracle import explicit_gemm as eg
+from oracle import neighbor as nb
+
+pytestmark = pytest.mark.gpu
+TOL = {torch.float16: 1e-2, torch.bfloat16: 1e-2, torch.float32: 1e-4}
+
+
+def _say(msg):
+    print(f"[case] {msg}", flush=True)
+    sys.stdout.flush()
+
+
+def _assert_close(got, ref64, dtype, what):
+    got = got.detach().cpu()
+    tol = TOL[dtype]
+    e_ref_metric = eg.calc_err(got, ref64)[0]
+    e_scaled = eg.max_rel_err(got, ref64)
+    assert e_ref_metric <= tol and e_scaled <= tol, f"{what}: min(abs,rel)={e_ref_metric:.3e} scaled={e_scaled:.3e} tol={tol}"
+    return e_ref_metric, e_scaled
+
+
+def _case(coords_np, ci, co, dtype, seed, ksize=(3, 3, 3), wscale=None):
+    g = torch.Generator().manual_seed(seed)
+    n = len(coords_np)
+    v = ksize[0] * ksize[1] * ksize[2]
+    feats = torch.randn(n, ci, generator=g).to(dtype)
+    weight = (torch.randn(co, *ksize, ci, generator=g) * (wscale or 1.0 / math.sqrt(v * ci))).to(dtype)
+    bias = torch.randn(co, generator=g).to(dtype)
+    grad = torch.randn(n, co, generator=g).to(dtype)
+    return feats, weight, bias, grad
+
+
+def _run_and_check(coords_np, shape, ci, co, dtype, dev, seed=0, ksize=(3, 3, 3), dilation=(1, 1, 1), use_bias=True,
+                   algo=Algorithm.MASKED_IMPLICIT_GEMM_SPLITK, cache=None):
+    feats, weight, bias, grad = _case(coords_np, ci, co, dtype, seed, ksize)
+    nmap = torch.from_numpy(nb.neighbor_map(coords_np, tuple(shape), ksize, dilation).view(np.int32))
+    f64, w64, b64, g64 = feats.double(), weight.double(), bias.double(), grad.double()
+    ref_out = eg.forward(f64, nmap, w64, b64 if use_bias else None)
+    ref_gi, ref_gw, ref_gb = eg.backward(g64, f64, nmap, w64)
+    flex_gemm.ops.spconv.set_algorithm(algo)
+    try:
+        f = feats.to(dev).requires_grad_(True)
+        w = weight.to(dev).requires_grad_(True)
+        b = bias.to(dev).requires_grad_(True) if use_bias else None
+        coords = torch.from_numpy(coords_np).to(dev)
+        out, cache = sparse_submanifold_conv3d(f, coords, shape, w, b, neighbor_cache=cache, dilation=dilation)
+        assert out.dtype == dtype and out.shape == (len(coords_np), co)
+        out.backward(grad.to(dev))
+        torch.cuda.synchronize()
+        errs = [_assert_close(out, ref_out, dtype, "forward"),
+                _assert_close(f.grad, ref_gi, dtype, "dgrad"),
+                _assert_close(w.grad, ref_gw, dtype, "wgrad")]
+        assert w.grad.shape == weight.shape
+        if use_bias:
+            errs.append(_assert_close(b.grad, ref_gb, dtype, "dbias"))
+    finally:
+        flex_gemm.ops.spconv.set_algorithm(Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
+    return cache, errs
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("res,ci,co", [(16, 32, 32), (16, 64, 64), (32, 128, 128), (24, 64, 128), (24, 256, 32), (8, 1024, 64)])
+def test_conv_matches_oracle(gpu_device, dtype, res, ci, co):
+    _say(f"conv res={res} ci={ci} co={co} {dtype}")
+    coords_np = reference_test_shell(res)
+    _run_and_check(coords_np, torch.Size([1, ci, res, res, res]), ci, co, dtype, gpu_device, seed=res + ci)
+
+
+@pytest.mark.parametrize("res", [1, 2, 4])
+def test_degenerate_sizes(gpu_device, res):
+    # fewer voxels than one tile; N = 1 at res 1
+    _say(f"conv degenerate res={res}")
+    coords_np = reference_test_shell(res)
+    for dtype in (torch.float16, torch.float32):
+        _run_and_check(coords_np, torch.Size([1, 64, res, res, res]), 64, 64, dtype, gpu_device, seed=res)
+
+
+def test_odd_channel_counts_batches_dilation_no_bias(gpu_device):
+    rng = np.random.default_rng(3)
+    res = 12
+    coords_np = reference_test_shell(res, batch=2)
+    coords_np = coords_np[rng.permutation(len(coords_np))]
+    shape = torch.Size([2, 0, res, res, res])
+    for ci, co, dtype in [(5, 7, torch.float32), (20, 12, torch.float16), (48, 96, torch.bfloat16), (3, 130, torch.float16)]:
+        _say(f"conv odd channels ci={ci} co={co} {dtype}")
+        _run_and_check(coords_np, shape, ci, co, dtype, gpu_device, seed=ci, dilation=(2, 1, 1), use_bias=False)
+    _say("conv 1x3x3 kernel")
+    _run_and_check(coords_np, shape, 32, 32, torch.float16, gpu_device, seed=1, ksize=(1, 3, 3))
+
+
+def test_algorithm_values_and_cache_reuse(gpu_device):
+    res, c = 16, 64
+    coords_np = reference_test_shell(res)
+    shape = torch.Size([1, c, res, res, res])
+    cache = None
+    for algo in (Algorithm.MASKED_IMPLICIT_GEMM_SPLITK, Algorithm.MASKED_IMPLICIT_GEMM, Algorithm.IMPLICIT_GEMM,
+                 Algorithm.IMPLICIT_GEMM_SPLITK, Algorithm.EXPLICIT_GEMM):
+        _say(f"conv algorithm {algo}")
+        cache, _ = _run_and_check(coords_np, shape, c, c, torch.float16, gpu_device, seed=5, algo=algo, cache=cache)
+    # a cache built without gradients (inference) is completed on demand when a training step reuses it
+    _say("inference cache reused for training")
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    inf_cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), False)
+    assert not hasattr(inf_cache, "valid_signal_i")
+    _run_and_check(coords_np, shape, c, c, torch.float16, gpu_device, seed=6, cache=inf_cache)
+    # under no_grad the operator builds the inference cache itself
+    with torch.no_grad():
+        f, w, b, _ = _case(coords_np, c, c, torch.float16, 7)
+        out, cch = sparse_submanifold_conv3d(f.to(gpu_device), coords, shape, w.to(gpu_device), b.to(gpu_device))
+    assert not hasattr(cch, "valid_signal_i") and out.shape == (len(coords_np), c)
+
+
+def test_forced_splitk_matches_unsplit(gpu_device):
+    """Split-K partial sums add up to the unsplit result (fp32 rounding apart)."""
+    import ctypes as C
+    from flexgemm_amd import _native as nat
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    res, c = 16, 128
+    _say("forced split-K")
+    coords_np = reference_test_shell(res)
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    shape = torch.Size([1, c, res, res, res])
+    f, w, b, _ = _case(coords_np, c, c, torch.float16, 9)
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), False)
+    outs = []
+    real = nat.table_lookup
+    for s in (1, 2, 5):
+        def forced(*a, _s=s):
+            sc = real(*a)
+            sc.splitk = _s
+            return sc
+        nat.table_lookup = forced
+        try:
+            outs.append(impl._gather_gemm(f.to(gpu_device), w.to(gpu_device).reshape(c, 27, c), b.to(gpu_device), cache, 0, True).float().cpu())
+        finally:
+            nat.table_lookup = real
+    assert eg.max_rel_err(outs[1], outs[0].double()) <= 2e-3 and eg.max_rel_err(outs[2], outs[0].double()) <= 2e-3
+
+
+@pytest.mark.parametrize("name,res,c", [("cfg2", 64, 256), ("cfg3", 128, 128), ("cfg4", 128, 32), ("cfg5", 32, 1024)])
+def test_scaled_down_benchmark_configs(gpu_device, name, res, c):
+    """The benchmark configurations at a resolution the float64 oracle finishes in seconds."""
+    _say(f"conv {name} at res {res}")
+    wl = make_workload(name, res=res, with_values=False)
+    _run_and_check(wl.coords.numpy(), wl.shape, c, c, wl.dtype, gpu_device, seed=11)
+
+
+def test_cfg5_fp32_variant(gpu_device):
+    _say("conv cfg5 fp32 variant at res 32")
+    wl = make_workload("cfg5", res=32, with_values=False)
+    _, errs = _run_and_check(wl.coords.numpy(), wl.shape, 1024, 1024, torch.float32, gpu_device, seed=12)
+    assert max(e[1] for e in errs) <= 1e-4
+
+
+def test_full_size_properties_cfg3(gpu_device):
+    """Configuration 3 at full size (669 288 voxels, C = 128, fp16): the float64 oracle is evaluated on a random
+    sample of output rows (forward, dgrad) and the closed-form identities <conv(f), g> = <f, dgrad(g)> = <W, wgrad>
+    tie the three passes together."""
+    _say("conv cfg3 full size")
+    wl = make_workload("cfg3")
+    dev = gpu_device
+    dt = torch.float16
+    f = wl.feats.to(dt).to(dev).requires_grad_(True)
+    w = wl.weight.to(dt).to(dev).requires_grad_(True)
+    b = wl.bias.to(dt).to(dev).requires_grad_(True)
+    g = wl.grad.to(dt)
+    coords = wl.coords.to(dev)
+    out, cache = sparse_submanifold_conv3d(f, coords, wl.shape, w, b)
+    out.backward(g.to(dev))
+    torch.cuda.synchronize()
+    nmap = cache.neighbor_map.cpu().view(torch.int32)
+    rows = torch.randperm(wl.n, generator=torch.Generator().manual_seed(0))[:4096]
+    f64, w64, b64, g64 = f.detach().cpu().double(), w.detach().cpu().double(), b.detach().cpu().double(), g.double()
+    ref_rows = eg.forward(f64, nmap[rows], w64, b64)
+    _assert_close(out[rows.to(dev)], ref_rows, dt, "forward sample")
+    ref_gi = torch.mm(eg._im2col(g64, torch.flip(nmap[rows].long(), [1])), w64.reshape(128, 27, 128).transpose(0, 1).reshape(27 * 128, 128))
+    _assert_close(f.grad[rows.to(dev)], ref_gi, dt, "dgrad sample")
+    # inner-product identities in float64 from the GPU results (bias-free part)
+    conv_nobias = out.detach().cpu().double() - b64
+    lhs = (conv_nobias * g64).sum()
+    mid = (f64 * f.grad.cpu().double()).sum()
+    rhs = (w64 * w.grad.cpu().double()).sum()
+    scale = float((conv_nobias.abs() * g64.abs()).sum())
+    assert abs(lhs - mid) / scale < 1e-3 and abs(lhs - rhs) / scale < 1e-3
+    assert eg.max_rel_err(b.grad.cpu(), g64.sum(0)) <= 1e-2
