@@ -1,0 +1,225 @@
+#!/usr/bin/env python3
+"""Benchmark of the submanifold sparse-conv hot path on one MI355X.
+
+One "step" is one training pass of a single 3x3x3 submanifold conv layer over one synthetic batch:
+forward + dgrad + wgrad (+ dbias) through the masked implicit GEMM, with the neighbor cache built once
+before the timed region and reused (the reference's benchmark does the same: tests/submconv/train_benchmark.py:152-160).
+Inputs are resident in HBM when the timed region starts.
+
+Headline workload (N = 1): configuration 3 -- res 512 shell (669 288 voxels), Ci = Co = 128, fp16.
+`value` = effective TFLOP/s = useful FLOP / time with useful FLOP = 6 * L * Ci * Co per step
+(L = valid neighbor pairs; the reference's accounting: tests/submconv/fwd.py:247-249, bwd.py:288-290).
+
+Prints ONE JSON line.  `--workload cfg2|cfg3|cfg4|cfg5` selects another configuration (cfg2 is forward only).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}   # MI355X dense MFMA peaks
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=50)
+    p.add_argument("--warmup", type=int, default=5)
+    p.add_argument("--workload", default="cfg3", choices=["cfg2", "cfg3", "cfg4", "cfg5"])
+    p.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (used under rocprofv3)")
+    p.add_argument("--cpu-rows", type=int, default=0, help="rows in the CPU baseline sample (0 = auto)")
+    p.add_argument("--build-only", action="store_true", help="time only the neighbor-cache build")
+    return p.parse_args()
+
+
+def cpu_baseline(wl, nmap_cpu, passes, rows_hint):
+    """Explicit gather-GEMM oracle (torch CPU, fp32) timed on a bounded row sample of the same workload."""
+    import torch
+    from oracle import explicit_gemm as eg
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    c = wl.channels
+    rows = rows_hint or max(1024, min(wl.n, int(3.0e8 / (27 * c))))     # im2col sample <= 0.3 G elements
+    rows = min(rows, wl.n)
+    sel = torch.arange(rows)
+    sub = nmap_cpu[sel]
+    f32, w32, b32, g32 = wl.feats.float(), wl.weight.float(), wl.bias.float(), wl.grad.float()
+    l_sample = int((sub >= 0).sum())
+
+    def run():
+        eg.forward(f32, sub, w32, b32)
+        if passes == 3:
+            # dgrad for the sampled output rows; wgrad contribution of the sampled rows; dbias of the sample
+            inv = torch.flip(sub.long(), [1])
+            wt = w32.reshape(c, 27, c).transpose(0, 1).reshape(27 * c, c)
+            torch.mm(eg._im2col(g32, inv), wt)
+            torch.mm(eg._im2col(f32, sub.long()).t(), g32[sel])
+            g32[sel].sum(0)
+
+    run()                                   # warm-up (page faults, thread pool)
+    t0 = time.perf_counter()
+    iters = 0
+    while True:
+        run()
+        iters += 1
+        if time.perf_counter() - t0 > 10.0 or iters >= 20:
+            break
+    dt = (time.perf_counter() - t0) / iters
+    flop = 2.0 * l_sample * c * c * passes
+    return {
+        "value": flop / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+        "sample": f"first {rows} rows of {wl.name} ({l_sample} valid pairs), {'fwd+dgrad+wgrad' if passes == 3 else 'fwd'}, "
+                  f"explicit gather-GEMM in torch CPU fp32 (substituted for {str(wl.dtype).split('.')[-1]}), {iters} iters, "
+                  f"{dt * 1e3:.1f} ms/iter",
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (the hot path is a single-device operator); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import flex_gemm
+    from flex_gemm.ops.spconv import Algorithm, SubMConv3dFunction
+    from flexgemm_amd import _native as nat
+    from flexgemm_amd.workloads import make_workload
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    nat.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    flex_gemm.ops.spconv.set_algorithm(Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
+
+    wl = make_workload(args.workload)
+    dt = wl.dtype
+    dname = {torch.float16: "f16", torch.bfloat16: "bf16", torch.float32: "f32"}[dt]
+    c = wl.channels
+    passes = 1 if args.workload == "cfg2" else 3
+    coords = wl.coords.to(dev)
+    feats = wl.feats.to(dt).to(dev).requires_grad_(passes == 3)
+    weight = wl.weight.to(dt).to(dev).requires_grad_(passes == 3)
+    bias = wl.bias.to(dt).to(dev).requires_grad_(passes == 3)
+    grad = wl.grad.to(dt).to(dev)
+
+    # ---- neighbor cache: built once, timed separately ----
+    def build_cache():
+        return SubMConv3dFunction._compute_neighbor_cache(coords, wl.shape, (3, 3, 3), (1, 1, 1), passes == 3)
+
+    cache = build_cache()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    build_ms = []
+    for _ in range(5):
+        ev0.record()
+        cache = build_cache()
+        ev1.record()
+        torch.cuda.synchronize()
+        build_ms.append(ev0.elapsed_time(ev1))
+    build_ms.sort()
+    pairs = int(cache.valid_signal_seg.view(torch.int32)[-1].item()) if passes == 3 else \
+        int((cache.neighbor_map.view(torch.int32) != -1).sum().item())
+    n = wl.n
+    build_bytes = 152.0 * n + (8.0 * pairs + 4 * 28 if passes == 3 else 0.0)
+    if args.build_only:
+        print(json.dumps({"metric": "neighbor-cache build", "workload": args.workload, "n": n, "pairs": pairs,
+                          "build_ms_median": build_ms[len(build_ms) // 2], "build_ms_min": build_ms[0],
+                          "algorithmic_GBps": build_bytes / (build_ms[len(build_ms) // 2] * 1e-3) / 1e9}))
+        return
+
+    # ---- the step ----
+    def step():
+        out = SubMConv3dFunction._sparse_submanifold_conv_forward(feats, cache, weight, bias)
+        if passes == 3:
+            return out, SubMConv3dFunction._sparse_submanifold_conv_backward(grad, feats, cache, weight, bias)
+        return out, None
+
+    for _ in range(max(args.warmup, 1)):
+        step()
+    torch.cuda.synchronize()
+
+    # HIP events around the dominant kernel's launches, on the stream they are launched on
+    events = {}
+
+    def hook(name, phase):
+        e = torch.cuda.Event(enable_timing=True)
+        e.record(torch.cuda.current_stream())
+        events.setdefault(name, []).append(e)
+
+    nat.EVENT_HOOK = hook
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    nat.EVENT_HOOK = None
+
+    ms_per_step = elapsed * 1e3 / args.steps
+    flop_pass = 2.0 * pairs * c * c
+    value = flop_pass * passes / (ms_per_step * 1e-3) / 1e12
+
+    def avg_ms(names):
+        tot, cnt = 0.0, 0
+        for nm in names:
+            ev = events.get(nm, [])
+            for i in range(0, len(ev) - 1, 2):
+                tot += ev[i].elapsed_time(ev[i + 1])
+                cnt += 1
+        return (tot / cnt if cnt else float("nan")), cnt
+
+    gemm_ms, gemm_launches = avg_ms(["gather_gemm_fwd", "gather_gemm_dgrad"])
+    wgrad_ms, _ = avg_ms(["wgrad"])
+    es = 2 if dname != "f32" else 4
+    gemm_bytes = es * n * (c + c) + es * 27 * c * c + 108.0 * n + 8.0 * n
+    roof = {
+        "bound": "mfma", "kernel": "gather_gemm_kernel (forward and dgrad launches)",
+        "achieved": flop_pass / (gemm_ms * 1e-3) / 1e12, "peak": PEAK_TFLOPS[dname], "unit": "TFLOP/s",
+        "frac": flop_pass / (gemm_ms * 1e-3) / 1e12 / PEAK_TFLOPS[dname],
+        "avg_launch_ms": gemm_ms, "launches_timed": gemm_launches,
+        "algorithmic_flop_per_launch": flop_pass,
+        "algorithmic_bytes_per_launch": gemm_bytes,
+        "algorithmic_hbm_GBps": gemm_bytes / (gemm_ms * 1e-3) / 1e9,
+        "traffic": None,
+    }
+    if args.workload == "cfg4":   # C = 32: every pass is HBM bound
+        roof.update({"bound": "hbm", "achieved": gemm_bytes / (gemm_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": gemm_bytes / (gemm_ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
+
+    result = {
+        "metric": "effective TFLOPS (useful MACs over valid neighbor pairs), submconv3d 3^3 "
+                  + ("fwd+dgrad+wgrad" if passes == 3 else "fwd") + f", res{wl.res} C={c}",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dname, "data": "synthetic",
+        "config": {"workload": f"{args.workload}: res {wl.res} shell, N={n}, L={pairs}, Ci=Co={c}, {dname}, "
+                               + ("fwd+dgrad+wgrad+dbias, neighbor cache prebuilt and reused" if passes == 3 else "forward"),
+                   "n_voxels": n, "valid_pairs": pairs, "useful_gflop_per_step": flop_pass * passes / 1e9},
+        "frac_of_mfma_peak": value / PEAK_TFLOPS[dname],
+        "pass_ms": {"gather_gemm_avg": gemm_ms, "wgrad_incl_reduce": wgrad_ms},
+        "neighbor_cache_build": {"ms_median": build_ms[len(build_ms) // 2], "ms_min": build_ms[0],
+                                 "algorithmic_bytes": build_bytes,
+                                 "algorithmic_GBps": build_bytes / (build_ms[len(build_ms) // 2] * 1e-3) / 1e9,
+                                 "frac_of_hbm_peak": build_bytes / (build_ms[len(build_ms) // 2] * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        "roofline": roof,
+    }
+    if not args.no_cpu_baseline:
+        nmap_cpu = cache.neighbor_map.cpu().view(torch.int32)
+        result["cpu_baseline"] = cpu_baseline(wl, nmap_cpu, passes, args.cpu_rows)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

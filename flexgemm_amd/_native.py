@@ -35,8 +35,18 @@ EXPORTS = [
 ]
 
 
+# Optional profiling hook: callable(name, phase) with phase "start"/"stop", invoked on the launching thread right
+# before / after the named native call is enqueued (bench.py records HIP events on the current stream from it).
+EVENT_HOOK = None
+
+
+def mark(name: str, phase: str) -> None:
+    if EVENT_HOOK is not None:
+        EVENT_HOOK(name, phase)
+
+
 class Schedule(C.Structure):
-    _fields_ = [("tile_rows", C.c_int), ("tile_cols", C.c_int), ("splitk", C.c_int), ("chunk_pairs", C.c_int)]
+    _fields_ = [("tile_rows", C.c_int), ("tile_cols", C.c_int), ("splitk", C.c_int), ("block_rows", C.c_int)]
 
 
 class NativeError(RuntimeError):

@@ -3,16 +3,24 @@
 //   out[sorted[r], :] = sum over offsets v present for row r of src[map[sorted[r], v], :] x panel_v (+ bias)
 //
 // One workgroup owns a tile of BM consecutive rows of the mask-sorted voxel order and BN output
-// channels.  Offsets whose bit is clear in the tile's OR-mask are skipped altogether.  For every
-// remaining (offset, K-slab) step the gathered source rows (A, BM x 128 bytes) and the matching
-// panel slice (B, BN x 128 bytes) are staged in LDS with an XOR swizzle on 16-byte chunks, and each
-// of the WAVES_M x WAVES_N wavefronts multiplies its (BM/WAVES_M) x (BN/WAVES_N) sub-tile with
-// 32x32 MFMA instructions, accumulating in fp32.  Global loads of step s+1 are issued before the
-// MFMAs of step s (register-staged double buffering, one barrier per step).
+// channels.  Offsets whose bit is clear in the tile's OR-mask are skipped altogether.  The remaining
+// (offset, K-slab) steps stream through an S-stage ring in LDS: a stage holds the gathered source rows
+// (A, BM x 64 bytes) and the matching weight-panel slice (B, BN x 64 bytes).  Stages are filled by
+// direct global->LDS loads (global_load_lds_dwordx4: lane i of a wavefront deposits its 16 bytes at
+// LDS base + 16 i), issued S-1 steps ahead of their use, so several gathers are in flight per
+// workgroup while the wavefronts multiply.  The only vector-memory operations in the main loop are
+// these loads, which makes the outstanding-load counter exact: "step k has landed" is
+// s_waitcnt vmcnt((S-2) * loads_per_step), followed by one workgroup barrier per step.  Steps past the
+// end still issue (dummy) loads so that the count never changes.
 //
-// Both operands are K-contiguous per row, and A and B fragments are read from LDS with the same
-// (chunk, lane-group) -> k assignment, so the contraction is independent of how the hardware
-// numbers k inside a fragment.
+// The gather is a per-lane choice of global address, so a missing neighbor (or a K tail) simply reads
+// a block of zeros, and the bank-conflict swizzle of the 16-byte chunks is applied on the global side
+// (lane -> which chunk of the row it fetches) since the LDS side of the load is fixed.
+//
+// Each of the WAVES_M x WAVES_N wavefronts multiplies its (BM/WAVES_M) x (BN/WAVES_N) sub-tile with
+// 32x32 MFMA instructions, accumulating in fp32.  Both operands are K-contiguous per row, and A and B
+// fragments are read from LDS with the same (chunk, lane-group) -> k assignment, so the contraction is
+// independent of how the hardware numbers k inside a fragment.
 //
 // dgrad is the same kernel: src = grad_output and a panel packed with the mirrored, transposed
 // weight (fgx_pack_weight mode 1).
@@ -27,9 +35,24 @@ using f32x4 = float __attribute__((ext_vector_type(4)));
 using f32x16 = float __attribute__((ext_vector_type(16)));
 using u32x4 = uint32_t __attribute__((ext_vector_type(4)));
 
-constexpr int kSlabBytes = 128;   // bytes of K per row and step
-constexpr int kChunks = 8;        // 16-byte chunks per slab row
+constexpr int kSlabBytes = 64;    // bytes of K per row and step
+constexpr int kChunks = 4;        // 16-byte chunks per slab row
 constexpr int kXcds = 8;
+constexpr int kStages = 4;        // LDS ring depth
+
+// 16 zero bytes every lane may read: missing neighbors, K tails, dummy loads past the last step
+__device__ __attribute__((aligned(256))) unsigned char g_zero_block[256];
+
+#define FGX_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define FGX_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+
+// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding: vmcnt = imm[3:0] | imm[15:14] << 4,
+// expcnt = imm[6:4], lgkmcnt = imm[11:8]; all-ones = unconstrained)
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
 
 struct F16 { using type = _Float16; };
 struct BF16 { using type = __bf16; };
@@ -67,7 +90,11 @@ template <> __device__ __forceinline__ float to_float<__bf16>(__bf16 x) {
     return __builtin_bit_cast(float, (uint32_t)__builtin_bit_cast(uint16_t, x) << 16);
 }
 
-__device__ __forceinline__ int swz(int row, int chunk) { return row * kSlabBytes + ((chunk ^ (row & 7)) << 4); }
+// Physical position of logical chunk `chunk` of slab row `row`.  With 64-byte rows two rows share a 128-byte
+// bank line; the XOR key makes any 8 (and any 16) consecutive rows reading the same logical chunk hit
+// distinct 16-byte bank groups.
+__device__ __forceinline__ int swz_key(int row) { return ((row >> 1) + (row >> 3)) & 3; }
+__device__ __forceinline__ int swz(int row, int chunk) { return row * kSlabBytes + ((chunk ^ swz_key(row)) << 4); }
 
 // ------------------------------------------------------------------------------------------------
 // Weight panels
@@ -103,16 +130,21 @@ __global__ void __launch_bounds__(256) pack_weight_kernel(const T* __restrict__ 
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N>
 struct GemmCfg {
     using T = typename Tag::type;
-    static constexpr int NT = 64 * WAVES_M * WAVES_N;
+    static constexpr int NW = WAVES_M * WAVES_N;
+    static constexpr int NT = 64 * NW;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     static constexpr int TM = WM / 32, TN = WN / 32;
     static constexpr int SK = kSlabBytes / (int)sizeof(T);
-    static constexpr int A_CHUNKS = BM * kChunks, B_CHUNKS = BN * kChunks;
-    static constexpr int A_PER = (A_CHUNKS + NT - 1) / NT, B_PER = (B_CHUNKS + NT - 1) / NT;
+    static constexpr int ROWS_PER_INST = 64 / kChunks;              // slab rows one wave-wide load covers
+    static constexpr int A_INST = BM / ROWS_PER_INST, B_INST = BN / ROWS_PER_INST;
+    static constexpr int A_PER = (A_INST + NW - 1) / NW, B_PER = (B_INST + NW - 1) / NW;  // loads per wavefront and step
+    static constexpr int LPS = A_PER + B_PER;
+    static constexpr int STAGE_BYTES = (BM + BN) * kSlabBytes;
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
-    static_assert(A_CHUNKS % NT == 0 && B_CHUNKS % NT == 0, "tile must split evenly over the workgroup");
+    static_assert(BM % ROWS_PER_INST == 0 && BN % ROWS_PER_INST == 0, "tile must be whole wave-wide loads");
+    static_assert((kStages - 2) * LPS < 64, "outstanding loads exceed the vmcnt range");
     static constexpr size_t lds_bytes(int V) {
-        return (size_t)2 * (BM + BN) * kSlabBytes + (size_t)BM * V * 4 + (size_t)BM * 4 + 32 * 4;
+        return (size_t)kStages * STAGE_BYTES + 1024 + (size_t)BM * V * 4 + (size_t)BM * 4 + 32 * 4;
     }
 };
 
@@ -126,9 +158,10 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
     using C = GemmCfg<Tag, BM, BN, WAVES_M, WAVES_N>;
     using T = typename Tag::type;
     constexpr int NT = C::NT;
+    constexpr int S = kStages;
 
     // XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs, so give each XCD a
-    // contiguous run of tiles (neighbouring tiles gather overlapping rows -> same L2).
+    // contiguous run of tiles (all column tiles of a row tile share their gathered rows -> same L2).
     const unsigned total_tiles = row_tiles * col_tiles;
     const unsigned per_xcd = (total_tiles + kXcds - 1) / kXcds;
     const unsigned logical = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
@@ -138,11 +171,11 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
     const int kid = blockIdx.y;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-    unsigned char* a_lds = lds_raw;                                   // [2][BM * 128]
-    unsigned char* b_lds = a_lds + 2 * BM * kSlabBytes;               // [2][BN * 128]
-    uint32_t* nbr_lds = (uint32_t*)(b_lds + 2 * BN * kSlabBytes);     // [V][BM]
-    uint32_t* row_lds = nbr_lds + (size_t)BM * V;                     // [BM] output row or EMPTY
-    int* v_lds = (int*)(row_lds + BM);                                // [32] offsets present in this tile
+    unsigned char* ring = lds_raw;                                        // [S][A: BM x 64 | B: BN x 64]
+    unsigned char* dump = ring + S * C::STAGE_BYTES;                      // 1 KiB sink of surplus loads
+    uint32_t* nbr_lds = (uint32_t*)(dump + 1024);                         // [V][BM]
+    uint32_t* row_lds = nbr_lds + (size_t)BM * V;                         // [BM] output row or EMPTY
+    int* v_lds = (int*)(row_lds + BM);                                    // [32] offsets present in this tile
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -176,7 +209,7 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
         if (row != FGX_EMPTY32 && ((code >> v) & 1u)) m = map[(size_t)row * V + v];
         nbr_lds[v * BM + r] = m;
     }
-    __syncthreads();
+    __syncthreads();   // also drains every outstanding vector-memory load: the counter starts at zero below
 
     f32x16 acc[C::TM][C::TN];
 #pragma unroll
@@ -186,74 +219,141 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    u32x4 a_reg[C::A_PER], b_reg[C::B_PER];
     const size_t row_bytes = (size_t)K * sizeof(T);
     const unsigned char* src_b = (const unsigned char*)src;
     const unsigned char* panel_b = (const unsigned char*)panel;
+    const unsigned char* zero_b = g_zero_block;
+    const int sub_row = lane / kChunks, pch = lane % kChunks;
+    const bool ragged = (row_bytes % kSlabBytes) != 0;   // last slab of a row is partly past the row end
 
-    auto load_step = [&](int step) {
-        const int v = v_lds[step / slabs];
-        const int slab = step - (step / slabs) * slabs;
+    // ---- issue stream: runs S-1 steps ahead of the multiply stream and keeps per-lane source pointers that
+    // advance by one slab per step; they are re-derived only when the offset changes ----
+    int a_row[C::A_PER], a_choff[C::A_PER], a_inc[C::A_PER], b_off[C::B_PER];
+    bool a_mine[C::A_PER], b_mine[C::B_PER];
+    const unsigned char* a_ptr[C::A_PER];
 #pragma unroll
-        for (int i = 0; i < C::A_PER; ++i) {
-            int c = tid + i * NT;
-            int row = c >> 3, ch = c & 7;
-            uint32_t m = nbr_lds[v * BM + row];
-            int kbyte = slab * kSlabBytes + ch * 16;
-            u32x4 val = {0u, 0u, 0u, 0u};
-            if (m != FGX_EMPTY32 && (size_t)kbyte < row_bytes) val = *(const u32x4*)(src_b + (size_t)m * row_bytes + kbyte);
-            a_reg[i] = val;
-        }
-        const unsigned char* pb = panel_b + (((size_t)v * slabs + slab) * cols_pad + (size_t)col_tile * BN) * kSlabBytes;
-#pragma unroll
-        for (int i = 0; i < C::B_PER; ++i) {
-            int c = tid + i * NT;
-            b_reg[i] = *(const u32x4*)(pb + (size_t)c * 16);
-        }
-    };
-    auto store_step = [&](int buf) {
-        unsigned char* a_dst = a_lds + buf * BM * kSlabBytes;
-        unsigned char* b_dst = b_lds + buf * BN * kSlabBytes;
-#pragma unroll
-        for (int i = 0; i < C::A_PER; ++i) {
-            int c = tid + i * NT;
-            *(u32x4*)(a_dst + swz(c >> 3, c & 7)) = a_reg[i];
-        }
-#pragma unroll
-        for (int i = 0; i < C::B_PER; ++i) {
-            int c = tid + i * NT;
-            *(u32x4*)(b_dst + swz(c >> 3, c & 7)) = b_reg[i];
-        }
-    };
-
-    if (step_lo < step_hi) {
-        load_step(step_lo);
-        store_step(0);
+    for (int i = 0; i < C::A_PER; ++i) {
+        const int inst = i * C::NW + wave;
+        a_mine[i] = C::A_INST % C::NW == 0 || inst < C::A_INST;          // wave-uniform
+        a_row[i] = (a_mine[i] ? inst : 0) * C::ROWS_PER_INST + sub_row;
+        a_choff[i] = (pch ^ swz_key(a_row[i])) << 4;
+        a_ptr[i] = zero_b;
+        a_inc[i] = 0;
     }
-    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < C::B_PER; ++i) {
+        const int inst = i * C::NW + wave;
+        b_mine[i] = C::B_INST % C::NW == 0 || inst < C::B_INST;          // wave-uniform
+        const int col = (b_mine[i] ? inst : 0) * C::ROWS_PER_INST + sub_row;
+        b_off[i] = col * kSlabBytes + ((pch ^ swz_key(col)) << 4);
+    }
+    const size_t b_slab_stride = (size_t)cols_pad * kSlabBytes;
+    const unsigned char* b_ptr = zero_b;   // panel slice of the issue stream's (offset, slab), column tile applied
+    size_t b_inc = 0;
+    int is_step = step_lo;                 // next step to enqueue
+    int is_vi = slabs > 0 ? step_lo / slabs : 0;
+    int is_slab = step_lo - is_vi * slabs;
+    bool is_fresh = true;                  // pointers must be (re)derived before the next enqueue
+
+    auto issue = [&]() {
+        unsigned char* stage = ring + ((is_step - step_lo) % S) * C::STAGE_BYTES;
+        if (is_fresh) {                    // wave-uniform: first call, offset change, or running off the end
+            const bool live = is_step < step_hi;
+            const int v = v_lds[live ? is_vi : 0];
+#pragma unroll
+            for (int i = 0; i < C::A_PER; ++i) {
+                const uint32_t m = nbr_lds[v * BM + a_row[i]];
+                const bool real = live && a_mine[i] && m != FGX_EMPTY32;
+                const size_t off = real ? (size_t)m * row_bytes + (size_t)(is_slab * kSlabBytes + a_choff[i]) : (size_t)0;
+                a_ptr[i] = real ? src_b + off : zero_b;
+                a_inc[i] = real ? kSlabBytes : 0;
+            }
+            b_ptr = live ? panel_b + (((size_t)v * slabs + is_slab) * cols_pad + (size_t)col_tile * BN) * kSlabBytes : zero_b;
+            b_inc = live ? b_slab_stride : 0;
+            is_fresh = false;
+        }
+        const bool tail = ragged && is_slab == slabs - 1;   // wave-uniform
+#pragma unroll
+        for (int i = 0; i < C::A_PER; ++i) {
+            const unsigned char* p = a_ptr[i];
+            if (tail) p = (size_t)(is_slab * kSlabBytes + a_choff[i]) < row_bytes ? p : zero_b;
+            unsigned char* dst = a_mine[i] ? stage + (i * C::NW + wave) * 1024 : dump;
+#ifndef FGX_DBG_NO_LOAD
+            __builtin_amdgcn_global_load_lds(FGX_GLOBAL_PTR(p), FGX_LDS_PTR(dst), 16, 0, 0);
+#else
+            asm volatile("" :: "v"(p), "v"(dst));
+#endif
+            a_ptr[i] += a_inc[i];
+        }
+#pragma unroll
+        for (int i = 0; i < C::B_PER; ++i) {
+            const unsigned char* p = (b_inc != 0 && b_mine[i]) ? b_ptr + b_off[i] : zero_b;
+            unsigned char* dst = b_mine[i] ? stage + BM * kSlabBytes + (i * C::NW + wave) * 1024 : dump;
+#ifndef FGX_DBG_NO_LOAD
+            __builtin_amdgcn_global_load_lds(FGX_GLOBAL_PTR(p), FGX_LDS_PTR(dst), 16, 0, 0);
+#else
+            asm volatile("" :: "v"(p), "v"(dst));
+#endif
+        }
+        b_ptr += b_inc;
+        ++is_step;
+        if (++is_slab == slabs) {
+            is_slab = 0;
+            ++is_vi;
+            is_fresh = true;
+        }
+        if (is_step == step_hi) is_fresh = true;
+    };
+
+#pragma unroll
+    for (int s = 0; s < S - 1; ++s) issue();
+
     const int g = lane >> 5;        // lane group inside the MFMA fragment
     const int l32 = lane & 31;
+    int a_frag[kChunks / 2][C::TM], b_frag[kChunks / 2][C::TN];   // byte offsets of this lane's fragments in a stage
+#pragma unroll
+    for (int kk = 0; kk < kChunks / 2; ++kk) {
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i) a_frag[kk][i] = swz(wave_m * C::WM + i * 32 + l32, kk * 2 + g);
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) b_frag[kk][j] = BM * kSlabBytes + swz(wave_n * C::WN + j * 32 + l32, kk * 2 + g);
+    }
     for (int step = step_lo; step < step_hi; ++step) {
-        const int buf = (step - step_lo) & 1;
-        if (step + 1 < step_hi) load_step(step + 1);
-        const unsigned char* a_cur = a_lds + buf * BM * kSlabBytes;
-        const unsigned char* b_cur = b_lds + buf * BN * kSlabBytes;
+        // step's own loads are the oldest (S-1) * LPS still counted; everything older has been waited for
+        wait_vmcnt<(S - 2) * C::LPS>();
+        asm volatile("" ::: "memory");
+#ifndef FGX_DBG_NO_BARRIER
+        __builtin_amdgcn_s_barrier();      // all lanes' loads of `step` landed; stage (step-1) % S is free again
+#endif
+        asm volatile("" ::: "memory");
+#ifndef FGX_DBG_NO_ISSUE
+        issue();
+#endif
+#ifndef FGX_DBG_NO_MMA
+        const unsigned char* cur = ring + ((step - step_lo) % S) * C::STAGE_BYTES;
+        u32x4 af[kChunks / 2][C::TM], bf[kChunks / 2][C::TN];
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-            const int chunk = kk * 2 + g;
-            u32x4 af[C::TM], bf[C::TN];
+        for (int kk = 0; kk < kChunks / 2; ++kk) {
 #pragma unroll
-            for (int i = 0; i < C::TM; ++i) af[i] = *(const u32x4*)(a_cur + swz(wave_m * C::WM + i * 32 + l32, chunk));
+#ifndef FGX_DBG_NO_LDSREAD
+            for (int i = 0; i < C::TM; ++i) af[kk][i] = *(const u32x4*)(cur + a_frag[kk][i]);
 #pragma unroll
-            for (int j = 0; j < C::TN; ++j) bf[j] = *(const u32x4*)(b_cur + swz(wave_n * C::WN + j * 32 + l32, chunk));
+            for (int j = 0; j < C::TN; ++j) bf[kk][j] = *(const u32x4*)(cur + b_frag[kk][j]);
+#else
+            for (int i = 0; i < C::TM; ++i) { u32x4 t = {(uint32_t)step, (uint32_t)kk, (uint32_t)i, (uint32_t)(size_t)cur}; af[kk][i] = t; }
+#pragma unroll
+            for (int j = 0; j < C::TN; ++j) { u32x4 t = {(uint32_t)step, (uint32_t)kk, (uint32_t)j, 1u}; bf[kk][j] = t; }
+#endif
+        }
+#pragma unroll
+        for (int kk = 0; kk < kChunks / 2; ++kk)
 #pragma unroll
             for (int i = 0; i < C::TM; ++i)
 #pragma unroll
-                for (int j = 0; j < C::TN; ++j) mma<Tag>(acc[i][j], af[i], bf[j]);
-        }
-        if (step + 1 < step_hi) store_step(buf ^ 1);
-        __syncthreads();
+                for (int j = 0; j < C::TN; ++j) mma<Tag>(acc[i][j], af[kk][i], bf[kk][j]);
+#endif
     }
+    wait_vmcnt<0>();   // the trailing dummy loads
 
     // ---- epilogue: 32x32 accumulator tile, element e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32 ----
 #pragma unroll
@@ -288,27 +388,68 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restr
     }
 }
 
-// Column sums with fp32 accumulation: stage 1 sums a slice of rows per block, stage 2 adds the slices.
-constexpr int kColsumRows = 1024;
-template <typename T>
+// Column sums with fp32 accumulation.  Stage 1: kColsumSlices blocks each sum a contiguous slice of rows with
+// 16-byte loads (a thread owns VEC adjacent columns, the block's row lanes are added through LDS); stage 2 adds
+// the slices in a fixed order, so the result is deterministic.
+constexpr int kColsumSlices = 1024;
+template <typename T, int VEC>
 __global__ void __launch_bounds__(256) colsum_partial_kernel(const T* __restrict__ x, size_t n, int cols,
                                                              float* __restrict__ partial) {
-    const size_t r0 = (size_t)blockIdx.x * kColsumRows;
-    const size_t r1 = r0 + kColsumRows < n ? r0 + kColsumRows : n;
-    for (int c = threadIdx.x; c < cols; c += 256) {
-        float s = 0.f;
-        for (size_t r = r0; r < r1; ++r) s += to_float<T>(x[r * cols + c]);
-        partial[(size_t)blockIdx.x * cols + c] = s;
+    __shared__ float red[256 * VEC];
+    const int groups = (cols + VEC - 1) / VEC;
+    const int tpr = groups < 256 ? groups : 256;    // threads across one row
+    const int lanes = 256 / tpr;                    // row lanes of the block
+    const int cg0 = threadIdx.x % tpr, rl = threadIdx.x / tpr;
+    const size_t per = (n + gridDim.x - 1) / gridDim.x;
+    const size_t r0 = (size_t)blockIdx.x * per;
+    const size_t r1 = r0 + per < n ? r0 + per : n;
+    for (int cg = cg0; cg < groups; cg += tpr) {
+        float acc[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+        if (rl < lanes) {
+            for (size_t r = r0 + rl; r < r1; r += lanes) {
+                const T* src = x + r * cols + (size_t)cg * VEC;
+                if constexpr (VEC == 1) {
+                    acc[0] += to_float<T>(src[0]);
+                } else {
+                    u32x4 raw = *(const u32x4*)src;
+                    const T* v = (const T*)&raw;
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) acc[e] += to_float<T>(v[e]);
+                }
+            }
+        }
+        if (lanes > 1) {   // uniform over the block: groups <= 128, a single pass of the cg loop
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) red[threadIdx.x * VEC + e] = acc[e];
+            __syncthreads();
+            if (rl == 0) {
+                for (int l = 1; l < lanes; ++l)
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) acc[e] += red[(l * tpr + cg0) * VEC + e];
+            }
+        }
+        if (rl == 0) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+                if (cg * VEC + e < cols) partial[(size_t)blockIdx.x * cols + cg * VEC + e] = acc[e];
+        }
     }
 }
+// 64 columns per block, 4 threads per column each adding a quarter of the slices
 template <typename T>
 __global__ void __launch_bounds__(256) colsum_final_kernel(const float* __restrict__ partial, unsigned slices, int cols,
                                                            T* __restrict__ out) {
-    int c = blockIdx.x * 256 + threadIdx.x;
-    if (c >= cols) return;
+    __shared__ float red[256];
+    const int c = blockIdx.x * 64 + (threadIdx.x & 63);
+    const int part = threadIdx.x >> 6;
     float s = 0.f;
-    for (unsigned b = 0; b < slices; ++b) s += partial[(size_t)b * cols + c];
-    out[c] = from_float<T>(s);
+    if (c < cols)
+        for (unsigned b = part; b < slices; b += 4) s += partial[(size_t)b * cols + c];
+    red[threadIdx.x] = s;
+    __syncthreads();
+    if (part == 0 && c < cols) out[c] = from_float<T>(red[threadIdx.x] + red[threadIdx.x + 64] + red[threadIdx.x + 128] + red[threadIdx.x + 192]);
 }
 
 int elem_size(int dtype) { return dtype == FGX_F32 ? 4 : 2; }
@@ -429,7 +570,8 @@ int fgx_conv_gather_gemm(int dtype, const void* src, const void* panel, const vo
 }
 
 size_t fgx_colsum_scratch_bytes(size_t n, int cols) {
-    return (size_t)cdiv(n ? n : 1, kColsumRows) * (size_t)(cols > 0 ? cols : 1) * sizeof(float);
+    (void)n;
+    return (size_t)kColsumSlices * (size_t)(cols > 0 ? cols : 1) * sizeof(float);
 }
 
 int fgx_colsum(int dtype, const void* x, size_t n, int cols, void* scratch, void* out, fgx_stream_t stream) {
@@ -437,16 +579,19 @@ int fgx_colsum(int dtype, const void* x, size_t n, int cols, void* scratch, void
     FGX_CHECK_ARG(cols > 0 && out != nullptr, "fgx_colsum: bad shape or null output");
     FGX_CHECK_ARG(scratch != nullptr && (n == 0 || x != nullptr), "fgx_colsum: null buffer");
     hipStream_t s = (hipStream_t)stream;
-    const unsigned slices = n ? cdiv(n, kColsumRows) : 0u;
-    const unsigned gfin = cdiv(cols, 256);
-#define FGX_COLSUM(T)                                                                                     \
-    do {                                                                                                  \
-        if (slices) colsum_partial_kernel<T><<<slices, 256, 0, s>>>((const T*)x, n, cols, (float*)scratch); \
-        colsum_final_kernel<T><<<gfin, 256, 0, s>>>((const float*)scratch, slices, cols, (T*)out);        \
+    unsigned slices = n ? (unsigned)((n + 255) / 256) : 0u;     // at least 256 rows per slice
+    if (slices > (unsigned)kColsumSlices) slices = kColsumSlices;
+    const unsigned gfin = cdiv(cols, 64);
+    const int es = elem_size(dtype);
+    const bool vec = ((size_t)cols * es) % 16 == 0 && ((uintptr_t)x & 15) == 0;
+#define FGX_COLSUM(T, VEC)                                                                                        \
+    do {                                                                                                          \
+        if (slices) colsum_partial_kernel<T, VEC><<<slices, 256, 0, s>>>((const T*)x, n, cols, (float*)scratch);   \
+        colsum_final_kernel<T><<<gfin, 256, 0, s>>>((const float*)scratch, slices, cols, (T*)out);                \
     } while (0)
-    if (dtype == FGX_F16) FGX_COLSUM(_Float16);
-    else if (dtype == FGX_BF16) FGX_COLSUM(__bf16);
-    else FGX_COLSUM(float);
+    if (dtype == FGX_F16) { if (vec) FGX_COLSUM(_Float16, 8); else FGX_COLSUM(_Float16, 1); }
+    else if (dtype == FGX_BF16) { if (vec) FGX_COLSUM(__bf16, 8); else FGX_COLSUM(__bf16, 1); }
+    else { if (vec) FGX_COLSUM(float, 4); else FGX_COLSUM(float, 1); }
 #undef FGX_COLSUM
     FGX_CHECK_LAUNCH("fgx_colsum");
     return FGX_OK;

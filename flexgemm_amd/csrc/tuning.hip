@@ -19,7 +19,7 @@ struct Entry {
 
 // Measured entries (MI355X).  Rows are matched exactly on (pass, element size, floor(log2 N), Ci, Co).
 const Entry kTable[] = {
-    // pass dtype log2n  Ci    Co    {rows, cols, splitk, chunk_pairs}
+    // pass dtype log2n  Ci    Co    {rows, cols, splitk, block_rows}
     {0, 2, 19, 128, 128, {128, 128, 1, 0}},
     {1, 2, 19, 128, 128, {128, 128, 1, 0}},
     {2, 2, 19, 128, 128, {128, 128, 1, 4096}},
@@ -28,10 +28,10 @@ const Entry kTable[] = {
     {2, 2, 17, 256, 256, {128, 128, 1, 4096}},
     {0, 2, 21, 32, 32, {128, 32, 1, 0}},
     {1, 2, 21, 32, 32, {128, 32, 1, 0}},
-    {2, 2, 21, 32, 32, {32, 32, 1, 16384}},
+    {2, 2, 21, 32, 32, {32, 32, 1, 4096}},
     {0, 2, 15, 1024, 1024, {128, 128, 1, 0}},
     {1, 2, 15, 1024, 1024, {128, 128, 1, 0}},
-    {2, 2, 15, 1024, 1024, {128, 128, 1, 16384}},
+    {2, 2, 15, 1024, 1024, {128, 128, 1, 65536}},
 };
 
 int floor_log2(size_t n) {
@@ -46,19 +46,19 @@ size_t round_up(size_t x, size_t m) { return (x + m - 1) / m * m; }
 
 void rule(int pass_kind, size_t n, int Ci, int Co, int V, fgx_schedule* out) {
     if (pass_kind == 2) {
-        // wgrad: square tiles over (Co, Ci); chunk the pair lists so that about 8 workgroups per CU exist.
+        // wgrad: square tiles over (Co, Ci); voxel blocks of at least 4096 rows, enlarged until the fp32 partial
+        // products (blocks x V x Co x Ci) stay below 256 MiB.
         int t = pick_cols(Ci < Co ? Ci : Co);
         out->tile_rows = t;
         out->tile_cols = t;
         out->splitk = 1;
-        size_t tiles = (size_t)cdiv(Co, t) * cdiv(Ci, t);
-        size_t pairs = n * (size_t)(V > 2 ? (V * 2) / 5 : 1);   // about 40 % of the offsets are present on surfaces
-        size_t want_chunks = (size_t)kCUs * 8 / (tiles ? tiles : 1);
-        if (want_chunks < (size_t)V) want_chunks = V;
-        size_t cp = round_up(pairs / want_chunks + 1, 64);
-        if (cp < 256) cp = 256;
-        if (cp > 65536) cp = 65536;
-        out->chunk_pairs = (int)cp;
+        const double per_block = 4.0 * V * (double)Co * (double)Ci;
+        size_t max_blocks = (size_t)(268435456.0 / per_block);
+        if (max_blocks < 1) max_blocks = 1;
+        size_t rows = round_up((n + max_blocks - 1) / max_blocks, 1024);
+        if (rows < 4096) rows = 4096;
+        if (rows > 0x40000000) rows = 0x40000000;
+        out->block_rows = (int)rows;
         return;
     }
     const int cols = pass_kind == 0 ? Co : Ci;
@@ -66,7 +66,7 @@ void rule(int pass_kind, size_t n, int Ci, int Co, int V, fgx_schedule* out) {
     out->tile_rows = n >= 4096 ? 128 : (n >= 1024 ? 64 : 32);
     if (out->tile_rows == 64 && out->tile_cols == 128) out->tile_rows = 128;
     if (out->tile_rows == 32 && out->tile_cols != 32) out->tile_rows = out->tile_cols == 64 ? 64 : 128;
-    out->chunk_pairs = 0;
+    out->block_rows = 0;
     // split K only when the tiles cannot fill the chip (reference: candidates start at #SM / blocks)
     size_t tiles = (size_t)cdiv(n, out->tile_rows) * cdiv(cols, out->tile_cols);
     int s = 1;

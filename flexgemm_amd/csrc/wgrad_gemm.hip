@@ -3,14 +3,29 @@
 //   grad_weight[co, v, ci] = sum over pairs k of offset v of grad_out[sig_o[k], co] * feats[sig_i[k], ci]
 //
 // The contraction runs over pairs, i.e. over ROWS of both operands, while MFMA fragments want the
-// contraction index contiguous inside a lane.  Rows are therefore staged in LDS pair-major exactly as
-// they arrive from memory (coalesced 16-byte stores) and the fragments are assembled with 16/32-bit
-// LDS reads down a column ("transpose on read").
+// contraction index contiguous inside a lane.  Rows are staged in LDS pair-major, exactly as they sit in
+// memory; 16-bit fragments are then read with the gfx950 transposing LDS load (ds_read_b64_tr_b16: a
+// 16-lane group reads a 4-pair x 16-channel block and each lane receives the 4 pair values of its own
+// channel), fp32 fragments with plain 32-bit reads.
 //
-// Work decomposition: every offset's pair segment is cut into chunks of `chunk_pairs` pairs; one
-// workgroup computes one (chunk, Co-tile, Ci-tile) partial product in fp32 and writes it to scratch;
-// a second kernel adds an offset's chunks in a fixed order (deterministic) and casts to the output type.
-// Equal-sized chunks balance the very unequal segment lengths (the centre offset has N pairs).
+// Pipeline.  Both operands are gathers, and each gather depends on an index (sig_o / sig_i) that has to
+// be fetched first.  Everything moves with direct global->LDS loads (lane i of a wavefront deposits its
+// data at LDS base + size * i) through two rings: an index ring (32 + 32 indices per step) that runs
+// 2 (S-1) steps ahead, and a row ring of S stages (32 pair rows of each operand) that runs S-1 steps ahead
+// and takes its addresses from the index ring.  These loads are the only vector-memory operations in the
+// main loop and every wavefront issues the same number per step (dummy loads past the end), so
+// s_waitcnt vmcnt((S-2) * loads_per_step) means "this step's rows and the indices needed for the next
+// enqueue have landed"; one workgroup barrier per step publishes them.
+//
+// Work decomposition and locality.  Inside one offset's segment the pairs are ordered by output row,
+// and the matching input rows are that row's neighbors, so the pairs of ALL offsets that belong to one
+// block of `block_rows` consecutive voxels touch the same few megabytes of grad_out / feats.  A work item
+// is therefore (voxel block b, offset v, Co-tile, Ci-tile); the items of one voxel block are dispatched
+// back to back onto the SAME XCD (workgroup ids are dealt round-robin over the 8 XCDs), so that the rows
+// are fetched from HBM once and then served by that XCD's L2 to the other offsets.  Each item writes an
+// fp32 partial product; a second kernel adds an offset's partials in block order (deterministic) and
+// casts to the output type.  The per-(offset, block) pair ranges are found by a small binary-search
+// kernel over sig_o.
 #include "fgx_common.h"
 
 namespace fgx {
@@ -20,11 +35,12 @@ using f16x8 = _Float16 __attribute__((ext_vector_type(8)));
 using bf16x8 = __bf16 __attribute__((ext_vector_type(8)));
 using f32x16 = float __attribute__((ext_vector_type(16)));
 using u32x4 = uint32_t __attribute__((ext_vector_type(4)));
-using u16x8 = uint16_t __attribute__((ext_vector_type(8)));
+using i16x4 = short __attribute__((ext_vector_type(4)));
+using i16x8 = short __attribute__((ext_vector_type(8)));
 
-struct F16 { using type = _Float16; using bits = uint16_t; };
-struct BF16 { using type = __bf16; using bits = uint16_t; };
-struct F32 { using type = float; using bits = uint32_t; };
+struct F16 { using type = _Float16; };
+struct BF16 { using type = __bf16; };
+struct F32 { using type = float; };
 
 template <typename T> __device__ __forceinline__ T from_float(float x);
 template <> __device__ __forceinline__ _Float16 from_float<_Float16>(float x) { return (_Float16)x; }
@@ -38,71 +54,122 @@ template <> __device__ __forceinline__ __bf16 from_float<__bf16>(float x) {
 }
 
 constexpr int kMaxV = 32;
+constexpr int kXcds = 8;
+constexpr int kStages = 4;      // row ring depth
+constexpr int kIdxSlots = 8;    // index ring depth (>= kStages, power of two)
 
-struct ChunkTable {
-    uint32_t seg[kMaxV + 1];          // pair offsets per kernel offset
-    uint32_t chunk_begin[kMaxV + 1];  // first chunk id of every offset
+// 16 zero bytes every lane may read: pairs past the end of an item, columns past the tensor width
+__device__ __attribute__((aligned(256))) unsigned char g_zero_block_w[256];
+
+#define FGX_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define FGX_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
+struct SegTable {
+    uint32_t seg[kMaxV + 1];   // pair offsets per kernel offset
 };
 
-// Pair-major staging: stage[p][c], p < PAIRS, c < W (tile width in elements), row pitch padded by
-// 16 bytes so that the lane groups of a column read hit different banks.
+// bounds[v * (nb + 1) + b] = first pair of offset v whose output row is >= b * block_rows
+__global__ void __launch_bounds__(256) block_bounds_kernel(const uint32_t* __restrict__ sig_o, SegTable tab, int V,
+                                                           unsigned nb, unsigned block_rows,
+                                                           uint32_t* __restrict__ bounds) {
+    const unsigned t = blockIdx.x * 256 + threadIdx.x;
+    if (t >= (unsigned)V * (nb + 1)) return;
+    const unsigned v = t / (nb + 1), b = t % (nb + 1);
+    uint32_t lo = tab.seg[v], hi = tab.seg[v + 1];
+    const uint64_t target = (uint64_t)b * block_rows;
+    while (lo < hi) {
+        uint32_t mid = lo + ((hi - lo) >> 1);
+        if ((uint64_t)sig_o[mid] < target) lo = mid + 1;
+        else hi = mid;
+    }
+    bounds[t] = lo;
+}
+
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N>
 struct WgradCfg {
     using T = typename Tag::type;
-    using B = typename Tag::bits;
     static constexpr int ES = (int)sizeof(T);
-    static constexpr int NT = 64 * WAVES_M * WAVES_N;
+    static constexpr int NW = WAVES_M * WAVES_N;
+    static constexpr int NT = 64 * NW;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     static constexpr int TM = WM / 32, TN = WN / 32;
-    static constexpr int KV = 16 / ES;              // elements per fragment vector (8 or 4)
-    static constexpr int PAIRS = 2 * KV * 2;        // pairs per step: 2 MFMA k-steps of 2 lane groups x KV
-    static constexpr int PITCH_A = BM * ES + 16, PITCH_B = BN * ES + 16;   // bytes
-    static constexpr int A_CHUNKS = PAIRS * BM * ES / 16, B_CHUNKS = PAIRS * BN * ES / 16;
-    static constexpr int A_PER = (A_CHUNKS + NT - 1) / NT, B_PER = (B_CHUNKS + NT - 1) / NT;
-    static constexpr size_t lds_bytes = (size_t)2 * PAIRS * (PITCH_A + PITCH_B) + 2 * PAIRS * 2 * 4;
+    static constexpr int PAIRS = 32;                                   // pairs per pipeline step
+    static constexpr int ROWB_A = BM * ES, ROWB_B = BN * ES;           // bytes of one staged pair row
+    static constexpr int CH_A = ROWB_A / 16, CH_B = ROWB_B / 16;       // 16-byte chunks per row
+    static constexpr int RPI_A = 64 / CH_A, RPI_B = 64 / CH_B;         // pair rows one wave-wide load covers
+    static constexpr int A_INST = PAIRS / RPI_A, B_INST = PAIRS / RPI_B;
+    static constexpr int A_PER = (A_INST + NW - 1) / NW, B_PER = (B_INST + NW - 1) / NW;
+    static constexpr int LPS = A_PER + B_PER + 1;                      // + one index load
+    static constexpr int A_BYTES = PAIRS * ROWB_A, B_BYTES = PAIRS * ROWB_B;
+    static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+    static constexpr int IDX_SLOT_BYTES = 64 * 4;                      // 32 sig_o + 32 sig_i
+    static constexpr size_t lds_bytes = (size_t)kStages * STAGE_BYTES + (size_t)kIdxSlots * IDX_SLOT_BYTES + 1024;
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
+    static_assert(CH_A <= 64 && CH_B <= 64 && 64 % CH_A == 0 && 64 % CH_B == 0, "row slice must divide a wave-wide load");
+    static_assert((kStages - 2) * LPS < 64, "outstanding loads exceed the vmcnt range");
+    // XOR key on the 16-byte chunk index: the transposing read touches 4 consecutive pair rows x 32 bytes, which
+    // must fall into distinct bank groups
+    static constexpr int key_a(int row) { return ES == 2 && CH_A >= 8 ? 2 * (row & 3) : 0; }
+    static constexpr int key_b(int row) { return ES == 2 && CH_B >= 8 ? 2 * (row & 3) : 0; }
 };
 
-template <typename Tag> struct Frag;
-template <> struct Frag<F16> {
-    static __device__ __forceinline__ void mma(f32x16& acc, const u16x8& a, const u16x8& b) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), acc, 0, 0, 0);
-    }
-};
-template <> struct Frag<BF16> {
-    static __device__ __forceinline__ void mma(f32x16& acc, const u16x8& a, const u16x8& b) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
-    }
-};
+__device__ __forceinline__ i16x4 lds_read_tr16(const unsigned char* p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((i16x4 __attribute__((address_space(3)))*)p);
+}
+
+template <typename Tag> __device__ __forceinline__ void mma16(f32x16& acc, const i16x8& a, const i16x8& b);
+template <> __device__ __forceinline__ void mma16<F16>(f32x16& acc, const i16x8& a, const i16x8& b) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), acc, 0, 0, 0);
+}
+template <> __device__ __forceinline__ void mma16<BF16>(f32x16& acc, const i16x8& a, const i16x8& b) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
+}
+template <> __device__ __forceinline__ void mma16<F32>(f32x16&, const i16x8&, const i16x8&) {}
 
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N>
 __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N)
 wgrad_kernel(const typename Tag::type* __restrict__ gout, const typename Tag::type* __restrict__ feats,
-             const uint32_t* __restrict__ sig_i, const uint32_t* __restrict__ sig_o, ChunkTable tab, int V, int Ci,
-             int Co, int chunk_pairs, unsigned co_tiles, unsigned ci_tiles, float* __restrict__ partial) {
+             const uint32_t* __restrict__ sig_i, const uint32_t* __restrict__ sig_o,
+             const uint32_t* __restrict__ bounds, int V, int Ci, int Co, unsigned nb, unsigned co_tiles,
+             unsigned ci_tiles, float* __restrict__ partial) {
     using C = WgradCfg<Tag, BM, BN, WAVES_M, WAVES_N>;
-    using Bits = typename Tag::bits;
-    constexpr int NT = C::NT;
     constexpr int ES = C::ES;
+    constexpr int S = kStages;
 
-    const unsigned chunk = blockIdx.y;
-    const unsigned co_tile = blockIdx.x % co_tiles;
-    const unsigned ci_tile = blockIdx.x / co_tiles;
-    int v = 0;
-    while (v + 1 < V && tab.chunk_begin[v + 1] <= chunk) ++v;
-    const uint32_t k_lo = tab.seg[v] + (chunk - tab.chunk_begin[v]) * (uint32_t)chunk_pairs;
-    const uint32_t seg_hi = tab.seg[v + 1];
-    const uint32_t k_hi = k_lo + (uint32_t)chunk_pairs < seg_hi ? k_lo + (uint32_t)chunk_pairs : seg_hi;
+    // XCD-aware item order: all (offset, tile) items of one voxel block run on one XCD, back to back.
+    const unsigned tiles = co_tiles * ci_tiles;
+    const unsigned per_block = (unsigned)V * tiles;
+    const unsigned xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
+    const unsigned b = (slot / per_block) * kXcds + xcd;
+    if (b >= nb) return;
+    const unsigned within = slot % per_block;
+    const unsigned v = within / tiles;
+    const unsigned tile = within % tiles;
+    const unsigned co_tile = tile % co_tiles, ci_tile = tile / co_tiles;
+    const uint32_t k_lo = bounds[v * (nb + 1) + b];
+    const uint32_t k_hi = bounds[v * (nb + 1) + b + 1];
+    if (k_lo >= k_hi) return;   // the reduction skips empty items
+    const int nsteps = (int)((k_hi - k_lo + C::PAIRS - 1) / C::PAIRS);
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-    unsigned char* a_lds = lds_raw;                                     // [2][PAIRS][PITCH_A]
-    unsigned char* b_lds = a_lds + 2 * C::PAIRS * C::PITCH_A;           // [2][PAIRS][PITCH_B]
-    uint32_t* idx_lds = (uint32_t*)(b_lds + 2 * C::PAIRS * C::PITCH_B); // [2][2][PAIRS]: (o, i) rows per buffer
+    unsigned char* ring = lds_raw;                                              // [S][A rows | B rows]
+    unsigned char* idx_ring = ring + S * C::STAGE_BYTES;                        // [kIdxSlots][o x 32 | i x 32]
+    unsigned char* dump = idx_ring + kIdxSlots * C::IDX_SLOT_BYTES;             // sink of surplus loads
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
     const int g = lane >> 5, l32 = lane & 31;
     const int m0 = (int)co_tile * BM, n0 = (int)ci_tile * BN;
+    const unsigned char* gout_b = (const unsigned char*)gout;
+    const unsigned char* feats_b = (const unsigned char*)feats;
+    const unsigned char* zero_b = g_zero_block_w;
+    const size_t rowb_o = (size_t)Co * ES, rowb_i = (size_t)Ci * ES;
 
     f32x16 acc[C::TM][C::TN];
 #pragma unroll
@@ -112,112 +179,129 @@ wgrad_kernel(const typename Tag::type* __restrict__ gout, const typename Tag::ty
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    u32x4 a_reg[C::A_PER], b_reg[C::B_PER];
-    const unsigned char* gout_b = (const unsigned char*)gout;
-    const unsigned char* feats_b = (const unsigned char*)feats;
-    constexpr int A_ROW_CHUNKS = BM * ES / 16, B_ROW_CHUNKS = BN * ES / 16;
-
-    // 16-byte chunk `c` of a tile row: columns [c*KV, c*KV+KV) of the tile; zero when the pair is past
-    // the chunk end or the columns are past the tensor width.
-    auto load_step = [&](uint32_t k0) {
+    // index slot of step j: lanes 0-31 fetch sig_o, lanes 32-63 sig_i of the step's 32 pairs and deposit them at
+    // slot + 4 * lane.  Every wavefront issues the same load (same data, same place) so that all of them count alike.
+    auto issue_idx = [&](int j) {
+        uint32_t k = k_lo + (uint32_t)j * C::PAIRS + (uint32_t)(lane & 31);
+        k = k < k_hi ? k : k_hi - 1;                       // past the end: any valid address, the row load ignores it
+        const uint32_t* src = (lane & 32) ? sig_i + k : sig_o + k;
+        unsigned char* dst = idx_ring + (j & (kIdxSlots - 1)) * C::IDX_SLOT_BYTES;
+        __builtin_amdgcn_global_load_lds(FGX_GLOBAL_PTR(src), FGX_LDS_PTR(dst), 4, 0, 0);
+    };
+    auto idx_of = [&](int j, int p, int which) -> uint32_t {   // which: 0 = sig_o, 1 = sig_i
+        const uint32_t* slot_p = (const uint32_t*)(idx_ring + (j & (kIdxSlots - 1)) * C::IDX_SLOT_BYTES);
+        return slot_p[which * 32 + p];
+    };
+    // rows of step j into stage j % S; exactly A_PER + B_PER loads per wavefront
+    auto issue_rows = [&](int j) {
+        unsigned char* stage = ring + (j & (S - 1)) * C::STAGE_BYTES;
+        const bool live = j < nsteps;
+        const uint32_t kbase = k_lo + (uint32_t)j * C::PAIRS;
 #pragma unroll
         for (int i = 0; i < C::A_PER; ++i) {
-            int c = tid + i * NT;
-            u32x4 val = {0u, 0u, 0u, 0u};
-            if (c < C::A_CHUNKS) {
-                int p = c / A_ROW_CHUNKS, ch = c % A_ROW_CHUNKS;
-                int col = m0 + ch * C::KV;
-                if (k0 + p < k_hi && col < Co) val = *(const u32x4*)(gout_b + ((size_t)sig_o[k0 + p] * Co + col) * ES);
-            }
-            a_reg[i] = val;
+            const int inst = i * C::NW + wave;
+            const bool mine = C::A_INST % C::NW == 0 || inst < C::A_INST;      // wave-uniform
+            const int row = (mine ? inst : 0) * C::RPI_A + lane / C::CH_A;
+            const int c = (lane % C::CH_A) ^ C::key_a(row);
+            const int col = m0 + c * (16 / ES);
+            const uint32_t o = idx_of(j, row, 0);
+            const bool real = live && mine && kbase + (uint32_t)row < k_hi && col < Co;
+            const size_t off = real ? (size_t)o * rowb_o + (size_t)col * ES : (size_t)0;
+            const unsigned char* p = real ? gout_b + off : zero_b;
+            unsigned char* dst = mine ? stage + inst * 1024 : dump;
+            __builtin_amdgcn_global_load_lds(FGX_GLOBAL_PTR(p), FGX_LDS_PTR(dst), 16, 0, 0);
         }
 #pragma unroll
         for (int i = 0; i < C::B_PER; ++i) {
-            int c = tid + i * NT;
-            u32x4 val = {0u, 0u, 0u, 0u};
-            if (c < C::B_CHUNKS) {
-                int p = c / B_ROW_CHUNKS, ch = c % B_ROW_CHUNKS;
-                int col = n0 + ch * C::KV;
-                if (k0 + p < k_hi && col < Ci) val = *(const u32x4*)(feats_b + ((size_t)sig_i[k0 + p] * Ci + col) * ES);
-            }
-            b_reg[i] = val;
+            const int inst = i * C::NW + wave;
+            const bool mine = C::B_INST % C::NW == 0 || inst < C::B_INST;      // wave-uniform
+            const int row = (mine ? inst : 0) * C::RPI_B + lane / C::CH_B;
+            const int c = (lane % C::CH_B) ^ C::key_b(row);
+            const int col = n0 + c * (16 / ES);
+            const uint32_t ii = idx_of(j, row, 1);
+            const bool real = live && mine && kbase + (uint32_t)row < k_hi && col < Ci;
+            const size_t off = real ? (size_t)ii * rowb_i + (size_t)col * ES : (size_t)0;
+            const unsigned char* p = real ? feats_b + off : zero_b;
+            unsigned char* dst = mine ? stage + C::A_BYTES + inst * 1024 : dump;
+            __builtin_amdgcn_global_load_lds(FGX_GLOBAL_PTR(p), FGX_LDS_PTR(dst), 16, 0, 0);
         }
     };
-    auto store_step = [&](int buf) {
-        unsigned char* a_dst = a_lds + buf * C::PAIRS * C::PITCH_A;
-        unsigned char* b_dst = b_lds + buf * C::PAIRS * C::PITCH_B;
-#pragma unroll
-        for (int i = 0; i < C::A_PER; ++i) {
-            int c = tid + i * NT;
-            if (c < C::A_CHUNKS) *(u32x4*)(a_dst + (c / A_ROW_CHUNKS) * C::PITCH_A + (c % A_ROW_CHUNKS) * 16) = a_reg[i];
-        }
-#pragma unroll
-        for (int i = 0; i < C::B_PER; ++i) {
-            int c = tid + i * NT;
-            if (c < C::B_CHUNKS) *(u32x4*)(b_dst + (c / B_ROW_CHUNKS) * C::PITCH_B + (c % B_ROW_CHUNKS) * 16) = b_reg[i];
-        }
-    };
-    (void)idx_lds;
 
-    if (k_lo < k_hi) {
-        load_step(k_lo);
-        store_step(0);
+    // ---- prologue: indices of the first S-1 steps, then S-1 enqueue rounds ----
+#pragma unroll
+    for (int j = 0; j < S - 1; ++j) issue_idx(j);
+    wait_vmcnt<0>();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int j = 0; j < S - 1; ++j) {
+        issue_rows(j);
+        issue_idx(j + S - 1);
     }
-    __syncthreads();
-    int it = 0;
-    for (uint32_t k0 = k_lo; k0 < k_hi; k0 += C::PAIRS, ++it) {
-        const int buf = it & 1;
-        const bool more = k0 + C::PAIRS < k_hi;
-        if (more) load_step(k0 + C::PAIRS);
-        const unsigned char* a_cur = a_lds + buf * C::PAIRS * C::PITCH_A;
-        const unsigned char* b_cur = b_lds + buf * C::PAIRS * C::PITCH_B;
+
+    // fragment addressing (constant per lane)
+    const int s16 = lane & 15, mb = (lane >> 4) & 1;
+    for (int k = 0; k < nsteps; ++k) {
+        wait_vmcnt<(S - 2) * C::LPS>();    // rows of step k and the indices of step k+S-1 have landed
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        issue_rows(k + S - 1);
+        issue_idx(k + 2 * (S - 1));
+        const unsigned char* a_cur = ring + (k & (S - 1)) * C::STAGE_BYTES;
+        const unsigned char* b_cur = a_cur + C::A_BYTES;
+        if constexpr (ES == 2) {
+            // Transposing read: in a 16-lane group, lane s supplies the address of 4 adjacent channels of pair
+            // row (s / 4) and receives the 4 pair values of channel (group base + s).  Lanes 0-15 / 16-31 cover
+            // fragment rows 0-15 / 16-31, the two wave halves take pair rows [0, 8) / [8, 16) of the k-step.
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-            // lane group g of k-step kk owns pairs [(kk*2+g)*KV, +KV)
-            const int p0 = (kk * 2 + g) * C::KV;
-            if constexpr (ES == 2) {
-                u16x8 af[C::TM], bf[C::TN];
+            for (int kk = 0; kk < C::PAIRS / 16; ++kk) {
+                const int prow = kk * 16 + g * 8 + (s16 >> 2);
+                i16x8 af[C::TM], bf[C::TN];
+#pragma unroll
+                for (int i = 0; i < C::TM; ++i) {
+                    const int byte = (wave_m * C::WM + i * 32 + mb * 16 + (s16 & 3) * 4) * 2;
+                    const int c = byte >> 4, w = byte & 15;
+                    i16x4 lo = lds_read_tr16(a_cur + prow * C::ROWB_A + ((c ^ C::key_a(prow)) << 4) + w);
+                    i16x4 hi = lds_read_tr16(a_cur + (prow + 4) * C::ROWB_A + ((c ^ C::key_a(prow + 4)) << 4) + w);
+                    af[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
+#pragma unroll
+                for (int j = 0; j < C::TN; ++j) {
+                    const int byte = (wave_n * C::WN + j * 32 + mb * 16 + (s16 & 3) * 4) * 2;
+                    const int c = byte >> 4, w = byte & 15;
+                    i16x4 lo = lds_read_tr16(b_cur + prow * C::ROWB_B + ((c ^ C::key_b(prow)) << 4) + w);
+                    i16x4 hi = lds_read_tr16(b_cur + (prow + 4) * C::ROWB_B + ((c ^ C::key_b(prow + 4)) << 4) + w);
+                    bf[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
 #pragma unroll
                 for (int i = 0; i < C::TM; ++i)
 #pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        af[i][e] = *(const Bits*)(a_cur + (p0 + e) * C::PITCH_A + (wave_m * C::WM + i * 32 + l32) * 2);
+                    for (int j = 0; j < C::TN; ++j) mma16<Tag>(acc[i][j], af[i], bf[j]);
+            }
+        } else {
+            // fp32: one value per lane and MFMA (32x32x2); lane group g takes the odd / even pair of each couple
 #pragma unroll
-                for (int j = 0; j < C::TN; ++j)
+            for (int kk = 0; kk < C::PAIRS / 2; ++kk) {
+                const int p = kk * 2 + g;
+                float af[C::TM], bf[C::TN];
 #pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        bf[j][e] = *(const Bits*)(b_cur + (p0 + e) * C::PITCH_B + (wave_n * C::WN + j * 32 + l32) * 2);
+                for (int i = 0; i < C::TM; ++i) af[i] = *(const float*)(a_cur + p * C::ROWB_A + (wave_m * C::WM + i * 32 + l32) * 4);
 #pragma unroll
-                for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < C::TN; ++j) Frag<Tag>::mma(acc[i][j], af[i], bf[j]);
-            } else {
-                float af[C::TM][4], bf[C::TN][4];
-#pragma unroll
-                for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        af[i][e] = *(const float*)(a_cur + (p0 + e) * C::PITCH_A + (wave_m * C::WM + i * 32 + l32) * 4);
-#pragma unroll
-                for (int j = 0; j < C::TN; ++j)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        bf[j][e] = *(const float*)(b_cur + (p0 + e) * C::PITCH_B + (wave_n * C::WN + j * 32 + l32) * 4);
+                for (int j = 0; j < C::TN; ++j) bf[j] = *(const float*)(b_cur + p * C::ROWB_B + (wave_n * C::WN + j * 32 + l32) * 4);
 #pragma unroll
                 for (int i = 0; i < C::TM; ++i)
 #pragma unroll
                     for (int j = 0; j < C::TN; ++j)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][e], bf[j][e], acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
             }
         }
-        if (more) store_step(buf ^ 1);
-        __syncthreads();
     }
+    wait_vmcnt<0>();   // the trailing dummy loads
 
-    // partial[chunk][co][ci], fp32
-    float* dst = partial + (size_t)chunk * Co * Ci;
+    // partial[b][v][co][ci], fp32
+    float* dst = partial + ((size_t)b * V + v) * ((size_t)Co * Ci);
 #pragma unroll
     for (int j = 0; j < C::TN; ++j) {
         const int ci = n0 + wave_n * C::WN + j * 32 + l32;
@@ -232,10 +316,11 @@ wgrad_kernel(const typename Tag::type* __restrict__ gout, const typename Tag::ty
     }
 }
 
-// grad_weight[co][v][ci] = sum over the chunks of offset v, in chunk order
+// grad_weight[co][v][ci] = sum over voxel blocks with pairs for offset v, in block order
 template <typename T>
-__global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restrict__ partial, ChunkTable tab, int V,
-                                                           int Ci, int Co, T* __restrict__ gw) {
+__global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restrict__ partial,
+                                                           const uint32_t* __restrict__ bounds, int V, int Ci, int Co,
+                                                           unsigned nb, T* __restrict__ gw) {
     const size_t per = (size_t)Co * Ci;
     const size_t total = per * V;
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
@@ -243,56 +328,71 @@ __global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restri
         size_t t = i / Ci;
         int v = (int)(t % V);
         int co = (int)(t / V);
+        const uint32_t* bd = bounds + (size_t)v * (nb + 1);
         float s = 0.f;
-        for (uint32_t c = tab.chunk_begin[v]; c < tab.chunk_begin[v + 1]; ++c) s += partial[(size_t)c * per + (size_t)co * Ci + ci];
+        for (unsigned b = 0; b < nb; ++b)
+            if (bd[b] < bd[b + 1]) s += partial[((size_t)b * V + v) * per + (size_t)co * Ci + ci];
         gw[i] = from_float<T>(s);
     }
 }
 
 bool dtype_ok(int dtype) { return dtype == FGX_F16 || dtype == FGX_BF16 || dtype == FGX_F32; }
 
-int make_table(const uint32_t* seg_host, int V, int chunk_pairs, ChunkTable* tab) {
-    uint32_t chunks = 0;
-    for (int v = 0; v < V; ++v) {
-        if (seg_host[v + 1] < seg_host[v]) return -1;
-        tab->seg[v] = seg_host[v];
-        tab->chunk_begin[v] = chunks;
-        uint32_t len = seg_host[v + 1] - seg_host[v];
-        chunks += (len + (uint32_t)chunk_pairs - 1) / (uint32_t)chunk_pairs;
-    }
-    tab->seg[V] = seg_host[V];
-    tab->chunk_begin[V] = chunks;
-    for (int v = V + 1; v <= kMaxV; ++v) { tab->seg[v] = seg_host[V]; tab->chunk_begin[v] = chunks; }
-    return (int)chunks;
+struct Layout {
+    unsigned nb;
+    size_t bounds_off, partial_off, total;
+};
+
+Layout layout(size_t n, int V, int Ci, int Co, int block_rows) {
+    Layout L{};
+    L.nb = n ? cdiv(n, (size_t)block_rows) : 0u;
+    size_t off = 0;
+    L.bounds_off = off;
+    off = align_up(off + (size_t)V * (L.nb + 1) * sizeof(uint32_t), 256);
+    L.partial_off = off;
+    off += (size_t)(L.nb ? L.nb : 1) * V * Co * Ci * sizeof(float);
+    L.total = off;
+    return L;
 }
 
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N>
-int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o, const ChunkTable& tab,
-                 int chunks, int V, int Ci, int Co, int chunk_pairs, void* scratch, void* gw, hipStream_t s) {
+int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o, const SegTable& tab,
+                 const Layout& L, int V, int Ci, int Co, int block_rows, void* scratch, void* gw, hipStream_t s) {
     using C = WgradCfg<Tag, BM, BN, WAVES_M, WAVES_N>;
     using T = typename Tag::type;
-    if (chunks > 0) {
+    uint32_t* bounds = (uint32_t*)((char*)scratch + L.bounds_off);
+    float* partial = (float*)((char*)scratch + L.partial_off);
+    if (L.nb > 0) {
+        block_bounds_kernel<<<cdiv((size_t)V * (L.nb + 1), 256), 256, 0, s>>>(sig_o, tab, V, L.nb, (unsigned)block_rows, bounds);
+        FGX_CHECK_LAUNCH("fgx_conv_wgrad(bounds)");
         const unsigned co_tiles = cdiv(Co, BM), ci_tiles = cdiv(Ci, BN);
-        dim3 grid(co_tiles * ci_tiles, (unsigned)chunks, 1);
-        wgrad_kernel<Tag, BM, BN, WAVES_M, WAVES_N><<<grid, C::NT, C::lds_bytes, s>>>(
-            (const T*)gout, (const T*)feats, sig_i, sig_o, tab, V, Ci, Co, chunk_pairs, co_tiles, ci_tiles, (float*)scratch);
+        const size_t grid = (size_t)cdiv(L.nb, kXcds) * V * co_tiles * ci_tiles * kXcds;
+        FGX_CHECK_ARG(grid < 0x7FFFFFFFull, "fgx_conv_wgrad: too many work items (%zu); use larger voxel blocks", grid);
+        auto kern = wgrad_kernel<Tag, BM, BN, WAVES_M, WAVES_N>;
+        static thread_local bool lds_raised = false;   // one raise of the dynamic LDS limit per thread and instantiation
+        if (C::lds_bytes > 64 * 1024 && !lds_raised) {
+            FGX_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::lds_bytes));
+            lds_raised = true;
+        }
+        kern<<<(unsigned)grid, C::NT, C::lds_bytes, s>>>(
+            (const T*)gout, (const T*)feats, sig_i, sig_o, bounds, V, Ci, Co, L.nb, co_tiles, ci_tiles, partial);
         FGX_CHECK_LAUNCH("fgx_conv_wgrad");
     }
     size_t total = (size_t)Co * V * Ci;
     unsigned g = cdiv(total, 256);
     if (g > 65536u) g = 65536u;
-    wgrad_reduce_kernel<T><<<g, 256, 0, s>>>((const float*)scratch, tab, V, Ci, Co, (T*)gw);
+    wgrad_reduce_kernel<T><<<g, 256, 0, s>>>(partial, bounds, V, Ci, Co, L.nb, (T*)gw);
     FGX_CHECK_LAUNCH("fgx_conv_wgrad(reduce)");
     return FGX_OK;
 }
 
 template <typename Tag>
 int dispatch_wgrad(int tile_rows, int tile_cols, const void* gout, const void* feats, const uint32_t* sig_i,
-                   const uint32_t* sig_o, const ChunkTable& tab, int chunks, int V, int Ci, int Co, int chunk_pairs,
+                   const uint32_t* sig_o, const SegTable& tab, const Layout& L, int V, int Ci, int Co, int block_rows,
                    void* scratch, void* gw, hipStream_t s) {
-#define FGX_TILE(BM, BN, WMv, WNv)               \
-    if (tile_rows == BM && tile_cols == BN)      \
-        return launch_wgrad<Tag, BM, BN, WMv, WNv>(gout, feats, sig_i, sig_o, tab, chunks, V, Ci, Co, chunk_pairs, scratch, gw, s);
+#define FGX_TILE(BM, BN, WMv, WNv)          \
+    if (tile_rows == BM && tile_cols == BN) \
+        return launch_wgrad<Tag, BM, BN, WMv, WNv>(gout, feats, sig_i, sig_o, tab, L, V, Ci, Co, block_rows, scratch, gw, s);
     FGX_TILE(128, 128, 2, 2)
     FGX_TILE(64, 64, 2, 2)
     FGX_TILE(32, 32, 1, 1)
@@ -308,37 +408,40 @@ using namespace fgx;
 
 extern "C" {
 
-size_t fgx_wgrad_scratch_bytes(const uint32_t* seg_host, int V, int Ci, int Co, int chunk_pairs) {
-    if (!seg_host || V < 1 || V > kMaxV || Ci <= 0 || Co <= 0 || chunk_pairs <= 0) return 0;
-    ChunkTable tab;
-    int chunks = make_table(seg_host, V, chunk_pairs, &tab);
-    if (chunks < 0) return 0;
-    return (size_t)(chunks > 0 ? chunks : 1) * (size_t)Co * (size_t)Ci * sizeof(float);
+size_t fgx_wgrad_scratch_bytes(size_t n, int V, int Ci, int Co, int block_rows) {
+    if (V < 1 || V > kMaxV || Ci <= 0 || Co <= 0 || block_rows <= 0) return 0;
+    return layout(n, V, Ci, Co, block_rows).total;
 }
 
 int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
-                   const uint32_t* seg_host, size_t n, int Ci, int Co, int V, int tile_rows, int tile_cols, int chunk_pairs,
+                   const uint32_t* seg_host, size_t n, int Ci, int Co, int V, int tile_rows, int tile_cols, int block_rows,
                    void* scratch, void* grad_weight, fgx_stream_t stream) {
     FGX_CHECK_ARG(dtype_ok(dtype), "fgx_conv_wgrad: unknown dtype %d", dtype);
     FGX_CHECK_ARG(Ci > 0 && Co > 0 && V >= 1 && V <= kMaxV, "fgx_conv_wgrad: bad shape Ci=%d Co=%d V=%d", Ci, Co, V);
-    FGX_CHECK_ARG(chunk_pairs >= 64 && chunk_pairs % 64 == 0, "fgx_conv_wgrad: chunk_pairs must be a positive multiple of 64, got %d", chunk_pairs);
+    FGX_CHECK_ARG(block_rows >= 1, "fgx_conv_wgrad: block_rows must be positive, got %d", block_rows);
     FGX_CHECK_ARG(seg_host && scratch && grad_weight, "fgx_conv_wgrad: null buffer");
+    FGX_CHECK_ARG(n < 0xFFFFFFFFull, "fgx_conv_wgrad: too many rows");
     const int es = dtype == FGX_F32 ? 4 : 2;
     FGX_CHECK_ARG(((size_t)Ci * es) % 16 == 0 && ((size_t)Co * es) % 16 == 0,
                   "fgx_conv_wgrad: rows of %d / %d elements are not multiples of 16 bytes", Ci, Co);
-    ChunkTable tab;
-    int chunks = make_table(seg_host, V, chunk_pairs, &tab);
-    FGX_CHECK_ARG(chunks >= 0 && chunks <= 65535, "fgx_conv_wgrad: segment table is not monotone or needs more than 65535 chunks");
-    if (chunks > 0) {
+    FGX_CHECK_ARG(((uintptr_t)scratch & 255) == 0, "fgx_conv_wgrad: scratch must be 256-byte aligned");
+    SegTable tab;
+    for (int v = 0; v <= V; ++v) {
+        FGX_CHECK_ARG(v == 0 || seg_host[v] >= seg_host[v - 1], "fgx_conv_wgrad: segment table is not monotone");
+        tab.seg[v] = seg_host[v];
+    }
+    for (int v = V + 1; v <= kMaxV; ++v) tab.seg[v] = seg_host[V];
+    const bool any = seg_host[V] > seg_host[0];
+    if (any) {
         FGX_CHECK_ARG(grad_out && feats && sig_i && sig_o, "fgx_conv_wgrad: null buffer");
         FGX_CHECK_ARG((((uintptr_t)grad_out | (uintptr_t)feats) & 15) == 0, "fgx_conv_wgrad: grad_out and feats must be 16-byte aligned");
     }
-    (void)n;
+    Layout L = layout(any ? n : 0, V, Ci, Co, block_rows);
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
-        case FGX_F16: return dispatch_wgrad<F16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, chunks, V, Ci, Co, chunk_pairs, scratch, grad_weight, s);
-        case FGX_BF16: return dispatch_wgrad<BF16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, chunks, V, Ci, Co, chunk_pairs, scratch, grad_weight, s);
-        default: return dispatch_wgrad<F32>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, chunks, V, Ci, Co, chunk_pairs, scratch, grad_weight, s);
+        case FGX_F16: return dispatch_wgrad<F16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, L, V, Ci, Co, block_rows, scratch, grad_weight, s);
+        case FGX_BF16: return dispatch_wgrad<BF16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, L, V, Ci, Co, block_rows, scratch, grad_weight, s);
+        default: return dispatch_wgrad<F32>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, L, V, Ci, Co, block_rows, scratch, grad_weight, s);
     }
 }
 

@@ -233,11 +233,13 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
         scratch = None
         if splitk > 1:
             scratch = nat.workspace(L.fgx_conv_scratch_bytes(nat.sz(n), C.c_int(cols), C.c_int(splitk)), dev)
+        nat.mark("gather_gemm_fwd" if mode == 0 else "gather_gemm_dgrad", "start")
         nat.check(L.fgx_conv_gather_gemm(
             C.c_int(code), nat.ptr(src), nat.ptr(panel), nat.ptr(bias), nat.ptr(cache["neighbor_map"]),
             nat.ptr(cache["sorted_idx"]), nat.ptr(tile_code), nat.sz(n), C.c_int(k), C.c_int(cols), C.c_int(v),
             C.c_int(sched.tile_rows), C.c_int(sched.tile_cols), C.c_int(splitk), nat.ptr(scratch), nat.ptr(out),
             nat.stream()))
+        nat.mark("gather_gemm_fwd" if mode == 0 else "gather_gemm_dgrad", "stop")
     return out
 
 
@@ -258,12 +260,14 @@ def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int) -> tor
     L = nat.lib()
     code = nat.DTYPE_CODE[dt]
     with torch.cuda.device(dev):
-        scratch = nat.workspace(L.fgx_wgrad_scratch_bytes(seg_arr, C.c_int(v), C.c_int(cip), C.c_int(cop),
-                                                          C.c_int(sched.chunk_pairs)), dev)
+        scratch = nat.workspace(L.fgx_wgrad_scratch_bytes(nat.sz(n), C.c_int(v), C.c_int(cip), C.c_int(cop),
+                                                          C.c_int(sched.block_rows)), dev)
+        nat.mark("wgrad", "start")
         nat.check(L.fgx_conv_wgrad(
             C.c_int(code), nat.ptr(g), nat.ptr(f), nat.ptr(cache["valid_signal_i"]), nat.ptr(cache["valid_signal_o"]),
             seg_arr, nat.sz(n), C.c_int(cip), C.c_int(cop), C.c_int(v), C.c_int(sched.tile_rows), C.c_int(sched.tile_cols),
-            C.c_int(sched.chunk_pairs), nat.ptr(scratch), nat.ptr(gw), nat.stream()))
+            C.c_int(sched.block_rows), nat.ptr(scratch), nat.ptr(gw), nat.stream()))
+        nat.mark("wgrad", "stop")
     if cip != ci or cop != co:
         gw = gw[:co, :, :ci].contiguous()
     return gw

@@ -134,7 +134,7 @@ typedef struct fgx_schedule {
     int tile_rows;      /* fwd/dgrad: sorted voxel rows per tile (B1); wgrad: Co rows per tile */
     int tile_cols;      /* fwd/dgrad: output channels per tile (B2);   wgrad: Ci columns per tile */
     int splitk;         /* fwd/dgrad: number of K splits (1 = none) */
-    int chunk_pairs;    /* wgrad: pairs per partial-sum chunk */
+    int block_rows;     /* wgrad: voxel rows per partial-sum block */
 } fgx_schedule;
 int fgx_table_lookup(int pass_kind, int dtype, size_t n, int Ci, int Co, int V, fgx_schedule* out);
 
@@ -165,14 +165,16 @@ int fgx_conv_gather_gemm(int dtype, const void* src, const void* panel, const vo
                          void* scratch, void* out, fgx_stream_t stream);
 
 /* grad_weight[co, v, ci] = sum over pairs k in [seg[v], seg[v+1]) of grad_out[sig_o[k], co] * feats[sig_i[k], ci].
- * seg_host is the HOST copy of valid_signal_seg (V+1 entries).  Partial sums of `chunk_pairs` pairs go to
- * `scratch` (fgx_wgrad_scratch_bytes bytes, fp32) and are reduced per offset in a second kernel.
+ * seg_host is the HOST copy of valid_signal_seg (V+1 entries); sig_o must ascend inside every segment (it does
+ * when it comes from fgx_pair_fill).  The voxels are cut into blocks of `block_rows` rows; every (block, offset)
+ * partial product goes to `scratch` in fp32 (fgx_wgrad_scratch_bytes bytes, 256-byte aligned) and a second kernel
+ * adds them per offset in block order.
  * Replaces: sparse_submanifold_conv_bwd_weight_masked_implicit_gemm[_splitk]
  *           (..._bwd_masked_implicit_gemm.py:99-170, ..._splitk.py:108-182, 278-317). */
-size_t fgx_wgrad_scratch_bytes(const uint32_t* seg_host, int V, int Ci, int Co, int chunk_pairs);
+size_t fgx_wgrad_scratch_bytes(size_t n, int V, int Ci, int Co, int block_rows);
 int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats,
                    const uint32_t* sig_i, const uint32_t* sig_o, const uint32_t* seg_host,
-                   size_t n, int Ci, int Co, int V, int tile_rows, int tile_cols, int chunk_pairs,
+                   size_t n, int Ci, int Co, int V, int tile_rows, int tile_cols, int block_rows,
                    void* scratch, void* grad_weight, fgx_stream_t stream);
 
 /* grad_bias[co] = sum over rows of grad_out[:, co], accumulated in fp32.

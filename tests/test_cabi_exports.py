@@ -42,15 +42,15 @@ def test_host_only_entry_points(library):
     s = nat.table_lookup(nat.PASS_FWD, torch.float16, 669288, 128, 128, 27)
     assert (s.tile_rows, s.tile_cols, s.splitk) == (128, 128, 1)
     s = nat.table_lookup(nat.PASS_WGRAD, torch.float16, 669288, 128, 128, 27)
-    assert s.chunk_pairs % 64 == 0 and s.chunk_pairs > 0
+    assert s.block_rows >= 1024
     s = nat.table_lookup(nat.PASS_FWD, torch.float32, 100, 16, 16, 27)
     assert s.tile_rows in (32, 64, 128) and s.tile_cols == 32 and s.splitk >= 1
     assert L.fgx_weight_panel_bytes(0, 0, 128, 128, 27, 128) == 27 * 2 * 128 * 128
     assert L.fgx_weight_panel_bytes(2, 1, 40, 24, 27, 32) == 27 * 1 * 64 * 128      # K=24 -> 1 slab, cols 40 -> 64
     assert L.fgx_conv_scratch_bytes(ctypes.c_size_t(1000), 64, 1) == 0
     assert L.fgx_conv_scratch_bytes(ctypes.c_size_t(1000), 64, 4) == 4 * 1000 * 64 * 4
-    seg = (ctypes.c_uint32 * 4)(0, 100, 100, 300)
-    assert L.fgx_wgrad_scratch_bytes(seg, 3, 8, 16, 64) == (2 + 0 + 4) * 8 * 16 * 4
+    # 1000 rows in blocks of 256 -> 4 blocks: bounds table (3 * 5 uint32, padded to 256 B) + 4 * 3 partial products
+    assert L.fgx_wgrad_scratch_bytes(ctypes.c_size_t(1000), 3, 8, 16, 256) == 256 + 4 * 3 * 8 * 16 * 4
 
 
 def test_argument_errors_map_to_exceptions(library):
@@ -62,7 +62,7 @@ def test_argument_errors_map_to_exceptions(library):
         nat.check(L.fgx_subm_neighbor_map(None, 32, None, ctypes.c_size_t(0), None, ctypes.c_size_t(0), 4, 4, 4,
                                           2, 3, 3, 1, 1, 1, None, None, None, None))
     with pytest.raises(ValueError):
-        nat.check(L.fgx_conv_wgrad(0, None, None, None, None, None, ctypes.c_size_t(0), 8, 8, 27, 128, 128, 100,
+        nat.check(L.fgx_conv_wgrad(0, None, None, None, None, None, ctypes.c_size_t(0), 8, 8, 27, 128, 128, 0,
                                    None, None, None))
 
 
