@@ -25,7 +25,7 @@ EXPORTS = [
     "fgx_hash_init", "fgx_hash_insert_3d_idx_as_val", "fgx_hash_insert", "fgx_hash_lookup",
     "fgx_hash_insert_3d", "fgx_hash_lookup_3d",
     "fgx_subm_neighbor_map", "fgx_mask_codes",
-    "fgx_sort_workspace_bytes", "fgx_sort_by_code",
+    "fgx_sort_workspace_bytes", "fgx_sort_by_code", "fgx_locality_workspace_bytes", "fgx_locality_order",
     "fgx_pair_workspace_bytes", "fgx_pair_count", "fgx_pair_fill",
     "fgx_tile_workspace_bytes", "fgx_tile_codes", "fgx_tile_fill",
     "fgx_table_lookup", "fgx_weight_panel_bytes", "fgx_pack_weight",
@@ -46,7 +46,8 @@ def mark(name: str, phase: str) -> None:
 
 
 class Schedule(C.Structure):
-    _fields_ = [("tile_rows", C.c_int), ("tile_cols", C.c_int), ("splitk", C.c_int), ("block_rows", C.c_int)]
+    _fields_ = [("tile_rows", C.c_int), ("tile_cols", C.c_int), ("slab_bytes", C.c_int), ("splitk", C.c_int),
+                ("block_rows", C.c_int)]
 
 
 class NativeError(RuntimeError):
@@ -67,7 +68,7 @@ def lib() -> C.CDLL:
                 "(hipcc --offload-arch=gfx950).  There is no fallback implementation.")
         L = C.CDLL(_LIB_PATH)
         L.fgx_last_error.restype = C.c_char_p
-        for name in ("fgx_sort_workspace_bytes", "fgx_pair_workspace_bytes", "fgx_tile_workspace_bytes",
+        for name in ("fgx_sort_workspace_bytes", "fgx_locality_workspace_bytes", "fgx_pair_workspace_bytes", "fgx_tile_workspace_bytes",
                      "fgx_weight_panel_bytes", "fgx_conv_scratch_bytes", "fgx_wgrad_scratch_bytes",
                      "fgx_colsum_scratch_bytes"):
             getattr(L, name).restype = C.c_size_t

@@ -5,17 +5,21 @@
 // One workgroup owns a tile of BM consecutive rows of the mask-sorted voxel order and BN output
 // channels.  Offsets whose bit is clear in the tile's OR-mask are skipped altogether.  The remaining
 // (offset, K-slab) steps stream through an S-stage ring in LDS: a stage holds the gathered source rows
-// (A, BM x 64 bytes) and the matching weight-panel slice (B, BN x 64 bytes).  Stages are filled by
-// direct global->LDS loads (global_load_lds_dwordx4: lane i of a wavefront deposits its 16 bytes at
-// LDS base + 16 i), issued S-1 steps ahead of their use, so several gathers are in flight per
-// workgroup while the wavefronts multiply.  The only vector-memory operations in the main loop are
-// these loads, which makes the outstanding-load counter exact: "step k has landed" is
-// s_waitcnt vmcnt((S-2) * loads_per_step), followed by one workgroup barrier per step.  Steps past the
-// end still issue (dummy) loads so that the count never changes.
+// (A, BM x 64 bytes) and the matching weight-panel slice (B, BN x 64 bytes).  The neighbor indices of
+// an offset (one column of the map, gathered through the sorted order) travel through a small ring of
+// their own, S-1 steps ahead of the rows that need them.  All of it is moved by direct global->LDS loads
+// (lane i of a wavefront deposits its data at LDS base + size * i), so several gathers are in flight
+// per workgroup while the wavefronts multiply and nothing waits for an index table to be staged first.
+// These loads are the only vector-memory operations in the main loop and every wavefront issues the
+// same number per step (dummy loads where it has nothing to fetch), which makes the outstanding-load
+// counter exact: "step k's rows and the indices for the next enqueue have landed" is
+// s_waitcnt vmcnt((S-2) * loads_per_step), followed by one workgroup barrier per step.
 //
 // The gather is a per-lane choice of global address, so a missing neighbor (or a K tail) simply reads
 // a block of zeros, and the bank-conflict swizzle of the 16-byte chunks is applied on the global side
 // (lane -> which chunk of the row it fetches) since the LDS side of the load is fixed.
+//
+// The output tile is converted, passed through LDS and written as whole 16-byte pieces of a row.
 //
 // Each of the WAVES_M x WAVES_N wavefronts multiplies its (BM/WAVES_M) x (BN/WAVES_N) sub-tile with
 // 32x32 MFMA instructions, accumulating in fp32.  Both operands are K-contiguous per row, and A and B
@@ -35,13 +39,14 @@ using f32x4 = float __attribute__((ext_vector_type(4)));
 using f32x16 = float __attribute__((ext_vector_type(16)));
 using u32x4 = uint32_t __attribute__((ext_vector_type(4)));
 
-constexpr int kSlabBytes = 64;    // bytes of K per row and step
-constexpr int kChunks = 4;        // 16-byte chunks per slab row
+// K-slab per row and step: 64 or 128 bytes (4 or 8 chunks of 16 bytes), a template parameter of the kernel
 constexpr int kXcds = 8;
-constexpr int kStages = 4;        // LDS ring depth
+constexpr int kIdxSlots = 4;      // neighbor-index ring depth (>= row ring depth)
 
 // 16 zero bytes every lane may read: missing neighbors, K tails, dummy loads past the last step
 __device__ __attribute__((aligned(256))) unsigned char g_zero_block[256];
+// the "no neighbor" word: index loads of rows past the end and dummy index loads read it
+__device__ __attribute__((aligned(16))) const uint32_t g_empty_word[4] = {FGX_EMPTY32, FGX_EMPTY32, FGX_EMPTY32, FGX_EMPTY32};
 
 #define FGX_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 #define FGX_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
@@ -90,11 +95,15 @@ template <> __device__ __forceinline__ float to_float<__bf16>(__bf16 x) {
     return __builtin_bit_cast(float, (uint32_t)__builtin_bit_cast(uint16_t, x) << 16);
 }
 
-// Physical position of logical chunk `chunk` of slab row `row`.  With 64-byte rows two rows share a 128-byte
-// bank line; the XOR key makes any 8 (and any 16) consecutive rows reading the same logical chunk hit
-// distinct 16-byte bank groups.
-__device__ __forceinline__ int swz_key(int row) { return ((row >> 1) + (row >> 3)) & 3; }
-__device__ __forceinline__ int swz(int row, int chunk) { return row * kSlabBytes + ((chunk ^ swz_key(row)) << 4); }
+// Physical position of logical chunk `chunk` of slab row `row` (CH chunks per row).  The XOR key makes rows that
+// read the same logical chunk in one LDS pass hit distinct 16-byte bank groups: with 128-byte rows any 8 consecutive
+// rows (and the even / odd rows of any 16), with 64-byte rows (two per bank line) any 8 and any 16 consecutive rows.
+template <int CH> __device__ __forceinline__ int swz_key(int row) {
+    return CH == 8 ? ((row + (row >> 3)) & 7) : (((row >> 1) + (row >> 3)) & 3);
+}
+template <int CH> __device__ __forceinline__ int swz(int row, int chunk) {
+    return row * (CH * 16) + ((chunk ^ swz_key<CH>(row)) << 4);
+}
 
 // ------------------------------------------------------------------------------------------------
 // Weight panels
@@ -102,8 +111,8 @@ __device__ __forceinline__ int swz(int row, int chunk) { return row * kSlabBytes
 // panel[v][slab][col][k] with k in [0, SK); mode 0: w[col][v][slab*SK+k]; mode 1: w[slab*SK+k][V-1-v][col].
 template <typename T>
 __global__ void __launch_bounds__(256) pack_weight_kernel(const T* __restrict__ w, int Ci, int Co, int V, int mode,
-                                                          int slabs, int cols_pad, T* __restrict__ panel) {
-    constexpr int SK = kSlabBytes / (int)sizeof(T);
+                                                          int slab_bytes, int slabs, int cols_pad, T* __restrict__ panel) {
+    const int SK = slab_bytes / (int)sizeof(T);
     const int K = mode == 0 ? Ci : Co;
     const int cols = mode == 0 ? Co : Ci;
     const size_t total = (size_t)V * slabs * cols_pad * SK;
@@ -127,38 +136,45 @@ __global__ void __launch_bounds__(256) pack_weight_kernel(const T* __restrict__ 
 // ------------------------------------------------------------------------------------------------
 // Gather GEMM
 // ------------------------------------------------------------------------------------------------
-template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N>
+template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int S, int CH>
 struct GemmCfg {
     using T = typename Tag::type;
+    static constexpr int ES = (int)sizeof(T);
     static constexpr int NW = WAVES_M * WAVES_N;
     static constexpr int NT = 64 * NW;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     static constexpr int TM = WM / 32, TN = WN / 32;
-    static constexpr int SK = kSlabBytes / (int)sizeof(T);
-    static constexpr int ROWS_PER_INST = 64 / kChunks;              // slab rows one wave-wide load covers
+    static constexpr int SLAB = CH * 16;                             // bytes of K per row and step
+    static constexpr int SK = SLAB / ES;
+    static constexpr int ROWS_PER_INST = 64 / CH;                    // slab rows one wave-wide load covers
     static constexpr int A_INST = BM / ROWS_PER_INST, B_INST = BN / ROWS_PER_INST;
-    static constexpr int A_PER = (A_INST + NW - 1) / NW, B_PER = (B_INST + NW - 1) / NW;  // loads per wavefront and step
-    static constexpr int LPS = A_PER + B_PER;
-    static constexpr int STAGE_BYTES = (BM + BN) * kSlabBytes;
+    static constexpr int A_PER = (A_INST + NW - 1) / NW, B_PER = (B_INST + NW - 1) / NW;  // row loads per wavefront and step
+    static constexpr int IDX_INST = (BM + 63) / 64;                  // wave-wide loads per index column
+    static constexpr int LPS = A_PER + B_PER + 1;                    // + one index load
+    static constexpr int STAGE_BYTES = (BM + BN) * SLAB;
+    static constexpr int IDX_SLOT_BYTES = IDX_INST * 256;
+    static constexpr int OUT_PITCH = WN * ES + 16;                   // epilogue band: 32 rows of a wave tile
+    static constexpr int OUT_BAND_BYTES = 32 * OUT_PITCH;
+    static constexpr int RING_BYTES = S * STAGE_BYTES > NW * OUT_BAND_BYTES ? S * STAGE_BYTES : NW * OUT_BAND_BYTES;
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
     static_assert(BM % ROWS_PER_INST == 0 && BN % ROWS_PER_INST == 0, "tile must be whole wave-wide loads");
-    static_assert((kStages - 2) * LPS < 64, "outstanding loads exceed the vmcnt range");
-    static constexpr size_t lds_bytes(int V) {
-        return (size_t)kStages * STAGE_BYTES + 1024 + (size_t)BM * V * 4 + (size_t)BM * 4 + 32 * 4;
-    }
+    static_assert((S - 2) * LPS < 64 && S >= 3 && S <= kIdxSlots, "ring depth out of range");
+    static_assert(CH == 4 || CH == 8, "slab must be 64 or 128 bytes");
+    static_assert((WN * ES) % 16 == 0, "a band row must be whole 16-byte pieces");
+    static constexpr size_t lds_bytes = (size_t)RING_BYTES + (size_t)kIdxSlots * IDX_SLOT_BYTES + 1024 + (size_t)BM * 4 + 32 * 4;
 };
 
-template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N>
+template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int S, int CH>
 __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N)
 gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Tag::type* __restrict__ panel,
                    const typename Tag::type* __restrict__ bias, const uint32_t* __restrict__ map,
                    const int64_t* __restrict__ sorted_idx, const int32_t* __restrict__ tile_code, uint32_t n, int K,
                    int cols, int cols_pad, int V, int splitk, unsigned row_tiles, unsigned col_tiles,
                    float* __restrict__ partial, typename Tag::type* __restrict__ out) {
-    using C = GemmCfg<Tag, BM, BN, WAVES_M, WAVES_N>;
+    using C = GemmCfg<Tag, BM, BN, WAVES_M, WAVES_N, S, CH>;
     using T = typename Tag::type;
     constexpr int NT = C::NT;
-    constexpr int S = kStages;
+    constexpr int kSlabBytes = C::SLAB, kChunks = CH;
 
     // XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs, so give each XCD a
     // contiguous run of tiles (all column tiles of a row tile share their gathered rows -> same L2).
@@ -171,10 +187,10 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
     const int kid = blockIdx.y;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-    unsigned char* ring = lds_raw;                                        // [S][A: BM x 64 | B: BN x 64]
-    unsigned char* dump = ring + S * C::STAGE_BYTES;                      // 1 KiB sink of surplus loads
-    uint32_t* nbr_lds = (uint32_t*)(dump + 1024);                         // [V][BM]
-    uint32_t* row_lds = nbr_lds + (size_t)BM * V;                         // [BM] output row or EMPTY
+    unsigned char* ring = lds_raw;                                        // [S][A: BM x 64 | B: BN x 64]; epilogue bands later
+    unsigned char* idx_ring = ring + C::RING_BYTES;                       // [kIdxSlots][BM] neighbor rows of one offset
+    unsigned char* dump = idx_ring + kIdxSlots * C::IDX_SLOT_BYTES;       // 1 KiB sink of surplus loads
+    uint32_t* row_lds = (uint32_t*)(dump + 1024);                         // [BM] output row or EMPTY
     int* v_lds = (int*)(row_lds + BM);                                    // [32] offsets present in this tile
 
     const int tid = threadIdx.x;
@@ -188,10 +204,18 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
     const int step_lo = (int)(((long long)steps_total * kid + splitk - 1) / splitk);
     const int step_hi = (int)(((long long)steps_total * (kid + 1) + splitk - 1) / splitk);
 
-    // ---- stage the tile's output rows, present offsets and neighbor indices ----
+    // ---- the tile's output rows; every wavefront also keeps the rows whose indices it will fetch ----
+    const int idx_inst = wave % C::IDX_INST;
+    const bool idx_owner = wave < C::IDX_INST;               // the other wavefronts only issue dummy index loads
+    const int idx_row = idx_inst * 64 + lane;
+    uint32_t my_row = FGX_EMPTY32;
+    {
+        const size_t gr = (size_t)row_tile * BM + idx_row;
+        if (idx_row < BM && gr < n) my_row = (uint32_t)sorted_idx[gr];
+    }
     for (int r = tid; r < BM; r += NT) {
-        size_t g = (size_t)row_tile * BM + r;
-        row_lds[r] = g < n ? (uint32_t)sorted_idx[g] : FGX_EMPTY32;
+        size_t gr = (size_t)row_tile * BM + r;
+        row_lds[r] = gr < n ? (uint32_t)sorted_idx[gr] : FGX_EMPTY32;
     }
     if (tid == 0) {
         uint32_t c = code;
@@ -200,14 +224,6 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
             v_lds[i++] = __ffs((int)c) - 1;
             c &= c - 1;
         }
-    }
-    __syncthreads();
-    for (int i = tid; i < BM * V; i += NT) {
-        int r = i / V, v = i - r * V;
-        uint32_t row = row_lds[r];
-        uint32_t m = FGX_EMPTY32;
-        if (row != FGX_EMPTY32 && ((code >> v) & 1u)) m = map[(size_t)row * V + v];
-        nbr_lds[v * BM + r] = m;
     }
     __syncthreads();   // also drains every outstanding vector-memory load: the counter starts at zero below
 
@@ -226,7 +242,31 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
     const int sub_row = lane / kChunks, pch = lane % kChunks;
     const bool ragged = (row_bytes % kSlabBytes) != 0;   // last slab of a row is partly past the row end
 
-    // ---- issue stream: runs S-1 steps ahead of the multiply stream and keeps per-lane source pointers that
+    // ---- index stream: one load per wavefront and step; a real one when a new offset comes into view ----
+    const uint32_t* my_map = my_row != FGX_EMPTY32 ? map + (size_t)my_row * V : nullptr;
+    int ix_step = step_lo, ix_vi = slabs > 0 ? step_lo / slabs : 0, ix_slab = step_lo - ix_vi * slabs;
+    int ix_done = -1;                                      // last offset slot whose load has been enqueued
+    auto issue_idx = [&]() {
+        const bool need = ix_step < step_hi && ix_vi > ix_done;      // wave-uniform
+        const uint32_t* p = g_empty_word;
+        unsigned char* dst = dump;
+        if (need) {
+            if (idx_owner) {
+                const int v = v_lds[ix_vi];
+                if (my_map != nullptr) p = my_map + v;
+                dst = idx_ring + (ix_vi % kIdxSlots) * C::IDX_SLOT_BYTES + idx_inst * 256;
+            }
+            ix_done = ix_vi;
+        }
+        __builtin_amdgcn_global_load_lds(FGX_GLOBAL_PTR(p), FGX_LDS_PTR(dst), 4, 0, 0);
+        ++ix_step;
+        if (++ix_slab == slabs) {
+            ix_slab = 0;
+            ++ix_vi;
+        }
+    };
+
+    // ---- row stream: runs S-1 steps ahead of the multiply stream and keeps per-lane source pointers that
     // advance by one slab per step; they are re-derived only when the offset changes ----
     int a_row[C::A_PER], a_choff[C::A_PER], a_inc[C::A_PER], b_off[C::B_PER];
     bool a_mine[C::A_PER], b_mine[C::B_PER];
@@ -236,7 +276,7 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
         const int inst = i * C::NW + wave;
         a_mine[i] = C::A_INST % C::NW == 0 || inst < C::A_INST;          // wave-uniform
         a_row[i] = (a_mine[i] ? inst : 0) * C::ROWS_PER_INST + sub_row;
-        a_choff[i] = (pch ^ swz_key(a_row[i])) << 4;
+        a_choff[i] = (pch ^ swz_key<CH>(a_row[i])) << 4;
         a_ptr[i] = zero_b;
         a_inc[i] = 0;
     }
@@ -245,24 +285,26 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
         const int inst = i * C::NW + wave;
         b_mine[i] = C::B_INST % C::NW == 0 || inst < C::B_INST;          // wave-uniform
         const int col = (b_mine[i] ? inst : 0) * C::ROWS_PER_INST + sub_row;
-        b_off[i] = col * kSlabBytes + ((pch ^ swz_key(col)) << 4);
+        b_off[i] = col * kSlabBytes + ((pch ^ swz_key<CH>(col)) << 4);
     }
     const size_t b_slab_stride = (size_t)cols_pad * kSlabBytes;
-    const unsigned char* b_ptr = zero_b;   // panel slice of the issue stream's (offset, slab), column tile applied
+    const unsigned char* b_ptr = zero_b;   // panel slice of the row stream's (offset, slab), column tile applied
     size_t b_inc = 0;
     int is_step = step_lo;                 // next step to enqueue
     int is_vi = slabs > 0 ? step_lo / slabs : 0;
     int is_slab = step_lo - is_vi * slabs;
+    int is_stage = 0;
     bool is_fresh = true;                  // pointers must be (re)derived before the next enqueue
 
-    auto issue = [&]() {
-        unsigned char* stage = ring + ((is_step - step_lo) % S) * C::STAGE_BYTES;
+    auto issue_rows = [&]() {
+        unsigned char* stage = ring + is_stage * C::STAGE_BYTES;
         if (is_fresh) {                    // wave-uniform: first call, offset change, or running off the end
             const bool live = is_step < step_hi;
             const int v = v_lds[live ? is_vi : 0];
+            const uint32_t* slot = (const uint32_t*)(idx_ring + ((live ? is_vi : 0) % kIdxSlots) * C::IDX_SLOT_BYTES);
 #pragma unroll
             for (int i = 0; i < C::A_PER; ++i) {
-                const uint32_t m = nbr_lds[v * BM + a_row[i]];
+                const uint32_t m = slot[a_row[i]];
                 const bool real = live && a_mine[i] && m != FGX_EMPTY32;
                 const size_t off = real ? (size_t)m * row_bytes + (size_t)(is_slab * kSlabBytes + a_choff[i]) : (size_t)0;
                 a_ptr[i] = real ? src_b + off : zero_b;
@@ -278,25 +320,18 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
             const unsigned char* p = a_ptr[i];
             if (tail) p = (size_t)(is_slab * kSlabBytes + a_choff[i]) < row_bytes ? p : zero_b;
             unsigned char* dst = a_mine[i] ? stage + (i * C::NW + wave) * 1024 : dump;
-#ifndef FGX_DBG_NO_LOAD
             __builtin_amdgcn_global_load_lds(FGX_GLOBAL_PTR(p), FGX_LDS_PTR(dst), 16, 0, 0);
-#else
-            asm volatile("" :: "v"(p), "v"(dst));
-#endif
             a_ptr[i] += a_inc[i];
         }
 #pragma unroll
         for (int i = 0; i < C::B_PER; ++i) {
             const unsigned char* p = (b_inc != 0 && b_mine[i]) ? b_ptr + b_off[i] : zero_b;
             unsigned char* dst = b_mine[i] ? stage + BM * kSlabBytes + (i * C::NW + wave) * 1024 : dump;
-#ifndef FGX_DBG_NO_LOAD
             __builtin_amdgcn_global_load_lds(FGX_GLOBAL_PTR(p), FGX_LDS_PTR(dst), 16, 0, 0);
-#else
-            asm volatile("" :: "v"(p), "v"(dst));
-#endif
         }
         b_ptr += b_inc;
         ++is_step;
+        is_stage = is_stage + 1 == S ? 0 : is_stage + 1;
         if (++is_slab == slabs) {
             is_slab = 0;
             ++is_vi;
@@ -305,8 +340,18 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
         if (is_step == step_hi) is_fresh = true;
     };
 
+    // ---- prologue: indices of the first S-1 steps, then S-1 enqueue rounds ----
 #pragma unroll
-    for (int s = 0; s < S - 1; ++s) issue();
+    for (int s = 0; s < S - 1; ++s) issue_idx();
+    wait_vmcnt<0>();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int s = 0; s < S - 1; ++s) {
+        issue_rows();
+        issue_idx();
+    }
 
     const int g = lane >> 5;        // lane group inside the MFMA fragment
     const int l32 = lane & 31;
@@ -314,36 +359,28 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
 #pragma unroll
     for (int kk = 0; kk < kChunks / 2; ++kk) {
 #pragma unroll
-        for (int i = 0; i < C::TM; ++i) a_frag[kk][i] = swz(wave_m * C::WM + i * 32 + l32, kk * 2 + g);
+        for (int i = 0; i < C::TM; ++i) a_frag[kk][i] = swz<CH>(wave_m * C::WM + i * 32 + l32, kk * 2 + g);
 #pragma unroll
-        for (int j = 0; j < C::TN; ++j) b_frag[kk][j] = BM * kSlabBytes + swz(wave_n * C::WN + j * 32 + l32, kk * 2 + g);
+        for (int j = 0; j < C::TN; ++j) b_frag[kk][j] = BM * kSlabBytes + swz<CH>(wave_n * C::WN + j * 32 + l32, kk * 2 + g);
     }
+    int cur_stage = 0;
     for (int step = step_lo; step < step_hi; ++step) {
-        // step's own loads are the oldest (S-1) * LPS still counted; everything older has been waited for
+        // rows of `step` and the indices the next enqueue needs are older than the (S-2) * LPS newest loads
         wait_vmcnt<(S - 2) * C::LPS>();
         asm volatile("" ::: "memory");
-#ifndef FGX_DBG_NO_BARRIER
-        __builtin_amdgcn_s_barrier();      // all lanes' loads of `step` landed; stage (step-1) % S is free again
-#endif
+        __builtin_amdgcn_s_barrier();      // everybody's loads landed; the stage read in the previous step is free again
         asm volatile("" ::: "memory");
-#ifndef FGX_DBG_NO_ISSUE
-        issue();
-#endif
-#ifndef FGX_DBG_NO_MMA
-        const unsigned char* cur = ring + ((step - step_lo) % S) * C::STAGE_BYTES;
+        issue_rows();
+        issue_idx();
+        const unsigned char* cur = ring + cur_stage * C::STAGE_BYTES;
+        cur_stage = cur_stage + 1 == S ? 0 : cur_stage + 1;
         u32x4 af[kChunks / 2][C::TM], bf[kChunks / 2][C::TN];
 #pragma unroll
         for (int kk = 0; kk < kChunks / 2; ++kk) {
 #pragma unroll
-#ifndef FGX_DBG_NO_LDSREAD
             for (int i = 0; i < C::TM; ++i) af[kk][i] = *(const u32x4*)(cur + a_frag[kk][i]);
 #pragma unroll
             for (int j = 0; j < C::TN; ++j) bf[kk][j] = *(const u32x4*)(cur + b_frag[kk][j]);
-#else
-            for (int i = 0; i < C::TM; ++i) { u32x4 t = {(uint32_t)step, (uint32_t)kk, (uint32_t)i, (uint32_t)(size_t)cur}; af[kk][i] = t; }
-#pragma unroll
-            for (int j = 0; j < C::TN; ++j) { u32x4 t = {(uint32_t)step, (uint32_t)kk, (uint32_t)j, 1u}; bf[kk][j] = t; }
-#endif
         }
 #pragma unroll
         for (int kk = 0; kk < kChunks / 2; ++kk)
@@ -351,27 +388,64 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
             for (int i = 0; i < C::TM; ++i)
 #pragma unroll
                 for (int j = 0; j < C::TN; ++j) mma<Tag>(acc[i][j], af[kk][i], bf[kk][j]);
-#endif
     }
     wait_vmcnt<0>();   // the trailing dummy loads
+    __syncthreads();   // the ring is reused below
 
-    // ---- epilogue: 32x32 accumulator tile, element e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32 ----
+    // ---- epilogue.  32x32 accumulator tile: element e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32. ----
+    if (splitk > 1) {
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) {
+            const int col = (int)col_tile * BN + wave_n * C::WN + j * 32 + l32;
+            if (col >= cols) continue;
+            const float bv = (bias != nullptr && kid == 0) ? to_float<T>(bias[col]) : 0.f;
+#pragma unroll
+            for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int r = wave_m * C::WM + i * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
+                    const uint32_t orow = row_lds[r];
+                    if (orow != FGX_EMPTY32) partial[((size_t)kid * n + orow) * cols + col] = acc[i][j][e] + bv;
+                }
+        }
+        return;
+    }
+    // One 32-row band of the wave tile at a time: add the bias, convert, park the band in LDS (each wavefront has
+    // its own area), then write whole 16-byte pieces of output rows.
+    unsigned char* band = ring + wave * C::OUT_BAND_BYTES;
+    float bv[C::TN];
 #pragma unroll
     for (int j = 0; j < C::TN; ++j) {
         const int col = (int)col_tile * BN + wave_n * C::WN + j * 32 + l32;
-        if (col >= cols) continue;
-        float bv = 0.f;
-        if (bias != nullptr && kid == 0) bv = to_float<T>(bias[col]);
+        bv[j] = (bias != nullptr && col < cols) ? to_float<T>(bias[col]) : 0.f;
+    }
+    constexpr int PIECES = C::WN * C::ES / 16;                // 16-byte pieces per band row
+    constexpr int ROWS_PER_PASS = 64 / PIECES;
+    const int col0 = (int)col_tile * BN + wave_n * C::WN;     // first output column of the wave tile
+    const bool vec_ok = (cols * C::ES) % 16 == 0;             // output rows start on 16-byte boundaries
 #pragma unroll
-        for (int i = 0; i < C::TM; ++i) {
+    for (int i = 0; i < C::TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                int r = wave_m * C::WM + i * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
-                uint32_t orow = row_lds[r];
-                if (orow == FGX_EMPTY32) continue;
-                float val = acc[i][j][e] + bv;
-                if (splitk > 1) partial[((size_t)kid * n + orow) * cols + col] = val;
-                else out[(size_t)orow * cols + col] = from_float<T>(val);
+                const int r = (e >> 2) * 8 + g * 4 + (e & 3);
+                *(T*)(band + r * C::OUT_PITCH + (j * 32 + l32) * C::ES) = from_float<T>(acc[i][j][e] + bv[j]);
+            }
+        // same wavefront wrote and reads: program order inside the wavefront suffices for LDS
+#pragma unroll
+        for (int pass = 0; pass < 32 / ROWS_PER_PASS; ++pass) {
+            const int r = pass * ROWS_PER_PASS + lane / PIECES;
+            const int piece = lane % PIECES;
+            const uint32_t orow = row_lds[wave_m * C::WM + i * 32 + r];
+            const int col = col0 + piece * (16 / C::ES);
+            if (orow == FGX_EMPTY32 || col >= cols) continue;
+            const unsigned char* sp = band + r * C::OUT_PITCH + piece * 16;
+            T* dp = out + (size_t)orow * cols + col;
+            if (vec_ok && col + 16 / C::ES <= cols) {
+                *(u32x4*)dp = *(const u32x4*)sp;
+            } else {
+                for (int t = 0; t < 16 / C::ES && col + t < cols; ++t) dp[t] = ((const T*)sp)[t];
             }
         }
     }
@@ -455,19 +529,19 @@ __global__ void __launch_bounds__(256) colsum_final_kernel(const float* __restri
 int elem_size(int dtype) { return dtype == FGX_F32 ? 4 : 2; }
 bool dtype_ok(int dtype) { return dtype == FGX_F16 || dtype == FGX_BF16 || dtype == FGX_F32; }
 
-template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N>
+template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int S, int CH>
 int launch_gemm(const void* src, const void* panel, const void* bias, const uint32_t* map, const int64_t* sorted_idx,
                 const int32_t* tile_code, size_t n, int K, int cols, int cols_pad, int V, int splitk, void* scratch,
                 void* out, hipStream_t s) {
-    using C = GemmCfg<Tag, BM, BN, WAVES_M, WAVES_N>;
+    using C = GemmCfg<Tag, BM, BN, WAVES_M, WAVES_N, S, CH>;
     using T = typename Tag::type;
-    auto kern = gather_gemm_kernel<Tag, BM, BN, WAVES_M, WAVES_N>;
-    const size_t lds = C::lds_bytes(V);
-    FGX_CHECK_ARG(lds <= 160 * 1024, "fgx_conv_gather_gemm: tile needs %zu bytes of LDS", lds);
-    static thread_local size_t lds_set = 0;   // raise the dynamic LDS limit once per thread and size
-    if (lds > 64 * 1024 && lds > lds_set) {
+    auto kern = gather_gemm_kernel<Tag, BM, BN, WAVES_M, WAVES_N, S, CH>;
+    constexpr size_t lds = C::lds_bytes;
+    static_assert(lds <= 160 * 1024, "tile does not fit the 160 KiB LDS");
+    static thread_local bool lds_raised = false;   // raise the dynamic LDS limit once per thread and instantiation
+    if (lds > 64 * 1024 && !lds_raised) {
         FGX_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        lds_set = lds;
+        lds_raised = true;
     }
     const unsigned row_tiles = cdiv(n, BM), col_tiles = cdiv(cols, BN);
     const unsigned total = row_tiles * col_tiles;
@@ -487,21 +561,23 @@ int launch_gemm(const void* src, const void* panel, const void* bias, const uint
 }
 
 template <typename Tag>
-int dispatch_tile(int tile_rows, int tile_cols, const void* src, const void* panel, const void* bias,
+int dispatch_tile(int tile_rows, int tile_cols, int slab_bytes, const void* src, const void* panel, const void* bias,
                   const uint32_t* map, const int64_t* sorted_idx, const int32_t* tile_code, size_t n, int K, int cols,
                   int cols_pad, int V, int splitk, void* scratch, void* out, hipStream_t s) {
-#define FGX_TILE(BM, BN, WMv, WNv)                                                                                    \
-    if (tile_rows == BM && tile_cols == BN)                                                                           \
-        return launch_gemm<Tag, BM, BN, WMv, WNv>(src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, \
-                                                  V, splitk, scratch, out, s);
-    FGX_TILE(128, 128, 2, 2)
-    FGX_TILE(128, 64, 2, 2)
-    FGX_TILE(128, 32, 4, 1)
-    FGX_TILE(64, 64, 2, 2)
-    FGX_TILE(64, 32, 2, 1)
-    FGX_TILE(32, 32, 1, 1)
+#define FGX_TILE(BM, BN, WMv, WNv, Sv, CHv)                                                                        \
+    if (tile_rows == BM && tile_cols == BN && slab_bytes == CHv * 16)                                              \
+        return launch_gemm<Tag, BM, BN, WMv, WNv, Sv, CHv>(src, panel, bias, map, sorted_idx, tile_code, n, K, cols, \
+                                                           cols_pad, V, splitk, scratch, out, s);
+    FGX_TILE(256, 128, 2, 2, 3, 4)
+    FGX_TILE(256, 128, 4, 2, 3, 8)
+    FGX_TILE(128, 128, 2, 2, 3, 4)
+    FGX_TILE(128, 64, 2, 2, 3, 4)
+    FGX_TILE(128, 32, 4, 1, 3, 4)
+    FGX_TILE(64, 64, 2, 2, 3, 4)
+    FGX_TILE(64, 32, 2, 1, 3, 4)
+    FGX_TILE(32, 32, 1, 1, 3, 4)
 #undef FGX_TILE
-    set_error("fgx_conv_gather_gemm: no kernel for tile %dx%d", tile_rows, tile_cols);
+    set_error("fgx_conv_gather_gemm: no kernel for tile %dx%d with %d-byte slabs", tile_rows, tile_cols, slab_bytes);
     return FGX_ERR_UNSUPPORTED;
 }
 
@@ -512,32 +588,33 @@ using namespace fgx;
 
 extern "C" {
 
-size_t fgx_weight_panel_bytes(int dtype, int mode, int Ci, int Co, int V, int col_pad) {
-    if (!dtype_ok(dtype) || Ci <= 0 || Co <= 0 || V <= 0 || col_pad <= 0) return 0;
+size_t fgx_weight_panel_bytes(int dtype, int mode, int Ci, int Co, int V, int slab_bytes, int col_pad) {
+    if (!dtype_ok(dtype) || Ci <= 0 || Co <= 0 || V <= 0 || col_pad <= 0 || (slab_bytes != 64 && slab_bytes != 128)) return 0;
     const int K = mode == 0 ? Ci : Co, cols = mode == 0 ? Co : Ci;
-    const int es = elem_size(dtype), SK = kSlabBytes / es;
+    const int es = elem_size(dtype), SK = slab_bytes / es;
     const size_t slabs = (size_t)(K + SK - 1) / SK;
     const size_t cols_pad = align_up((size_t)cols, (size_t)col_pad);
-    return (size_t)V * slabs * cols_pad * kSlabBytes;
+    return (size_t)V * slabs * cols_pad * slab_bytes;
 }
 
-int fgx_pack_weight(int dtype, int mode, const void* weight, int Ci, int Co, int V, int col_pad, void* panel,
-                    fgx_stream_t stream) {
+int fgx_pack_weight(int dtype, int mode, const void* weight, int Ci, int Co, int V, int slab_bytes, int col_pad,
+                    void* panel, fgx_stream_t stream) {
     FGX_CHECK_ARG(dtype_ok(dtype), "fgx_pack_weight: unknown dtype %d", dtype);
     FGX_CHECK_ARG(mode == 0 || mode == 1, "fgx_pack_weight: mode must be 0 (forward) or 1 (dgrad)");
     FGX_CHECK_ARG(Ci > 0 && Co > 0 && V > 0, "fgx_pack_weight: bad shape Ci=%d Co=%d V=%d", Ci, Co, V);
     FGX_CHECK_ARG(col_pad > 0 && col_pad % 32 == 0, "fgx_pack_weight: col_pad must be a positive multiple of 32");
+    FGX_CHECK_ARG(slab_bytes == 64 || slab_bytes == 128, "fgx_pack_weight: slab_bytes must be 64 or 128, got %d", slab_bytes);
     FGX_CHECK_ARG(weight && panel, "fgx_pack_weight: null buffer");
     const int K = mode == 0 ? Ci : Co, cols = mode == 0 ? Co : Ci;
-    const int es = elem_size(dtype), SK = kSlabBytes / es;
+    const int es = elem_size(dtype), SK = slab_bytes / es;
     const int slabs = (K + SK - 1) / SK;
     const int cols_pad = (int)align_up((size_t)cols, (size_t)col_pad);
     const size_t total = (size_t)V * slabs * cols_pad * SK;
     unsigned grid = cdiv(total, 256);
     if (grid > 32768u) grid = 32768u;
     hipStream_t s = (hipStream_t)stream;
-    if (dtype == FGX_F32) pack_weight_kernel<float><<<grid, 256, 0, s>>>((const float*)weight, Ci, Co, V, mode, slabs, cols_pad, (float*)panel);
-    else pack_weight_kernel<uint16_t><<<grid, 256, 0, s>>>((const uint16_t*)weight, Ci, Co, V, mode, slabs, cols_pad, (uint16_t*)panel);
+    if (dtype == FGX_F32) pack_weight_kernel<float><<<grid, 256, 0, s>>>((const float*)weight, Ci, Co, V, mode, slab_bytes, slabs, cols_pad, (float*)panel);
+    else pack_weight_kernel<uint16_t><<<grid, 256, 0, s>>>((const uint16_t*)weight, Ci, Co, V, mode, slab_bytes, slabs, cols_pad, (uint16_t*)panel);
     FGX_CHECK_LAUNCH("fgx_pack_weight");
     return FGX_OK;
 }
@@ -548,7 +625,8 @@ size_t fgx_conv_scratch_bytes(size_t n, int cols, int splitk) {
 
 int fgx_conv_gather_gemm(int dtype, const void* src, const void* panel, const void* bias, const uint32_t* map,
                          const int64_t* sorted_idx, const int32_t* tile_code, size_t n, int K, int cols, int V,
-                         int tile_rows, int tile_cols, int splitk, void* scratch, void* out, fgx_stream_t stream) {
+                         int tile_rows, int tile_cols, int slab_bytes, int splitk, void* scratch, void* out,
+                         fgx_stream_t stream) {
     FGX_CHECK_ARG(dtype_ok(dtype), "fgx_conv_gather_gemm: unknown dtype %d", dtype);
     FGX_CHECK_ARG(K > 0 && cols > 0 && V >= 1 && V <= 32, "fgx_conv_gather_gemm: bad shape K=%d cols=%d V=%d", K, cols, V);
     FGX_CHECK_ARG(splitk >= 1 && splitk <= 1024, "fgx_conv_gather_gemm: splitk %d out of range", splitk);
@@ -563,9 +641,9 @@ int fgx_conv_gather_gemm(int dtype, const void* src, const void* panel, const vo
     const int cols_pad = (int)align_up((size_t)cols, (size_t)tile_cols);
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
-        case FGX_F16: return dispatch_tile<F16>(tile_rows, tile_cols, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, out, s);
-        case FGX_BF16: return dispatch_tile<BF16>(tile_rows, tile_cols, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, out, s);
-        default: return dispatch_tile<F32>(tile_rows, tile_cols, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, out, s);
+        case FGX_F16: return dispatch_tile<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, out, s);
+        case FGX_BF16: return dispatch_tile<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, out, s);
+        default: return dispatch_tile<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, out, s);
     }
 }
 

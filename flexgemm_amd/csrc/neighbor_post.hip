@@ -31,6 +31,62 @@ __global__ void __launch_bounds__(kBlock) widen_u32_i64_kernel(const uint32_t* i
     if (i < n) out[i] = (int64_t)in[i];
 }
 
+// 16 bits of x, y, z interleaved (x highest), batch index on top: voxels close in space get close keys
+__device__ __forceinline__ uint64_t spread16(uint32_t x) {
+    uint64_t v = x & 0xFFFFu;
+    v = (v | (v << 16)) & 0x0000FF0000FFull;
+    v = (v | (v << 8)) & 0x00F00F00F00Full;
+    v = (v | (v << 4)) & 0x0C30C30C30C3ull;
+    v = (v | (v << 2)) & 0x249249249249ull;
+    return v;
+}
+
+__global__ void __launch_bounds__(kBlock) morton_key_kernel(const int32_t* __restrict__ coords, size_t n,
+                                                            uint64_t* __restrict__ keys, uint32_t* __restrict__ vals) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    int4 c = reinterpret_cast<const int4*>(coords)[i];
+    keys[i] = ((uint64_t)((uint32_t)c.x & 0xFFFFu) << 48) | (spread16((uint32_t)c.y) << 2) | (spread16((uint32_t)c.z) << 1) |
+              spread16((uint32_t)c.w);
+    vals[i] = (uint32_t)i;
+}
+
+// position p of the spatial order -> (chunk of p, mask code of its voxel)
+__global__ void __launch_bounds__(kBlock) chunk_code_key_kernel(const uint32_t* __restrict__ perm,
+                                                                const int32_t* __restrict__ binary, size_t n,
+                                                                uint32_t chunk_rows, uint64_t* __restrict__ keys) {
+    size_t p = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (p >= n) return;
+    keys[p] = ((uint64_t)(p / chunk_rows) << 32) | (uint32_t)binary[perm[p]];
+}
+
+struct LocalityLayout {
+    size_t keys_a, keys_b, vals_a, vals_b, temp, temp_bytes, total;
+};
+
+LocalityLayout locality_layout(size_t n) {
+    LocalityLayout L{};
+    size_t nn = n ? n : 1;
+    size_t temp_bytes = 0;
+    (void)rocprim::radix_sort_pairs(nullptr, temp_bytes, (const uint64_t*)nullptr, (uint64_t*)nullptr,
+                                    (const uint32_t*)nullptr, (uint32_t*)nullptr, nn, 0u, 64u, (hipStream_t)0);
+    size_t off = 0;
+    L.keys_a = off; off = align_up(off + nn * 8, 256);
+    L.keys_b = off; off = align_up(off + nn * 8, 256);
+    L.vals_a = off; off = align_up(off + nn * 4, 256);
+    L.vals_b = off; off = align_up(off + nn * 4, 256);
+    L.temp = off;   off = align_up(off + temp_bytes, 256);
+    L.temp_bytes = temp_bytes;
+    L.total = off;
+    return L;
+}
+
+int bits_for(size_t x) {   // smallest b with 2^b > x
+    int b = 0;
+    while (b < 63 && ((size_t)1 << b) <= x) ++b;
+    return b;
+}
+
 struct SortLayout {
     size_t keys_out, vals_in, vals_out, temp, temp_bytes, total;
 };
@@ -224,6 +280,40 @@ int fgx_sort_by_code(const int32_t* binary, size_t n, int V, int64_t* sorted_idx
     FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp_bytes, binary, keys_out, vals_in, vals_out, n, 0u, end_bit, s));
     widen_u32_i64_kernel<<<cdiv(n, kBlock), kBlock, 0, s>>>(vals_out, sorted_idx, n);
     FGX_CHECK_LAUNCH("fgx_sort_by_code(widen)");
+    return FGX_OK;
+}
+
+size_t fgx_locality_workspace_bytes(size_t n) { return locality_layout(n).total; }
+
+int fgx_locality_order(const int32_t* coords, const int32_t* binary, size_t n, int V, int chunk_rows, int64_t* order,
+                       void* workspace, size_t workspace_bytes, fgx_stream_t stream) {
+    FGX_CHECK_ARG(V >= 1 && V <= 32, "fgx_locality_order: kernel volume must be in [1, 32], got %d", V);
+    FGX_CHECK_ARG(chunk_rows >= 1, "fgx_locality_order: chunk_rows must be positive, got %d", chunk_rows);
+    FGX_CHECK_ARG(n < 0xFFFFFFFFull, "fgx_locality_order: too many rows");
+    if (n == 0) return FGX_OK;
+    LocalityLayout L = locality_layout(n);
+    FGX_CHECK_ARG(coords && binary && order && workspace, "fgx_locality_order: null buffer");
+    FGX_CHECK_ARG(((uintptr_t)coords & 15) == 0, "fgx_locality_order: coords must be 16-byte aligned");
+    FGX_CHECK_ARG(workspace_bytes >= L.total, "fgx_locality_order: workspace of %zu bytes, need %zu", workspace_bytes, L.total);
+    FGX_CHECK_ARG(((uintptr_t)workspace & 255) == 0, "fgx_locality_order: workspace must be 256-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    char* ws = (char*)workspace;
+    uint64_t* keys_a = (uint64_t*)(ws + L.keys_a);
+    uint64_t* keys_b = (uint64_t*)(ws + L.keys_b);
+    uint32_t* vals_a = (uint32_t*)(ws + L.vals_a);
+    uint32_t* vals_b = (uint32_t*)(ws + L.vals_b);
+    const unsigned grid = cdiv(n, kBlock);
+    morton_key_kernel<<<grid, kBlock, 0, s>>>(coords, n, keys_a, vals_a);
+    FGX_CHECK_LAUNCH("fgx_locality_order(keys)");
+    size_t temp_bytes = L.temp_bytes;
+    FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp_bytes, keys_a, keys_b, vals_a, vals_b, n, 0u, 64u, s));
+    chunk_code_key_kernel<<<grid, kBlock, 0, s>>>(vals_b, binary, n, (uint32_t)chunk_rows, keys_a);
+    FGX_CHECK_LAUNCH("fgx_locality_order(chunk keys)");
+    const unsigned end_bit = 32u + (unsigned)bits_for((n - 1) / (size_t)chunk_rows);
+    temp_bytes = L.temp_bytes;
+    FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp_bytes, keys_a, keys_b, vals_b, vals_a, n, 0u, end_bit, s));
+    widen_u32_i64_kernel<<<grid, kBlock, 0, s>>>(vals_a, order, n);
+    FGX_CHECK_LAUNCH("fgx_locality_order(widen)");
     return FGX_OK;
 }
 

@@ -20,9 +20,10 @@
 // Work decomposition and locality.  Inside one offset's segment the pairs are ordered by output row,
 // and the matching input rows are that row's neighbors, so the pairs of ALL offsets that belong to one
 // block of `block_rows` consecutive voxels touch the same few megabytes of grad_out / feats.  A work item
-// is therefore (voxel block b, offset v, Co-tile, Ci-tile); the items of one voxel block are dispatched
-// back to back onto the SAME XCD (workgroup ids are dealt round-robin over the 8 XCDs), so that the rows
-// are fetched from HBM once and then served by that XCD's L2 to the other offsets.  Each item writes an
+// is therefore (voxel block b, offset v, Co-tile, Ci-tile); the item list is block-major and each XCD takes
+// a contiguous eighth of it (workgroup ids are dealt round-robin over the 8 XCDs), so the items of one voxel
+// block run back to back on one XCD: the rows are fetched from HBM once and then served by that XCD's L2 to
+// the other offsets.  Each item writes an
 // fp32 partial product; a second kernel adds an offset's partials in block order (deterministic) and
 // casts to the output type.  The per-(offset, block) pair ranges are found by a small binary-search
 // kernel over sig_o.
@@ -142,13 +143,17 @@ wgrad_kernel(const typename Tag::type* __restrict__ gout, const typename Tag::ty
     constexpr int ES = C::ES;
     constexpr int S = kStages;
 
-    // XCD-aware item order: all (offset, tile) items of one voxel block run on one XCD, back to back.
+    // XCD-aware item order.  Items are listed block-major (block, offset, tile); workgroup ids are dealt round-robin
+    // over the 8 XCDs, so XCD x takes the x-th contiguous eighth of the list: the items of one voxel block run on one
+    // XCD back to back (or on a few neighbouring XCDs when there are fewer blocks than XCDs).
     const unsigned tiles = co_tiles * ci_tiles;
     const unsigned per_block = (unsigned)V * tiles;
-    const unsigned xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
-    const unsigned b = (slot / per_block) * kXcds + xcd;
-    if (b >= nb) return;
-    const unsigned within = slot % per_block;
+    const unsigned total_items = nb * per_block;
+    const unsigned per_xcd = (total_items + kXcds - 1) / kXcds;
+    const unsigned item = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
+    if (blockIdx.x / kXcds >= per_xcd || item >= total_items) return;
+    const unsigned b = item / per_block;
+    const unsigned within = item % per_block;
     const unsigned v = within / tiles;
     const unsigned tile = within % tiles;
     const unsigned co_tile = tile % co_tiles, ci_tile = tile / co_tiles;
@@ -366,7 +371,7 @@ int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, con
         block_bounds_kernel<<<cdiv((size_t)V * (L.nb + 1), 256), 256, 0, s>>>(sig_o, tab, V, L.nb, (unsigned)block_rows, bounds);
         FGX_CHECK_LAUNCH("fgx_conv_wgrad(bounds)");
         const unsigned co_tiles = cdiv(Co, BM), ci_tiles = cdiv(Ci, BN);
-        const size_t grid = (size_t)cdiv(L.nb, kXcds) * V * co_tiles * ci_tiles * kXcds;
+        const size_t grid = (size_t)cdiv((size_t)L.nb * V * co_tiles * ci_tiles, kXcds) * kXcds;
         FGX_CHECK_ARG(grid < 0x7FFFFFFFull, "fgx_conv_wgrad: too many work items (%zu); use larger voxel blocks", grid);
         auto kern = wgrad_kernel<Tag, BM, BN, WAVES_M, WAVES_N>;
         static thread_local bool lds_raised = false;   // one raise of the dynamic LDS limit per thread and instantiation

@@ -54,11 +54,20 @@ class SubMConv3dNeighborCache:
         return hasattr(self, key)
 
     # -- per-tile offset lists -------------------------------------------------------------------
-    def _tile_tables(self, block_size: int):
-        """(tile_code int32 [nb], seg int32 [nb+1]) for tiles of `block_size` sorted rows; no host sync."""
-        key = f"_tile_code_{block_size}"
+    def _tile_tables(self, block_size: int, private: bool):
+        """(order int64 [N], tile_code int32 [nb], seg int32 [nb+1]) for tiles of `block_size` rows; no host sync.
+
+        private=False: tiles of the public `sorted_idx` (what `valid_kernel_{B}` describes).
+        private=True : tiles of the cache-friendly row order the gfx950 kernels walk (`_tile_order` when the cache
+        was built from coordinates, otherwise the public order)."""
+        if private:
+            self._ensure_tile_order()
+        use_private = private and hasattr(self, "_tile_order")
+        order = self["_tile_order"] if use_private else self["sorted_idx"]
+        key = f"_tile_code_{block_size}" if use_private else f"_mask_code_{block_size}"
+        seg_key = f"_tile_seg_{block_size}" if use_private else f"valid_kernel_seg_{block_size}"
         if not hasattr(self, key):
-            gray, order = self["gray_code"], self["sorted_idx"]
+            gray = self["gray_code"]
             n = gray.shape[0]
             nb = (n + block_size - 1) // block_size
             code = torch.empty((nb,), dtype=torch.int32, device=gray.device)
@@ -70,8 +79,8 @@ class SubMConv3dNeighborCache:
                 nat.check(L.fgx_tile_codes(nat.ptr(gray), nat.ptr(order), nat.sz(n), C.c_int(block_size),
                                            nat.ptr(code), nat.ptr(seg), nat.ptr(ws), nat.sz(ws.numel()), nat.stream()))
             setattr(self, key, code)
-            setattr(self, f"valid_kernel_seg_{block_size}", seg)
-        return getattr(self, key), getattr(self, f"valid_kernel_seg_{block_size}")
+            setattr(self, seg_key, seg)
+        return order, getattr(self, key), getattr(self, seg_key)
 
     def compute_kernel_idx(self, block_size: int):
         """Fill `valid_kernel_{B}` / `valid_kernel_seg_{B}` (reference: submanifold_conv3d.py:20-23,
@@ -79,7 +88,7 @@ class SubMConv3dNeighborCache:
         block_size = int(block_size)
         if block_size < 1:
             raise ValueError(f"block_size must be positive, got {block_size}")
-        code, seg = self._tile_tables(block_size)
+        _, code, seg = self._tile_tables(block_size, private=False)
         nb = code.shape[0]
         total = int(seg[-1].item())
         vk = torch.empty((total,), dtype=torch.int32, device=code.device)
@@ -99,12 +108,23 @@ class SubMConv3dNeighborCache:
         return self[f"valid_kernel_seg_{block_size}"]
 
     # -- lazily completed fields -----------------------------------------------------------------
+    def _ensure_tile_order(self):
+        """Z-order-chunked, mask-sorted row order (private); needs the coordinates the cache was built from."""
+        if hasattr(self, "_tile_order") or not hasattr(self, "_coords"):
+            return
+        self._ensure_sorted()
+        if not hasattr(self, "_binary_code"):
+            _, binary, _ = _codes_and_order(self["neighbor_map"], None, None)
+            self["_binary_code"] = binary
+        self["_tile_order"] = _locality_order(self["_coords"], self["_binary_code"], self["neighbor_map"].shape[1])
+
+
     def _ensure_sorted(self):
         """gray_code / sorted_idx for a cache that only carries `neighbor_map`."""
         if hasattr(self, "gray_code") and hasattr(self, "sorted_idx"):
             return
         nmap = self["neighbor_map"]
-        gray, order = _codes_and_order(nmap, None, None)
+        gray, _, order = _codes_and_order(nmap, None, None)
         self["gray_code"], self["sorted_idx"] = gray, order
 
     def _ensure_pairs(self):
@@ -127,7 +147,7 @@ class SubMConv3dNeighborCache:
 # native helpers
 # ------------------------------------------------------------------------------------------------
 def _codes_and_order(nmap: torch.Tensor, gray: Optional[torch.Tensor], binary: Optional[torch.Tensor]):
-    """(gray_code, sorted_idx) from a neighbor map; gray/binary may come precomputed from the fused builder."""
+    """(gray_code, binary_code, sorted_idx) from a neighbor map; gray/binary may come precomputed from the fused builder."""
     n, v = nmap.shape
     dev = nmap.device
     L = nat.lib()
@@ -140,7 +160,26 @@ def _codes_and_order(nmap: torch.Tensor, gray: Optional[torch.Tensor], binary: O
         ws = nat.workspace(L.fgx_sort_workspace_bytes(nat.sz(n)), dev)
         nat.check(L.fgx_sort_by_code(nat.ptr(binary), nat.sz(n), C.c_int(v), nat.ptr(order), nat.ptr(ws),
                                      nat.sz(ws.numel()), nat.stream()))
-    return gray, order
+    return gray, binary, order
+
+
+# The kernels' private row order (Z-order chunks, mask-sorted inside a chunk) trades ~12 % more padded MFMA work for
+# gathers that stay inside an XCD's L2.  It pays when rows are short and the pass is bandwidth bound.
+LOCALITY_CHUNK_ROWS = 8192      # rows per spatial chunk
+LOCALITY_MAX_ROW_BYTES = 128    # use the private order when a gathered row is at most this long
+
+
+def _locality_order(coords: torch.Tensor, binary: torch.Tensor, v: int) -> torch.Tensor:
+    """Z-order chunks, mask-sorted inside each chunk (int64 permutation)."""
+    n = coords.shape[0]
+    dev = coords.device
+    order = torch.empty((n,), dtype=torch.int64, device=dev)
+    L = nat.lib()
+    with torch.cuda.device(dev):
+        ws = nat.workspace(L.fgx_locality_workspace_bytes(nat.sz(n)), dev)
+        nat.check(L.fgx_locality_order(nat.ptr(coords), nat.ptr(binary), nat.sz(n), C.c_int(v), C.c_int(LOCALITY_CHUNK_ROWS),
+                                       nat.ptr(order), nat.ptr(ws), nat.sz(ws.numel()), nat.stream()))
+    return order
 
 
 def _pair_lists(nmap: torch.Tensor, gray: torch.Tensor):
@@ -219,7 +258,7 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
     sched = nat.table_lookup(nat.PASS_FWD if mode == 0 else nat.PASS_DGRAD, dt, n, ci, co, v)
     splitk = sched.splitk if allow_splitk else 1
     cache._ensure_sorted()
-    tile_code, _ = cache._tile_tables(sched.tile_rows)
+    order, tile_code, _ = cache._tile_tables(sched.tile_rows, private=k * src.element_size() <= LOCALITY_MAX_ROW_BYTES)
     out = torch.empty((n, cols), dtype=dt, device=dev)
     if n == 0:
         return out
@@ -227,18 +266,18 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
     code = nat.DTYPE_CODE[dt]
     with torch.cuda.device(dev):
         panel = nat.workspace(L.fgx_weight_panel_bytes(C.c_int(code), C.c_int(mode), C.c_int(ci), C.c_int(co), C.c_int(v),
-                                                       C.c_int(sched.tile_cols)), dev)
+                                                       C.c_int(sched.slab_bytes), C.c_int(sched.tile_cols)), dev)
         nat.check(L.fgx_pack_weight(C.c_int(code), C.c_int(mode), nat.ptr(weight_cvk), C.c_int(ci), C.c_int(co), C.c_int(v),
-                                    C.c_int(sched.tile_cols), nat.ptr(panel), nat.stream()))
+                                    C.c_int(sched.slab_bytes), C.c_int(sched.tile_cols), nat.ptr(panel), nat.stream()))
         scratch = None
         if splitk > 1:
             scratch = nat.workspace(L.fgx_conv_scratch_bytes(nat.sz(n), C.c_int(cols), C.c_int(splitk)), dev)
         nat.mark("gather_gemm_fwd" if mode == 0 else "gather_gemm_dgrad", "start")
         nat.check(L.fgx_conv_gather_gemm(
             C.c_int(code), nat.ptr(src), nat.ptr(panel), nat.ptr(bias), nat.ptr(cache["neighbor_map"]),
-            nat.ptr(cache["sorted_idx"]), nat.ptr(tile_code), nat.sz(n), C.c_int(k), C.c_int(cols), C.c_int(v),
-            C.c_int(sched.tile_rows), C.c_int(sched.tile_cols), C.c_int(splitk), nat.ptr(scratch), nat.ptr(out),
-            nat.stream()))
+            nat.ptr(order), nat.ptr(tile_code), nat.sz(n), C.c_int(k), C.c_int(cols), C.c_int(v),
+            C.c_int(sched.tile_rows), C.c_int(sched.tile_cols), C.c_int(sched.slab_bytes), C.c_int(splitk),
+            nat.ptr(scratch), nat.ptr(out), nat.stream()))
         nat.mark("gather_gemm_fwd" if mode == 0 else "gather_gemm_dgrad", "stop")
     return out
 
@@ -317,8 +356,10 @@ class SubMConv3dFunction(Function):
             return SubMConv3dNeighborCache(neighbor_map=nmap)
         assert v <= 32, "Currently, the max kernel volume is 32 because kernel mask is encoded as uint32"
         nmap, gray, binary = _build_neighbor_map(coords, shape, kernel_size, dilation, with_codes=True)
-        gray, order = _codes_and_order(nmap, gray, binary)
+        gray, binary, order = _codes_and_order(nmap, gray, binary)
         cache = SubMConv3dNeighborCache(neighbor_map=nmap, gray_code=gray, sorted_idx=order)
+        cache["_coords"] = coords           # for the private row order, built on first use by a short-row layer
+        cache["_binary_code"] = binary
         if needs_grad:
             sig_i, sig_o, seg, seg_host = _pair_lists(nmap, gray)
             cache["valid_signal_seg"] = seg

@@ -100,6 +100,16 @@ size_t fgx_sort_workspace_bytes(size_t n);
 int fgx_sort_by_code(const int32_t* binary, size_t n, int V, int64_t* sorted_idx,
                      void* workspace, size_t workspace_bytes, fgx_stream_t stream);
 
+/* Row order for the gather GEMM that keeps gathers cache-resident: voxels are ranked along a Z-order curve of their
+ * coordinates, cut into chunks of `chunk_rows` consecutive ranks, and sorted by mask key inside each chunk (stable).
+ * Tiles of this order are still mask-homogeneous (their OR-masks come from fgx_tile_codes on this order) but all rows
+ * a run of tiles gathers lie in one small region, so an XCD's L2 serves the ~10 re-reads of every feature row.
+ * No counterpart in the reference, whose kernels walk the globally mask-sorted order (migemm_neighmap_pp.cu:79,221).
+ * Workspace: fgx_locality_workspace_bytes(n) bytes, 256-byte aligned. */
+size_t fgx_locality_workspace_bytes(size_t n);
+int fgx_locality_order(const int32_t* coords, const int32_t* binary, size_t n, int V, int chunk_rows, int64_t* order,
+                       void* workspace, size_t workspace_bytes, fgx_stream_t stream);
+
 /* Pair lists for wgrad: all (v, n) with map[n, v] present, ordered by v then n.
  *   count: seg[V+1] <- exclusive offsets per v (seg[V] = L); caller reads seg[V] back, allocates
  *          sig_i / sig_o of L uint32 each, then calls fill with the same workspace.
@@ -133,6 +143,7 @@ int fgx_tile_fill(const int32_t* tile_code, const int32_t* seg, size_t num_tiles
 typedef struct fgx_schedule {
     int tile_rows;      /* fwd/dgrad: sorted voxel rows per tile (B1); wgrad: Co rows per tile */
     int tile_cols;      /* fwd/dgrad: output channels per tile (B2);   wgrad: Ci columns per tile */
+    int slab_bytes;     /* fwd/dgrad: bytes of K staged per row and pipeline step (64 or 128) */
     int splitk;         /* fwd/dgrad: number of K splits (1 = none) */
     int block_rows;     /* wgrad: voxel rows per partial-sum block */
 } fgx_schedule;
@@ -141,15 +152,17 @@ int fgx_table_lookup(int pass_kind, int dtype, size_t n, int Ci, int Co, int V, 
 /* Re-layout the [Co, V, Ci] weight into K-slab-major panels consumed by fgx_conv_gather_gemm.
  *   mode 0 (forward): panel[v][slab][co][k]  = w[co][v][slab*SK + k]          (K = Ci, cols = Co)
  *   mode 1 (dgrad)  : panel[v][slab][ci][k]  = w[slab*SK + k][V-1-v][ci]      (K = Co, cols = Ci)
- * SK = 128 bytes / element size; K is zero-padded to a whole slab and cols to a multiple of col_pad
- * (a multiple of 32; pass the tile_cols the GEMM will run with).
+ * SK = slab_bytes / element size (slab_bytes = 64 or 128: the schedule's value); K is zero-padded to a whole
+ * slab and cols to a multiple of col_pad (a multiple of 32; pass the tile_cols the GEMM will run with).
  * Replaces: the strided weight-tile loads of the Triton kernels
  *           (..._fwd_masked_implicit_gemm.py:79, ..._bwd_masked_implicit_gemm.py:74). */
-size_t fgx_weight_panel_bytes(int dtype, int mode, int Ci, int Co, int V, int col_pad);
-int fgx_pack_weight(int dtype, int mode, const void* weight, int Ci, int Co, int V, int col_pad, void* panel,
-                    fgx_stream_t stream);
+size_t fgx_weight_panel_bytes(int dtype, int mode, int Ci, int Co, int V, int slab_bytes, int col_pad);
+int fgx_pack_weight(int dtype, int mode, const void* weight, int Ci, int Co, int V, int slab_bytes, int col_pad,
+                    void* panel, fgx_stream_t stream);
 
-/* out[sorted[r], :] = sum over offsets v present in row r of src[map[sorted[r], v], :] . panel_v  (+ bias)
+/* `sorted_idx` may be ANY permutation of the rows (the mask-sorted order or fgx_locality_order's); `tile_code` must
+ * come from fgx_tile_codes on that same permutation with block = tile_rows.
+ * out[sorted[r], :] = sum over offsets v present in row r of src[map[sorted[r], v], :] . panel_v  (+ bias)
  * for K = src channels, cols = out channels.  Forward: src = feats, panel mode 0, bias optional.
  * dgrad: src = grad_output, panel mode 1, bias = NULL.  Tiles of `tile_rows` sorted rows skip every
  * offset whose bit is clear in tile_code[tile].  splitk > 1 needs `scratch` of
@@ -161,7 +174,7 @@ int fgx_pack_weight(int dtype, int mode, const void* weight, int Ci, int Co, int
 size_t fgx_conv_scratch_bytes(size_t n, int cols, int splitk);
 int fgx_conv_gather_gemm(int dtype, const void* src, const void* panel, const void* bias,
                          const uint32_t* map, const int64_t* sorted_idx, const int32_t* tile_code,
-                         size_t n, int K, int cols, int V, int tile_rows, int tile_cols, int splitk,
+                         size_t n, int K, int cols, int V, int tile_rows, int tile_cols, int slab_bytes, int splitk,
                          void* scratch, void* out, fgx_stream_t stream);
 
 /* grad_weight[co, v, ci] = sum over pairs k in [seg[v], seg[v+1]) of grad_out[sig_o[k], co] * feats[sig_i[k], ci].

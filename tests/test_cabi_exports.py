@@ -40,13 +40,14 @@ def test_host_only_entry_points(library):
     L = nat.lib()
     import torch
     s = nat.table_lookup(nat.PASS_FWD, torch.float16, 669288, 128, 128, 27)
-    assert (s.tile_rows, s.tile_cols, s.splitk) == (128, 128, 1)
+    assert s.tile_rows in (128, 256) and s.tile_cols == 128 and s.splitk == 1 and s.slab_bytes in (64, 128)
     s = nat.table_lookup(nat.PASS_WGRAD, torch.float16, 669288, 128, 128, 27)
     assert s.block_rows >= 1024
     s = nat.table_lookup(nat.PASS_FWD, torch.float32, 100, 16, 16, 27)
     assert s.tile_rows in (32, 64, 128) and s.tile_cols == 32 and s.splitk >= 1
-    assert L.fgx_weight_panel_bytes(0, 0, 128, 128, 27, 128) == 27 * 2 * 128 * 128
-    assert L.fgx_weight_panel_bytes(2, 1, 40, 24, 27, 32) == 27 * 1 * 64 * 128      # K=24 -> 1 slab, cols 40 -> 64
+    assert L.fgx_weight_panel_bytes(0, 0, 128, 128, 27, 64, 128) == 27 * 2 * 128 * 128
+    assert L.fgx_weight_panel_bytes(2, 1, 40, 24, 27, 128, 32) == 27 * 1 * 64 * 128  # K=24 -> 1 slab, cols 40 -> 64
+    assert L.fgx_weight_panel_bytes(2, 1, 40, 24, 27, 64, 32) == 27 * 2 * 64 * 64    # 16 floats per slab -> 2 slabs
     assert L.fgx_conv_scratch_bytes(ctypes.c_size_t(1000), 64, 1) == 0
     assert L.fgx_conv_scratch_bytes(ctypes.c_size_t(1000), 64, 4) == 4 * 1000 * 64 * 4
     # 1000 rows in blocks of 256 -> 4 blocks: bounds table (3 * 5 uint32, padded to 256 B) + 4 * 3 partial products

@@ -129,6 +129,32 @@ def test_algorithm_values_and_cache_reuse(gpu_device):
     assert not hasattr(cch, "valid_signal_i") and out.shape == (len(coords_np), c)
 
 
+def test_private_row_order_is_used_and_equivalent(gpu_device):
+    """Short rows (<= 128 bytes) run on the Z-order-chunked private row order, long rows on the public mask-sorted one;
+    both give the oracle's result (checked by _run_and_check) and agree with each other."""
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    res = 24
+    coords_np = reference_test_shell(res)
+    coords_np = coords_np[np.random.default_rng(0).permutation(len(coords_np))]
+    shape = torch.Size([1, 0, res, res, res])
+    _say("private row order: C=32 fp16 (64-byte rows)")
+    cache, _ = _run_and_check(coords_np, shape, 32, 32, torch.float16, gpu_device, seed=21)
+    assert hasattr(cache, "_tile_order")
+    _say("public row order: C=128 fp16 (256-byte rows)")
+    cache2, _ = _run_and_check(coords_np, shape, 128, 128, torch.float16, gpu_device, seed=22)
+    assert not hasattr(cache2, "_tile_order")
+    f, w, b, _ = _case(coords_np, 32, 32, torch.float16, 23)
+    old = impl.LOCALITY_MAX_ROW_BYTES
+    outs = []
+    try:
+        for limit in (0, 1 << 20):
+            impl.LOCALITY_MAX_ROW_BYTES = limit
+            outs.append(impl._gather_gemm(f.to(gpu_device), w.to(gpu_device).reshape(32, 27, 32), b.to(gpu_device), cache, 0, True).float().cpu())
+    finally:
+        impl.LOCALITY_MAX_ROW_BYTES = old
+    assert eg.max_rel_err(outs[0], outs[1].double()) <= 2e-3
+
+
 def test_forced_splitk_matches_unsplit(gpu_device):
     """Split-K partial sums add up to the unsplit result (fp32 rounding apart)."""
     import ctypes as C

@@ -212,3 +212,44 @@ def test_standalone_hash_round_trip(gpu_device, kbits, vbits):
             t.keys[:] = _np(keys.view(torch.int32) if kbits == 32 else keys.view(torch.int64)).view(t.keys.dtype)
             t.vals[:] = _np(vals).view(np.uint32)
             assert np.array_equal(t.lookup_3d(coords_np, res, res, res), _np(values).view(np.uint32))
+
+
+def _morton_keys(coords_np):
+    def spread(x):
+        v = x.astype(np.uint64) & np.uint64(0xFFFF)
+        v = (v | (v << np.uint64(16))) & np.uint64(0x0000FF0000FF)
+        v = (v | (v << np.uint64(8))) & np.uint64(0x00F00F00F00F)
+        v = (v | (v << np.uint64(4))) & np.uint64(0x0C30C30C30C3)
+        v = (v | (v << np.uint64(2))) & np.uint64(0x249249249249)
+        return v
+    c = coords_np.astype(np.int64)
+    return (c[:, 0].astype(np.uint64) << np.uint64(48)) | (spread(c[:, 1]) << np.uint64(2)) | (spread(c[:, 2]) << np.uint64(1)) | spread(c[:, 3])
+
+
+@pytest.mark.parametrize("res,batch,shuffle", [(8, 1, False), (48, 2, True), (128, 1, True)])
+def test_private_tile_order(gpu_device, res, batch, shuffle):
+    """The kernels' private row order: Z-order ranks cut into chunks, stable mask sort inside each chunk."""
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    _say(f"private tile order res={res} batch={batch} shuffle={shuffle}")
+    coords_np = shell_coords(res, batch=batch)
+    if shuffle:
+        coords_np = coords_np[np.random.default_rng(res).permutation(len(coords_np))]
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    shape = torch.Size([batch, 0, res, res, res])
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), False)
+    assert not hasattr(cache, "_tile_order")      # built on first use by a short-row layer
+    cache._ensure_tile_order()
+    order = _np(cache._tile_order)
+    n = len(coords_np)
+    assert order.dtype == np.int64 and np.array_equal(np.sort(order), np.arange(n))
+    binary = df.gray_to_binary(_np(cache.gray_code)).astype(np.int64)
+    rank_order = np.argsort(_morton_keys(coords_np), kind="stable")          # position -> voxel
+    chunk = impl.LOCALITY_CHUNK_ROWS
+    key = (np.arange(n) // chunk).astype(np.int64) << 32 | binary[rank_order]
+    expect = rank_order[np.argsort(key, kind="stable")]
+    assert np.array_equal(order, expect)
+    # the public order is untouched and the public tile tables still describe it
+    assert np.array_equal(_np(cache.sorted_idx), np.argsort(binary, kind="stable"))
+    vk, seg = nb.tile_masks(_np(cache.gray_code), _np(cache.sorted_idx), 128)
+    assert np.array_equal(_np(cache.valid_kernel_callback(128)), vk)
+    assert np.array_equal(_np(cache.valid_kernel_seg_callback(128)), seg)
