@@ -38,6 +38,8 @@ def parse():
     p.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (used under rocprofv3)")
     p.add_argument("--cpu-rows", type=int, default=0, help="rows in the CPU baseline sample (0 = auto)")
     p.add_argument("--build-only", action="store_true", help="time only the neighbor-cache build")
+    p.add_argument("--calibrate-copy", action="store_true",
+                   help="also run a plain 1 GiB device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     return p.parse_args()
 
 
@@ -147,6 +149,14 @@ def main():
     for _ in range(max(args.warmup, 1)):
         step()
     torch.cuda.synchronize()
+    if args.calibrate_copy:
+        # a plain copy kernel of known size: reads 1 GiB, writes 1 GiB per launch
+        a = torch.empty(1 << 29, dtype=torch.float16, device=dev).fill_(1.0)
+        b = torch.empty_like(a)
+        for _ in range(3):
+            torch.neg(a, out=b)
+        torch.cuda.synchronize()
+        del a, b
 
     # HIP events around the dominant kernel's launches, on the stream they are launched on
     events = {}

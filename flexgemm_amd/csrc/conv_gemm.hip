@@ -465,7 +465,7 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restr
 // Column sums with fp32 accumulation.  Stage 1: kColsumSlices blocks each sum a contiguous slice of rows with
 // 16-byte loads (a thread owns VEC adjacent columns, the block's row lanes are added through LDS); stage 2 adds
 // the slices in a fixed order, so the result is deterministic.
-constexpr int kColsumSlices = 1024;
+constexpr int kColsumSlices = 512;
 template <typename T, int VEC>
 __global__ void __launch_bounds__(256) colsum_partial_kernel(const T* __restrict__ x, size_t n, int cols,
                                                              float* __restrict__ partial) {
@@ -511,19 +511,24 @@ __global__ void __launch_bounds__(256) colsum_partial_kernel(const T* __restrict
         }
     }
 }
-// 64 columns per block, 4 threads per column each adding a quarter of the slices
+// 16 columns per block, 16 threads per column each adding a sixteenth of the slices, then a fixed-order LDS sum
 template <typename T>
 __global__ void __launch_bounds__(256) colsum_final_kernel(const float* __restrict__ partial, unsigned slices, int cols,
                                                            T* __restrict__ out) {
     __shared__ float red[256];
-    const int c = blockIdx.x * 64 + (threadIdx.x & 63);
-    const int part = threadIdx.x >> 6;
+    const int c = blockIdx.x * 16 + (threadIdx.x & 15);
+    const int part = threadIdx.x >> 4;
     float s = 0.f;
     if (c < cols)
-        for (unsigned b = part; b < slices; b += 4) s += partial[(size_t)b * cols + c];
+        for (unsigned b = part; b < slices; b += 16) s += partial[(size_t)b * cols + c];
     red[threadIdx.x] = s;
     __syncthreads();
-    if (part == 0 && c < cols) out[c] = from_float<T>(red[threadIdx.x] + red[threadIdx.x + 64] + red[threadIdx.x + 128] + red[threadIdx.x + 192]);
+    if (part == 0 && c < cols) {
+        float t = 0.f;
+#pragma unroll
+        for (int p = 0; p < 16; ++p) t += red[p * 16 + threadIdx.x];
+        out[c] = from_float<T>(t);
+    }
 }
 
 int elem_size(int dtype) { return dtype == FGX_F32 ? 4 : 2; }
@@ -659,7 +664,7 @@ int fgx_colsum(int dtype, const void* x, size_t n, int cols, void* scratch, void
     hipStream_t s = (hipStream_t)stream;
     unsigned slices = n ? (unsigned)((n + 255) / 256) : 0u;     // at least 256 rows per slice
     if (slices > (unsigned)kColsumSlices) slices = kColsumSlices;
-    const unsigned gfin = cdiv(cols, 64);
+    const unsigned gfin = cdiv(cols, 16);
     const int es = elem_size(dtype);
     const bool vec = ((size_t)cols * es) % 16 == 0 && ((uintptr_t)x & 15) == 0;
 #define FGX_COLSUM(T, VEC)                                                                                        \

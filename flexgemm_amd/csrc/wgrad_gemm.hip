@@ -334,9 +334,19 @@ __global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restri
         int v = (int)(t % V);
         int co = (int)(t / V);
         const uint32_t* bd = bounds + (size_t)v * (nb + 1);
+        const float* src = partial + (size_t)v * per + (size_t)co * Ci + ci;
+        const size_t stride = (size_t)V * per;
         float s = 0.f;
-        for (unsigned b = 0; b < nb; ++b)
-            if (bd[b] < bd[b + 1]) s += partial[((size_t)b * V + v) * per + (size_t)co * Ci + ci];
+        unsigned b = 0;
+        for (; b + 4 <= nb; b += 4) {     // four independent loads in flight; the sum order stays b-ascending
+            const float x0 = bd[b] < bd[b + 1] ? src[(size_t)b * stride] : 0.f;
+            const float x1 = bd[b + 1] < bd[b + 2] ? src[(size_t)(b + 1) * stride] : 0.f;
+            const float x2 = bd[b + 2] < bd[b + 3] ? src[(size_t)(b + 2) * stride] : 0.f;
+            const float x3 = bd[b + 3] < bd[b + 4] ? src[(size_t)(b + 3) * stride] : 0.f;
+            s = (((s + x0) + x1) + x2) + x3;
+        }
+        for (; b < nb; ++b)
+            if (bd[b] < bd[b + 1]) s += src[(size_t)b * stride];
         gw[i] = from_float<T>(s);
     }
 }
