@@ -120,8 +120,22 @@ struct WgradCfg {
     static constexpr int key_b(int row) { return ES == 2 && CH_B >= 8 ? 2 * (row & 3) : 0; }
 };
 
+// Transposing LDS read, issued as inline assembly: through the compiler builtin every such read is preceded by a
+// conservative s_waitcnt vmcnt(0) (the compiler cannot tell it apart from the LDS areas the in-flight direct-to-LDS
+// loads are filling), which would drain the whole ring each step.  The price is that the result must be waited
+// for by hand: lds_wait_all() below ties the fragment registers to an s_waitcnt lgkmcnt(0).
 __device__ __forceinline__ i16x4 lds_read_tr16(const unsigned char* p) {
-    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((i16x4 __attribute__((address_space(3)))*)p);
+    const uint32_t addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const unsigned char*)p;
+    i16x4 r;
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(r) : "v"(addr));
+    return r;
+}
+template <int N>
+__device__ __forceinline__ void lds_wait_all(i16x4 (&r)[N]) {
+    static_assert(N % 4 == 0, "fragments come in groups of four registers pairs");
+#pragma unroll
+    for (int i = 0; i < N; i += 4)
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[i]), "+v"(r[i + 1]), "+v"(r[i + 2]), "+v"(r[i + 3]));
 }
 
 template <typename Tag> __device__ __forceinline__ void mma16(f32x16& acc, const i16x8& a, const i16x8& b);
@@ -138,7 +152,7 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N)
 wgrad_kernel(const typename Tag::type* __restrict__ gout, const typename Tag::type* __restrict__ feats,
              const uint32_t* __restrict__ sig_i, const uint32_t* __restrict__ sig_o,
              const uint32_t* __restrict__ bounds, int V, int Ci, int Co, unsigned nb, unsigned co_tiles,
-             unsigned ci_tiles, float* __restrict__ partial) {
+             unsigned ci_tiles, bool small_tensors, float* __restrict__ partial) {
     using C = WgradCfg<Tag, BM, BN, WAVES_M, WAVES_N>;
     constexpr int ES = C::ES;
     constexpr int S = kStages;
@@ -193,41 +207,63 @@ wgrad_kernel(const typename Tag::type* __restrict__ gout, const typename Tag::ty
         unsigned char* dst = idx_ring + (j & (kIdxSlots - 1)) * C::IDX_SLOT_BYTES;
         __builtin_amdgcn_global_load_lds(FGX_GLOBAL_PTR(src), FGX_LDS_PTR(dst), 4, 0, 0);
     };
-    auto idx_of = [&](int j, int p, int which) -> uint32_t {   // which: 0 = sig_o, 1 = sig_i
-        const uint32_t* slot_p = (const uint32_t*)(idx_ring + (j & (kIdxSlots - 1)) * C::IDX_SLOT_BYTES);
-        return slot_p[which * 32 + p];
-    };
-    // rows of step j into stage j % S; exactly A_PER + B_PER loads per wavefront
+    // rows of step j into stage j % S; exactly A_PER + B_PER loads per wavefront.  Steps whose 32 pairs all exist,
+    // in tiles that lie fully inside tensors of less than 4 GiB, take a lean path (32-bit offsets from a uniform base,
+    // no validity selects); the last partial step, edge tiles, huge tensors and the dummy steps take the general one.
+    int a_row[C::A_PER], a_colb[C::A_PER], b_row[C::B_PER], b_colb[C::B_PER];
+    bool a_mine[C::A_PER], b_mine[C::B_PER];
+#pragma unroll
+    for (int i = 0; i < C::A_PER; ++i) {
+        const int inst = i * C::NW + wave;
+        a_mine[i] = C::A_INST % C::NW == 0 || inst < C::A_INST;               // wave-uniform
+        a_row[i] = (a_mine[i] ? inst : 0) * C::RPI_A + lane / C::CH_A;
+        a_colb[i] = (m0 + ((lane % C::CH_A) ^ C::key_a(a_row[i])) * (16 / ES)) * ES;   // byte column in the tensor row
+    }
+#pragma unroll
+    for (int i = 0; i < C::B_PER; ++i) {
+        const int inst = i * C::NW + wave;
+        b_mine[i] = C::B_INST % C::NW == 0 || inst < C::B_INST;               // wave-uniform
+        b_row[i] = (b_mine[i] ? inst : 0) * C::RPI_B + lane / C::CH_B;
+        b_colb[i] = (n0 + ((lane % C::CH_B) ^ C::key_b(b_row[i])) * (16 / ES)) * ES;
+    }
+    const int full_steps = (int)((k_hi - k_lo) / C::PAIRS);
+    const bool lean_ok = m0 + BM <= Co && n0 + BN <= Ci && small_tensors &&
+                         C::A_INST % C::NW == 0 && C::B_INST % C::NW == 0;      // uniform
     auto issue_rows = [&](int j) {
         unsigned char* stage = ring + (j & (S - 1)) * C::STAGE_BYTES;
+        const uint32_t* slot_p = (const uint32_t*)(idx_ring + (j & (kIdxSlots - 1)) * C::IDX_SLOT_BYTES);
+        if (lean_ok && j < full_steps) {
+            uint32_t oa[C::A_PER], ob[C::B_PER];
+#pragma unroll
+            for (int i = 0; i < C::A_PER; ++i) oa[i] = slot_p[a_row[i]] * (uint32_t)rowb_o + (uint32_t)a_colb[i];
+#pragma unroll
+            for (int i = 0; i < C::B_PER; ++i) ob[i] = slot_p[32 + b_row[i]] * (uint32_t)rowb_i + (uint32_t)b_colb[i];
+#pragma unroll
+            for (int i = 0; i < C::A_PER; ++i)
+                __builtin_amdgcn_global_load_lds(FGX_GLOBAL_PTR(gout_b + oa[i]), FGX_LDS_PTR(stage + (i * C::NW + wave) * 1024), 16, 0, 0);
+#pragma unroll
+            for (int i = 0; i < C::B_PER; ++i)
+                __builtin_amdgcn_global_load_lds(FGX_GLOBAL_PTR(feats_b + ob[i]), FGX_LDS_PTR(stage + C::A_BYTES + (i * C::NW + wave) * 1024), 16, 0, 0);
+            return;
+        }
         const bool live = j < nsteps;
         const uint32_t kbase = k_lo + (uint32_t)j * C::PAIRS;
 #pragma unroll
         for (int i = 0; i < C::A_PER; ++i) {
-            const int inst = i * C::NW + wave;
-            const bool mine = C::A_INST % C::NW == 0 || inst < C::A_INST;      // wave-uniform
-            const int row = (mine ? inst : 0) * C::RPI_A + lane / C::CH_A;
-            const int c = (lane % C::CH_A) ^ C::key_a(row);
-            const int col = m0 + c * (16 / ES);
-            const uint32_t o = idx_of(j, row, 0);
-            const bool real = live && mine && kbase + (uint32_t)row < k_hi && col < Co;
-            const size_t off = real ? (size_t)o * rowb_o + (size_t)col * ES : (size_t)0;
+            const uint32_t o = slot_p[a_row[i]];
+            const bool real = live && a_mine[i] && kbase + (uint32_t)a_row[i] < k_hi && a_colb[i] < Co * ES;
+            const size_t off = real ? (size_t)o * rowb_o + (size_t)a_colb[i] : (size_t)0;
             const unsigned char* p = real ? gout_b + off : zero_b;
-            unsigned char* dst = mine ? stage + inst * 1024 : dump;
+            unsigned char* dst = a_mine[i] ? stage + (i * C::NW + wave) * 1024 : dump;
             __builtin_amdgcn_global_load_lds(FGX_GLOBAL_PTR(p), FGX_LDS_PTR(dst), 16, 0, 0);
         }
 #pragma unroll
         for (int i = 0; i < C::B_PER; ++i) {
-            const int inst = i * C::NW + wave;
-            const bool mine = C::B_INST % C::NW == 0 || inst < C::B_INST;      // wave-uniform
-            const int row = (mine ? inst : 0) * C::RPI_B + lane / C::CH_B;
-            const int c = (lane % C::CH_B) ^ C::key_b(row);
-            const int col = n0 + c * (16 / ES);
-            const uint32_t ii = idx_of(j, row, 1);
-            const bool real = live && mine && kbase + (uint32_t)row < k_hi && col < Ci;
-            const size_t off = real ? (size_t)ii * rowb_i + (size_t)col * ES : (size_t)0;
+            const uint32_t ii = slot_p[32 + b_row[i]];
+            const bool real = live && b_mine[i] && kbase + (uint32_t)b_row[i] < k_hi && b_colb[i] < Ci * ES;
+            const size_t off = real ? (size_t)ii * rowb_i + (size_t)b_colb[i] : (size_t)0;
             const unsigned char* p = real ? feats_b + off : zero_b;
-            unsigned char* dst = mine ? stage + C::A_BYTES + inst * 1024 : dump;
+            unsigned char* dst = b_mine[i] ? stage + C::A_BYTES + (i * C::NW + wave) * 1024 : dump;
             __builtin_amdgcn_global_load_lds(FGX_GLOBAL_PTR(p), FGX_LDS_PTR(dst), 16, 0, 0);
         }
     };
@@ -260,31 +296,38 @@ wgrad_kernel(const typename Tag::type* __restrict__ gout, const typename Tag::ty
             // Transposing read: in a 16-lane group, lane s supplies the address of 4 adjacent channels of pair
             // row (s / 4) and receives the 4 pair values of channel (group base + s).  Lanes 0-15 / 16-31 cover
             // fragment rows 0-15 / 16-31, the two wave halves take pair rows [0, 8) / [8, 16) of the k-step.
+            constexpr int NK = C::PAIRS / 16;
+            i16x4 ar[NK * C::TM * 2], br[NK * C::TN * 2];      // (lo, hi) halves of every fragment of the step
 #pragma unroll
-            for (int kk = 0; kk < C::PAIRS / 16; ++kk) {
+            for (int kk = 0; kk < NK; ++kk) {
                 const int prow = kk * 16 + g * 8 + (s16 >> 2);
-                i16x8 af[C::TM], bf[C::TN];
 #pragma unroll
                 for (int i = 0; i < C::TM; ++i) {
                     const int byte = (wave_m * C::WM + i * 32 + mb * 16 + (s16 & 3) * 4) * 2;
                     const int c = byte >> 4, w = byte & 15;
-                    i16x4 lo = lds_read_tr16(a_cur + prow * C::ROWB_A + ((c ^ C::key_a(prow)) << 4) + w);
-                    i16x4 hi = lds_read_tr16(a_cur + (prow + 4) * C::ROWB_A + ((c ^ C::key_a(prow + 4)) << 4) + w);
-                    af[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    ar[(kk * C::TM + i) * 2] = lds_read_tr16(a_cur + prow * C::ROWB_A + ((c ^ C::key_a(prow)) << 4) + w);
+                    ar[(kk * C::TM + i) * 2 + 1] = lds_read_tr16(a_cur + (prow + 4) * C::ROWB_A + ((c ^ C::key_a(prow + 4)) << 4) + w);
                 }
 #pragma unroll
                 for (int j = 0; j < C::TN; ++j) {
                     const int byte = (wave_n * C::WN + j * 32 + mb * 16 + (s16 & 3) * 4) * 2;
                     const int c = byte >> 4, w = byte & 15;
-                    i16x4 lo = lds_read_tr16(b_cur + prow * C::ROWB_B + ((c ^ C::key_b(prow)) << 4) + w);
-                    i16x4 hi = lds_read_tr16(b_cur + (prow + 4) * C::ROWB_B + ((c ^ C::key_b(prow + 4)) << 4) + w);
-                    bf[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    br[(kk * C::TN + j) * 2] = lds_read_tr16(b_cur + prow * C::ROWB_B + ((c ^ C::key_b(prow)) << 4) + w);
+                    br[(kk * C::TN + j) * 2 + 1] = lds_read_tr16(b_cur + (prow + 4) * C::ROWB_B + ((c ^ C::key_b(prow + 4)) << 4) + w);
                 }
+            }
+            lds_wait_all(ar);
+            lds_wait_all(br);
+#pragma unroll
+            for (int kk = 0; kk < NK; ++kk)
 #pragma unroll
                 for (int i = 0; i < C::TM; ++i)
 #pragma unroll
-                    for (int j = 0; j < C::TN; ++j) mma16<Tag>(acc[i][j], af[i], bf[j]);
-            }
+                    for (int j = 0; j < C::TN; ++j) {
+                        const i16x8 af = __builtin_shufflevector(ar[(kk * C::TM + i) * 2], ar[(kk * C::TM + i) * 2 + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                        const i16x8 bf = __builtin_shufflevector(br[(kk * C::TN + j) * 2], br[(kk * C::TN + j) * 2 + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                        mma16<Tag>(acc[i][j], af, bf);
+                    }
         } else {
             // fp32: one value per lane and MFMA (32x32x2); lane group g takes the odd / even pair of each couple
 #pragma unroll
@@ -372,7 +415,7 @@ Layout layout(size_t n, int V, int Ci, int Co, int block_rows) {
 
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N>
 int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o, const SegTable& tab,
-                 const Layout& L, int V, int Ci, int Co, int block_rows, void* scratch, void* gw, hipStream_t s) {
+                 const Layout& L, bool small, int V, int Ci, int Co, int block_rows, void* scratch, void* gw, hipStream_t s) {
     using C = WgradCfg<Tag, BM, BN, WAVES_M, WAVES_N>;
     using T = typename Tag::type;
     uint32_t* bounds = (uint32_t*)((char*)scratch + L.bounds_off);
@@ -390,7 +433,7 @@ int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, con
             lds_raised = true;
         }
         kern<<<(unsigned)grid, C::NT, C::lds_bytes, s>>>(
-            (const T*)gout, (const T*)feats, sig_i, sig_o, bounds, V, Ci, Co, L.nb, co_tiles, ci_tiles, partial);
+            (const T*)gout, (const T*)feats, sig_i, sig_o, bounds, V, Ci, Co, L.nb, co_tiles, ci_tiles, small, partial);
         FGX_CHECK_LAUNCH("fgx_conv_wgrad");
     }
     size_t total = (size_t)Co * V * Ci;
@@ -403,11 +446,11 @@ int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, con
 
 template <typename Tag>
 int dispatch_wgrad(int tile_rows, int tile_cols, const void* gout, const void* feats, const uint32_t* sig_i,
-                   const uint32_t* sig_o, const SegTable& tab, const Layout& L, int V, int Ci, int Co, int block_rows,
-                   void* scratch, void* gw, hipStream_t s) {
+                   const uint32_t* sig_o, const SegTable& tab, const Layout& L, bool small, int V, int Ci, int Co,
+                   int block_rows, void* scratch, void* gw, hipStream_t s) {
 #define FGX_TILE(BM, BN, WMv, WNv)          \
     if (tile_rows == BM && tile_cols == BN) \
-        return launch_wgrad<Tag, BM, BN, WMv, WNv>(gout, feats, sig_i, sig_o, tab, L, V, Ci, Co, block_rows, scratch, gw, s);
+        return launch_wgrad<Tag, BM, BN, WMv, WNv>(gout, feats, sig_i, sig_o, tab, L, small, V, Ci, Co, block_rows, scratch, gw, s);
     FGX_TILE(128, 128, 2, 2)
     FGX_TILE(64, 64, 2, 2)
     FGX_TILE(32, 32, 1, 1)
@@ -452,11 +495,13 @@ int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uin
         FGX_CHECK_ARG((((uintptr_t)grad_out | (uintptr_t)feats) & 15) == 0, "fgx_conv_wgrad: grad_out and feats must be 16-byte aligned");
     }
     Layout L = layout(any ? n : 0, V, Ci, Co, block_rows);
+    // 32-bit byte offsets into grad_out / feats are enough below 4 GiB
+    const bool small = (double)n * Co * es < 4294967296.0 && (double)n * Ci * es < 4294967296.0;
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
-        case FGX_F16: return dispatch_wgrad<F16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, L, V, Ci, Co, block_rows, scratch, grad_weight, s);
-        case FGX_BF16: return dispatch_wgrad<BF16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, L, V, Ci, Co, block_rows, scratch, grad_weight, s);
-        default: return dispatch_wgrad<F32>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, L, V, Ci, Co, block_rows, scratch, grad_weight, s);
+        case FGX_F16: return dispatch_wgrad<F16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);
+        case FGX_BF16: return dispatch_wgrad<BF16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);
+        default: return dispatch_wgrad<F32>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);
     }
 }
 
