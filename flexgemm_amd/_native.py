@@ -30,6 +30,7 @@ EXPORTS = [
     "fgx_tile_workspace_bytes", "fgx_tile_codes", "fgx_tile_fill",
     "fgx_table_lookup", "fgx_weight_panel_bytes", "fgx_pack_weight",
     "fgx_conv_scratch_bytes", "fgx_conv_gather_gemm",
+    "fgx_gather_plan_count", "fgx_gather_plan_fill", "fgx_conv_gather_gemm_stream",
     "fgx_wgrad_scratch_bytes", "fgx_conv_wgrad",
     "fgx_colsum_scratch_bytes", "fgx_colsum",
 ]
@@ -47,7 +48,7 @@ def mark(name: str, phase: str) -> None:
 
 class Schedule(C.Structure):
     _fields_ = [("tile_rows", C.c_int), ("tile_cols", C.c_int), ("slab_bytes", C.c_int), ("splitk", C.c_int),
-                ("block_rows", C.c_int)]
+                ("block_rows", C.c_int), ("stream", C.c_int)]
 
 
 class NativeError(RuntimeError):

@@ -1,0 +1,478 @@
+// Streaming masked implicit GEMM (forward and dgrad) for large voxel counts on gfx950.
+//
+//   out[order[r], :] = sum over offsets v present for row r of src[map[order[r], v], :] x panel_v (+ bias)
+//
+// Same arithmetic as the tiled kernel in conv_gemm.hip, organised for one resident workgroup per CU:
+//
+//  * A workgroup is persistent.  It walks its share of the (row tile, column tile) items -- item g, g + G, ... for
+//    workgroup g of G -- and treats all their (offset, K-slab) steps as ONE stream: the loads of the next item's first
+//    steps are in flight while the last steps of the current item are multiplied and its output tile is written, so
+//    neither the start-up latency of a tile nor its epilogue leaves the memory pipeline empty.
+//  * The per-tile neighbor indices come from the gather plan (fgx_gather_plan_fill): for every tile and every offset
+//    present in it, the tile's source rows as one contiguous run.  An index column is therefore one small contiguous
+//    load, fetched two offsets ahead of the rows that need it.
+//  * Every vector-memory load is a buffer load that writes straight into LDS (lane i deposits 16 bytes at LDS base
+//    + 16 * i).  A missing neighbor is an out-of-range buffer offset, which the hardware answers with zeros; the
+//    per-lane address of a row is a 32-bit offset computed once per offset and reused for all its K-slabs through the
+//    scalar offset operand, and the weight-panel and index loads use lane-constant offsets, so the steady state
+//    spends almost no vector ALU time on addressing.
+//  * No load returns into a register, so the only vector-memory counter traffic in the loop is this kernel's own:
+//    "the rows of step c have landed" is s_waitcnt vmcnt(number of loads this wavefront issued in the last
+//    iteration), chosen among a few immediates by a scalar branch, followed by one workgroup barrier per step.
+//    Output stores also count; they only make that wait stricter.
+//
+// Stage layout, swizzle, MFMA fragment mapping and the epilogue through LDS are those of the tiled kernel.  The
+// output tile is staged in the ring stage that was multiplied last (free until the next enqueue targets it).
+#include "gemm_device.h"
+
+namespace fgx {
+namespace {
+
+constexpr int kPlanSlots = 4;        // index ring depth
+constexpr int kPlanAhead = 2;        // the index stream runs this many offsets ahead of the row stream
+constexpr uint32_t kOobOffset = 0xFF000000u;   // buffer offset no source tensor reaches: the load returns zeros
+constexpr int kStreamStages = 3;
+
+using rsrc_t = __amdgpu_buffer_rsrc_t;
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), (short)0, (int)bytes, 0x00020000);
+}
+
+template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int CH>
+struct StreamCfg {
+    using T = typename Tag::type;
+    static constexpr int S = kStreamStages;
+    static constexpr int ES = (int)sizeof(T);
+    static constexpr int NW = WAVES_M * WAVES_N;
+    static constexpr int NT = 64 * NW;
+    static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    static constexpr int TM = WM / 32, TN = WN / 32;
+    static constexpr int SLAB = CH * 16;
+    static constexpr int SK = SLAB / ES;
+    static constexpr int ROWS_PER_INST = 64 / CH;
+    static constexpr int A_PER = BM / ROWS_PER_INST / NW, B_PER = BN / ROWS_PER_INST / NW;
+    static constexpr int LPS = A_PER + B_PER;                  // row loads per wavefront and step
+    static constexpr int IDX_INST = BM / 64;                   // wave-wide dword loads per index column
+    static constexpr int OROW_INST = (WM + 63) / 64;           // wave-wide dword loads for a wave tile's output rows
+    static constexpr int STAGE_BYTES = (BM + BN) * SLAB;
+    static constexpr int IDX_SLOT_BYTES = BM * 4;
+    static constexpr int OUT_PITCH = WN * ES + 16;
+    static constexpr int BAND_ROWS = NW * 32 * OUT_PITCH <= (BM + BN) * SLAB ? 32 : 16;   // rows staged per epilogue pass
+    static constexpr int OUT_BAND_BYTES = BAND_ROWS * OUT_PITCH;
+    static constexpr int OROW_BYTES = 2 * NW * OROW_INST * 256;
+    static constexpr int MAX_OPS = LPS + 1 + OROW_INST;        // most loads a wavefront issues in one iteration
+    static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
+    static_assert(BM % (ROWS_PER_INST * NW) == 0 && BN % (ROWS_PER_INST * NW) == 0, "every wavefront issues the same row loads");
+    static_assert(BM % 64 == 0 && IDX_INST <= NW, "index column must be whole wave-wide loads, one per wavefront");
+    static_assert(NW * OUT_BAND_BYTES <= STAGE_BYTES, "the output bands must fit one ring stage");
+    static_assert(MAX_OPS < 64, "vmcnt is a 6-bit counter");
+    static_assert(CH == 4 || CH == 8, "slab must be 64 or 128 bytes");
+    static constexpr size_t fixed_lds = (size_t)S * STAGE_BYTES + (size_t)kPlanSlots * IDX_SLOT_BYTES + OROW_BYTES;
+};
+
+// wait until at most `n` of this wavefront's vector-memory operations are outstanding.  n is wave-uniform; the
+// immediate used is the largest of 0, LPS, LPS + 1, ..., LPS + EXTRA that does not exceed n (smaller is merely stricter)
+template <int LPS, int K>
+struct WaitChain {
+    static __device__ __forceinline__ void run(int n) {
+        if (n >= LPS + K) wait_vmcnt<LPS + K>();
+        else WaitChain<LPS, K - 1>::run(n);
+    }
+};
+template <int LPS>
+struct WaitChain<LPS, -1> {
+    static __device__ __forceinline__ void run(int) { wait_vmcnt<0>(); }
+};
+template <int LPS, int EXTRA>
+__device__ __forceinline__ void wait_outstanding(int n) {
+    WaitChain<LPS, EXTRA>::run(n);
+}
+
+__device__ __forceinline__ void wg_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int CH>
+__global__ void __launch_bounds__(64 * WAVES_M * WAVES_N)
+gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const typename Tag::type* __restrict__ panel,
+                          const typename Tag::type* __restrict__ bias, const int64_t* __restrict__ order,
+                          const int32_t* __restrict__ plan_seg, const int32_t* __restrict__ plan_v,
+                          const uint32_t* __restrict__ plan_idx, uint32_t n, int K, int cols, int cols_pad,
+                          unsigned row_tiles, unsigned col_tiles, uint32_t src_bytes, uint32_t panel_bytes,
+                          uint32_t plan_bytes, typename Tag::type* __restrict__ out) {
+    using C = StreamCfg<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
+    using T = typename Tag::type;
+    constexpr int S = C::S, kSlabBytes = C::SLAB, kChunks = CH;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    unsigned char* ring = lds_raw;                                          // [S][A: BM x SLAB | B: BN x SLAB]
+    uint32_t* idx_ring = (uint32_t*)(ring + S * C::STAGE_BYTES);            // [kPlanSlots][BM] source rows of one offset
+    uint32_t* orow_lds = idx_ring + kPlanSlots * BM;                        // [2][NW][OROW_INST * 64] output rows
+    float* bias_lds = (float*)(orow_lds + C::OROW_BYTES / 4);               // [cols_pad]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+    const int g = lane >> 5, l32 = lane & 31;
+
+    const unsigned total_items = row_tiles * col_tiles;
+    const unsigned G = gridDim.x;
+    const unsigned dt = G / col_tiles, dct = G % col_tiles;     // item -> (row tile, column tile) increments
+    const int slabs = (K + C::SK - 1) / C::SK;
+    const uint32_t row_bytes = (uint32_t)K * sizeof(T);
+    const bool ragged = (row_bytes % kSlabBytes) != 0;
+
+    const rsrc_t src_rs = make_rsrc(src, src_bytes);
+    const rsrc_t panel_rs = make_rsrc(panel, panel_bytes);
+    const rsrc_t plan_rs = make_rsrc(plan_idx, plan_bytes);
+    const rsrc_t order_rs = make_rsrc(order, n * 8u);
+
+    for (int c = tid; c < cols_pad; c += C::NT) bias_lds[c] = (bias != nullptr && c < cols) ? to_float<T>(bias[c]) : 0.f;
+
+    // ---- lane constants ----
+    const int sub_row = lane / kChunks, pch = lane % kChunks;
+    int a_row[C::A_PER];
+    uint32_t a_choff[C::A_PER], a_voff[C::A_PER], b_voff[C::B_PER];
+#pragma unroll
+    for (int i = 0; i < C::A_PER; ++i) {
+        a_row[i] = (i * C::NW + wave) * C::ROWS_PER_INST + sub_row;
+        a_choff[i] = (uint32_t)((pch ^ swz_key<CH>(a_row[i])) << 4);
+        a_voff[i] = kOobOffset;
+    }
+#pragma unroll
+    for (int i = 0; i < C::B_PER; ++i) {
+        const int col = (i * C::NW + wave) * C::ROWS_PER_INST + sub_row;
+        b_voff[i] = (uint32_t)(col * kSlabBytes + ((pch ^ swz_key<CH>(col)) << 4));
+    }
+    const uint32_t idx_voff = (uint32_t)((wave * 64 + lane) * 4);           // used by wavefronts < IDX_INST only
+    const bool idx_wave = wave < C::IDX_INST;
+
+    // ---- the index stream: walks the plan rows of this workgroup's items, kPlanAhead offsets ahead of the rows ----
+    unsigned f_it = blockIdx.x, f_t = blockIdx.x / col_tiles, f_ct = blockIdx.x % col_tiles;
+    bool f_live = f_it < total_items;
+    int f_pos = 0, f_end = 0, f_ring = 0;
+    if (f_live) {
+        f_pos = plan_seg[f_t];
+        f_end = plan_seg[f_t + 1];
+    }
+    // queue of offsets the row stream has not started yet (head first)
+    int q_v[kPlanAhead], q_ct[kPlanAhead];
+    bool q_live[kPlanAhead];
+    auto fetch_slot = [&](int& v, int& ct, bool& live) -> int {     // returns the loads this wavefront issued
+        live = f_live;
+        v = 0;
+        ct = 0;
+        if (!f_live) return 0;
+        v = plan_v[f_pos];
+        ct = (int)f_ct;
+        int ops = 0;
+        if (idx_wave) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(plan_rs, FGX_LDS_PTR(idx_ring + f_ring * BM + wave * 64), 4, idx_voff,
+                                                     (uint32_t)f_pos * (uint32_t)(BM * 4), 0, 0);
+            ops = 1;
+        }
+        f_ring = (f_ring + 1) & (kPlanSlots - 1);
+        if (++f_pos == f_end) {
+            f_it += G;
+            f_live = f_it < total_items;
+            if (f_live) {
+                f_t += dt;
+                f_ct += dct;
+                if (f_ct >= col_tiles) {
+                    f_ct -= col_tiles;
+                    ++f_t;
+                }
+                f_pos = plan_seg[f_t];
+                f_end = plan_seg[f_t + 1];
+            }
+        }
+        return ops;
+    };
+
+    // ---- the row stream: S-1 steps ahead of the multiply stream ----
+    bool p_done = false;
+    int p_slab = 0, p_ring = 0, p_stage = 0;
+    uint32_t b_soff = 0;
+    const uint32_t b_slab_stride = (uint32_t)cols_pad * kSlabBytes;
+    auto produce = [&]() -> int {
+        if (p_done) return 0;
+        int ops = 0;
+        if (p_slab == 0) {
+            if (!q_live[0]) {
+                p_done = true;
+                return 0;
+            }
+            const int v = q_v[0], ct = q_ct[0];
+#pragma unroll
+            for (int i = 0; i + 1 < kPlanAhead; ++i) {
+                q_v[i] = q_v[i + 1];
+                q_ct[i] = q_ct[i + 1];
+                q_live[i] = q_live[i + 1];
+            }
+            const uint32_t* slot = idx_ring + p_ring * BM;
+#pragma unroll
+            for (int i = 0; i < C::A_PER; ++i) {
+                const uint32_t m = slot[a_row[i]];
+                a_voff[i] = m == FGX_EMPTY32 ? kOobOffset : m * row_bytes + a_choff[i];
+            }
+            b_soff = ((uint32_t)(v * slabs) * (uint32_t)cols_pad + (uint32_t)(ct * BN)) * kSlabBytes;
+            ops += fetch_slot(q_v[kPlanAhead - 1], q_ct[kPlanAhead - 1], q_live[kPlanAhead - 1]);
+        }
+        unsigned char* stage = ring + p_stage * C::STAGE_BYTES;
+        const uint32_t a_soff = (uint32_t)(p_slab * kSlabBytes);
+        const bool tail = ragged && p_slab == slabs - 1;     // wave-uniform
+#pragma unroll
+        for (int i = 0; i < C::A_PER; ++i) {
+            uint32_t vo = a_voff[i];
+            if (tail) vo = a_soff + a_choff[i] < row_bytes ? vo : kOobOffset;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(src_rs, FGX_LDS_PTR(stage + (i * C::NW + wave) * 1024), 16, vo, a_soff, 0, 0);
+        }
+        unsigned char* stage_b = stage + BM * kSlabBytes;
+#pragma unroll
+        for (int i = 0; i < C::B_PER; ++i) {
+            const uint32_t vo = b_voff[i];
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(panel_rs, FGX_LDS_PTR(stage_b + (i * C::NW + wave) * 1024), 16, vo, b_soff, 0, 0);
+        }
+        ops += C::LPS;
+        b_soff += b_slab_stride;
+        p_stage = p_stage + 1 == S ? 0 : p_stage + 1;
+        if (++p_slab == slabs) {
+            p_slab = 0;
+            p_ring = (p_ring + 1) & (kPlanSlots - 1);
+        }
+        return ops;
+    };
+
+    // ---- output rows of an item's wave tile: one (or two) small loads into this wavefront's own LDS area ----
+    auto fetch_orow = [&](unsigned t, int parity) {
+#pragma unroll
+        for (int j = 0; j < C::OROW_INST; ++j) {
+            const int r = j * 64 + lane;
+            const uint32_t row = t * (uint32_t)BM + (uint32_t)(wave_m * C::WM + r);
+            const uint32_t vo = (r < C::WM && row < n) ? row * 8u : kOobOffset;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(order_rs, FGX_LDS_PTR(orow_lds + ((parity * C::NW + wave) * C::OROW_INST + j) * 64),
+                                                     4, vo, 0, 0, 0);
+        }
+    };
+
+    // ---- multiply stream state ----
+    unsigned c_it = blockIdx.x, c_t = blockIdx.x / col_tiles, c_ct = blockIdx.x % col_tiles;
+    if (c_it >= total_items) return;                                   // whole workgroup
+    int c_lo = plan_seg[c_t], c_hi = plan_seg[c_t + 1];
+
+    // ---- prologue ----
+#pragma unroll
+    for (int i = 0; i < kPlanAhead; ++i) (void)fetch_slot(q_v[i], q_ct[i], q_live[i]);
+    fetch_orow(c_t, 0);
+    int ops_prev = 0;
+#pragma unroll
+    for (int s = 0; s < S - 1; ++s) {
+        wait_vmcnt<0>();
+        __syncthreads();      // also publishes bias_lds
+        ops_prev = produce();
+    }
+
+    int a_frag[kChunks / 2][C::TM], b_frag[kChunks / 2][C::TN];   // byte offsets of this lane's fragments in a stage
+#pragma unroll
+    for (int kk = 0; kk < kChunks / 2; ++kk) {
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i) a_frag[kk][i] = swz<CH>(wave_m * C::WM + i * 32 + l32, kk * 2 + g);
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) b_frag[kk][j] = BM * kSlabBytes + swz<CH>(wave_n * C::WN + j * 32 + l32, kk * 2 + g);
+    }
+    constexpr int PIECES = C::WN * C::ES / 16;                // 16-byte pieces per band row
+    constexpr int ROWS_PER_PASS = 64 / PIECES;
+    const bool vec_ok = (cols * C::ES) % 16 == 0;             // output rows start on 16-byte boundaries
+
+    int cur_stage = 0, parity = 0;
+    while (true) {
+        const int nsteps = (c_hi - c_lo) * slabs;
+        // the item after this one (its output rows are fetched now, its plan bounds are read now)
+        unsigned n_it = c_it + G, n_t = c_t + dt, n_ct = c_ct + dct;
+        if (n_ct >= col_tiles) {
+            n_ct -= col_tiles;
+            ++n_t;
+        }
+        const bool has_next = n_it < total_items;
+        int n_lo = 0, n_hi = 0;
+        if (has_next) {
+            n_lo = plan_seg[n_t];
+            n_hi = plan_seg[n_t + 1];
+        }
+
+        f32x16 acc[C::TM][C::TN];
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+            for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+        for (int s = 0; s < nsteps; ++s) {
+            // everything this wavefront issued before its previous iteration has landed: the rows of this step among it
+            wait_outstanding<C::LPS, 1 + C::OROW_INST>(ops_prev);
+            wg_barrier();                  // ... and everybody else's; the stage multiplied in the previous step is free
+            int ops = produce();
+            if (s == 0 && has_next) {
+                fetch_orow(n_t, parity ^ 1);
+                ops += C::OROW_INST;
+            }
+            ops_prev = ops;
+            const unsigned char* cur = ring + cur_stage * C::STAGE_BYTES;
+            cur_stage = cur_stage + 1 == S ? 0 : cur_stage + 1;
+            u32x4 af[kChunks / 2][C::TM], bf[kChunks / 2][C::TN];
+#pragma unroll
+            for (int kk = 0; kk < kChunks / 2; ++kk) {
+#pragma unroll
+                for (int i = 0; i < C::TM; ++i) af[kk][i] = *(const u32x4*)(cur + a_frag[kk][i]);
+#pragma unroll
+                for (int j = 0; j < C::TN; ++j) bf[kk][j] = *(const u32x4*)(cur + b_frag[kk][j]);
+            }
+#pragma unroll
+            for (int kk = 0; kk < kChunks / 2; ++kk)
+#pragma unroll
+                for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < C::TN; ++j) mma<Tag>(acc[i][j], af[kk][i], bf[kk][j]);
+        }
+
+        // ---- epilogue: 32x32 accumulator tile: element e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32 ----
+        wait_outstanding<C::LPS, 1 + C::OROW_INST>(ops_prev);   // this item's output rows have landed (fetched an item ago)
+        wg_barrier();                                           // everybody is done reading the last stage
+        {
+            const int last = cur_stage == 0 ? S - 1 : cur_stage - 1;
+            unsigned char* band = ring + last * C::STAGE_BYTES + wave * C::OUT_BAND_BYTES;
+            const uint32_t* my_orow = orow_lds + (parity * C::NW + wave) * C::OROW_INST * 64;
+            const int col0 = (int)c_ct * BN + wave_n * C::WN;
+            float bv[C::TN];
+#pragma unroll
+            for (int j = 0; j < C::TN; ++j) bv[j] = bias_lds[col0 + j * 32 + l32];
+#pragma unroll
+            for (int ih = 0; ih < C::TM * (32 / C::BAND_ROWS); ++ih) {
+                const int i = ih / (32 / C::BAND_ROWS), h = ih % (32 / C::BAND_ROWS);   // 32-row tile, half of it
+#pragma unroll
+                for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+                    for (int e = h * (C::BAND_ROWS / 2); e < (h + 1) * (C::BAND_ROWS / 2); ++e) {
+                        const int r = (e >> 2) * 8 + g * 4 + (e & 3) - h * C::BAND_ROWS;
+                        *(T*)(band + r * C::OUT_PITCH + (j * 32 + l32) * C::ES) = from_float<T>(acc[i][j][e] + bv[j]);
+                    }
+                // same wavefront wrote and reads: program order inside the wavefront suffices for LDS
+#pragma unroll
+                for (int pass = 0; pass < C::BAND_ROWS / ROWS_PER_PASS; ++pass) {
+                    const int r = pass * ROWS_PER_PASS + lane / PIECES;
+                    const int piece = lane % PIECES;
+                    const int tr = i * 32 + h * C::BAND_ROWS + r;                      // row inside the wave tile
+                    const bool live = c_t * (uint32_t)BM + (uint32_t)(wave_m * C::WM + tr) < n;
+                    const uint32_t orow = my_orow[tr];
+                    const int col = col0 + piece * (16 / C::ES);
+                    if (!live || col >= cols) continue;
+                    const unsigned char* sp = band + r * C::OUT_PITCH + piece * 16;
+                    T* dp = out + (size_t)orow * cols + col;
+                    if (vec_ok && col + 16 / C::ES <= cols) {
+                        *(u32x4*)dp = *(const u32x4*)sp;
+                    } else {
+                        for (int t = 0; t < 16 / C::ES && col + t < cols; ++t) dp[t] = ((const T*)sp)[t];
+                    }
+                }
+            }
+        }
+        if (!has_next) break;
+        c_it = n_it;
+        c_t = n_t;
+        c_ct = n_ct;
+        c_lo = n_lo;
+        c_hi = n_hi;
+        parity ^= 1;
+    }
+    wait_vmcnt<0>();
+}
+
+template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int CH>
+int launch_stream(const void* src, const void* panel, const void* bias, const int64_t* order, const int32_t* plan_seg,
+                  const int32_t* plan_v, const uint32_t* plan_idx, size_t plan_rows, size_t n, int K, int cols,
+                  int cols_pad, size_t panel_bytes, int max_groups, void* out, hipStream_t s) {
+    using C = StreamCfg<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
+    using T = typename Tag::type;
+    auto kern = gather_gemm_stream_kernel<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
+    const size_t lds = C::fixed_lds + (size_t)cols_pad * sizeof(float);
+    if (lds > 160 * 1024) {
+        set_error("fgx_conv_gather_gemm_stream: %d output columns need %zu bytes of LDS (limit 163840)", cols, lds);
+        return FGX_ERR_UNSUPPORTED;
+    }
+    static thread_local size_t lds_raised = 0;   // raise the dynamic LDS limit once per thread, instantiation and size
+    if (lds > 64 * 1024 && lds > lds_raised) {
+        FGX_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        lds_raised = lds;
+    }
+    const unsigned row_tiles = cdiv(n, BM), col_tiles = cdiv(cols, BN);
+    const size_t total = (size_t)row_tiles * col_tiles;
+    unsigned groups = (unsigned)(total < (size_t)max_groups ? total : (size_t)max_groups);
+    kern<<<groups, C::NT, lds, s>>>((const T*)src, (const T*)panel, (const T*)bias, order, plan_seg, plan_v, plan_idx,
+                                    (uint32_t)n, K, cols, cols_pad, row_tiles, col_tiles,
+                                    (uint32_t)(n * (size_t)K * sizeof(T)), (uint32_t)panel_bytes,
+                                    (uint32_t)(plan_rows * BM * 4), (T*)out);
+    FGX_CHECK_LAUNCH("fgx_conv_gather_gemm_stream");
+    return FGX_OK;
+}
+
+template <typename Tag>
+int dispatch_stream(int tile_rows, int tile_cols, int slab_bytes, const void* src, const void* panel, const void* bias,
+                    const int64_t* order, const int32_t* plan_seg, const int32_t* plan_v, const uint32_t* plan_idx,
+                    size_t plan_rows, size_t n, int K, int cols, int cols_pad, size_t panel_bytes, int max_groups,
+                    void* out, hipStream_t s) {
+#define FGX_STREAM_TILE(BM, BN, WMv, WNv, CHv)                                                                          \
+    if (tile_rows == BM && tile_cols == BN && slab_bytes == CHv * 16)                                                   \
+        return launch_stream<Tag, BM, BN, WMv, WNv, CHv>(src, panel, bias, order, plan_seg, plan_v, plan_idx, plan_rows, \
+                                                         n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
+    FGX_STREAM_TILE(256, 128, 4, 2, 8)
+#undef FGX_STREAM_TILE
+    set_error("fgx_conv_gather_gemm_stream: no kernel for tile %dx%d with %d-byte slabs", tile_rows, tile_cols, slab_bytes);
+    return FGX_ERR_UNSUPPORTED;
+}
+
+}  // namespace
+}  // namespace fgx
+
+using namespace fgx;
+
+extern "C" int fgx_conv_gather_gemm_stream(int dtype, const void* src, const void* panel, const void* bias,
+                                           const int64_t* order, const int32_t* plan_seg, const int32_t* plan_v,
+                                           const uint32_t* plan_idx, size_t plan_rows, size_t n, int K, int cols, int V,
+                                           int tile_rows, int tile_cols, int slab_bytes, int max_groups, void* out,
+                                           fgx_stream_t stream) {
+    FGX_CHECK_ARG(dtype == FGX_F16 || dtype == FGX_BF16 || dtype == FGX_F32, "fgx_conv_gather_gemm_stream: unknown dtype %d", dtype);
+    FGX_CHECK_ARG(K > 0 && cols > 0 && V >= 1 && V <= 32, "fgx_conv_gather_gemm_stream: bad shape K=%d cols=%d V=%d", K, cols, V);
+    if (n == 0) return FGX_OK;
+    const int es = dtype == FGX_F32 ? 4 : 2;
+    FGX_CHECK_ARG(((size_t)K * es) % 16 == 0, "fgx_conv_gather_gemm_stream: source row of %d elements is not a multiple of 16 bytes", K);
+    FGX_CHECK_ARG(src && panel && order && plan_seg && plan_v && plan_idx && out, "fgx_conv_gather_gemm_stream: null buffer");
+    FGX_CHECK_ARG((((uintptr_t)src | (uintptr_t)panel | (uintptr_t)plan_idx) & 15) == 0,
+                  "fgx_conv_gather_gemm_stream: src, panel and plan_idx must be 16-byte aligned");
+    FGX_CHECK_ARG(tile_rows > 0 && tile_cols > 0 && (slab_bytes == 64 || slab_bytes == 128), "fgx_conv_gather_gemm_stream: bad schedule");
+    if (max_groups <= 0) {
+        int dev = 0, cus = 0;
+        FGX_CHECK_HIP(hipGetDevice(&dev));
+        FGX_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        max_groups = cus > 0 ? cus : 256;
+    }
+    // 32-bit buffer offsets: every operand must stay below the out-of-range marker
+    const size_t src_bytes = n * (size_t)K * es;
+    const int cols_pad = (int)align_up((size_t)cols, (size_t)tile_cols);
+    const size_t slabs = ((size_t)K * es + slab_bytes - 1) / slab_bytes;
+    const size_t panel_bytes = (size_t)V * slabs * cols_pad * slab_bytes;
+    if (src_bytes > kOobOffset || panel_bytes > kOobOffset || plan_rows * (size_t)tile_rows * 4 > kOobOffset || n * 8 > kOobOffset) {
+        set_error("fgx_conv_gather_gemm_stream: an operand exceeds the 32-bit offset range (src %zu bytes); use fgx_conv_gather_gemm", src_bytes);
+        return FGX_ERR_UNSUPPORTED;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case FGX_F16: return dispatch_stream<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, plan_v, plan_idx, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
+        case FGX_BF16: return dispatch_stream<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, plan_v, plan_idx, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
+        default: return dispatch_stream<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, plan_v, plan_idx, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
+    }
+}

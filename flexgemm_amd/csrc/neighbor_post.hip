@@ -209,6 +209,47 @@ __global__ void __launch_bounds__(kBlock) tile_fill_kernel(const int32_t* __rest
     }
 }
 
+// Rows of the gather plan a tile contributes: one per offset present, and one (all rows missing) for a tile
+// without any, so that every tile owns at least one step of the streaming GEMM.
+__global__ void __launch_bounds__(kBlock) plan_count_kernel(const int32_t* __restrict__ tile_code, size_t num_tiles,
+                                                            uint32_t* __restrict__ cnt) {
+    size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= num_tiles) return;
+    const int c = __popc((uint32_t)tile_code[t]);
+    cnt[t] = (uint32_t)(c > 0 ? c : 1);
+}
+
+// One workgroup per tile: plan_v[seg[t] + k] = k-th offset present in the tile,
+// plan_idx[seg[t] + k][r] = map[order[t * tile_rows + r]][that offset] (EMPTY for rows past the end).
+__global__ void __launch_bounds__(kBlock) plan_fill_kernel(const uint32_t* __restrict__ map,
+                                                           const int64_t* __restrict__ order,
+                                                           const int32_t* __restrict__ tile_code,
+                                                           const int32_t* __restrict__ seg, size_t n, int V, int tile_rows,
+                                                           int32_t* __restrict__ plan_v, uint32_t* __restrict__ plan_idx) {
+    const size_t t = blockIdx.x;
+    uint32_t code = (uint32_t)tile_code[t];
+    size_t slot = (size_t)seg[t];
+    if (code == 0) {
+        if (threadIdx.x == 0) plan_v[slot] = 0;
+        for (int r = threadIdx.x; r < tile_rows; r += kBlock) plan_idx[slot * tile_rows + r] = FGX_EMPTY32;
+        return;
+    }
+    for (int r0 = 0; r0 < tile_rows; r0 += kBlock) {
+        const int r = r0 + threadIdx.x;
+        const size_t row = t * (size_t)tile_rows + r;
+        const uint32_t* mrow = (r < tile_rows && row < n) ? map + (size_t)order[row] * V : nullptr;
+        uint32_t c = code;
+        size_t s = slot;
+        while (c) {
+            const int v = __ffs((int)c) - 1;
+            c &= c - 1;
+            if (r0 == 0 && threadIdx.x == 0) plan_v[s] = v;
+            if (r < tile_rows) plan_idx[s * tile_rows + r] = mrow ? mrow[v] : FGX_EMPTY32;
+            ++s;
+        }
+    }
+}
+
 size_t scan_temp_bytes(size_t count) {
     size_t bytes = 0;
     (void)rocprim::exclusive_scan(nullptr, bytes, (const uint32_t*)nullptr, (uint32_t*)nullptr, 0u, count ? count : 1,
@@ -393,6 +434,44 @@ int fgx_tile_fill(const int32_t* tile_code, const int32_t* seg, size_t num_tiles
     FGX_CHECK_ARG(tile_code && seg && valid_kernel, "fgx_tile_fill: null buffer");
     tile_fill_kernel<<<cdiv(num_tiles, kBlock), kBlock, 0, (hipStream_t)stream>>>(tile_code, seg, num_tiles, valid_kernel);
     FGX_CHECK_LAUNCH("fgx_tile_fill");
+    return FGX_OK;
+}
+
+int fgx_gather_plan_count(const int32_t* tile_code, size_t num_tiles, int32_t* plan_seg, void* workspace,
+                          size_t workspace_bytes, fgx_stream_t stream) {
+    FGX_CHECK_ARG(plan_seg != nullptr, "fgx_gather_plan_count: null segment table");
+    hipStream_t s = (hipStream_t)stream;
+    if (num_tiles == 0) {
+        set_i32_kernel<<<1, 64, 0, s>>>(plan_seg, 0);
+        FGX_CHECK_LAUNCH("fgx_gather_plan_count(empty)");
+        return FGX_OK;
+    }
+    TileLayout L = tile_layout(num_tiles, 1);
+    FGX_CHECK_ARG(tile_code && workspace, "fgx_gather_plan_count: null buffer");
+    FGX_CHECK_ARG(workspace_bytes >= L.total, "fgx_gather_plan_count: workspace of %zu bytes, need %zu", workspace_bytes, L.total);
+    FGX_CHECK_ARG(((uintptr_t)workspace & 255) == 0, "fgx_gather_plan_count: workspace must be 256-byte aligned");
+    unsigned char* ws = (unsigned char*)workspace;
+    uint32_t* cnt = (uint32_t*)(ws + L.popc);
+    plan_count_kernel<<<cdiv(num_tiles, kBlock), kBlock, 0, s>>>(tile_code, num_tiles, cnt);
+    FGX_CHECK_LAUNCH("fgx_gather_plan_count(count)");
+    size_t temp_bytes = L.temp_bytes;
+    FGX_CHECK_HIP(rocprim::exclusive_scan(ws + L.temp, temp_bytes, cnt, (uint32_t*)plan_seg, 0u, num_tiles,
+                                          rocprim::plus<uint32_t>(), s));
+    tile_seg_tail_kernel<<<1, 64, 0, s>>>(cnt, plan_seg, num_tiles);
+    FGX_CHECK_LAUNCH("fgx_gather_plan_count(tail)");
+    return FGX_OK;
+}
+
+int fgx_gather_plan_fill(const uint32_t* map, const int64_t* order, const int32_t* tile_code, const int32_t* plan_seg,
+                         size_t n, int V, int tile_rows, int32_t* plan_v, uint32_t* plan_idx, fgx_stream_t stream) {
+    FGX_CHECK_ARG(tile_rows >= 1 && V >= 1 && V <= 32, "fgx_gather_plan_fill: bad shape tile_rows=%d V=%d", tile_rows, V);
+    if (n == 0) return FGX_OK;
+    FGX_CHECK_ARG(map && order && tile_code && plan_seg && plan_v && plan_idx, "fgx_gather_plan_fill: null buffer");
+    const size_t num_tiles = (n + tile_rows - 1) / tile_rows;
+    FGX_CHECK_ARG(num_tiles <= 0x7FFFFFFFu, "fgx_gather_plan_fill: too many tiles");
+    plan_fill_kernel<<<(unsigned)num_tiles, kBlock, 0, (hipStream_t)stream>>>(map, order, tile_code, plan_seg, n, V, tile_rows,
+                                                                              plan_v, plan_idx);
+    FGX_CHECK_LAUNCH("fgx_gather_plan_fill");
     return FGX_OK;
 }
 

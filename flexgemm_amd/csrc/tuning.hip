@@ -19,19 +19,19 @@ struct Entry {
 
 // Measured entries (MI355X).  Rows are matched exactly on (pass, element size, floor(log2 N), Ci, Co).
 const Entry kTable[] = {
-    // pass dtype log2n  Ci    Co    {rows, cols, slab_bytes, splitk, block_rows}
-    {0, 2, 19, 128, 128, {128, 128, 64, 1, 0}},
-    {1, 2, 19, 128, 128, {128, 128, 64, 1, 0}},
-    {2, 2, 19, 128, 128, {128, 128, 64, 1, 8192}},
-    {0, 2, 17, 256, 256, {128, 128, 64, 1, 0}},
-    {1, 2, 17, 256, 256, {128, 128, 64, 1, 0}},
-    {2, 2, 17, 256, 256, {128, 128, 64, 1, 4096}},
-    {0, 2, 21, 32, 32, {128, 32, 64, 1, 0}},
-    {1, 2, 21, 32, 32, {128, 32, 64, 1, 0}},
-    {2, 2, 21, 32, 32, {32, 32, 64, 1, 4096}},
-    {0, 2, 15, 1024, 1024, {128, 128, 64, 1, 0}},
-    {1, 2, 15, 1024, 1024, {128, 128, 64, 1, 0}},
-    {2, 2, 15, 1024, 1024, {128, 128, 64, 1, 65536}},
+    // pass dtype log2n  Ci    Co    {rows, cols, slab_bytes, splitk, block_rows, stream}
+    {0, 2, 19, 128, 128, {256, 128, 128, 1, 0, 1}},
+    {1, 2, 19, 128, 128, {256, 128, 128, 1, 0, 1}},
+    {2, 2, 19, 128, 128, {128, 128, 64, 1, 8192, 0}},
+    {0, 2, 17, 256, 256, {128, 128, 64, 1, 0, 0}},
+    {1, 2, 17, 256, 256, {128, 128, 64, 1, 0, 0}},
+    {2, 2, 17, 256, 256, {128, 128, 64, 1, 4096, 0}},
+    {0, 2, 21, 32, 32, {128, 32, 64, 1, 0, 0}},
+    {1, 2, 21, 32, 32, {128, 32, 64, 1, 0, 0}},
+    {2, 2, 21, 32, 32, {32, 32, 64, 1, 4096, 0}},
+    {0, 2, 15, 1024, 1024, {128, 128, 64, 1, 0, 0}},
+    {1, 2, 15, 1024, 1024, {128, 128, 64, 1, 0, 0}},
+    {2, 2, 15, 1024, 1024, {128, 128, 64, 1, 65536, 0}},
 };
 
 int floor_log2(size_t n) {
@@ -53,6 +53,7 @@ void rule(int pass_kind, size_t n, int Ci, int Co, int V, fgx_schedule* out) {
         out->tile_cols = t;
         out->slab_bytes = 64;
         out->splitk = 1;
+        out->stream = 0;
         const double per_block = 4.0 * V * (double)Co * (double)Ci;
         size_t max_blocks = (size_t)(268435456.0 / per_block);
         if (max_blocks < 1) max_blocks = 1;
@@ -68,6 +69,7 @@ void rule(int pass_kind, size_t n, int Ci, int Co, int V, fgx_schedule* out) {
     if (out->tile_rows == 64 && out->tile_cols == 128) out->tile_rows = 128;
     if (out->tile_rows == 32 && out->tile_cols != 32) out->tile_rows = out->tile_cols == 64 ? 64 : 128;
     out->block_rows = 0;
+    out->stream = 0;
     out->slab_bytes = 64;
     // split K only when the tiles cannot fill the chip (reference: candidates start at #SM / blocks)
     size_t tiles = (size_t)cdiv(n, out->tile_rows) * cdiv(cols, out->tile_cols);

@@ -82,6 +82,33 @@ class SubMConv3dNeighborCache:
             setattr(self, seg_key, seg)
         return order, getattr(self, key), getattr(self, seg_key)
 
+    def _gather_plan(self, block_size: int, private: bool):
+        """(order, plan_seg int32 [nb+1], plan_v int32 [P], plan_idx uint32 [P, block_size]) for the streaming GEMM:
+        per tile and offset present in it, the tile's source rows as one contiguous run.  Built once per tile size
+        (one 4-byte read-back sizes it) and kept with the cache."""
+        order, code, _ = self._tile_tables(block_size, private)
+        use_private = private and hasattr(self, "_tile_order")
+        key = f"_plan_{'t' if use_private else 'm'}_{block_size}"
+        if not hasattr(self, key):
+            nmap = self["neighbor_map"]
+            n, v = nmap.shape
+            nb = code.shape[0]
+            dev = nmap.device
+            seg = torch.empty((nb + 1,), dtype=torch.int32, device=dev)
+            with torch.cuda.device(dev):
+                L = nat.lib()
+                ws = nat.workspace(L.fgx_tile_workspace_bytes(nat.sz(nb), C.c_int(1)), dev)
+                nat.check(L.fgx_gather_plan_count(nat.ptr(code), nat.sz(nb), nat.ptr(seg), nat.ptr(ws), nat.sz(ws.numel()),
+                                                  nat.stream()))
+                rows = int(seg[-1].item())
+                plan_v = torch.empty((rows,), dtype=torch.int32, device=dev)
+                plan_idx = torch.empty((rows, block_size), dtype=torch.uint32, device=dev)
+                nat.check(L.fgx_gather_plan_fill(nat.ptr(nmap), nat.ptr(order), nat.ptr(code), nat.ptr(seg), nat.sz(n),
+                                                 C.c_int(v), C.c_int(block_size), nat.ptr(plan_v), nat.ptr(plan_idx),
+                                                 nat.stream()))
+            setattr(self, key, (seg, plan_v, plan_idx))
+        return (order,) + getattr(self, key)
+
     def compute_kernel_idx(self, block_size: int):
         """Fill `valid_kernel_{B}` / `valid_kernel_seg_{B}` (reference: submanifold_conv3d.py:20-23,
         native side migemm_neighmap_pp.cu:330-368).  One 4-byte read-back sizes the list."""
@@ -258,28 +285,45 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
     sched = nat.table_lookup(nat.PASS_FWD if mode == 0 else nat.PASS_DGRAD, dt, n, ci, co, v)
     splitk = sched.splitk if allow_splitk else 1
     cache._ensure_sorted()
-    order, tile_code, _ = cache._tile_tables(sched.tile_rows, private=k * src.element_size() <= LOCALITY_MAX_ROW_BYTES)
+    private = k * src.element_size() <= LOCALITY_MAX_ROW_BYTES
     out = torch.empty((n, cols), dtype=dt, device=dev)
     if n == 0:
         return out
     L = nat.lib()
     code = nat.DTYPE_CODE[dt]
+    name = "gather_gemm_fwd" if mode == 0 else "gather_gemm_dgrad"
     with torch.cuda.device(dev):
         panel = nat.workspace(L.fgx_weight_panel_bytes(C.c_int(code), C.c_int(mode), C.c_int(ci), C.c_int(co), C.c_int(v),
                                                        C.c_int(sched.slab_bytes), C.c_int(sched.tile_cols)), dev)
         nat.check(L.fgx_pack_weight(C.c_int(code), C.c_int(mode), nat.ptr(weight_cvk), C.c_int(ci), C.c_int(co), C.c_int(v),
                                     C.c_int(sched.slab_bytes), C.c_int(sched.tile_cols), nat.ptr(panel), nat.stream()))
+        if sched.stream and _stream_fits(n, k * src.element_size()):
+            order, plan_seg, plan_v, plan_idx = cache._gather_plan(sched.tile_rows, private)
+            nat.mark(name, "start")
+            nat.check(L.fgx_conv_gather_gemm_stream(
+                C.c_int(code), nat.ptr(src), nat.ptr(panel), nat.ptr(bias), nat.ptr(order), nat.ptr(plan_seg),
+                nat.ptr(plan_v), nat.ptr(plan_idx), nat.sz(plan_v.shape[0]), nat.sz(n), C.c_int(k), C.c_int(cols), C.c_int(v),
+                C.c_int(sched.tile_rows), C.c_int(sched.tile_cols), C.c_int(sched.slab_bytes), C.c_int(0), nat.ptr(out),
+                nat.stream()))
+            nat.mark(name, "stop")
+            return out
+        order, tile_code, _ = cache._tile_tables(sched.tile_rows, private)
         scratch = None
         if splitk > 1:
             scratch = nat.workspace(L.fgx_conv_scratch_bytes(nat.sz(n), C.c_int(cols), C.c_int(splitk)), dev)
-        nat.mark("gather_gemm_fwd" if mode == 0 else "gather_gemm_dgrad", "start")
+        nat.mark(name, "start")
         nat.check(L.fgx_conv_gather_gemm(
             C.c_int(code), nat.ptr(src), nat.ptr(panel), nat.ptr(bias), nat.ptr(cache["neighbor_map"]),
             nat.ptr(order), nat.ptr(tile_code), nat.sz(n), C.c_int(k), C.c_int(cols), C.c_int(v),
             C.c_int(sched.tile_rows), C.c_int(sched.tile_cols), C.c_int(sched.slab_bytes), C.c_int(splitk),
             nat.ptr(scratch), nat.ptr(out), nat.stream()))
-        nat.mark("gather_gemm_fwd" if mode == 0 else "gather_gemm_dgrad", "stop")
+        nat.mark(name, "stop")
     return out
+
+
+def _stream_fits(n: int, row_bytes: int) -> bool:
+    """The streaming kernel addresses its operands with 32-bit byte offsets."""
+    return n * row_bytes <= 0xFF000000 and n * 8 <= 0xFF000000 and n * 27 * 4 * 2 <= 0xFF000000
 
 
 def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int) -> torch.Tensor:
