@@ -8,18 +8,20 @@
 //    workgroup g of G -- and treats all their (offset, K-slab) steps as ONE stream: the loads of the next item's first
 //    steps are in flight while the last steps of the current item are multiplied and its output tile is written, so
 //    neither the start-up latency of a tile nor its epilogue leaves the memory pipeline empty.
+//  * The wavefronts are specialised.  WAVES_M x WAVES_N of them only multiply (LDS fragment reads + MFMA) and write
+//    the output tiles; kLoaders more (one per SIMD) only enqueue loads.  Issuing a vector-memory instruction blocks
+//    its wavefront while the address pipeline is busy, and the loads of a step keep that pipeline busy for about as
+//    long as its MFMAs take -- in separate wavefronts the two run side by side instead of one after the other.
 //  * The per-tile neighbor indices come from the gather plan (fgx_gather_plan_fill): for every tile and every offset
 //    present in it, the tile's source rows as one contiguous run.  An index column is therefore one small contiguous
-//    load, fetched two offsets ahead of the rows that need it.
-//  * Every vector-memory load is a buffer load that writes straight into LDS (lane i deposits 16 bytes at LDS base
-//    + 16 * i).  A missing neighbor is an out-of-range buffer offset, which the hardware answers with zeros; the
-//    per-lane address of a row is a 32-bit offset computed once per offset and reused for all its K-slabs through the
-//    scalar offset operand, and the weight-panel and index loads use lane-constant offsets, so the steady state
-//    spends almost no vector ALU time on addressing.
-//  * No load returns into a register, so the only vector-memory counter traffic in the loop is this kernel's own:
+//    load, fetched kPlanAhead offsets ahead of the rows that need it.
+//  * Every load is a buffer load that writes straight into LDS (lane i deposits 16 bytes at LDS base + 16 * i).  A
+//    missing neighbor is an out-of-range buffer offset, which the hardware answers with zeros; the per-lane address
+//    of a row is a 32-bit offset computed once per offset and reused for all its K-slabs through the scalar offset
+//    operand, and the weight-panel and index loads use lane-constant offsets.
+//  * No load returns into a register, so a loader's vector-memory counter sees only its own loads in issue order:
 //    "the rows of step c have landed" is s_waitcnt vmcnt(number of loads this wavefront issued in the last
 //    iteration), chosen among a few immediates by a scalar branch, followed by one workgroup barrier per step.
-//    Output stores also count; they only make that wait stricter.
 //
 // Stage layout, swizzle, MFMA fragment mapping and the epilogue through LDS are those of the tiled kernel.  The
 // output tile is staged in the ring stage that was multiplied last (free until the next enqueue targets it).
@@ -29,9 +31,10 @@ namespace fgx {
 namespace {
 
 constexpr int kPlanSlots = 4;        // index ring depth
-constexpr int kPlanAhead = 2;        // the index stream runs this many offsets ahead of the row stream
+constexpr int kPlanAhead = 3;        // the index stream runs this many offsets ahead of the row stream
 constexpr uint32_t kOobOffset = 0xFF000000u;   // buffer offset no source tensor reaches: the load returns zeros
 constexpr int kStreamStages = 3;
+constexpr int kLoaders = 4;          // loader wavefronts per workgroup (one per SIMD)
 
 using rsrc_t = __amdgpu_buffer_rsrc_t;
 
@@ -44,15 +47,16 @@ struct StreamCfg {
     using T = typename Tag::type;
     static constexpr int S = kStreamStages;
     static constexpr int ES = (int)sizeof(T);
-    static constexpr int NW = WAVES_M * WAVES_N;
-    static constexpr int NT = 64 * NW;
+    static constexpr int NW = WAVES_M * WAVES_N;               // multiplying wavefronts
+    static constexpr int NL = kLoaders;
+    static constexpr int NT = 64 * (NW + NL);
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     static constexpr int TM = WM / 32, TN = WN / 32;
     static constexpr int SLAB = CH * 16;
     static constexpr int SK = SLAB / ES;
     static constexpr int ROWS_PER_INST = 64 / CH;
-    static constexpr int A_PER = BM / ROWS_PER_INST / NW, B_PER = BN / ROWS_PER_INST / NW;
-    static constexpr int LPS = A_PER + B_PER;                  // row loads per wavefront and step
+    static constexpr int A_PER = BM / ROWS_PER_INST / NL, B_PER = BN / ROWS_PER_INST / NL;
+    static constexpr int LPS = A_PER + B_PER;                  // row loads per loader and step
     static constexpr int IDX_INST = BM / 64;                   // wave-wide dword loads per index column
     static constexpr int OROW_INST = (WM + 63) / 64;           // wave-wide dword loads for a wave tile's output rows
     static constexpr int STAGE_BYTES = (BM + BN) * SLAB;
@@ -61,33 +65,14 @@ struct StreamCfg {
     static constexpr int BAND_ROWS = NW * 32 * OUT_PITCH <= (BM + BN) * SLAB ? 32 : 16;   // rows staged per epilogue pass
     static constexpr int OUT_BAND_BYTES = BAND_ROWS * OUT_PITCH;
     static constexpr int OROW_BYTES = 2 * NW * OROW_INST * 256;
-    static constexpr int MAX_OPS = LPS + 1 + OROW_INST;        // most loads a wavefront issues in one iteration
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
-    static_assert(BM % (ROWS_PER_INST * NW) == 0 && BN % (ROWS_PER_INST * NW) == 0, "every wavefront issues the same row loads");
-    static_assert(BM % 64 == 0 && IDX_INST <= NW, "index column must be whole wave-wide loads, one per wavefront");
+    static_assert(BM % (ROWS_PER_INST * NL) == 0 && BN % (ROWS_PER_INST * NL) == 0, "every loader issues the same row loads");
+    static_assert(BM % 64 == 0 && IDX_INST <= NL, "index column must be whole wave-wide loads, one per loader");
     static_assert(NW * OUT_BAND_BYTES <= STAGE_BYTES, "the output bands must fit one ring stage");
-    static_assert(MAX_OPS < 64, "vmcnt is a 6-bit counter");
+    static_assert(LPS + 1 < 64, "vmcnt is a 6-bit counter");
     static_assert(CH == 4 || CH == 8, "slab must be 64 or 128 bytes");
     static constexpr size_t fixed_lds = (size_t)S * STAGE_BYTES + (size_t)kPlanSlots * IDX_SLOT_BYTES + OROW_BYTES;
 };
-
-// wait until at most `n` of this wavefront's vector-memory operations are outstanding.  n is wave-uniform; the
-// immediate used is the largest of 0, LPS, LPS + 1, ..., LPS + EXTRA that does not exceed n (smaller is merely stricter)
-template <int LPS, int K>
-struct WaitChain {
-    static __device__ __forceinline__ void run(int n) {
-        if (n >= LPS + K) wait_vmcnt<LPS + K>();
-        else WaitChain<LPS, K - 1>::run(n);
-    }
-};
-template <int LPS>
-struct WaitChain<LPS, -1> {
-    static __device__ __forceinline__ void run(int) { wait_vmcnt<0>(); }
-};
-template <int LPS, int EXTRA>
-__device__ __forceinline__ void wait_outstanding(int n) {
-    WaitChain<LPS, EXTRA>::run(n);
-}
 
 __device__ __forceinline__ void wg_barrier() {
     asm volatile("" ::: "memory");
@@ -96,10 +81,10 @@ __device__ __forceinline__ void wg_barrier() {
 }
 
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int CH>
-__global__ void __launch_bounds__(64 * WAVES_M * WAVES_N)
+__global__ void __launch_bounds__(64 * (WAVES_M * WAVES_N + kLoaders))
 gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const typename Tag::type* __restrict__ panel,
                           const typename Tag::type* __restrict__ bias, const int64_t* __restrict__ order,
-                          const int32_t* __restrict__ plan_seg, const int32_t* __restrict__ plan_v,
+                          const int32_t* __restrict__ plan_seg, const int32_t* __restrict__ tile_code,
                           const uint32_t* __restrict__ plan_idx, uint32_t n, int K, int cols, int cols_pad,
                           unsigned row_tiles, unsigned col_tiles, uint32_t src_bytes, uint32_t panel_bytes,
                           uint32_t plan_bytes, typename Tag::type* __restrict__ out) {
@@ -116,7 +101,10 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+    const bool loader = wave >= C::NW;                          // wave-uniform role
+    const int lw = loader ? wave - C::NW : 0;                   // loader number
+    const int mw = loader ? 0 : wave;                           // multiplier number
+    const int wave_m = mw / WAVES_N, wave_n = mw % WAVES_N;
     const int g = lane >> 5, l32 = lane & 31;
 
     const unsigned total_items = row_tiles * col_tiles;
@@ -125,6 +113,7 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     const int slabs = (K + C::SK - 1) / C::SK;
     const uint32_t row_bytes = (uint32_t)K * sizeof(T);
     const bool ragged = (row_bytes % kSlabBytes) != 0;
+    if (blockIdx.x >= total_items) return;                      // whole workgroup
 
     const rsrc_t src_rs = make_rsrc(src, src_bytes);
     const rsrc_t panel_rs = make_rsrc(panel, panel_bytes);
@@ -133,32 +122,34 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
 
     for (int c = tid; c < cols_pad; c += C::NT) bias_lds[c] = (bias != nullptr && c < cols) ? to_float<T>(bias[c]) : 0.f;
 
-    // ---- lane constants ----
+    // =================================================================================================
+    // Loader state (meaningful in loader wavefronts only)
+    // =================================================================================================
     const int sub_row = lane / kChunks, pch = lane % kChunks;
     int a_row[C::A_PER];
     uint32_t a_choff[C::A_PER], a_voff[C::A_PER], b_voff[C::B_PER];
 #pragma unroll
     for (int i = 0; i < C::A_PER; ++i) {
-        a_row[i] = (i * C::NW + wave) * C::ROWS_PER_INST + sub_row;
+        a_row[i] = (i * C::NL + lw) * C::ROWS_PER_INST + sub_row;
         a_choff[i] = (uint32_t)((pch ^ swz_key<CH>(a_row[i])) << 4);
         a_voff[i] = kOobOffset;
     }
 #pragma unroll
     for (int i = 0; i < C::B_PER; ++i) {
-        const int col = (i * C::NW + wave) * C::ROWS_PER_INST + sub_row;
+        const int col = (i * C::NL + lw) * C::ROWS_PER_INST + sub_row;
         b_voff[i] = (uint32_t)(col * kSlabBytes + ((pch ^ swz_key<CH>(col)) << 4));
     }
-    const uint32_t idx_voff = (uint32_t)((wave * 64 + lane) * 4);           // used by wavefronts < IDX_INST only
-    const bool idx_wave = wave < C::IDX_INST;
+    const uint32_t idx_voff = (uint32_t)((lw * 64 + lane) * 4);             // used by loaders < IDX_INST only
+    const bool idx_wave = loader && lw < C::IDX_INST;
 
     // ---- the index stream: walks the plan rows of this workgroup's items, kPlanAhead offsets ahead of the rows ----
+    // The offsets of a tile are the set bits of its code (a tile without any owns one all-missing plan row, walked as
+    // offset 0), so one scalar load per item feeds the whole walk.
     unsigned f_it = blockIdx.x, f_t = blockIdx.x / col_tiles, f_ct = blockIdx.x % col_tiles;
-    bool f_live = f_it < total_items;
-    int f_pos = 0, f_end = 0, f_ring = 0;
-    if (f_live) {
-        f_pos = plan_seg[f_t];
-        f_end = plan_seg[f_t + 1];
-    }
+    bool f_live = true;
+    int f_pos = plan_seg[f_t], f_ring = 0;
+    uint32_t f_code = (uint32_t)tile_code[f_t];
+    f_code = f_code ? f_code : 1u;
     // queue of offsets the row stream has not started yet (head first)
     int q_v[kPlanAhead], q_ct[kPlanAhead];
     bool q_live[kPlanAhead];
@@ -167,16 +158,18 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
         v = 0;
         ct = 0;
         if (!f_live) return 0;
-        v = plan_v[f_pos];
+        v = __builtin_ctz(f_code);
+        f_code &= f_code - 1;
         ct = (int)f_ct;
         int ops = 0;
         if (idx_wave) {
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(plan_rs, FGX_LDS_PTR(idx_ring + f_ring * BM + wave * 64), 4, idx_voff,
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(plan_rs, FGX_LDS_PTR(idx_ring + f_ring * BM + lw * 64), 4, idx_voff,
                                                      (uint32_t)f_pos * (uint32_t)(BM * 4), 0, 0);
             ops = 1;
         }
         f_ring = (f_ring + 1) & (kPlanSlots - 1);
-        if (++f_pos == f_end) {
+        ++f_pos;
+        if (f_code == 0) {
             f_it += G;
             f_live = f_it < total_items;
             if (f_live) {
@@ -187,95 +180,87 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
                     ++f_t;
                 }
                 f_pos = plan_seg[f_t];
-                f_end = plan_seg[f_t + 1];
+                f_code = (uint32_t)tile_code[f_t];
+                f_code = f_code ? f_code : 1u;
             }
         }
         return ops;
     };
 
     // ---- the row stream: S-1 steps ahead of the multiply stream ----
-    bool p_done = false;
+    // slot_begin() makes the next offset current (per-lane row offsets from its index column, panel offset) and
+    // starts the index load of the offset kPlanAhead further on; issue_step() enqueues the loads of the current step
+    // and moves on by one K-slab.
+    bool p_ready = false;
     int p_slab = 0, p_ring = 0, p_stage = 0;
-    uint32_t b_soff = 0;
+    uint32_t a_soff = 0, b_soff = 0;
     const uint32_t b_slab_stride = (uint32_t)cols_pad * kSlabBytes;
-    auto produce = [&]() -> int {
-        if (p_done) return 0;
-        int ops = 0;
-        if (p_slab == 0) {
-            if (!q_live[0]) {
-                p_done = true;
-                return 0;
-            }
-            const int v = q_v[0], ct = q_ct[0];
+    auto slot_begin = [&]() -> int {
+        p_ready = q_live[0];
+        if (!p_ready) return 0;
+        const int v = q_v[0], ct = q_ct[0];
 #pragma unroll
-            for (int i = 0; i + 1 < kPlanAhead; ++i) {
-                q_v[i] = q_v[i + 1];
-                q_ct[i] = q_ct[i + 1];
-                q_live[i] = q_live[i + 1];
-            }
-            const uint32_t* slot = idx_ring + p_ring * BM;
-#pragma unroll
-            for (int i = 0; i < C::A_PER; ++i) {
-                const uint32_t m = slot[a_row[i]];
-                a_voff[i] = m == FGX_EMPTY32 ? kOobOffset : m * row_bytes + a_choff[i];
-            }
-            b_soff = ((uint32_t)(v * slabs) * (uint32_t)cols_pad + (uint32_t)(ct * BN)) * kSlabBytes;
-            ops += fetch_slot(q_v[kPlanAhead - 1], q_ct[kPlanAhead - 1], q_live[kPlanAhead - 1]);
+        for (int i = 0; i + 1 < kPlanAhead; ++i) {
+            q_v[i] = q_v[i + 1];
+            q_ct[i] = q_ct[i + 1];
+            q_live[i] = q_live[i + 1];
         }
+        const uint32_t* slot = idx_ring + p_ring * BM;
+        p_ring = (p_ring + 1) & (kPlanSlots - 1);
+#pragma unroll
+        for (int i = 0; i < C::A_PER; ++i) {
+            const uint32_t m = slot[a_row[i]];
+            a_voff[i] = m == FGX_EMPTY32 ? kOobOffset : m * row_bytes + a_choff[i];
+        }
+        p_slab = 0;
+        a_soff = 0;
+        b_soff = ((uint32_t)(v * slabs) * (uint32_t)cols_pad + (uint32_t)(ct * BN)) * kSlabBytes;
+        return fetch_slot(q_v[kPlanAhead - 1], q_ct[kPlanAhead - 1], q_live[kPlanAhead - 1]);
+    };
+    auto issue_step = [&]() -> int {                     // returns the loads this wavefront issued
+        if (!p_ready) return 0;
         unsigned char* stage = ring + p_stage * C::STAGE_BYTES;
-        const uint32_t a_soff = (uint32_t)(p_slab * kSlabBytes);
         const bool tail = ragged && p_slab == slabs - 1;     // wave-uniform
 #pragma unroll
         for (int i = 0; i < C::A_PER; ++i) {
             uint32_t vo = a_voff[i];
             if (tail) vo = a_soff + a_choff[i] < row_bytes ? vo : kOobOffset;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(src_rs, FGX_LDS_PTR(stage + (i * C::NW + wave) * 1024), 16, vo, a_soff, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(src_rs, FGX_LDS_PTR(stage + (i * C::NL + lw) * 1024), 16, vo, a_soff, 0, 0);
         }
         unsigned char* stage_b = stage + BM * kSlabBytes;
 #pragma unroll
         for (int i = 0; i < C::B_PER; ++i) {
             const uint32_t vo = b_voff[i];
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(panel_rs, FGX_LDS_PTR(stage_b + (i * C::NW + wave) * 1024), 16, vo, b_soff, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(panel_rs, FGX_LDS_PTR(stage_b + (i * C::NL + lw) * 1024), 16, vo, b_soff, 0, 0);
         }
-        ops += C::LPS;
+        int ops = C::LPS;
+        a_soff += kSlabBytes;
         b_soff += b_slab_stride;
         p_stage = p_stage + 1 == S ? 0 : p_stage + 1;
-        if (++p_slab == slabs) {
-            p_slab = 0;
-            p_ring = (p_ring + 1) & (kPlanSlots - 1);
-        }
+        if (++p_slab == slabs) ops += slot_begin();
         return ops;
     };
+    // at most `n` of this loader's loads may still be outstanding; n is 0, LPS or LPS + 1
+    auto wait_loads = [&](int n) {
+        if (n > C::LPS) wait_vmcnt<C::LPS + 1>();
+        else if (n == C::LPS) wait_vmcnt<C::LPS>();
+        else wait_vmcnt<0>();
+    };
 
-    // ---- output rows of an item's wave tile: one (or two) small loads into this wavefront's own LDS area ----
+    // =================================================================================================
+    // Multiplier state
+    // =================================================================================================
+    // output rows of an item's wave tile: one (or two) small loads into this wavefront's own LDS area
     auto fetch_orow = [&](unsigned t, int parity) {
 #pragma unroll
         for (int j = 0; j < C::OROW_INST; ++j) {
             const int r = j * 64 + lane;
             const uint32_t row = t * (uint32_t)BM + (uint32_t)(wave_m * C::WM + r);
             const uint32_t vo = (r < C::WM && row < n) ? row * 8u : kOobOffset;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(order_rs, FGX_LDS_PTR(orow_lds + ((parity * C::NW + wave) * C::OROW_INST + j) * 64),
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(order_rs, FGX_LDS_PTR(orow_lds + ((parity * C::NW + mw) * C::OROW_INST + j) * 64),
                                                      4, vo, 0, 0, 0);
         }
     };
-
-    // ---- multiply stream state ----
-    unsigned c_it = blockIdx.x, c_t = blockIdx.x / col_tiles, c_ct = blockIdx.x % col_tiles;
-    if (c_it >= total_items) return;                                   // whole workgroup
-    int c_lo = plan_seg[c_t], c_hi = plan_seg[c_t + 1];
-
-    // ---- prologue ----
-#pragma unroll
-    for (int i = 0; i < kPlanAhead; ++i) (void)fetch_slot(q_v[i], q_ct[i], q_live[i]);
-    fetch_orow(c_t, 0);
-    int ops_prev = 0;
-#pragma unroll
-    for (int s = 0; s < S - 1; ++s) {
-        wait_vmcnt<0>();
-        __syncthreads();      // also publishes bias_lds
-        ops_prev = produce();
-    }
-
     int a_frag[kChunks / 2][C::TM], b_frag[kChunks / 2][C::TN];   // byte offsets of this lane's fragments in a stage
 #pragma unroll
     for (int kk = 0; kk < kChunks / 2; ++kk) {
@@ -288,65 +273,84 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     constexpr int ROWS_PER_PASS = 64 / PIECES;
     const bool vec_ok = (cols * C::ES) % 16 == 0;             // output rows start on 16-byte boundaries
 
+    // ---- item walk shared by both roles (same barriers in the same order) ----
+    unsigned c_it = blockIdx.x, c_t = blockIdx.x / col_tiles, c_ct = blockIdx.x % col_tiles;
+    int c_slots = __popc((uint32_t)tile_code[c_t]);
+
+    // ---- prologue ----
+    int ops_prev = 0;
+    if (loader) {
+#pragma unroll
+        for (int i = 0; i < kPlanAhead; ++i) (void)fetch_slot(q_v[i], q_ct[i], q_live[i]);
+    } else {
+        fetch_orow(c_t, 0);
+    }
+    wait_vmcnt<0>();
+    __syncthreads();          // index columns landed; also publishes bias_lds
+    if (loader) (void)slot_begin();
+#pragma unroll
+    for (int s = 0; s < S - 1; ++s) {
+        wait_vmcnt<0>();
+        __syncthreads();
+        if (loader) ops_prev = issue_step();
+    }
+
     int cur_stage = 0, parity = 0;
     while (true) {
-        const int nsteps = (c_hi - c_lo) * slabs;
-        // the item after this one (its output rows are fetched now, its plan bounds are read now)
+        const int nsteps = (c_slots > 0 ? c_slots : 1) * slabs;
+        // the item after this one (its output rows are fetched now, its size is read now)
         unsigned n_it = c_it + G, n_t = c_t + dt, n_ct = c_ct + dct;
         if (n_ct >= col_tiles) {
             n_ct -= col_tiles;
             ++n_t;
         }
         const bool has_next = n_it < total_items;
-        int n_lo = 0, n_hi = 0;
-        if (has_next) {
-            n_lo = plan_seg[n_t];
-            n_hi = plan_seg[n_t + 1];
-        }
+        int n_slots = 0;
+        if (has_next) n_slots = __popc((uint32_t)tile_code[n_t]);
 
-        f32x16 acc[C::TM][C::TN];
-#pragma unroll
-        for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-            for (int j = 0; j < C::TN; ++j)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-
-        for (int s = 0; s < nsteps; ++s) {
-            // everything this wavefront issued before its previous iteration has landed: the rows of this step among it
-            wait_outstanding<C::LPS, 1 + C::OROW_INST>(ops_prev);
-            wg_barrier();                  // ... and everybody else's; the stage multiplied in the previous step is free
-            int ops = produce();
-            if (s == 0 && has_next) {
-                fetch_orow(n_t, parity ^ 1);
-                ops += C::OROW_INST;
+        if (loader) {
+            for (int s = 0; s < nsteps; ++s) {
+                // everything this loader issued before its previous iteration has landed: its share of this step's rows
+                wait_loads(ops_prev);
+                wg_barrier();              // ... and everybody else's; the stage multiplied in the previous step is free
+                ops_prev = issue_step();
             }
-            ops_prev = ops;
-            const unsigned char* cur = ring + cur_stage * C::STAGE_BYTES;
-            cur_stage = cur_stage + 1 == S ? 0 : cur_stage + 1;
-            u32x4 af[kChunks / 2][C::TM], bf[kChunks / 2][C::TN];
+            wg_barrier();                  // the multipliers' "done reading the last stage"
+        } else {
+            f32x16 acc[C::TM][C::TN];
 #pragma unroll
-            for (int kk = 0; kk < kChunks / 2; ++kk) {
+            for (int i = 0; i < C::TM; ++i)
 #pragma unroll
-                for (int i = 0; i < C::TM; ++i) af[kk][i] = *(const u32x4*)(cur + a_frag[kk][i]);
+                for (int j = 0; j < C::TN; ++j)
 #pragma unroll
-                for (int j = 0; j < C::TN; ++j) bf[kk][j] = *(const u32x4*)(cur + b_frag[kk][j]);
+                    for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+            if (has_next) fetch_orow(n_t, parity ^ 1);
+            for (int s = 0; s < nsteps; ++s) {
+                wg_barrier();              // the loaders saw this step's rows land
+                const unsigned char* cur = ring + cur_stage * C::STAGE_BYTES;
+                cur_stage = cur_stage + 1 == S ? 0 : cur_stage + 1;
+                u32x4 af[kChunks / 2][C::TM], bf[kChunks / 2][C::TN];
+#pragma unroll
+                for (int kk = 0; kk < kChunks / 2; ++kk) {
+#pragma unroll
+                    for (int i = 0; i < C::TM; ++i) af[kk][i] = *(const u32x4*)(cur + a_frag[kk][i]);
+#pragma unroll
+                    for (int j = 0; j < C::TN; ++j) bf[kk][j] = *(const u32x4*)(cur + b_frag[kk][j]);
+                }
+#pragma unroll
+                for (int kk = 0; kk < kChunks / 2; ++kk)
+#pragma unroll
+                    for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+                        for (int j = 0; j < C::TN; ++j) mma<Tag>(acc[i][j], af[kk][i], bf[kk][j]);
             }
-#pragma unroll
-            for (int kk = 0; kk < kChunks / 2; ++kk)
-#pragma unroll
-                for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < C::TN; ++j) mma<Tag>(acc[i][j], af[kk][i], bf[kk][j]);
-        }
 
-        // ---- epilogue: 32x32 accumulator tile: element e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32 ----
-        wait_outstanding<C::LPS, 1 + C::OROW_INST>(ops_prev);   // this item's output rows have landed (fetched an item ago)
-        wg_barrier();                                           // everybody is done reading the last stage
-        {
+            // ---- epilogue: 32x32 accumulator tile: element e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32
+            wait_vmcnt<0>();               // this item's output rows (fetched an item ago) and older stores
+            wg_barrier();                  // everybody is done reading the last stage
             const int last = cur_stage == 0 ? S - 1 : cur_stage - 1;
-            unsigned char* band = ring + last * C::STAGE_BYTES + wave * C::OUT_BAND_BYTES;
-            const uint32_t* my_orow = orow_lds + (parity * C::NW + wave) * C::OROW_INST * 64;
+            unsigned char* band = ring + last * C::STAGE_BYTES + mw * C::OUT_BAND_BYTES;
+            const uint32_t* my_orow = orow_lds + (parity * C::NW + mw) * C::OROW_INST * 64;
             const int col0 = (int)c_ct * BN + wave_n * C::WN;
             float bv[C::TN];
 #pragma unroll
@@ -385,8 +389,7 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
         c_it = n_it;
         c_t = n_t;
         c_ct = n_ct;
-        c_lo = n_lo;
-        c_hi = n_hi;
+        c_slots = n_slots;
         parity ^= 1;
     }
     wait_vmcnt<0>();
@@ -394,7 +397,7 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
 
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int CH>
 int launch_stream(const void* src, const void* panel, const void* bias, const int64_t* order, const int32_t* plan_seg,
-                  const int32_t* plan_v, const uint32_t* plan_idx, size_t plan_rows, size_t n, int K, int cols,
+                  const int32_t* tile_code, const uint32_t* plan_idx, size_t plan_rows, size_t n, int K, int cols,
                   int cols_pad, size_t panel_bytes, int max_groups, void* out, hipStream_t s) {
     using C = StreamCfg<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
     using T = typename Tag::type;
@@ -412,7 +415,7 @@ int launch_stream(const void* src, const void* panel, const void* bias, const in
     const unsigned row_tiles = cdiv(n, BM), col_tiles = cdiv(cols, BN);
     const size_t total = (size_t)row_tiles * col_tiles;
     unsigned groups = (unsigned)(total < (size_t)max_groups ? total : (size_t)max_groups);
-    kern<<<groups, C::NT, lds, s>>>((const T*)src, (const T*)panel, (const T*)bias, order, plan_seg, plan_v, plan_idx,
+    kern<<<groups, C::NT, lds, s>>>((const T*)src, (const T*)panel, (const T*)bias, order, plan_seg, tile_code, plan_idx,
                                     (uint32_t)n, K, cols, cols_pad, row_tiles, col_tiles,
                                     (uint32_t)(n * (size_t)K * sizeof(T)), (uint32_t)panel_bytes,
                                     (uint32_t)(plan_rows * BM * 4), (T*)out);
@@ -422,12 +425,12 @@ int launch_stream(const void* src, const void* panel, const void* bias, const in
 
 template <typename Tag>
 int dispatch_stream(int tile_rows, int tile_cols, int slab_bytes, const void* src, const void* panel, const void* bias,
-                    const int64_t* order, const int32_t* plan_seg, const int32_t* plan_v, const uint32_t* plan_idx,
+                    const int64_t* order, const int32_t* plan_seg, const int32_t* tile_code, const uint32_t* plan_idx,
                     size_t plan_rows, size_t n, int K, int cols, int cols_pad, size_t panel_bytes, int max_groups,
                     void* out, hipStream_t s) {
 #define FGX_STREAM_TILE(BM, BN, WMv, WNv, CHv)                                                                          \
     if (tile_rows == BM && tile_cols == BN && slab_bytes == CHv * 16)                                                   \
-        return launch_stream<Tag, BM, BN, WMv, WNv, CHv>(src, panel, bias, order, plan_seg, plan_v, plan_idx, plan_rows, \
+        return launch_stream<Tag, BM, BN, WMv, WNv, CHv>(src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_rows, \
                                                          n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
     FGX_STREAM_TILE(256, 128, 4, 2, 8)
 #undef FGX_STREAM_TILE
@@ -441,7 +444,7 @@ int dispatch_stream(int tile_rows, int tile_cols, int slab_bytes, const void* sr
 using namespace fgx;
 
 extern "C" int fgx_conv_gather_gemm_stream(int dtype, const void* src, const void* panel, const void* bias,
-                                           const int64_t* order, const int32_t* plan_seg, const int32_t* plan_v,
+                                           const int64_t* order, const int32_t* tile_code, const int32_t* plan_seg,
                                            const uint32_t* plan_idx, size_t plan_rows, size_t n, int K, int cols, int V,
                                            int tile_rows, int tile_cols, int slab_bytes, int max_groups, void* out,
                                            fgx_stream_t stream) {
@@ -450,7 +453,7 @@ extern "C" int fgx_conv_gather_gemm_stream(int dtype, const void* src, const voi
     if (n == 0) return FGX_OK;
     const int es = dtype == FGX_F32 ? 4 : 2;
     FGX_CHECK_ARG(((size_t)K * es) % 16 == 0, "fgx_conv_gather_gemm_stream: source row of %d elements is not a multiple of 16 bytes", K);
-    FGX_CHECK_ARG(src && panel && order && plan_seg && plan_v && plan_idx && out, "fgx_conv_gather_gemm_stream: null buffer");
+    FGX_CHECK_ARG(src && panel && order && plan_seg && tile_code && plan_idx && out, "fgx_conv_gather_gemm_stream: null buffer");
     FGX_CHECK_ARG((((uintptr_t)src | (uintptr_t)panel | (uintptr_t)plan_idx) & 15) == 0,
                   "fgx_conv_gather_gemm_stream: src, panel and plan_idx must be 16-byte aligned");
     FGX_CHECK_ARG(tile_rows > 0 && tile_cols > 0 && (slab_bytes == 64 || slab_bytes == 128), "fgx_conv_gather_gemm_stream: bad schedule");
@@ -471,8 +474,8 @@ extern "C" int fgx_conv_gather_gemm_stream(int dtype, const void* src, const voi
     }
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
-        case FGX_F16: return dispatch_stream<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, plan_v, plan_idx, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
-        case FGX_BF16: return dispatch_stream<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, plan_v, plan_idx, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
-        default: return dispatch_stream<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, plan_v, plan_idx, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
+        case FGX_F16: return dispatch_stream<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
+        case FGX_BF16: return dispatch_stream<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
+        default: return dispatch_stream<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
     }
 }

@@ -219,18 +219,17 @@ __global__ void __launch_bounds__(kBlock) plan_count_kernel(const int32_t* __res
     cnt[t] = (uint32_t)(c > 0 ? c : 1);
 }
 
-// One workgroup per tile: plan_v[seg[t] + k] = k-th offset present in the tile,
-// plan_idx[seg[t] + k][r] = map[order[t * tile_rows + r]][that offset] (EMPTY for rows past the end).
+// One workgroup per tile: plan_idx[seg[t] + k][r] = map[order[t * tile_rows + r]][k-th offset present in the tile]
+// (EMPTY for rows past the end).
 __global__ void __launch_bounds__(kBlock) plan_fill_kernel(const uint32_t* __restrict__ map,
                                                            const int64_t* __restrict__ order,
                                                            const int32_t* __restrict__ tile_code,
                                                            const int32_t* __restrict__ seg, size_t n, int V, int tile_rows,
-                                                           int32_t* __restrict__ plan_v, uint32_t* __restrict__ plan_idx) {
+                                                           uint32_t* __restrict__ plan_idx) {
     const size_t t = blockIdx.x;
     uint32_t code = (uint32_t)tile_code[t];
     size_t slot = (size_t)seg[t];
     if (code == 0) {
-        if (threadIdx.x == 0) plan_v[slot] = 0;
         for (int r = threadIdx.x; r < tile_rows; r += kBlock) plan_idx[slot * tile_rows + r] = FGX_EMPTY32;
         return;
     }
@@ -243,7 +242,6 @@ __global__ void __launch_bounds__(kBlock) plan_fill_kernel(const uint32_t* __res
         while (c) {
             const int v = __ffs((int)c) - 1;
             c &= c - 1;
-            if (r0 == 0 && threadIdx.x == 0) plan_v[s] = v;
             if (r < tile_rows) plan_idx[s * tile_rows + r] = mrow ? mrow[v] : FGX_EMPTY32;
             ++s;
         }
@@ -463,14 +461,14 @@ int fgx_gather_plan_count(const int32_t* tile_code, size_t num_tiles, int32_t* p
 }
 
 int fgx_gather_plan_fill(const uint32_t* map, const int64_t* order, const int32_t* tile_code, const int32_t* plan_seg,
-                         size_t n, int V, int tile_rows, int32_t* plan_v, uint32_t* plan_idx, fgx_stream_t stream) {
+                         size_t n, int V, int tile_rows, uint32_t* plan_idx, fgx_stream_t stream) {
     FGX_CHECK_ARG(tile_rows >= 1 && V >= 1 && V <= 32, "fgx_gather_plan_fill: bad shape tile_rows=%d V=%d", tile_rows, V);
     if (n == 0) return FGX_OK;
-    FGX_CHECK_ARG(map && order && tile_code && plan_seg && plan_v && plan_idx, "fgx_gather_plan_fill: null buffer");
+    FGX_CHECK_ARG(map && order && tile_code && plan_seg && plan_idx, "fgx_gather_plan_fill: null buffer");
     const size_t num_tiles = (n + tile_rows - 1) / tile_rows;
     FGX_CHECK_ARG(num_tiles <= 0x7FFFFFFFu, "fgx_gather_plan_fill: too many tiles");
     plan_fill_kernel<<<(unsigned)num_tiles, kBlock, 0, (hipStream_t)stream>>>(map, order, tile_code, plan_seg, n, V, tile_rows,
-                                                                              plan_v, plan_idx);
+                                                                              plan_idx);
     FGX_CHECK_LAUNCH("fgx_gather_plan_fill");
     return FGX_OK;
 }

@@ -83,8 +83,8 @@ class SubMConv3dNeighborCache:
         return order, getattr(self, key), getattr(self, seg_key)
 
     def _gather_plan(self, block_size: int, private: bool):
-        """(order, plan_seg int32 [nb+1], plan_v int32 [P], plan_idx uint32 [P, block_size]) for the streaming GEMM:
-        per tile and offset present in it, the tile's source rows as one contiguous run.  Built once per tile size
+        """(order, tile_code int32 [nb], plan_seg int32 [nb+1], plan_idx uint32 [P, block_size]) for the streaming
+        GEMM: per tile and offset present in it, the tile's source rows as one contiguous run.  Built once per tile size
         (one 4-byte read-back sizes it) and kept with the cache."""
         order, code, _ = self._tile_tables(block_size, private)
         use_private = private and hasattr(self, "_tile_order")
@@ -101,13 +101,11 @@ class SubMConv3dNeighborCache:
                 nat.check(L.fgx_gather_plan_count(nat.ptr(code), nat.sz(nb), nat.ptr(seg), nat.ptr(ws), nat.sz(ws.numel()),
                                                   nat.stream()))
                 rows = int(seg[-1].item())
-                plan_v = torch.empty((rows,), dtype=torch.int32, device=dev)
                 plan_idx = torch.empty((rows, block_size), dtype=torch.uint32, device=dev)
                 nat.check(L.fgx_gather_plan_fill(nat.ptr(nmap), nat.ptr(order), nat.ptr(code), nat.ptr(seg), nat.sz(n),
-                                                 C.c_int(v), C.c_int(block_size), nat.ptr(plan_v), nat.ptr(plan_idx),
-                                                 nat.stream()))
-            setattr(self, key, (seg, plan_v, plan_idx))
-        return (order,) + getattr(self, key)
+                                                 C.c_int(v), C.c_int(block_size), nat.ptr(plan_idx), nat.stream()))
+            setattr(self, key, (seg, plan_idx))
+        return (order, code) + getattr(self, key)
 
     def compute_kernel_idx(self, block_size: int):
         """Fill `valid_kernel_{B}` / `valid_kernel_seg_{B}` (reference: submanifold_conv3d.py:20-23,
@@ -298,11 +296,11 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
         nat.check(L.fgx_pack_weight(C.c_int(code), C.c_int(mode), nat.ptr(weight_cvk), C.c_int(ci), C.c_int(co), C.c_int(v),
                                     C.c_int(sched.slab_bytes), C.c_int(sched.tile_cols), nat.ptr(panel), nat.stream()))
         if sched.stream and _stream_fits(n, k * src.element_size()):
-            order, plan_seg, plan_v, plan_idx = cache._gather_plan(sched.tile_rows, private)
+            order, tile_code, plan_seg, plan_idx = cache._gather_plan(sched.tile_rows, private)
             nat.mark(name, "start")
             nat.check(L.fgx_conv_gather_gemm_stream(
-                C.c_int(code), nat.ptr(src), nat.ptr(panel), nat.ptr(bias), nat.ptr(order), nat.ptr(plan_seg),
-                nat.ptr(plan_v), nat.ptr(plan_idx), nat.sz(plan_v.shape[0]), nat.sz(n), C.c_int(k), C.c_int(cols), C.c_int(v),
+                C.c_int(code), nat.ptr(src), nat.ptr(panel), nat.ptr(bias), nat.ptr(order), nat.ptr(tile_code),
+                nat.ptr(plan_seg), nat.ptr(plan_idx), nat.sz(plan_idx.shape[0]), nat.sz(n), C.c_int(k), C.c_int(cols), C.c_int(v),
                 C.c_int(sched.tile_rows), C.c_int(sched.tile_cols), C.c_int(sched.slab_bytes), C.c_int(0), nat.ptr(out),
                 nat.stream()))
             nat.mark(name, "stop")

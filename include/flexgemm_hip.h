@@ -179,19 +179,19 @@ int fgx_conv_gather_gemm(int dtype, const void* src, const void* panel, const vo
                          void* scratch, void* out, fgx_stream_t stream);
 
 /* Gather plan of a row order for tiles of `tile_rows` rows: for tile t and the k-th offset v present in it
- * (ascending; a tile whose code is 0 gets one row with every neighbor missing),
- *   plan_v[plan_seg[t] + k] = v,   plan_idx[(plan_seg[t] + k) * tile_rows + r] = map[order[t * tile_rows + r], v]
- * (0xFFFFFFFF for rows past n).  count: plan_seg[num_tiles + 1] <- exclusive offsets, plan_seg[num_tiles] = plan
- * rows; the caller reads that back, allocates plan_v (int32 per plan row) and plan_idx (tile_rows uint32 per plan
- * row, 16-byte aligned) and calls fill.  `tile_code` comes from fgx_tile_codes on the same order and tile size;
- * workspace: fgx_tile_workspace_bytes(num_tiles, 1) bytes, 256-byte aligned.
+ * (the set bits of tile_code[t], ascending; a tile whose code is 0 gets one row with every neighbor missing),
+ *   plan_idx[(plan_seg[t] + k) * tile_rows + r] = map[order[t * tile_rows + r], v]     (0xFFFFFFFF for rows past n).
+ * count: plan_seg[num_tiles + 1] <- exclusive offsets, plan_seg[num_tiles] = plan rows; the caller reads that back,
+ * allocates plan_idx (tile_rows uint32 per plan row, 16-byte aligned) and calls fill.  `tile_code` comes from
+ * fgx_tile_codes on the same order and tile size; workspace: fgx_tile_workspace_bytes(num_tiles, 1) bytes,
+ * 256-byte aligned.
  * Replaces: the neighbor[sorted_idx[rows], v] double gather inside the Triton kernels
  *           (..._fwd_masked_implicit_gemm.py:69-76, ..._bwd_masked_implicit_gemm.py:64-71) by a table built once per
  *           coordinate set. */
 int fgx_gather_plan_count(const int32_t* tile_code, size_t num_tiles, int32_t* plan_seg, void* workspace,
                           size_t workspace_bytes, fgx_stream_t stream);
 int fgx_gather_plan_fill(const uint32_t* map, const int64_t* order, const int32_t* tile_code, const int32_t* plan_seg,
-                         size_t n, int V, int tile_rows, int32_t* plan_v, uint32_t* plan_idx, fgx_stream_t stream);
+                         size_t n, int V, int tile_rows, uint32_t* plan_idx, fgx_stream_t stream);
 
 /* Same result as fgx_conv_gather_gemm (splitk = 1) from the gather plan of `order`, by persistent workgroups that
  * stream all their tiles' (offset, K-slab) steps back to back; meant for voxel counts that give every CU several
@@ -200,7 +200,7 @@ int fgx_gather_plan_fill(const uint32_t* map, const int64_t* order, const int32_
  * schedule -- callers then use fgx_conv_gather_gemm.
  * Replaces: the same reference kernels as fgx_conv_gather_gemm. */
 int fgx_conv_gather_gemm_stream(int dtype, const void* src, const void* panel, const void* bias,
-                                const int64_t* order, const int32_t* plan_seg, const int32_t* plan_v,
+                                const int64_t* order, const int32_t* tile_code, const int32_t* plan_seg,
                                 const uint32_t* plan_idx, size_t plan_rows, size_t n, int K, int cols, int V,
                                 int tile_rows, int tile_cols, int slab_bytes, int max_groups, void* out,
                                 fgx_stream_t stream);
