@@ -114,6 +114,9 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     const uint32_t row_bytes = (uint32_t)K * sizeof(T);
     const bool ragged = (row_bytes % kSlabBytes) != 0;
     if (blockIdx.x >= total_items) return;                      // whole workgroup
+    // Workgroups are dealt round-robin to the 8 XCDs.  Give the workgroups of one XCD neighboring items in every
+    // round (first items (g % 8) * G/8 + g / 8), so that tiles which gather from the same region share an L2.
+    const unsigned first_item = G % kXcds == 0 ? (blockIdx.x % kXcds) * (G / kXcds) + blockIdx.x / kXcds : blockIdx.x;
 
     const rsrc_t src_rs = make_rsrc(src, src_bytes);
     const rsrc_t panel_rs = make_rsrc(panel, panel_bytes);
@@ -145,7 +148,7 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     // ---- the index stream: walks the plan rows of this workgroup's items, kPlanAhead offsets ahead of the rows ----
     // The offsets of a tile are the set bits of its code (a tile without any owns one all-missing plan row, walked as
     // offset 0), so one scalar load per item feeds the whole walk.
-    unsigned f_it = blockIdx.x, f_t = blockIdx.x / col_tiles, f_ct = blockIdx.x % col_tiles;
+    unsigned f_it = first_item, f_t = first_item / col_tiles, f_ct = first_item % col_tiles;
     bool f_live = true;
     int f_pos = plan_seg[f_t], f_ring = 0;
     uint32_t f_code = (uint32_t)tile_code[f_t];
@@ -274,7 +277,7 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     const bool vec_ok = (cols * C::ES) % 16 == 0;             // output rows start on 16-byte boundaries
 
     // ---- item walk shared by both roles (same barriers in the same order) ----
-    unsigned c_it = blockIdx.x, c_t = blockIdx.x / col_tiles, c_ct = blockIdx.x % col_tiles;
+    unsigned c_it = first_item, c_t = first_item / col_tiles, c_ct = first_item % col_tiles;
     int c_slots = __popc((uint32_t)tile_code[c_t]);
 
     // ---- prologue ----

@@ -182,6 +182,69 @@ def test_forced_splitk_matches_unsplit(gpu_device):
     assert eg.max_rel_err(outs[1], outs[0].double()) <= 2e-3 and eg.max_rel_err(outs[2], outs[0].double()) <= 2e-3
 
 
+def _force_schedule(**fields):
+    """Context manager: fwd/dgrad schedules from the table with the given fields overridden."""
+    import contextlib
+    from flexgemm_amd import _native as nat
+
+    @contextlib.contextmanager
+    def cm():
+        real = nat.table_lookup
+
+        def forced(pass_kind, *a):
+            sc = real(pass_kind, *a)
+            if pass_kind != nat.PASS_WGRAD:
+                for k, v in fields.items():
+                    setattr(sc, k, v)
+            return sc
+        nat.table_lookup = forced
+        try:
+            yield
+        finally:
+            nat.table_lookup = real
+    return cm()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("res,ci,co", [(32, 128, 128), (24, 64, 256), (24, 96, 40), (16, 8, 136), (48, 256, 128)])
+def test_streaming_kernel_matches_oracle(gpu_device, dtype, res, ci, co):
+    """Forward, dgrad (and the untouched wgrad) with the persistent streaming GEMM forced: several column tiles,
+    contraction widths that are not whole K-slabs, fewer tiles than workgroups, rows past the last tile."""
+    _say(f"stream res={res} ci={ci} co={co} {dtype}")
+    coords_np = reference_test_shell(res)
+    shape = torch.Size([1, ci, res, res, res])
+    with _force_schedule(tile_rows=256, tile_cols=128, slab_bytes=128, splitk=1, stream=1):
+        _run_and_check(coords_np, shape, ci, co, dtype, gpu_device, seed=21)
+
+
+def test_streaming_kernel_equals_tiled_kernel_bitwise(gpu_device):
+    """Both kernels add the same products in the same order (offsets ascending, K ascending), so their outputs
+    agree bit for bit; isolated voxels (only the centre offset) and a batch dimension are in the mix."""
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    _say("stream vs tiled, bitwise")
+    res, c = 40, 128
+    shell = reference_test_shell(res)
+    rng = np.random.default_rng(5)
+    lonely = np.stack([np.zeros(40, np.int32), rng.integers(0, 4, 40), rng.integers(0, 4, 40), rng.integers(0, 4, 40)], 1).astype(np.int32) * 9
+    lonely = lonely[np.unique(lonely, axis=0, return_index=True)[1]]
+    second = shell.copy()
+    second[:, 0] = 1
+    coords_np = np.concatenate([shell, second, lonely + np.array([2, 0, 0, 0], np.int32)], 0).astype(np.int32)
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    shape = torch.Size([3, c, res, res, res])
+    f, w, b, g = _case(coords_np, c, c, torch.float16, 31)
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+    outs = []
+    for stream in (0, 1):
+        fields = dict(tile_rows=256, tile_cols=128, slab_bytes=128, splitk=1, stream=1) if stream else \
+            dict(tile_rows=128, tile_cols=128, slab_bytes=64, splitk=1, stream=0)
+        with _force_schedule(**fields):
+            o = impl._gather_gemm(f.to(gpu_device), w.to(gpu_device).reshape(c, 27, c), b.to(gpu_device), cache, 0, False)
+            gi = impl._gather_gemm(g.to(gpu_device), w.to(gpu_device).reshape(c, 27, c), None, cache, 1, False)
+        outs.append((o.cpu(), gi.cpu()))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+
+
 @pytest.mark.parametrize("name,res,c", [("cfg2", 64, 256), ("cfg3", 128, 128), ("cfg4", 128, 32), ("cfg5", 32, 1024)])
 def test_scaled_down_benchmark_configs(gpu_device, name, res, c):
     """The benchmark configurations at a resolution the float64 oracle finishes in seconds."""
