@@ -345,29 +345,40 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
 #pragma unroll
                     for (int i = 0; i < C::TM; ++i)
 #pragma unroll
-                        for (int j = 0; j < C::TN; ++j) mma<Tag>(acc[i][j], af[kk][i], bf[kk][j]);
+                        for (int j = 0; j < C::TN; ++j) mma<Tag>(acc[i][j], bf[kk][j], af[kk][i]);   // transposed tile
             }
 
-            // ---- epilogue: 32x32 accumulator tile: element e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32
+            // ---- epilogue.  The MFMAs ran with the operands swapped, so a 32x32 accumulator holds the TRANSPOSED
+            // tile: element e of lane l belongs to output row l%32 and column 8*(e/4) + 4*(l/32) + e%4 -- four
+            // adjacent columns per (lane, e/4), which go to LDS as one 8- or 16-byte store.
             wait_vmcnt<0>();               // this item's output rows (fetched an item ago) and older stores
             wg_barrier();                  // everybody is done reading the last stage
             const int last = cur_stage == 0 ? S - 1 : cur_stage - 1;
             unsigned char* band = ring + last * C::STAGE_BYTES + mw * C::OUT_BAND_BYTES;
             const uint32_t* my_orow = orow_lds + (parity * C::NW + mw) * C::OROW_INST * 64;
             const int col0 = (int)c_ct * BN + wave_n * C::WN;
-            float bv[C::TN];
+            constexpr int HALVES = 32 / C::BAND_ROWS;
 #pragma unroll
-            for (int j = 0; j < C::TN; ++j) bv[j] = bias_lds[col0 + j * 32 + l32];
+            for (int ih = 0; ih < C::TM * HALVES; ++ih) {
+                const int i = ih / HALVES, h = ih % HALVES;      // 32-row tile, half of it
+                if (HALVES == 1 || (l32 >> 4) == h) {
+                    const int r = l32 - h * C::BAND_ROWS;
 #pragma unroll
-            for (int ih = 0; ih < C::TM * (32 / C::BAND_ROWS); ++ih) {
-                const int i = ih / (32 / C::BAND_ROWS), h = ih % (32 / C::BAND_ROWS);   // 32-row tile, half of it
+                    for (int j = 0; j < C::TN; ++j)
 #pragma unroll
-                for (int j = 0; j < C::TN; ++j)
-#pragma unroll
-                    for (int e = h * (C::BAND_ROWS / 2); e < (h + 1) * (C::BAND_ROWS / 2); ++e) {
-                        const int r = (e >> 2) * 8 + g * 4 + (e & 3) - h * C::BAND_ROWS;
-                        *(T*)(band + r * C::OUT_PITCH + (j * 32 + l32) * C::ES) = from_float<T>(acc[i][j][e] + bv[j]);
-                    }
+                        for (int q = 0; q < 4; ++q) {
+                            const int c = j * 32 + q * 8 + g * 4;                   // first of four columns
+                            const f32x4 bv = *(const f32x4*)(bias_lds + col0 + c);
+                            T pk[4];
+                            pk[0] = from_float<T>(acc[i][j][q * 4 + 0] + bv.x);
+                            pk[1] = from_float<T>(acc[i][j][q * 4 + 1] + bv.y);
+                            pk[2] = from_float<T>(acc[i][j][q * 4 + 2] + bv.z);
+                            pk[3] = from_float<T>(acc[i][j][q * 4 + 3] + bv.w);
+                            unsigned char* dstp = band + r * C::OUT_PITCH + c * C::ES;
+                            if constexpr (C::ES == 2) *(uint64_t*)dstp = __builtin_bit_cast(uint64_t, pk);
+                            else *(u32x4*)dstp = __builtin_bit_cast(u32x4, pk);
+                        }
+                }
                 // same wavefront wrote and reads: program order inside the wavefront suffices for LDS
 #pragma unroll
                 for (int pass = 0; pass < C::BAND_ROWS / ROWS_PER_PASS; ++pass) {
