@@ -117,6 +117,9 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     // Workgroups are dealt round-robin to the 8 XCDs.  Give the workgroups of one XCD neighboring items in every
     // round (first items (g % 8) * G/8 + g / 8), so that tiles which gather from the same region share an L2.
     const unsigned first_item = G % kXcds == 0 ? (blockIdx.x % kXcds) * (G / kXcds) + blockIdx.x / kXcds : blockIdx.x;
+    // Items are walked from the LAST tile down: in the mask-sorted order the late tiles carry the most offsets, so the
+    // incomplete final round (total_items % G workgroups get one item more) is made of the cheapest tiles.
+    const unsigned first_rev = total_items - 1 - first_item;
 
     const rsrc_t src_rs = make_rsrc(src, src_bytes);
     const rsrc_t panel_rs = make_rsrc(panel, panel_bytes);
@@ -148,7 +151,7 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     // ---- the index stream: walks the plan rows of this workgroup's items, kPlanAhead offsets ahead of the rows ----
     // The offsets of a tile are the set bits of its code (a tile without any owns one all-missing plan row, walked as
     // offset 0), so one scalar load per item feeds the whole walk.
-    unsigned f_it = first_item, f_t = first_item / col_tiles, f_ct = first_item % col_tiles;
+    unsigned f_it = first_item, f_t = first_rev / col_tiles, f_ct = first_rev % col_tiles;
     bool f_live = true;
     int f_pos = plan_seg[f_t], f_ring = 0;
     uint32_t f_code = (uint32_t)tile_code[f_t];
@@ -176,12 +179,12 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
             f_it += G;
             f_live = f_it < total_items;
             if (f_live) {
-                f_t += dt;
-                f_ct += dct;
-                if (f_ct >= col_tiles) {
-                    f_ct -= col_tiles;
-                    ++f_t;
+                f_t -= dt;
+                if (f_ct < dct) {
+                    f_ct += col_tiles;
+                    --f_t;
                 }
+                f_ct -= dct;
                 f_pos = plan_seg[f_t];
                 f_code = (uint32_t)tile_code[f_t];
                 f_code = f_code ? f_code : 1u;
@@ -277,7 +280,7 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     const bool vec_ok = (cols * C::ES) % 16 == 0;             // output rows start on 16-byte boundaries
 
     // ---- item walk shared by both roles (same barriers in the same order) ----
-    unsigned c_it = first_item, c_t = first_item / col_tiles, c_ct = first_item % col_tiles;
+    unsigned c_it = first_item, c_t = first_rev / col_tiles, c_ct = first_rev % col_tiles;
     int c_slots = __popc((uint32_t)tile_code[c_t]);
 
     // ---- prologue ----
@@ -302,11 +305,12 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     while (true) {
         const int nsteps = (c_slots > 0 ? c_slots : 1) * slabs;
         // the item after this one (its output rows are fetched now, its size is read now)
-        unsigned n_it = c_it + G, n_t = c_t + dt, n_ct = c_ct + dct;
-        if (n_ct >= col_tiles) {
-            n_ct -= col_tiles;
-            ++n_t;
+        unsigned n_it = c_it + G, n_t = c_t - dt, n_ct = c_ct;
+        if (n_ct < dct) {
+            n_ct += col_tiles;
+            --n_t;
         }
+        n_ct -= dct;
         const bool has_next = n_it < total_items;
         int n_slots = 0;
         if (has_next) n_slots = __popc((uint32_t)tile_code[n_t]);

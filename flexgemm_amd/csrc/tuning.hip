@@ -22,7 +22,7 @@ const Entry kTable[] = {
     // pass dtype log2n  Ci    Co    {rows, cols, slab_bytes, splitk, block_rows, stream}
     {0, 2, 19, 128, 128, {256, 128, 128, 1, 0, 1}},
     {1, 2, 19, 128, 128, {256, 128, 128, 1, 0, 1}},
-    {2, 2, 19, 128, 128, {128, 128, 64, 1, 8192, 0}},
+    {2, 2, 19, 128, 128, {128, 128, 64, 1, 8192, 1}},
     {0, 2, 17, 256, 256, {128, 128, 64, 1, 0, 0}},
     {1, 2, 17, 256, 256, {128, 128, 64, 1, 0, 0}},
     {2, 2, 17, 256, 256, {128, 128, 64, 1, 4096, 0}},

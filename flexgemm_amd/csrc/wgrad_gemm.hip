@@ -364,6 +364,354 @@ wgrad_kernel(const typename Tag::type* __restrict__ gout, const typename Tag::ty
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Streaming variant (16-bit types): one persistent workgroup per CU, specialised wavefronts.
+// ------------------------------------------------------------------------------------------------
+// Four wavefronts multiply (2 x 2 over the Co x Ci tile), four more only enqueue loads: issuing a vector-memory
+// instruction blocks its wavefront while the address pipeline is busy, and a step's gathers keep that pipeline busy
+// for longer than its MFMAs take, so the two kinds of work sit in different wavefronts.  A workgroup walks its share
+// of the block-major item list (XCD x takes the x-th eighth, its workgroups interleave inside it) and treats the
+// 64-pair steps of all its items as one stream through a 4-stage row ring and an 8-slot index ring, so the loads of
+// the next item are in flight while the current one finishes.  Loads are buffer loads into LDS: a pair past the end
+// of an item or a column past the tensor is an out-of-range offset and arrives as zeros.  A loader's outstanding-
+// load counter sees only its own loads in issue order: "step c has landed" is s_waitcnt vmcnt(loads issued in the
+// last two iterations).
+constexpr int kWsStages = 4;
+constexpr int kWsIdxSlots = 8;
+constexpr int kWsIdxAhead = 3;       // index loads run this many steps ahead of the row loads (> kWsStages - 2)
+constexpr int kWsLoaders = 4;
+constexpr int kWsPairs = 64;         // pairs per step
+constexpr uint32_t kOobOffset = 0xFF000000u;
+
+using rsrc_t = __amdgpu_buffer_rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), (short)0, (int)bytes, 0x00020000);
+}
+
+template <typename Tag, int BM, int BN>
+struct WStreamCfg {
+    using T = typename Tag::type;
+    static constexpr int ES = (int)sizeof(T);
+    static constexpr int P = kWsPairs, S = kWsStages;
+    static constexpr int NW = 4, NL = kWsLoaders, NT = 64 * (NW + NL);
+    static constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+    static constexpr int ROWB_A = BM * ES, ROWB_B = BN * ES;
+    static constexpr int CH_A = ROWB_A / 16, CH_B = ROWB_B / 16;
+    static constexpr int RPI_A = 64 / CH_A, RPI_B = 64 / CH_B;
+    static constexpr int A_PER = P / RPI_A / NL, B_PER = P / RPI_B / NL;
+    static constexpr int LPS = A_PER + B_PER;
+    static constexpr int A_BYTES = P * ROWB_A, B_BYTES = P * ROWB_B, STAGE_BYTES = A_BYTES + B_BYTES;
+    static constexpr int IDX_SLOT_BYTES = 2 * P * 4;               // sig_o x P | sig_i x P
+    static constexpr size_t lds_bytes = (size_t)S * STAGE_BYTES + (size_t)kWsIdxSlots * IDX_SLOT_BYTES;
+    static_assert(ES == 2, "the streaming kernel handles 16-bit types");
+    static_assert(P == 64, "one wave-wide index load per operand and step");
+    static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
+    static_assert(P % (RPI_A * NL) == 0 && P % (RPI_B * NL) == 0, "every loader issues the same row loads");
+    static_assert(2 * (LPS + 1) < 64, "outstanding loads exceed the vmcnt range");
+    static constexpr int key_a(int row) { return CH_A >= 8 ? 2 * (row & 3) : 0; }
+    static constexpr int key_b(int row) { return CH_B >= 8 ? 2 * (row & 3) : 0; }
+};
+
+// wait until the LDS reads before the newest N have returned; the registers are tied to the wait so that the
+// compiler cannot move their first use above it
+template <int N, int R>
+__device__ __forceinline__ void lds_wait_but(i16x4 (&r)[R]) {
+    static_assert(N >= 0 && N < 16 && R % 4 == 0, "lgkmcnt is a 4-bit counter");
+#if defined(__HIP_DEVICE_COMPILE__)   // (the host pass only needs the kernel's signature; it has no such registers)
+#pragma unroll
+    for (int i = 0; i < R; i += 4)
+        asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(r[i]), "+v"(r[i + 1]), "+v"(r[i + 2]), "+v"(r[i + 3]) : "n"(N));
+#endif
+}
+
+template <typename Tag, int BM, int BN>
+__global__ void __launch_bounds__(64 * (4 + kWsLoaders))
+wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename Tag::type* __restrict__ feats,
+                    const uint32_t* __restrict__ sig_i, const uint32_t* __restrict__ sig_o,
+                    const uint32_t* __restrict__ bounds, int V, int Ci, int Co, unsigned nb, unsigned co_tiles,
+                    unsigned ci_tiles, uint32_t n_pairs, uint32_t gout_bytes, uint32_t feats_bytes,
+                    float* __restrict__ partial) {
+    using C = WStreamCfg<Tag, BM, BN>;
+    constexpr int ES = C::ES, S = C::S, P = C::P;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    unsigned char* ring = lds_raw;                                              // [S][A rows | B rows]
+    uint32_t* idx_ring = (uint32_t*)(ring + S * C::STAGE_BYTES);                // [kWsIdxSlots][o x P | i x P]
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool loader = wave >= C::NW;
+    const int lw = loader ? wave - C::NW : 0, mw = loader ? 0 : wave;
+    const int wave_m = mw >> 1, wave_n = mw & 1;
+    const int g = lane >> 5, l32 = lane & 31;
+
+    // ---- item list: block-major (block, offset, tile); XCD x owns the x-th eighth, its workgroups interleave ----
+    const unsigned tiles = co_tiles * ci_tiles;
+    const unsigned per_block = (unsigned)V * tiles;
+    const unsigned total_items = nb * per_block;
+    const unsigned per_xcd = (total_items + kXcds - 1) / kXcds;
+    const unsigned xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds, stride = gridDim.x / kXcds;
+    const unsigned range_end = (xcd + 1) * per_xcd < total_items ? (xcd + 1) * per_xcd : total_items;
+
+    struct Walk {
+        unsigned item;
+        uint32_t k, k_hi;       // next pair to hand out, end of the item's pairs
+        unsigned b, v, tile;
+        bool live;
+    };
+    auto seek = [&](Walk& w) {                      // settle on the first non-empty item at or after w.item
+        w.live = false;
+        while (w.item < range_end) {
+            const unsigned b = w.item / per_block, within = w.item % per_block;
+            const unsigned v = within / tiles;
+            const uint32_t lo = bounds[v * (nb + 1) + b], hi = bounds[v * (nb + 1) + b + 1];
+            if (lo < hi) {
+                w.k = lo;
+                w.k_hi = hi;
+                w.b = b;
+                w.v = v;
+                w.tile = within % tiles;
+                w.live = true;
+                return;
+            }
+            w.item += stride;
+        }
+    };
+    auto advance = [&](Walk& w) {                   // one step further
+        w.k += P;
+        if (w.k >= w.k_hi) {
+            w.item += stride;
+            seek(w);
+        }
+    };
+    Walk first;
+    first.item = xcd * per_xcd + slot;
+    seek(first);
+    if (!first.live) return;                        // whole workgroup: nothing to do
+
+    const rsrc_t gout_rs = make_rsrc(gout, gout_bytes);
+    const rsrc_t feats_rs = make_rsrc(feats, feats_bytes);
+    const rsrc_t sigo_rs = make_rsrc(sig_o, n_pairs * 4u);
+    const rsrc_t sigi_rs = make_rsrc(sig_i, n_pairs * 4u);
+    const uint32_t rowb_o = (uint32_t)Co * ES, rowb_i = (uint32_t)Ci * ES;
+
+    if (loader) {
+        // =============================================================================================
+        // loaders
+        // =============================================================================================
+        int a_row[C::A_PER], b_row[C::B_PER];
+        uint32_t a_chb[C::A_PER], b_chb[C::B_PER];          // byte column inside the tile, swizzle applied
+#pragma unroll
+        for (int i = 0; i < C::A_PER; ++i) {
+            a_row[i] = (i * C::NL + lw) * C::RPI_A + lane / C::CH_A;
+            a_chb[i] = (uint32_t)(((lane % C::CH_A) ^ C::key_a(a_row[i])) * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < C::B_PER; ++i) {
+            b_row[i] = (i * C::NL + lw) * C::RPI_B + lane / C::CH_B;
+            b_chb[i] = (uint32_t)(((lane % C::CH_B) ^ C::key_b(b_row[i])) * 16);
+        }
+        Walk f = first, r = first;                  // index stream, row stream
+        unsigned f_step = 0, r_step = 0;            // steps handed out so far (ring positions)
+        auto issue_idx = [&]() -> int {             // index loads of the index stream's next step
+            if (!f.live) return 0;
+            int ops = 0;
+            uint32_t* dst = idx_ring + (f_step & (kWsIdxSlots - 1)) * (2 * P);
+            if (lw == 0) {
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(sigo_rs, FGX_LDS_PTR(dst), 4, (f.k + (uint32_t)lane) * 4u, 0, 0, 0);
+                ops = 1;
+            } else if (lw == 1) {
+                uint32_t* dst_i = dst + P;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(sigi_rs, FGX_LDS_PTR(dst_i), 4, (f.k + (uint32_t)lane) * 4u, 0, 0, 0);
+                ops = 1;
+            }
+            ++f_step;
+            advance(f);
+            return ops;
+        };
+        auto issue_rows = [&]() -> int {            // row loads of the row stream's next step; 0 when the stream is over
+            if (!r.live) return 0;
+            unsigned char* stage = ring + (r_step & (S - 1)) * C::STAGE_BYTES;
+            const uint32_t* slot_p = idx_ring + (r_step & (kWsIdxSlots - 1)) * (2 * P);
+            const unsigned co_tile = r.tile % co_tiles, ci_tile = r.tile / co_tiles;
+            const uint32_t m0b = co_tile * (uint32_t)(BM * ES), n0b = ci_tile * (uint32_t)(BN * ES);
+            const uint32_t left = r.k_hi - r.k;                                   // pairs left in the item
+            const bool ragged = left < (uint32_t)P || m0b + BM * ES > rowb_o || n0b + BN * ES > rowb_i;   // uniform
+            uint32_t va[C::A_PER], vb[C::B_PER];
+#pragma unroll
+            for (int i = 0; i < C::A_PER; ++i) va[i] = slot_p[a_row[i]] * rowb_o + (m0b + a_chb[i]);
+#pragma unroll
+            for (int i = 0; i < C::B_PER; ++i) vb[i] = slot_p[P + b_row[i]] * rowb_i + (n0b + b_chb[i]);
+            if (ragged) {
+#pragma unroll
+                for (int i = 0; i < C::A_PER; ++i)
+                    va[i] = ((uint32_t)a_row[i] < left && m0b + a_chb[i] < rowb_o) ? va[i] : kOobOffset;
+#pragma unroll
+                for (int i = 0; i < C::B_PER; ++i)
+                    vb[i] = ((uint32_t)b_row[i] < left && n0b + b_chb[i] < rowb_i) ? vb[i] : kOobOffset;
+            }
+            // (offsets go through a scalar local: the host pass of hipcc silently drops a kernel whose body hands an
+            // array element straight to this builtin)
+#pragma unroll
+            for (int i = 0; i < C::A_PER; ++i) {
+                const uint32_t vo = va[i];
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(gout_rs, FGX_LDS_PTR(stage + (i * C::NL + lw) * 1024), 16, vo, 0, 0, 0);
+            }
+            unsigned char* stage_b = stage + C::A_BYTES;
+#pragma unroll
+            for (int i = 0; i < C::B_PER; ++i) {
+                const uint32_t vo = vb[i];
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(feats_rs, FGX_LDS_PTR(stage_b + (i * C::NL + lw) * 1024), 16, vo, 0, 0, 0);
+            }
+            ++r_step;
+            advance(r);
+            return C::LPS;
+        };
+        // at most `n` of this loader's loads may be outstanding; n is a sum of two per-iteration counts, each 0, LPS
+        // or LPS + 1 (rounded down to the next value handled here, which is merely stricter)
+        auto wait_loads = [&](int n) {
+            if (n >= 2 * C::LPS + 2) wait_vmcnt<2 * C::LPS + 2>();
+            else if (n == 2 * C::LPS + 1) wait_vmcnt<2 * C::LPS + 1>();
+            else if (n == 2 * C::LPS) wait_vmcnt<2 * C::LPS>();
+            else if (n > C::LPS) wait_vmcnt<C::LPS + 1>();
+            else if (n == C::LPS) wait_vmcnt<C::LPS>();
+            else wait_vmcnt<0>();
+        };
+
+        // prologue: indices of the first kWsIdxAhead steps, then S-1 row rounds
+#pragma unroll
+        for (int j = 0; j < kWsIdxAhead; ++j) (void)issue_idx();
+        wait_vmcnt<0>();
+        __syncthreads();
+        int drained = 0, ops1 = 0, ops2 = 0;        // ops1: loads issued in the previous round, ops2: the one before
+#pragma unroll
+        for (int j = 0; j < S - 1; ++j) {
+            int ops = issue_rows();
+            if (ops == 0) ++drained;
+            ops += issue_idx();
+            ops2 = ops1;
+            ops1 = ops;
+        }
+        while (true) {
+            wait_loads(ops1 + ops2);               // everything issued before the last two rounds has landed
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();          // ... everybody's; the stage multiplied in the previous step is free
+            asm volatile("" ::: "memory");
+            int ops = issue_rows();
+            if (ops == 0) ++drained;
+            ops += issue_idx();
+            ops2 = ops1;
+            ops1 = ops;
+            if (drained >= S - 1) break;           // that was the barrier of the stream's last step
+        }
+        wait_vmcnt<0>();
+        return;
+    }
+
+    // =================================================================================================
+    // multipliers
+    // =================================================================================================
+    __syncthreads();                                // the loaders' prologue barrier
+    const int s16 = lane & 15, mb = (lane >> 4) & 1;
+    // per-lane byte offsets of the transposing reads inside a stage, for k-block 0 (a k-block is 16 pair rows)
+    int a_off[C::TM][2], b_off[C::TN][2];
+    {
+        const int prow = g * 8 + (s16 >> 2);
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i) {
+            const int byte = (wave_m * C::WM + i * 32 + mb * 16 + (s16 & 3) * 4) * 2;
+            const int c = byte >> 4, w = byte & 15;
+            a_off[i][0] = prow * C::ROWB_A + ((c ^ C::key_a(prow)) << 4) + w;
+            a_off[i][1] = (prow + 4) * C::ROWB_A + ((c ^ C::key_a(prow + 4)) << 4) + w;
+        }
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) {
+            const int byte = (wave_n * C::WN + j * 32 + mb * 16 + (s16 & 3) * 4) * 2;
+            const int c = byte >> 4, w = byte & 15;
+            b_off[j][0] = C::A_BYTES + prow * C::ROWB_B + ((c ^ C::key_b(prow)) << 4) + w;
+            b_off[j][1] = C::A_BYTES + (prow + 4) * C::ROWB_B + ((c ^ C::key_b(prow + 4)) << 4) + w;
+        }
+    }
+    constexpr int NK = P / 16;
+    constexpr int RK = 2 * (C::TM + C::TN);         // LDS reads per k-block
+    Walk m = first;
+    unsigned step = 0;
+    while (m.live) {
+        const unsigned b = m.b, v = m.v, tile = m.tile;
+        const int nsteps = (int)((m.k_hi - m.k + P - 1) / P);
+        f32x16 acc[C::TM][C::TN];
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+            for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        for (int s = 0; s < nsteps; ++s) {
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();           // the loaders saw this step's rows land
+            asm volatile("" ::: "memory");
+            const unsigned char* cur = ring + (step & (S - 1)) * C::STAGE_BYTES;
+            ++step;
+            // Transposing read: in a 16-lane group, lane s supplies the address of 4 adjacent channels of pair row
+            // (s / 4) and receives the 4 pair values of channel (group base + s).  Lanes 0-15 / 16-31 cover fragment
+            // rows 0-15 / 16-31, the two wave halves take pair rows [0, 8) / [8, 16) of the k-block.  The reads of
+            // k-block kk+1 are in flight while k-block kk is multiplied.
+            i16x4 fr[2][RK];
+            auto read_block = [&](int kk, i16x4 (&dst)[RK]) {
+                const unsigned char* base = cur + kk * 16 * C::ROWB_A;      // ROWB_A == ROWB_B is not assumed below
+#pragma unroll
+                for (int i = 0; i < C::TM; ++i) {
+                    dst[i * 2] = lds_read_tr16(base + a_off[i][0]);
+                    dst[i * 2 + 1] = lds_read_tr16(base + a_off[i][1]);
+                }
+                const unsigned char* base_b = cur + kk * 16 * C::ROWB_B;
+#pragma unroll
+                for (int j = 0; j < C::TN; ++j) {
+                    dst[(C::TM + j) * 2] = lds_read_tr16(base_b + b_off[j][0]);
+                    dst[(C::TM + j) * 2 + 1] = lds_read_tr16(base_b + b_off[j][1]);
+                }
+            };
+            read_block(0, fr[0]);
+#pragma unroll
+            for (int kk = 0; kk < NK; ++kk) {
+                if (kk + 1 < NK) {
+                    read_block(kk + 1, fr[(kk + 1) & 1]);
+                    lds_wait_but<RK>(fr[kk & 1]);
+                } else {
+                    lds_wait_but<0>(fr[kk & 1]);
+                }
+#pragma unroll
+                for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < C::TN; ++j) {
+                        const i16x8 af = __builtin_shufflevector(fr[kk & 1][i * 2], fr[kk & 1][i * 2 + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                        const i16x8 bf = __builtin_shufflevector(fr[kk & 1][(C::TM + j) * 2], fr[kk & 1][(C::TM + j) * 2 + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                        mma16<Tag>(acc[i][j], af, bf);
+                    }
+            }
+        }
+        // partial[b][v][co][ci], fp32
+        const unsigned co_tile = tile % co_tiles, ci_tile = tile / co_tiles;
+        const int m0 = (int)co_tile * BM, n0 = (int)ci_tile * BN;
+        float* dst = partial + ((size_t)b * V + v) * ((size_t)Co * Ci);
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) {
+            const int ci = n0 + wave_n * C::WN + j * 32 + l32;
+            if (ci >= Ci) continue;
+#pragma unroll
+            for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    int co = m0 + wave_m * C::WM + i * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
+                    if (co < Co) dst[(size_t)co * Ci + ci] = acc[i][j][e];
+                }
+        }
+        m.k = m.k_hi;                               // on to the next non-empty item
+        m.item += stride;
+        seek(m);
+    }
+}
+
 // grad_weight[co][v][ci] = sum over voxel blocks with pairs for offset v, in block order
 template <typename T>
 __global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restrict__ partial,
@@ -444,6 +792,67 @@ int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, con
     return FGX_OK;
 }
 
+template <typename Tag, int BM, int BN>
+int launch_wgrad_stream(const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
+                        const SegTable& tab, const Layout& L, size_t n, int V, int Ci, int Co, int block_rows,
+                        void* scratch, void* gw, hipStream_t s) {
+    using C = WStreamCfg<Tag, BM, BN>;
+    using T = typename Tag::type;
+    uint32_t* bounds = (uint32_t*)((char*)scratch + L.bounds_off);
+    float* partial = (float*)((char*)scratch + L.partial_off);
+    if (L.nb > 0) {
+        block_bounds_kernel<<<cdiv((size_t)V * (L.nb + 1), 256), 256, 0, s>>>(sig_o, tab, V, L.nb, (unsigned)block_rows, bounds);
+        FGX_CHECK_LAUNCH("fgx_conv_wgrad(bounds)");
+        const unsigned co_tiles = cdiv(Co, BM), ci_tiles = cdiv(Ci, BN);
+        const size_t items = (size_t)L.nb * V * co_tiles * ci_tiles;
+        FGX_CHECK_ARG(items < 0x7FFFFFFFull, "fgx_conv_wgrad: too many work items (%zu); use larger voxel blocks", items);
+        int dev = 0, cus = 0;
+        FGX_CHECK_HIP(hipGetDevice(&dev));
+        FGX_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        unsigned groups = (unsigned)(cus > 0 ? cus : 256);
+        groups = groups / kXcds * kXcds;                      // whole rounds over the XCDs
+        if (groups < (unsigned)kXcds) groups = kXcds;
+        auto kern = wgrad_stream_kernel<Tag, BM, BN>;
+        static thread_local bool lds_raised = false;
+        if (C::lds_bytes > 64 * 1024 && !lds_raised) {
+            FGX_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::lds_bytes));
+            lds_raised = true;
+        }
+        kern<<<groups, C::NT, C::lds_bytes, s>>>((const T*)gout, (const T*)feats, sig_i, sig_o, bounds, V, Ci, Co, L.nb, co_tiles,
+                                                 ci_tiles, tab.seg[V], (uint32_t)(n * (size_t)Co * sizeof(T)),
+                                                 (uint32_t)(n * (size_t)Ci * sizeof(T)), partial);
+        FGX_CHECK_LAUNCH("fgx_conv_wgrad(stream)");
+    }
+    size_t total = (size_t)Co * V * Ci;
+    unsigned g = cdiv(total, 256);
+    if (g > 65536u) g = 65536u;
+    wgrad_reduce_kernel<T><<<g, 256, 0, s>>>(partial, bounds, V, Ci, Co, L.nb, (T*)gw);
+    FGX_CHECK_LAUNCH("fgx_conv_wgrad(reduce)");
+    return FGX_OK;
+}
+
+// the streaming kernel: 16-bit types, tiles of 128x128 or 64x64, operands addressable with 32-bit offsets
+template <typename Tag>
+bool stream_ok(int tile_rows, int tile_cols, size_t n, int Ci, int Co, uint32_t n_pairs) {
+    if (sizeof(typename Tag::type) != 2) return false;
+    if (!((tile_rows == 128 && tile_cols == 128) || (tile_rows == 64 && tile_cols == 64))) return false;
+    return (double)n * Co * 2 <= (double)kOobOffset && (double)n * Ci * 2 <= (double)kOobOffset &&
+           (double)n_pairs * 4 + 256 <= (double)kOobOffset;
+}
+
+template <typename Tag>
+int dispatch_wgrad_stream(int tile_rows, const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
+                          const SegTable& tab, const Layout& L, size_t n, int V, int Ci, int Co, int block_rows, void* scratch,
+                          void* gw, hipStream_t s) {
+    if constexpr (sizeof(typename Tag::type) == 2) {
+        if (tile_rows == 128) return launch_wgrad_stream<Tag, 128, 128>(gout, feats, sig_i, sig_o, tab, L, n, V, Ci, Co, block_rows, scratch, gw, s);
+        return launch_wgrad_stream<Tag, 64, 64>(gout, feats, sig_i, sig_o, tab, L, n, V, Ci, Co, block_rows, scratch, gw, s);
+    } else {
+        set_error("fgx_conv_wgrad: the streaming kernel handles 16-bit types only");
+        return FGX_ERR_UNSUPPORTED;
+    }
+}
+
 template <typename Tag>
 int dispatch_wgrad(int tile_rows, int tile_cols, const void* gout, const void* feats, const uint32_t* sig_i,
                    const uint32_t* sig_o, const SegTable& tab, const Layout& L, bool small, int V, int Ci, int Co,
@@ -473,7 +882,7 @@ size_t fgx_wgrad_scratch_bytes(size_t n, int V, int Ci, int Co, int block_rows) 
 
 int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
                    const uint32_t* seg_host, size_t n, int Ci, int Co, int V, int tile_rows, int tile_cols, int block_rows,
-                   void* scratch, void* grad_weight, fgx_stream_t stream) {
+                   int streaming, void* scratch, void* grad_weight, fgx_stream_t stream) {
     FGX_CHECK_ARG(dtype_ok(dtype), "fgx_conv_wgrad: unknown dtype %d", dtype);
     FGX_CHECK_ARG(Ci > 0 && Co > 0 && V >= 1 && V <= kMaxV, "fgx_conv_wgrad: bad shape Ci=%d Co=%d V=%d", Ci, Co, V);
     FGX_CHECK_ARG(block_rows >= 1, "fgx_conv_wgrad: block_rows must be positive, got %d", block_rows);
@@ -498,6 +907,13 @@ int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uin
     // 32-bit byte offsets into grad_out / feats are enough below 4 GiB
     const bool small = (double)n * Co * es < 4294967296.0 && (double)n * Ci * es < 4294967296.0;
     hipStream_t s = (hipStream_t)stream;
+    if (streaming && any) {
+        // falls through to the tiled kernel when the problem is outside the streaming kernel's range
+        if (dtype == FGX_F16 && stream_ok<F16>(tile_rows, tile_cols, n, Ci, Co, tab.seg[V]))
+            return dispatch_wgrad_stream<F16>(tile_rows, grad_out, feats, sig_i, sig_o, tab, L, n, V, Ci, Co, block_rows, scratch, grad_weight, s);
+        if (dtype == FGX_BF16 && stream_ok<BF16>(tile_rows, tile_cols, n, Ci, Co, tab.seg[V]))
+            return dispatch_wgrad_stream<BF16>(tile_rows, grad_out, feats, sig_i, sig_o, tab, L, n, V, Ci, Co, block_rows, scratch, grad_weight, s);
+    }
     switch (dtype) {
         case FGX_F16: return dispatch_wgrad<F16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);
         case FGX_BF16: return dispatch_wgrad<BF16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);

@@ -347,7 +347,7 @@ def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int) -> tor
         nat.check(L.fgx_conv_wgrad(
             C.c_int(code), nat.ptr(g), nat.ptr(f), nat.ptr(cache["valid_signal_i"]), nat.ptr(cache["valid_signal_o"]),
             seg_arr, nat.sz(n), C.c_int(cip), C.c_int(cop), C.c_int(v), C.c_int(sched.tile_rows), C.c_int(sched.tile_cols),
-            C.c_int(sched.block_rows), nat.ptr(scratch), nat.ptr(gw), nat.stream()))
+            C.c_int(sched.block_rows), C.c_int(sched.stream), nat.ptr(scratch), nat.ptr(gw), nat.stream()))
         nat.mark("wgrad", "stop")
     if cip != ci or cop != co:
         gw = gw[:co, :, :ci].contiguous()

@@ -146,7 +146,8 @@ typedef struct fgx_schedule {
     int slab_bytes;     /* fwd/dgrad: bytes of K staged per row and pipeline step (64 or 128) */
     int splitk;         /* fwd/dgrad: number of K splits (1 = none) */
     int block_rows;     /* wgrad: voxel rows per partial-sum block */
-    int stream;         /* fwd/dgrad: 1 = persistent streaming kernel (fgx_conv_gather_gemm_stream), 0 = tiled kernel */
+    int stream;         /* 1 = persistent streaming kernel (fwd/dgrad: fgx_conv_gather_gemm_stream; wgrad: the
+                         * `streaming` argument of fgx_conv_wgrad), 0 = tiled kernel */
 } fgx_schedule;
 int fgx_table_lookup(int pass_kind, int dtype, size_t n, int Ci, int Co, int V, fgx_schedule* out);
 
@@ -209,13 +210,14 @@ int fgx_conv_gather_gemm_stream(int dtype, const void* src, const void* panel, c
  * seg_host is the HOST copy of valid_signal_seg (V+1 entries); sig_o must ascend inside every segment (it does
  * when it comes from fgx_pair_fill).  The voxels are cut into blocks of `block_rows` rows; every (block, offset)
  * partial product goes to `scratch` in fp32 (fgx_wgrad_scratch_bytes bytes, 256-byte aligned) and a second kernel
- * adds them per offset in block order.
+ * adds them per offset in block order.  `streaming` != 0 asks for the persistent kernel with loader / multiplier
+ * wavefronts (16-bit types, 128x128 or 64x64 tiles, operands below ~4 GB); outside that range the tiled kernel runs.
  * Replaces: sparse_submanifold_conv_bwd_weight_masked_implicit_gemm[_splitk]
  *           (..._bwd_masked_implicit_gemm.py:99-170, ..._splitk.py:108-182, 278-317). */
 size_t fgx_wgrad_scratch_bytes(size_t n, int V, int Ci, int Co, int block_rows);
 int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats,
                    const uint32_t* sig_i, const uint32_t* sig_o, const uint32_t* seg_host,
-                   size_t n, int Ci, int Co, int V, int tile_rows, int tile_cols, int block_rows,
+                   size_t n, int Ci, int Co, int V, int tile_rows, int tile_cols, int block_rows, int streaming,
                    void* scratch, void* grad_weight, fgx_stream_t stream);
 
 /* grad_bias[co] = sum over rows of grad_out[:, co], accumulated in fp32.
