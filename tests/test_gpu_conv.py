@@ -182,8 +182,8 @@ def test_forced_splitk_matches_unsplit(gpu_device):
     assert eg.max_rel_err(outs[1], outs[0].double()) <= 2e-3 and eg.max_rel_err(outs[2], outs[0].double()) <= 2e-3
 
 
-def _force_schedule(**fields):
-    """Context manager: fwd/dgrad schedules from the table with the given fields overridden."""
+def _force_schedule(wgrad=False, **fields):
+    """Context manager: fwd/dgrad (or, with wgrad=True, wgrad) schedules from the table with the given fields overridden."""
     import contextlib
     from flexgemm_amd import _native as nat
 
@@ -193,7 +193,7 @@ def _force_schedule(**fields):
 
         def forced(pass_kind, *a):
             sc = real(pass_kind, *a)
-            if pass_kind != nat.PASS_WGRAD:
+            if (pass_kind == nat.PASS_WGRAD) == wgrad:
                 for k, v in fields.items():
                     setattr(sc, k, v)
             return sc
@@ -243,6 +243,37 @@ def test_streaming_kernel_equals_tiled_kernel_bitwise(gpu_device):
             gi = impl._gather_gemm(g.to(gpu_device), w.to(gpu_device).reshape(c, 27, c), None, cache, 1, False)
         outs.append((o.cpu(), gi.cpu()))
     assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("res,ci,co,tile,block_rows", [(32, 128, 128, 128, 1024), (24, 64, 64, 64, 512), (24, 96, 40, 128, 300),
+                                                       (16, 256, 136, 128, 100000), (48, 128, 128, 128, 37)])
+def test_streaming_wgrad_matches_oracle(gpu_device, dtype, res, ci, co, tile, block_rows):
+    """wgrad with the persistent streaming kernel forced: edge tiles, several Co / Ci tiles, voxel blocks smaller
+    than a 64-pair step (most steps partial, many empty items) and one block for everything."""
+    _say(f"stream wgrad res={res} ci={ci} co={co} tile={tile} block_rows={block_rows} {dtype}")
+    coords_np = reference_test_shell(res)
+    shape = torch.Size([1, ci, res, res, res])
+    with _force_schedule(wgrad=True, tile_rows=tile, tile_cols=tile, block_rows=block_rows, stream=1):
+        _run_and_check(coords_np, shape, ci, co, dtype, gpu_device, seed=23)
+
+
+def test_streaming_wgrad_equals_tiled_wgrad_bitwise(gpu_device):
+    """Same 16-pair MFMA blocks in the same order inside every (voxel block, offset) item, same block-ordered
+    reduction: the two wgrad kernels agree bit for bit."""
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    _say("stream wgrad vs tiled wgrad, bitwise")
+    res, c = 40, 128
+    coords_np = reference_test_shell(res)
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    shape = torch.Size([1, c, res, res, res])
+    f, _, _, g = _case(coords_np, c, c, torch.float16, 33)
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+    outs = []
+    for stream in (0, 1):
+        with _force_schedule(wgrad=True, tile_rows=128, tile_cols=128, block_rows=1024, stream=stream):
+            outs.append(impl._wgrad(g.to(gpu_device), f.to(gpu_device), cache, 27).cpu())
+    assert torch.equal(outs[0], outs[1])
 
 
 @pytest.mark.parametrize("name,res,c", [("cfg2", 64, 256), ("cfg3", 128, 128), ("cfg4", 128, 32), ("cfg5", 32, 1024)])
