@@ -378,7 +378,7 @@ wgrad_kernel(const typename Tag::type* __restrict__ gout, const typename Tag::ty
 // last two iterations).
 constexpr int kWsStages = 4;
 constexpr int kWsIdxSlots = 8;
-constexpr int kWsIdxAhead = 3;       // index loads run this many steps ahead of the row loads (> kWsStages - 2)
+constexpr int kWsIdxAhead = 4;       // index loads run this many steps ahead of the row loads (> kWsStages - 1)
 constexpr int kWsLoaders = 4;
 constexpr int kWsPairs = 64;         // pairs per step
 constexpr uint32_t kOobOffset = 0xFF000000u;
@@ -529,15 +529,22 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
             advance(f);
             return ops;
         };
-        auto issue_rows = [&]() -> int {            // row loads of the row stream's next step; 0 when the stream is over
-            if (!r.live) return 0;
-            unsigned char* stage = ring + (r_step & (S - 1)) * C::STAGE_BYTES;
+        // Row loads come in two halves.  prep_rows() turns the next step's indices into per-lane buffer offsets (LDS
+        // reads, multiplies, range checks) and is run right AFTER the previous step's loads were enqueued, i.e. while the
+        // multipliers work and this wavefront would only wait for the next barrier; fire_rows() then enqueues the
+        // prepared loads first thing after that barrier.
+        bool pr_live = false;
+        unsigned pr_stage = 0;
+        uint32_t va[C::A_PER], vb[C::B_PER];
+        auto prep_rows = [&]() {
+            pr_live = r.live;
+            if (!r.live) return;
+            pr_stage = r_step & (S - 1);
             const uint32_t* slot_p = idx_ring + (r_step & (kWsIdxSlots - 1)) * (2 * P);
             const unsigned co_tile = r.tile % co_tiles, ci_tile = r.tile / co_tiles;
             const uint32_t m0b = co_tile * (uint32_t)(BM * ES), n0b = ci_tile * (uint32_t)(BN * ES);
             const uint32_t left = r.k_hi - r.k;                                   // pairs left in the item
             const bool ragged = left < (uint32_t)P || m0b + BM * ES > rowb_o || n0b + BN * ES > rowb_i;   // uniform
-            uint32_t va[C::A_PER], vb[C::B_PER];
 #pragma unroll
             for (int i = 0; i < C::A_PER; ++i) va[i] = slot_p[a_row[i]] * rowb_o + (m0b + a_chb[i]);
 #pragma unroll
@@ -550,6 +557,12 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
                 for (int i = 0; i < C::B_PER; ++i)
                     vb[i] = ((uint32_t)b_row[i] < left && n0b + b_chb[i] < rowb_i) ? vb[i] : kOobOffset;
             }
+            ++r_step;
+            advance(r);
+        };
+        auto fire_rows = [&]() -> int {             // 0 when the stream is over
+            if (!pr_live) return 0;
+            unsigned char* stage = ring + pr_stage * C::STAGE_BYTES;
             // (offsets go through a scalar local: the host pass of hipcc silently drops a kernel whose body hands an
             // array element straight to this builtin)
 #pragma unroll
@@ -563,8 +576,6 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
                 const uint32_t vo = vb[i];
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(feats_rs, FGX_LDS_PTR(stage_b + (i * C::NL + lw) * 1024), 16, vo, 0, 0, 0);
             }
-            ++r_step;
-            advance(r);
             return C::LPS;
         };
         // at most `n` of this loader's loads may be outstanding; n is a sum of two per-iteration counts, each 0, LPS
@@ -583,11 +594,13 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
         for (int j = 0; j < kWsIdxAhead; ++j) (void)issue_idx();
         wait_vmcnt<0>();
         __syncthreads();
+        prep_rows();
         int drained = 0, ops1 = 0, ops2 = 0;        // ops1: loads issued in the previous round, ops2: the one before
 #pragma unroll
         for (int j = 0; j < S - 1; ++j) {
-            int ops = issue_rows();
+            int ops = fire_rows();
             if (ops == 0) ++drained;
+            prep_rows();                            // indices of steps 1 .. S-1 came with the first batch
             ops += issue_idx();
             ops2 = ops1;
             ops1 = ops;
@@ -597,12 +610,13 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
             asm volatile("" ::: "memory");
             __builtin_amdgcn_s_barrier();          // ... everybody's; the stage multiplied in the previous step is free
             asm volatile("" ::: "memory");
-            int ops = issue_rows();
+            int ops = fire_rows();
             if (ops == 0) ++drained;
+            if (drained >= S - 1) break;           // that was the barrier of the stream's last step
+            prep_rows();
             ops += issue_idx();
             ops2 = ops1;
             ops1 = ops;
-            if (drained >= S - 1) break;           // that was the barrier of the stream's last step
         }
         wait_vmcnt<0>();
         return;
