@@ -23,15 +23,15 @@ const Entry kTable[] = {
     {0, 2, 19, 128, 128, {256, 128, 128, 1, 0, 1}},
     {1, 2, 19, 128, 128, {256, 128, 128, 1, 0, 1}},
     {2, 2, 19, 128, 128, {128, 128, 64, 1, 8192, 1}},
-    {0, 2, 17, 256, 256, {128, 128, 64, 1, 0, 0}},
-    {1, 2, 17, 256, 256, {128, 128, 64, 1, 0, 0}},
-    {2, 2, 17, 256, 256, {128, 128, 64, 1, 4096, 0}},
+    {0, 2, 17, 256, 256, {256, 128, 128, 1, 0, 1}},
+    {1, 2, 17, 256, 256, {256, 128, 128, 1, 0, 1}},
+    {2, 2, 17, 256, 256, {128, 128, 64, 1, 4096, 1}},
     {0, 2, 21, 32, 32, {128, 32, 64, 1, 0, 0}},
     {1, 2, 21, 32, 32, {128, 32, 64, 1, 0, 0}},
     {2, 2, 21, 32, 32, {32, 32, 64, 1, 4096, 0}},
-    {0, 2, 15, 1024, 1024, {128, 128, 64, 1, 0, 0}},
-    {1, 2, 15, 1024, 1024, {128, 128, 64, 1, 0, 0}},
-    {2, 2, 15, 1024, 1024, {128, 128, 64, 1, 65536, 0}},
+    {0, 2, 15, 1024, 1024, {256, 128, 128, 1, 0, 1}},
+    {1, 2, 15, 1024, 1024, {256, 128, 128, 1, 0, 1}},
+    {2, 2, 15, 1024, 1024, {128, 128, 64, 1, 65536, 1}},
 };
 
 int floor_log2(size_t n) {
@@ -44,7 +44,7 @@ int pick_cols(int c) { return c > 64 ? 128 : (c > 32 ? 64 : 32); }
 
 size_t round_up(size_t x, size_t m) { return (x + m - 1) / m * m; }
 
-void rule(int pass_kind, size_t n, int Ci, int Co, int V, fgx_schedule* out) {
+void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* out) {
     if (pass_kind == 2) {
         // wgrad: square tiles over (Co, Ci); voxel blocks of at least 4096 rows, enlarged until the fp32 partial
         // products (blocks x V x Co x Ci) stay below 256 MiB.
@@ -53,7 +53,8 @@ void rule(int pass_kind, size_t n, int Ci, int Co, int V, fgx_schedule* out) {
         out->tile_cols = t;
         out->slab_bytes = 64;
         out->splitk = 1;
-        out->stream = 0;
+        // persistent streaming kernel: 16-bit types, tiles of at least 64, enough voxels to give every CU several items
+        out->stream = (es == 2 && t >= 64 && n >= 32768) ? 1 : 0;
         const double per_block = 4.0 * V * (double)Co * (double)Ci;
         size_t max_blocks = (size_t)(268435456.0 / per_block);
         if (max_blocks < 1) max_blocks = 1;
@@ -76,6 +77,16 @@ void rule(int pass_kind, size_t n, int Ci, int Co, int V, fgx_schedule* out) {
     int s = 1;
     while (tiles * s < (size_t)kCUs && s < 16) s *= 2;
     out->splitk = s;
+    // persistent streaming kernel (256 x 128 tiles, 128-byte K-slabs): rows of at least one slab, full-width column
+    // tiles, and at least two items per CU
+    const int K = pass_kind == 0 ? Ci : Co;
+    if ((size_t)K * es >= 128 && cols >= 128 && (size_t)cdiv(n, 256) * cdiv(cols, 128) >= 2 * (size_t)kCUs) {
+        out->tile_rows = 256;
+        out->tile_cols = 128;
+        out->slab_bytes = 128;
+        out->splitk = 1;
+        out->stream = 1;
+    }
 }
 
 }  // namespace
@@ -96,6 +107,6 @@ extern "C" int fgx_table_lookup(int pass_kind, int dtype, size_t n, int Ci, int 
             return FGX_OK;
         }
     }
-    rule(pass_kind, n, Ci, Co, V, out);
+    rule(pass_kind, es, n, Ci, Co, V, out);
     return FGX_OK;
 }
