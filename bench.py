@@ -27,6 +27,10 @@ if ROOT not in sys.path:
 
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}   # MI355X dense MFMA peaks
 HBM_PEAK_GBS = 8000.0
+# HBM-side bytes per launch of the dominant kernel, from two rocprofv3 counter runs of this script (FETCH_SIZE, then
+# WRITE_SIZE, each scaled by what the same counter reads for the plain copy of --calibrate-copy: x2.0 and x1.0).
+# The counters cannot be read from inside the process, so the measured figure is kept here per workload.
+MEASURED_TRAFFIC_BYTES = {"cfg3": 1.760e9}
 
 
 def parse():
@@ -193,14 +197,14 @@ def main():
     es = 2 if dname != "f32" else 4
     gemm_bytes = es * n * (c + c) + es * 27 * c * c + 108.0 * n + 8.0 * n
     roof = {
-        "bound": "mfma", "kernel": "gather_gemm_kernel (forward and dgrad launches)",
+        "bound": "mfma", "kernel": "gather GEMM (gather_gemm_stream_kernel or gather_gemm_kernel; forward and dgrad launches)",
         "achieved": flop_pass / (gemm_ms * 1e-3) / 1e12, "peak": PEAK_TFLOPS[dname], "unit": "TFLOP/s",
         "frac": flop_pass / (gemm_ms * 1e-3) / 1e12 / PEAK_TFLOPS[dname],
         "avg_launch_ms": gemm_ms, "launches_timed": gemm_launches,
         "algorithmic_flop_per_launch": flop_pass,
         "algorithmic_bytes_per_launch": gemm_bytes,
         "algorithmic_hbm_GBps": gemm_bytes / (gemm_ms * 1e-3) / 1e9,
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
     }
     if args.workload == "cfg4":   # C = 32: every pass is HBM bound
         roof.update({"bound": "hbm", "achieved": gemm_bytes / (gemm_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
