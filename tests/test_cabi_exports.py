@@ -41,10 +41,18 @@ def test_host_only_entry_points(library):
     import torch
     s = nat.table_lookup(nat.PASS_FWD, torch.float16, 669288, 128, 128, 27)
     assert s.tile_rows in (128, 256) and s.tile_cols == 128 and s.splitk == 1 and s.slab_bytes in (64, 128)
+    # the persistent streaming kernel has exactly one tile shape
+    assert (s.stream, s.tile_rows, s.slab_bytes) in ((1, 256, 128), (0, s.tile_rows, s.slab_bytes))
     s = nat.table_lookup(nat.PASS_WGRAD, torch.float16, 669288, 128, 128, 27)
-    assert s.block_rows >= 1024
+    assert s.block_rows >= 1024 and s.stream in (0, 1)
     s = nat.table_lookup(nat.PASS_FWD, torch.float32, 100, 16, 16, 27)
-    assert s.tile_rows in (32, 64, 128) and s.tile_cols == 32 and s.splitk >= 1
+    assert s.tile_rows in (32, 64, 128) and s.tile_cols == 32 and s.splitk >= 1 and s.stream == 0
+    # rule (no table entry): big 16-bit problems stream, small ones and short rows do not
+    s = nat.table_lookup(nat.PASS_DGRAD, torch.bfloat16, 300000, 192, 160, 27)
+    assert (s.stream, s.tile_rows, s.tile_cols, s.slab_bytes, s.splitk) == (1, 256, 128, 128, 1)
+    assert nat.table_lookup(nat.PASS_FWD, torch.bfloat16, 300000, 32, 32, 27).stream == 0
+    assert nat.table_lookup(nat.PASS_FWD, torch.float16, 5000, 192, 160, 27).stream == 0
+    assert nat.table_lookup(nat.PASS_WGRAD, torch.float32, 300000, 192, 160, 27).stream == 0
     assert L.fgx_weight_panel_bytes(0, 0, 128, 128, 27, 64, 128) == 27 * 2 * 128 * 128
     assert L.fgx_weight_panel_bytes(2, 1, 40, 24, 27, 128, 32) == 27 * 1 * 64 * 128  # K=24 -> 1 slab, cols 40 -> 64
     assert L.fgx_weight_panel_bytes(2, 1, 40, 24, 27, 64, 32) == 27 * 2 * 64 * 64    # 16 floats per slab -> 2 slabs
@@ -63,8 +71,12 @@ def test_argument_errors_map_to_exceptions(library):
         nat.check(L.fgx_subm_neighbor_map(None, 32, None, ctypes.c_size_t(0), None, ctypes.c_size_t(0), 4, 4, 4,
                                           2, 3, 3, 1, 1, 1, None, None, None, None))
     with pytest.raises(ValueError):
-        nat.check(L.fgx_conv_wgrad(0, None, None, None, None, None, ctypes.c_size_t(0), 8, 8, 27, 128, 128, 0,
+        nat.check(L.fgx_conv_wgrad(0, None, None, None, None, None, ctypes.c_size_t(0), 8, 8, 27, 128, 128, 0, 0,
                                    None, None, None))
+    with pytest.raises(ValueError):   # the streaming GEMM checks its arguments before touching the device
+        nat.check(L.fgx_conv_gather_gemm_stream(0, None, None, None, None, None, None, None, ctypes.c_size_t(0),
+                                                ctypes.c_size_t(10), 128, 128, 27, 256, 128, 128, 0, None, None))
+    assert b"null buffer" in L.fgx_last_error()
 
 
 def test_host_logic_without_gpu():
