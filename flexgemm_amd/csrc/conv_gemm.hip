@@ -401,7 +401,7 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restr
 // Column sums with fp32 accumulation.  Stage 1: kColsumSlices blocks each sum a contiguous slice of rows with
 // 16-byte loads (a thread owns VEC adjacent columns, the block's row lanes are added through LDS); stage 2 adds
 // the slices in a fixed order, so the result is deterministic.
-constexpr int kColsumSlices = 512;
+constexpr int kColsumSlices = 1024;
 template <typename T, int VEC>
 __global__ void __launch_bounds__(256) colsum_partial_kernel(const T* __restrict__ x, size_t n, int cols,
                                                              float* __restrict__ partial) {
@@ -418,7 +418,22 @@ __global__ void __launch_bounds__(256) colsum_partial_kernel(const T* __restrict
 #pragma unroll
         for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
         if (rl < lanes) {
-            for (size_t r = r0 + rl; r < r1; r += lanes) {
+            size_t r = r0 + rl;
+            if constexpr (VEC > 1) {
+                // four rows per trip: four independent 16-byte loads in flight, added in row order
+                for (; r + 3 * (size_t)lanes < r1; r += 4 * (size_t)lanes) {
+                    u32x4 raw[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) raw[q] = *(const u32x4*)(x + (r + (size_t)q * lanes) * cols + (size_t)cg * VEC);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const T* v = (const T*)&raw[q];
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) acc[e] += to_float<T>(v[e]);
+                    }
+                }
+            }
+            for (; r < r1; r += lanes) {
                 const T* src = x + r * cols + (size_t)cg * VEC;
                 if constexpr (VEC == 1) {
                     acc[0] += to_float<T>(src[0]);
@@ -455,8 +470,17 @@ __global__ void __launch_bounds__(256) colsum_final_kernel(const float* __restri
     const int c = blockIdx.x * 16 + (threadIdx.x & 15);
     const int part = threadIdx.x >> 4;
     float s = 0.f;
-    if (c < cols)
-        for (unsigned b = part; b < slices; b += 16) s += partial[(size_t)b * cols + c];
+    if (c < cols) {
+        unsigned b = part;
+        for (; b + 7 * 16 < slices; b += 8 * 16) {     // eight independent loads in flight, added in slice order
+            float x[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) x[q] = partial[(size_t)(b + q * 16) * cols + c];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) s += x[q];
+        }
+        for (; b < slices; b += 16) s += partial[(size_t)b * cols + c];
+    }
     red[threadIdx.x] = s;
     __syncthreads();
     if (part == 0 && c < cols) {

@@ -743,12 +743,12 @@ __global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restri
         const size_t stride = (size_t)V * per;
         float s = 0.f;
         unsigned b = 0;
-        for (; b + 4 <= nb; b += 4) {     // four independent loads in flight; the sum order stays b-ascending
-            const float x0 = bd[b] < bd[b + 1] ? src[(size_t)b * stride] : 0.f;
-            const float x1 = bd[b + 1] < bd[b + 2] ? src[(size_t)(b + 1) * stride] : 0.f;
-            const float x2 = bd[b + 2] < bd[b + 3] ? src[(size_t)(b + 2) * stride] : 0.f;
-            const float x3 = bd[b + 3] < bd[b + 4] ? src[(size_t)(b + 3) * stride] : 0.f;
-            s = (((s + x0) + x1) + x2) + x3;
+        for (; b + 8 <= nb; b += 8) {     // eight independent loads in flight; the sum order stays b-ascending
+            float x[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) x[q] = bd[b + q] < bd[b + q + 1] ? src[(size_t)(b + q) * stride] : 0.f;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) s += x[q];
         }
         for (; b < nb; ++b)
             if (bd[b] < bd[b + 1]) s += src[(size_t)b * stride];
