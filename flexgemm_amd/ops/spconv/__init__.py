@@ -5,9 +5,11 @@
 class Algorithm:
     """Algorithm choices for sparse convolution.
 
-    On gfx950 the four implicit-GEMM values all run the masked implicit GEMM kernels (the plain
-    values without the split-K search); EXPLICIT_GEMM is the gather + dense-GEMM formulation in
-    torch ops."""
+    On gfx950 the four implicit-GEMM values share the same gather-GEMM kernels.  MASKED_* walk the
+    mask-sorted row order and skip, tile by tile, the offsets no row of the tile has; IMPLICIT_GEMM*
+    walk the rows in their natural order and every tile visits all offsets (for inputs so dense that
+    sorting buys nothing), and their neighbor cache is the map alone.  The values without _SPLITK never
+    split K.  EXPLICIT_GEMM is the gather + dense-GEMM formulation in torch ops."""
     EXPLICIT_GEMM = "explicit_gemm"
     IMPLICIT_GEMM = "implicit_gemm"
     IMPLICIT_GEMM_SPLITK = "implicit_gemm_splitk"

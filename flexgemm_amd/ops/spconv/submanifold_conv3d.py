@@ -23,6 +23,7 @@ EMPTY = 0xFFFFFFFF
 _IMPLICIT = (Algorithm.IMPLICIT_GEMM, Algorithm.IMPLICIT_GEMM_SPLITK,
              Algorithm.MASKED_IMPLICIT_GEMM, Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
 _NO_SPLITK = (Algorithm.IMPLICIT_GEMM, Algorithm.MASKED_IMPLICIT_GEMM)
+_MASKED = (Algorithm.MASKED_IMPLICIT_GEMM, Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
 
 
 def _require_cuda(t: torch.Tensor, what: str) -> None:
@@ -82,13 +83,33 @@ class SubMConv3dNeighborCache:
             setattr(self, seg_key, seg)
         return order, getattr(self, key), getattr(self, seg_key)
 
-    def _gather_plan(self, block_size: int, private: bool):
+    def _dense_tile_tables(self, block_size: int):
+        """(order, tile_code) of the non-masked schedule (reference: ..._fwd_implicit_gemm.py:18-89): rows in their
+        natural order, every tile walks all V offsets."""
+        key = f"_dense_code_{block_size}"
+        if not hasattr(self, key):
+            nmap = self["neighbor_map"]
+            n, v = nmap.shape
+            nb = (n + block_size - 1) // block_size
+            full = (1 << v) - 1
+            if full >= 1 << 31:
+                full -= 1 << 32                  # V = 32: all ones as int32
+            if not hasattr(self, "_dense_order"):
+                self["_dense_order"] = torch.arange(n, dtype=torch.int64, device=nmap.device)
+            setattr(self, key, torch.full((nb,), full, dtype=torch.int32, device=nmap.device))
+        return self["_dense_order"], getattr(self, key)
+
+    def _gather_plan(self, block_size: int, private: bool, dense: bool = False):
         """(order, tile_code int32 [nb], plan_seg int32 [nb+1], plan_idx uint32 [P, block_size]) for the streaming
         GEMM: per tile and offset present in it, the tile's source rows as one contiguous run.  Built once per tile size
         (one 4-byte read-back sizes it) and kept with the cache."""
-        order, code, _ = self._tile_tables(block_size, private)
-        use_private = private and hasattr(self, "_tile_order")
-        key = f"_plan_{'t' if use_private else 'm'}_{block_size}"
+        if dense:
+            order, code = self._dense_tile_tables(block_size)
+            key = f"_plan_d_{block_size}"
+        else:
+            order, code, _ = self._tile_tables(block_size, private)
+            use_private = private and hasattr(self, "_tile_order")
+            key = f"_plan_{'t' if use_private else 'm'}_{block_size}"
         if not hasattr(self, key):
             nmap = self["neighbor_map"]
             n, v = nmap.shape
@@ -257,8 +278,9 @@ def _pad_cols(t: torch.Tensor, mult: int) -> torch.Tensor:
 
 
 def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[torch.Tensor], cache, mode: int,
-                 allow_splitk: bool) -> torch.Tensor:
-    """mode 0: out = conv(src) with weight [Co, V, Ci] (+bias); mode 1: grad_input from src = grad_output."""
+                 allow_splitk: bool, masked: bool = True) -> torch.Tensor:
+    """mode 0: out = conv(src) with weight [Co, V, Ci] (+bias); mode 1: grad_input from src = grad_output.
+    masked=False: the non-masked schedule (natural row order, all offsets per tile)."""
     co, v, ci = weight_cvk.shape
     n = src.shape[0]
     dt = src.dtype
@@ -282,8 +304,9 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
     weight_cvk = weight_cvk.contiguous()
     sched = nat.table_lookup(nat.PASS_FWD if mode == 0 else nat.PASS_DGRAD, dt, n, ci, co, v)
     splitk = sched.splitk if allow_splitk else 1
-    cache._ensure_sorted()
-    private = k * src.element_size() <= LOCALITY_MAX_ROW_BYTES
+    if masked:
+        cache._ensure_sorted()
+    private = masked and k * src.element_size() <= LOCALITY_MAX_ROW_BYTES
     out = torch.empty((n, cols), dtype=dt, device=dev)
     if n == 0:
         return out
@@ -296,7 +319,7 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
         nat.check(L.fgx_pack_weight(C.c_int(code), C.c_int(mode), nat.ptr(weight_cvk), C.c_int(ci), C.c_int(co), C.c_int(v),
                                     C.c_int(sched.slab_bytes), C.c_int(sched.tile_cols), nat.ptr(panel), nat.stream()))
         if sched.stream and _stream_fits(n, k * src.element_size()):
-            order, tile_code, plan_seg, plan_idx = cache._gather_plan(sched.tile_rows, private)
+            order, tile_code, plan_seg, plan_idx = cache._gather_plan(sched.tile_rows, private, dense=not masked)
             nat.mark(name, "start")
             nat.check(L.fgx_conv_gather_gemm_stream(
                 C.c_int(code), nat.ptr(src), nat.ptr(panel), nat.ptr(bias), nat.ptr(order), nat.ptr(tile_code),
@@ -305,7 +328,10 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
                 nat.stream()))
             nat.mark(name, "stop")
             return out
-        order, tile_code, _ = cache._tile_tables(sched.tile_rows, private)
+        if masked:
+            order, tile_code, _ = cache._tile_tables(sched.tile_rows, private)
+        else:
+            order, tile_code = cache._dense_tile_tables(sched.tile_rows)
         scratch = None
         if splitk > 1:
             scratch = nat.workspace(L.fgx_conv_scratch_bytes(nat.sz(n), C.c_int(cols), C.c_int(splitk)), dev)
@@ -397,6 +423,11 @@ class SubMConv3dFunction(Function):
             nmap, _, _ = _build_neighbor_map(coords, shape, kernel_size, dilation, with_codes=False)
             return SubMConv3dNeighborCache(neighbor_map=nmap)
         assert v <= 32, "Currently, the max kernel volume is 32 because kernel mask is encoded as uint32"
+        if algo not in _MASKED:
+            # non-masked implicit GEMM: the cache is the map alone (reference: submanifold_conv3d.py:59-71); the
+            # pair lists wgrad needs are derived from it on first use
+            nmap, _, _ = _build_neighbor_map(coords, shape, kernel_size, dilation, with_codes=False)
+            return SubMConv3dNeighborCache(neighbor_map=nmap)
         nmap, gray, binary = _build_neighbor_map(coords, shape, kernel_size, dilation, with_codes=True)
         gray, binary, order = _codes_and_order(nmap, gray, binary)
         cache = SubMConv3dNeighborCache(neighbor_map=nmap, gray_code=gray, sorted_idx=order)
@@ -463,7 +494,8 @@ class SubMConv3dFunction(Function):
             return torch.addmm(bias, col, w) if bias is not None else torch.mm(col, w)
         if algo in _IMPLICIT:
             _require_cuda(feats, "sparse_submanifold_conv3d")
-            return _gather_gemm(feats, weight.reshape(co, v, ci), bias, neighbor_cache, 0, algo not in _NO_SPLITK)
+            return _gather_gemm(feats, weight.reshape(co, v, ci), bias, neighbor_cache, 0, algo not in _NO_SPLITK,
+                                masked=algo in _MASKED)
         raise ValueError(f"Unsupported algorithm {algo}")
 
     @staticmethod
@@ -495,7 +527,7 @@ class SubMConv3dFunction(Function):
             grad_output = grad_output.contiguous()
             if feats.requires_grad:
                 grad_input = _gather_gemm(grad_output, weight.detach().reshape(co, v, ci), None, neighbor_cache, 1,
-                                          algo not in _NO_SPLITK)
+                                          algo not in _NO_SPLITK, masked=algo in _MASKED)
             if weight.requires_grad:
                 grad_weight = _wgrad(grad_output, feats.detach(), neighbor_cache, v).reshape(co, kw, kh, kd, ci)
             if bias is not None and bias.requires_grad:

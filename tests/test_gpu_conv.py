@@ -129,6 +129,28 @@ def test_algorithm_values_and_cache_reuse(gpu_device):
     assert not hasattr(cch, "valid_signal_i") and out.shape == (len(coords_np), c)
 
 
+@pytest.mark.parametrize("stream", [0, 1])
+def test_non_masked_schedule(gpu_device, stream):
+    """IMPLICIT_GEMM[_SPLITK]: the cache is the neighbor map alone (reference submanifold_conv3d.py:59-71) and the
+    kernels walk the natural row order with all 27 offsets per tile; same results as the oracle."""
+    res, c = 24, 128
+    coords_np = reference_test_shell(res)
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    shape = torch.Size([1, c, res, res, res])
+    for algo in (Algorithm.IMPLICIT_GEMM, Algorithm.IMPLICIT_GEMM_SPLITK):
+        _say(f"non-masked schedule {algo} stream={stream}")
+        flex_gemm.ops.spconv.set_algorithm(algo)
+        try:
+            cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+        finally:
+            flex_gemm.ops.spconv.set_algorithm(Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
+        assert [k for k in vars(cache) if not k.startswith("_")] == ["neighbor_map"]
+        fields = dict(tile_rows=256, tile_cols=128, slab_bytes=128, splitk=1, stream=1) if stream else dict(stream=0)
+        with _force_schedule(**fields):
+            _run_and_check(coords_np, shape, c, c, torch.float16, gpu_device, seed=41, algo=algo, cache=cache)
+        assert hasattr(cache, "_dense_order") and (stream == 0 or hasattr(cache, "_plan_d_256"))
+
+
 def test_private_row_order_is_used_and_equivalent(gpu_device):
     """Short rows (<= 128 bytes) run on the Z-order-chunked private row order, long rows on the public mask-sorted one;
     both give the oracle's result (checked by _run_and_check) and agree with each other."""
