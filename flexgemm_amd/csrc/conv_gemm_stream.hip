@@ -451,6 +451,7 @@ int dispatch_stream(int tile_rows, int tile_cols, int slab_bytes, const void* sr
         return launch_stream<Tag, BM, BN, WMv, WNv, CHv>(src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_rows, \
                                                          n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
     FGX_STREAM_TILE(256, 128, 4, 2, 8)
+    FGX_STREAM_TILE(256, 64, 4, 2, 8)
 #undef FGX_STREAM_TILE
     set_error("fgx_conv_gather_gemm_stream: no kernel for tile %dx%d with %d-byte slabs", tile_rows, tile_cols, slab_bytes);
     return FGX_ERR_UNSUPPORTED;

@@ -77,12 +77,13 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
     int s = 1;
     while (tiles * s < (size_t)kCUs && s < 16) s *= 2;
     out->splitk = s;
-    // persistent streaming kernel (256 x 128 tiles, 128-byte K-slabs): rows of at least one slab, full-width column
-    // tiles, and at least two items per CU
+    // persistent streaming kernel (256 x 128 or 256 x 64 tiles, 128-byte K-slabs): rows of at least one slab, at least
+    // 64 columns, and at least two items per CU
     const int K = pass_kind == 0 ? Ci : Co;
-    if ((size_t)K * es >= 128 && cols >= 128 && (size_t)cdiv(n, 256) * cdiv(cols, 128) >= 2 * (size_t)kCUs) {
+    const int scols = cols > 64 ? 128 : 64;
+    if ((size_t)K * es >= 128 && cols >= 64 && (size_t)cdiv(n, 256) * cdiv(cols, scols) >= 2 * (size_t)kCUs) {
         out->tile_rows = 256;
-        out->tile_cols = 128;
+        out->tile_cols = scols;
         out->slab_bytes = 128;
         out->splitk = 1;
         out->stream = 1;

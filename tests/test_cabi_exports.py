@@ -51,6 +51,8 @@ def test_host_only_entry_points(library):
     s = nat.table_lookup(nat.PASS_DGRAD, torch.bfloat16, 300000, 192, 160, 27)
     assert (s.stream, s.tile_rows, s.tile_cols, s.slab_bytes, s.splitk) == (1, 256, 128, 128, 1)
     assert nat.table_lookup(nat.PASS_FWD, torch.bfloat16, 300000, 32, 32, 27).stream == 0
+    s = nat.table_lookup(nat.PASS_FWD, torch.float16, 300000, 64, 64, 27)
+    assert (s.stream, s.tile_rows, s.tile_cols, s.slab_bytes) == (1, 256, 64, 128)
     assert nat.table_lookup(nat.PASS_FWD, torch.float16, 5000, 192, 160, 27).stream == 0
     assert nat.table_lookup(nat.PASS_WGRAD, torch.float32, 300000, 192, 160, 27).stream == 0
     assert L.fgx_weight_panel_bytes(0, 0, 128, 128, 27, 64, 128) == 27 * 2 * 128 * 128

@@ -237,6 +237,9 @@ def test_streaming_kernel_matches_oracle(gpu_device, dtype, res, ci, co):
     shape = torch.Size([1, ci, res, res, res])
     with _force_schedule(tile_rows=256, tile_cols=128, slab_bytes=128, splitk=1, stream=1):
         _run_and_check(coords_np, shape, ci, co, dtype, gpu_device, seed=21)
+    if co <= 136:   # the narrow-tile variant of the streaming kernel (64 columns per tile)
+        with _force_schedule(tile_rows=256, tile_cols=64, slab_bytes=128, splitk=1, stream=1):
+            _run_and_check(coords_np, shape, ci, co, dtype, gpu_device, seed=22)
 
 
 def test_streaming_kernel_equals_tiled_kernel_bitwise(gpu_device):
