@@ -71,8 +71,21 @@ struct StreamCfg {
     static_assert(NW * OUT_BAND_BYTES <= STAGE_BYTES, "the output bands must fit one ring stage");
     static_assert(LPS + 1 < 64, "vmcnt is a 6-bit counter");
     static_assert(CH == 4 || CH == 8, "slab must be 64 or 128 bytes");
-    static constexpr size_t fixed_lds = (size_t)S * STAGE_BYTES + (size_t)kPlanSlots * IDX_SLOT_BYTES + OROW_BYTES;
+    static constexpr size_t fixed_lds = (size_t)S * STAGE_BYTES + (size_t)kPlanSlots * IDX_SLOT_BYTES + OROW_BYTES + kPlanSlots * 4;
 };
+
+// s_waitcnt vmcnt(n) for a wave-uniform n in [LO, HI]: the count is an immediate, so a binary tree of scalar branches
+// picks the instruction.
+template <int LO, int HI>
+__device__ __forceinline__ void wait_vmcnt_in(int n) {
+    if constexpr (LO == HI) {
+        wait_vmcnt<LO>();
+    } else {
+        constexpr int MID = (LO + HI) / 2;
+        if (n <= MID) wait_vmcnt_in<LO, MID>(n);
+        else wait_vmcnt_in<MID + 1, HI>(n);
+    }
+}
 
 __device__ __forceinline__ void wg_barrier() {
     asm volatile("" ::: "memory");
@@ -85,7 +98,8 @@ __global__ void __launch_bounds__(64 * (WAVES_M * WAVES_N + kLoaders))
 gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const typename Tag::type* __restrict__ panel,
                           const typename Tag::type* __restrict__ bias, const int64_t* __restrict__ order,
                           const int32_t* __restrict__ plan_seg, const int32_t* __restrict__ tile_code,
-                          const uint32_t* __restrict__ plan_idx, uint32_t n, int K, int cols, int cols_pad,
+                          const uint32_t* __restrict__ plan_idx, const uint32_t* __restrict__ plan_band, uint32_t n, int K,
+                          int cols, int cols_pad,
                           unsigned row_tiles, unsigned col_tiles, uint32_t src_bytes, uint32_t panel_bytes,
                           uint32_t plan_bytes, typename Tag::type* __restrict__ out) {
     using C = StreamCfg<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
@@ -96,7 +110,8 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     unsigned char* ring = lds_raw;                                          // [S][A: BM x SLAB | B: BN x SLAB]
     uint32_t* idx_ring = (uint32_t*)(ring + S * C::STAGE_BYTES);            // [kPlanSlots][BM] source rows of one offset
     uint32_t* orow_lds = idx_ring + kPlanSlots * BM;                        // [2][NW][OROW_INST * 64] output rows
-    float* bias_lds = (float*)(orow_lds + C::OROW_BYTES / 4);               // [cols_pad]
+    uint32_t* band_lds = orow_lds + C::OROW_BYTES / 4;                      // [kPlanSlots] band masks, loaders -> multipliers
+    float* bias_lds = (float*)(band_lds + kPlanSlots);                      // [cols_pad]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -158,12 +173,15 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     f_code = f_code ? f_code : 1u;
     // queue of offsets the row stream has not started yet (head first)
     int q_v[kPlanAhead], q_ct[kPlanAhead];
+    uint32_t q_band[kPlanAhead];
     bool q_live[kPlanAhead];
-    auto fetch_slot = [&](int& v, int& ct, bool& live) -> int {     // returns the loads this wavefront issued
+    auto fetch_slot = [&](int& v, int& ct, uint32_t& band, bool& live) -> int {     // returns the loads this wavefront issued
         live = f_live;
         v = 0;
         ct = 0;
+        band = 0;
         if (!f_live) return 0;
+        band = plan_band != nullptr ? plan_band[f_pos] : 0xFFFFFFFFu;
         v = __builtin_ctz(f_code);
         f_code &= f_code - 1;
         ct = (int)f_ct;
@@ -199,19 +217,24 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     // and moves on by one K-slab.
     bool p_ready = false;
     int p_slab = 0, p_ring = 0, p_stage = 0;
-    uint32_t a_soff = 0, b_soff = 0;
+    uint32_t a_soff = 0, b_soff = 0, cur_band = 0;
     const uint32_t b_slab_stride = (uint32_t)cols_pad * kSlabBytes;
     auto slot_begin = [&]() -> int {
         p_ready = q_live[0];
         if (!p_ready) return 0;
         const int v = q_v[0], ct = q_ct[0];
+        cur_band = q_band[0];
 #pragma unroll
         for (int i = 0; i + 1 < kPlanAhead; ++i) {
             q_v[i] = q_v[i + 1];
             q_ct[i] = q_ct[i + 1];
+            q_band[i] = q_band[i + 1];
             q_live[i] = q_live[i + 1];
         }
         const uint32_t* slot = idx_ring + p_ring * BM;
+        // for the multipliers, who fetch it at least two barriers from now; the reads of the index column below are
+        // waited for before this wavefront reaches its next barrier, and LDS finishes a wavefront's accesses in order
+        if (lw == 0 && lane == 0) band_lds[p_ring] = cur_band;
         p_ring = (p_ring + 1) & (kPlanSlots - 1);
 #pragma unroll
         for (int i = 0; i < C::A_PER; ++i) {
@@ -220,18 +243,27 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
         }
         p_slab = 0;
         a_soff = 0;
-        b_soff = ((uint32_t)(v * slabs) * (uint32_t)cols_pad + (uint32_t)(ct * BN)) * kSlabBytes;
-        return fetch_slot(q_v[kPlanAhead - 1], q_ct[kPlanAhead - 1], q_live[kPlanAhead - 1]);
+        // wave-uniform by construction; saying so keeps the panel loads from being wrapped in per-lane loops
+        b_soff = __builtin_amdgcn_readfirstlane(((uint32_t)(v * slabs) * (uint32_t)cols_pad + (uint32_t)(ct * BN)) * kSlabBytes);
+        return fetch_slot(q_v[kPlanAhead - 1], q_ct[kPlanAhead - 1], q_band[kPlanAhead - 1], q_live[kPlanAhead - 1]);
     };
     auto issue_step = [&]() -> int {                     // returns the loads this wavefront issued
         if (!p_ready) return 0;
         unsigned char* stage = ring + p_stage * C::STAGE_BYTES;
         const bool tail = ragged && p_slab == slabs - 1;     // wave-uniform
+        int ops = C::B_PER;
 #pragma unroll
         for (int i = 0; i < C::A_PER; ++i) {
+            // 32-row band of this load's rows (a constant when the loaders' loads of one round make up one band)
+            const int band = C::NL * C::ROWS_PER_INST == 32 ? i : ((i * C::NL + lw) * C::ROWS_PER_INST) >> 5;
+            // a multiplier wavefront skips all TM bands of its tile or none, so the loaders skip on the same groups:
+            // no row of the group has the offset -> nothing to load, and the stage keeps stale data nobody reads
+            constexpr uint32_t kWaveBands = (1u << C::TM) - 1u;
+            if (!((cur_band >> (band / C::TM * C::TM)) & kWaveBands)) continue;
             uint32_t vo = a_voff[i];
             if (tail) vo = a_soff + a_choff[i] < row_bytes ? vo : kOobOffset;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(src_rs, FGX_LDS_PTR(stage + (i * C::NL + lw) * 1024), 16, vo, a_soff, 0, 0);
+            ++ops;
         }
         unsigned char* stage_b = stage + BM * kSlabBytes;
 #pragma unroll
@@ -239,19 +271,14 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
             const uint32_t vo = b_voff[i];
             __builtin_amdgcn_raw_ptr_buffer_load_lds(panel_rs, FGX_LDS_PTR(stage_b + (i * C::NL + lw) * 1024), 16, vo, b_soff, 0, 0);
         }
-        int ops = C::LPS;
         a_soff += kSlabBytes;
-        b_soff += b_slab_stride;
+        b_soff = __builtin_amdgcn_readfirstlane(b_soff + b_slab_stride);
         p_stage = p_stage + 1 == S ? 0 : p_stage + 1;
         if (++p_slab == slabs) ops += slot_begin();
         return ops;
     };
-    // at most `n` of this loader's loads may still be outstanding; n is 0, LPS or LPS + 1
-    auto wait_loads = [&](int n) {
-        if (n > C::LPS) wait_vmcnt<C::LPS + 1>();
-        else if (n == C::LPS) wait_vmcnt<C::LPS>();
-        else wait_vmcnt<0>();
-    };
+    // at most `n` of this loader's loads may still be outstanding; n is wave-uniform, 0 .. LPS + 1
+    auto wait_loads = [&](int n) { wait_vmcnt_in<0, C::LPS + 1>(n); };
 
     // =================================================================================================
     // Multiplier state
@@ -279,43 +306,47 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     constexpr int ROWS_PER_PASS = 64 / PIECES;
     const bool vec_ok = (cols * C::ES) % 16 == 0;             // output rows start on 16-byte boundaries
 
-    // ---- item walk shared by both roles (same barriers in the same order) ----
-    unsigned c_it = first_item, c_t = first_rev / col_tiles, c_ct = first_rev % col_tiles;
-    int c_slots = __popc((uint32_t)tile_code[c_t]);
-
-    // ---- prologue ----
-    int ops_prev = 0;
-    if (loader) {
-#pragma unroll
-        for (int i = 0; i < kPlanAhead; ++i) (void)fetch_slot(q_v[i], q_ct[i], q_live[i]);
-    } else {
-        fetch_orow(c_t, 0);
-    }
-    wait_vmcnt<0>();
-    __syncthreads();          // index columns landed; also publishes bias_lds
-    if (loader) (void)slot_begin();
-#pragma unroll
-    for (int s = 0; s < S - 1; ++s) {
-        wait_vmcnt<0>();
-        __syncthreads();
-        if (loader) ops_prev = issue_step();
-    }
-
-    int cur_stage = 0, parity = 0;
-    while (true) {
-        const int nsteps = (c_slots > 0 ? c_slots : 1) * slabs;
-        // the item after this one (its output rows are fetched now, its size is read now)
-        unsigned n_it = c_it + G, n_t = c_t - dt, n_ct = c_ct;
-        if (n_ct < dct) {
-            n_ct += col_tiles;
-            --n_t;
+    // ---- item walk.  Both roles walk the same items and meet at the same barriers in the same order, but each runs
+    // its own loop, so that neither role's registers stay live through the other's code. ----
+    struct Item {
+        unsigned it, t, ct;
+        int slots;
+    };
+    Item cur_item{first_item, first_rev / col_tiles, first_rev % col_tiles, 0};
+    cur_item.slots = __popc((uint32_t)tile_code[cur_item.t]);
+    auto following = [&](const Item& c, Item& nx) -> bool {     // the item G further on; false past the end
+        nx.it = c.it + G;
+        nx.t = c.t - dt;
+        nx.ct = c.ct;
+        if (nx.ct < dct) {
+            nx.ct += col_tiles;
+            --nx.t;
         }
-        n_ct -= dct;
-        const bool has_next = n_it < total_items;
-        int n_slots = 0;
-        if (has_next) n_slots = __popc((uint32_t)tile_code[n_t]);
+        nx.ct -= dct;
+        nx.slots = 0;
+        if (nx.it >= total_items) return false;
+        nx.slots = __popc((uint32_t)tile_code[nx.t]);
+        return true;
+    };
 
-        if (loader) {
+    if (loader) {
+        // ---- prologue: index columns of the first kPlanAhead offsets, then the rows of the first S-1 steps ----
+#pragma unroll
+        for (int i = 0; i < kPlanAhead; ++i) (void)fetch_slot(q_v[i], q_ct[i], q_band[i], q_live[i]);
+        wait_vmcnt<0>();
+        __syncthreads();          // index columns landed; also publishes bias_lds
+        (void)slot_begin();
+        int ops_prev = 0;
+#pragma unroll
+        for (int s = 0; s < S - 1; ++s) {
+            wait_vmcnt<0>();
+            __syncthreads();
+            ops_prev = issue_step();
+        }
+        while (true) {
+            const int nsteps = (cur_item.slots > 0 ? cur_item.slots : 1) * slabs;
+            Item nx;
+            const bool has_next = following(cur_item, nx);
             for (int s = 0; s < nsteps; ++s) {
                 // everything this loader issued before its previous iteration has landed: its share of this step's rows
                 wait_loads(ops_prev);
@@ -323,19 +354,52 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
                 ops_prev = issue_step();
             }
             wg_barrier();                  // the multipliers' "done reading the last stage"
-        } else {
-            f32x16 acc[C::TM][C::TN];
+            if (!has_next) break;
+            cur_item = nx;
+        }
+        wait_vmcnt<0>();
+        return;
+    }
+
+    // ---- multipliers ----
+    fetch_orow(cur_item.t, 0);
+    wait_vmcnt<0>();
+    __syncthreads();
 #pragma unroll
-            for (int i = 0; i < C::TM; ++i)
+    for (int s = 0; s < S - 1; ++s) __syncthreads();
+
+    int cur_stage = 0, parity = 0;
+    // position in the band-mask ring, K-slab inside the current offset, this wavefront's bits of the offset's mask
+    constexpr uint32_t kMineAll = (1u << C::TM) - 1u;
+    int m_ring = 1, m_slab = 0;
+    uint32_t m_mine = kMineAll, m_next = band_lds[0];
+    while (true) {
+        const int nsteps = (cur_item.slots > 0 ? cur_item.slots : 1) * slabs;
+        // the item after this one (its output rows are fetched now, its size is read now)
+        Item nx;
+        const bool has_next = following(cur_item, nx);
+        const unsigned c_t = cur_item.t, c_ct = cur_item.ct, n_t = nx.t;
+        f32x16 acc[C::TM][C::TN];
 #pragma unroll
-                for (int j = 0; j < C::TN; ++j)
+        for (int i = 0; i < C::TM; ++i)
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-            if (has_next) fetch_orow(n_t, parity ^ 1);
-            for (int s = 0; s < nsteps; ++s) {
-                wg_barrier();              // the loaders saw this step's rows land
-                const unsigned char* cur = ring + cur_stage * C::STAGE_BYTES;
-                cur_stage = cur_stage + 1 == S ? 0 : cur_stage + 1;
+            for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        if (has_next) fetch_orow(n_t, parity ^ 1);
+        for (int s = 0; s < nsteps; ++s) {
+            wg_barrier();              // the loaders saw this step's rows land
+            const unsigned char* cur = ring + cur_stage * C::STAGE_BYTES;
+            cur_stage = cur_stage + 1 == S ? 0 : cur_stage + 1;
+            if (m_slab == 0) m_mine = (__builtin_amdgcn_readfirstlane(m_next) >> (wave_m * C::TM)) & kMineAll;
+            m_slab = m_slab + 1 == slabs ? 0 : m_slab + 1;
+            // last K-slab of an offset: fetch the mask of the next one (published at least two barriers ago); the
+            // wait for this step's fragments covers it
+            if (m_slab == 0) {
+                m_next = band_lds[m_ring];
+                m_ring = (m_ring + 1) & (kPlanSlots - 1);
+            }
+            if (m_mine != 0) {
                 u32x4 af[kChunks / 2][C::TM], bf[kChunks / 2][C::TN];
 #pragma unroll
                 for (int kk = 0; kk < kChunks / 2; ++kk) {
@@ -351,63 +415,60 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
 #pragma unroll
                         for (int j = 0; j < C::TN; ++j) mma<Tag>(acc[i][j], bf[kk][j], af[kk][i]);   // transposed tile
             }
+        }
 
-            // ---- epilogue.  The MFMAs ran with the operands swapped, so a 32x32 accumulator holds the TRANSPOSED
-            // tile: element e of lane l belongs to output row l%32 and column 8*(e/4) + 4*(l/32) + e%4 -- four
-            // adjacent columns per (lane, e/4), which go to LDS as one 8- or 16-byte store.
-            wait_vmcnt<0>();               // this item's output rows (fetched an item ago) and older stores
-            wg_barrier();                  // everybody is done reading the last stage
-            const int last = cur_stage == 0 ? S - 1 : cur_stage - 1;
-            unsigned char* band = ring + last * C::STAGE_BYTES + mw * C::OUT_BAND_BYTES;
-            const uint32_t* my_orow = orow_lds + (parity * C::NW + mw) * C::OROW_INST * 64;
-            const int col0 = (int)c_ct * BN + wave_n * C::WN;
-            constexpr int HALVES = 32 / C::BAND_ROWS;
+        // ---- epilogue.  The MFMAs ran with the operands swapped, so a 32x32 accumulator holds the TRANSPOSED
+        // tile: element e of lane l belongs to output row l%32 and column 8*(e/4) + 4*(l/32) + e%4 -- four
+        // adjacent columns per (lane, e/4), which go to LDS as one 8- or 16-byte store.
+        wait_vmcnt<0>();               // this item's output rows (fetched an item ago) and older stores
+        wg_barrier();                  // everybody is done reading the last stage
+        const int last = cur_stage == 0 ? S - 1 : cur_stage - 1;
+        unsigned char* band = ring + last * C::STAGE_BYTES + mw * C::OUT_BAND_BYTES;
+        const uint32_t* my_orow = orow_lds + (parity * C::NW + mw) * C::OROW_INST * 64;
+        const int col0 = (int)c_ct * BN + wave_n * C::WN;
+        constexpr int HALVES = 32 / C::BAND_ROWS;
 #pragma unroll
-            for (int ih = 0; ih < C::TM * HALVES; ++ih) {
-                const int i = ih / HALVES, h = ih % HALVES;      // 32-row tile, half of it
-                if (HALVES == 1 || (l32 >> 4) == h) {
-                    const int r = l32 - h * C::BAND_ROWS;
+        for (int ih = 0; ih < C::TM * HALVES; ++ih) {
+            const int i = ih / HALVES, h = ih % HALVES;      // 32-row tile, half of it
+            if (HALVES == 1 || (l32 >> 4) == h) {
+                const int r = l32 - h * C::BAND_ROWS;
 #pragma unroll
-                    for (int j = 0; j < C::TN; ++j)
+                for (int j = 0; j < C::TN; ++j)
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) {
-                            const int c = j * 32 + q * 8 + g * 4;                   // first of four columns
-                            const f32x4 bv = *(const f32x4*)(bias_lds + col0 + c);
-                            T pk[4];
-                            pk[0] = from_float<T>(acc[i][j][q * 4 + 0] + bv.x);
-                            pk[1] = from_float<T>(acc[i][j][q * 4 + 1] + bv.y);
-                            pk[2] = from_float<T>(acc[i][j][q * 4 + 2] + bv.z);
-                            pk[3] = from_float<T>(acc[i][j][q * 4 + 3] + bv.w);
-                            unsigned char* dstp = band + r * C::OUT_PITCH + c * C::ES;
-                            if constexpr (C::ES == 2) *(uint64_t*)dstp = __builtin_bit_cast(uint64_t, pk);
-                            else *(u32x4*)dstp = __builtin_bit_cast(u32x4, pk);
-                        }
-                }
-                // same wavefront wrote and reads: program order inside the wavefront suffices for LDS
-#pragma unroll
-                for (int pass = 0; pass < C::BAND_ROWS / ROWS_PER_PASS; ++pass) {
-                    const int r = pass * ROWS_PER_PASS + lane / PIECES;
-                    const int piece = lane % PIECES;
-                    const int tr = i * 32 + h * C::BAND_ROWS + r;                      // row inside the wave tile
-                    const bool live = c_t * (uint32_t)BM + (uint32_t)(wave_m * C::WM + tr) < n;
-                    const uint32_t orow = my_orow[tr];
-                    const int col = col0 + piece * (16 / C::ES);
-                    if (!live || col >= cols) continue;
-                    const unsigned char* sp = band + r * C::OUT_PITCH + piece * 16;
-                    T* dp = out + (size_t)orow * cols + col;
-                    if (vec_ok && col + 16 / C::ES <= cols) {
-                        *(u32x4*)dp = *(const u32x4*)sp;
-                    } else {
-                        for (int t = 0; t < 16 / C::ES && col + t < cols; ++t) dp[t] = ((const T*)sp)[t];
+                    for (int q = 0; q < 4; ++q) {
+                        const int c = j * 32 + q * 8 + g * 4;                   // first of four columns
+                        const f32x4 bv = *(const f32x4*)(bias_lds + col0 + c);
+                        T pk[4];
+                        pk[0] = from_float<T>(acc[i][j][q * 4 + 0] + bv.x);
+                        pk[1] = from_float<T>(acc[i][j][q * 4 + 1] + bv.y);
+                        pk[2] = from_float<T>(acc[i][j][q * 4 + 2] + bv.z);
+                        pk[3] = from_float<T>(acc[i][j][q * 4 + 3] + bv.w);
+                        unsigned char* dstp = band + r * C::OUT_PITCH + c * C::ES;
+                        if constexpr (C::ES == 2) *(uint64_t*)dstp = __builtin_bit_cast(uint64_t, pk);
+                        else *(u32x4*)dstp = __builtin_bit_cast(u32x4, pk);
                     }
+            }
+            // same wavefront wrote and reads: program order inside the wavefront suffices for LDS
+#pragma unroll
+            for (int pass = 0; pass < C::BAND_ROWS / ROWS_PER_PASS; ++pass) {
+                const int r = pass * ROWS_PER_PASS + lane / PIECES;
+                const int piece = lane % PIECES;
+                const int tr = i * 32 + h * C::BAND_ROWS + r;                      // row inside the wave tile
+                const bool live = c_t * (uint32_t)BM + (uint32_t)(wave_m * C::WM + tr) < n;
+                const uint32_t orow = my_orow[tr];
+                const int col = col0 + piece * (16 / C::ES);
+                if (!live || col >= cols) continue;
+                const unsigned char* sp = band + r * C::OUT_PITCH + piece * 16;
+                T* dp = out + (size_t)orow * cols + col;
+                if (vec_ok && col + 16 / C::ES <= cols) {
+                    *(u32x4*)dp = *(const u32x4*)sp;
+                } else {
+                    for (int t = 0; t < 16 / C::ES && col + t < cols; ++t) dp[t] = ((const T*)sp)[t];
                 }
             }
         }
         if (!has_next) break;
-        c_it = n_it;
-        c_t = n_t;
-        c_ct = n_ct;
-        c_slots = n_slots;
+        cur_item = nx;
         parity ^= 1;
     }
     wait_vmcnt<0>();
@@ -415,8 +476,8 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
 
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int CH>
 int launch_stream(const void* src, const void* panel, const void* bias, const int64_t* order, const int32_t* plan_seg,
-                  const int32_t* tile_code, const uint32_t* plan_idx, size_t plan_rows, size_t n, int K, int cols,
-                  int cols_pad, size_t panel_bytes, int max_groups, void* out, hipStream_t s) {
+                  const int32_t* tile_code, const uint32_t* plan_idx, const uint32_t* plan_band, size_t plan_rows, size_t n,
+                  int K, int cols, int cols_pad, size_t panel_bytes, int max_groups, void* out, hipStream_t s) {
     using C = StreamCfg<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
     using T = typename Tag::type;
     auto kern = gather_gemm_stream_kernel<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
@@ -434,7 +495,7 @@ int launch_stream(const void* src, const void* panel, const void* bias, const in
     const size_t total = (size_t)row_tiles * col_tiles;
     unsigned groups = (unsigned)(total < (size_t)max_groups ? total : (size_t)max_groups);
     kern<<<groups, C::NT, lds, s>>>((const T*)src, (const T*)panel, (const T*)bias, order, plan_seg, tile_code, plan_idx,
-                                    (uint32_t)n, K, cols, cols_pad, row_tiles, col_tiles,
+                                    plan_band, (uint32_t)n, K, cols, cols_pad, row_tiles, col_tiles,
                                     (uint32_t)(n * (size_t)K * sizeof(T)), (uint32_t)panel_bytes,
                                     (uint32_t)(plan_rows * BM * 4), (T*)out);
     FGX_CHECK_LAUNCH("fgx_conv_gather_gemm_stream");
@@ -444,12 +505,12 @@ int launch_stream(const void* src, const void* panel, const void* bias, const in
 template <typename Tag>
 int dispatch_stream(int tile_rows, int tile_cols, int slab_bytes, const void* src, const void* panel, const void* bias,
                     const int64_t* order, const int32_t* plan_seg, const int32_t* tile_code, const uint32_t* plan_idx,
-                    size_t plan_rows, size_t n, int K, int cols, int cols_pad, size_t panel_bytes, int max_groups,
-                    void* out, hipStream_t s) {
+                    const uint32_t* plan_band, size_t plan_rows, size_t n, int K, int cols, int cols_pad,
+                    size_t panel_bytes, int max_groups, void* out, hipStream_t s) {
 #define FGX_STREAM_TILE(BM, BN, WMv, WNv, CHv)                                                                          \
     if (tile_rows == BM && tile_cols == BN && slab_bytes == CHv * 16)                                                   \
-        return launch_stream<Tag, BM, BN, WMv, WNv, CHv>(src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_rows, \
-                                                         n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
+        return launch_stream<Tag, BM, BN, WMv, WNv, CHv>(src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band,  \
+                                                         plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
     FGX_STREAM_TILE(256, 128, 4, 2, 8)
     FGX_STREAM_TILE(256, 64, 4, 2, 8)
 #undef FGX_STREAM_TILE
@@ -464,7 +525,8 @@ using namespace fgx;
 
 extern "C" int fgx_conv_gather_gemm_stream(int dtype, const void* src, const void* panel, const void* bias,
                                            const int64_t* order, const int32_t* tile_code, const int32_t* plan_seg,
-                                           const uint32_t* plan_idx, size_t plan_rows, size_t n, int K, int cols, int V,
+                                           const uint32_t* plan_idx, const uint32_t* plan_band, size_t plan_rows, size_t n,
+                                           int K, int cols, int V,
                                            int tile_rows, int tile_cols, int slab_bytes, int max_groups, void* out,
                                            fgx_stream_t stream) {
     FGX_CHECK_ARG(dtype == FGX_F16 || dtype == FGX_BF16 || dtype == FGX_F32, "fgx_conv_gather_gemm_stream: unknown dtype %d", dtype);
@@ -476,6 +538,7 @@ extern "C" int fgx_conv_gather_gemm_stream(int dtype, const void* src, const voi
     FGX_CHECK_ARG((((uintptr_t)src | (uintptr_t)panel | (uintptr_t)plan_idx) & 15) == 0,
                   "fgx_conv_gather_gemm_stream: src, panel and plan_idx must be 16-byte aligned");
     FGX_CHECK_ARG(tile_rows > 0 && tile_cols > 0 && (slab_bytes == 64 || slab_bytes == 128), "fgx_conv_gather_gemm_stream: bad schedule");
+    FGX_CHECK_ARG(plan_band == nullptr || tile_rows <= 1024, "fgx_conv_gather_gemm_stream: band masks cover tiles of at most 1024 rows");
     if (max_groups <= 0) {
         int dev = 0, cus = 0;
         FGX_CHECK_HIP(hipGetDevice(&dev));
@@ -493,8 +556,8 @@ extern "C" int fgx_conv_gather_gemm_stream(int dtype, const void* src, const voi
     }
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
-        case FGX_F16: return dispatch_stream<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
-        case FGX_BF16: return dispatch_stream<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
-        default: return dispatch_stream<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
+        case FGX_F16: return dispatch_stream<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
+        case FGX_BF16: return dispatch_stream<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
+        default: return dispatch_stream<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
     }
 }

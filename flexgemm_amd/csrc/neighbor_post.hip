@@ -220,31 +220,54 @@ __global__ void __launch_bounds__(kBlock) plan_count_kernel(const int32_t* __res
 }
 
 // One workgroup per tile: plan_idx[seg[t] + k][r] = map[order[t * tile_rows + r]][k-th offset present in the tile]
-// (EMPTY for rows past the end).
+// (EMPTY for rows past the end); plan_band[seg[t] + k] (optional) has bit b set when rows [32 b, 32 b + 32) of the
+// tile hold at least one present neighbor for that offset.
 __global__ void __launch_bounds__(kBlock) plan_fill_kernel(const uint32_t* __restrict__ map,
                                                            const int64_t* __restrict__ order,
                                                            const int32_t* __restrict__ tile_code,
                                                            const int32_t* __restrict__ seg, size_t n, int V, int tile_rows,
-                                                           uint32_t* __restrict__ plan_idx) {
+                                                           uint32_t* __restrict__ plan_idx, uint32_t* __restrict__ plan_band) {
+    __shared__ uint32_t bands[32];
     const size_t t = blockIdx.x;
     uint32_t code = (uint32_t)tile_code[t];
     size_t slot = (size_t)seg[t];
     if (code == 0) {
         for (int r = threadIdx.x; r < tile_rows; r += kBlock) plan_idx[slot * tile_rows + r] = FGX_EMPTY32;
+        if (plan_band != nullptr && threadIdx.x == 0) plan_band[slot] = 0u;
         return;
     }
+    if (threadIdx.x < 32) bands[threadIdx.x] = 0u;
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
     for (int r0 = 0; r0 < tile_rows; r0 += kBlock) {
         const int r = r0 + threadIdx.x;
         const size_t row = t * (size_t)tile_rows + r;
         const uint32_t* mrow = (r < tile_rows && row < n) ? map + (size_t)order[row] * V : nullptr;
         uint32_t c = code;
         size_t s = slot;
+        int k = 0;
         while (c) {
             const int v = __ffs((int)c) - 1;
             c &= c - 1;
-            if (r < tile_rows) plan_idx[s * tile_rows + r] = mrow ? mrow[v] : FGX_EMPTY32;
+            const uint32_t m = mrow ? mrow[v] : FGX_EMPTY32;
+            if (r < tile_rows) plan_idx[s * tile_rows + r] = m;
+            if (plan_band != nullptr) {
+                const unsigned long long live = __ballot(m != FGX_EMPTY32);    // all 64 lanes take part
+                if (lane == 0) {
+                    const int b0 = (r0 + (int)(threadIdx.x & ~63u)) >> 5;          // band of this wavefront's lanes 0-31
+                    uint32_t bits = ((live & 0xFFFFFFFFull) ? 1u : 0u) << (b0 & 31);
+                    bits |= ((live >> 32) ? 1u : 0u) << ((b0 + 1) & 31);
+                    if (bits) atomicOr(&bands[k], bits);
+                }
+            }
             ++s;
+            ++k;
         }
+    }
+    if (plan_band != nullptr) {
+        __syncthreads();
+        const int cnt = __popc(code);
+        if ((int)threadIdx.x < cnt) plan_band[slot + threadIdx.x] = bands[threadIdx.x];
     }
 }
 
@@ -461,14 +484,15 @@ int fgx_gather_plan_count(const int32_t* tile_code, size_t num_tiles, int32_t* p
 }
 
 int fgx_gather_plan_fill(const uint32_t* map, const int64_t* order, const int32_t* tile_code, const int32_t* plan_seg,
-                         size_t n, int V, int tile_rows, uint32_t* plan_idx, fgx_stream_t stream) {
+                         size_t n, int V, int tile_rows, uint32_t* plan_idx, uint32_t* plan_band, fgx_stream_t stream) {
     FGX_CHECK_ARG(tile_rows >= 1 && V >= 1 && V <= 32, "fgx_gather_plan_fill: bad shape tile_rows=%d V=%d", tile_rows, V);
     if (n == 0) return FGX_OK;
     FGX_CHECK_ARG(map && order && tile_code && plan_seg && plan_idx, "fgx_gather_plan_fill: null buffer");
     const size_t num_tiles = (n + tile_rows - 1) / tile_rows;
     FGX_CHECK_ARG(num_tiles <= 0x7FFFFFFFu, "fgx_gather_plan_fill: too many tiles");
+    FGX_CHECK_ARG(plan_band == nullptr || tile_rows <= 1024, "fgx_gather_plan_fill: band masks need tile_rows <= 1024");
     plan_fill_kernel<<<(unsigned)num_tiles, kBlock, 0, (hipStream_t)stream>>>(map, order, tile_code, plan_seg, n, V, tile_rows,
-                                                                              plan_idx);
+                                                                              plan_idx, plan_band);
     FGX_CHECK_LAUNCH("fgx_gather_plan_fill");
     return FGX_OK;
 }

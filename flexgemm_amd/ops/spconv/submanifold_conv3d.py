@@ -100,9 +100,10 @@ class SubMConv3dNeighborCache:
         return self["_dense_order"], getattr(self, key)
 
     def _gather_plan(self, block_size: int, private: bool, dense: bool = False):
-        """(order, tile_code int32 [nb], plan_seg int32 [nb+1], plan_idx uint32 [P, block_size]) for the streaming
-        GEMM: per tile and offset present in it, the tile's source rows as one contiguous run.  Built once per tile size
-        (one 4-byte read-back sizes it) and kept with the cache."""
+        """(order, tile_code int32 [nb], plan_seg int32 [nb+1], plan_idx uint32 [P, block_size], plan_band uint32 [P])
+        for the streaming GEMM: per tile and offset present in it, the tile's source rows as one contiguous run and the
+        mask of its 32-row bands that hold any.  Built once per tile size (one 4-byte read-back sizes it) and kept with
+        the cache."""
         if dense:
             order, code = self._dense_tile_tables(block_size)
             key = f"_plan_d_{block_size}"
@@ -123,9 +124,11 @@ class SubMConv3dNeighborCache:
                                                   nat.stream()))
                 rows = int(seg[-1].item())
                 plan_idx = torch.empty((rows, block_size), dtype=torch.uint32, device=dev)
+                plan_band = torch.empty((rows,), dtype=torch.uint32, device=dev)
                 nat.check(L.fgx_gather_plan_fill(nat.ptr(nmap), nat.ptr(order), nat.ptr(code), nat.ptr(seg), nat.sz(n),
-                                                 C.c_int(v), C.c_int(block_size), nat.ptr(plan_idx), nat.stream()))
-            setattr(self, key, (seg, plan_idx))
+                                                 C.c_int(v), C.c_int(block_size), nat.ptr(plan_idx), nat.ptr(plan_band),
+                                                 nat.stream()))
+            setattr(self, key, (seg, plan_idx, plan_band))
         return (order, code) + getattr(self, key)
 
     def compute_kernel_idx(self, block_size: int):
@@ -319,11 +322,12 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
         nat.check(L.fgx_pack_weight(C.c_int(code), C.c_int(mode), nat.ptr(weight_cvk), C.c_int(ci), C.c_int(co), C.c_int(v),
                                     C.c_int(sched.slab_bytes), C.c_int(sched.tile_cols), nat.ptr(panel), nat.stream()))
         if sched.stream and _stream_fits(n, k * src.element_size()):
-            order, tile_code, plan_seg, plan_idx = cache._gather_plan(sched.tile_rows, private, dense=not masked)
+            order, tile_code, plan_seg, plan_idx, plan_band = cache._gather_plan(sched.tile_rows, private, dense=not masked)
             nat.mark(name, "start")
             nat.check(L.fgx_conv_gather_gemm_stream(
                 C.c_int(code), nat.ptr(src), nat.ptr(panel), nat.ptr(bias), nat.ptr(order), nat.ptr(tile_code),
-                nat.ptr(plan_seg), nat.ptr(plan_idx), nat.sz(plan_idx.shape[0]), nat.sz(n), C.c_int(k), C.c_int(cols), C.c_int(v),
+                nat.ptr(plan_seg), nat.ptr(plan_idx), nat.ptr(plan_band), nat.sz(plan_idx.shape[0]), nat.sz(n), C.c_int(k),
+                C.c_int(cols), C.c_int(v),
                 C.c_int(sched.tile_rows), C.c_int(sched.tile_cols), C.c_int(sched.slab_bytes), C.c_int(0), nat.ptr(out),
                 nat.stream()))
             nat.mark(name, "stop")

@@ -181,9 +181,11 @@ int fgx_conv_gather_gemm(int dtype, const void* src, const void* panel, const vo
 
 /* Gather plan of a row order for tiles of `tile_rows` rows: for tile t and the k-th offset v present in it
  * (the set bits of tile_code[t], ascending; a tile whose code is 0 gets one row with every neighbor missing),
- *   plan_idx[(plan_seg[t] + k) * tile_rows + r] = map[order[t * tile_rows + r], v]     (0xFFFFFFFF for rows past n).
+ *   plan_idx[(plan_seg[t] + k) * tile_rows + r] = map[order[t * tile_rows + r], v]     (0xFFFFFFFF for rows past n),
+ *   plan_band[plan_seg[t] + k] bit b = 1 iff rows [32 b, 32 b + 32) of the tile have a neighbor at v   (optional).
  * count: plan_seg[num_tiles + 1] <- exclusive offsets, plan_seg[num_tiles] = plan rows; the caller reads that back,
- * allocates plan_idx (tile_rows uint32 per plan row, 16-byte aligned) and calls fill.  `tile_code` comes from
+ * allocates plan_idx (tile_rows uint32 per plan row, 16-byte aligned) and plan_band (one uint32 per plan row, may be
+ * NULL; needs tile_rows <= 1024) and calls fill.  `tile_code` comes from
  * fgx_tile_codes on the same order and tile size; workspace: fgx_tile_workspace_bytes(num_tiles, 1) bytes,
  * 256-byte aligned.
  * Replaces: the neighbor[sorted_idx[rows], v] double gather inside the Triton kernels
@@ -192,17 +194,19 @@ int fgx_conv_gather_gemm(int dtype, const void* src, const void* panel, const vo
 int fgx_gather_plan_count(const int32_t* tile_code, size_t num_tiles, int32_t* plan_seg, void* workspace,
                           size_t workspace_bytes, fgx_stream_t stream);
 int fgx_gather_plan_fill(const uint32_t* map, const int64_t* order, const int32_t* tile_code, const int32_t* plan_seg,
-                         size_t n, int V, int tile_rows, uint32_t* plan_idx, fgx_stream_t stream);
+                         size_t n, int V, int tile_rows, uint32_t* plan_idx, uint32_t* plan_band, fgx_stream_t stream);
 
 /* Same result as fgx_conv_gather_gemm (splitk = 1) from the gather plan of `order`, by persistent workgroups that
  * stream all their tiles' (offset, K-slab) steps back to back; meant for voxel counts that give every CU several
  * tiles.  `max_groups`: workgroups to launch (<= 0: one per CU).  Operands are addressed with 32-bit offsets:
  * returns FGX_ERR_UNSUPPORTED when src, the panel or the plan exceed ~4 GB, or when no kernel exists for the
- * schedule -- callers then use fgx_conv_gather_gemm.
+ * schedule -- callers then use fgx_conv_gather_gemm.  `plan_band` (from fgx_gather_plan_fill; NULL = every band
+ * present) lets the kernel skip the loads and products of 32-row bands without a neighbor at an offset.
  * Replaces: the same reference kernels as fgx_conv_gather_gemm. */
 int fgx_conv_gather_gemm_stream(int dtype, const void* src, const void* panel, const void* bias,
                                 const int64_t* order, const int32_t* tile_code, const int32_t* plan_seg,
-                                const uint32_t* plan_idx, size_t plan_rows, size_t n, int K, int cols, int V,
+                                const uint32_t* plan_idx, const uint32_t* plan_band, size_t plan_rows, size_t n,
+                                int K, int cols, int V,
                                 int tile_rows, int tile_cols, int slab_bytes, int max_groups, void* out,
                                 fgx_stream_t stream);
 

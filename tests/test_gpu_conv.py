@@ -270,6 +270,33 @@ def test_streaming_kernel_equals_tiled_kernel_bitwise(gpu_device):
     assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
 
 
+def test_gather_plan_band_masks(gpu_device):
+    """plan_band bit b of a plan row says whether rows [32 b, 32 b + 32) of that row's index column hold a neighbor;
+    the shell with scattered isolated voxels gives full, partial and (for the tail tile) sparse masks."""
+    _say("gather plan band masks")
+    res = 40
+    shell = reference_test_shell(res)
+    rng = np.random.default_rng(11)
+    lonely = (np.stack([np.zeros(300, np.int32), rng.integers(0, 13, 300), rng.integers(0, 13, 300), rng.integers(0, 13, 300)], 1) * 3).astype(np.int32)
+    lonely = lonely[np.unique(lonely, axis=0, return_index=True)[1]]
+    lonely[:, 0] = 1
+    coords_np = np.concatenate([shell, lonely], 0).astype(np.int32)
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    shape = torch.Size([2, 8, res, res, res])
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+    for dense in (False, True):
+        order, code, seg, plan_idx, plan_band = cache._gather_plan(256, False, dense=dense)
+        torch.cuda.synchronize()
+        idx = plan_idx.cpu().numpy()
+        got = plan_band.cpu().numpy()
+        live = (idx != 0xFFFFFFFF).reshape(idx.shape[0], 8, 32).any(axis=2)
+        want = (live.astype(np.uint32) << np.arange(8, dtype=np.uint32)).sum(axis=1).astype(np.uint32)
+        assert np.array_equal(got, want)
+        assert idx.shape[0] == int(seg.cpu()[-1])
+        if not dense:
+            assert (got != 0xFF).any() and (got == 0xFF).any()
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("res,ci,co,tile,block_rows", [(32, 128, 128, 128, 1024), (24, 64, 64, 64, 512), (24, 96, 40, 128, 300),
                                                        (16, 256, 136, 128, 100000), (48, 128, 128, 128, 37)])

@@ -57,16 +57,21 @@ def test_cache_matches_oracle_reference_geometry(gpu_device, res, needs_grad):
     coords_np = reference_test_shell(res)
     coords = torch.from_numpy(coords_np).to(gpu_device)
     shape = torch.Size([1, 0, res, res, res])
-    for algo in (Algorithm.MASKED_IMPLICIT_GEMM_SPLITK, Algorithm.MASKED_IMPLICIT_GEMM, Algorithm.IMPLICIT_GEMM):
-        flex_gemm.ops.spconv.set_algorithm(algo)
-        cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), needs_grad)
-        _check_cache(cache, coords_np, shape, needs_grad)
-    flex_gemm.ops.spconv.set_algorithm(Algorithm.EXPLICIT_GEMM)
-    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), needs_grad)
-    assert np.array_equal(_np(cache.neighbor_map), nb.neighbor_map(coords_np, tuple(shape)))
-    torch_cache = SubMConv3dFunction._compute_neighbor_cache_torch(coords, shape, (3, 3, 3), (1, 1, 1))
-    assert torch.equal(cache.neighbor_map.view(torch.int32), torch_cache.neighbor_map.view(torch.int32))
-    flex_gemm.ops.spconv.set_algorithm(Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
+    try:
+        for algo in (Algorithm.MASKED_IMPLICIT_GEMM_SPLITK, Algorithm.MASKED_IMPLICIT_GEMM):
+            flex_gemm.ops.spconv.set_algorithm(algo)
+            cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), needs_grad)
+            _check_cache(cache, coords_np, shape, needs_grad)
+        # the other algorithms keep the neighbor map alone (reference submanifold_conv3d.py:59-71)
+        for algo in (Algorithm.IMPLICIT_GEMM, Algorithm.IMPLICIT_GEMM_SPLITK, Algorithm.EXPLICIT_GEMM):
+            flex_gemm.ops.spconv.set_algorithm(algo)
+            cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), needs_grad)
+            assert [k for k in vars(cache) if not k.startswith("_")] == ["neighbor_map"]
+            assert np.array_equal(_np(cache.neighbor_map), nb.neighbor_map(coords_np, tuple(shape)))
+        torch_cache = SubMConv3dFunction._compute_neighbor_cache_torch(coords, shape, (3, 3, 3), (1, 1, 1))
+        assert torch.equal(cache.neighbor_map.view(torch.int32), torch_cache.neighbor_map.view(torch.int32))
+    finally:
+        flex_gemm.ops.spconv.set_algorithm(Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
 
 
 def test_cache_shuffled_batched_dilated(gpu_device):
