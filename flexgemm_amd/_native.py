@@ -33,6 +33,8 @@ EXPORTS = [
     "fgx_gather_plan_count", "fgx_gather_plan_fill", "fgx_conv_gather_gemm_stream",
     "fgx_wgrad_scratch_bytes", "fgx_conv_wgrad",
     "fgx_colsum_scratch_bytes", "fgx_colsum",
+    "fgx_spconv_out_dims", "fgx_spconv_out_coords_workspace_bytes", "fgx_spconv_out_coords_keys",
+    "fgx_spconv_out_coords_decode", "fgx_spconv_neighbor_map",
 ]
 
 
@@ -71,7 +73,7 @@ def lib() -> C.CDLL:
         L.fgx_last_error.restype = C.c_char_p
         for name in ("fgx_sort_workspace_bytes", "fgx_locality_workspace_bytes", "fgx_pair_workspace_bytes", "fgx_tile_workspace_bytes",
                      "fgx_weight_panel_bytes", "fgx_conv_scratch_bytes", "fgx_wgrad_scratch_bytes",
-                     "fgx_colsum_scratch_bytes"):
+                     "fgx_colsum_scratch_bytes", "fgx_spconv_out_coords_workspace_bytes"):
             getattr(L, name).restype = C.c_size_t
         _lib = L
     return _lib

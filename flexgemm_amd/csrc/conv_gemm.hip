@@ -44,7 +44,8 @@ __device__ __attribute__((aligned(16))) const uint32_t g_empty_word[4] = {FGX_EM
 // ------------------------------------------------------------------------------------------------
 // Weight panels
 // ------------------------------------------------------------------------------------------------
-// panel[v][slab][col][k] with k in [0, SK); mode 0: w[col][v][slab*SK+k]; mode 1: w[slab*SK+k][V-1-v][col].
+// panel[v][slab][col][k] with k in [0, SK); mode 0: w[col][v][slab*SK+k]; mode 1: w[slab*SK+k][V-1-v][col];
+// mode 2: w[slab*SK+k][v][col] (input gradient through a separate backward map, no mirroring of v).
 template <typename T>
 __global__ void __launch_bounds__(256) pack_weight_kernel(const T* __restrict__ w, int Ci, int Co, int V, int mode,
                                                           int slab_bytes, int slabs, int cols_pad, T* __restrict__ panel) {
@@ -63,7 +64,7 @@ __global__ void __launch_bounds__(256) pack_weight_kernel(const T* __restrict__ 
         T val = (T)0;
         if (kk < K && col < cols) {
             if (mode == 0) val = w[((size_t)col * V + v) * Ci + kk];
-            else val = w[((size_t)kk * V + (V - 1 - v)) * Ci + col];
+            else val = w[((size_t)kk * V + (mode == 1 ? V - 1 - v : v)) * Ci + col];
         }
         panel[i] = val;
     }
@@ -565,7 +566,7 @@ size_t fgx_weight_panel_bytes(int dtype, int mode, int Ci, int Co, int V, int sl
 int fgx_pack_weight(int dtype, int mode, const void* weight, int Ci, int Co, int V, int slab_bytes, int col_pad,
                     void* panel, fgx_stream_t stream) {
     FGX_CHECK_ARG(dtype_ok(dtype), "fgx_pack_weight: unknown dtype %d", dtype);
-    FGX_CHECK_ARG(mode == 0 || mode == 1, "fgx_pack_weight: mode must be 0 (forward) or 1 (dgrad)");
+    FGX_CHECK_ARG(mode >= 0 && mode <= 2, "fgx_pack_weight: mode must be 0 (forward), 1 (dgrad, mirrored offsets) or 2 (dgrad)");
     FGX_CHECK_ARG(Ci > 0 && Co > 0 && V > 0, "fgx_pack_weight: bad shape Ci=%d Co=%d V=%d", Ci, Co, V);
     FGX_CHECK_ARG(col_pad > 0 && col_pad % 32 == 0, "fgx_pack_weight: col_pad must be a positive multiple of 32");
     FGX_CHECK_ARG(slab_bytes == 64 || slab_bytes == 128, "fgx_pack_weight: slab_bytes must be 64 or 128, got %d", slab_bytes);

@@ -477,7 +477,7 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int CH>
 int launch_stream(const void* src, const void* panel, const void* bias, const int64_t* order, const int32_t* plan_seg,
                   const int32_t* tile_code, const uint32_t* plan_idx, const uint32_t* plan_band, size_t plan_rows, size_t n,
-                  int K, int cols, int cols_pad, size_t panel_bytes, int max_groups, void* out, hipStream_t s) {
+                  size_t n_src, int K, int cols, int cols_pad, size_t panel_bytes, int max_groups, void* out, hipStream_t s) {
     using C = StreamCfg<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
     using T = typename Tag::type;
     auto kern = gather_gemm_stream_kernel<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
@@ -496,7 +496,7 @@ int launch_stream(const void* src, const void* panel, const void* bias, const in
     unsigned groups = (unsigned)(total < (size_t)max_groups ? total : (size_t)max_groups);
     kern<<<groups, C::NT, lds, s>>>((const T*)src, (const T*)panel, (const T*)bias, order, plan_seg, tile_code, plan_idx,
                                     plan_band, (uint32_t)n, K, cols, cols_pad, row_tiles, col_tiles,
-                                    (uint32_t)(n * (size_t)K * sizeof(T)), (uint32_t)panel_bytes,
+                                    (uint32_t)(n_src * (size_t)K * sizeof(T)), (uint32_t)panel_bytes,
                                     (uint32_t)(plan_rows * BM * 4), (T*)out);
     FGX_CHECK_LAUNCH("fgx_conv_gather_gemm_stream");
     return FGX_OK;
@@ -505,12 +505,12 @@ int launch_stream(const void* src, const void* panel, const void* bias, const in
 template <typename Tag>
 int dispatch_stream(int tile_rows, int tile_cols, int slab_bytes, const void* src, const void* panel, const void* bias,
                     const int64_t* order, const int32_t* plan_seg, const int32_t* tile_code, const uint32_t* plan_idx,
-                    const uint32_t* plan_band, size_t plan_rows, size_t n, int K, int cols, int cols_pad,
+                    const uint32_t* plan_band, size_t plan_rows, size_t n, size_t n_src, int K, int cols, int cols_pad,
                     size_t panel_bytes, int max_groups, void* out, hipStream_t s) {
 #define FGX_STREAM_TILE(BM, BN, WMv, WNv, CHv)                                                                          \
     if (tile_rows == BM && tile_cols == BN && slab_bytes == CHv * 16)                                                   \
         return launch_stream<Tag, BM, BN, WMv, WNv, CHv>(src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band,  \
-                                                         plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
+                                                         plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, max_groups, out, s);
     FGX_STREAM_TILE(256, 128, 4, 2, 8)
     FGX_STREAM_TILE(256, 64, 4, 2, 8)
 #undef FGX_STREAM_TILE
@@ -526,7 +526,7 @@ using namespace fgx;
 extern "C" int fgx_conv_gather_gemm_stream(int dtype, const void* src, const void* panel, const void* bias,
                                            const int64_t* order, const int32_t* tile_code, const int32_t* plan_seg,
                                            const uint32_t* plan_idx, const uint32_t* plan_band, size_t plan_rows, size_t n,
-                                           int K, int cols, int V,
+                                           size_t n_src, int K, int cols, int V,
                                            int tile_rows, int tile_cols, int slab_bytes, int max_groups, void* out,
                                            fgx_stream_t stream) {
     FGX_CHECK_ARG(dtype == FGX_F16 || dtype == FGX_BF16 || dtype == FGX_F32, "fgx_conv_gather_gemm_stream: unknown dtype %d", dtype);
@@ -546,7 +546,7 @@ extern "C" int fgx_conv_gather_gemm_stream(int dtype, const void* src, const voi
         max_groups = cus > 0 ? cus : 256;
     }
     // 32-bit buffer offsets: every operand must stay below the out-of-range marker
-    const size_t src_bytes = n * (size_t)K * es;
+    const size_t src_bytes = n_src * (size_t)K * es;
     const int cols_pad = (int)align_up((size_t)cols, (size_t)tile_cols);
     const size_t slabs = ((size_t)K * es + slab_bytes - 1) / slab_bytes;
     const size_t panel_bytes = (size_t)V * slabs * cols_pad * slab_bytes;
@@ -556,8 +556,8 @@ extern "C" int fgx_conv_gather_gemm_stream(int dtype, const void* src, const voi
     }
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
-        case FGX_F16: return dispatch_stream<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
-        case FGX_BF16: return dispatch_stream<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
-        default: return dispatch_stream<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, K, cols, cols_pad, panel_bytes, max_groups, out, s);
+        case FGX_F16: return dispatch_stream<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, max_groups, out, s);
+        case FGX_BF16: return dispatch_stream<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, max_groups, out, s);
+        default: return dispatch_stream<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, max_groups, out, s);
     }
 }

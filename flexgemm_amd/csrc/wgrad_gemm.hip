@@ -808,7 +808,7 @@ int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, con
 
 template <typename Tag, int BM, int BN>
 int launch_wgrad_stream(const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
-                        const SegTable& tab, const Layout& L, size_t n, int V, int Ci, int Co, int block_rows,
+                        const SegTable& tab, const Layout& L, size_t n, size_t n_in, int V, int Ci, int Co, int block_rows,
                         void* scratch, void* gw, hipStream_t s) {
     using C = WStreamCfg<Tag, BM, BN>;
     using T = typename Tag::type;
@@ -834,7 +834,7 @@ int launch_wgrad_stream(const void* gout, const void* feats, const uint32_t* sig
         }
         kern<<<groups, C::NT, C::lds_bytes, s>>>((const T*)gout, (const T*)feats, sig_i, sig_o, bounds, V, Ci, Co, L.nb, co_tiles,
                                                  ci_tiles, tab.seg[V], (uint32_t)(n * (size_t)Co * sizeof(T)),
-                                                 (uint32_t)(n * (size_t)Ci * sizeof(T)), partial);
+                                                 (uint32_t)(n_in * (size_t)Ci * sizeof(T)), partial);
         FGX_CHECK_LAUNCH("fgx_conv_wgrad(stream)");
     }
     size_t total = (size_t)Co * V * Ci;
@@ -847,20 +847,20 @@ int launch_wgrad_stream(const void* gout, const void* feats, const uint32_t* sig
 
 // the streaming kernel: 16-bit types, tiles of 128x128 or 64x64, operands addressable with 32-bit offsets
 template <typename Tag>
-bool stream_ok(int tile_rows, int tile_cols, size_t n, int Ci, int Co, uint32_t n_pairs) {
+bool stream_ok(int tile_rows, int tile_cols, size_t n, size_t n_in, int Ci, int Co, uint32_t n_pairs) {
     if (sizeof(typename Tag::type) != 2) return false;
     if (!((tile_rows == 128 && tile_cols == 128) || (tile_rows == 64 && tile_cols == 64))) return false;
-    return (double)n * Co * 2 <= (double)kOobOffset && (double)n * Ci * 2 <= (double)kOobOffset &&
+    return (double)n * Co * 2 <= (double)kOobOffset && (double)n_in * Ci * 2 <= (double)kOobOffset &&
            (double)n_pairs * 4 + 256 <= (double)kOobOffset;
 }
 
 template <typename Tag>
 int dispatch_wgrad_stream(int tile_rows, const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
-                          const SegTable& tab, const Layout& L, size_t n, int V, int Ci, int Co, int block_rows, void* scratch,
-                          void* gw, hipStream_t s) {
+                          const SegTable& tab, const Layout& L, size_t n, size_t n_in, int V, int Ci, int Co, int block_rows,
+                          void* scratch, void* gw, hipStream_t s) {
     if constexpr (sizeof(typename Tag::type) == 2) {
-        if (tile_rows == 128) return launch_wgrad_stream<Tag, 128, 128>(gout, feats, sig_i, sig_o, tab, L, n, V, Ci, Co, block_rows, scratch, gw, s);
-        return launch_wgrad_stream<Tag, 64, 64>(gout, feats, sig_i, sig_o, tab, L, n, V, Ci, Co, block_rows, scratch, gw, s);
+        if (tile_rows == 128) return launch_wgrad_stream<Tag, 128, 128>(gout, feats, sig_i, sig_o, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, s);
+        return launch_wgrad_stream<Tag, 64, 64>(gout, feats, sig_i, sig_o, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, s);
     } else {
         set_error("fgx_conv_wgrad: the streaming kernel handles 16-bit types only");
         return FGX_ERR_UNSUPPORTED;
@@ -895,13 +895,13 @@ size_t fgx_wgrad_scratch_bytes(size_t n, int V, int Ci, int Co, int block_rows) 
 }
 
 int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
-                   const uint32_t* seg_host, size_t n, int Ci, int Co, int V, int tile_rows, int tile_cols, int block_rows,
-                   int streaming, void* scratch, void* grad_weight, fgx_stream_t stream) {
+                   const uint32_t* seg_host, size_t n, size_t n_in, int Ci, int Co, int V, int tile_rows, int tile_cols,
+                   int block_rows, int streaming, void* scratch, void* grad_weight, fgx_stream_t stream) {
     FGX_CHECK_ARG(dtype_ok(dtype), "fgx_conv_wgrad: unknown dtype %d", dtype);
     FGX_CHECK_ARG(Ci > 0 && Co > 0 && V >= 1 && V <= kMaxV, "fgx_conv_wgrad: bad shape Ci=%d Co=%d V=%d", Ci, Co, V);
     FGX_CHECK_ARG(block_rows >= 1, "fgx_conv_wgrad: block_rows must be positive, got %d", block_rows);
     FGX_CHECK_ARG(seg_host && scratch && grad_weight, "fgx_conv_wgrad: null buffer");
-    FGX_CHECK_ARG(n < 0xFFFFFFFFull, "fgx_conv_wgrad: too many rows");
+    FGX_CHECK_ARG(n < 0xFFFFFFFFull && n_in < 0xFFFFFFFFull, "fgx_conv_wgrad: too many rows");
     const int es = dtype == FGX_F32 ? 4 : 2;
     FGX_CHECK_ARG(((size_t)Ci * es) % 16 == 0 && ((size_t)Co * es) % 16 == 0,
                   "fgx_conv_wgrad: rows of %d / %d elements are not multiples of 16 bytes", Ci, Co);
@@ -919,14 +919,14 @@ int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uin
     }
     Layout L = layout(any ? n : 0, V, Ci, Co, block_rows);
     // 32-bit byte offsets into grad_out / feats are enough below 4 GiB
-    const bool small = (double)n * Co * es < 4294967296.0 && (double)n * Ci * es < 4294967296.0;
+    const bool small = (double)n * Co * es < 4294967296.0 && (double)n_in * Ci * es < 4294967296.0;
     hipStream_t s = (hipStream_t)stream;
     if (streaming && any) {
         // falls through to the tiled kernel when the problem is outside the streaming kernel's range
-        if (dtype == FGX_F16 && stream_ok<F16>(tile_rows, tile_cols, n, Ci, Co, tab.seg[V]))
-            return dispatch_wgrad_stream<F16>(tile_rows, grad_out, feats, sig_i, sig_o, tab, L, n, V, Ci, Co, block_rows, scratch, grad_weight, s);
-        if (dtype == FGX_BF16 && stream_ok<BF16>(tile_rows, tile_cols, n, Ci, Co, tab.seg[V]))
-            return dispatch_wgrad_stream<BF16>(tile_rows, grad_out, feats, sig_i, sig_o, tab, L, n, V, Ci, Co, block_rows, scratch, grad_weight, s);
+        if (dtype == FGX_F16 && stream_ok<F16>(tile_rows, tile_cols, n, n_in, Ci, Co, tab.seg[V]))
+            return dispatch_wgrad_stream<F16>(tile_rows, grad_out, feats, sig_i, sig_o, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, s);
+        if (dtype == FGX_BF16 && stream_ok<BF16>(tile_rows, tile_cols, n, n_in, Ci, Co, tab.seg[V]))
+            return dispatch_wgrad_stream<BF16>(tile_rows, grad_out, feats, sig_i, sig_o, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, s);
     }
     switch (dtype) {
         case FGX_F16: return dispatch_wgrad<F16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);

@@ -17,8 +17,26 @@ class Algorithm:
     MASKED_IMPLICIT_GEMM_SPLITK = "masked_implicit_gemm_splitk"
 
 
+class SerializationMode:
+    """How 3-D coordinates are flattened into the key that orders generated output coordinates
+    (flex_gemm/ops/spconv/__init__.py:10-14).  Only BXYZ is implemented here."""
+    BXYZ = 0
+    Z_ORDER = 1
+    HILBERT = 2
+
+
+class SparseConv3dOutCoordAlgorithm:
+    """Algorithm choices for generating output coordinates (flex_gemm/ops/spconv/__init__.py:17-20).  Both values give
+    the same sorted list; on gfx950 they share one streaming implementation (candidate keys, radix sort, unique)."""
+    HASHMAP = 0
+    EXPAND_UNIQUE = 1
+
+
 ALGORITHM = Algorithm.MASKED_IMPLICIT_GEMM_SPLITK  # Default algorithm
 HASHMAP_RATIO = 2.0                                 # Ratio of hashmap size to input size
+OUT_COORD_HASHMAP_RATIO = 1.1                       # kept for interface parity; the sort-based builder has no table
+OUT_COORD_ALGO = SparseConv3dOutCoordAlgorithm.HASHMAP
+SERIALIZATION_MODE = SerializationMode.BXYZ
 
 
 def set_algorithm(algorithm: str):
@@ -32,3 +50,4 @@ def set_hashmap_ratio(ratio: float):
 
 
 from .submanifold_conv3d import SubMConv3dFunction, SubMConv3dNeighborCache, sparse_submanifold_conv3d  # noqa: E402
+from .sparse_conv3d import SparseConv3dFunction, SparseConv3dNeighborCache, sparse_conv3d  # noqa: E402

@@ -282,10 +282,13 @@ def _pad_cols(t: torch.Tensor, mult: int) -> torch.Tensor:
 
 def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[torch.Tensor], cache, mode: int,
                  allow_splitk: bool, masked: bool = True) -> torch.Tensor:
-    """mode 0: out = conv(src) with weight [Co, V, Ci] (+bias); mode 1: grad_input from src = grad_output.
-    masked=False: the non-masked schedule (natural row order, all offsets per tile)."""
+    """mode 0: out = conv(src) with weight [Co, V, Ci] (+bias); mode 1: grad_input from src = grad_output through the
+    same map with the offsets mirrored (submanifold); mode 2: grad_input through a map of its own, offsets as they
+    are (generic sparse convolution).  The result has one row per row of cache["neighbor_map"]; src may have a
+    different number of rows.  masked=False: the non-masked schedule (natural row order, all offsets per tile)."""
     co, v, ci = weight_cvk.shape
-    n = src.shape[0]
+    n = cache["neighbor_map"].shape[0]
+    n_src = src.shape[0]
     dt = src.dtype
     if dt not in nat.DTYPE_CODE:
         raise TypeError(f"unsupported feature dtype {dt}; expected float16, bfloat16 or float32")
@@ -293,6 +296,9 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
         raise TypeError("features, weight and bias must share one dtype")
     k_true, cols = (ci, co) if mode == 0 else (co, ci)
     dev = src.device
+    if n_src == 0:      # nothing to gather: the bias alone
+        out = torch.zeros((n, cols), dtype=dt, device=dev)
+        return out if bias is None else out + bias
     # rows must be whole 16-byte chunks: zero-pad the contraction dimension when they are not
     align = 16 // src.element_size()
     if k_true % align:
@@ -321,13 +327,13 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
                                                        C.c_int(sched.slab_bytes), C.c_int(sched.tile_cols)), dev)
         nat.check(L.fgx_pack_weight(C.c_int(code), C.c_int(mode), nat.ptr(weight_cvk), C.c_int(ci), C.c_int(co), C.c_int(v),
                                     C.c_int(sched.slab_bytes), C.c_int(sched.tile_cols), nat.ptr(panel), nat.stream()))
-        if sched.stream and _stream_fits(n, k * src.element_size()):
+        if sched.stream and _stream_fits(n, n_src, k * src.element_size()):
             order, tile_code, plan_seg, plan_idx, plan_band = cache._gather_plan(sched.tile_rows, private, dense=not masked)
             nat.mark(name, "start")
             nat.check(L.fgx_conv_gather_gemm_stream(
                 C.c_int(code), nat.ptr(src), nat.ptr(panel), nat.ptr(bias), nat.ptr(order), nat.ptr(tile_code),
-                nat.ptr(plan_seg), nat.ptr(plan_idx), nat.ptr(plan_band), nat.sz(plan_idx.shape[0]), nat.sz(n), C.c_int(k),
-                C.c_int(cols), C.c_int(v),
+                nat.ptr(plan_seg), nat.ptr(plan_idx), nat.ptr(plan_band), nat.sz(plan_idx.shape[0]), nat.sz(n), nat.sz(n_src),
+                C.c_int(k), C.c_int(cols), C.c_int(v),
                 C.c_int(sched.tile_rows), C.c_int(sched.tile_cols), C.c_int(sched.slab_bytes), C.c_int(0), nat.ptr(out),
                 nat.stream()))
             nat.mark(name, "stop")
@@ -349,14 +355,16 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
     return out
 
 
-def _stream_fits(n: int, row_bytes: int) -> bool:
+def _stream_fits(n: int, n_src: int, row_bytes: int) -> bool:
     """The streaming kernel addresses its operands with 32-bit byte offsets."""
-    return n * row_bytes <= 0xFF000000 and n * 8 <= 0xFF000000 and n * 27 * 4 * 2 <= 0xFF000000
+    return n_src * row_bytes <= 0xFF000000 and n * 8 <= 0xFF000000 and n * 27 * 4 * 2 <= 0xFF000000
 
 
 def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int) -> torch.Tensor:
-    n, ci = feats.shape
-    co = grad_output.shape[1]
+    """[Co, V, Ci] weight gradient from the pair lists of cache["neighbor_map"]: grad_output has one row per row of
+    that map, feats one per row the map points at."""
+    n_in, ci = feats.shape
+    n, co = grad_output.shape
     dt = feats.dtype
     dev = feats.device
     align = 16 // feats.element_size()
@@ -376,7 +384,7 @@ def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int) -> tor
         nat.mark("wgrad", "start")
         nat.check(L.fgx_conv_wgrad(
             C.c_int(code), nat.ptr(g), nat.ptr(f), nat.ptr(cache["valid_signal_i"]), nat.ptr(cache["valid_signal_o"]),
-            seg_arr, nat.sz(n), C.c_int(cip), C.c_int(cop), C.c_int(v), C.c_int(sched.tile_rows), C.c_int(sched.tile_cols),
+            seg_arr, nat.sz(n), nat.sz(n_in), C.c_int(cip), C.c_int(cop), C.c_int(v), C.c_int(sched.tile_rows), C.c_int(sched.tile_cols),
             C.c_int(sched.block_rows), C.c_int(sched.stream), nat.ptr(scratch), nat.ptr(gw), nat.stream()))
         nat.mark("wgrad", "stop")
     if cip != ci or cop != co:

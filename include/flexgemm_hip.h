@@ -154,6 +154,8 @@ int fgx_table_lookup(int pass_kind, int dtype, size_t n, int Ci, int Co, int V, 
 /* Re-layout the [Co, V, Ci] weight into K-slab-major panels consumed by fgx_conv_gather_gemm.
  *   mode 0 (forward): panel[v][slab][co][k]  = w[co][v][slab*SK + k]          (K = Ci, cols = Co)
  *   mode 1 (dgrad)  : panel[v][slab][ci][k]  = w[slab*SK + k][V-1-v][ci]      (K = Co, cols = Ci)
+ *   mode 2 (dgrad through a separate backward map, generic sparse convolution):
+ *                     panel[v][slab][ci][k]  = w[slab*SK + k][v][ci]          (K = Co, cols = Ci)
  * SK = slab_bytes / element size (slab_bytes = 64 or 128: the schedule's value); K is zero-padded to a whole
  * slab and cols to a multiple of col_pad (a multiple of 32; pass the tile_cols the GEMM will run with).
  * Replaces: the strided weight-tile loads of the Triton kernels
@@ -202,11 +204,13 @@ int fgx_gather_plan_fill(const uint32_t* map, const int64_t* order, const int32_
  * returns FGX_ERR_UNSUPPORTED when src, the panel or the plan exceed ~4 GB, or when no kernel exists for the
  * schedule -- callers then use fgx_conv_gather_gemm.  `plan_band` (from fgx_gather_plan_fill; NULL = every band
  * present) lets the kernel skip the loads and products of 32-row bands without a neighbor at an offset.
+ * `n` counts the output rows (rows of the map behind the plan), `n_src` the rows of `src`; they differ for the
+ * generic sparse convolution only.
  * Replaces: the same reference kernels as fgx_conv_gather_gemm. */
 int fgx_conv_gather_gemm_stream(int dtype, const void* src, const void* panel, const void* bias,
                                 const int64_t* order, const int32_t* tile_code, const int32_t* plan_seg,
                                 const uint32_t* plan_idx, const uint32_t* plan_band, size_t plan_rows, size_t n,
-                                int K, int cols, int V,
+                                size_t n_src, int K, int cols, int V,
                                 int tile_rows, int tile_cols, int slab_bytes, int max_groups, void* out,
                                 fgx_stream_t stream);
 
@@ -216,13 +220,15 @@ int fgx_conv_gather_gemm_stream(int dtype, const void* src, const void* panel, c
  * partial product goes to `scratch` in fp32 (fgx_wgrad_scratch_bytes bytes, 256-byte aligned) and a second kernel
  * adds them per offset in block order.  `streaming` != 0 asks for the persistent kernel with loader / multiplier
  * wavefronts (16-bit types, 128x128 or 64x64 tiles, operands below ~4 GB); outside that range the tiled kernel runs.
+ * `n` = rows of grad_out (the range of sig_o), `n_in` = rows of feats (the range of sig_i); equal for the submanifold
+ * convolution.
  * Replaces: sparse_submanifold_conv_bwd_weight_masked_implicit_gemm[_splitk]
  *           (..._bwd_masked_implicit_gemm.py:99-170, ..._splitk.py:108-182, 278-317). */
 size_t fgx_wgrad_scratch_bytes(size_t n, int V, int Ci, int Co, int block_rows);
 int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats,
                    const uint32_t* sig_i, const uint32_t* sig_o, const uint32_t* seg_host,
-                   size_t n, int Ci, int Co, int V, int tile_rows, int tile_cols, int block_rows, int streaming,
-                   void* scratch, void* grad_weight, fgx_stream_t stream);
+                   size_t n, size_t n_in, int Ci, int Co, int V, int tile_rows, int tile_cols, int block_rows,
+                   int streaming, void* scratch, void* grad_weight, fgx_stream_t stream);
 
 /* grad_bias[co] = sum over rows of grad_out[:, co], accumulated in fp32.
  * `scratch`: fgx_colsum_scratch_bytes bytes of fp32 partial sums.
@@ -230,6 +236,48 @@ int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats,
 size_t fgx_colsum_scratch_bytes(size_t n, int cols);
 int fgx_colsum(int dtype, const void* grad_out, size_t n, int cols, void* scratch, void* out,
                fgx_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Generic sparse convolution (stride / padding / dilation): output coordinates and neighbor maps.
+ * The GEMM passes are the ones above: forward gathers feats through map_fwd (n = output rows, n_src = input
+ * rows), the input gradient gathers grad_out through map_bwd with the mode-2 weight panel, wgrad takes the pair
+ * lists of map_fwd.
+ * ------------------------------------------------------------------------------------------- */
+
+/* (Wo, Ho, Do) = floor((N + 2P - D(K-1) - 1) / S) + 1 per axis.
+ * Replaces: the size formula in flex_gemm/kernels/cuda/spconv/sparse_neighbor_map.cu:86-88. */
+int fgx_spconv_out_dims(int W, int H, int D, int Kw, int Kh, int Kd, int Sw, int Sh, int Sd,
+                        int Pw, int Ph, int Pd, int Dw, int Dh, int Dd, int* Wo, int* Ho, int* Do);
+
+/* Output coordinates, two steps around the one read-back that sizes the result:
+ *   fgx_spconv_out_coords_keys    every cell o = (i + P - k*D) / S reached by an input voxel i through a kernel
+ *                                 position k (exact division, inside the output grid) as a flattened key
+ *                                 ((b*Wo + x)*Ho + y)*Do + z, sorted ascending and unique, left at the start of
+ *                                 `workspace`; their number goes to `count` (DEVICE memory, 8 bytes).
+ *   fgx_spconv_out_coords_decode  keys -> int32 (b, x, y, z) rows, `count` of them (the value read back).
+ * key_bits: 32 when B*Wo*Ho*Do < 2^32 - 1, else 64.  workspace: fgx_spconv_out_coords_workspace_bytes bytes,
+ * 256-byte aligned.  The order is the reference's with BXYZ serialisation (its default), i.e. torch.unique(dim=0).
+ * Replaces: hashmap_build_sparse_conv_out_coords and expand_unique_build_sparse_conv_out_coords,
+ *           flex_gemm/kernels/cuda/spconv/sparse_neighbor_map.h:42-86 (.cu:76-131, 275-345). */
+size_t fgx_spconv_out_coords_workspace_bytes(size_t n_in, int V, int key_bits);
+int fgx_spconv_out_coords_keys(const int32_t* coords, size_t n_in, int B, int W, int H, int D,
+                               int Kw, int Kh, int Kd, int Sw, int Sh, int Sd, int Pw, int Ph, int Pd,
+                               int Dw, int Dh, int Dd, int key_bits, void* workspace, size_t workspace_bytes,
+                               uint64_t* count, fgx_stream_t stream);
+int fgx_spconv_out_coords_decode(const void* workspace, int key_bits, size_t count, int Wo, int Ho, int Do,
+                                 int32_t* out_coords, fgx_stream_t stream);
+
+/* map_fwd[o, v] = row of the input voxel at out_coords[o]*S - P + k_v*D (same batch, inside the input grid), all
+ * ones when there is none; map_bwd[i, v] = o for every map_fwd[o, v] = i, all ones elsewhere (NULL = not wanted;
+ * [n_in, V], filled here).  `keys` / `vals` is the hash table of the INPUT voxels (fgx_hash_init +
+ * fgx_hash_insert_3d_idx_as_val over the input grid).  gray / binary (optional, V <= 32): validity mask of every
+ * map_fwd row and its Gray-decoded sort key, as fgx_mask_codes would give.
+ * Replaces: hashmap_build_sparse_conv_neighbour_map, sparse_neighbor_map.h:88-131 (.cu:431-567). */
+int fgx_spconv_neighbor_map(const void* keys, int key_bits, const uint32_t* vals, size_t table_size,
+                            const int32_t* out_coords, size_t n_out, size_t n_in, int W, int H, int D,
+                            int Kw, int Kh, int Kd, int Sw, int Sh, int Sd, int Pw, int Ph, int Pd,
+                            int Dw, int Dh, int Dd, uint32_t* map_fwd, uint32_t* map_bwd,
+                            int32_t* gray, int32_t* binary, fgx_stream_t stream);
 
 #ifdef __cplusplus
 }
