@@ -55,18 +55,21 @@ struct StreamCfg {
     static constexpr int SLAB = CH * 16;
     static constexpr int SK = SLAB / ES;
     static constexpr int ROWS_PER_INST = 64 / CH;
-    static constexpr int A_PER = BM / ROWS_PER_INST / NL, B_PER = BN / ROWS_PER_INST / NL;
-    static constexpr int LPS = A_PER + B_PER;                  // row loads per loader and step
+    static constexpr int A_PER = BM / ROWS_PER_INST / NL;
+    static constexpr int B_INST = BN / ROWS_PER_INST;          // wave-wide loads per panel slab, dealt round-robin to the loaders
+    static constexpr int B_PER = (B_INST + NL - 1) / NL;       // ... so a loader issues B_PER of them, or one fewer
+    static constexpr int LPS = A_PER + B_PER;                  // most row loads per loader and step
     static constexpr int IDX_INST = BM / 64;                   // wave-wide dword loads per index column
     static constexpr int OROW_INST = (WM + 63) / 64;           // wave-wide dword loads for a wave tile's output rows
     static constexpr int STAGE_BYTES = (BM + BN) * SLAB;
     static constexpr int IDX_SLOT_BYTES = BM * 4;
     static constexpr int OUT_PITCH = WN * ES + 16;
-    static constexpr int BAND_ROWS = NW * 32 * OUT_PITCH <= (BM + BN) * SLAB ? 32 : 16;   // rows staged per epilogue pass
+    // rows staged per epilogue pass: the most of 32, 16, 8 whose bands (one per multiplier) fit one ring stage
+    static constexpr int BAND_ROWS = NW * 32 * OUT_PITCH <= (BM + BN) * SLAB ? 32 : (NW * 16 * OUT_PITCH <= (BM + BN) * SLAB ? 16 : 8);
     static constexpr int OUT_BAND_BYTES = BAND_ROWS * OUT_PITCH;
     static constexpr int OROW_BYTES = 2 * NW * OROW_INST * 256;
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
-    static_assert(BM % (ROWS_PER_INST * NL) == 0 && BN % (ROWS_PER_INST * NL) == 0, "every loader issues the same row loads");
+    static_assert(BM % (ROWS_PER_INST * NL) == 0 && BN % ROWS_PER_INST == 0, "rows and panel columns must be whole wave-wide loads");
     static_assert(BM % 64 == 0 && IDX_INST <= NL, "index column must be whole wave-wide loads, one per loader");
     static_assert(NW * OUT_BAND_BYTES <= STAGE_BYTES, "the output bands must fit one ring stage");
     static_assert(LPS + 1 < 64, "vmcnt is a 6-bit counter");
@@ -251,7 +254,7 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
         if (!p_ready) return 0;
         unsigned char* stage = ring + p_stage * C::STAGE_BYTES;
         const bool tail = ragged && p_slab == slabs - 1;     // wave-uniform
-        int ops = C::B_PER;
+        int ops = 0;
 #pragma unroll
         for (int i = 0; i < C::A_PER; ++i) {
             // 32-row band of this load's rows (a constant when the loaders' loads of one round make up one band)
@@ -268,8 +271,10 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
         unsigned char* stage_b = stage + BM * kSlabBytes;
 #pragma unroll
         for (int i = 0; i < C::B_PER; ++i) {
+            if (C::B_INST % C::NL != 0 && i * C::NL + lw >= C::B_INST) continue;     // narrow panels: not every loader has one
             const uint32_t vo = b_voff[i];
             __builtin_amdgcn_raw_ptr_buffer_load_lds(panel_rs, FGX_LDS_PTR(stage_b + (i * C::NL + lw) * 1024), 16, vo, b_soff, 0, 0);
+            ++ops;
         }
         a_soff += kSlabBytes;
         b_soff = __builtin_amdgcn_readfirstlane(b_soff + b_slab_stride);
@@ -430,7 +435,7 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
 #pragma unroll
         for (int ih = 0; ih < C::TM * HALVES; ++ih) {
             const int i = ih / HALVES, h = ih % HALVES;      // 32-row tile, half of it
-            if (HALVES == 1 || (l32 >> 4) == h) {
+            if (HALVES == 1 || l32 / C::BAND_ROWS == h) {
                 const int r = l32 - h * C::BAND_ROWS;
 #pragma unroll
                 for (int j = 0; j < C::TN; ++j)
@@ -493,6 +498,22 @@ int launch_stream(const void* src, const void* panel, const void* bias, const in
     }
     const unsigned row_tiles = cdiv(n, BM), col_tiles = cdiv(cols, BN);
     const size_t total = (size_t)row_tiles * col_tiles;
+    if (max_groups <= 0) {
+        // as many resident workgroups as the CUs hold (the narrow tiles leave room for two per CU: their steps are
+        // short, and a second stream fills the time the first spends at its barriers)
+        static thread_local int per_cu = 0;          // per thread and instantiation, for the LDS size it was asked with
+        static thread_local size_t per_cu_lds = 0;
+        int dev = 0, cus = 0;
+        FGX_CHECK_HIP(hipGetDevice(&dev));
+        FGX_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        if (per_cu == 0 || per_cu_lds != lds) {
+            int q = 1;
+            FGX_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&q, (const void*)kern, C::NT, lds));
+            per_cu = q < 1 ? 1 : (q > 2 ? 2 : q);
+            per_cu_lds = lds;
+        }
+        max_groups = (cus > 0 ? cus : 256) * per_cu;
+    }
     unsigned groups = (unsigned)(total < (size_t)max_groups ? total : (size_t)max_groups);
     kern<<<groups, C::NT, lds, s>>>((const T*)src, (const T*)panel, (const T*)bias, order, plan_seg, tile_code, plan_idx,
                                     plan_band, (uint32_t)n, K, cols, cols_pad, row_tiles, col_tiles,
@@ -513,6 +534,9 @@ int dispatch_stream(int tile_rows, int tile_cols, int slab_bytes, const void* sr
                                                          plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, max_groups, out, s);
     FGX_STREAM_TILE(256, 128, 4, 2, 8)
     FGX_STREAM_TILE(256, 64, 4, 2, 8)
+    FGX_STREAM_TILE(256, 128, 4, 2, 4)      // 64-byte K-slabs: rows shorter than 128 bytes
+    FGX_STREAM_TILE(256, 64, 4, 2, 4)
+    FGX_STREAM_TILE(256, 32, 8, 1, 4)
 #undef FGX_STREAM_TILE
     set_error("fgx_conv_gather_gemm_stream: no kernel for tile %dx%d with %d-byte slabs", tile_rows, tile_cols, slab_bytes);
     return FGX_ERR_UNSUPPORTED;
@@ -539,12 +563,6 @@ extern "C" int fgx_conv_gather_gemm_stream(int dtype, const void* src, const voi
                   "fgx_conv_gather_gemm_stream: src, panel and plan_idx must be 16-byte aligned");
     FGX_CHECK_ARG(tile_rows > 0 && tile_cols > 0 && (slab_bytes == 64 || slab_bytes == 128), "fgx_conv_gather_gemm_stream: bad schedule");
     FGX_CHECK_ARG(plan_band == nullptr || tile_rows <= 1024, "fgx_conv_gather_gemm_stream: band masks cover tiles of at most 1024 rows");
-    if (max_groups <= 0) {
-        int dev = 0, cus = 0;
-        FGX_CHECK_HIP(hipGetDevice(&dev));
-        FGX_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-        max_groups = cus > 0 ? cus : 256;
-    }
     // 32-bit buffer offsets: every operand must stay below the out-of-range marker
     const size_t src_bytes = n_src * (size_t)K * es;
     const int cols_pad = (int)align_up((size_t)cols, (size_t)tile_cols);

@@ -26,8 +26,8 @@ const Entry kTable[] = {
     {0, 2, 17, 256, 256, {256, 128, 128, 1, 0, 1}},
     {1, 2, 17, 256, 256, {256, 128, 128, 1, 0, 1}},
     {2, 2, 17, 256, 256, {128, 128, 64, 1, 4096, 1}},
-    {0, 2, 21, 32, 32, {128, 32, 64, 1, 0, 0}},
-    {1, 2, 21, 32, 32, {128, 32, 64, 1, 0, 0}},
+    {0, 2, 21, 32, 32, {256, 32, 64, 1, 0, 1}},
+    {1, 2, 21, 32, 32, {256, 32, 64, 1, 0, 1}},
     {2, 2, 21, 32, 32, {32, 32, 64, 1, 4096, 0}},
     {0, 2, 15, 1024, 1024, {256, 128, 128, 1, 0, 1}},
     {1, 2, 15, 1024, 1024, {256, 128, 128, 1, 0, 1}},
@@ -77,14 +77,16 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
     int s = 1;
     while (tiles * s < (size_t)kCUs && s < 16) s *= 2;
     out->splitk = s;
-    // persistent streaming kernel (256 x 128 or 256 x 64 tiles, 128-byte K-slabs): rows of at least one slab, at least
-    // 64 columns, and at least two items per CU
+    // persistent streaming kernel (256-row tiles): rows of at least 64 bytes -- 128-byte K-slabs from 128 bytes on, 64-byte
+    // ones below, where 32 output columns get a tile of their own -- and at least two items per CU
     const int K = pass_kind == 0 ? Ci : Co;
-    const int scols = cols > 64 ? 128 : 64;
-    if ((size_t)K * es >= 128 && cols >= 64 && (size_t)cdiv(n, 256) * cdiv(cols, scols) >= 2 * (size_t)kCUs) {
+    const size_t row_bytes = (size_t)K * es;
+    const int slab = row_bytes >= 128 ? 128 : 64;
+    const int scols = cols > 64 ? 128 : ((cols > 32 || slab == 128) ? 64 : 32);
+    if (row_bytes >= 64 && (slab == 64 || cols >= 64) && (size_t)cdiv(n, 256) * cdiv(cols, scols) >= 2 * (size_t)kCUs) {
         out->tile_rows = 256;
         out->tile_cols = scols;
-        out->slab_bytes = 128;
+        out->slab_bytes = slab;
         out->splitk = 1;
         out->stream = 1;
     }

@@ -726,33 +726,54 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
     }
 }
 
-// grad_weight[co][v][ci] = sum over voxel blocks with pairs for offset v, in block order
+// grad_weight[co][v][ci] = sum over the voxel blocks that have pairs for offset v.  A workgroup owns kReduceElems
+// consecutive elements (ci fastest: one 128-byte piece per block for fp32 partials) and cuts the blocks into
+// kReduceSlices contiguous ranges, one per group of threads; a slice adds its blocks in ascending order (eight loads in
+// flight) and the slice sums are added in ascending order as well, so the result depends on nb alone, not on which
+// kernel wrote the partial products.
+constexpr int kReduceElems = 32, kReduceSlices = 8;
+
 template <typename T>
 __global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restrict__ partial,
                                                            const uint32_t* __restrict__ bounds, int V, int Ci, int Co,
                                                            unsigned nb, T* __restrict__ gw) {
+    __shared__ float sums[kReduceSlices][kReduceElems];
     const size_t per = (size_t)Co * Ci;
     const size_t total = per * V;
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
-        int ci = (int)(i % Ci);
-        size_t t = i / Ci;
-        int v = (int)(t % V);
-        int co = (int)(t / V);
-        const uint32_t* bd = bounds + (size_t)v * (nb + 1);
-        const float* src = partial + (size_t)v * per + (size_t)co * Ci + ci;
-        const size_t stride = (size_t)V * per;
+    const int e = threadIdx.x % kReduceElems, slice = threadIdx.x / kReduceElems;
+    const unsigned chunk = (nb + kReduceSlices - 1) / kReduceSlices;
+    for (size_t base = (size_t)blockIdx.x * kReduceElems; base < total; base += (size_t)gridDim.x * kReduceElems) {
+        const size_t i = base + e;
         float s = 0.f;
-        unsigned b = 0;
-        for (; b + 8 <= nb; b += 8) {     // eight independent loads in flight; the sum order stays b-ascending
-            float x[8];
+        if (i < total) {
+            int ci = (int)(i % Ci);
+            size_t t = i / Ci;
+            int v = (int)(t % V);
+            int co = (int)(t / V);
+            const uint32_t* bd = bounds + (size_t)v * (nb + 1);
+            const float* src = partial + (size_t)v * per + (size_t)co * Ci + ci;
+            const size_t stride = (size_t)V * per;
+            unsigned b = slice * chunk;
+            const unsigned end = b + chunk < nb ? b + chunk : nb;
+            for (; b + 8 <= end; b += 8) {
+                float x[8];
 #pragma unroll
-            for (int q = 0; q < 8; ++q) x[q] = bd[b + q] < bd[b + q + 1] ? src[(size_t)(b + q) * stride] : 0.f;
+                for (int q = 0; q < 8; ++q) x[q] = bd[b + q] < bd[b + q + 1] ? src[(size_t)(b + q) * stride] : 0.f;
 #pragma unroll
-            for (int q = 0; q < 8; ++q) s += x[q];
+                for (int q = 0; q < 8; ++q) s += x[q];
+            }
+            for (; b < end; ++b)
+                if (bd[b] < bd[b + 1]) s += src[(size_t)b * stride];
         }
-        for (; b < nb; ++b)
-            if (bd[b] < bd[b + 1]) s += src[(size_t)b * stride];
-        gw[i] = from_float<T>(s);
+        sums[slice][e] = s;
+        __syncthreads();
+        if (slice == 0 && i < total) {
+            float r = sums[0][e];
+#pragma unroll
+            for (int q = 1; q < kReduceSlices; ++q) r += sums[q][e];
+            gw[i] = from_float<T>(r);
+        }
+        __syncthreads();
     }
 }
 
@@ -799,7 +820,7 @@ int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, con
         FGX_CHECK_LAUNCH("fgx_conv_wgrad");
     }
     size_t total = (size_t)Co * V * Ci;
-    unsigned g = cdiv(total, 256);
+    unsigned g = cdiv(total, kReduceElems);
     if (g > 65536u) g = 65536u;
     wgrad_reduce_kernel<T><<<g, 256, 0, s>>>(partial, bounds, V, Ci, Co, L.nb, (T*)gw);
     FGX_CHECK_LAUNCH("fgx_conv_wgrad(reduce)");
@@ -838,7 +859,7 @@ int launch_wgrad_stream(const void* gout, const void* feats, const uint32_t* sig
         FGX_CHECK_LAUNCH("fgx_conv_wgrad(stream)");
     }
     size_t total = (size_t)Co * V * Ci;
-    unsigned g = cdiv(total, 256);
+    unsigned g = cdiv(total, kReduceElems);
     if (g > 65536u) g = 65536u;
     wgrad_reduce_kernel<T><<<g, 256, 0, s>>>(partial, bounds, V, Ci, Co, L.nb, (T*)gw);
     FGX_CHECK_LAUNCH("fgx_conv_wgrad(reduce)");

@@ -200,7 +200,7 @@ int fgx_gather_plan_fill(const uint32_t* map, const int64_t* order, const int32_
 
 /* Same result as fgx_conv_gather_gemm (splitk = 1) from the gather plan of `order`, by persistent workgroups that
  * stream all their tiles' (offset, K-slab) steps back to back; meant for voxel counts that give every CU several
- * tiles.  `max_groups`: workgroups to launch (<= 0: one per CU).  Operands are addressed with 32-bit offsets:
+ * tiles.  `max_groups`: workgroups to launch (<= 0: as many as are resident at once, at most two per CU).  Operands are addressed with 32-bit offsets:
  * returns FGX_ERR_UNSUPPORTED when src, the panel or the plan exceed ~4 GB, or when no kernel exists for the
  * schedule -- callers then use fgx_conv_gather_gemm.  `plan_band` (from fgx_gather_plan_fill; NULL = every band
  * present) lets the kernel skip the loads and products of 32-row bands without a neighbor at an offset.

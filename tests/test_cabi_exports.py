@@ -41,16 +41,21 @@ def test_host_only_entry_points(library):
     import torch
     s = nat.table_lookup(nat.PASS_FWD, torch.float16, 669288, 128, 128, 27)
     assert s.tile_rows in (128, 256) and s.tile_cols == 128 and s.splitk == 1 and s.slab_bytes in (64, 128)
-    # the persistent streaming kernel has exactly one tile shape
+    # the persistent streaming kernel walks 256-row tiles; rows of 128 bytes or more use 128-byte K-slabs
     assert (s.stream, s.tile_rows, s.slab_bytes) in ((1, 256, 128), (0, s.tile_rows, s.slab_bytes))
     s = nat.table_lookup(nat.PASS_WGRAD, torch.float16, 669288, 128, 128, 27)
     assert s.block_rows >= 1024 and s.stream in (0, 1)
     s = nat.table_lookup(nat.PASS_FWD, torch.float32, 100, 16, 16, 27)
     assert s.tile_rows in (32, 64, 128) and s.tile_cols == 32 and s.splitk >= 1 and s.stream == 0
-    # rule (no table entry): big 16-bit problems stream, small ones and short rows do not
+    # rule (no table entry): big problems stream, small ones and rows below 64 bytes do not
     s = nat.table_lookup(nat.PASS_DGRAD, torch.bfloat16, 300000, 192, 160, 27)
     assert (s.stream, s.tile_rows, s.tile_cols, s.slab_bytes, s.splitk) == (1, 256, 128, 128, 1)
-    assert nat.table_lookup(nat.PASS_FWD, torch.bfloat16, 300000, 32, 32, 27).stream == 0
+    s = nat.table_lookup(nat.PASS_FWD, torch.bfloat16, 300000, 32, 32, 27)      # 64-byte rows: 64-byte slabs, 32-column tiles
+    assert (s.stream, s.tile_rows, s.tile_cols, s.slab_bytes, s.splitk) == (1, 256, 32, 64, 1)
+    s = nat.table_lookup(nat.PASS_DGRAD, torch.bfloat16, 300000, 96, 32, 27)    # K = Co = 32, 96 input-gradient columns
+    assert (s.stream, s.tile_rows, s.tile_cols, s.slab_bytes) == (1, 256, 128, 64)
+    assert nat.table_lookup(nat.PASS_FWD, torch.float16, 300000, 16, 64, 27).stream == 0
+    assert nat.table_lookup(nat.PASS_FWD, torch.float16, 300000, 128, 32, 27).stream == 0   # no 32-column tile for long rows
     s = nat.table_lookup(nat.PASS_FWD, torch.float16, 300000, 64, 64, 27)
     assert (s.stream, s.tile_rows, s.tile_cols, s.slab_bytes) == (1, 256, 64, 128)
     assert nat.table_lookup(nat.PASS_FWD, torch.float16, 5000, 192, 160, 27).stream == 0

@@ -242,6 +242,19 @@ def test_streaming_kernel_matches_oracle(gpu_device, dtype, res, ci, co):
             _run_and_check(coords_np, shape, ci, co, dtype, gpu_device, seed=22)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("res,ci,co,tile_cols", [(32, 32, 32, 32), (24, 32, 64, 64), (24, 16, 96, 128), (24, 128, 40, 32),
+                                                 (16, 24, 32, 32), (40, 32, 32, 32)])
+def test_streaming_kernel_with_64_byte_slabs(gpu_device, dtype, res, ci, co, tile_cols):
+    """The streaming GEMM on 64-byte K-slabs (rows shorter than 128 bytes) with 32-, 64- and 128-column tiles: panels
+    narrower than one round of loader instructions, several slabs per row, ragged last slabs, several column tiles."""
+    _say(f"stream slab64 res={res} ci={ci} co={co} tile_cols={tile_cols} {dtype}")
+    coords_np = reference_test_shell(res)
+    shape = torch.Size([1, ci, res, res, res])
+    with _force_schedule(tile_rows=256, tile_cols=tile_cols, slab_bytes=64, splitk=1, stream=1):
+        _run_and_check(coords_np, shape, ci, co, dtype, gpu_device, seed=29)
+
+
 def test_streaming_kernel_equals_tiled_kernel_bitwise(gpu_device):
     """Both kernels add the same products in the same order (offsets ascending, K ascending), so their outputs
     agree bit for bit; isolated voxels (only the centre offset) and a batch dimension are in the mix."""
