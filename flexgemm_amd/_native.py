@@ -24,7 +24,7 @@ EXPORTS = [
     "fgx_abi_version", "fgx_last_error",
     "fgx_hash_init", "fgx_hash_insert_3d_idx_as_val", "fgx_hash_insert", "fgx_hash_lookup",
     "fgx_hash_insert_3d", "fgx_hash_lookup_3d",
-    "fgx_subm_neighbor_map", "fgx_mask_codes",
+    "fgx_subm_neighbor_map", "fgx_subm_neighbor_map_sorted_workspace_bytes", "fgx_subm_neighbor_map_sorted", "fgx_mask_codes",
     "fgx_sort_workspace_bytes", "fgx_sort_by_code", "fgx_locality_workspace_bytes", "fgx_locality_order",
     "fgx_pair_workspace_bytes", "fgx_pair_count", "fgx_pair_fill",
     "fgx_tile_workspace_bytes", "fgx_tile_codes", "fgx_tile_fill",
@@ -73,7 +73,8 @@ def lib() -> C.CDLL:
         L.fgx_last_error.restype = C.c_char_p
         for name in ("fgx_sort_workspace_bytes", "fgx_locality_workspace_bytes", "fgx_pair_workspace_bytes", "fgx_tile_workspace_bytes",
                      "fgx_weight_panel_bytes", "fgx_conv_scratch_bytes", "fgx_wgrad_scratch_bytes",
-                     "fgx_colsum_scratch_bytes", "fgx_spconv_out_coords_workspace_bytes"):
+                     "fgx_colsum_scratch_bytes", "fgx_spconv_out_coords_workspace_bytes",
+                     "fgx_subm_neighbor_map_sorted_workspace_bytes"):
             getattr(L, name).restype = C.c_size_t
         _lib = L
     return _lib

@@ -33,7 +33,10 @@ namespace {
 constexpr int kPlanSlots = 4;        // index ring depth
 constexpr int kPlanAhead = 3;        // the index stream runs this many offsets ahead of the row stream
 constexpr uint32_t kOobOffset = 0xFF000000u;   // buffer offset no source tensor reaches: the load returns zeros
-constexpr int kStreamStages = 3;
+constexpr int kBandSlots = 8;        // band-mask ring depth: a mask is read up to (stages - 2) steps after it was written
+#ifndef FGX_EXP_SHORT_STAGES
+#define FGX_EXP_SHORT_STAGES 3
+#endif
 constexpr int kLoaders = 4;          // loader wavefronts per workgroup (one per SIMD)
 
 using rsrc_t = __amdgpu_buffer_rsrc_t;
@@ -45,7 +48,7 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint32_t bytes) {
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int CH>
 struct StreamCfg {
     using T = typename Tag::type;
-    static constexpr int S = kStreamStages;
+    static constexpr int S = CH == 4 ? FGX_EXP_SHORT_STAGES : 3;   // ring stages
     static constexpr int ES = (int)sizeof(T);
     static constexpr int NW = WAVES_M * WAVES_N;               // multiplying wavefronts
     static constexpr int NL = kLoaders;
@@ -74,7 +77,8 @@ struct StreamCfg {
     static_assert(NW * OUT_BAND_BYTES <= STAGE_BYTES, "the output bands must fit one ring stage");
     static_assert(LPS + 1 < 64, "vmcnt is a 6-bit counter");
     static_assert(CH == 4 || CH == 8, "slab must be 64 or 128 bytes");
-    static constexpr size_t fixed_lds = (size_t)S * STAGE_BYTES + (size_t)kPlanSlots * IDX_SLOT_BYTES + OROW_BYTES + kPlanSlots * 4;
+    static_assert(S >= 3 && S - 1 < kBandSlots, "a band mask must outlive the S - 2 steps between its writing and its reading");
+    static constexpr size_t fixed_lds = (size_t)S * STAGE_BYTES + (size_t)kPlanSlots * IDX_SLOT_BYTES + OROW_BYTES + kBandSlots * 4;
 };
 
 // s_waitcnt vmcnt(n) for a wave-uniform n in [LO, HI]: the count is an immediate, so a binary tree of scalar branches
@@ -113,8 +117,8 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     unsigned char* ring = lds_raw;                                          // [S][A: BM x SLAB | B: BN x SLAB]
     uint32_t* idx_ring = (uint32_t*)(ring + S * C::STAGE_BYTES);            // [kPlanSlots][BM] source rows of one offset
     uint32_t* orow_lds = idx_ring + kPlanSlots * BM;                        // [2][NW][OROW_INST * 64] output rows
-    uint32_t* band_lds = orow_lds + C::OROW_BYTES / 4;                      // [kPlanSlots] band masks, loaders -> multipliers
-    float* bias_lds = (float*)(band_lds + kPlanSlots);                      // [cols_pad]
+    uint32_t* band_lds = orow_lds + C::OROW_BYTES / 4;                      // [kBandSlots] band masks, loaders -> multipliers
+    float* bias_lds = (float*)(band_lds + kBandSlots);                      // [cols_pad]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -219,7 +223,7 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     // starts the index load of the offset kPlanAhead further on; issue_step() enqueues the loads of the current step
     // and moves on by one K-slab.
     bool p_ready = false;
-    int p_slab = 0, p_ring = 0, p_stage = 0;
+    int p_slab = 0, p_ring = 0, p_band = 0, p_stage = 0;
     uint32_t a_soff = 0, b_soff = 0, cur_band = 0;
     const uint32_t b_slab_stride = (uint32_t)cols_pad * kSlabBytes;
     auto slot_begin = [&]() -> int {
@@ -237,7 +241,8 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
         const uint32_t* slot = idx_ring + p_ring * BM;
         // for the multipliers, who fetch it at least two barriers from now; the reads of the index column below are
         // waited for before this wavefront reaches its next barrier, and LDS finishes a wavefront's accesses in order
-        if (lw == 0 && lane == 0) band_lds[p_ring] = cur_band;
+        if (lw == 0 && lane == 0) band_lds[p_band] = cur_band;
+        p_band = (p_band + 1) & (kBandSlots - 1);
         p_ring = (p_ring + 1) & (kPlanSlots - 1);
 #pragma unroll
         for (int i = 0; i < C::A_PER; ++i) {
@@ -402,7 +407,7 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
             // wait for this step's fragments covers it
             if (m_slab == 0) {
                 m_next = band_lds[m_ring];
-                m_ring = (m_ring + 1) & (kPlanSlots - 1);
+                m_ring = (m_ring + 1) & (kBandSlots - 1);
             }
             if (m_mine != 0) {
                 u32x4 af[kChunks / 2][C::TM], bf[kChunks / 2][C::TN];

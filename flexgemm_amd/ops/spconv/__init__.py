@@ -39,6 +39,20 @@ OUT_COORD_ALGO = SparseConv3dOutCoordAlgorithm.HASHMAP
 SERIALIZATION_MODE = SerializationMode.BXYZ
 
 
+# How the submanifold neighbor map is found (no counterpart in the reference, which always hashes; the map is the same
+# either way): "hash" = open-addressing table and probes, "sort" = radix sort of the flattened keys and windowed merges,
+# "auto" = "sort" from SORT_BUILDER_MIN_VOXELS voxels on.
+NEIGHBOR_MAP_BUILDER = "auto"
+SORT_BUILDER_MIN_VOXELS = 32768
+
+
+def set_neighbor_map_builder(builder: str):
+    global NEIGHBOR_MAP_BUILDER
+    if builder not in ("auto", "hash", "sort"):
+        raise ValueError(f"unknown neighbor map builder {builder!r}; expected 'auto', 'hash' or 'sort'")
+    NEIGHBOR_MAP_BUILDER = builder
+
+
 def set_algorithm(algorithm: str):
     global ALGORITHM
     ALGORITHM = algorithm

@@ -252,19 +252,33 @@ def _pair_lists(nmap: torch.Tensor, gray: torch.Tensor):
 
 def _build_neighbor_map(coords: torch.Tensor, shape, kernel_size, dilation, with_codes: bool):
     n = coords.shape[0]
-    _, _, W, H, D = [int(s) for s in shape]
+    B, _, W, H, D = [int(s) for s in shape]
     kw, kh, kd = [int(k) for k in kernel_size]
     v = kw * kh * kd
     dev = coords.device
-    table = int(spconv.HASHMAP_RATIO * n)
-    if n > 0 and table < n:
-        raise ValueError(f"hashmap ratio {spconv.HASHMAP_RATIO} gives a table smaller than the input")
-    keys, vals = utils.init_hashmap(shape, table, dev)
     nmap = torch.empty((n, v), dtype=torch.uint32, device=dev)
     gray = binary = None
     if with_codes:
         gray = torch.empty((n,), dtype=torch.int32, device=dev)
         binary = torch.empty((n,), dtype=torch.int32, device=dev)
+    builder = spconv.NEIGHBOR_MAP_BUILDER
+    if builder == "auto":
+        builder = "sort" if n >= spconv.SORT_BUILDER_MIN_VOXELS else "hash"
+    vol = B * W * H * D
+    if builder == "sort" and kw * kh <= 128 and vol <= 2 ** 63:
+        key_bits = 32 if vol <= 2 ** 32 else 64
+        with torch.cuda.device(dev):
+            L = nat.lib()
+            ws = nat.workspace(L.fgx_subm_neighbor_map_sorted_workspace_bytes(nat.sz(n), C.c_int(key_bits), C.c_int(kw), C.c_int(kh)), dev)
+            nat.check(L.fgx_subm_neighbor_map_sorted(
+                nat.ptr(coords), nat.sz(n), C.c_int(B), C.c_int(W), C.c_int(H), C.c_int(D), C.c_int(kw), C.c_int(kh), C.c_int(kd),
+                C.c_int(int(dilation[0])), C.c_int(int(dilation[1])), C.c_int(int(dilation[2])), C.c_int(key_bits),
+                nat.ptr(ws), nat.sz(ws.numel()), nat.ptr(nmap), nat.ptr(gray), nat.ptr(binary), nat.stream()))
+        return nmap, gray, binary
+    table = int(spconv.HASHMAP_RATIO * n)
+    if n > 0 and table < n:
+        raise ValueError(f"hashmap ratio {spconv.HASHMAP_RATIO} gives a table smaller than the input")
+    keys, vals = utils.init_hashmap(shape, table, dev)
     with torch.cuda.device(dev):
         nat.check(nat.lib().fgx_subm_neighbor_map(
             nat.ptr(keys), C.c_int(32 if keys.dtype == torch.uint32 else 64), nat.ptr(vals), nat.sz(table),

@@ -88,6 +88,19 @@ int fgx_subm_neighbor_map(void* keys, int key_bits, uint32_t* vals, size_t table
                           int Kw, int Kh, int Kd, int Dw, int Dh, int Dd,
                           uint32_t* out_map, int32_t* gray, int32_t* binary, fgx_stream_t stream);
 
+/* The same table as fgx_subm_neighbor_map without a hash table: (flattened key, row) pairs are radix-sorted, and a
+ * workgroup of 256 consecutive sorted voxels finds, for every (dx, dy), all its neighbors in one contiguous window of
+ * the sorted array (two binary searches, one coalesced read into LDS, per-lane searches there).  Meant for large or
+ * shuffled coordinate sets, where hash probes are cache-line fetches at random addresses.  key_bits: 32 when
+ * B*W*H*D <= 2^32, else 64 (grids up to 2^63 cells).  workspace: fgx_subm_neighbor_map_sorted_workspace_bytes bytes,
+ * 256-byte aligned.  gray / binary as above.
+ * Replaces: the same reference function as fgx_subm_neighbor_map (the result is identical; only the search differs). */
+size_t fgx_subm_neighbor_map_sorted_workspace_bytes(size_t n, int key_bits, int Kw, int Kh);
+int fgx_subm_neighbor_map_sorted(const int32_t* coords, size_t n, int B, int W, int H, int D,
+                                 int Kw, int Kh, int Kd, int Dw, int Dh, int Dd, int key_bits,
+                                 void* workspace, size_t workspace_bytes,
+                                 uint32_t* out_map, int32_t* gray, int32_t* binary, fgx_stream_t stream);
+
 /* Validity mask (bit v <=> map[n, v] present) and Gray-decoded key from an existing map.
  * Replaces: neighbor_map_to_gray_binary_code_kernel, migemm_neighmap_pp.cu:19-44. */
 int fgx_mask_codes(const uint32_t* map, size_t n, int V, int32_t* gray, int32_t* binary, fgx_stream_t stream);

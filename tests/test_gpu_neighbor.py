@@ -23,6 +23,14 @@ def _say(msg):
     sys.stdout.flush()
 
 
+@pytest.fixture(params=["hash", "sort"], autouse=True)
+def neighbor_map_builder(request):
+    """Every test of this file runs once per way of finding the neighbors: the tables must not depend on it."""
+    flex_gemm.ops.spconv.set_neighbor_map_builder(request.param)
+    yield request.param
+    flex_gemm.ops.spconv.set_neighbor_map_builder("auto")
+
+
 def _np(t):
     if t.dtype == torch.uint32:
         return t.cpu().view(torch.int32).numpy().view(np.uint32)
