@@ -28,7 +28,7 @@ const Entry kTable[] = {
     {2, 2, 17, 256, 256, {128, 128, 64, 1, 4096, 1}},
     {0, 2, 21, 32, 32, {256, 32, 64, 1, 0, 1}},
     {1, 2, 21, 32, 32, {256, 32, 64, 1, 0, 1}},
-    {2, 2, 21, 32, 32, {32, 32, 64, 1, 4096, 0}},
+    {2, 2, 21, 32, 32, {32, 32, 64, 1, 16384, 1}},
     {0, 2, 15, 1024, 1024, {256, 128, 128, 1, 0, 1}},
     {1, 2, 15, 1024, 1024, {256, 128, 128, 1, 0, 1}},
     {2, 2, 15, 1024, 1024, {128, 128, 64, 1, 65536, 1}},
@@ -53,13 +53,16 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
         out->tile_cols = t;
         out->slab_bytes = 64;
         out->splitk = 1;
-        // persistent streaming kernel: 16-bit types, tiles of at least 64, enough voxels to give every CU several items
-        out->stream = (es == 2 && t >= 64 && n >= 32768) ? 1 : 0;
-        const double per_block = 4.0 * V * (double)Co * (double)Ci;
+        // persistent streaming kernel: 16-bit types, enough voxels to give every CU several items.  Its 32 x 32 tile
+        // writes four partial products per voxel block (one per multiplying wavefront), so its blocks are four times
+        // as long.
+        out->stream = (es == 2 && n >= 32768) ? 1 : 0;
+        const int slices = (out->stream && t == 32) ? 4 : 1;
+        const double per_block = 4.0 * V * (double)Co * (double)Ci * slices;
         size_t max_blocks = (size_t)(268435456.0 / per_block);
         if (max_blocks < 1) max_blocks = 1;
         size_t rows = round_up((n + max_blocks - 1) / max_blocks, 1024);
-        if (rows < 4096) rows = 4096;
+        if (rows < (size_t)4096 * slices) rows = (size_t)4096 * slices;
         if (rows > 0x40000000) rows = 0x40000000;
         out->block_rows = (int)rows;
         return;

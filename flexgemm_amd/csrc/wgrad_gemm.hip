@@ -392,9 +392,15 @@ template <typename Tag, int BM, int BN>
 struct WStreamCfg {
     using T = typename Tag::type;
     static constexpr int ES = (int)sizeof(T);
-    static constexpr int P = kWsPairs, S = kWsStages;
+    // A 32 x 32 tile is one MFMA tile: the four multipliers then split the PAIRS of a step among themselves (each owns a
+    // quarter of the pair rows and keeps its own accumulator, written out as a partial product of its own), and a step
+    // carries four times the pairs so that its loads are as many bytes as a wide tile's.
+    static constexpr bool KSPLIT = BM == 32 && BN == 32;
+    static constexpr int SLICES = KSPLIT ? 4 : 1;                  // partial products per (voxel block, offset, tile)
+    static constexpr int P = KSPLIT ? 4 * kWsPairs : kWsPairs, S = kWsStages;
     static constexpr int NW = 4, NL = kWsLoaders, NT = 64 * (NW + NL);
-    static constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+    static constexpr int WM = KSPLIT ? BM : BM / 2, WN = KSPLIT ? BN : BN / 2, TM = WM / 32, TN = WN / 32;
+    static constexpr int IDX_PER = P / 64;                         // wave-wide index loads per operand and step
     static constexpr int ROWB_A = BM * ES, ROWB_B = BN * ES;
     static constexpr int CH_A = ROWB_A / 16, CH_B = ROWB_B / 16;
     static constexpr int RPI_A = 64 / CH_A, RPI_B = 64 / CH_B;
@@ -404,7 +410,7 @@ struct WStreamCfg {
     static constexpr int IDX_SLOT_BYTES = 2 * P * 4;               // sig_o x P | sig_i x P
     static constexpr size_t lds_bytes = (size_t)S * STAGE_BYTES + (size_t)kWsIdxSlots * IDX_SLOT_BYTES;
     static_assert(ES == 2, "the streaming kernel handles 16-bit types");
-    static_assert(P == 64, "one wave-wide index load per operand and step");
+    static_assert(IDX_PER == 1 || IDX_PER == NL, "index loads: one loader per operand, or every loader a quarter of both");
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
     static_assert(P % (RPI_A * NL) == 0 && P % (RPI_B * NL) == 0, "every loader issues the same row loads");
     static_assert(2 * (LPS + 1) < 64, "outstanding loads exceed the vmcnt range");
@@ -442,7 +448,7 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const bool loader = wave >= C::NW;
     const int lw = loader ? wave - C::NW : 0, mw = loader ? 0 : wave;
-    const int wave_m = mw >> 1, wave_n = mw & 1;
+    const int wave_m = C::KSPLIT ? 0 : mw >> 1, wave_n = C::KSPLIT ? 0 : mw & 1;
     const int g = lane >> 5, l32 = lane & 31;
 
     // ---- item list: block-major (block, offset, tile); XCD x owns the x-th eighth, its workgroups interleave ----
@@ -517,13 +523,22 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
             if (!f.live) return 0;
             int ops = 0;
             uint32_t* dst = idx_ring + (f_step & (kWsIdxSlots - 1)) * (2 * P);
-            if (lw == 0) {
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(sigo_rs, FGX_LDS_PTR(dst), 4, (f.k + (uint32_t)lane) * 4u, 0, 0, 0);
-                ops = 1;
-            } else if (lw == 1) {
-                uint32_t* dst_i = dst + P;
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(sigi_rs, FGX_LDS_PTR(dst_i), 4, (f.k + (uint32_t)lane) * 4u, 0, 0, 0);
-                ops = 1;
+            if constexpr (C::IDX_PER == 1) {
+                if (lw == 0) {
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(sigo_rs, FGX_LDS_PTR(dst), 4, (f.k + (uint32_t)lane) * 4u, 0, 0, 0);
+                    ops = 1;
+                } else if (lw == 1) {
+                    uint32_t* dst_i = dst + P;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(sigi_rs, FGX_LDS_PTR(dst_i), 4, (f.k + (uint32_t)lane) * 4u, 0, 0, 0);
+                    ops = 1;
+                }
+            } else {        // every loader fetches its quarter of both index columns
+                const uint32_t vo = (f.k + (uint32_t)(lw * 64 + lane)) * 4u;
+                uint32_t* dst_o = dst + lw * 64;
+                uint32_t* dst_i = dst + P + lw * 64;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(sigo_rs, FGX_LDS_PTR(dst_o), 4, vo, 0, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(sigi_rs, FGX_LDS_PTR(dst_i), 4, vo, 0, 0, 0);
+                ops = 2;
             }
             ++f_step;
             advance(f);
@@ -646,7 +661,8 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
             b_off[j][1] = C::A_BYTES + (prow + 4) * C::ROWB_B + ((c ^ C::key_b(prow + 4)) << 4) + w;
         }
     }
-    constexpr int NK = P / 16;
+    constexpr int NK = P / 16 / C::SLICES;          // k-blocks (16 pair rows) this wavefront multiplies per step
+    const int kk0 = C::KSPLIT ? mw * NK : 0;        // ... starting at this one
     constexpr int RK = 2 * (C::TM + C::TN);         // LDS reads per k-block
     Walk m = first;
     unsigned step = 0;
@@ -671,7 +687,8 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
             // rows 0-15 / 16-31, the two wave halves take pair rows [0, 8) / [8, 16) of the k-block.  The reads of
             // k-block kk+1 are in flight while k-block kk is multiplied.
             i16x4 fr[2][RK];
-            auto read_block = [&](int kk, i16x4 (&dst)[RK]) {
+            auto read_block = [&](int kl, i16x4 (&dst)[RK]) {
+                const int kk = kk0 + kl;
                 const unsigned char* base = cur + kk * 16 * C::ROWB_A;      // ROWB_A == ROWB_B is not assumed below
 #pragma unroll
                 for (int i = 0; i < C::TM; ++i) {
@@ -707,7 +724,7 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
         // partial[b][v][co][ci], fp32
         const unsigned co_tile = tile % co_tiles, ci_tile = tile / co_tiles;
         const int m0 = (int)co_tile * BM, n0 = (int)ci_tile * BN;
-        float* dst = partial + ((size_t)b * V + v) * ((size_t)Co * Ci);
+        float* dst = partial + (((size_t)b * C::SLICES + (C::KSPLIT ? mw : 0)) * V + v) * ((size_t)Co * Ci);
 #pragma unroll
         for (int j = 0; j < C::TN; ++j) {
             const int ci = n0 + wave_n * C::WN + j * 32 + l32;
@@ -736,7 +753,8 @@ constexpr int kReduceElems = 32, kReduceSlices = 8;
 template <typename T>
 __global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restrict__ partial,
                                                            const uint32_t* __restrict__ bounds, int V, int Ci, int Co,
-                                                           unsigned nb, T* __restrict__ gw) {
+                                                           unsigned nb, unsigned per_block, T* __restrict__ gw) {
+    // `per_block` partial products per voxel block (consecutive in `partial`); nb counts the partial products
     __shared__ float sums[kReduceSlices][kReduceElems];
     const size_t per = (size_t)Co * Ci;
     const size_t total = per * V;
@@ -750,7 +768,7 @@ __global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restri
             size_t t = i / Ci;
             int v = (int)(t % V);
             int co = (int)(t / V);
-            const uint32_t* bd = bounds + (size_t)v * (nb + 1);
+            const uint32_t* bd = bounds + (size_t)v * (nb / per_block + 1);
             const float* src = partial + (size_t)v * per + (size_t)co * Ci + ci;
             const size_t stride = (size_t)V * per;
             unsigned b = slice * chunk;
@@ -758,12 +776,17 @@ __global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restri
             for (; b + 8 <= end; b += 8) {
                 float x[8];
 #pragma unroll
-                for (int q = 0; q < 8; ++q) x[q] = bd[b + q] < bd[b + q + 1] ? src[(size_t)(b + q) * stride] : 0.f;
+                for (int q = 0; q < 8; ++q) {
+                    const unsigned blk = (b + q) / per_block;
+                    x[q] = bd[blk] < bd[blk + 1] ? src[(size_t)(b + q) * stride] : 0.f;
+                }
 #pragma unroll
                 for (int q = 0; q < 8; ++q) s += x[q];
             }
-            for (; b < end; ++b)
-                if (bd[b] < bd[b + 1]) s += src[(size_t)b * stride];
+            for (; b < end; ++b) {
+                const unsigned blk = b / per_block;
+                if (bd[blk] < bd[blk + 1]) s += src[(size_t)b * stride];
+            }
         }
         sums[slice][e] = s;
         __syncthreads();
@@ -784,14 +807,15 @@ struct Layout {
     size_t bounds_off, partial_off, total;
 };
 
-Layout layout(size_t n, int V, int Ci, int Co, int block_rows) {
+// `slices`: partial products per (voxel block, offset, tile)
+Layout layout(size_t n, int V, int Ci, int Co, int block_rows, int slices) {
     Layout L{};
     L.nb = n ? cdiv(n, (size_t)block_rows) : 0u;
     size_t off = 0;
     L.bounds_off = off;
     off = align_up(off + (size_t)V * (L.nb + 1) * sizeof(uint32_t), 256);
     L.partial_off = off;
-    off += (size_t)(L.nb ? L.nb : 1) * V * Co * Ci * sizeof(float);
+    off += (size_t)(L.nb ? L.nb : 1) * slices * V * Co * Ci * sizeof(float);
     L.total = off;
     return L;
 }
@@ -822,7 +846,7 @@ int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, con
     size_t total = (size_t)Co * V * Ci;
     unsigned g = cdiv(total, kReduceElems);
     if (g > 65536u) g = 65536u;
-    wgrad_reduce_kernel<T><<<g, 256, 0, s>>>(partial, bounds, V, Ci, Co, L.nb, (T*)gw);
+    wgrad_reduce_kernel<T><<<g, 256, 0, s>>>(partial, bounds, V, Ci, Co, L.nb, 1u, (T*)gw);
     FGX_CHECK_LAUNCH("fgx_conv_wgrad(reduce)");
     return FGX_OK;
 }
@@ -861,7 +885,7 @@ int launch_wgrad_stream(const void* gout, const void* feats, const uint32_t* sig
     size_t total = (size_t)Co * V * Ci;
     unsigned g = cdiv(total, kReduceElems);
     if (g > 65536u) g = 65536u;
-    wgrad_reduce_kernel<T><<<g, 256, 0, s>>>(partial, bounds, V, Ci, Co, L.nb, (T*)gw);
+    wgrad_reduce_kernel<T><<<g, 256, 0, s>>>(partial, bounds, V, Ci, Co, L.nb * C::SLICES, (unsigned)C::SLICES, (T*)gw);
     FGX_CHECK_LAUNCH("fgx_conv_wgrad(reduce)");
     return FGX_OK;
 }
@@ -870,7 +894,8 @@ int launch_wgrad_stream(const void* gout, const void* feats, const uint32_t* sig
 template <typename Tag>
 bool stream_ok(int tile_rows, int tile_cols, size_t n, size_t n_in, int Ci, int Co, uint32_t n_pairs) {
     if (sizeof(typename Tag::type) != 2) return false;
-    if (!((tile_rows == 128 && tile_cols == 128) || (tile_rows == 64 && tile_cols == 64))) return false;
+    if (!((tile_rows == 128 && tile_cols == 128) || (tile_rows == 64 && tile_cols == 64) || (tile_rows == 32 && tile_cols == 32)))
+        return false;
     return (double)n * Co * 2 <= (double)kOobOffset && (double)n_in * Ci * 2 <= (double)kOobOffset &&
            (double)n_pairs * 4 + 256 <= (double)kOobOffset;
 }
@@ -881,7 +906,8 @@ int dispatch_wgrad_stream(int tile_rows, const void* gout, const void* feats, co
                           void* scratch, void* gw, hipStream_t s) {
     if constexpr (sizeof(typename Tag::type) == 2) {
         if (tile_rows == 128) return launch_wgrad_stream<Tag, 128, 128>(gout, feats, sig_i, sig_o, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, s);
-        return launch_wgrad_stream<Tag, 64, 64>(gout, feats, sig_i, sig_o, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, s);
+        if (tile_rows == 64) return launch_wgrad_stream<Tag, 64, 64>(gout, feats, sig_i, sig_o, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, s);
+        return launch_wgrad_stream<Tag, 32, 32>(gout, feats, sig_i, sig_o, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, s);
     } else {
         set_error("fgx_conv_wgrad: the streaming kernel handles 16-bit types only");
         return FGX_ERR_UNSUPPORTED;
@@ -912,7 +938,8 @@ extern "C" {
 
 size_t fgx_wgrad_scratch_bytes(size_t n, int V, int Ci, int Co, int block_rows) {
     if (V < 1 || V > kMaxV || Ci <= 0 || Co <= 0 || block_rows <= 0) return 0;
-    return layout(n, V, Ci, Co, block_rows).total;
+    // room for the four partial products per block of the pair-splitting 32 x 32 streaming tile wherever it could run
+    return layout(n, V, Ci, Co, block_rows, (Ci < Co ? Ci : Co) <= 32 ? 4 : 1).total;
 }
 
 int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
@@ -938,17 +965,17 @@ int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uin
         FGX_CHECK_ARG(grad_out && feats && sig_i && sig_o, "fgx_conv_wgrad: null buffer");
         FGX_CHECK_ARG((((uintptr_t)grad_out | (uintptr_t)feats) & 15) == 0, "fgx_conv_wgrad: grad_out and feats must be 16-byte aligned");
     }
-    Layout L = layout(any ? n : 0, V, Ci, Co, block_rows);
+    const bool stream_f16 = streaming && any && dtype == FGX_F16 && stream_ok<F16>(tile_rows, tile_cols, n, n_in, Ci, Co, tab.seg[V]);
+    const bool stream_bf16 = streaming && any && dtype == FGX_BF16 && stream_ok<BF16>(tile_rows, tile_cols, n, n_in, Ci, Co, tab.seg[V]);
+    Layout L = layout(any ? n : 0, V, Ci, Co, block_rows, (stream_f16 || stream_bf16) && tile_rows == 32 ? 4 : 1);
     // 32-bit byte offsets into grad_out / feats are enough below 4 GiB
     const bool small = (double)n * Co * es < 4294967296.0 && (double)n_in * Ci * es < 4294967296.0;
     hipStream_t s = (hipStream_t)stream;
-    if (streaming && any) {
-        // falls through to the tiled kernel when the problem is outside the streaming kernel's range
-        if (dtype == FGX_F16 && stream_ok<F16>(tile_rows, tile_cols, n, n_in, Ci, Co, tab.seg[V]))
-            return dispatch_wgrad_stream<F16>(tile_rows, grad_out, feats, sig_i, sig_o, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, s);
-        if (dtype == FGX_BF16 && stream_ok<BF16>(tile_rows, tile_cols, n, n_in, Ci, Co, tab.seg[V]))
-            return dispatch_wgrad_stream<BF16>(tile_rows, grad_out, feats, sig_i, sig_o, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, s);
-    }
+    // (outside the streaming kernel's range the tiled kernel runs)
+    if (stream_f16)
+        return dispatch_wgrad_stream<F16>(tile_rows, grad_out, feats, sig_i, sig_o, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, s);
+    if (stream_bf16)
+        return dispatch_wgrad_stream<BF16>(tile_rows, grad_out, feats, sig_i, sig_o, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, s);
     switch (dtype) {
         case FGX_F16: return dispatch_wgrad<F16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);
         case FGX_BF16: return dispatch_wgrad<BF16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);

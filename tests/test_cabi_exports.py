@@ -66,7 +66,9 @@ def test_host_only_entry_points(library):
     assert L.fgx_conv_scratch_bytes(ctypes.c_size_t(1000), 64, 1) == 0
     assert L.fgx_conv_scratch_bytes(ctypes.c_size_t(1000), 64, 4) == 4 * 1000 * 64 * 4
     # 1000 rows in blocks of 256 -> 4 blocks: bounds table (3 * 5 uint32, padded to 256 B) + 4 * 3 partial products
-    assert L.fgx_wgrad_scratch_bytes(ctypes.c_size_t(1000), 3, 8, 16, 256) == 256 + 4 * 3 * 8 * 16 * 4
+    assert L.fgx_wgrad_scratch_bytes(ctypes.c_size_t(1000), 3, 48, 64, 256) == 256 + 4 * 3 * 48 * 64 * 4
+    # up to 32 channels on either side: room for the four partial products per block of the 32 x 32 streaming tile
+    assert L.fgx_wgrad_scratch_bytes(ctypes.c_size_t(1000), 3, 8, 16, 256) == 256 + 4 * 4 * 3 * 8 * 16 * 4
 
 
 def test_argument_errors_map_to_exceptions(library):

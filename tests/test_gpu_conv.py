@@ -312,10 +312,13 @@ def test_gather_plan_band_masks(gpu_device):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("res,ci,co,tile,block_rows", [(32, 128, 128, 128, 1024), (24, 64, 64, 64, 512), (24, 96, 40, 128, 300),
-                                                       (16, 256, 136, 128, 100000), (48, 128, 128, 128, 37)])
+                                                       (16, 256, 136, 128, 100000), (48, 128, 128, 128, 37),
+                                                       (32, 32, 32, 32, 2048), (24, 24, 72, 32, 300), (40, 32, 32, 32, 100000),
+                                                       (24, 16, 32, 32, 50)])
 def test_streaming_wgrad_matches_oracle(gpu_device, dtype, res, ci, co, tile, block_rows):
     """wgrad with the persistent streaming kernel forced: edge tiles, several Co / Ci tiles, voxel blocks smaller
-    than a 64-pair step (most steps partial, many empty items) and one block for everything."""
+    than a 64-pair step (most steps partial, many empty items) and one block for everything; the 32 x 32 tile splits
+    the pairs of a step over its four multiplying wavefronts (ragged steps, channel counts below the tile)."""
     _say(f"stream wgrad res={res} ci={ci} co={co} tile={tile} block_rows={block_rows} {dtype}")
     coords_np = reference_test_shell(res)
     shape = torch.Size([1, ci, res, res, res])
