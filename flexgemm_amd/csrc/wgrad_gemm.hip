@@ -800,6 +800,50 @@ __global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restri
     }
 }
 
+// The same sum with one thread per element, for few partial products (the sliced kernel's eight thread groups
+// per element would mostly idle).  Which of the two runs depends on the number of partial products alone.
+template <typename T>
+__global__ void __launch_bounds__(256) wgrad_reduce_flat_kernel(const float* __restrict__ partial,
+                                                                const uint32_t* __restrict__ bounds, int V, int Ci, int Co,
+                                                                unsigned nb, unsigned per_block, T* __restrict__ gw) {
+    const size_t per = (size_t)Co * Ci;
+    const size_t total = per * V;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        int ci = (int)(i % Ci);
+        size_t t = i / Ci;
+        int v = (int)(t % V);
+        int co = (int)(t / V);
+        const uint32_t* bd = bounds + (size_t)v * (nb / per_block + 1);
+        const float* src = partial + (size_t)v * per + (size_t)co * Ci + ci;
+        const size_t stride = (size_t)V * per;
+        float s = 0.f;
+        for (unsigned b = 0; b < nb; ++b) {
+            const unsigned blk = b / per_block;
+            if (bd[blk] < bd[blk + 1]) s += src[(size_t)b * stride];
+        }
+        gw[i] = from_float<T>(s);
+    }
+}
+
+constexpr unsigned kReduceSlicedFrom = 32;      // partial products from which the sliced reduction is used
+
+template <typename T>
+int launch_reduce(const float* partial, const uint32_t* bounds, int V, int Ci, int Co, unsigned nb, unsigned per_block, T* gw,
+                  hipStream_t s) {
+    const size_t total = (size_t)Co * V * Ci;
+    if (nb >= kReduceSlicedFrom) {
+        unsigned g = cdiv(total, kReduceElems);
+        if (g > 65536u) g = 65536u;
+        wgrad_reduce_kernel<T><<<g, 256, 0, s>>>(partial, bounds, V, Ci, Co, nb, per_block, gw);
+    } else {
+        unsigned g = cdiv(total, 256);
+        if (g > 65536u) g = 65536u;
+        wgrad_reduce_flat_kernel<T><<<g, 256, 0, s>>>(partial, bounds, V, Ci, Co, nb, per_block, gw);
+    }
+    FGX_CHECK_LAUNCH("fgx_conv_wgrad(reduce)");
+    return FGX_OK;
+}
+
 bool dtype_ok(int dtype) { return dtype == FGX_F16 || dtype == FGX_BF16 || dtype == FGX_F32; }
 
 struct Layout {
@@ -843,12 +887,7 @@ int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, con
             (const T*)gout, (const T*)feats, sig_i, sig_o, bounds, V, Ci, Co, L.nb, co_tiles, ci_tiles, small, partial);
         FGX_CHECK_LAUNCH("fgx_conv_wgrad");
     }
-    size_t total = (size_t)Co * V * Ci;
-    unsigned g = cdiv(total, kReduceElems);
-    if (g > 65536u) g = 65536u;
-    wgrad_reduce_kernel<T><<<g, 256, 0, s>>>(partial, bounds, V, Ci, Co, L.nb, 1u, (T*)gw);
-    FGX_CHECK_LAUNCH("fgx_conv_wgrad(reduce)");
-    return FGX_OK;
+    return launch_reduce<T>(partial, bounds, V, Ci, Co, L.nb, 1u, (T*)gw, s);
 }
 
 template <typename Tag, int BM, int BN>
@@ -882,12 +921,7 @@ int launch_wgrad_stream(const void* gout, const void* feats, const uint32_t* sig
                                                  (uint32_t)(n_in * (size_t)Ci * sizeof(T)), partial);
         FGX_CHECK_LAUNCH("fgx_conv_wgrad(stream)");
     }
-    size_t total = (size_t)Co * V * Ci;
-    unsigned g = cdiv(total, kReduceElems);
-    if (g > 65536u) g = 65536u;
-    wgrad_reduce_kernel<T><<<g, 256, 0, s>>>(partial, bounds, V, Ci, Co, L.nb * C::SLICES, (unsigned)C::SLICES, (T*)gw);
-    FGX_CHECK_LAUNCH("fgx_conv_wgrad(reduce)");
-    return FGX_OK;
+    return launch_reduce<T>(partial, bounds, V, Ci, Co, L.nb * C::SLICES, (unsigned)C::SLICES, (T*)gw, s);
 }
 
 // the streaming kernel: 16-bit types, tiles of 128x128 or 64x64, operands addressable with 32-bit offsets
