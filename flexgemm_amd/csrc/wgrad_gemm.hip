@@ -800,8 +800,9 @@ __global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restri
     }
 }
 
-// The same sum with one thread per element, for few partial products (the sliced kernel's eight thread groups
-// per element would mostly idle).  Which of the two runs depends on the number of partial products alone.
+// The same sum with one thread per element: 1 KiB contiguous per workgroup and block.  Used unless the weight is so small
+// that this leaves most CUs idle while every thread walks a long list of blocks.  Which of the two runs depends on the
+// problem's shape alone, not on which kernel wrote the partial products.
 template <typename T>
 __global__ void __launch_bounds__(256) wgrad_reduce_flat_kernel(const float* __restrict__ partial,
                                                                 const uint32_t* __restrict__ bounds, int V, int Ci, int Co,
@@ -817,7 +818,18 @@ __global__ void __launch_bounds__(256) wgrad_reduce_flat_kernel(const float* __r
         const float* src = partial + (size_t)v * per + (size_t)co * Ci + ci;
         const size_t stride = (size_t)V * per;
         float s = 0.f;
-        for (unsigned b = 0; b < nb; ++b) {
+        unsigned b = 0;
+        for (; b + 8 <= nb; b += 8) {     // eight independent loads in flight; the sum order stays b-ascending
+            float x[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const unsigned blk = (b + q) / per_block;
+                x[q] = bd[blk] < bd[blk + 1] ? src[(size_t)(b + q) * stride] : 0.f;
+            }
+#pragma unroll
+            for (int q = 0; q < 8; ++q) s += x[q];
+        }
+        for (; b < nb; ++b) {
             const unsigned blk = b / per_block;
             if (bd[blk] < bd[blk + 1]) s += src[(size_t)b * stride];
         }
@@ -825,13 +837,14 @@ __global__ void __launch_bounds__(256) wgrad_reduce_flat_kernel(const float* __r
     }
 }
 
-constexpr unsigned kReduceSlicedFrom = 32;      // partial products from which the sliced reduction is used
+constexpr unsigned kReduceSlicedFrom = 32;      // partial products from which the sliced reduction is considered
+constexpr unsigned kReduceFlatGroups = 1024;    // ... when the flat kernel would launch fewer workgroups than this
 
 template <typename T>
 int launch_reduce(const float* partial, const uint32_t* bounds, int V, int Ci, int Co, unsigned nb, unsigned per_block, T* gw,
                   hipStream_t s) {
     const size_t total = (size_t)Co * V * Ci;
-    if (nb >= kReduceSlicedFrom) {
+    if (nb >= kReduceSlicedFrom && cdiv(total, 256) < kReduceFlatGroups) {
         unsigned g = cdiv(total, kReduceElems);
         if (g > 65536u) g = 65536u;
         wgrad_reduce_kernel<T><<<g, 256, 0, s>>>(partial, bounds, V, Ci, Co, nb, per_block, gw);
