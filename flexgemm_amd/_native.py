@@ -31,7 +31,7 @@ EXPORTS = [
     "fgx_table_lookup", "fgx_weight_panel_bytes", "fgx_pack_weight",
     "fgx_conv_scratch_bytes", "fgx_conv_gather_gemm",
     "fgx_gather_plan_count", "fgx_gather_plan_fill", "fgx_conv_gather_gemm_stream",
-    "fgx_wgrad_scratch_bytes", "fgx_conv_wgrad",
+    "fgx_wgrad_scratch_bytes", "fgx_wgrad_block_bounds_count", "fgx_wgrad_block_bounds", "fgx_conv_wgrad",
     "fgx_colsum_scratch_bytes", "fgx_colsum",
     "fgx_spconv_out_dims", "fgx_spconv_out_coords_workspace_bytes", "fgx_spconv_out_coords_keys",
     "fgx_spconv_out_coords_decode", "fgx_spconv_neighbor_map",
@@ -74,7 +74,7 @@ def lib() -> C.CDLL:
         for name in ("fgx_sort_workspace_bytes", "fgx_locality_workspace_bytes", "fgx_pair_workspace_bytes", "fgx_tile_workspace_bytes",
                      "fgx_weight_panel_bytes", "fgx_conv_scratch_bytes", "fgx_wgrad_scratch_bytes",
                      "fgx_colsum_scratch_bytes", "fgx_spconv_out_coords_workspace_bytes",
-                     "fgx_subm_neighbor_map_sorted_workspace_bytes"):
+                     "fgx_subm_neighbor_map_sorted_workspace_bytes", "fgx_wgrad_block_bounds_count"):
             getattr(L, name).restype = C.c_size_t
         _lib = L
     return _lib

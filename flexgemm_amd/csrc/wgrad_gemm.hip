@@ -878,15 +878,20 @@ Layout layout(size_t n, int V, int Ci, int Co, int block_rows, int slices) {
 }
 
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N>
-int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o, const SegTable& tab,
+int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
+                 const uint32_t* given_bounds, const SegTable& tab,
                  const Layout& L, bool small, int V, int Ci, int Co, int block_rows, void* scratch, void* gw, hipStream_t s) {
     using C = WgradCfg<Tag, BM, BN, WAVES_M, WAVES_N>;
     using T = typename Tag::type;
-    uint32_t* bounds = (uint32_t*)((char*)scratch + L.bounds_off);
+    // the block table depends on the pair lists and block_rows alone: callers that keep it pass it in
+    const uint32_t* bounds = given_bounds ? given_bounds : (const uint32_t*)((char*)scratch + L.bounds_off);
     float* partial = (float*)((char*)scratch + L.partial_off);
     if (L.nb > 0) {
-        block_bounds_kernel<<<cdiv((size_t)V * (L.nb + 1), 256), 256, 0, s>>>(sig_o, tab, V, L.nb, (unsigned)block_rows, bounds);
-        FGX_CHECK_LAUNCH("fgx_conv_wgrad(bounds)");
+        if (!given_bounds) {
+            block_bounds_kernel<<<cdiv((size_t)V * (L.nb + 1), 256), 256, 0, s>>>(sig_o, tab, V, L.nb, (unsigned)block_rows,
+                                                                                 (uint32_t*)((char*)scratch + L.bounds_off));
+            FGX_CHECK_LAUNCH("fgx_conv_wgrad(bounds)");
+        }
         const unsigned co_tiles = cdiv(Co, BM), ci_tiles = cdiv(Ci, BN);
         const size_t grid = (size_t)cdiv((size_t)L.nb * V * co_tiles * ci_tiles, kXcds) * kXcds;
         FGX_CHECK_ARG(grid < 0x7FFFFFFFull, "fgx_conv_wgrad: too many work items (%zu); use larger voxel blocks", grid);
@@ -905,15 +910,19 @@ int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, con
 
 template <typename Tag, int BM, int BN>
 int launch_wgrad_stream(const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
-                        const SegTable& tab, const Layout& L, size_t n, size_t n_in, int V, int Ci, int Co, int block_rows,
+                        const uint32_t* given_bounds, const SegTable& tab, const Layout& L, size_t n, size_t n_in, int V, int Ci, int Co, int block_rows,
                         void* scratch, void* gw, hipStream_t s) {
     using C = WStreamCfg<Tag, BM, BN>;
     using T = typename Tag::type;
-    uint32_t* bounds = (uint32_t*)((char*)scratch + L.bounds_off);
+    // the block table depends on the pair lists and block_rows alone: callers that keep it pass it in
+    const uint32_t* bounds = given_bounds ? given_bounds : (const uint32_t*)((char*)scratch + L.bounds_off);
     float* partial = (float*)((char*)scratch + L.partial_off);
     if (L.nb > 0) {
-        block_bounds_kernel<<<cdiv((size_t)V * (L.nb + 1), 256), 256, 0, s>>>(sig_o, tab, V, L.nb, (unsigned)block_rows, bounds);
-        FGX_CHECK_LAUNCH("fgx_conv_wgrad(bounds)");
+        if (!given_bounds) {
+            block_bounds_kernel<<<cdiv((size_t)V * (L.nb + 1), 256), 256, 0, s>>>(sig_o, tab, V, L.nb, (unsigned)block_rows,
+                                                                                 (uint32_t*)((char*)scratch + L.bounds_off));
+            FGX_CHECK_LAUNCH("fgx_conv_wgrad(bounds)");
+        }
         const unsigned co_tiles = cdiv(Co, BM), ci_tiles = cdiv(Ci, BN);
         const size_t items = (size_t)L.nb * V * co_tiles * ci_tiles;
         FGX_CHECK_ARG(items < 0x7FFFFFFFull, "fgx_conv_wgrad: too many work items (%zu); use larger voxel blocks", items);
@@ -949,12 +958,12 @@ bool stream_ok(int tile_rows, int tile_cols, size_t n, size_t n_in, int Ci, int 
 
 template <typename Tag>
 int dispatch_wgrad_stream(int tile_rows, const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
-                          const SegTable& tab, const Layout& L, size_t n, size_t n_in, int V, int Ci, int Co, int block_rows,
+                          const uint32_t* given_bounds, const SegTable& tab, const Layout& L, size_t n, size_t n_in, int V, int Ci, int Co, int block_rows,
                           void* scratch, void* gw, hipStream_t s) {
     if constexpr (sizeof(typename Tag::type) == 2) {
-        if (tile_rows == 128) return launch_wgrad_stream<Tag, 128, 128>(gout, feats, sig_i, sig_o, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, s);
-        if (tile_rows == 64) return launch_wgrad_stream<Tag, 64, 64>(gout, feats, sig_i, sig_o, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, s);
-        return launch_wgrad_stream<Tag, 32, 32>(gout, feats, sig_i, sig_o, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, s);
+        if (tile_rows == 128) return launch_wgrad_stream<Tag, 128, 128>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, s);
+        if (tile_rows == 64) return launch_wgrad_stream<Tag, 64, 64>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, s);
+        return launch_wgrad_stream<Tag, 32, 32>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, s);
     } else {
         set_error("fgx_conv_wgrad: the streaming kernel handles 16-bit types only");
         return FGX_ERR_UNSUPPORTED;
@@ -963,11 +972,11 @@ int dispatch_wgrad_stream(int tile_rows, const void* gout, const void* feats, co
 
 template <typename Tag>
 int dispatch_wgrad(int tile_rows, int tile_cols, const void* gout, const void* feats, const uint32_t* sig_i,
-                   const uint32_t* sig_o, const SegTable& tab, const Layout& L, bool small, int V, int Ci, int Co,
+                   const uint32_t* sig_o, const uint32_t* given_bounds, const SegTable& tab, const Layout& L, bool small, int V, int Ci, int Co,
                    int block_rows, void* scratch, void* gw, hipStream_t s) {
 #define FGX_TILE(BM, BN, WMv, WNv)          \
     if (tile_rows == BM && tile_cols == BN) \
-        return launch_wgrad<Tag, BM, BN, WMv, WNv>(gout, feats, sig_i, sig_o, tab, L, small, V, Ci, Co, block_rows, scratch, gw, s);
+        return launch_wgrad<Tag, BM, BN, WMv, WNv>(gout, feats, sig_i, sig_o, given_bounds, tab, L, small, V, Ci, Co, block_rows, scratch, gw, s);
     FGX_TILE(128, 128, 2, 2)
     FGX_TILE(64, 64, 2, 2)
     FGX_TILE(32, 32, 1, 1)
@@ -989,9 +998,35 @@ size_t fgx_wgrad_scratch_bytes(size_t n, int V, int Ci, int Co, int block_rows) 
     return layout(n, V, Ci, Co, block_rows, (Ci < Co ? Ci : Co) <= 32 ? 4 : 1).total;
 }
 
+size_t fgx_wgrad_block_bounds_count(size_t n, int V, int block_rows) {
+    if (V < 1 || V > kMaxV || block_rows <= 0) return 0;
+    return (size_t)V * ((size_t)cdiv(n, (size_t)block_rows) + 1);
+}
+
+int fgx_wgrad_block_bounds(const uint32_t* sig_o, const uint32_t* seg_host, size_t n, int V, int block_rows,
+                           uint32_t* block_bounds, fgx_stream_t stream) {
+    FGX_CHECK_ARG(V >= 1 && V <= kMaxV, "fgx_wgrad_block_bounds: bad kernel volume %d", V);
+    FGX_CHECK_ARG(block_rows >= 1, "fgx_wgrad_block_bounds: block_rows must be positive, got %d", block_rows);
+    FGX_CHECK_ARG(seg_host && block_bounds, "fgx_wgrad_block_bounds: null buffer");
+    FGX_CHECK_ARG(n < 0xFFFFFFFFull, "fgx_wgrad_block_bounds: too many rows");
+    SegTable tab;
+    for (int v = 0; v <= V; ++v) {
+        FGX_CHECK_ARG(v == 0 || seg_host[v] >= seg_host[v - 1], "fgx_wgrad_block_bounds: segment table is not monotone");
+        tab.seg[v] = seg_host[v];
+    }
+    for (int v = V + 1; v <= kMaxV; ++v) tab.seg[v] = seg_host[V];
+    FGX_CHECK_ARG(seg_host[V] == seg_host[0] || sig_o != nullptr, "fgx_wgrad_block_bounds: null pair list");
+    const unsigned nb = cdiv(n, (size_t)block_rows);
+    block_bounds_kernel<<<cdiv((size_t)V * (nb + 1), 256), 256, 0, (hipStream_t)stream>>>(sig_o, tab, V, nb, (unsigned)block_rows,
+                                                                                         block_bounds);
+    FGX_CHECK_LAUNCH("fgx_wgrad_block_bounds");
+    return FGX_OK;
+}
+
 int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
-                   const uint32_t* seg_host, size_t n, size_t n_in, int Ci, int Co, int V, int tile_rows, int tile_cols,
-                   int block_rows, int streaming, void* scratch, void* grad_weight, fgx_stream_t stream) {
+                   const uint32_t* seg_host, const uint32_t* block_bounds, size_t n, size_t n_in, int Ci, int Co, int V,
+                   int tile_rows, int tile_cols, int block_rows, int streaming, void* scratch, void* grad_weight,
+                   fgx_stream_t stream) {
     FGX_CHECK_ARG(dtype_ok(dtype), "fgx_conv_wgrad: unknown dtype %d", dtype);
     FGX_CHECK_ARG(Ci > 0 && Co > 0 && V >= 1 && V <= kMaxV, "fgx_conv_wgrad: bad shape Ci=%d Co=%d V=%d", Ci, Co, V);
     FGX_CHECK_ARG(block_rows >= 1, "fgx_conv_wgrad: block_rows must be positive, got %d", block_rows);
@@ -1020,13 +1055,13 @@ int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uin
     hipStream_t s = (hipStream_t)stream;
     // (outside the streaming kernel's range the tiled kernel runs)
     if (stream_f16)
-        return dispatch_wgrad_stream<F16>(tile_rows, grad_out, feats, sig_i, sig_o, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, s);
+        return dispatch_wgrad_stream<F16>(tile_rows, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, s);
     if (stream_bf16)
-        return dispatch_wgrad_stream<BF16>(tile_rows, grad_out, feats, sig_i, sig_o, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, s);
+        return dispatch_wgrad_stream<BF16>(tile_rows, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, s);
     switch (dtype) {
-        case FGX_F16: return dispatch_wgrad<F16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);
-        case FGX_BF16: return dispatch_wgrad<BF16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);
-        default: return dispatch_wgrad<F32>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);
+        case FGX_F16: return dispatch_wgrad<F16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);
+        case FGX_BF16: return dispatch_wgrad<BF16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);
+        default: return dispatch_wgrad<F32>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);
     }
 }
 

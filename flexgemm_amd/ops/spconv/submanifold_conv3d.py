@@ -185,6 +185,23 @@ class SubMConv3dNeighborCache:
         self["valid_signal_i"], self["valid_signal_o"], self["valid_signal_seg"] = sig_i, sig_o, seg
         self["_valid_signal_seg_host"] = seg_host
 
+    def _wgrad_bounds(self, block_rows: int):
+        """First pair of every (offset, voxel block) for wgrad's blocks of `block_rows` rows: a function of the pair lists
+        alone, so it is made once per block size and kept."""
+        key = f"_wgrad_bounds_{block_rows}"
+        if not hasattr(self, key):
+            sig_o = self["valid_signal_o"]
+            n, v = self["neighbor_map"].shape
+            seg_host = self._seg_host()
+            L = nat.lib()
+            count = L.fgx_wgrad_block_bounds_count(nat.sz(n), C.c_int(v), C.c_int(block_rows))
+            bounds = torch.empty((max(int(count), 1),), dtype=torch.uint32, device=sig_o.device)
+            with torch.cuda.device(sig_o.device):
+                nat.check(L.fgx_wgrad_block_bounds(nat.ptr(sig_o), (C.c_uint32 * (v + 1))(*seg_host), nat.sz(n), C.c_int(v),
+                                                   C.c_int(block_rows), nat.ptr(bounds), nat.stream()))
+            setattr(self, key, bounds)
+        return getattr(self, key)
+
     def _seg_host(self):
         if not hasattr(self, "_valid_signal_seg_host"):
             seg = self["valid_signal_seg"]
@@ -392,13 +409,14 @@ def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int) -> tor
     gw = torch.empty((cop, v, cip), dtype=dt, device=dev)
     L = nat.lib()
     code = nat.DTYPE_CODE[dt]
+    bounds = cache._wgrad_bounds(sched.block_rows)
     with torch.cuda.device(dev):
         scratch = nat.workspace(L.fgx_wgrad_scratch_bytes(nat.sz(n), C.c_int(v), C.c_int(cip), C.c_int(cop),
                                                           C.c_int(sched.block_rows)), dev)
         nat.mark("wgrad", "start")
         nat.check(L.fgx_conv_wgrad(
             C.c_int(code), nat.ptr(g), nat.ptr(f), nat.ptr(cache["valid_signal_i"]), nat.ptr(cache["valid_signal_o"]),
-            seg_arr, nat.sz(n), nat.sz(n_in), C.c_int(cip), C.c_int(cop), C.c_int(v), C.c_int(sched.tile_rows), C.c_int(sched.tile_cols),
+            seg_arr, nat.ptr(bounds), nat.sz(n), nat.sz(n_in), C.c_int(cip), C.c_int(cop), C.c_int(v), C.c_int(sched.tile_rows), C.c_int(sched.tile_cols),
             C.c_int(sched.block_rows), C.c_int(sched.stream), nat.ptr(scratch), nat.ptr(gw), nat.stream()))
         nat.mark("wgrad", "stop")
     if cip != ci or cop != co:

@@ -234,12 +234,18 @@ int fgx_conv_gather_gemm_stream(int dtype, const void* src, const void* panel, c
  * adds them per offset in block order.  `streaming` != 0 asks for the persistent kernel with loader / multiplier
  * wavefronts (16-bit types, 128x128 or 64x64 tiles, operands below ~4 GB); outside that range the tiled kernel runs.
  * `n` = rows of grad_out (the range of sig_o), `n_in` = rows of feats (the range of sig_i); equal for the submanifold
- * convolution.
+ * convolution.  `block_bounds` (optional): the table fgx_wgrad_block_bounds makes from the same pair lists and
+ * block_rows -- block_bounds[v * (nb + 1) + b] = first pair of offset v whose grad_out row is >= b * block_rows,
+ * nb = ceil(n / block_rows) -- for callers that keep it with their neighbor cache; NULL = computed here, per call.
+ * The 32x32 streaming tile writes four partial products per block (the scratch size accounts for it).
  * Replaces: sparse_submanifold_conv_bwd_weight_masked_implicit_gemm[_splitk]
  *           (..._bwd_masked_implicit_gemm.py:99-170, ..._splitk.py:108-182, 278-317). */
 size_t fgx_wgrad_scratch_bytes(size_t n, int V, int Ci, int Co, int block_rows);
+size_t fgx_wgrad_block_bounds_count(size_t n, int V, int block_rows);
+int fgx_wgrad_block_bounds(const uint32_t* sig_o, const uint32_t* seg_host, size_t n, int V, int block_rows,
+                           uint32_t* block_bounds, fgx_stream_t stream);
 int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats,
-                   const uint32_t* sig_i, const uint32_t* sig_o, const uint32_t* seg_host,
+                   const uint32_t* sig_i, const uint32_t* sig_o, const uint32_t* seg_host, const uint32_t* block_bounds,
                    size_t n, size_t n_in, int Ci, int Co, int V, int tile_rows, int tile_cols, int block_rows,
                    int streaming, void* scratch, void* grad_weight, fgx_stream_t stream);
 

@@ -80,7 +80,7 @@ def test_argument_errors_map_to_exceptions(library):
         nat.check(L.fgx_subm_neighbor_map(None, 32, None, ctypes.c_size_t(0), None, ctypes.c_size_t(0), 4, 4, 4,
                                           2, 3, 3, 1, 1, 1, None, None, None, None))
     with pytest.raises(ValueError):
-        nat.check(L.fgx_conv_wgrad(0, None, None, None, None, None, ctypes.c_size_t(0), ctypes.c_size_t(0), 8, 8, 27, 128, 128, 0, 0,
+        nat.check(L.fgx_conv_wgrad(0, None, None, None, None, None, None, ctypes.c_size_t(0), ctypes.c_size_t(0), 8, 8, 27, 128, 128, 0, 0,
                                    None, None, None))
     with pytest.raises(ValueError):   # the streaming GEMM checks its arguments before touching the device
         nat.check(L.fgx_conv_gather_gemm_stream(0, None, None, None, None, None, None, None, None, ctypes.c_size_t(0),
