@@ -34,9 +34,7 @@ constexpr int kPlanSlots = 4;        // index ring depth
 constexpr int kPlanAhead = 3;        // the index stream runs this many offsets ahead of the row stream
 constexpr uint32_t kOobOffset = 0xFF000000u;   // buffer offset no source tensor reaches: the load returns zeros
 constexpr int kBandSlots = 8;        // band-mask ring depth: a mask is read up to (stages - 2) steps after it was written
-#ifndef FGX_EXP_SHORT_STAGES
-#define FGX_EXP_SHORT_STAGES 3
-#endif
+constexpr int kStreamStages = 3;     // ring stages (for the short-row tiles 4, 5 and 7 measured the same)
 constexpr int kLoaders = 4;          // loader wavefronts per workgroup (one per SIMD)
 
 using rsrc_t = __amdgpu_buffer_rsrc_t;
@@ -48,7 +46,7 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint32_t bytes) {
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int CH>
 struct StreamCfg {
     using T = typename Tag::type;
-    static constexpr int S = CH == 4 ? FGX_EXP_SHORT_STAGES : 3;   // ring stages
+    static constexpr int S = kStreamStages;
     static constexpr int ES = (int)sizeof(T);
     static constexpr int NW = WAVES_M * WAVES_N;               // multiplying wavefronts
     static constexpr int NL = kLoaders;
@@ -77,6 +75,7 @@ struct StreamCfg {
     static_assert(NW * OUT_BAND_BYTES <= STAGE_BYTES, "the output bands must fit one ring stage");
     static_assert(LPS + 1 < 64, "vmcnt is a 6-bit counter");
     static_assert(CH == 4 || CH == 8, "slab must be 64 or 128 bytes");
+    // (the loaders' wait -- "all but the last iteration's loads have landed" -- is what fixes S at 3 or more)
     static_assert(S >= 3 && S - 1 < kBandSlots, "a band mask must outlive the S - 2 steps between its writing and its reading");
     static constexpr size_t fixed_lds = (size_t)S * STAGE_BYTES + (size_t)kPlanSlots * IDX_SLOT_BYTES + OROW_BYTES + kBandSlots * 4;
 };
