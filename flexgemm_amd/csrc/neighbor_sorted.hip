@@ -129,83 +129,90 @@ __global__ void __launch_bounds__(kGroup) merge_neighbor_kernel(const K* __restr
     }
     __syncthreads();
 
-    // The window of row r + 1 travels from memory to registers while row r is searched in LDS.
-    K pk[kPer];
-    uint32_t pr[kPer];
-    auto fetch = [&](int r) {
-        if (r >= R) return;
-        const size_t lo = win_lo[r], hi = win_hi[r];
-        const size_t w = hi > lo ? hi - lo : 0;
-        if (w > (size_t)kWindow) return;            // searched in place
-#pragma unroll
-        for (int i = 0; i < kPer; ++i) {
-            const size_t j = (size_t)tid + (size_t)i * kGroup;
-            if (j < w) {
-                pk[i] = skeys[lo + j];
-                pr[i] = srows[lo + j];
-            }
-        }
-    };
-    fetch(0);
+    // The windows of the next kAhead (dx, dy) rows travel from memory to registers together, so their latencies overlap;
+    // each is then put into LDS and searched in turn.
+    constexpr int kAhead = 9;
+    K pk[kAhead][kPer];
+    uint32_t pr[kAhead][kPer];
     uint32_t mask = 0;
-    for (int r = 0; r < R; ++r) {
-        const size_t lo = win_lo[r], hi = win_hi[r];
-        const size_t w = hi > lo ? hi - lo : 0;
-        const bool staged = w <= (size_t)kWindow;
-        if (staged) {
+    for (int r0 = 0; r0 < R; r0 += kAhead) {
+#pragma unroll
+        for (int a = 0; a < kAhead; ++a) {
+            const int r = r0 + a;
+            if (r >= R) break;
+            const size_t lo = win_lo[r], hi = win_hi[r];
+            const size_t w = hi > lo ? hi - lo : 0;
+            if (w > (size_t)kWindow) continue;          // searched in place
 #pragma unroll
             for (int i = 0; i < kPer; ++i) {
                 const size_t j = (size_t)tid + (size_t)i * kGroup;
                 if (j < w) {
-                    wkeys[j] = pk[i];
-                    wrows[j] = pr[i];
+                    pk[a][i] = skeys[lo + j];
+                    pr[a][i] = srows[lo + j];
                 }
             }
         }
-        __syncthreads();
-        fetch(r + 1);
-        if (live) {
-            const int kx = r / g.Kh, ky = r % g.Kh;
-            const int x2 = x + (kx - g.Kw / 2) * g.Dw, y2 = y + (ky - g.Kh / 2) * g.Dh;
-            const bool row_in = x2 >= 0 && x2 < g.W && y2 >= 0 && y2 < g.H;
-            const long long off = (long long)(kx - g.Kw / 2) * g.Dw * HD + (long long)(ky - g.Kh / 2) * g.Dh * g.D;
-            uint32_t* out_row = stage_out ? out_rows + tid * (kStageV + 1) + r * g.Kd
-                                          : out_map + (size_t)me * g.V + (size_t)r * g.Kd;
-            // the Kd targets of a row ascend by Dd: one binary search for the first, then a short walk to each next one
-            unsigned pos = 0;
-            bool searched = false;
-            const unsigned wn = (unsigned)w;
-            for (int kz = 0; kz < g.Kd; ++kz) {
-                const int dz = (kz - g.Kd / 2) * g.Dd;
-                const int z2 = z + dz;
-                uint32_t value = FGX_EMPTY32;
-                if (row_in && z2 >= 0 && z2 < g.D && w > 0) {
-                    const K target = (K)((long long)key + off + dz);
-                    if (staged) {
-                        if (!searched) {
-                            unsigned a = 0, b = wn;
-                            while (a < b) {
-                                const unsigned mid = (a + b) >> 1;
-                                if (wkeys[mid] < target) a = mid + 1;
-                                else b = mid;
-                            }
-                            pos = a;
-                            searched = true;
-                        } else {
-                            while (pos < wn && wkeys[pos] < target) ++pos;
-                        }
-                        if (pos < wn && wkeys[pos] == target) value = wrows[pos];
-                    } else {
-                        const size_t q = lower_bound_at<K>(skeys, lo, hi, target);
-                        if (q < hi && skeys[q] == target) value = srows[q];
+#pragma unroll
+        for (int a = 0; a < kAhead; ++a) {
+            const int r = r0 + a;
+            if (r >= R) break;
+            const size_t lo = win_lo[r], hi = win_hi[r];
+            const size_t w = hi > lo ? hi - lo : 0;
+            const bool staged = w <= (size_t)kWindow;
+            if (staged) {
+#pragma unroll
+                for (int i = 0; i < kPer; ++i) {
+                    const size_t j = (size_t)tid + (size_t)i * kGroup;
+                    if (j < w) {
+                        wkeys[j] = pk[a][i];
+                        wrows[j] = pr[a][i];
                     }
                 }
-                out_row[kz] = value;
-                const int v = r * g.Kd + kz;
-                if (v < 32 && value != FGX_EMPTY32) mask |= 1u << v;
             }
+            __syncthreads();
+            if (live) {
+                const int kx = r / g.Kh, ky = r % g.Kh;
+                const int x2 = x + (kx - g.Kw / 2) * g.Dw, y2 = y + (ky - g.Kh / 2) * g.Dh;
+                const bool row_in = x2 >= 0 && x2 < g.W && y2 >= 0 && y2 < g.H;
+                const long long off = (long long)(kx - g.Kw / 2) * g.Dw * HD + (long long)(ky - g.Kh / 2) * g.Dh * g.D;
+                uint32_t* out_row = stage_out ? out_rows + tid * (kStageV + 1) + r * g.Kd
+                                              : out_map + (size_t)me * g.V + (size_t)r * g.Kd;
+                // the Kd targets of a row ascend by Dd: one binary search for the first, then a short walk to each next one
+                unsigned pos = 0;
+                bool searched = false;
+                const unsigned wn = (unsigned)w;
+                for (int kz = 0; kz < g.Kd; ++kz) {
+                    const int dz = (kz - g.Kd / 2) * g.Dd;
+                    const int z2 = z + dz;
+                    uint32_t value = FGX_EMPTY32;
+                    if (row_in && z2 >= 0 && z2 < g.D && w > 0) {
+                        const K target = (K)((long long)key + off + dz);
+                        if (staged) {
+                            if (!searched) {
+                                unsigned a = 0, b = wn;
+                                while (a < b) {
+                                    const unsigned mid = (a + b) >> 1;
+                                    if (wkeys[mid] < target) a = mid + 1;
+                                    else b = mid;
+                                }
+                                pos = a;
+                                searched = true;
+                            } else {
+                                while (pos < wn && wkeys[pos] < target) ++pos;
+                            }
+                            if (pos < wn && wkeys[pos] == target) value = wrows[pos];
+                        } else {
+                            const size_t q = lower_bound_at<K>(skeys, lo, hi, target);
+                            if (q < hi && skeys[q] == target) value = srows[q];
+                        }
+                    }
+                    out_row[kz] = value;
+                    const int v = r * g.Kd + kz;
+                    if (v < 32 && value != FGX_EMPTY32) mask |= 1u << v;
+                }
+            }
+            __syncthreads();       // the window is overwritten by the next row
         }
-        __syncthreads();       // the window is overwritten by the next row
     }
     if (live && gray != nullptr) {
         gray[me] = (int32_t)mask;
