@@ -35,6 +35,7 @@ EXPORTS = [
     "fgx_colsum_scratch_bytes", "fgx_colsum",
     "fgx_spconv_out_dims", "fgx_spconv_out_coords_workspace_bytes", "fgx_spconv_out_coords_keys",
     "fgx_spconv_out_coords_decode", "fgx_spconv_neighbor_map",
+    "fgx_spconv_neighbor_map_sorted_workspace_bytes", "fgx_spconv_neighbor_map_sorted",
 ]
 
 
@@ -74,7 +75,8 @@ def lib() -> C.CDLL:
         for name in ("fgx_sort_workspace_bytes", "fgx_locality_workspace_bytes", "fgx_pair_workspace_bytes", "fgx_tile_workspace_bytes",
                      "fgx_weight_panel_bytes", "fgx_conv_scratch_bytes", "fgx_wgrad_scratch_bytes",
                      "fgx_colsum_scratch_bytes", "fgx_spconv_out_coords_workspace_bytes",
-                     "fgx_subm_neighbor_map_sorted_workspace_bytes", "fgx_wgrad_block_bounds_count"):
+                     "fgx_subm_neighbor_map_sorted_workspace_bytes", "fgx_wgrad_block_bounds_count",
+                     "fgx_spconv_neighbor_map_sorted_workspace_bytes"):
             getattr(L, name).restype = C.c_size_t
         _lib = L
     return _lib

@@ -292,6 +292,274 @@ int build_sorted(const int32_t* coords, size_t n, uint64_t vol, const SubmGeom& 
     return FGX_OK;
 }
 
+// ------------------------------------------------------------------------------------------------
+// Generic sparse convolution: the same search with the OUTPUT voxels as queries.
+//
+// Output voxel o = (b, x, y, z) reads the input voxel at (x*Sw - Pw + kx*Dw, ...): for a fixed kernel position that is its
+// "base" cell (x*Sw - Pw, y*Sh - Ph, z*Sd - Pd) plus a constant, and in flattened input keys base(o) + constant, even when
+// the base cell itself lies outside the grid (the sum is linear).  So the queries are sorted by base(o) (biased to be
+// non-negative), and a group of 256 consecutive ones again finds all its (kx, ky) neighbors in one window of the sorted
+// input keys.  A query that cannot reach the grid at all (any base coordinate further out than the kernel spans, or a
+// batch index outside [0, B)) gets the largest key and an all-empty row.
+// ------------------------------------------------------------------------------------------------
+struct ConvGeomS {
+    int B, W, H, D;
+    int Kw, Kh, Kd, V;
+    int Sw, Sh, Sd;
+    int Pw, Ph, Pd;
+    int Dw, Dh, Dd;
+};
+
+__device__ __forceinline__ bool query_base(const int4 c, const ConvGeomS& g, int& xi, int& yi, int& zi, long long& base) {
+    xi = c.y * g.Sw - g.Pw;
+    yi = c.z * g.Sh - g.Ph;
+    zi = c.w * g.Sd - g.Pd;
+    base = (((long long)c.x * g.W + xi) * g.H + yi) * g.D + zi;
+    return c.x >= 0 && c.x < g.B && xi > -g.Kw * g.Dw && xi < g.W && yi > -g.Kh * g.Dh && yi < g.H && zi > -g.Kd * g.Dd && zi < g.D;
+}
+
+__global__ void __launch_bounds__(256) query_keys_kernel(const int32_t* __restrict__ out_coords, size_t n_out, ConvGeomS g,
+                                                         unsigned long long bias, unsigned long long dead_key,
+                                                         uint64_t* __restrict__ keys, uint32_t* __restrict__ rows) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n_out) return;
+    int xi, yi, zi;
+    long long base;
+    const bool live = query_base(reinterpret_cast<const int4*>(out_coords)[i], g, xi, yi, zi, base);
+    keys[i] = live ? (uint64_t)(base + (long long)bias) : (uint64_t)dead_key;
+    rows[i] = (uint32_t)i;
+}
+
+// as window_bounds_kernel, with the group's range taken from the sorted query keys (dead queries, at the end, excluded)
+template <typename K>
+__global__ void __launch_bounds__(256) query_bounds_kernel(const K* __restrict__ skeys, size_t n_in, unsigned long long vol,
+                                                           const uint64_t* __restrict__ qkeys, size_t n_out,
+                                                           unsigned long long bias, unsigned long long dead_key, ConvGeomS g,
+                                                           unsigned groups, uint32_t* __restrict__ bounds) {
+    const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const int R = g.Kw * g.Kh;
+    if (t >= (size_t)groups * R * 2) return;
+    const size_t grp = t / (2 * R);
+    const int r = (int)(t % (2 * R)) >> 1;
+    const size_t p0 = grp * kGroup;
+    size_t p1 = (n_out - p0 < (size_t)kGroup ? n_out : p0 + kGroup) - 1;      // last query of the group
+    uint32_t pos = 0;
+    if (qkeys[p0] != dead_key) {
+        // the last live query of the group (dead keys are the largest)
+        if (qkeys[p1] == dead_key) p1 = lower_bound_at<uint64_t>(qkeys, p0, p1, dead_key) - 1;
+        const long long HD = (long long)g.H * g.D;
+        const long long off = (long long)(r / g.Kh) * g.Dw * HD + (long long)(r % g.Kh) * g.Dh * g.D;
+        const long long lo_t = (long long)(qkeys[p0] - bias) + off, hi_t = (long long)(qkeys[p1] - bias) + off + (long long)(g.Kd - 1) * g.Dd;
+        if ((t & 1) == 0) pos = (uint32_t)(hi_t < 0 ? 0 : (lo_t >= (long long)vol ? n_in : lower_bound_at<K>(skeys, 0, n_in, (K)(lo_t < 0 ? 0 : lo_t))));
+        else pos = (uint32_t)(hi_t < 0 ? 0 : (hi_t + 1 >= (long long)vol ? n_in : lower_bound_at<K>(skeys, 0, n_in, (K)(hi_t + 1))));
+    }
+    bounds[t] = pos;
+}
+
+template <typename K>
+__global__ void __launch_bounds__(kGroup) merge_query_kernel(const K* __restrict__ skeys, const uint32_t* __restrict__ srows,
+                                                             const uint64_t* __restrict__ qkeys, const uint32_t* __restrict__ qrows,
+                                                             const int32_t* __restrict__ out_coords, const uint32_t* __restrict__ bounds,
+                                                             size_t n_out, unsigned long long dead_key, ConvGeomS g,
+                                                             uint32_t* __restrict__ map_fwd, uint32_t* __restrict__ map_bwd,
+                                                             int32_t* __restrict__ gray, int32_t* __restrict__ binary) {
+    constexpr int kPer = kWindow / kGroup;
+    __shared__ K wkeys[kWindow];
+    __shared__ uint32_t wrows[kWindow];
+    __shared__ uint32_t win_lo[kMaxRows], win_hi[kMaxRows];
+    __shared__ uint32_t out_rows[kGroup * (kStageV + 1)];
+    __shared__ uint32_t out_dst[kGroup];
+    const bool stage_out = g.V <= kStageV;
+    const size_t p0 = (size_t)blockIdx.x * kGroup;
+    const int cnt = (int)(n_out - p0 < (size_t)kGroup ? n_out - p0 : (size_t)kGroup);
+    const int tid = threadIdx.x;
+    const bool present = tid < cnt;
+    const int R = g.Kw * g.Kh;
+    const long long HD = (long long)g.H * g.D;
+    for (int j = tid; j < R; j += kGroup) {
+        win_lo[j] = bounds[((size_t)blockIdx.x * R + j) * 2];
+        win_hi[j] = bounds[((size_t)blockIdx.x * R + j) * 2 + 1];
+    }
+    uint32_t me = 0;
+    int xi = 0, yi = 0, zi = 0;
+    long long base = 0;
+    bool live = false;
+    if (present) {
+        me = qrows[p0 + tid];
+        live = qkeys[p0 + tid] != dead_key;
+        bool ok = query_base(reinterpret_cast<const int4*>(out_coords)[me], g, xi, yi, zi, base);
+        live = live && ok;
+    }
+    __syncthreads();
+
+    constexpr int kAhead = 9;
+    K pk[kAhead][kPer];
+    uint32_t pr[kAhead][kPer];
+    uint32_t mask = 0;
+    for (int r0 = 0; r0 < R; r0 += kAhead) {
+#pragma unroll
+        for (int a = 0; a < kAhead; ++a) {
+            const int r = r0 + a;
+            if (r >= R) break;
+            const size_t lo = win_lo[r], hi = win_hi[r];
+            const size_t w = hi > lo ? hi - lo : 0;
+            if (w > (size_t)kWindow) continue;
+#pragma unroll
+            for (int i = 0; i < kPer; ++i) {
+                const size_t j = (size_t)tid + (size_t)i * kGroup;
+                if (j < w) {
+                    pk[a][i] = skeys[lo + j];
+                    pr[a][i] = srows[lo + j];
+                }
+            }
+        }
+#pragma unroll
+        for (int a = 0; a < kAhead; ++a) {
+            const int r = r0 + a;
+            if (r >= R) break;
+            const size_t lo = win_lo[r], hi = win_hi[r];
+            const size_t w = hi > lo ? hi - lo : 0;
+            const bool staged = w <= (size_t)kWindow;
+            if (staged) {
+#pragma unroll
+                for (int i = 0; i < kPer; ++i) {
+                    const size_t j = (size_t)tid + (size_t)i * kGroup;
+                    if (j < w) {
+                        wkeys[j] = pk[a][i];
+                        wrows[j] = pr[a][i];
+                    }
+                }
+            }
+            __syncthreads();
+            if (present) {
+                const int kx = r / g.Kh, ky = r % g.Kh;
+                const int x2 = xi + kx * g.Dw, y2 = yi + ky * g.Dh;
+                const bool row_in = live && x2 >= 0 && x2 < g.W && y2 >= 0 && y2 < g.H;
+                const long long off = (long long)kx * g.Dw * HD + (long long)ky * g.Dh * g.D;
+                uint32_t* out_row = stage_out ? out_rows + tid * (kStageV + 1) + r * g.Kd
+                                              : map_fwd + (size_t)me * g.V + (size_t)r * g.Kd;
+                unsigned pos = 0;
+                bool searched = false;
+                const unsigned wn = (unsigned)w;
+                for (int kz = 0; kz < g.Kd; ++kz) {
+                    const int z2 = zi + kz * g.Dd;
+                    uint32_t value = FGX_EMPTY32;
+                    if (row_in && z2 >= 0 && z2 < g.D && w > 0) {
+                        const K target = (K)(base + off + (long long)kz * g.Dd);
+                        if (staged) {
+                            if (!searched) {
+                                unsigned a2 = 0, b2 = wn;
+                                while (a2 < b2) {
+                                    const unsigned mid = (a2 + b2) >> 1;
+                                    if (wkeys[mid] < target) a2 = mid + 1;
+                                    else b2 = mid;
+                                }
+                                pos = a2;
+                                searched = true;
+                            } else {
+                                while (pos < wn && wkeys[pos] < target) ++pos;
+                            }
+                            if (pos < wn && wkeys[pos] == target) value = wrows[pos];
+                        } else {
+                            const size_t q = lower_bound_at<K>(skeys, lo, hi, target);
+                            if (q < hi && skeys[q] == target) value = srows[q];
+                        }
+                    }
+                    out_row[kz] = value;
+                    const int v = r * g.Kd + kz;
+                    if (value != FGX_EMPTY32) {
+                        if (v < 32) mask |= 1u << v;
+                        if (map_bwd != nullptr) map_bwd[(size_t)value * g.V + v] = me;
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    }
+    if (present && gray != nullptr) {
+        gray[me] = (int32_t)mask;
+        binary[me] = (int32_t)gray_decode(mask);
+    }
+    if (stage_out) {
+        out_dst[tid] = me;
+        __syncthreads();
+        const int lane32 = tid & 31;
+        for (int row = tid >> 5; row < cnt; row += kGroup / 32)
+            if (lane32 < g.V) map_fwd[(size_t)out_dst[row] * g.V + lane32] = out_rows[row * (kStageV + 1) + lane32];
+    }
+}
+
+__global__ void __launch_bounds__(256) fill_words_kernel(uint32_t* p, size_t count, uint32_t value) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (; i < count; i += stride) p[i] = value;
+}
+
+struct QueryLayout {
+    SortedLayout in;            // the input voxels' sort (bounds sized for the query groups)
+    size_t qkeys_in, qkeys_out, qrows_in, qrows_out, qtemp, qtemp_bytes, total;
+};
+
+QueryLayout query_layout(size_t n_in, size_t n_out, int key_bits, int rows_xy) {
+    QueryLayout Q{};
+    Q.in = sorted_layout(n_in, key_bits, 0);
+    size_t off = Q.in.total;
+    const size_t nq = n_out ? n_out : 1;
+    Q.qkeys_in = off;
+    off = align_up(off + nq * 8, 256);
+    Q.qkeys_out = off;
+    off = align_up(off + nq * 8, 256);
+    Q.qrows_in = off;
+    off = align_up(off + nq * 4, 256);
+    Q.qrows_out = off;
+    off = align_up(off + nq * 4, 256);
+    Q.in.bounds = off;
+    off = align_up(off + (size_t)cdiv(nq, kGroup) * rows_xy * 2 * sizeof(uint32_t), 256);
+    Q.qtemp = off;
+    Q.qtemp_bytes = pair_sort_temp_bytes<uint64_t>(n_out);
+    Q.total = off + align_up(Q.qtemp_bytes, 256);
+    return Q;
+}
+
+template <typename K>
+int build_query_sorted(const int32_t* in_coords, size_t n_in, const int32_t* out_coords, size_t n_out, uint64_t vol,
+                       const ConvGeomS& g, char* ws, const QueryLayout& Q, uint32_t* map_fwd, uint32_t* map_bwd, int32_t* gray,
+                       int32_t* binary, hipStream_t s) {
+    K* keys_in = (K*)(ws + Q.in.keys_in);
+    K* keys_out = (K*)(ws + Q.in.keys_out);
+    uint32_t* rows_in = (uint32_t*)(ws + Q.in.rows_in);
+    uint32_t* rows_out = (uint32_t*)(ws + Q.in.rows_out);
+    flat_keys_kernel<K><<<cdiv(n_in, 256), 256, 0, s>>>(in_coords, n_in, g.W, g.H, g.D, keys_in, rows_in);
+    FGX_CHECK_LAUNCH("fgx_spconv_neighbor_map_sorted(keys)");
+    size_t temp_bytes = Q.in.temp_bytes;
+    unsigned end_bit = bit_length(vol - 1);
+    if (end_bit == 0) end_bit = 1;
+    FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + Q.in.temp, temp_bytes, (const K*)keys_in, keys_out, (const uint32_t*)rows_in, rows_out,
+                                            n_in, 0u, end_bit, s));
+    // queries: base keys biased by the furthest a live base cell can lie below the grid origin
+    const long long HD = (long long)g.H * g.D;
+    const unsigned long long bias = (unsigned long long)((long long)g.Kw * g.Dw * HD + (long long)g.Kh * g.Dh * g.D + (long long)g.Kd * g.Dd);
+    const unsigned long long dead_key = vol + 2 * bias + 1;
+    uint64_t* qkeys_in = (uint64_t*)(ws + Q.qkeys_in);
+    uint64_t* qkeys_out = (uint64_t*)(ws + Q.qkeys_out);
+    uint32_t* qrows_in = (uint32_t*)(ws + Q.qrows_in);
+    uint32_t* qrows_out = (uint32_t*)(ws + Q.qrows_out);
+    query_keys_kernel<<<cdiv(n_out, 256), 256, 0, s>>>(out_coords, n_out, g, bias, dead_key, qkeys_in, qrows_in);
+    FGX_CHECK_LAUNCH("fgx_spconv_neighbor_map_sorted(query keys)");
+    temp_bytes = Q.qtemp_bytes;
+    FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + Q.qtemp, temp_bytes, (const uint64_t*)qkeys_in, qkeys_out, (const uint32_t*)qrows_in,
+                                            qrows_out, n_out, 0u, bit_length(dead_key), s));
+    const unsigned groups = cdiv(n_out, kGroup);
+    uint32_t* bounds = (uint32_t*)(ws + Q.in.bounds);
+    query_bounds_kernel<K><<<cdiv((size_t)groups * g.Kw * g.Kh * 2, 256), 256, 0, s>>>(keys_out, n_in, (unsigned long long)vol, qkeys_out,
+                                                                                      n_out, bias, dead_key, g, groups, bounds);
+    FGX_CHECK_LAUNCH("fgx_spconv_neighbor_map_sorted(bounds)");
+    merge_query_kernel<K><<<groups, kGroup, 0, s>>>(keys_out, rows_out, qkeys_out, qrows_out, out_coords, bounds, n_out, dead_key, g,
+                                                    map_fwd, map_bwd, gray, binary);
+    FGX_CHECK_LAUNCH("fgx_spconv_neighbor_map_sorted");
+    return FGX_OK;
+}
+
 }  // namespace
 }  // namespace fgx
 
@@ -332,6 +600,61 @@ int fgx_subm_neighbor_map_sorted(const int32_t* coords, size_t n, int B, int W, 
     char* ws = (char*)workspace;
     return key_bits == 32 ? build_sorted<uint32_t>(coords, n, vol, g, ws, L, out_map, gray, binary, s)
                           : build_sorted<uint64_t>(coords, n, vol, g, ws, L, out_map, gray, binary, s);
+}
+
+size_t fgx_spconv_neighbor_map_sorted_workspace_bytes(size_t n_in, size_t n_out, int key_bits, int Kw, int Kh) {
+    if ((key_bits != 32 && key_bits != 64) || Kw < 1 || Kh < 1 || Kw * Kh > kMaxRows) return 0;
+    return query_layout(n_in, n_out, key_bits, Kw * Kh).total;
+}
+
+int fgx_spconv_neighbor_map_sorted(const int32_t* in_coords, size_t n_in, const int32_t* out_coords, size_t n_out, int B, int W,
+                                   int H, int D, int Kw, int Kh, int Kd, int Sw, int Sh, int Sd, int Pw, int Ph, int Pd, int Dw,
+                                   int Dh, int Dd, int key_bits, void* workspace, size_t workspace_bytes, uint32_t* map_fwd,
+                                   uint32_t* map_bwd, int32_t* gray, int32_t* binary, fgx_stream_t stream) {
+    FGX_CHECK_ARG(key_bits == 32 || key_bits == 64, "fgx_spconv_neighbor_map_sorted: key_bits must be 32 or 64, got %d", key_bits);
+    FGX_CHECK_ARG(B > 0 && W > 0 && H > 0 && D > 0, "fgx_spconv_neighbor_map_sorted: grid extents must be positive");
+    FGX_CHECK_ARG(Kw > 0 && Kh > 0 && Kd > 0 && Sw > 0 && Sh > 0 && Sd > 0 && Dw > 0 && Dh > 0 && Dd > 0 && Pw >= 0 && Ph >= 0 && Pd >= 0,
+                  "fgx_spconv_neighbor_map_sorted: bad kernel geometry");
+    FGX_CHECK_ARG(Kw * Kh <= kMaxRows && (long long)Kw * Kh * Kd <= 1 << 20, "fgx_spconv_neighbor_map_sorted: kernel too large");
+    const int V = Kw * Kh * Kd;
+    FGX_CHECK_ARG((gray == nullptr) == (binary == nullptr), "fgx_spconv_neighbor_map_sorted: gray and binary go together");
+    FGX_CHECK_ARG(gray == nullptr || V <= 32, "fgx_spconv_neighbor_map_sorted: mask codes need a kernel volume <= 32, got %d", V);
+    FGX_CHECK_ARG(n_in < 0xFFFFFFFFull && n_out < 0xFFFFFFFFull, "fgx_spconv_neighbor_map_sorted: row indices must fit below 2^32-1");
+    const long double vol_ld = (long double)B * W * H * D;
+    FGX_CHECK_ARG(vol_ld <= (key_bits == 32 ? 4294967296.0L : 4611686018427387904.0L),
+                  "fgx_spconv_neighbor_map_sorted: the grid needs wider keys than %d bits", key_bits);
+    hipStream_t s = (hipStream_t)stream;
+    if (map_bwd != nullptr && n_in > 0) {
+        const size_t cells = n_in * (size_t)V;
+        unsigned grid = cdiv(cells, 256);
+        if (grid > 65536u) grid = 65536u;
+        fill_words_kernel<<<grid, 256, 0, s>>>(map_bwd, cells, FGX_EMPTY32);
+        FGX_CHECK_LAUNCH("fgx_spconv_neighbor_map_sorted(fill)");
+    }
+    if (n_out == 0) return FGX_OK;
+    FGX_CHECK_ARG(out_coords && map_fwd, "fgx_spconv_neighbor_map_sorted: null buffer");
+    FGX_CHECK_ARG(((uintptr_t)out_coords & 15) == 0 && ((uintptr_t)in_coords & 15) == 0, "fgx_spconv_neighbor_map_sorted: coords must be 16-byte aligned");
+    if (n_in == 0) {
+        const size_t cells = n_out * (size_t)V;
+        unsigned grid = cdiv(cells, 256);
+        if (grid > 65536u) grid = 65536u;
+        fill_words_kernel<<<grid, 256, 0, s>>>(map_fwd, cells, FGX_EMPTY32);
+        if (gray != nullptr) {
+            fill_words_kernel<<<cdiv(n_out, 256), 256, 0, s>>>((uint32_t*)gray, n_out, 0u);
+            fill_words_kernel<<<cdiv(n_out, 256), 256, 0, s>>>((uint32_t*)binary, n_out, 0u);
+        }
+        FGX_CHECK_LAUNCH("fgx_spconv_neighbor_map_sorted(fill)");
+        return FGX_OK;
+    }
+    FGX_CHECK_ARG(in_coords && workspace, "fgx_spconv_neighbor_map_sorted: null buffer");
+    QueryLayout Q = query_layout(n_in, n_out, key_bits, Kw * Kh);
+    FGX_CHECK_ARG(workspace_bytes >= Q.total, "fgx_spconv_neighbor_map_sorted: workspace of %zu bytes, need %zu", workspace_bytes, Q.total);
+    FGX_CHECK_ARG(((uintptr_t)workspace & 255) == 0, "fgx_spconv_neighbor_map_sorted: workspace must be 256-byte aligned");
+    const uint64_t vol = (uint64_t)B * (uint64_t)W * (uint64_t)H * (uint64_t)D;
+    ConvGeomS g{B, W, H, D, Kw, Kh, Kd, V, Sw, Sh, Sd, Pw, Ph, Pd, Dw, Dh, Dd};
+    char* ws = (char*)workspace;
+    return key_bits == 32 ? build_query_sorted<uint32_t>(in_coords, n_in, out_coords, n_out, vol, g, ws, Q, map_fwd, map_bwd, gray, binary, s)
+                          : build_query_sorted<uint64_t>(in_coords, n_in, out_coords, n_out, vol, g, ws, Q, map_fwd, map_bwd, gray, binary, s);
 }
 
 }  // extern "C"

@@ -41,9 +41,10 @@ SERIALIZATION_MODE = SerializationMode.BXYZ
 
 # How the submanifold neighbor map is found (no counterpart in the reference, which always hashes; the map is the same
 # either way): "hash" = open-addressing table and probes, "sort" = radix sort of the flattened keys and windowed merges,
-# "auto" = "sort" from SORT_BUILDER_MIN_VOXELS voxels on.
+# "auto" = "sort" once the searches outweigh the two sorts: from SORT_BUILDER_MIN_PROBES (voxel, kernel position)
+# questions on (131 072 voxels of a 3x3x3 kernel).
 NEIGHBOR_MAP_BUILDER = "auto"
-SORT_BUILDER_MIN_VOXELS = 32768
+SORT_BUILDER_MIN_PROBES = 27 * 131072
 
 
 def set_neighbor_map_builder(builder: str):

@@ -79,21 +79,40 @@ class SparseConv3dNeighborCache(SubMConv3dNeighborCache):
 
 def _build_maps(coords: torch.Tensor, out_coords: torch.Tensor, shape, kernel_size, stride, padding, dilation,
                 with_bwd: bool, with_codes: bool):
-    """(map_fwd [L, V], map_bwd [M, V] | None, gray | None, binary | None) from a hash table of the input voxels."""
+    """(map_fwd [L, V], map_bwd [M, V] | None, gray | None, binary | None), by hash probes or by sort and merge."""
     m, l = coords.shape[0], out_coords.shape[0]
     _, _, W, H, D = [int(s) for s in shape]
     kw, kh, kd = kernel_size
     v = kw * kh * kd
     dev = coords.device
-    table = int(spconv.HASHMAP_RATIO * m)
-    if m > 0 and table < m:
-        raise ValueError(f"hashmap ratio {spconv.HASHMAP_RATIO} gives a table smaller than the input")
     nmap = torch.empty((l, v), dtype=torch.uint32, device=dev)
     nmap_bwd = torch.empty((m, v), dtype=torch.uint32, device=dev) if with_bwd else None
     gray = binary = None
     if with_codes:
         gray = torch.empty((l,), dtype=torch.int32, device=dev)
         binary = torch.empty((l,), dtype=torch.int32, device=dev)
+    B = int(shape[0])
+    builder = spconv.NEIGHBOR_MAP_BUILDER
+    if builder == "auto":
+        # (the generic builder sorts the queries as well, with wider keys: it needs more questions to pay off)
+        builder = "sort" if l * v >= 4 * spconv.SORT_BUILDER_MIN_PROBES else "hash"
+    vol = B * W * H * D
+    geom = [C.c_int(x) for x in (kw, kh, kd, stride[0], stride[1], stride[2], padding[0], padding[1], padding[2],
+                                 dilation[0], dilation[1], dilation[2])]
+    if builder == "sort" and kw * kh <= 128 and vol <= 2 ** 62:
+        key_bits = 32 if vol <= 2 ** 32 else 64
+        with torch.cuda.device(dev):
+            L = nat.lib()
+            ws = nat.workspace(L.fgx_spconv_neighbor_map_sorted_workspace_bytes(nat.sz(m), nat.sz(l), C.c_int(key_bits),
+                                                                                 C.c_int(kw), C.c_int(kh)), dev)
+            nat.check(L.fgx_spconv_neighbor_map_sorted(
+                nat.ptr(coords), nat.sz(m), nat.ptr(out_coords), nat.sz(l), C.c_int(B), C.c_int(W), C.c_int(H), C.c_int(D), *geom,
+                C.c_int(key_bits), nat.ptr(ws), nat.sz(ws.numel()), nat.ptr(nmap), nat.ptr(nmap_bwd), nat.ptr(gray), nat.ptr(binary),
+                nat.stream()))
+        return nmap, nmap_bwd, gray, binary
+    table = int(spconv.HASHMAP_RATIO * m)
+    if m > 0 and table < m:
+        raise ValueError(f"hashmap ratio {spconv.HASHMAP_RATIO} gives a table smaller than the input")
     keys = vals = None
     key_bits = 32
     with torch.cuda.device(dev):
@@ -106,10 +125,7 @@ def _build_maps(coords: torch.Tensor, out_coords: torch.Tensor, shape, kernel_si
                                                       C.c_int(D), nat.stream()))
         nat.check(L.fgx_spconv_neighbor_map(
             nat.ptr(keys), C.c_int(key_bits), nat.ptr(vals), nat.sz(table), nat.ptr(out_coords), nat.sz(l), nat.sz(m),
-            C.c_int(W), C.c_int(H), C.c_int(D), C.c_int(kw), C.c_int(kh), C.c_int(kd),
-            C.c_int(stride[0]), C.c_int(stride[1]), C.c_int(stride[2]),
-            C.c_int(padding[0]), C.c_int(padding[1]), C.c_int(padding[2]),
-            C.c_int(dilation[0]), C.c_int(dilation[1]), C.c_int(dilation[2]),
+            C.c_int(W), C.c_int(H), C.c_int(D), *geom,
             nat.ptr(nmap), nat.ptr(nmap_bwd), nat.ptr(gray), nat.ptr(binary), nat.stream()))
     return nmap, nmap_bwd, gray, binary
 

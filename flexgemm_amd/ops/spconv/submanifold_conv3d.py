@@ -280,7 +280,7 @@ def _build_neighbor_map(coords: torch.Tensor, shape, kernel_size, dilation, with
         binary = torch.empty((n,), dtype=torch.int32, device=dev)
     builder = spconv.NEIGHBOR_MAP_BUILDER
     if builder == "auto":
-        builder = "sort" if n >= spconv.SORT_BUILDER_MIN_VOXELS else "hash"
+        builder = "sort" if n * v >= spconv.SORT_BUILDER_MIN_PROBES else "hash"
     vol = B * W * H * D
     if builder == "sort" and kw * kh <= 128 and vol <= 2 ** 63:
         key_bits = 32 if vol <= 2 ** 32 else 64

@@ -298,6 +298,20 @@ int fgx_spconv_neighbor_map(const void* keys, int key_bits, const uint32_t* vals
                             int Dw, int Dh, int Dd, uint32_t* map_fwd, uint32_t* map_bwd,
                             int32_t* gray, int32_t* binary, fgx_stream_t stream);
 
+/* The same two maps (and codes) without a hash table, as fgx_subm_neighbor_map_sorted finds the submanifold map: the
+ * input voxels are sorted by flattened key, the output voxels by the key of the cell their kernel position (0, 0, 0)
+ * reads, and every group of 256 consecutive output voxels finds its neighbors of one (kx, ky) in one window of the
+ * sorted inputs.  Takes the coordinates themselves; out_coords may be in any order.  key_bits: 32 when
+ * B*W*H*D <= 2^32, else 64 (grids up to 2^62 cells).  workspace: fgx_spconv_neighbor_map_sorted_workspace_bytes bytes,
+ * 256-byte aligned.
+ * Replaces: the same reference function as fgx_spconv_neighbor_map. */
+size_t fgx_spconv_neighbor_map_sorted_workspace_bytes(size_t n_in, size_t n_out, int key_bits, int Kw, int Kh);
+int fgx_spconv_neighbor_map_sorted(const int32_t* in_coords, size_t n_in, const int32_t* out_coords, size_t n_out,
+                                   int B, int W, int H, int D, int Kw, int Kh, int Kd, int Sw, int Sh, int Sd,
+                                   int Pw, int Ph, int Pd, int Dw, int Dh, int Dd, int key_bits,
+                                   void* workspace, size_t workspace_bytes, uint32_t* map_fwd, uint32_t* map_bwd,
+                                   int32_t* gray, int32_t* binary, fgx_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -32,6 +32,14 @@ GEOMS = [
 ]
 
 
+@pytest.fixture(params=["hash", "sort"], autouse=True)
+def neighbor_map_builder(request):
+    """Every test of this file runs once per way of finding the neighbors: nothing may depend on it."""
+    flex_gemm.ops.spconv.set_neighbor_map_builder(request.param)
+    yield request.param
+    flex_gemm.ops.spconv.set_neighbor_map_builder("auto")
+
+
 def _say(msg):
     print(f"[case] {msg}", flush=True)
     sys.stdout.flush()
