@@ -6,7 +6,7 @@ import sys
 
 import flexgemm_amd as _impl
 
-for _name in ("ops", "ops.utils", "ops.spconv", "ops.spconv.submanifold_conv3d", "ops.spconv.sparse_conv3d"):
+for _name in ("ops", "ops.utils", "ops.serialize", "ops.spconv", "ops.spconv.submanifold_conv3d", "ops.spconv.sparse_conv3d"):
     sys.modules[__name__ + "." + _name] = importlib.import_module("flexgemm_amd." + _name)
 
 ops = _impl.ops

@@ -36,6 +36,8 @@ EXPORTS = [
     "fgx_spconv_out_dims", "fgx_spconv_out_coords_workspace_bytes", "fgx_spconv_out_coords_keys",
     "fgx_spconv_out_coords_decode", "fgx_spconv_neighbor_map",
     "fgx_spconv_neighbor_map_sorted_workspace_bytes", "fgx_spconv_neighbor_map_sorted",
+    "fgx_serialize_encode", "fgx_serialize_decode", "fgx_serialize_reorder_workspace_bytes",
+    "fgx_serialize_reorder_coords",
 ]
 
 
@@ -76,7 +78,7 @@ def lib() -> C.CDLL:
                      "fgx_weight_panel_bytes", "fgx_conv_scratch_bytes", "fgx_wgrad_scratch_bytes",
                      "fgx_colsum_scratch_bytes", "fgx_spconv_out_coords_workspace_bytes",
                      "fgx_subm_neighbor_map_sorted_workspace_bytes", "fgx_wgrad_block_bounds_count",
-                     "fgx_spconv_neighbor_map_sorted_workspace_bytes"):
+                     "fgx_spconv_neighbor_map_sorted_workspace_bytes", "fgx_serialize_reorder_workspace_bytes"):
             getattr(L, name).restype = C.c_size_t
         _lib = L
     return _lib

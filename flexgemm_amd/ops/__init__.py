@@ -1,1 +1,1 @@
-from . import spconv, utils
+from . import serialize, spconv, utils

@@ -16,6 +16,7 @@ from torch.autograd import Function
 
 from ... import _native as nat
 from .. import spconv, utils
+from .. import serialize
 from . import Algorithm, SerializationMode, SparseConv3dOutCoordAlgorithm
 from .submanifold_conv3d import (EMPTY, _IMPLICIT, _MASKED, _NO_SPLITK, SubMConv3dNeighborCache, _codes_and_order, _colsum,
                                  _gather_gemm, _gathered_rows, _pair_lists, _require_cuda, _wgrad)
@@ -140,18 +141,21 @@ class SparseConv3dFunction(Function):
         padding: Tuple[int, int, int],
         dilation: Tuple[int, int, int],
     ) -> torch.Tensor:
-        """int32 [L, 4] output coordinates, sorted by (b, x, y, z) (reference: sparse_conv3d.py:60-94).
+        """int32 [L, 4] output coordinates (reference: sparse_conv3d.py:60-94), sorted by (b, x, y, z) under
+        SerializationMode.BXYZ, along the z-order or Hilbert curve under the other two modes.
 
         Both of the reference's OUT_COORD_ALGO values name the same result; on gfx950 one streaming pass (candidate
-        keys, radix sort, unique) serves both.  Only BXYZ serialisation, the reference's default, is available."""
+        keys, radix sort, unique) serves both.  The curve modes re-sort the unique coordinates by their code; the bits
+        per axis come from the INPUT grid, as in the reference (sparse_neighbor_map.cu:157-160), which fixes the
+        orientation of the Hilbert curve."""
         assert coords.is_contiguous(), "Coords should be contiguous"
         assert coords.dtype in [torch.int32], "Unsupported coords dtype. Expect int32"
         if not coords.is_cuda:
             raise NotImplementedError("CPU version is not implemented")
         if spconv.OUT_COORD_ALGO not in (SparseConv3dOutCoordAlgorithm.HASHMAP, SparseConv3dOutCoordAlgorithm.EXPAND_UNIQUE):
             raise ValueError(f"Unsupported output-coordinate algorithm {spconv.OUT_COORD_ALGO}")
-        if spconv.SERIALIZATION_MODE != SerializationMode.BXYZ:
-            raise NotImplementedError("only SerializationMode.BXYZ orders the output coordinates on this build")
+        if spconv.SERIALIZATION_MODE not in (SerializationMode.BXYZ, SerializationMode.Z_ORDER, SerializationMode.HILBERT):
+            raise ValueError("Unsupported serialize mode.")
         B, _, W, H, D = [int(s) for s in shape]
         ks, st, pd, dl = _triple(kernel_size), _triple(stride), _triple(padding), _triple(dilation)
         wo, ho, do = _out_dims(shape, ks, st, pd, dl)
@@ -177,6 +181,11 @@ class SparseConv3dFunction(Function):
             out = torch.empty((total, 4), dtype=torch.int32, device=dev)
             nat.check(L.fgx_spconv_out_coords_decode(nat.ptr(ws), C.c_int(key_bits), nat.sz(total), C.c_int(wo), C.c_int(ho),
                                                      C.c_int(do), nat.ptr(out), nat.stream()))
+        if spconv.SERIALIZATION_MODE != SerializationMode.BXYZ:
+            bit_length = (max(W, H, D) - 1).bit_length()
+            if max(wo, ho, do) > (1 << bit_length):
+                raise ValueError("output grid exceeds the bits per axis of the input grid: curve codes would collide")
+            out = serialize.reorder_coords(out, bit_length, (B - 1).bit_length(), int(spconv.SERIALIZATION_MODE))
         return out
 
     @staticmethod

@@ -312,6 +312,28 @@ int fgx_spconv_neighbor_map_sorted(const int32_t* in_coords, size_t n_in, const 
                                    void* workspace, size_t workspace_bytes, uint32_t* map_fwd, uint32_t* map_bwd,
                                    int32_t* gray, int32_t* binary, fgx_stream_t stream);
 
+/* ---- Space-filling-curve codes of voxel coordinates -----------------------------------------------------------
+ * mode: 1 = z-order (Morton), 2 = Hilbert (the values of SerializationMode, flex_gemm/ops/spconv/__init__.py:20-24).
+ * coords int32[n, 4] = (b, x, y, z), 16-byte aligned.  bit_length = bits per spatial coordinate; x, y, z give bit i to
+ * code bits 3i+2, 3i+1, 3i, the batch index sits above bit 3*bit_length.  code_bits: 32 (uint32 codes,
+ * bit_length <= 10) or 64 (uint64, bit_length <= 21) -- the caller applies the width rule of
+ * flex_gemm/ops/serialize.py:26-31.
+ * Replace: z_order_encode / hilbert_encode and z_order_decode / hilbert_decode, flex_gemm/kernels/cuda/serialize/api.h:22-76
+ * (device code z_order.h:22-40, hilbert.h:22-118).  Unlike z_order.h:29 the batch index is widened before the shift. */
+int fgx_serialize_encode(int mode, const int32_t* coords, size_t n, int bit_length, int code_bits, void* codes,
+                         fgx_stream_t stream);
+int fgx_serialize_decode(int mode, const void* codes, size_t n, int bit_length, int code_bits, int32_t* coords,
+                         fgx_stream_t stream);
+
+/* out_coords = coords sorted by code (unsigned, ascending): encode, radix sort over batch_bits + 3*bit_length bits,
+ * decode.  This is the order the reference leaves the output coordinates of the generic convolution in when
+ * SERIALIZATION_MODE is Z_ORDER or HILBERT (its keys are these codes: sparse_neighbor_map.cu:156-187,
+ * spconv/utils.h:47-107).  Coordinates must fit bit_length bits, batch indices batch_bits bits.
+ * workspace: fgx_serialize_reorder_workspace_bytes(n, code_bits) bytes, 256-byte aligned; out_coords != coords. */
+size_t fgx_serialize_reorder_workspace_bytes(size_t n, int code_bits);
+int fgx_serialize_reorder_coords(int mode, const int32_t* coords, size_t n, int bit_length, int batch_bits, int code_bits,
+                                 void* workspace, size_t workspace_bytes, int32_t* out_coords, fgx_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
