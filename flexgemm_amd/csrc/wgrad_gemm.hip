@@ -800,9 +800,10 @@ __global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restri
     }
 }
 
-// The same sum with one thread per element: 1 KiB contiguous per workgroup and block.  Used unless the weight is so small
-// that this leaves most CUs idle while every thread walks a long list of blocks.  Which of the two runs depends on the
-// problem's shape alone, not on which kernel wrote the partial products.
+// The same sum with one thread per element: 1 KiB contiguous per workgroup and block.  For weights whose rows are not a
+// multiple of 128 channels (wider ones take the row-per-wavefront kernel below) and that are not so small that this
+// leaves most CUs idle while every thread walks a long list of blocks.  Which kernel runs depends on the problem's shape
+// alone, not on which kernel wrote the partial products.
 template <typename T>
 __global__ void __launch_bounds__(256) wgrad_reduce_flat_kernel(const float* __restrict__ partial,
                                                                 const uint32_t* __restrict__ bounds, int V, int Ci, int Co,
@@ -837,6 +838,61 @@ __global__ void __launch_bounds__(256) wgrad_reduce_flat_kernel(const float* __r
     }
 }
 
+// The same sum with one wavefront per (co, v) row of the result: which blocks have a partial product for this v is
+// one ballot over the block table (64 blocks per turn), so the loads of the partial products depend on nothing but
+// that mask and eight of them (VEC floats per lane each) are in flight per lane.  Needs Ci to be a multiple of VEC.
+// Sums in ascending block order like the other two kernels: same result bit for bit.
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256) wgrad_reduce_rows_kernel(const float* __restrict__ partial,
+                                                                const uint32_t* __restrict__ bounds, int V, int Ci, int Co,
+                                                                unsigned nb, unsigned per_block, T* __restrict__ gw) {
+    using vec_t = float __attribute__((ext_vector_type(VEC)));
+    const int lane = threadIdx.x & 63;
+    const size_t rows = (size_t)Co * V;
+    const size_t per = (size_t)Co * Ci;
+    const size_t stride = (size_t)V * per;
+    const unsigned blocks = nb / per_block;
+    for (size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6); row < rows; row += (size_t)gridDim.x * 4) {
+        const int v = (int)(row % V);
+        const size_t co = row / V;
+        const uint32_t* bd = bounds + (size_t)v * (blocks + 1);
+        const float* src_row = partial + (size_t)v * per + co * Ci;
+        T* dst_row = gw + row * Ci;
+        for (int c0 = lane * VEC; c0 < Ci; c0 += 64 * VEC) {
+            vec_t s = 0.f;
+            for (unsigned blk0 = 0; blk0 < blocks; blk0 += 64) {
+                const unsigned mine = blk0 + lane;
+                uint64_t live = __ballot(mine < blocks && bd[mine] < bd[mine + 1]);
+                while (live) {
+                    // up to eight live blocks at a time, ascending
+                    unsigned idx[8];
+                    int cnt = 0;
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) {
+                        idx[q] = 0;
+                        if (live) {
+                            idx[q] = blk0 + (unsigned)__builtin_ctzll(live);
+                            live &= live - 1;
+                            cnt = q + 1;
+                        }
+                    }
+                    for (unsigned sl = 0; sl < per_block; ++sl) {
+                        vec_t x[8];
+#pragma unroll
+                        for (int q = 0; q < 8; ++q)
+                            if (q < cnt) x[q] = *reinterpret_cast<const vec_t*>(src_row + (size_t)(idx[q] * per_block + sl) * stride + c0);
+#pragma unroll
+                        for (int q = 0; q < 8; ++q)
+                            if (q < cnt) s += x[q];
+                    }
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) dst_row[c0 + e] = from_float<T>(s[e]);
+        }
+    }
+}
+
 constexpr unsigned kReduceSlicedFrom = 32;      // partial products from which the sliced reduction is considered
 constexpr unsigned kReduceFlatGroups = 1024;    // ... when the flat kernel would launch fewer workgroups than this
 
@@ -844,7 +900,18 @@ template <typename T>
 int launch_reduce(const float* partial, const uint32_t* bounds, int V, int Ci, int Co, unsigned nb, unsigned per_block, T* gw,
                   hipStream_t s) {
     const size_t total = (size_t)Co * V * Ci;
-    if (nb >= kReduceSlicedFrom && cdiv(total, 256) < kReduceFlatGroups) {
+    const bool few_groups = nb >= kReduceSlicedFrom && cdiv(total, 256) < kReduceFlatGroups;
+    if (Ci % 128 == 0 && per_block == 1 && !few_groups) {
+        unsigned g = cdiv((size_t)Co * V, 4);
+        if (g > 65536u) g = 65536u;
+        if (Ci % 256 == 0)
+            wgrad_reduce_rows_kernel<T, 4><<<g, 256, 0, s>>>(partial, bounds, V, Ci, Co, nb, per_block, gw);
+        else
+            wgrad_reduce_rows_kernel<T, 2><<<g, 256, 0, s>>>(partial, bounds, V, Ci, Co, nb, per_block, gw);
+        FGX_CHECK_LAUNCH("fgx_conv_wgrad(reduce)");
+        return FGX_OK;
+    }
+    if (few_groups) {
         unsigned g = cdiv(total, kReduceElems);
         if (g > 65536u) g = 65536u;
         wgrad_reduce_kernel<T><<<g, 256, 0, s>>>(partial, bounds, V, Ci, Co, nb, per_block, gw);
