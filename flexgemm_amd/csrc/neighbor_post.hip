@@ -19,7 +19,8 @@ namespace fgx {
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kPairRows = 256;   // voxels per block in the pair-list passes
+constexpr int kPairRows = 256;       // voxels per block in the pair-list passes (larger blocks were not faster)
+constexpr int kPairThreads = 256;    // ... walked in chunks of this many
 
 __global__ void __launch_bounds__(kBlock) iota_u32_kernel(uint32_t* out, size_t n) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
@@ -108,21 +109,29 @@ SortLayout sort_layout(size_t n) {
     return L;
 }
 
-// counts[v * nblk + blk] = number of voxels of block blk whose mask has bit v set
-__global__ void __launch_bounds__(kPairRows) pair_count_kernel(const int32_t* __restrict__ gray, size_t n, int V,
-                                                               unsigned nblk, uint32_t* __restrict__ counts) {
-    __shared__ uint32_t wave_cnt[kPairRows / 64][32];
-    const size_t row = (size_t)blockIdx.x * kPairRows + threadIdx.x;
-    const uint32_t g = row < n ? (uint32_t)gray[row] : 0u;
+// counts[v * nblk + blk] = number of voxels of block blk whose mask has bit v set.  A block is kPairRows voxels, walked
+// by kPairThreads threads in kPairRows / kPairThreads chunks.
+__global__ void __launch_bounds__(kPairThreads) pair_count_kernel(const int32_t* __restrict__ gray, size_t n, int V,
+                                                                  unsigned nblk, uint32_t* __restrict__ counts) {
+    __shared__ uint32_t wave_cnt[kPairThreads / 64][32];
+    constexpr int kChunks = kPairRows / kPairThreads;
+    uint32_t g[kChunks];
+#pragma unroll
+    for (int c = 0; c < kChunks; ++c) {
+        const size_t row = (size_t)blockIdx.x * kPairRows + c * kPairThreads + threadIdx.x;
+        g[c] = row < n ? (uint32_t)gray[row] : 0u;
+    }
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     for (int v = 0; v < V; ++v) {
-        unsigned long long b = __ballot((g >> v) & 1u);
-        if (lane == 0) wave_cnt[wave][v] = (uint32_t)__popcll(b);
+        uint32_t cnt = 0;
+#pragma unroll
+        for (int c = 0; c < kChunks; ++c) cnt += (uint32_t)__popcll(__ballot((g[c] >> v) & 1u));
+        if (lane == 0) wave_cnt[wave][v] = cnt;
     }
     __syncthreads();
     if (threadIdx.x < V) {
         uint32_t c = 0;
-        for (int w = 0; w < kPairRows / 64; ++w) c += wave_cnt[w][threadIdx.x];
+        for (int w = 0; w < kPairThreads / 64; ++w) c += wave_cnt[w][threadIdx.x];
         counts[(size_t)threadIdx.x * nblk + blockIdx.x] = c;
     }
 }
@@ -135,36 +144,69 @@ __global__ void pair_seg_kernel(const uint32_t* __restrict__ offsets, const uint
     if (v == V) seg[V] = nblk ? offsets[(size_t)V * nblk - 1] + counts[(size_t)V * nblk - 1] : 0u;
 }
 
-// Stage the block's map rows in LDS with coalesced loads, then for every offset rank the present
-// voxels (wave ballot + prefix of the wave totals) and write (n, map[n, v]) at offsets[v, blk] + rank.
-__global__ void __launch_bounds__(kPairRows) pair_fill_kernel(const uint32_t* __restrict__ map,
-                                                              const int32_t* __restrict__ gray, size_t n, int V,
-                                                              unsigned nblk, const uint32_t* __restrict__ offsets,
-                                                              uint32_t* __restrict__ sig_i, uint32_t* __restrict__ sig_o) {
+// A block takes kPairRows voxels in chunks of kPairThreads: the chunk's map rows are staged in LDS with coalesced loads,
+// then for every offset the present voxels are ranked (wave ballot + prefix of the wave totals) and (n, map[n, v]) goes
+// to first[v] + rank, where first[v] starts at offsets[v, blk] and moves on by the chunk's count.  The pairs a block
+// adds to one offset's list are therefore one run of up to kPairRows entries written by one workgroup within a few
+// microseconds: the partial cache lines at the seams of the chunks' pieces meet in L2.
+__global__ void __launch_bounds__(kPairThreads) pair_fill_kernel(const uint32_t* __restrict__ map,
+                                                                 const int32_t* __restrict__ gray, size_t n, int V,
+                                                                 unsigned nblk, const uint32_t* __restrict__ offsets,
+                                                                 uint32_t* __restrict__ sig_i, uint32_t* __restrict__ sig_o) {
     extern __shared__ uint32_t lds[];
-    uint32_t* rows = lds;                                 // [kPairRows * V]
-    uint32_t* wave_cnt = lds + (size_t)kPairRows * V;     // [4][32]
-    const size_t base = (size_t)blockIdx.x * kPairRows;
-    const size_t len = (n - base < (size_t)kPairRows ? n - base : (size_t)kPairRows) * V;
-    for (size_t i = threadIdx.x; i < len; i += kPairRows) rows[i] = map[base * V + i];
-    const size_t row = base + threadIdx.x;
-    const uint32_t g = row < n ? (uint32_t)gray[row] : 0u;
+    constexpr int kWaves = kPairThreads / 64;
+    uint32_t* rows = lds;                                    // [kPairThreads * V]
+    uint32_t* wave_cnt2 = lds + (size_t)kPairThreads * V;    // [2][kWaves][32], by chunk parity
+    uint32_t* first = wave_cnt2 + 2 * kWaves * 32;           // [32] where the next pairs of each offset go
+    // fetched once, up front: a load inside the offset loop below would put a memory round trip into each of its turns
+    if (threadIdx.x < V) first[threadIdx.x] = offsets[(size_t)threadIdx.x * nblk + blockIdx.x];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-    for (int v = 0; v < V; ++v) {
-        unsigned long long b = __ballot((g >> v) & 1u);
-        if (lane == 0) wave_cnt[wave * 32 + v] = (uint32_t)__popcll(b);
-    }
-    __syncthreads();
-    for (int v = 0; v < V; ++v) {
-        unsigned long long b = __ballot((g >> v) & 1u);
-        if ((g >> v) & 1u) {
-            uint32_t r = (uint32_t)__popcll(b & below);
-            for (int w = 0; w < wave; ++w) r += wave_cnt[w * 32 + v];
-            size_t to = (size_t)offsets[(size_t)v * nblk + blockIdx.x] + r;
-            sig_o[to] = (uint32_t)row;
-            sig_i[to] = rows[(size_t)threadIdx.x * V + v];
+    for (int c = 0; c < kPairRows / kPairThreads; ++c) {
+        const size_t base = (size_t)blockIdx.x * kPairRows + (size_t)c * kPairThreads;
+        if (base >= n) break;                                // uniform
+        // two count tables: the first wavefront may still be adding up the previous chunk's counts (below) while the
+        // others write this chunk's
+        uint32_t* wave_cnt = wave_cnt2 + (c & 1) * kWaves * 32;
+        const size_t len = (n - base < (size_t)kPairThreads ? n - base : (size_t)kPairThreads) * V;
+        // eight loads in flight per thread: a plain copy loop waits for each load before it issues the next
+        for (size_t i0 = 0; i0 < len; i0 += 8 * kPairThreads) {
+            uint32_t t8[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const size_t i = i0 + (size_t)q * kPairThreads + threadIdx.x;
+                t8[q] = i < len ? map[base * V + i] : 0u;
+            }
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const size_t i = i0 + (size_t)q * kPairThreads + threadIdx.x;
+                if (i < len) rows[i] = t8[q];
+            }
         }
+        const size_t row = base + threadIdx.x;
+        const uint32_t g = row < n ? (uint32_t)gray[row] : 0u;
+        for (int v = 0; v < V; ++v) {
+            unsigned long long b = __ballot((g >> v) & 1u);
+            if (lane == 0) wave_cnt[wave * 32 + v] = (uint32_t)__popcll(b);
+        }
+        __syncthreads();
+        for (int v = 0; v < V; ++v) {
+            unsigned long long b = __ballot((g >> v) & 1u);
+            if ((g >> v) & 1u) {
+                uint32_t r = (uint32_t)__popcll(b & below);
+                for (int w = 0; w < wave; ++w) r += wave_cnt[w * 32 + v];
+                size_t to = (size_t)first[v] + r;
+                sig_o[to] = (uint32_t)row;
+                sig_i[to] = rows[(size_t)threadIdx.x * V + v];
+            }
+        }
+        __syncthreads();                                     // rows and first[] have been read by everyone
+        if (threadIdx.x < V) {
+            uint32_t add = 0;
+            for (int w = 0; w < kWaves; ++w) add += wave_cnt[w * 32 + threadIdx.x];
+            first[threadIdx.x] += add;
+        }
+        // the next chunk's first barrier orders these updates before they are read
     }
 }
 
@@ -228,6 +270,8 @@ __global__ void __launch_bounds__(kBlock) plan_fill_kernel(const uint32_t* __res
                                                            const int32_t* __restrict__ seg, size_t n, int V, int tile_rows,
                                                            uint32_t* __restrict__ plan_idx, uint32_t* __restrict__ plan_band) {
     __shared__ uint32_t bands[32];
+    __shared__ uint32_t stage[kBlock * 32];      // kBlock map rows of V <= 32 words
+    __shared__ int64_t src_row[kBlock];          // which map row each of them is (-1: past the end)
     const size_t t = blockIdx.x;
     uint32_t code = (uint32_t)tile_code[t];
     size_t slot = (size_t)seg[t];
@@ -237,12 +281,34 @@ __global__ void __launch_bounds__(kBlock) plan_fill_kernel(const uint32_t* __res
         return;
     }
     if (threadIdx.x < 32) bands[threadIdx.x] = 0u;
-    __syncthreads();
     const int lane = threadIdx.x & 63;
     for (int r0 = 0; r0 < tile_rows; r0 += kBlock) {
+        // The rows of this tile sit wherever the mask order put them.  A half-wave fetches one whole row (V consecutive
+        // words: one or two cache lines per request) into LDS; each thread then walks its own row there.  One thread
+        // per row reading straight from memory would ask for 64 different cache lines with every load instruction.
+        __syncthreads();                         // the previous chunk's rows have been consumed; bands[] is cleared
+        {
+            const size_t row = t * (size_t)tile_rows + r0 + threadIdx.x;
+            src_row[threadIdx.x] = (r0 + (int)threadIdx.x < tile_rows && row < n) ? order[row] : (int64_t)-1;
+        }
+        __syncthreads();
+        for (int i0 = 0; i0 < kBlock * 32; i0 += 8 * kBlock) {       // eight loads in flight per thread
+            uint32_t t8[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const int i = i0 + q * kBlock + threadIdx.x;
+                const int64_t src = src_row[i >> 5];
+                t8[q] = ((i & 31) < V && src >= 0) ? map[(size_t)src * V + (i & 31)] : FGX_EMPTY32;
+            }
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const int i = i0 + q * kBlock + threadIdx.x;
+                if ((i & 31) < V) stage[(i >> 5) * V + (i & 31)] = t8[q];
+            }
+        }
+        __syncthreads();
         const int r = r0 + threadIdx.x;
-        const size_t row = t * (size_t)tile_rows + r;
-        const uint32_t* mrow = (r < tile_rows && row < n) ? map + (size_t)order[row] * V : nullptr;
+        const uint32_t* mrow = src_row[threadIdx.x] >= 0 ? stage + threadIdx.x * V : nullptr;
         uint32_t c = code;
         size_t s = slot;
         int k = 0;
@@ -397,7 +463,7 @@ int fgx_pair_count(const int32_t* gray, size_t n, int V, uint32_t* seg, void* wo
     uint32_t* counts = n ? (uint32_t*)(ws + L.counts) : nullptr;
     uint32_t* offsets = n ? (uint32_t*)(ws + L.offsets) : nullptr;
     if (n > 0) {
-        pair_count_kernel<<<L.nblk, kPairRows, 0, s>>>(gray, n, V, L.nblk, counts);
+        pair_count_kernel<<<L.nblk, kPairThreads, 0, s>>>(gray, n, V, L.nblk, counts);
         FGX_CHECK_LAUNCH("fgx_pair_count(count)");
         size_t temp_bytes = L.temp_bytes;
         FGX_CHECK_HIP(rocprim::exclusive_scan(ws + L.temp, temp_bytes, counts, offsets, 0u, (size_t)L.nblk * V,
@@ -415,8 +481,8 @@ int fgx_pair_fill(const uint32_t* map, const int32_t* gray, size_t n, int V, con
     FGX_CHECK_ARG(map && gray && workspace && sig_i && sig_o, "fgx_pair_fill: null buffer");
     PairLayout L = pair_layout(n, V);
     const uint32_t* offsets = (const uint32_t*)((const char*)workspace + L.offsets);
-    size_t lds = ((size_t)kPairRows * V + 4 * 32) * sizeof(uint32_t);
-    pair_fill_kernel<<<L.nblk, kPairRows, lds, (hipStream_t)stream>>>(map, gray, n, V, L.nblk, offsets, sig_i, sig_o);
+    size_t lds = ((size_t)kPairThreads * V + 2 * (kPairThreads / 64) * 32 + 32) * sizeof(uint32_t);
+    pair_fill_kernel<<<L.nblk, kPairThreads, lds, (hipStream_t)stream>>>(map, gray, n, V, L.nblk, offsets, sig_i, sig_o);
     FGX_CHECK_LAUNCH("fgx_pair_fill");
     return FGX_OK;
 }
