@@ -89,6 +89,55 @@ __global__ void __launch_bounds__(256) window_bounds_kernel(const K* __restrict_
     bounds[t] = (uint32_t)pos;
 }
 
+// Which rows hold the keys first, first + Dd, ... (Kd of them, ascending) in the sorted window wkeys[0, wn), wn > 0?
+// emit(kz, row index or EMPTY) is called for every kz.  One binary search for the first key -- a fixed number of
+// halving steps, the same for every lane, no data-dependent branch -- then at most Dd steps forward to each next one
+// (keys are distinct integers).  `first` may lie below zero (next to the origin, or for a base cell outside the grid);
+// row_in tells whether the (x, y) of these targets lies inside the grid, target kz lies inside along z when
+// z_first + kz * Dd is in [0, D).  A lane outside searches too and discards what it finds.
+template <typename K, typename Emit>
+__device__ __forceinline__ void search_staged(const K* wkeys, const uint32_t* wrows, unsigned wn, long long first, bool row_in,
+                                              int z_first, int Kd, int Dd, int D, Emit emit) {
+    const K t0 = (K)(first < 0 ? 0 : first);
+    unsigned pos = 0;           // number of window keys below the current target
+    for (unsigned step = 1u << (31 - __clz((int)wn)); step > 0; step >>= 1) {
+        const unsigned cand = pos + step;
+        const unsigned at = (cand <= wn ? cand : wn) - 1;
+        if (wkeys[at] < t0 && cand <= wn) pos = cand;
+    }
+    for (int kz = 0; kz < Kd; ++kz) {
+        const long long t = first + (long long)kz * Dd;
+        const K tk = (K)t;
+        if (kz > 0 && t > 0) {
+            for (int s = 0; s < Dd; ++s) {
+                const unsigned at = pos < wn ? pos : wn - 1;
+                if (wkeys[at] < tk && pos < wn) ++pos;
+            }
+        }
+        const unsigned at = pos < wn ? pos : wn - 1;
+        const int z2 = z_first + kz * Dd;
+        const bool hit = wkeys[at] == tk && pos < wn && t >= 0 && row_in && z2 >= 0 && z2 < D;
+        emit(kz, hit ? wrows[at] : FGX_EMPTY32);
+    }
+}
+
+// The same questions for a window that is too long for LDS (or empty): searched where it lies in memory.
+template <typename K, typename Emit>
+__device__ __forceinline__ void search_in_place(const K* __restrict__ skeys, const uint32_t* __restrict__ srows, size_t lo,
+                                                size_t hi, long long first, bool row_in, int z_first, int Kd, int Dd, int D,
+                                                Emit emit) {
+    for (int kz = 0; kz < Kd; ++kz) {
+        const long long t = first + (long long)kz * Dd;
+        const int z2 = z_first + kz * Dd;
+        uint32_t value = FGX_EMPTY32;
+        if (lo < hi && row_in && z2 >= 0 && z2 < D && t >= 0) {
+            const size_t q = lower_bound_at<K>(skeys, lo, hi, (K)t);
+            if (q < hi && skeys[q] == (K)t) value = srows[q];
+        }
+        emit(kz, value);
+    }
+}
+
 template <typename K>
 __global__ void __launch_bounds__(kGroup) merge_neighbor_kernel(const K* __restrict__ skeys, const uint32_t* __restrict__ srows,
                                                                 const uint32_t* __restrict__ bounds, size_t n, SubmGeom g,
@@ -120,12 +169,21 @@ __global__ void __launch_bounds__(kGroup) merge_neighbor_kernel(const K* __restr
     if (live) {
         key = skeys[p0 + tid];
         me = srows[p0 + tid];
-        uint64_t t = (uint64_t)key;
-        z = (int)(t % (uint64_t)g.D);
-        t /= (uint64_t)g.D;
-        y = (int)(t % (uint64_t)g.H);
-        t /= (uint64_t)g.H;
-        x = (int)(t % (uint64_t)g.W);
+        if constexpr (sizeof(K) == 4) {         // 32-bit division is several times shorter than the 64-bit sequence
+            uint32_t t = (uint32_t)key;
+            z = (int)(t % (uint32_t)g.D);
+            t /= (uint32_t)g.D;
+            y = (int)(t % (uint32_t)g.H);
+            t /= (uint32_t)g.H;
+            x = (int)(t % (uint32_t)g.W);
+        } else {
+            uint64_t t = (uint64_t)key;
+            z = (int)(t % (uint64_t)g.D);
+            t /= (uint64_t)g.D;
+            y = (int)(t % (uint64_t)g.H);
+            t /= (uint64_t)g.H;
+            x = (int)(t % (uint64_t)g.W);
+        }
     }
     __syncthreads();
 
@@ -135,6 +193,7 @@ __global__ void __launch_bounds__(kGroup) merge_neighbor_kernel(const K* __restr
     K pk[kAhead][kPer];
     uint32_t pr[kAhead][kPer];
     uint32_t mask = 0;
+    const int z_first = z - (g.Kd / 2) * g.Dd;
     for (int r0 = 0; r0 < R; r0 += kAhead) {
 #pragma unroll
         for (int a = 0; a < kAhead; ++a) {
@@ -177,39 +236,14 @@ __global__ void __launch_bounds__(kGroup) merge_neighbor_kernel(const K* __restr
                 const long long off = (long long)(kx - g.Kw / 2) * g.Dw * HD + (long long)(ky - g.Kh / 2) * g.Dh * g.D;
                 uint32_t* out_row = stage_out ? out_rows + tid * (kStageV + 1) + r * g.Kd
                                               : out_map + (size_t)me * g.V + (size_t)r * g.Kd;
-                // the Kd targets of a row ascend by Dd: one binary search for the first, then a short walk to each next one
-                unsigned pos = 0;
-                bool searched = false;
-                const unsigned wn = (unsigned)w;
-                for (int kz = 0; kz < g.Kd; ++kz) {
-                    const int dz = (kz - g.Kd / 2) * g.Dd;
-                    const int z2 = z + dz;
-                    uint32_t value = FGX_EMPTY32;
-                    if (row_in && z2 >= 0 && z2 < g.D && w > 0) {
-                        const K target = (K)((long long)key + off + dz);
-                        if (staged) {
-                            if (!searched) {
-                                unsigned a = 0, b = wn;
-                                while (a < b) {
-                                    const unsigned mid = (a + b) >> 1;
-                                    if (wkeys[mid] < target) a = mid + 1;
-                                    else b = mid;
-                                }
-                                pos = a;
-                                searched = true;
-                            } else {
-                                while (pos < wn && wkeys[pos] < target) ++pos;
-                            }
-                            if (pos < wn && wkeys[pos] == target) value = wrows[pos];
-                        } else {
-                            const size_t q = lower_bound_at<K>(skeys, lo, hi, target);
-                            if (q < hi && skeys[q] == target) value = srows[q];
-                        }
-                    }
+                const long long first = (long long)key + off - (long long)(g.Kd / 2) * g.Dd;
+                auto emit = [&](int kz, uint32_t value) {
                     out_row[kz] = value;
                     const int v = r * g.Kd + kz;
                     if (v < 32 && value != FGX_EMPTY32) mask |= 1u << v;
-                }
+                };
+                if (staged && w > 0) search_staged<K>(wkeys, wrows, (unsigned)w, first, row_in, z_first, g.Kd, g.Dd, g.D, emit);
+                else search_in_place<K>(skeys, srows, lo, hi, first, row_in, z_first, g.Kd, g.Dd, g.D, emit);
             }
             __syncthreads();       // the window is overwritten by the next row
         }
@@ -438,40 +472,16 @@ __global__ void __launch_bounds__(kGroup) merge_query_kernel(const K* __restrict
                 const long long off = (long long)kx * g.Dw * HD + (long long)ky * g.Dh * g.D;
                 uint32_t* out_row = stage_out ? out_rows + tid * (kStageV + 1) + r * g.Kd
                                               : map_fwd + (size_t)me * g.V + (size_t)r * g.Kd;
-                unsigned pos = 0;
-                bool searched = false;
-                const unsigned wn = (unsigned)w;
-                for (int kz = 0; kz < g.Kd; ++kz) {
-                    const int z2 = zi + kz * g.Dd;
-                    uint32_t value = FGX_EMPTY32;
-                    if (row_in && z2 >= 0 && z2 < g.D && w > 0) {
-                        const K target = (K)(base + off + (long long)kz * g.Dd);
-                        if (staged) {
-                            if (!searched) {
-                                unsigned a2 = 0, b2 = wn;
-                                while (a2 < b2) {
-                                    const unsigned mid = (a2 + b2) >> 1;
-                                    if (wkeys[mid] < target) a2 = mid + 1;
-                                    else b2 = mid;
-                                }
-                                pos = a2;
-                                searched = true;
-                            } else {
-                                while (pos < wn && wkeys[pos] < target) ++pos;
-                            }
-                            if (pos < wn && wkeys[pos] == target) value = wrows[pos];
-                        } else {
-                            const size_t q = lower_bound_at<K>(skeys, lo, hi, target);
-                            if (q < hi && skeys[q] == target) value = srows[q];
-                        }
-                    }
+                auto emit = [&](int kz, uint32_t value) {
                     out_row[kz] = value;
                     const int v = r * g.Kd + kz;
                     if (value != FGX_EMPTY32) {
                         if (v < 32) mask |= 1u << v;
                         if (map_bwd != nullptr) map_bwd[(size_t)value * g.V + v] = me;
                     }
-                }
+                };
+                if (staged && w > 0) search_staged<K>(wkeys, wrows, (unsigned)w, base + off, row_in, zi, g.Kd, g.Dd, g.D, emit);
+                else search_in_place<K>(skeys, srows, lo, hi, base + off, row_in, zi, g.Kd, g.Dd, g.D, emit);
             }
             __syncthreads();
         }
