@@ -70,6 +70,51 @@ __global__ void __launch_bounds__(256) pack_weight_kernel(const T* __restrict__ 
     }
 }
 
+// The same panels for 16-bit types whose channel counts are multiples of 8, moved 16 bytes at a time.
+//
+// Forward panels copy runs: panel[v][slab][col][0, SK) is w[col][v][slab*SK, +SK), contiguous on both sides.  One thread
+// per 16-byte piece; grid = (pieces of a (v, slab) plane / 256, slabs, V), so no index needs a division.
+template <int SK>
+__global__ void __launch_bounds__(256) pack_weight_rows_kernel(const uint16_t* __restrict__ w, int Ci, int Co, int V,
+                                                               int cols_pad, uint16_t* __restrict__ panel) {
+    constexpr int PIECES = SK / 8;                          // 16-byte pieces per (col, slab) run
+    const int piece = blockIdx.x * 256 + threadIdx.x;       // inside the (v, slab) plane
+    if (piece >= cols_pad * PIECES) return;
+    const int col = piece / PIECES, kk = blockIdx.y * SK + (piece % PIECES) * 8, v = blockIdx.z;
+    uint4 val = make_uint4(0u, 0u, 0u, 0u);
+    if (col < Co && kk < Ci) val = *reinterpret_cast<const uint4*>(w + ((size_t)col * V + v) * Ci + kk);
+    *reinterpret_cast<uint4*>(panel + (((size_t)v * gridDim.y + blockIdx.y) * cols_pad) * SK + (size_t)piece * 8) = val;
+}
+
+// Input-gradient panels transpose: panel[v][slab][col][k] is w[slab*SK + k][v'][col] (v' = V-1-v when the offsets are
+// mirrored), contiguous along col in w and along k in the panel.  A workgroup moves one SK x 32 tile through LDS:
+// 16-byte reads along col, 2-byte LDS stores into the transposed tile, 16-byte LDS reads and stores along k.
+template <int SK>
+__global__ void __launch_bounds__(256) pack_weight_transpose_kernel(const uint16_t* __restrict__ w, int Ci, int Co, int V,
+                                                                    int mirror, int cols_pad, uint16_t* __restrict__ panel) {
+    constexpr int PITCH = SK + 8;                           // halfwords; keeps every row 16-byte aligned
+    __shared__ __attribute__((aligned(16))) uint16_t tile[32 * PITCH];
+    const int col0 = blockIdx.x * 32, slab = blockIdx.y, v = blockIdx.z;
+    const int vsrc = mirror ? V - 1 - v : v;
+    const int t = threadIdx.x;
+    if (t < SK * 4) {
+        const int r = t >> 2, c8 = (t & 3) * 8;             // row of the tile (a k value), first of 8 columns
+        const int kk = slab * SK + r, col = col0 + c8;
+        uint4 val = make_uint4(0u, 0u, 0u, 0u);
+        if (kk < Co && col < Ci) val = *reinterpret_cast<const uint4*>(w + ((size_t)kk * V + vsrc) * Ci + col);
+        const uint32_t words[4] = {val.x, val.y, val.z, val.w};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) tile[(c8 + j) * PITCH + r] = (uint16_t)(words[j >> 1] >> ((j & 1) * 16));
+    }
+    __syncthreads();
+    constexpr int PIECES = SK / 8;
+    if (t < 32 * PIECES) {
+        const int c = t / PIECES, k8 = (t % PIECES) * 8;
+        const uint4 val = *reinterpret_cast<const uint4*>(tile + c * PITCH + k8);
+        *reinterpret_cast<uint4*>(panel + ((((size_t)v * gridDim.y + slab) * cols_pad) + col0 + c) * SK + k8) = val;
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // Gather GEMM
 // ------------------------------------------------------------------------------------------------
@@ -579,6 +624,23 @@ int fgx_pack_weight(int dtype, int mode, const void* weight, int Ci, int Co, int
     unsigned grid = cdiv(total, 256);
     if (grid > 32768u) grid = 32768u;
     hipStream_t s = (hipStream_t)stream;
+    const bool wide = es == 2 && Ci % 8 == 0 && Co % 8 == 0 && (((uintptr_t)weight | (uintptr_t)panel) & 15) == 0 &&
+                      slabs <= 65535 && V <= 65535;
+    if (wide) {
+        const uint16_t* w16 = (const uint16_t*)weight;
+        uint16_t* p16 = (uint16_t*)panel;
+        if (mode == 0) {
+            const dim3 g(cdiv((size_t)cols_pad * (SK / 8), 256), slabs, V);
+            if (SK == 64) pack_weight_rows_kernel<64><<<g, 256, 0, s>>>(w16, Ci, Co, V, cols_pad, p16);
+            else pack_weight_rows_kernel<32><<<g, 256, 0, s>>>(w16, Ci, Co, V, cols_pad, p16);
+        } else {
+            const dim3 g(cols_pad / 32, slabs, V);
+            if (SK == 64) pack_weight_transpose_kernel<64><<<g, 256, 0, s>>>(w16, Ci, Co, V, mode == 1, cols_pad, p16);
+            else pack_weight_transpose_kernel<32><<<g, 256, 0, s>>>(w16, Ci, Co, V, mode == 1, cols_pad, p16);
+        }
+        FGX_CHECK_LAUNCH("fgx_pack_weight");
+        return FGX_OK;
+    }
     if (dtype == FGX_F32) pack_weight_kernel<float><<<grid, 256, 0, s>>>((const float*)weight, Ci, Co, V, mode, slab_bytes, slabs, cols_pad, (float*)panel);
     else pack_weight_kernel<uint16_t><<<grid, 256, 0, s>>>((const uint16_t*)weight, Ci, Co, V, mode, slab_bytes, slabs, cols_pad, (uint16_t*)panel);
     FGX_CHECK_LAUNCH("fgx_pack_weight");
