@@ -152,7 +152,8 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N)
 wgrad_kernel(const typename Tag::type* __restrict__ gout, const typename Tag::type* __restrict__ feats,
              const uint32_t* __restrict__ sig_i, const uint32_t* __restrict__ sig_o,
              const uint32_t* __restrict__ bounds, int V, int Ci, int Co, unsigned nb, unsigned co_tiles,
-             unsigned ci_tiles, bool small_tensors, float* __restrict__ partial) {
+             unsigned ci_tiles, bool small_tensors, float* __restrict__ partial,
+             typename Tag::type* __restrict__ direct) {
     using C = WgradCfg<Tag, BM, BN, WAVES_M, WAVES_N>;
     constexpr int ES = C::ES;
     constexpr int S = kStages;
@@ -348,8 +349,9 @@ wgrad_kernel(const typename Tag::type* __restrict__ gout, const typename Tag::ty
     }
     wait_vmcnt<0>();   // the trailing dummy loads
 
-    // partial[b][v][co][ci], fp32
+    // partial[b][v][co][ci], fp32 -- or, when there is a single voxel block, straight into grad_weight[co][v][ci]
     float* dst = partial + ((size_t)b * V + v) * ((size_t)Co * Ci);
+    typename Tag::type* out = direct ? direct + (size_t)v * Ci : nullptr;
 #pragma unroll
     for (int j = 0; j < C::TN; ++j) {
         const int ci = n0 + wave_n * C::WN + j * 32 + l32;
@@ -359,7 +361,10 @@ wgrad_kernel(const typename Tag::type* __restrict__ gout, const typename Tag::ty
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 int co = m0 + wave_m * C::WM + i * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
-                if (co < Co) dst[(size_t)co * Ci + ci] = acc[i][j][e];
+                if (co < Co) {
+                    if (out) out[(size_t)co * V * Ci + ci] = from_float<typename Tag::type>(acc[i][j][e]);
+                    else dst[(size_t)co * Ci + ci] = acc[i][j][e];
+                }
             }
     }
 }
@@ -436,7 +441,7 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
                     const uint32_t* __restrict__ sig_i, const uint32_t* __restrict__ sig_o,
                     const uint32_t* __restrict__ bounds, int V, int Ci, int Co, unsigned nb, unsigned co_tiles,
                     unsigned ci_tiles, uint32_t n_pairs, uint32_t gout_bytes, uint32_t feats_bytes,
-                    float* __restrict__ partial) {
+                    float* __restrict__ partial, typename Tag::type* __restrict__ direct) {
     using C = WStreamCfg<Tag, BM, BN>;
     constexpr int ES = C::ES, S = C::S, P = C::P;
 
@@ -725,6 +730,7 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
         const unsigned co_tile = tile % co_tiles, ci_tile = tile / co_tiles;
         const int m0 = (int)co_tile * BM, n0 = (int)ci_tile * BN;
         float* dst = partial + (((size_t)b * C::SLICES + (C::KSPLIT ? mw : 0)) * V + v) * ((size_t)Co * Ci);
+        typename Tag::type* out = direct ? direct + (size_t)v * Ci : nullptr;      // single voxel block: no partial products
 #pragma unroll
         for (int j = 0; j < C::TN; ++j) {
             const int ci = n0 + wave_n * C::WN + j * 32 + l32;
@@ -734,7 +740,10 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     int co = m0 + wave_m * C::WM + i * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
-                    if (co < Co) dst[(size_t)co * Ci + ci] = acc[i][j][e];
+                    if (co < Co) {
+                        if (out) out[(size_t)co * V * Ci + ci] = from_float<typename Tag::type>(acc[i][j][e]);
+                        else dst[(size_t)co * Ci + ci] = acc[i][j][e];
+                    }
                 }
         }
         m.k = m.k_hi;                               // on to the next non-empty item
@@ -924,6 +933,33 @@ int launch_reduce(const float* partial, const uint32_t* bounds, int V, int Ci, i
     return FGX_OK;
 }
 
+// grad_weight[:, v, :] = 0 for the offsets v of `mask`: offsets without a single pair when the kernels write
+// grad_weight themselves (they skip empty items)
+template <typename T>
+__global__ void __launch_bounds__(256) zero_offsets_kernel(T* __restrict__ gw, int Co, int V, int Ci, uint32_t mask) {
+    const size_t total = (size_t)Co * V * Ci;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        const int v = (int)(i / Ci % V);
+        if ((mask >> v) & 1u) gw[i] = from_float<T>(0.f);
+    }
+}
+
+// With a single voxel block there is one partial product per offset: the kernels round it and write grad_weight
+// themselves, and the reduction (and the fp32 scratch traffic) is skipped.  Same bits as the two-kernel path.
+template <typename T>
+int prepare_direct(const SegTable& tab, int V, int Ci, int Co, T* gw, hipStream_t s) {
+    uint32_t empty = 0;
+    for (int v = 0; v < V; ++v)
+        if (tab.seg[v + 1] == tab.seg[v]) empty |= 1u << v;
+    if (empty) {
+        unsigned g = cdiv((size_t)Co * V * Ci, 256);
+        if (g > 4096u) g = 4096u;
+        zero_offsets_kernel<T><<<g, 256, 0, s>>>(gw, Co, V, Ci, empty);
+        FGX_CHECK_LAUNCH("fgx_conv_wgrad(zero)");
+    }
+    return FGX_OK;
+}
+
 bool dtype_ok(int dtype) { return dtype == FGX_F16 || dtype == FGX_BF16 || dtype == FGX_F32; }
 
 struct Layout {
@@ -968,9 +1004,16 @@ int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, con
             FGX_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::lds_bytes));
             lds_raised = true;
         }
+        const bool direct = L.nb == 1;
+        if (direct) {
+            int rc = prepare_direct<T>(tab, V, Ci, Co, (T*)gw, s);
+            if (rc != FGX_OK) return rc;
+        }
         kern<<<(unsigned)grid, C::NT, C::lds_bytes, s>>>(
-            (const T*)gout, (const T*)feats, sig_i, sig_o, bounds, V, Ci, Co, L.nb, co_tiles, ci_tiles, small, partial);
+            (const T*)gout, (const T*)feats, sig_i, sig_o, bounds, V, Ci, Co, L.nb, co_tiles, ci_tiles, small, partial,
+            direct ? (T*)gw : nullptr);
         FGX_CHECK_LAUNCH("fgx_conv_wgrad");
+        if (direct) return FGX_OK;
     }
     return launch_reduce<T>(partial, bounds, V, Ci, Co, L.nb, 1u, (T*)gw, s);
 }
@@ -1005,10 +1048,16 @@ int launch_wgrad_stream(const void* gout, const void* feats, const uint32_t* sig
             FGX_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::lds_bytes));
             lds_raised = true;
         }
+        const bool direct = L.nb == 1 && C::SLICES == 1;
+        if (direct) {
+            int rc = prepare_direct<T>(tab, V, Ci, Co, (T*)gw, s);
+            if (rc != FGX_OK) return rc;
+        }
         kern<<<groups, C::NT, C::lds_bytes, s>>>((const T*)gout, (const T*)feats, sig_i, sig_o, bounds, V, Ci, Co, L.nb, co_tiles,
                                                  ci_tiles, tab.seg[V], (uint32_t)(n * (size_t)Co * sizeof(T)),
-                                                 (uint32_t)(n_in * (size_t)Ci * sizeof(T)), partial);
+                                                 (uint32_t)(n_in * (size_t)Ci * sizeof(T)), partial, direct ? (T*)gw : nullptr);
         FGX_CHECK_LAUNCH("fgx_conv_wgrad(stream)");
+        if (direct) return FGX_OK;
     }
     return launch_reduce<T>(partial, bounds, V, Ci, Co, L.nb * C::SLICES, (unsigned)C::SLICES, (T*)gw, s);
 }
