@@ -53,10 +53,11 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
         out->tile_cols = t;
         out->slab_bytes = 64;
         out->splitk = 1;
-        // persistent streaming kernel: 16-bit types, enough voxels to give every CU several items.  Its 32 x 32 tile
+        // persistent streaming kernel: 16-bit types; measured ahead of the tiled kernel from about two thousand voxels
+        // on (both walk the same item list).  Its 32 x 32 tile
         // writes four partial products per voxel block (one per multiplying wavefront), so its blocks are four times
         // as long.
-        out->stream = (es == 2 && n >= 32768) ? 1 : 0;
+        out->stream = (es == 2 && n >= 2048) ? 1 : 0;
         const int slices = (out->stream && t == 32) ? 4 : 1;
         const double per_block = 4.0 * V * (double)Co * (double)Ci * slices;
         size_t max_blocks = (size_t)(268435456.0 / per_block);
@@ -81,12 +82,15 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
     while (tiles * s < (size_t)kCUs && s < 16) s *= 2;
     out->splitk = s;
     // persistent streaming kernel (256-row tiles): rows of at least 64 bytes -- 128-byte K-slabs from 128 bytes on, 64-byte
-    // ones below, where 32 output columns get a tile of their own -- and at least two items per CU
+    // ones below, where 32 output columns get a tile of their own.  With 128-byte slabs it is ahead of the tiled kernel
+    // as soon as there is an item for a little under half of the CUs (measured: 120 items 10 % ahead, 64 items 13 %
+    // behind); the short-row form, two workgroups per CU, keeps the bar of two items per CU.
     const int K = pass_kind == 0 ? Ci : Co;
     const size_t row_bytes = (size_t)K * es;
     const int slab = row_bytes >= 128 ? 128 : 64;
     const int scols = cols > 64 ? 128 : ((cols > 32 || slab == 128) ? 64 : 32);
-    if (row_bytes >= 64 && (slab == 64 || cols >= 64) && (size_t)cdiv(n, 256) * cdiv(cols, scols) >= 2 * (size_t)kCUs) {
+    const size_t enough = slab == 128 ? (size_t)kCUs * 7 / 16 : 2 * (size_t)kCUs;
+    if (row_bytes >= 64 && (slab == 64 || cols >= 64) && (size_t)cdiv(n, 256) * cdiv(cols, scols) >= enough) {
         out->tile_rows = 256;
         out->tile_cols = scols;
         out->slab_bytes = slab;
