@@ -31,6 +31,7 @@ EXPORTS = [
     "fgx_table_lookup", "fgx_weight_panel_bytes", "fgx_pack_weight",
     "fgx_conv_scratch_bytes", "fgx_conv_gather_gemm",
     "fgx_gather_plan_count", "fgx_gather_plan_fill", "fgx_conv_gather_gemm_stream",
+    "fgx_conv_gather_gemm_stream_groups", "fgx_gather_item_order_workspace_bytes", "fgx_gather_item_order",
     "fgx_wgrad_scratch_bytes", "fgx_wgrad_block_bounds_count", "fgx_wgrad_block_bounds", "fgx_conv_wgrad",
     "fgx_colsum_scratch_bytes", "fgx_colsum",
     "fgx_spconv_out_dims", "fgx_spconv_out_coords_workspace_bytes", "fgx_spconv_out_coords_keys",
@@ -78,7 +79,8 @@ def lib() -> C.CDLL:
                      "fgx_weight_panel_bytes", "fgx_conv_scratch_bytes", "fgx_wgrad_scratch_bytes",
                      "fgx_colsum_scratch_bytes", "fgx_spconv_out_coords_workspace_bytes",
                      "fgx_subm_neighbor_map_sorted_workspace_bytes", "fgx_wgrad_block_bounds_count",
-                     "fgx_spconv_neighbor_map_sorted_workspace_bytes", "fgx_serialize_reorder_workspace_bytes"):
+                     "fgx_spconv_neighbor_map_sorted_workspace_bytes", "fgx_serialize_reorder_workspace_bytes",
+                     "fgx_gather_item_order_workspace_bytes"):
             getattr(L, name).restype = C.c_size_t
         _lib = L
     return _lib

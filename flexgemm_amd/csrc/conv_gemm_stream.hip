@@ -107,7 +107,8 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
                           const uint32_t* __restrict__ plan_idx, const uint32_t* __restrict__ plan_band, uint32_t n, int K,
                           int cols, int cols_pad,
                           unsigned row_tiles, unsigned col_tiles, uint32_t src_bytes, uint32_t panel_bytes,
-                          uint32_t plan_bytes, typename Tag::type* __restrict__ out) {
+                          uint32_t plan_bytes, const uint32_t* __restrict__ item_at,
+                          typename Tag::type* __restrict__ out) {
     using C = StreamCfg<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
     using T = typename Tag::type;
     constexpr int S = C::S, kSlabBytes = C::SLAB, kChunks = CH;
@@ -130,7 +131,6 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
 
     const unsigned total_items = row_tiles * col_tiles;
     const unsigned G = gridDim.x;
-    const unsigned dt = G / col_tiles, dct = G % col_tiles;     // item -> (row tile, column tile) increments
     const int slabs = (K + C::SK - 1) / C::SK;
     const uint32_t row_bytes = (uint32_t)K * sizeof(T);
     const bool ragged = (row_bytes % kSlabBytes) != 0;
@@ -138,9 +138,15 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     // Workgroups are dealt round-robin to the 8 XCDs.  Give the workgroups of one XCD neighboring items in every
     // round (first items (g % 8) * G/8 + g / 8), so that tiles which gather from the same region share an L2.
     const unsigned first_item = G % kXcds == 0 ? (blockIdx.x % kXcds) * (G / kXcds) + blockIdx.x / kXcds : blockIdx.x;
-    // Items are walked from the LAST tile down: in the mask-sorted order the late tiles carry the most offsets, so the
-    // incomplete final round (total_items % G workgroups get one item more) is made of the cheapest tiles.
-    const unsigned first_rev = total_items - 1 - first_item;
+    // A workgroup takes the positions first_item, first_item + G, ... of the item sequence.  Which (row tile, column
+    // tile) sits at a position is the caller's choice (item_at: a permutation of the items, made so that the workgroups'
+    // loads come out even); without one, items are walked from the LAST tile down: in the mask-sorted order the late
+    // tiles carry the most offsets, so the incomplete final round is made of the cheapest tiles.
+    auto locate = [&](unsigned position, unsigned& t, unsigned& ct) {
+        const unsigned item = item_at != nullptr ? item_at[position] : total_items - 1 - position;
+        t = item / col_tiles;
+        ct = item - t * col_tiles;
+    };
 
     const rsrc_t src_rs = make_rsrc(src, src_bytes);
     const rsrc_t panel_rs = make_rsrc(panel, panel_bytes);
@@ -172,7 +178,8 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     // ---- the index stream: walks the plan rows of this workgroup's items, kPlanAhead offsets ahead of the rows ----
     // The offsets of a tile are the set bits of its code (a tile without any owns one all-missing plan row, walked as
     // offset 0), so one scalar load per item feeds the whole walk.
-    unsigned f_it = first_item, f_t = first_rev / col_tiles, f_ct = first_rev % col_tiles;
+    unsigned f_it = first_item, f_t, f_ct;
+    locate(f_it, f_t, f_ct);
     bool f_live = true;
     int f_pos = plan_seg[f_t], f_ring = 0;
     uint32_t f_code = (uint32_t)tile_code[f_t];
@@ -203,12 +210,7 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
             f_it += G;
             f_live = f_it < total_items;
             if (f_live) {
-                f_t -= dt;
-                if (f_ct < dct) {
-                    f_ct += col_tiles;
-                    --f_t;
-                }
-                f_ct -= dct;
+                locate(f_it, f_t, f_ct);
                 f_pos = plan_seg[f_t];
                 f_code = (uint32_t)tile_code[f_t];
                 f_code = f_code ? f_code : 1u;
@@ -321,19 +323,15 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
         unsigned it, t, ct;
         int slots;
     };
-    Item cur_item{first_item, first_rev / col_tiles, first_rev % col_tiles, 0};
+    Item cur_item{first_item, 0, 0, 0};
+    locate(cur_item.it, cur_item.t, cur_item.ct);
     cur_item.slots = __popc((uint32_t)tile_code[cur_item.t]);
-    auto following = [&](const Item& c, Item& nx) -> bool {     // the item G further on; false past the end
+    auto following = [&](const Item& c, Item& nx) -> bool {     // the item G positions further on; false past the end
         nx.it = c.it + G;
-        nx.t = c.t - dt;
-        nx.ct = c.ct;
-        if (nx.ct < dct) {
-            nx.ct += col_tiles;
-            --nx.t;
-        }
-        nx.ct -= dct;
+        nx.t = nx.ct = 0;
         nx.slots = 0;
         if (nx.it >= total_items) return false;
+        locate(nx.it, nx.t, nx.ct);
         nx.slots = __popc((uint32_t)tile_code[nx.t]);
         return true;
     };
@@ -486,10 +484,33 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
     wait_vmcnt<0>();
 }
 
+// As many workgroups as the CUs hold at once (the narrow tiles leave room for two per CU: their steps are short, and a
+// second stream fills the time the first spends at its barriers).
+template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int CH>
+int resident_groups(size_t lds, int* groups) {
+    using C = StreamCfg<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
+    auto kern = gather_gemm_stream_kernel<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
+    static thread_local int per_cu = 0;          // per thread and instantiation, for the LDS size it was asked with
+    static thread_local size_t per_cu_lds = 0;
+    int dev = 0, cus = 0;
+    FGX_CHECK_HIP(hipGetDevice(&dev));
+    FGX_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    if (per_cu == 0 || per_cu_lds != lds) {
+        if (lds > 64 * 1024) FGX_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        int q = 1;
+        FGX_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&q, (const void*)kern, C::NT, lds));
+        per_cu = q < 1 ? 1 : (q > 2 ? 2 : q);
+        per_cu_lds = lds;
+    }
+    *groups = (cus > 0 ? cus : 256) * per_cu;
+    return FGX_OK;
+}
+
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int CH>
 int launch_stream(const void* src, const void* panel, const void* bias, const int64_t* order, const int32_t* plan_seg,
                   const int32_t* tile_code, const uint32_t* plan_idx, const uint32_t* plan_band, size_t plan_rows, size_t n,
-                  size_t n_src, int K, int cols, int cols_pad, size_t panel_bytes, int max_groups, void* out, hipStream_t s) {
+                  size_t n_src, int K, int cols, int cols_pad, size_t panel_bytes, const uint32_t* item_at, int max_groups,
+                  void* out, hipStream_t s) {
     using C = StreamCfg<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
     using T = typename Tag::type;
     auto kern = gather_gemm_stream_kernel<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
@@ -506,26 +527,14 @@ int launch_stream(const void* src, const void* panel, const void* bias, const in
     const unsigned row_tiles = cdiv(n, BM), col_tiles = cdiv(cols, BN);
     const size_t total = (size_t)row_tiles * col_tiles;
     if (max_groups <= 0) {
-        // as many resident workgroups as the CUs hold (the narrow tiles leave room for two per CU: their steps are
-        // short, and a second stream fills the time the first spends at its barriers)
-        static thread_local int per_cu = 0;          // per thread and instantiation, for the LDS size it was asked with
-        static thread_local size_t per_cu_lds = 0;
-        int dev = 0, cus = 0;
-        FGX_CHECK_HIP(hipGetDevice(&dev));
-        FGX_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-        if (per_cu == 0 || per_cu_lds != lds) {
-            int q = 1;
-            FGX_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&q, (const void*)kern, C::NT, lds));
-            per_cu = q < 1 ? 1 : (q > 2 ? 2 : q);
-            per_cu_lds = lds;
-        }
-        max_groups = (cus > 0 ? cus : 256) * per_cu;
+        int rc = resident_groups<Tag, BM, BN, WAVES_M, WAVES_N, CH>(lds, &max_groups);
+        if (rc != FGX_OK) return rc;
     }
     unsigned groups = (unsigned)(total < (size_t)max_groups ? total : (size_t)max_groups);
     kern<<<groups, C::NT, lds, s>>>((const T*)src, (const T*)panel, (const T*)bias, order, plan_seg, tile_code, plan_idx,
                                     plan_band, (uint32_t)n, K, cols, cols_pad, row_tiles, col_tiles,
                                     (uint32_t)(n_src * (size_t)K * sizeof(T)), (uint32_t)panel_bytes,
-                                    (uint32_t)(plan_rows * BM * 4), (T*)out);
+                                    (uint32_t)(plan_rows * BM * 4), item_at, (T*)out);
     FGX_CHECK_LAUNCH("fgx_conv_gather_gemm_stream");
     return FGX_OK;
 }
@@ -534,11 +543,11 @@ template <typename Tag>
 int dispatch_stream(int tile_rows, int tile_cols, int slab_bytes, const void* src, const void* panel, const void* bias,
                     const int64_t* order, const int32_t* plan_seg, const int32_t* tile_code, const uint32_t* plan_idx,
                     const uint32_t* plan_band, size_t plan_rows, size_t n, size_t n_src, int K, int cols, int cols_pad,
-                    size_t panel_bytes, int max_groups, void* out, hipStream_t s) {
+                    size_t panel_bytes, const uint32_t* item_at, int max_groups, void* out, hipStream_t s) {
 #define FGX_STREAM_TILE(BM, BN, WMv, WNv, CHv)                                                                          \
     if (tile_rows == BM && tile_cols == BN && slab_bytes == CHv * 16)                                                   \
         return launch_stream<Tag, BM, BN, WMv, WNv, CHv>(src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band,  \
-                                                         plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, max_groups, out, s);
+                                                         plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, out, s);
     FGX_STREAM_TILE(256, 128, 4, 2, 8)
     FGX_STREAM_TILE(256, 64, 4, 2, 8)
     FGX_STREAM_TILE(256, 128, 4, 2, 4)      // 64-byte K-slabs: rows shorter than 128 bytes
@@ -558,8 +567,8 @@ extern "C" int fgx_conv_gather_gemm_stream(int dtype, const void* src, const voi
                                            const int64_t* order, const int32_t* tile_code, const int32_t* plan_seg,
                                            const uint32_t* plan_idx, const uint32_t* plan_band, size_t plan_rows, size_t n,
                                            size_t n_src, int K, int cols, int V,
-                                           int tile_rows, int tile_cols, int slab_bytes, int max_groups, void* out,
-                                           fgx_stream_t stream) {
+                                           int tile_rows, int tile_cols, int slab_bytes, const uint32_t* item_at,
+                                           int max_groups, void* out, fgx_stream_t stream) {
     FGX_CHECK_ARG(dtype == FGX_F16 || dtype == FGX_BF16 || dtype == FGX_F32, "fgx_conv_gather_gemm_stream: unknown dtype %d", dtype);
     FGX_CHECK_ARG(K > 0 && cols > 0 && V >= 1 && V <= 32, "fgx_conv_gather_gemm_stream: bad shape K=%d cols=%d V=%d", K, cols, V);
     if (n == 0) return FGX_OK;
@@ -581,8 +590,31 @@ extern "C" int fgx_conv_gather_gemm_stream(int dtype, const void* src, const voi
     }
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
-        case FGX_F16: return dispatch_stream<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, max_groups, out, s);
-        case FGX_BF16: return dispatch_stream<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, max_groups, out, s);
-        default: return dispatch_stream<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, max_groups, out, s);
+        case FGX_F16: return dispatch_stream<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, out, s);
+        case FGX_BF16: return dispatch_stream<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, out, s);
+        default: return dispatch_stream<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, out, s);
     }
+}
+
+extern "C" int fgx_conv_gather_gemm_stream_groups(int dtype, int cols, int tile_rows, int tile_cols, int slab_bytes,
+                                                  int* groups) {
+    FGX_CHECK_ARG(dtype == FGX_F16 || dtype == FGX_BF16 || dtype == FGX_F32, "fgx_conv_gather_gemm_stream_groups: unknown dtype %d", dtype);
+    FGX_CHECK_ARG(groups != nullptr && cols > 0 && tile_cols > 0, "fgx_conv_gather_gemm_stream_groups: bad argument");
+    const size_t bias_bytes = align_up((size_t)cols, (size_t)tile_cols) * sizeof(float);
+#define FGX_STREAM_TILE(TAG, BM, BN, WMv, WNv, CHv)                                              \
+    if (tile_rows == BM && tile_cols == BN && slab_bytes == CHv * 16)                            \
+        return resident_groups<TAG, BM, BN, WMv, WNv, CHv>(StreamCfg<TAG, BM, BN, WMv, WNv, CHv>::fixed_lds + bias_bytes, groups);
+#define FGX_STREAM_TILES(TAG)            \
+    FGX_STREAM_TILE(TAG, 256, 128, 4, 2, 8) \
+    FGX_STREAM_TILE(TAG, 256, 64, 4, 2, 8)  \
+    FGX_STREAM_TILE(TAG, 256, 128, 4, 2, 4) \
+    FGX_STREAM_TILE(TAG, 256, 64, 4, 2, 4)  \
+    FGX_STREAM_TILE(TAG, 256, 32, 8, 1, 4)
+    if (dtype == FGX_F16) { FGX_STREAM_TILES(F16) }
+    else if (dtype == FGX_BF16) { FGX_STREAM_TILES(BF16) }
+    else { FGX_STREAM_TILES(F32) }
+#undef FGX_STREAM_TILES
+#undef FGX_STREAM_TILE
+    set_error("fgx_conv_gather_gemm_stream_groups: no kernel for tile %dx%d with %d-byte slabs", tile_rows, tile_cols, slab_bytes);
+    return FGX_ERR_UNSUPPORTED;
 }

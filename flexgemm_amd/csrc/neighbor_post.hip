@@ -337,6 +337,97 @@ __global__ void __launch_bounds__(kBlock) plan_fill_kernel(const uint32_t* __res
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Item order of the streaming GEMM (fgx_gather_item_order): one workgroup, no host round trip.
+// ---------------------------------------------------------------------------------------------------------------
+// Items (row tile * col_tiles + column tile) cost about max(popcount(tile_code), 1) offsets each.  Workgroup slot q of
+// `groups` works through the positions q, q + groups, ... of the sequence written here.  Step 1 sorts the items by
+// cost, most expensive first (stable counting sort over the 33 possible popcounts: per-thread counts of a contiguous
+// chunk, one scan, one placement pass).  Step 2 deals them round by round: the incomplete last round takes the
+// cheapest items, every full round gives its most expensive item to the least loaded slot (rank of each slot's load by
+// counting).  Everything is deterministic.
+constexpr int kOrderThreads = 1024;     // also the largest number of slots
+constexpr int kCostBins = 33;
+
+__global__ void __launch_bounds__(kOrderThreads) item_order_kernel(const int32_t* __restrict__ tile_code, unsigned num_tiles,
+                                                                   unsigned col_tiles, unsigned slabs, unsigned groups,
+                                                                   uint32_t* __restrict__ sorted, uint32_t* __restrict__ item_at) {
+    __shared__ uint32_t count[kCostBins][kOrderThreads / 4];     // [bin][chunk owner]; 256 owners
+    __shared__ uint32_t bin_start[kCostBins];
+    __shared__ uint32_t load[kOrderThreads];
+    constexpr unsigned kOwners = kOrderThreads / 4;
+    const unsigned tid = threadIdx.x;
+    const unsigned total = num_tiles * col_tiles;
+    auto bin_of = [&](unsigned item) -> unsigned {                // bin 0 = most expensive
+        const unsigned pc = (unsigned)__popc((uint32_t)tile_code[item / col_tiles]);
+        return 32u - pc;
+    };
+    // ---- step 1: stable counting sort, cost descending ----
+    for (unsigned i = tid; i < kCostBins * kOwners; i += kOrderThreads) (&count[0][0])[i] = 0u;
+    __syncthreads();
+    const unsigned chunk = (total + kOwners - 1) / kOwners;
+    if (tid < kOwners) {
+        const unsigned lo = tid * chunk, hi = lo + chunk < total ? lo + chunk : total;
+        for (unsigned i = lo; i < hi; ++i) ++count[bin_of(i)][tid];
+    }
+    __syncthreads();
+    if (tid < kCostBins) {                                        // per bin: exclusive prefix over the owners, total left in bin_start
+        uint32_t run = 0;
+        for (unsigned o = 0; o < kOwners; ++o) {
+            const uint32_t c = count[tid][o];
+            count[tid][o] = run;
+            run += c;
+        }
+        bin_start[tid] = run;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t run = 0;
+        for (int b = 0; b < kCostBins; ++b) {
+            const uint32_t c = bin_start[b];
+            bin_start[b] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+    if (tid < kOwners) {
+        const unsigned lo = tid * chunk, hi = lo + chunk < total ? lo + chunk : total;
+        for (unsigned i = lo; i < hi; ++i) {
+            const unsigned b = bin_of(i);
+            sorted[bin_start[b] + count[b][tid]++] = i;
+        }
+    }
+    __threadfence_block();
+    __syncthreads();
+    // ---- step 2: deal the rounds ----
+    const unsigned rounds = total / groups, rem = total % groups;
+    auto cost_of = [&](unsigned item) -> uint32_t {
+        const unsigned pc = (unsigned)__popc((uint32_t)tile_code[item / col_tiles]);
+        return (pc ? pc : 1u) * slabs + 3u;
+    };
+    uint32_t mine = 0;
+    if (tid < rem) {                                              // cheapest items: the positions of the last round
+        const unsigned item = sorted[total - rem + tid];
+        item_at[rounds * groups + tid] = item;
+        mine = cost_of(item);
+    }
+    for (unsigned r = 0; r < rounds; ++r) {
+        if (tid < groups) load[tid] = mine;
+        __syncthreads();
+        if (tid < groups) {
+            unsigned rank = 0;                                    // slots with a smaller load come first, ties by slot number
+            for (unsigned q = 0; q < groups; ++q) {
+                const uint32_t other = load[q];
+                rank += (other < mine || (other == mine && q < tid)) ? 1u : 0u;
+            }
+            const unsigned item = sorted[r * groups + rank];      // rank 0 = least loaded slot <- most expensive item
+            item_at[r * groups + tid] = item;
+            mine += cost_of(item);
+        }
+        __syncthreads();
+    }
+}
+
 size_t scan_temp_bytes(size_t count) {
     size_t bytes = 0;
     (void)rocprim::exclusive_scan(nullptr, bytes, (const uint32_t*)nullptr, (uint32_t*)nullptr, 0u, count ? count : 1,
@@ -560,6 +651,29 @@ int fgx_gather_plan_fill(const uint32_t* map, const int64_t* order, const int32_
     plan_fill_kernel<<<(unsigned)num_tiles, kBlock, 0, (hipStream_t)stream>>>(map, order, tile_code, plan_seg, n, V, tile_rows,
                                                                               plan_idx, plan_band);
     FGX_CHECK_LAUNCH("fgx_gather_plan_fill");
+    return FGX_OK;
+}
+
+size_t fgx_gather_item_order_workspace_bytes(size_t num_tiles, int col_tiles) {
+    if (col_tiles < 1) return 0;
+    return align_up((num_tiles * (size_t)col_tiles + 1) * sizeof(uint32_t), 256);
+}
+
+int fgx_gather_item_order(const int32_t* tile_code, size_t num_tiles, int col_tiles, int slabs, int groups, void* workspace,
+                          size_t workspace_bytes, uint32_t* item_at, fgx_stream_t stream) {
+    FGX_CHECK_ARG(col_tiles >= 1 && slabs >= 1, "fgx_gather_item_order: bad shape col_tiles=%d slabs=%d", col_tiles, slabs);
+    FGX_CHECK_ARG(groups >= 1 && groups <= kOrderThreads, "fgx_gather_item_order: groups must be in [1, %d], got %d", kOrderThreads,
+                  groups);
+    const size_t total = num_tiles * (size_t)col_tiles;
+    if (total == 0) return FGX_OK;
+    FGX_CHECK_ARG(total < 0x7FFFFFFFull, "fgx_gather_item_order: too many items");
+    FGX_CHECK_ARG(tile_code && workspace && item_at, "fgx_gather_item_order: null buffer");
+    FGX_CHECK_ARG(workspace_bytes >= fgx_gather_item_order_workspace_bytes(num_tiles, col_tiles),
+                  "fgx_gather_item_order: workspace of %zu bytes is too small", workspace_bytes);
+    FGX_CHECK_ARG(((uintptr_t)workspace & 255) == 0, "fgx_gather_item_order: workspace must be 256-byte aligned");
+    item_order_kernel<<<1, kOrderThreads, 0, (hipStream_t)stream>>>(tile_code, (unsigned)num_tiles, (unsigned)col_tiles,
+                                                                    (unsigned)slabs, (unsigned)groups, (uint32_t*)workspace, item_at);
+    FGX_CHECK_LAUNCH("fgx_gather_item_order");
     return FGX_OK;
 }
 

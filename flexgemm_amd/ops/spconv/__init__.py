@@ -45,6 +45,11 @@ SERIALIZATION_MODE = SerializationMode.BXYZ
 # questions on (131 072 voxels of a 3x3x3 kernel).
 NEIGHBOR_MAP_BUILDER = "auto"
 SORT_BUILDER_MIN_PROBES = 27 * 131072
+# How the streaming GEMM's tiles are dealt to its persistent workgroups: "balanced" (by cost, every round of tiles dealt
+# expensive-first to the least loaded workgroup), "default" (the kernel's own round-robin over the tile list) or "auto"
+# (balanced, except for the locality order of short-row layers, whose neighboring tiles are meant to share an XCD).
+# The result does not depend on it.
+GEMM_ITEM_ORDER = "auto"
 
 
 def set_neighbor_map_builder(builder: str):

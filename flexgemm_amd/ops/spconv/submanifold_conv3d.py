@@ -129,7 +129,34 @@ class SubMConv3dNeighborCache:
                                                  C.c_int(v), C.c_int(block_size), nat.ptr(plan_idx), nat.ptr(plan_band),
                                                  nat.stream()))
             setattr(self, key, (seg, plan_idx, plan_band))
-        return (order, code) + getattr(self, key)
+        return (order, code) + getattr(self, key) + (key,)
+
+    def _item_order(self, plan_key: str, code: torch.Tensor, col_tiles: int, groups: int, slabs: int):
+        """uint32 device tensor for fgx_conv_gather_gemm_stream's item_at (or None): the tiles dealt to the persistent
+        workgroups by cost, built on the device (no read-back) once per plan and shape and kept with the cache."""
+        mode = spconv.GEMM_ITEM_ORDER
+        if mode == "auto":
+            # the locality order of short-row layers lives on neighboring tiles sharing an XCD (dealing them by cost
+            # alone: 0.32 -> 0.42 ms per launch at C = 32); elsewhere balance wins (-6 % at C = 256, -8 % at C = 1024)
+            mode = "default" if plan_key.startswith("_plan_t_") else "balanced"
+        nb = code.shape[0]
+        # with fewer than four rounds of items there is little to even out (and the round-by-round dealing is not
+        # reliably better than the kernel's own order)
+        if mode == "default" or nb * col_tiles < 4 * groups or groups > 1024:
+            return None
+        if mode != "balanced":
+            raise ValueError(f"unknown GEMM_ITEM_ORDER {spconv.GEMM_ITEM_ORDER!r}; expected 'auto', 'balanced' or 'default'")
+        key = f"_items_{plan_key}_{col_tiles}_{groups}_{slabs}"
+        if not hasattr(self, key):
+            dev = code.device
+            item_at = torch.empty((nb * col_tiles,), dtype=torch.int32, device=dev)
+            with torch.cuda.device(dev):
+                L = nat.lib()
+                ws = nat.workspace(L.fgx_gather_item_order_workspace_bytes(nat.sz(nb), C.c_int(col_tiles)), dev)
+                nat.check(L.fgx_gather_item_order(nat.ptr(code), nat.sz(nb), C.c_int(col_tiles), C.c_int(slabs), C.c_int(groups),
+                                                  nat.ptr(ws), nat.sz(ws.numel()), nat.ptr(item_at), nat.stream()))
+            setattr(self, key, item_at)
+        return getattr(self, key)
 
     def compute_kernel_idx(self, block_size: int):
         """Fill `valid_kernel_{B}` / `valid_kernel_seg_{B}` (reference: submanifold_conv3d.py:20-23,
@@ -359,14 +386,20 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
         nat.check(L.fgx_pack_weight(C.c_int(code), C.c_int(mode), nat.ptr(weight_cvk), C.c_int(ci), C.c_int(co), C.c_int(v),
                                     C.c_int(sched.slab_bytes), C.c_int(sched.tile_cols), nat.ptr(panel), nat.stream()))
         if sched.stream and _stream_fits(n, n_src, k * src.element_size()):
-            order, tile_code, plan_seg, plan_idx, plan_band = cache._gather_plan(sched.tile_rows, private, dense=not masked)
+            order, tile_code, plan_seg, plan_idx, plan_band, plan_key = cache._gather_plan(sched.tile_rows, private,
+                                                                                           dense=not masked)
+            groups = C.c_int(0)
+            nat.check(L.fgx_conv_gather_gemm_stream_groups(C.c_int(code), C.c_int(cols), C.c_int(sched.tile_rows),
+                                                           C.c_int(sched.tile_cols), C.c_int(sched.slab_bytes), C.byref(groups)))
+            item_at = cache._item_order(plan_key, tile_code, -(-cols // sched.tile_cols), groups.value,
+                                        -(-(k * src.element_size()) // sched.slab_bytes))
             nat.mark(name, "start")
             nat.check(L.fgx_conv_gather_gemm_stream(
                 C.c_int(code), nat.ptr(src), nat.ptr(panel), nat.ptr(bias), nat.ptr(order), nat.ptr(tile_code),
                 nat.ptr(plan_seg), nat.ptr(plan_idx), nat.ptr(plan_band), nat.sz(plan_idx.shape[0]), nat.sz(n), nat.sz(n_src),
                 C.c_int(k), C.c_int(cols), C.c_int(v),
-                C.c_int(sched.tile_rows), C.c_int(sched.tile_cols), C.c_int(sched.slab_bytes), C.c_int(0), nat.ptr(out),
-                nat.stream()))
+                C.c_int(sched.tile_rows), C.c_int(sched.tile_cols), C.c_int(sched.slab_bytes), nat.ptr(item_at),
+                C.c_int(groups.value), nat.ptr(out), nat.stream()))
             nat.mark(name, "stop")
             return out
         if masked:

@@ -219,13 +219,29 @@ int fgx_gather_plan_fill(const uint32_t* map, const int64_t* order, const int32_
  * present) lets the kernel skip the loads and products of 32-row bands without a neighbor at an offset.
  * `n` counts the output rows (rows of the map behind the plan), `n_src` the rows of `src`; they differ for the
  * generic sparse convolution only.
+ * `item_at` (device, may be NULL): a permutation of the items 0 .. row_tiles * col_tiles - 1 (item = row tile *
+ * col_tiles + column tile, row_tiles = ceil(n / tile_rows), col_tiles = ceil(cols / tile_cols)).  Workgroup w of G
+ * works through the positions p(w), p(w) + G, ... of that sequence, p(w) = (w % 8) * (G / 8) + w / 8 when 8 divides
+ * G, else w: a caller that knows the tiles' costs (offsets per tile = popcount of tile_code) orders the items so that
+ * the workgroups' sums come out even.  NULL: last tile first.  The result does not depend on it.
+ * fgx_conv_gather_gemm_stream_groups tells G for max_groups <= 0.
  * Replaces: the same reference kernels as fgx_conv_gather_gemm. */
 int fgx_conv_gather_gemm_stream(int dtype, const void* src, const void* panel, const void* bias,
                                 const int64_t* order, const int32_t* tile_code, const int32_t* plan_seg,
                                 const uint32_t* plan_idx, const uint32_t* plan_band, size_t plan_rows, size_t n,
                                 size_t n_src, int K, int cols, int V,
-                                int tile_rows, int tile_cols, int slab_bytes, int max_groups, void* out,
-                                fgx_stream_t stream);
+                                int tile_rows, int tile_cols, int slab_bytes, const uint32_t* item_at,
+                                int max_groups, void* out, fgx_stream_t stream);
+int fgx_conv_gather_gemm_stream_groups(int dtype, int cols, int tile_rows, int tile_cols, int slab_bytes, int* groups);
+
+/* item_at for fgx_conv_gather_gemm_stream, made on the device from the tile codes: items sorted by cost (offsets per
+ * row tile x `slabs` K-slabs + an epilogue), the incomplete last round of `groups` positions filled with the cheapest,
+ * every full round dealt most-expensive-item to least-loaded-slot.  One workgroup, deterministic, no read-back;
+ * groups <= 1024.  workspace: fgx_gather_item_order_workspace_bytes bytes, 256-byte aligned; item_at: uint32 per item.
+ * No counterpart in the reference (Triton's grid is one program per tile). */
+size_t fgx_gather_item_order_workspace_bytes(size_t num_tiles, int col_tiles);
+int fgx_gather_item_order(const int32_t* tile_code, size_t num_tiles, int col_tiles, int slabs, int groups,
+                          void* workspace, size_t workspace_bytes, uint32_t* item_at, fgx_stream_t stream);
 
 /* grad_weight[co, v, ci] = sum over pairs k in [seg[v], seg[v+1]) of grad_out[sig_o[k], co] * feats[sig_i[k], ci].
  * seg_host is the HOST copy of valid_signal_seg (V+1 entries); sig_o must ascend inside every segment (it does

@@ -84,7 +84,7 @@ def test_argument_errors_map_to_exceptions(library):
                                    None, None, None))
     with pytest.raises(ValueError):   # the streaming GEMM checks its arguments before touching the device
         nat.check(L.fgx_conv_gather_gemm_stream(0, None, None, None, None, None, None, None, None, ctypes.c_size_t(0),
-                                                ctypes.c_size_t(10), ctypes.c_size_t(10), 128, 128, 27, 256, 128, 128, 0, None, None))
+                                                ctypes.c_size_t(10), ctypes.c_size_t(10), 128, 128, 27, 256, 128, 128, None, 0, None, None))
     assert b"null buffer" in L.fgx_last_error()
 
 

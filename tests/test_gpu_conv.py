@@ -283,6 +283,65 @@ def test_streaming_kernel_equals_tiled_kernel_bitwise(gpu_device):
     assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
 
 
+def test_item_order_changes_nothing(gpu_device):
+    """How the streaming GEMM's tiles are dealt to its workgroups is a scheduling choice: every order gives the same
+    bits (more items than resident workgroups, two column tiles per row tile)."""
+    import flex_gemm
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    res, ci, co = 192, 64, 256
+    coords_np = reference_test_shell(res)
+    assert -(-len(coords_np) // 256) * 2 >= 4 * 256          # enough rounds of items for the dealt order to be used
+    _say(f"item orders res={res} n={len(coords_np)}")
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    shape = torch.Size([1, ci, res, res, res])
+    f, w, b, g = _case(coords_np, ci, co, torch.float16, 41)
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+    outs = {}
+    try:
+        for mode in ("default", "balanced", "auto"):
+            flex_gemm.ops.spconv.GEMM_ITEM_ORDER = mode
+            with _force_schedule(tile_rows=256, tile_cols=128, slab_bytes=128, splitk=1, stream=1):
+                outs[mode] = impl._gather_gemm(f.to(gpu_device), w.to(gpu_device).reshape(co, 27, ci), b.to(gpu_device), cache, 0,
+                                               False).cpu()
+    finally:
+        flex_gemm.ops.spconv.GEMM_ITEM_ORDER = "auto"
+    assert any(k.startswith("_items_") for k in vars(cache))
+    for mode in ("balanced", "auto"):
+        assert torch.equal(outs[mode], outs["default"]), mode
+    rows = torch.from_numpy(np.random.default_rng(3).choice(len(coords_np), 4000, replace=False))
+    ref_rows = eg.forward(f.double(), cache.neighbor_map.cpu().view(torch.int32)[rows], w.double(), b.double())
+    assert eg.max_rel_err(outs["default"][rows], ref_rows) <= 1e-2          # fp16 tolerance
+
+
+def _load_spread(item_at, codes, col_tiles, groups, slabs):
+    """busiest workgroup / mean, with the cost model of the ordering kernel"""
+    offsets = np.array([bin(int(c)).count("1") for c in codes])
+    cost = np.maximum(offsets, 1) * slabs + 3
+    load = np.zeros(groups)
+    np.add.at(load, np.arange(len(item_at)) % groups, cost[np.asarray(item_at) // col_tiles])
+    return load.max() / load.mean()
+
+
+def test_item_order_evens_out_the_benchmark_shell(gpu_device):
+    """At the res-512 benchmark shape (2615 tiles of 256 rows for 256 workgroups) the kernel's own round-robin leaves the
+    busiest workgroup ~17 % above the mean; the dealt order brings it within 3 % (within 10 % when there are only five rounds of items)."""
+    from flexgemm_amd.workloads import shell_coords
+    res = 512
+    coords = torch.from_numpy(shell_coords(res)).to(gpu_device)
+    _say(f"item order at res {res}, n={coords.shape[0]}")
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, torch.Size([1, 128, res, res, res]), (3, 3, 3), (1, 1, 1), False)
+    _, code, _, _, _, key = cache._gather_plan(256, False)
+    for col_tiles, groups, slabs in ((1, 256, 2), (2, 256, 4), (1, 512, 1)):
+        item_at = cache._item_order(key, code, col_tiles, groups, slabs).cpu().numpy().astype(np.int64)
+        codes = code.cpu().numpy().view(np.uint32)
+        total = col_tiles * len(codes)
+        assert sorted(item_at.tolist()) == list(range(total))
+        own = _load_spread(np.arange(total - 1, -1, -1), codes, col_tiles, groups, slabs)
+        dealt = _load_spread(item_at, codes, col_tiles, groups, slabs)
+        _say(f"  col_tiles={col_tiles} groups={groups}: busiest/mean {own:.3f} -> {dealt:.3f}")
+        assert dealt < 1.12 and dealt < own - 0.05
+
+
 def test_gather_plan_band_masks(gpu_device):
     """plan_band bit b of a plan row says whether rows [32 b, 32 b + 32) of that row's index column hold a neighbor;
     the shell with scattered isolated voxels gives full, partial and (for the tail tile) sparse masks."""
@@ -298,7 +357,7 @@ def test_gather_plan_band_masks(gpu_device):
     shape = torch.Size([2, 8, res, res, res])
     cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
     for dense in (False, True):
-        order, code, seg, plan_idx, plan_band = cache._gather_plan(256, False, dense=dense)
+        order, code, seg, plan_idx, plan_band, _ = cache._gather_plan(256, False, dense=dense)
         torch.cuda.synchronize()
         idx = plan_idx.cpu().numpy()
         got = plan_band.cpu().numpy()
