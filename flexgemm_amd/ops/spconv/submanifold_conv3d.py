@@ -137,8 +137,10 @@ class SubMConv3dNeighborCache:
         mode = spconv.GEMM_ITEM_ORDER
         if mode == "auto":
             # the locality order of short-row layers lives on neighboring tiles sharing an XCD (dealing them by cost
-            # alone: 0.32 -> 0.42 ms per launch at C = 32); elsewhere balance wins (-6 % at C = 256, -8 % at C = 1024)
-            mode = "default" if plan_key.startswith("_plan_t_") else "balanced"
+            # alone: 0.32 -> 0.42 ms per launch at C = 32); with rows of 512 bytes and more balance wins (-6 % per
+            # launch at C = 256, -8 % at C = 1024); in between (-1 % at C = 128) it does not pay for the ordering
+            # kernel, which takes ~3 us per round of items
+            mode = "balanced" if slabs >= 4 and not plan_key.startswith("_plan_t_") else "default"
         nb = code.shape[0]
         # with fewer than four rounds of items there is little to even out (and the round-by-round dealing is not
         # reliably better than the kernel's own order)
