@@ -27,6 +27,8 @@
 // fp32 partial product; a second kernel adds an offset's partials in block order (deterministic) and
 // casts to the output type.  The per-(offset, block) pair ranges are found by a small binary-search
 // kernel over sig_o.
+#include <type_traits>
+
 #include "fgx_common.h"
 
 namespace fgx {
@@ -146,6 +148,12 @@ template <> __device__ __forceinline__ void mma16<BF16>(f32x16& acc, const i16x8
     acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
 }
 template <> __device__ __forceinline__ void mma16<F32>(f32x16&, const i16x8&, const i16x8&) {}
+
+// eight ones in the 16-bit type, as a fragment
+template <typename Tag> __device__ __forceinline__ i16x8 ones16() {
+    constexpr short one = sizeof(typename Tag::type) == 2 && __is_same(typename Tag::type, _Float16) ? (short)0x3C00 : (short)0x3F80;
+    return i16x8{one, one, one, one, one, one, one, one};
+}
 
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N>
 __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N)
@@ -441,7 +449,8 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
                     const uint32_t* __restrict__ sig_i, const uint32_t* __restrict__ sig_o,
                     const uint32_t* __restrict__ bounds, int V, int Ci, int Co, unsigned nb, unsigned co_tiles,
                     unsigned ci_tiles, uint32_t n_pairs, uint32_t gout_bytes, uint32_t feats_bytes,
-                    float* __restrict__ partial, typename Tag::type* __restrict__ direct) {
+                    float* __restrict__ partial, typename Tag::type* __restrict__ direct,
+                    float* __restrict__ bias_partial, int bias_offset) {
     using C = WStreamCfg<Tag, BM, BN>;
     constexpr int ES = C::ES, S = C::S, P = C::P;
 
@@ -681,51 +690,68 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
             for (int j = 0; j < C::TN; ++j)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-        for (int s = 0; s < nsteps; ++s) {
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_s_barrier();           // the loaders saw this step's rows land
-            asm volatile("" ::: "memory");
-            const unsigned char* cur = ring + (step & (S - 1)) * C::STAGE_BYTES;
-            ++step;
-            // Transposing read: in a 16-lane group, lane s supplies the address of 4 adjacent channels of pair row
-            // (s / 4) and receives the 4 pair values of channel (group base + s).  Lanes 0-15 / 16-31 cover fragment
-            // rows 0-15 / 16-31, the two wave halves take pair rows [0, 8) / [8, 16) of the k-block.  The reads of
-            // k-block kk+1 are in flight while k-block kk is multiplied.
-            i16x4 fr[2][RK];
-            auto read_block = [&](int kl, i16x4 (&dst)[RK]) {
-                const int kk = kk0 + kl;
-                const unsigned char* base = cur + kk * 16 * C::ROWB_A;      // ROWB_A == ROWB_B is not assumed below
+        // Column sums of grad_out (the bias gradient) ride along with the offset whose pairs hold every output row once:
+        // the grad_out fragments are multiplied by a fragment of ones as well, so every column of bacc is the sum.  Only
+        // the wavefronts of the first column of wave tiles do it, for the first Ci-tile.
+        const bool do_bias = bias_partial != nullptr && (int)v == bias_offset && wave_n == 0 && tile < co_tiles;
+        f32x16 bacc[C::TM];
 #pragma unroll
-                for (int i = 0; i < C::TM; ++i) {
-                    dst[i * 2] = lds_read_tr16(base + a_off[i][0]);
-                    dst[i * 2 + 1] = lds_read_tr16(base + a_off[i][1]);
-                }
-                const unsigned char* base_b = cur + kk * 16 * C::ROWB_B;
+        for (int i = 0; i < C::TM; ++i)
 #pragma unroll
-                for (int j = 0; j < C::TN; ++j) {
-                    dst[(C::TM + j) * 2] = lds_read_tr16(base_b + b_off[j][0]);
-                    dst[(C::TM + j) * 2 + 1] = lds_read_tr16(base_b + b_off[j][1]);
-                }
-            };
-            read_block(0, fr[0]);
-#pragma unroll
-            for (int kk = 0; kk < NK; ++kk) {
-                if (kk + 1 < NK) {
-                    read_block(kk + 1, fr[(kk + 1) & 1]);
-                    lds_wait_but<RK>(fr[kk & 1]);
-                } else {
-                    lds_wait_but<0>(fr[kk & 1]);
-                }
-#pragma unroll
-                for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < C::TN; ++j) {
-                        const i16x8 af = __builtin_shufflevector(fr[kk & 1][i * 2], fr[kk & 1][i * 2 + 1], 0, 1, 2, 3, 4, 5, 6, 7);
-                        const i16x8 bf = __builtin_shufflevector(fr[kk & 1][(C::TM + j) * 2], fr[kk & 1][(C::TM + j) * 2 + 1], 0, 1, 2, 3, 4, 5, 6, 7);
-                        mma16<Tag>(acc[i][j], af, bf);
+            for (int e = 0; e < 16; ++e) bacc[i][e] = 0.f;
+        // The steps of an item, in two compiled forms: the one with the extra products for the bias gradient runs for
+        // the few items that need it, so the other keeps the register allocation and instruction schedule it had.
+        auto run_steps = [&](auto with_bias) {
+            for (int s = 0; s < nsteps; ++s) {
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_s_barrier();           // the loaders saw this step's rows land
+                asm volatile("" ::: "memory");
+                const unsigned char* cur = ring + (step & (S - 1)) * C::STAGE_BYTES;
+                ++step;
+                // Transposing read: in a 16-lane group, lane s supplies the address of 4 adjacent channels of pair row
+                // (s / 4) and receives the 4 pair values of channel (group base + s).  Lanes 0-15 / 16-31 cover fragment
+                // rows 0-15 / 16-31, the two wave halves take pair rows [0, 8) / [8, 16) of the k-block.  The reads of
+                // k-block kk+1 are in flight while k-block kk is multiplied.
+                i16x4 fr[2][RK];
+                auto read_block = [&](int kl, i16x4 (&dst)[RK]) {
+                    const int kk = kk0 + kl;
+                    const unsigned char* base = cur + kk * 16 * C::ROWB_A;      // ROWB_A == ROWB_B is not assumed below
+    #pragma unroll
+                    for (int i = 0; i < C::TM; ++i) {
+                        dst[i * 2] = lds_read_tr16(base + a_off[i][0]);
+                        dst[i * 2 + 1] = lds_read_tr16(base + a_off[i][1]);
                     }
+                    const unsigned char* base_b = cur + kk * 16 * C::ROWB_B;
+    #pragma unroll
+                    for (int j = 0; j < C::TN; ++j) {
+                        dst[(C::TM + j) * 2] = lds_read_tr16(base_b + b_off[j][0]);
+                        dst[(C::TM + j) * 2 + 1] = lds_read_tr16(base_b + b_off[j][1]);
+                    }
+                };
+                read_block(0, fr[0]);
+    #pragma unroll
+                for (int kk = 0; kk < NK; ++kk) {
+                    if (kk + 1 < NK) {
+                        read_block(kk + 1, fr[(kk + 1) & 1]);
+                        lds_wait_but<RK>(fr[kk & 1]);
+                    } else {
+                        lds_wait_but<0>(fr[kk & 1]);
+                    }
+    #pragma unroll
+                    for (int i = 0; i < C::TM; ++i) {
+                        const i16x8 af = __builtin_shufflevector(fr[kk & 1][i * 2], fr[kk & 1][i * 2 + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                        if constexpr (decltype(with_bias)::value) mma16<Tag>(bacc[i], af, ones16<Tag>());
+    #pragma unroll
+                        for (int j = 0; j < C::TN; ++j) {
+                            const i16x8 bf = __builtin_shufflevector(fr[kk & 1][(C::TM + j) * 2], fr[kk & 1][(C::TM + j) * 2 + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                            mma16<Tag>(acc[i][j], af, bf);
+                        }
+                    }
+                }
             }
-        }
+        };
+        if (do_bias) run_steps(std::true_type{});
+        else run_steps(std::false_type{});
         // partial[b][v][co][ci], fp32
         const unsigned co_tile = tile % co_tiles, ci_tile = tile / co_tiles;
         const int m0 = (int)co_tile * BM, n0 = (int)ci_tile * BN;
@@ -744,6 +770,16 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
                         if (out) out[(size_t)co * V * Ci + ci] = from_float<typename Tag::type>(acc[i][j][e]);
                         else dst[(size_t)co * Ci + ci] = acc[i][j][e];
                     }
+                }
+        }
+        if (do_bias && l32 == 0) {                  // bias_partial[block * SLICES + slice][co]
+            float* bdst = bias_partial + ((size_t)b * C::SLICES + (C::KSPLIT ? mw : 0)) * Co;
+#pragma unroll
+            for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int co = m0 + wave_m * C::WM + i * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
+                    if (co < Co) bdst[co] = bacc[i][e];
                 }
         }
         m.k = m.k_hi;                               // on to the next non-empty item
@@ -933,6 +969,40 @@ int launch_reduce(const float* partial, const uint32_t* bounds, int V, int Ci, i
     return FGX_OK;
 }
 
+__global__ void __launch_bounds__(256) zero_f32_kernel(float* __restrict__ p, size_t count) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (size_t)gridDim.x * 256) p[i] = 0.f;
+}
+
+// grad_bias[co] = sum over the voxel blocks (and slices) of their column sums.  A workgroup owns 32 columns; its 32
+// groups of 32 threads each add every 32nd slot (four independent loads in flight), then the group sums are added in
+// group order: a fixed order, the same on every run.
+template <typename T>
+__global__ void __launch_bounds__(1024) bias_reduce_kernel(const float* __restrict__ bias_partial, unsigned slots, int Co,
+                                                           T* __restrict__ out) {
+    __shared__ float sums[32][33];
+    const int c = threadIdx.x & 31, grp = threadIdx.x >> 5;
+    const int co = blockIdx.x * 32 + c;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    if (co < Co) {
+        unsigned q = grp;
+        for (; q + 96 < slots; q += 128) {
+            s0 += bias_partial[(size_t)q * Co + co];
+            s1 += bias_partial[(size_t)(q + 32) * Co + co];
+            s2 += bias_partial[(size_t)(q + 64) * Co + co];
+            s3 += bias_partial[(size_t)(q + 96) * Co + co];
+        }
+        for (; q < slots; q += 32) s0 += bias_partial[(size_t)q * Co + co];
+    }
+    sums[grp][c] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (grp == 0 && co < Co) {
+        float s = 0.f;
+#pragma unroll
+        for (int k = 0; k < 32; ++k) s += sums[k][c];
+        out[co] = from_float<T>(s);
+    }
+}
+
 // grad_weight[:, v, :] = 0 for the offsets v of `mask`: offsets without a single pair when the kernels write
 // grad_weight themselves (they skip empty items)
 template <typename T>
@@ -964,8 +1034,15 @@ bool dtype_ok(int dtype) { return dtype == FGX_F16 || dtype == FGX_BF16 || dtype
 
 struct Layout {
     unsigned nb;
-    size_t bounds_off, partial_off, total;
+    size_t bounds_off, partial_off, bias_off, colsum_off, total;
 };
+
+// where the bias gradient goes, and the offset whose pairs hold every output row exactly once (-1: none does)
+struct BiasOut {
+    void* out = nullptr;
+    int offset = -1;
+};
+constexpr int kMaxSlices = 4;
 
 // `slices`: partial products per (voxel block, offset, tile)
 Layout layout(size_t n, int V, int Ci, int Co, int block_rows, int slices) {
@@ -975,7 +1052,11 @@ Layout layout(size_t n, int V, int Ci, int Co, int block_rows, int slices) {
     L.bounds_off = off;
     off = align_up(off + (size_t)V * (L.nb + 1) * sizeof(uint32_t), 256);
     L.partial_off = off;
-    off += (size_t)(L.nb ? L.nb : 1) * slices * V * Co * Ci * sizeof(float);
+    off = align_up(off + (size_t)(L.nb ? L.nb : 1) * slices * V * Co * Ci * sizeof(float), 256);
+    L.bias_off = off;           // fp32 column sums of grad_out per voxel block and slice
+    off = align_up(off + (size_t)(L.nb ? L.nb : 1) * kMaxSlices * Co * sizeof(float), 256);
+    L.colsum_off = off;         // scratch of the stand-alone column sum, for the paths that do not fuse it
+    off += fgx_colsum_scratch_bytes((size_t)1 << 40, Co);      // its largest size: the row count it serves is the caller's
     L.total = off;
     return L;
 }
@@ -1021,7 +1102,7 @@ int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, con
 template <typename Tag, int BM, int BN>
 int launch_wgrad_stream(const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
                         const uint32_t* given_bounds, const SegTable& tab, const Layout& L, size_t n, size_t n_in, int V, int Ci, int Co, int block_rows,
-                        void* scratch, void* gw, hipStream_t s) {
+                        void* scratch, void* gw, BiasOut bias, hipStream_t s) {
     using C = WStreamCfg<Tag, BM, BN>;
     using T = typename Tag::type;
     // the block table depends on the pair lists and block_rows alone: callers that keep it pass it in
@@ -1053,10 +1134,22 @@ int launch_wgrad_stream(const void* gout, const void* feats, const uint32_t* sig
             int rc = prepare_direct<T>(tab, V, Ci, Co, (T*)gw, s);
             if (rc != FGX_OK) return rc;
         }
+        float* bias_partial = bias.out ? (float*)((char*)scratch + L.bias_off) : nullptr;
+        const unsigned bias_slots = L.nb * C::SLICES;
+        if (bias_partial) {         // a block without a pair at that offset leaves its slot untouched
+            zero_f32_kernel<<<cdiv((size_t)bias_slots * Co, 256) < 1024u ? cdiv((size_t)bias_slots * Co, 256) : 1024u, 256, 0, s>>>(
+                bias_partial, (size_t)bias_slots * Co);
+            FGX_CHECK_LAUNCH("fgx_conv_wgrad(bias zero)");
+        }
         kern<<<groups, C::NT, C::lds_bytes, s>>>((const T*)gout, (const T*)feats, sig_i, sig_o, bounds, V, Ci, Co, L.nb, co_tiles,
                                                  ci_tiles, tab.seg[V], (uint32_t)(n * (size_t)Co * sizeof(T)),
-                                                 (uint32_t)(n_in * (size_t)Ci * sizeof(T)), partial, direct ? (T*)gw : nullptr);
+                                                 (uint32_t)(n_in * (size_t)Ci * sizeof(T)), partial, direct ? (T*)gw : nullptr,
+                                                 bias_partial, bias.offset);
         FGX_CHECK_LAUNCH("fgx_conv_wgrad(stream)");
+        if (bias_partial) {
+            bias_reduce_kernel<T><<<cdiv((size_t)Co, 32), 1024, 0, s>>>(bias_partial, bias_slots, Co, (T*)bias.out);
+            FGX_CHECK_LAUNCH("fgx_conv_wgrad(bias reduce)");
+        }
         if (direct) return FGX_OK;
     }
     return launch_reduce<T>(partial, bounds, V, Ci, Co, L.nb * C::SLICES, (unsigned)C::SLICES, (T*)gw, s);
@@ -1075,11 +1168,11 @@ bool stream_ok(int tile_rows, int tile_cols, size_t n, size_t n_in, int Ci, int 
 template <typename Tag>
 int dispatch_wgrad_stream(int tile_rows, const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
                           const uint32_t* given_bounds, const SegTable& tab, const Layout& L, size_t n, size_t n_in, int V, int Ci, int Co, int block_rows,
-                          void* scratch, void* gw, hipStream_t s) {
+                          void* scratch, void* gw, BiasOut bias, hipStream_t s) {
     if constexpr (sizeof(typename Tag::type) == 2) {
-        if (tile_rows == 128) return launch_wgrad_stream<Tag, 128, 128>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, s);
-        if (tile_rows == 64) return launch_wgrad_stream<Tag, 64, 64>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, s);
-        return launch_wgrad_stream<Tag, 32, 32>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, s);
+        if (tile_rows == 128) return launch_wgrad_stream<Tag, 128, 128>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, s);
+        if (tile_rows == 64) return launch_wgrad_stream<Tag, 64, 64>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, s);
+        return launch_wgrad_stream<Tag, 32, 32>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, s);
     } else {
         set_error("fgx_conv_wgrad: the streaming kernel handles 16-bit types only");
         return FGX_ERR_UNSUPPORTED;
@@ -1142,7 +1235,7 @@ int fgx_wgrad_block_bounds(const uint32_t* sig_o, const uint32_t* seg_host, size
 int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
                    const uint32_t* seg_host, const uint32_t* block_bounds, size_t n, size_t n_in, int Ci, int Co, int V,
                    int tile_rows, int tile_cols, int block_rows, int streaming, void* scratch, void* grad_weight,
-                   fgx_stream_t stream) {
+                   void* grad_bias, int bias_offset, fgx_stream_t stream) {
     FGX_CHECK_ARG(dtype_ok(dtype), "fgx_conv_wgrad: unknown dtype %d", dtype);
     FGX_CHECK_ARG(Ci > 0 && Co > 0 && V >= 1 && V <= kMaxV, "fgx_conv_wgrad: bad shape Ci=%d Co=%d V=%d", Ci, Co, V);
     FGX_CHECK_ARG(block_rows >= 1, "fgx_conv_wgrad: block_rows must be positive, got %d", block_rows);
@@ -1169,11 +1262,25 @@ int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uin
     // 32-bit byte offsets into grad_out / feats are enough below 4 GiB
     const bool small = (double)n * Co * es < 4294967296.0 && (double)n_in * Ci * es < 4294967296.0;
     hipStream_t s = (hipStream_t)stream;
+    // The bias gradient is the column sum of grad_out.  The streaming kernel makes it on the side when one offset's pairs
+    // hold every output row exactly once (the caller says which); every other path runs the stand-alone column sum.
+    BiasOut bias;
+    if (grad_bias != nullptr) {
+        const bool fuse = (stream_f16 || stream_bf16) && bias_offset >= 0 && bias_offset < V &&
+                          (size_t)(tab.seg[bias_offset + 1] - tab.seg[bias_offset]) == n;
+        if (fuse) {
+            bias.out = grad_bias;
+            bias.offset = bias_offset;
+        } else {
+            int rc = fgx_colsum(dtype, grad_out, n, Co, (char*)scratch + L.colsum_off, grad_bias, stream);
+            if (rc != FGX_OK) return rc;
+        }
+    }
     // (outside the streaming kernel's range the tiled kernel runs)
     if (stream_f16)
-        return dispatch_wgrad_stream<F16>(tile_rows, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, s);
+        return dispatch_wgrad_stream<F16>(tile_rows, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, bias, s);
     if (stream_bf16)
-        return dispatch_wgrad_stream<BF16>(tile_rows, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, s);
+        return dispatch_wgrad_stream<BF16>(tile_rows, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, bias, s);
     switch (dtype) {
         case FGX_F16: return dispatch_wgrad<F16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);
         case FGX_BF16: return dispatch_wgrad<BF16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);

@@ -50,6 +50,9 @@ SORT_BUILDER_MIN_PROBES = 27 * 131072
 # (balanced, except for the locality order of short-row layers, whose neighboring tiles are meant to share an XCD).
 # The result does not depend on it.
 GEMM_ITEM_ORDER = "auto"
+# The bias gradient of a submanifold layer comes out of the streaming wgrad kernel (which loads every grad_output row for
+# the centre offset anyway) instead of a column-sum pass of its own.  False: always the separate pass.
+FUSE_DBIAS = True
 
 
 def set_neighbor_map_builder(builder: str):

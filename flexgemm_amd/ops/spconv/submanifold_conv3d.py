@@ -426,9 +426,11 @@ def _stream_fits(n: int, n_src: int, row_bytes: int) -> bool:
     return n_src * row_bytes <= 0xFF000000 and n * 8 <= 0xFF000000 and n * 27 * 4 * 2 <= 0xFF000000
 
 
-def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int) -> torch.Tensor:
+def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int, with_bias: bool = False, bias_offset: int = -1):
     """[Co, V, Ci] weight gradient from the pair lists of cache["neighbor_map"]: grad_output has one row per row of
-    that map, feats one per row the map points at."""
+    that map, feats one per row the map points at.  with_bias: also the bias gradient (column sums of grad_output),
+    returned as a second value; bias_offset names an offset whose pairs hold every row of grad_output exactly once (the
+    centre of a submanifold convolution), which lets the streaming kernel sum the rows it loads anyway."""
     n_in, ci = feats.shape
     n, co = grad_output.shape
     dt = feats.dtype
@@ -442,6 +444,7 @@ def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int) -> tor
     seg_arr = (C.c_uint32 * (v + 1))(*seg_host)
     sched = nat.table_lookup(nat.PASS_WGRAD, dt, n, cip, cop, v)
     gw = torch.empty((cop, v, cip), dtype=dt, device=dev)
+    gb = torch.empty((cop,), dtype=dt, device=dev) if with_bias else None
     L = nat.lib()
     code = nat.DTYPE_CODE[dt]
     bounds = cache._wgrad_bounds(sched.block_rows)
@@ -452,11 +455,13 @@ def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int) -> tor
         nat.check(L.fgx_conv_wgrad(
             C.c_int(code), nat.ptr(g), nat.ptr(f), nat.ptr(cache["valid_signal_i"]), nat.ptr(cache["valid_signal_o"]),
             seg_arr, nat.ptr(bounds), nat.sz(n), nat.sz(n_in), C.c_int(cip), C.c_int(cop), C.c_int(v), C.c_int(sched.tile_rows), C.c_int(sched.tile_cols),
-            C.c_int(sched.block_rows), C.c_int(sched.stream), nat.ptr(scratch), nat.ptr(gw), nat.stream()))
+            C.c_int(sched.block_rows), C.c_int(sched.stream), nat.ptr(scratch), nat.ptr(gw), nat.ptr(gb), C.c_int(bias_offset),
+            nat.stream()))
         nat.mark("wgrad", "stop")
     if cip != ci or cop != co:
         gw = gw[:co, :, :ci].contiguous()
-    return gw
+        gb = gb[:co].contiguous() if with_bias else None
+    return (gw, gb) if with_bias else gw
 
 
 def _colsum(grad_output: torch.Tensor) -> torch.Tensor:
@@ -607,9 +612,15 @@ class SubMConv3dFunction(Function):
             if feats.requires_grad:
                 grad_input = _gather_gemm(grad_output, weight.detach().reshape(co, v, ci), None, neighbor_cache, 1,
                                           algo not in _NO_SPLITK, masked=algo in _MASKED)
-            if weight.requires_grad:
+            want_bias = bias is not None and bias.requires_grad
+            if weight.requires_grad and want_bias:
+                # odd kernel: the centre offset pairs every voxel with itself, so dbias rides along with wgrad
+                centre = v // 2 if (kw % 2 and kh % 2 and kd % 2 and spconv.FUSE_DBIAS) else -1
+                grad_weight, grad_bias = _wgrad(grad_output, feats.detach(), neighbor_cache, v, True, centre)
+                grad_weight = grad_weight.reshape(co, kw, kh, kd, ci)
+            elif weight.requires_grad:
                 grad_weight = _wgrad(grad_output, feats.detach(), neighbor_cache, v).reshape(co, kw, kh, kd, ci)
-            if bias is not None and bias.requires_grad:
+            elif want_bias:
                 grad_bias = _colsum(grad_output)
             return grad_input, grad_weight, grad_bias
         raise ValueError(f"Unsupported algorithm {algo}")

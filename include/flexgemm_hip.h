@@ -254,8 +254,14 @@ int fgx_gather_item_order(const int32_t* tile_code, size_t num_tiles, int col_ti
  * block_rows -- block_bounds[v * (nb + 1) + b] = first pair of offset v whose grad_out row is >= b * block_rows,
  * nb = ceil(n / block_rows) -- for callers that keep it with their neighbor cache; NULL = computed here, per call.
  * The 32x32 streaming tile writes four partial products per block (the scratch size accounts for it).
+ * `grad_bias` (optional, Co elements of the tensors' type): the column sums of grad_out over its n rows, the bias
+ * gradient.  `bias_offset` names an offset whose pairs hold every grad_out row exactly once (the centre offset of a
+ * submanifold convolution; -1 when there is none): the streaming kernel then sums the grad_out rows it loads for that
+ * offset anyway and grad_out is not read a third time.  Without such an offset, or on the tiled path, the call runs
+ * fgx_colsum itself (the scratch size accounts for that too).
  * Replaces: sparse_submanifold_conv_bwd_weight_masked_implicit_gemm[_splitk]
- *           (..._bwd_masked_implicit_gemm.py:99-170, ..._splitk.py:108-182, 278-317). */
+ *           (..._bwd_masked_implicit_gemm.py:99-170, ..._splitk.py:108-182, 278-317), and with grad_bias
+ *           grad_output.sum(0) (..._splitk.py:365-366). */
 size_t fgx_wgrad_scratch_bytes(size_t n, int V, int Ci, int Co, int block_rows);
 size_t fgx_wgrad_block_bounds_count(size_t n, int V, int block_rows);
 int fgx_wgrad_block_bounds(const uint32_t* sig_o, const uint32_t* seg_host, size_t n, int V, int block_rows,
@@ -263,7 +269,8 @@ int fgx_wgrad_block_bounds(const uint32_t* sig_o, const uint32_t* seg_host, size
 int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats,
                    const uint32_t* sig_i, const uint32_t* sig_o, const uint32_t* seg_host, const uint32_t* block_bounds,
                    size_t n, size_t n_in, int Ci, int Co, int V, int tile_rows, int tile_cols, int block_rows,
-                   int streaming, void* scratch, void* grad_weight, fgx_stream_t stream);
+                   int streaming, void* scratch, void* grad_weight, void* grad_bias, int bias_offset,
+                   fgx_stream_t stream);
 
 /* grad_bias[co] = sum over rows of grad_out[:, co], accumulated in fp32.
  * `scratch`: fgx_colsum_scratch_bytes bytes of fp32 partial sums.

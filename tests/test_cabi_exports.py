@@ -66,9 +66,12 @@ def test_host_only_entry_points(library):
     assert L.fgx_conv_scratch_bytes(ctypes.c_size_t(1000), 64, 1) == 0
     assert L.fgx_conv_scratch_bytes(ctypes.c_size_t(1000), 64, 4) == 4 * 1000 * 64 * 4
     # 1000 rows in blocks of 256 -> 4 blocks: bounds table (3 * 5 uint32, padded to 256 B) + 4 * 3 partial products
-    assert L.fgx_wgrad_scratch_bytes(ctypes.c_size_t(1000), 3, 48, 64, 256) == 256 + 4 * 3 * 48 * 64 * 4
+    # + the bias gradient's column sums per block and slice (4 blocks * 4 slices * Co floats) + the scratch of fgx_colsum
+    colsum = L.fgx_colsum_scratch_bytes(ctypes.c_size_t(1000), 64)
+    assert L.fgx_wgrad_scratch_bytes(ctypes.c_size_t(1000), 3, 48, 64, 256) == 256 + 4 * 3 * 48 * 64 * 4 + 4 * 4 * 64 * 4 + colsum
     # up to 32 channels on either side: room for the four partial products per block of the 32 x 32 streaming tile
-    assert L.fgx_wgrad_scratch_bytes(ctypes.c_size_t(1000), 3, 8, 16, 256) == 256 + 4 * 4 * 3 * 8 * 16 * 4
+    colsum = L.fgx_colsum_scratch_bytes(ctypes.c_size_t(1000), 16)
+    assert L.fgx_wgrad_scratch_bytes(ctypes.c_size_t(1000), 3, 8, 16, 256) == 256 + 4 * 4 * 3 * 8 * 16 * 4 + 4 * 4 * 16 * 4 + colsum
 
 
 def test_argument_errors_map_to_exceptions(library):
@@ -81,7 +84,7 @@ def test_argument_errors_map_to_exceptions(library):
                                           2, 3, 3, 1, 1, 1, None, None, None, None))
     with pytest.raises(ValueError):
         nat.check(L.fgx_conv_wgrad(0, None, None, None, None, None, None, ctypes.c_size_t(0), ctypes.c_size_t(0), 8, 8, 27, 128, 128, 0, 0,
-                                   None, None, None))
+                                   None, None, None, -1, None))
     with pytest.raises(ValueError):   # the streaming GEMM checks its arguments before touching the device
         nat.check(L.fgx_conv_gather_gemm_stream(0, None, None, None, None, None, None, None, None, ctypes.c_size_t(0),
                                                 ctypes.c_size_t(10), ctypes.c_size_t(10), 128, 128, 27, 256, 128, 128, None, 0, None, None))

@@ -283,6 +283,33 @@ def test_streaming_kernel_equals_tiled_kernel_bitwise(gpu_device):
     assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("res,ci,co,block_rows", [(48, 128, 128, 0), (48, 128, 128, 2048), (48, 32, 32, 0), (40, 64, 256, 1024),
+                                                   (40, 256, 64, 0), (64, 64, 64, 4096), (24, 128, 128, 0)])
+def test_bias_gradient_rides_along_with_wgrad(gpu_device, dtype, res, ci, co, block_rows):
+    """dbias from the streaming wgrad kernel (grad_out rows of the centre offset times a fragment of ones): equal to the
+    column sums within the operator's tolerance, for wide, narrow (pairs split over the multipliers), multi-tile and
+    single-block shapes, and the weight gradient itself is unchanged bit for bit.  The last shape is below the streaming
+    range: there the call falls back to the stand-alone column sum."""
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    _say(f"fused dbias res={res} ci={ci} co={co} block_rows={block_rows} {dtype}")
+    coords_np = reference_test_shell(res)
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    f, w, b, g = _case(coords_np, ci, co, dtype, 53)
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, torch.Size([1, ci, res, res, res]), (3, 3, 3), (1, 1, 1), True)
+    fields = dict(block_rows=block_rows) if block_rows else {}
+    with _force_schedule(wgrad=True, **fields):
+        gw_plain = impl._wgrad(g.to(gpu_device), f.to(gpu_device), cache, 27)
+        gw, gb = impl._wgrad(g.to(gpu_device), f.to(gpu_device), cache, 27, True, 13)
+        gw2, gb2 = impl._wgrad(g.to(gpu_device), f.to(gpu_device), cache, 27, True, -1)       # no such offset: column sum
+    assert torch.equal(gw, gw_plain) and torch.equal(gw2, gw_plain)
+    ref = g.double().sum(0)
+    assert gb.dtype == dtype and gb.shape == (co,)
+    assert eg.max_rel_err(gb.cpu(), ref) <= TOL[dtype]
+    assert eg.max_rel_err(gb2.cpu(), ref) <= TOL[dtype]
+    assert torch.equal(gb2, impl._colsum(g.to(gpu_device)))
+
+
 def test_item_order_changes_nothing(gpu_device):
     """How the streaming GEMM's tiles are dealt to its workgroups is a scheduling choice: every order gives the same
     bits (more items than resident workgroups, two column tiles per row tile)."""
@@ -330,9 +357,14 @@ def test_item_order_evens_out_the_benchmark_shell(gpu_device):
     coords = torch.from_numpy(shell_coords(res)).to(gpu_device)
     _say(f"item order at res {res}, n={coords.shape[0]}")
     cache = SubMConv3dFunction._compute_neighbor_cache(coords, torch.Size([1, 128, res, res, res]), (3, 3, 3), (1, 1, 1), False)
+    import flex_gemm
     _, code, _, _, _, key = cache._gather_plan(256, False)
     for col_tiles, groups, slabs in ((1, 256, 2), (2, 256, 4), (1, 512, 1)):
-        item_at = cache._item_order(key, code, col_tiles, groups, slabs).cpu().numpy().astype(np.int64)
+        flex_gemm.ops.spconv.GEMM_ITEM_ORDER = "balanced"       # ("auto" deals rows of 512 bytes and more only)
+        try:
+            item_at = cache._item_order(key, code, col_tiles, groups, slabs).cpu().numpy().astype(np.int64)
+        finally:
+            flex_gemm.ops.spconv.GEMM_ITEM_ORDER = "auto"
         codes = code.cpu().numpy().view(np.uint32)
         total = col_tiles * len(codes)
         assert sorted(item_at.tolist()) == list(range(total))
