@@ -481,3 +481,37 @@ def test_full_size_properties_cfg3(gpu_device):
     scale = float((conv_nobias.abs() * g64.abs()).sum())
     assert abs(lhs - mid) / scale < 1e-3 and abs(lhs - rhs) / scale < 1e-3
     assert eg.max_rel_err(b.grad.cpu(), g64.sum(0)) <= 1e-2
+
+
+@pytest.mark.parametrize("name,sample", [("cfg2", 2048), ("cfg4", 4096), ("cfg5", 512)])
+def test_full_size_properties_other_configurations(gpu_device, name, sample):
+    """Configurations 2, 4 and 5 at full size, in their own dtypes: a random sample of output rows against the float64
+    oracle (forward and input gradient), the inner-product identities <conv(f), g> = <f, dgrad(g)> = <W, wgrad> over the
+    whole tensors, and the bias gradient against the column sums."""
+    wl = make_workload(name)
+    dt = wl.dtype
+    c = wl.feats.shape[1]
+    _say(f"conv {name} full size, n={wl.n} C={c} {dt}")
+    dev = gpu_device
+    f = wl.feats.to(dt).to(dev).requires_grad_(True)
+    w = wl.weight.to(dt).to(dev).requires_grad_(True)
+    b = wl.bias.to(dt).to(dev).requires_grad_(True)
+    g = wl.grad.to(dt)
+    coords = wl.coords.to(dev)
+    out, cache = sparse_submanifold_conv3d(f, coords, wl.shape, w, b)
+    out.backward(g.to(dev))
+    torch.cuda.synchronize()
+    nmap = cache.neighbor_map.cpu().view(torch.int32)
+    rows = torch.randperm(wl.n, generator=torch.Generator().manual_seed(1))[:sample]
+    f64, w64, b64, g64 = f.detach().cpu().double(), w.detach().cpu().double(), b.detach().cpu().double(), g.double()
+    ref_rows = eg.forward(f64, nmap[rows], w64, b64)
+    _assert_close(out[rows.to(dev)], ref_rows, dt, "forward sample")
+    ref_gi = torch.mm(eg._im2col(g64, torch.flip(nmap[rows].long(), [1])), w64.reshape(c, 27, c).transpose(0, 1).reshape(27 * c, c))
+    _assert_close(f.grad[rows.to(dev)], ref_gi, dt, "dgrad sample")
+    conv_nobias = out.detach().cpu().double() - b64
+    lhs = (conv_nobias * g64).sum()
+    mid = (f64 * f.grad.cpu().double()).sum()
+    rhs = (w64 * w.grad.cpu().double()).sum()
+    scale = float((conv_nobias.abs() * g64.abs()).sum())
+    assert abs(lhs - mid) / scale < 1e-3 and abs(lhs - rhs) / scale < 1e-3
+    assert eg.max_rel_err(b.grad.cpu(), g64.sum(0)) <= 1e-2
