@@ -969,29 +969,31 @@ int launch_reduce(const float* partial, const uint32_t* bounds, int V, int Ci, i
     return FGX_OK;
 }
 
-__global__ void __launch_bounds__(256) zero_f32_kernel(float* __restrict__ p, size_t count) {
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (size_t)gridDim.x * 256) p[i] = 0.f;
-}
-
 // grad_bias[co] = sum over the voxel blocks (and slices) of their column sums.  A workgroup owns 32 columns; its 32
 // groups of 32 threads each add every 32nd slot (four independent loads in flight), then the group sums are added in
-// group order: a fixed order, the same on every run.
+// group order: a fixed order, the same on every run.  `live` is the block table row of the offset the sums were made
+// from: a block without a pair there was skipped by the kernel and its slots hold nothing.
 template <typename T>
-__global__ void __launch_bounds__(1024) bias_reduce_kernel(const float* __restrict__ bias_partial, unsigned slots, int Co,
-                                                           T* __restrict__ out) {
+__global__ void __launch_bounds__(1024) bias_reduce_kernel(const float* __restrict__ bias_partial,
+                                                           const uint32_t* __restrict__ live, unsigned slots, unsigned slices,
+                                                           int Co, T* __restrict__ out) {
     __shared__ float sums[32][33];
     const int c = threadIdx.x & 31, grp = threadIdx.x >> 5;
     const int co = blockIdx.x * 32 + c;
+    auto term = [&](unsigned q) -> float {
+        const unsigned blk = q / slices;
+        return live[blk] < live[blk + 1] ? bias_partial[(size_t)q * Co + co] : 0.f;
+    };
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
     if (co < Co) {
         unsigned q = grp;
         for (; q + 96 < slots; q += 128) {
-            s0 += bias_partial[(size_t)q * Co + co];
-            s1 += bias_partial[(size_t)(q + 32) * Co + co];
-            s2 += bias_partial[(size_t)(q + 64) * Co + co];
-            s3 += bias_partial[(size_t)(q + 96) * Co + co];
+            s0 += term(q);
+            s1 += term(q + 32);
+            s2 += term(q + 64);
+            s3 += term(q + 96);
         }
-        for (; q < slots; q += 32) s0 += bias_partial[(size_t)q * Co + co];
+        for (; q < slots; q += 32) s0 += term(q);
     }
     sums[grp][c] = (s0 + s1) + (s2 + s3);
     __syncthreads();
@@ -1136,18 +1138,14 @@ int launch_wgrad_stream(const void* gout, const void* feats, const uint32_t* sig
         }
         float* bias_partial = bias.out ? (float*)((char*)scratch + L.bias_off) : nullptr;
         const unsigned bias_slots = L.nb * C::SLICES;
-        if (bias_partial) {         // a block without a pair at that offset leaves its slot untouched
-            zero_f32_kernel<<<cdiv((size_t)bias_slots * Co, 256) < 1024u ? cdiv((size_t)bias_slots * Co, 256) : 1024u, 256, 0, s>>>(
-                bias_partial, (size_t)bias_slots * Co);
-            FGX_CHECK_LAUNCH("fgx_conv_wgrad(bias zero)");
-        }
         kern<<<groups, C::NT, C::lds_bytes, s>>>((const T*)gout, (const T*)feats, sig_i, sig_o, bounds, V, Ci, Co, L.nb, co_tiles,
                                                  ci_tiles, tab.seg[V], (uint32_t)(n * (size_t)Co * sizeof(T)),
                                                  (uint32_t)(n_in * (size_t)Ci * sizeof(T)), partial, direct ? (T*)gw : nullptr,
                                                  bias_partial, bias.offset);
         FGX_CHECK_LAUNCH("fgx_conv_wgrad(stream)");
         if (bias_partial) {
-            bias_reduce_kernel<T><<<cdiv((size_t)Co, 32), 1024, 0, s>>>(bias_partial, bias_slots, Co, (T*)bias.out);
+            bias_reduce_kernel<T><<<cdiv((size_t)Co, 32), 1024, 0, s>>>(bias_partial, bounds + (size_t)bias.offset * (L.nb + 1),
+                                                                         bias_slots, (unsigned)C::SLICES, Co, (T*)bias.out);
             FGX_CHECK_LAUNCH("fgx_conv_wgrad(bias reduce)");
         }
         if (direct) return FGX_OK;
