@@ -19,7 +19,8 @@ class Algorithm:
 
 class SerializationMode:
     """How 3-D coordinates are flattened into the key that orders generated output coordinates
-    (flex_gemm/ops/spconv/__init__.py:10-14).  Only BXYZ is implemented here."""
+    (flex_gemm/ops/spconv/__init__.py:10-14): by flattened (b, x, y, z) key, along the z-order curve or along the Hilbert
+    curve."""
     BXYZ = 0
     Z_ORDER = 1
     HILBERT = 2
