@@ -6,7 +6,7 @@ import sys
 
 import flexgemm_amd as _impl
 
-for _name in ("kernels", "kernels.cuda", "ops", "ops.utils", "ops.serialize", "ops.spconv", "ops.spconv.submanifold_conv3d", "ops.spconv.sparse_conv3d"):
+for _name in ("kernels", "kernels.cuda", "kernels.triton", "kernels.triton.spconv", "kernels.triton.spconv.config", "ops", "ops.utils", "ops.serialize", "ops.spconv", "ops.spconv.submanifold_conv3d", "ops.spconv.sparse_conv3d"):
     sys.modules[__name__ + "." + _name] = importlib.import_module("flexgemm_amd." + _name)
 
 kernels = _impl.kernels
