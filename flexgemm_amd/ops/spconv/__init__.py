@@ -56,6 +56,24 @@ GEMM_ITEM_ORDER = "auto"
 FUSE_DBIAS = True
 
 
+# Keep the repacked weight panels of the gather GEMMs with the weight tensor and reuse them while the weight is unchanged
+# (no counterpart in the reference, whose kernels read the weight as it lies).  For serving and for gradient
+# accumulation: a panel is kept from the second time a weight is seen at the same version counter and data pointer, so a
+# loop that updates its weights every step keeps nothing.  Off by default, because the check cannot see a weight changed
+# through `weight.data` (that path does not move the version counter): switch it on only where weights are updated
+# through the tensor itself (torch.optim does) or not at all.  WEIGHT_PANEL_CACHE_MAX_BYTES bounds what is kept per
+# process; beyond it panels are packed per call as without the cache.
+WEIGHT_PANEL_CACHE = False
+WEIGHT_PANEL_CACHE_MAX_BYTES = 4 << 30
+
+
+def set_weight_panel_cache(enabled: bool, max_bytes: int = None):
+    global WEIGHT_PANEL_CACHE, WEIGHT_PANEL_CACHE_MAX_BYTES
+    WEIGHT_PANEL_CACHE = bool(enabled)
+    if max_bytes is not None:
+        WEIGHT_PANEL_CACHE_MAX_BYTES = int(max_bytes)
+
+
 def set_neighbor_map_builder(builder: str):
     global NEIGHBOR_MAP_BUILDER
     if builder not in ("auto", "hash", "sort"):

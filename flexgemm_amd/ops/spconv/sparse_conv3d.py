@@ -9,6 +9,7 @@ include/flexgemm_hip.h; the three GEMM passes are the submanifold operator's ker
 from __future__ import annotations
 
 import ctypes as C
+import weakref
 from typing import Optional, Tuple
 
 import torch
@@ -321,7 +322,7 @@ class SparseConv3dFunction(Function):
         if algo in _IMPLICIT:
             _require_cuda(feats, "sparse_conv3d")
             return _gather_gemm(feats, weight.reshape(co, v, ci), bias, neighbor_cache, 0, algo not in _NO_SPLITK,
-                                masked=algo in _MASKED)
+                                masked=algo in _MASKED, weight_owner=weight)
         raise ValueError(f"Unsupported algorithm {algo}")
 
     @staticmethod
@@ -331,6 +332,7 @@ class SparseConv3dFunction(Function):
         neighbor_cache: SparseConv3dNeighborCache,
         weight: torch.Tensor,
         bias: Optional[torch.Tensor] = None,
+        weight_owner: Optional[torch.Tensor] = None,
     ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], Optional[torch.Tensor]]:
         co, kw, kh, kd, ci = weight.shape
         v = kw * kh * kd
@@ -355,7 +357,8 @@ class SparseConv3dFunction(Function):
                 # mask-sorted walk only where the cache carries the backward order (reference: sparse_conv3d.py:191-207)
                 masked = algo in _MASKED and hasattr(view, "sorted_idx")
                 grad_input = _gather_gemm(grad_output, weight.detach().reshape(co, v, ci), None, view, 2,
-                                          algo not in _NO_SPLITK, masked=masked)
+                                          algo not in _NO_SPLITK, masked=masked,
+                                          weight_owner=weight if weight_owner is None else weight_owner)
             if weight.requires_grad:
                 grad_weight = _wgrad(grad_output, feats.detach(), neighbor_cache, v).reshape(co, kw, kh, kd, ci)
             if bias is not None and bias.requires_grad:
@@ -389,6 +392,7 @@ class SparseConv3dFunction(Function):
         output = SparseConv3dFunction._sparse_conv_forward(feats, neighbor_cache, weight, bias)
         ctx.save_for_backward(feats, weight, bias)
         ctx.neighbor_cache = neighbor_cache
+        ctx.weight_owner = weakref.ref(weight)      # the caller's tensor object: kept weight panels hang on it
         ctx.mark_non_differentiable(out_coords)
         return output, out_coords, neighbor_cache
 
@@ -399,7 +403,8 @@ class SparseConv3dFunction(Function):
         f = feats.detach().requires_grad_(need_f)
         w = weight.detach().requires_grad_(need_w)
         b = None if bias is None else bias.detach().requires_grad_(need_b)
-        grad_input, grad_weight, grad_bias = SparseConv3dFunction._sparse_conv_backward(grad_output, f, ctx.neighbor_cache, w, b)
+        grad_input, grad_weight, grad_bias = SparseConv3dFunction._sparse_conv_backward(grad_output, f, ctx.neighbor_cache, w, b,
+                                                                                        weight_owner=ctx.weight_owner())
         return grad_input, None, None, None, grad_weight, grad_bias, None, None, None, None
 
 

@@ -9,6 +9,7 @@ include/flexgemm_hip.h; torch only allocates tensors and owns the stream.
 from __future__ import annotations
 
 import ctypes as C
+import weakref
 from typing import Optional, Tuple
 
 import torch
@@ -340,12 +341,57 @@ def _pad_cols(t: torch.Tensor, mult: int) -> torch.Tensor:
     return t if pad == 0 else torch.nn.functional.pad(t, (0, pad))
 
 
+_panel_bytes_kept = 0       # bytes of weight panels kept with their weights (all devices)
+
+
+def _release_panel_bytes(nbytes: int) -> None:
+    global _panel_bytes_kept
+    _panel_bytes_kept -= nbytes
+
+
+def _weight_panel(owner: Optional[torch.Tensor], weight_cvk: torch.Tensor, code: int, mode: int, sched, dev) -> torch.Tensor:
+    """The weight repacked for the gather GEMM of `mode` under schedule `sched`.  With spconv.WEIGHT_PANEL_CACHE and an
+    `owner` (the caller's weight tensor, whose version counter and data pointer say whether it changed) the panel is
+    kept on the owner from the second request at the same version and handed out without packing after that."""
+    global _panel_bytes_kept
+    co, v, ci = weight_cvk.shape
+    L = nat.lib()
+    nbytes = L.fgx_weight_panel_bytes(C.c_int(code), C.c_int(mode), C.c_int(ci), C.c_int(co), C.c_int(v),
+                                      C.c_int(sched.slab_bytes), C.c_int(sched.tile_cols))
+
+    def pack(panel):
+        nat.check(L.fgx_pack_weight(C.c_int(code), C.c_int(mode), nat.ptr(weight_cvk), C.c_int(ci), C.c_int(co), C.c_int(v),
+                                    C.c_int(sched.slab_bytes), C.c_int(sched.tile_cols), nat.ptr(panel), nat.stream()))
+        return panel
+
+    if owner is None or not spconv.WEIGHT_PANEL_CACHE:
+        return pack(nat.workspace(nbytes, dev))
+    kept = owner.__dict__.setdefault("_fgx_weight_panels", {})
+    key = (code, mode, ci, co, v, int(sched.slab_bytes), int(sched.tile_cols), str(dev))
+    stamp = (owner._version, owner.data_ptr())
+    entry = kept.get(key)
+    if entry is not None and entry[0] == stamp:
+        if entry[1] is not None:
+            # (a panel packed on another stream is ordered like any other tensor: by the caller's stream semantics)
+            return entry[1]
+        if _panel_bytes_kept + nbytes <= spconv.WEIGHT_PANEL_CACHE_MAX_BYTES:
+            panel = pack(nat.workspace(nbytes, dev))
+            kept[key] = (stamp, panel)
+            _panel_bytes_kept += panel.numel()
+            weakref.finalize(panel, _release_panel_bytes, panel.numel())
+            return panel
+        return pack(nat.workspace(nbytes, dev))
+    kept[key] = (stamp, None)           # first sight of this version (a stale panel, if any, is dropped here)
+    return pack(nat.workspace(nbytes, dev))
+
+
 def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[torch.Tensor], cache, mode: int,
-                 allow_splitk: bool, masked: bool = True) -> torch.Tensor:
+                 allow_splitk: bool, masked: bool = True, weight_owner: Optional[torch.Tensor] = None) -> torch.Tensor:
     """mode 0: out = conv(src) with weight [Co, V, Ci] (+bias); mode 1: grad_input from src = grad_output through the
     same map with the offsets mirrored (submanifold); mode 2: grad_input through a map of its own, offsets as they
     are (generic sparse convolution).  The result has one row per row of cache["neighbor_map"]; src may have a
-    different number of rows.  masked=False: the non-masked schedule (natural row order, all offsets per tile)."""
+    different number of rows.  masked=False: the non-masked schedule (natural row order, all offsets per tile).
+    weight_owner: the tensor the caller's weight lives in, for the optional panel cache (see _weight_panel)."""
     co, v, ci = weight_cvk.shape
     n = cache["neighbor_map"].shape[0]
     n_src = src.shape[0]
@@ -363,6 +409,7 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
     align = 16 // src.element_size()
     if k_true % align:
         src = _pad_cols(src, align)
+        weight_owner = None             # the padded copy is made per call: nothing to key a kept panel on
         if mode == 0:
             weight_cvk = _pad_cols(weight_cvk, align)
         else:
@@ -383,10 +430,7 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
     code = nat.DTYPE_CODE[dt]
     name = "gather_gemm_fwd" if mode == 0 else "gather_gemm_dgrad"
     with torch.cuda.device(dev):
-        panel = nat.workspace(L.fgx_weight_panel_bytes(C.c_int(code), C.c_int(mode), C.c_int(ci), C.c_int(co), C.c_int(v),
-                                                       C.c_int(sched.slab_bytes), C.c_int(sched.tile_cols)), dev)
-        nat.check(L.fgx_pack_weight(C.c_int(code), C.c_int(mode), nat.ptr(weight_cvk), C.c_int(ci), C.c_int(co), C.c_int(v),
-                                    C.c_int(sched.slab_bytes), C.c_int(sched.tile_cols), nat.ptr(panel), nat.stream()))
+        panel = _weight_panel(weight_owner, weight_cvk, code, mode, sched, dev)
         if sched.stream and _stream_fits(n, n_src, k * src.element_size()):
             order, tile_code, plan_seg, plan_idx, plan_band, plan_key = cache._gather_plan(sched.tile_rows, private,
                                                                                            dense=not masked)
@@ -579,7 +623,7 @@ class SubMConv3dFunction(Function):
         if algo in _IMPLICIT:
             _require_cuda(feats, "sparse_submanifold_conv3d")
             return _gather_gemm(feats, weight.reshape(co, v, ci), bias, neighbor_cache, 0, algo not in _NO_SPLITK,
-                                masked=algo in _MASKED)
+                                masked=algo in _MASKED, weight_owner=weight)
         raise ValueError(f"Unsupported algorithm {algo}")
 
     @staticmethod
@@ -589,6 +633,7 @@ class SubMConv3dFunction(Function):
         neighbor_cache: SubMConv3dNeighborCache,
         weight: torch.Tensor,
         bias: Optional[torch.Tensor] = None,
+        weight_owner: Optional[torch.Tensor] = None,
     ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], Optional[torch.Tensor]]:
         co, kw, kh, kd, ci = weight.shape
         v = kw * kh * kd
@@ -611,7 +656,8 @@ class SubMConv3dFunction(Function):
             grad_output = grad_output.contiguous()
             if feats.requires_grad:
                 grad_input = _gather_gemm(grad_output, weight.detach().reshape(co, v, ci), None, neighbor_cache, 1,
-                                          algo not in _NO_SPLITK, masked=algo in _MASKED)
+                                          algo not in _NO_SPLITK, masked=algo in _MASKED,
+                                          weight_owner=weight if weight_owner is None else weight_owner)
             want_bias = bias is not None and bias.requires_grad
             if weight.requires_grad and want_bias:
                 # odd kernel: the centre offset pairs every voxel with itself, so dbias rides along with wgrad
@@ -644,6 +690,7 @@ class SubMConv3dFunction(Function):
         output = SubMConv3dFunction._sparse_submanifold_conv_forward(feats, neighbor_cache, weight, bias)
         ctx.save_for_backward(feats, weight, bias)
         ctx.neighbor_cache = neighbor_cache
+        ctx.weight_owner = weakref.ref(weight)      # the caller's tensor object: kept weight panels hang on it
         return output, neighbor_cache
 
     @staticmethod
@@ -655,7 +702,7 @@ class SubMConv3dFunction(Function):
         w = weight.detach().requires_grad_(need_w)
         b = None if bias is None else bias.detach().requires_grad_(need_b)
         grad_input, grad_weight, grad_bias = SubMConv3dFunction._sparse_submanifold_conv_backward(
-            grad_output, f, ctx.neighbor_cache, w, b)
+            grad_output, f, ctx.neighbor_cache, w, b, weight_owner=ctx.weight_owner())
         return grad_input, None, None, None, grad_weight, grad_bias, None
 
 

@@ -515,3 +515,102 @@ def test_full_size_properties_other_configurations(gpu_device, name, sample):
     scale = float((conv_nobias.abs() * g64.abs()).sum())
     assert abs(lhs - mid) / scale < 1e-3 and abs(lhs - rhs) / scale < 1e-3
     assert eg.max_rel_err(b.grad.cpu(), g64.sum(0)) <= 1e-2
+
+
+def test_weight_panel_cache_keeps_results_and_follows_weight_updates(gpu_device):
+    """Opt-in reuse of the repacked weight panels: same bits as without it, a panel kept from the second call on, an
+    in-place weight update seen through the version counter, the byte budget respected, bytes released with the weight."""
+    import gc
+    from flexgemm_amd.ops import spconv as cfg
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    res, c = 32, 64
+    coords_np = reference_test_shell(res)
+    shape = torch.Size([1, c, res, res, res])
+    feats, weight, bias, grad = _case(coords_np, c, c, torch.float16, seed=11)
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+
+    def step(w, b):
+        f = feats.to(gpu_device).requires_grad_(True)
+        w.grad = None
+        out, _ = sparse_submanifold_conv3d(f, coords, shape, w, b, neighbor_cache=cache)
+        out.backward(grad.to(gpu_device))
+        return out.detach().clone(), f.grad.clone(), w.grad.clone()
+
+    w = weight.to(gpu_device).requires_grad_(True)
+    b = bias.to(gpu_device)
+    plain = step(w, b)
+    kept_before = impl._panel_bytes_kept
+    cfg.set_weight_panel_cache(True)
+    try:
+        _say("panel cache: three steps with one weight")
+        for i in range(3):
+            got = step(w, b)
+            assert all(torch.equal(x, y) for x, y in zip(got, plain)), f"step {i} differs from the uncached result"
+            panels = [e for e in w._fgx_weight_panels.values() if e[1] is not None]
+            assert len(panels) == (0 if i == 0 else 2), f"step {i}: {len(panels)} panels kept"      # forward and dgrad
+        assert impl._panel_bytes_kept > kept_before
+        _say("panel cache: in-place update")
+        with torch.no_grad():
+            w.mul_(0.5)
+        got = step(w, b)
+        cfg.set_weight_panel_cache(False)
+        want = step(w, b)
+        cfg.set_weight_panel_cache(True)
+        assert all(torch.equal(x, y) for x, y in zip(got, want))
+        assert not torch.equal(got[0], plain[0])
+        assert all(e[1] is None for e in w._fgx_weight_panels.values())       # the stale panels are gone
+        _say("panel cache: zero budget keeps nothing")
+        cfg.set_weight_panel_cache(True, max_bytes=0)
+        w2 = weight.to(gpu_device).requires_grad_(True)
+        for _ in range(3):
+            got = step(w2, b)
+        assert all(torch.equal(x, y) for x, y in zip(got, plain))
+        assert all(e[1] is None for e in w2._fgx_weight_panels.values())
+        del w, w2, got, want, panels
+        gc.collect()
+        assert impl._panel_bytes_kept == kept_before
+    finally:
+        cfg.set_weight_panel_cache(False, max_bytes=4 << 30)
+
+
+@pytest.mark.parametrize("res,c", [(24, 64), (64, 128), (16, 1024)])
+def test_forward_replays_from_a_hip_graph(gpu_device, res, c):
+    """Two stacked layers captured into a HIP graph (the library calls no allocation, memset, copy or synchronisation,
+    so a warmed-up forward records kernels only): every replay, with new input values and eager work of the same
+    operator between the replays, equals the eager result bit for bit.  Sizes cover the tiled kernel with split-K, the
+    streaming kernel and the wide-channel case."""
+    coords_np = reference_test_shell(res)
+    shape = torch.Size([1, c, res, res, res])
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    n = len(coords_np)
+    g = torch.Generator().manual_seed(res * c)
+    ws = [(torch.randn(c, 3, 3, 3, c, generator=g) / math.sqrt(27 * c)).half().to(gpu_device) for _ in range(2)]
+    bs = [torch.randn(c, generator=g).half().to(gpu_device) for _ in range(2)]
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), False)
+
+    def stack(x):
+        for w, b in zip(ws, bs):
+            x = sparse_submanifold_conv3d(x, coords, shape, w, b, cache)[0]
+        return x
+
+    static_in = torch.randn(n, c, generator=g).half().to(gpu_device)
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                stack(static_in)                 # builds the plans and the schedule lookups the capture must not build
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        _say(f"graph capture res={res} c={c}")
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_out = stack(static_in)
+        for k in range(4):
+            x = torch.randn(n, c, generator=g).half().to(gpu_device)
+            static_in.copy_(x)
+            graph.replay()
+            eager = stack(x)                     # the program's own eager work between the replays
+            torch.cuda.synchronize()
+            assert torch.equal(static_out, eager), f"replay {k} differs from the eager result"
