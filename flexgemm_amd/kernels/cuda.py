@@ -206,18 +206,12 @@ def neighbor_map_post_process_for_masked_implicit_gemm_2(gray_code: torch.Tensor
 
 
 def _out_coords(in_coords: torch.Tensor, serialize_mode: int, B, W, H, D, Kw, Kh, Kd, Sw, Sh, Sd, Pw, Ph, Pd, Dw, Dh, Dd):
-    from ..ops import spconv
     from ..ops.spconv.sparse_conv3d import SparseConv3dFunction
     _on_gpu(in_coords)
     if serialize_mode not in (0, 1, 2):
         raise RuntimeError("Unsupported serialize mode.")
-    saved = spconv.SERIALIZATION_MODE
-    spconv.SERIALIZATION_MODE = serialize_mode
-    try:
-        return SparseConv3dFunction._get_output_coords(in_coords.contiguous(), torch.Size([B, 0, W, H, D]), (Kw, Kh, Kd),
-                                                       (Sw, Sh, Sd), (Pw, Ph, Pd), (Dw, Dh, Dd))
-    finally:
-        spconv.SERIALIZATION_MODE = saved
+    return SparseConv3dFunction._get_output_coords(in_coords.contiguous(), torch.Size([B, 0, W, H, D]), (Kw, Kh, Kd),
+                                                   (Sw, Sh, Sd), (Pw, Ph, Pd), (Dw, Dh, Dd), serialization_mode=serialize_mode)
 
 
 def hashmap_build_sparse_conv_out_coords(in_coords: torch.Tensor, hashmap_ratio: float, serialize_mode: int, B: int, W: int,
@@ -242,16 +236,11 @@ def hashmap_build_sparse_conv_neighbour_map(in_coords: torch.Tensor, out_coords:
                                             Dd: int):
     """(neighbor_map uint32 [L, V], neighbor_map_bwd uint32 [M, V] -- an empty tensor when include_bwd is false)
     (sparse_neighbor_map.h:88-131)."""
-    from ..ops import spconv
     from ..ops.spconv.sparse_conv3d import _build_maps
     dev = _on_gpu(in_coords, out_coords)
-    saved = spconv.HASHMAP_RATIO
-    spconv.HASHMAP_RATIO = float(hashmap_ratio)
-    try:
-        fwd, bwd, _, _ = _build_maps(in_coords.contiguous(), out_coords.contiguous(), torch.Size([B, 0, W, H, D]), (Kw, Kh, Kd),
-                                     (Sw, Sh, Sd), (Pw, Ph, Pd), (Dw, Dh, Dd), bool(include_bwd), False)
-    finally:
-        spconv.HASHMAP_RATIO = saved
+    fwd, bwd, _, _ = _build_maps(in_coords.contiguous(), out_coords.contiguous(), torch.Size([B, 0, W, H, D]), (Kw, Kh, Kd),
+                                 (Sw, Sh, Sd), (Pw, Ph, Pd), (Dw, Dh, Dd), bool(include_bwd), False,
+                                 hashmap_ratio=hashmap_ratio)
     if bwd is None:
         bwd = torch.empty((0,), dtype=torch.uint32, device=dev)
     return fwd, bwd

@@ -80,8 +80,10 @@ class SparseConv3dNeighborCache(SubMConv3dNeighborCache):
 
 
 def _build_maps(coords: torch.Tensor, out_coords: torch.Tensor, shape, kernel_size, stride, padding, dilation,
-                with_bwd: bool, with_codes: bool):
-    """(map_fwd [L, V], map_bwd [M, V] | None, gray | None, binary | None), by hash probes or by sort and merge."""
+                with_bwd: bool, with_codes: bool, hashmap_ratio: Optional[float] = None):
+    """(map_fwd [L, V], map_bwd [M, V] | None, gray | None, binary | None), by hash probes or by sort and merge.
+    hashmap_ratio: table slots per input voxel for the hash builder (default: spconv.HASHMAP_RATIO)."""
+    ratio = spconv.HASHMAP_RATIO if hashmap_ratio is None else float(hashmap_ratio)
     m, l = coords.shape[0], out_coords.shape[0]
     _, _, W, H, D = [int(s) for s in shape]
     kw, kh, kd = kernel_size
@@ -112,9 +114,9 @@ def _build_maps(coords: torch.Tensor, out_coords: torch.Tensor, shape, kernel_si
                 C.c_int(key_bits), nat.ptr(ws), nat.sz(ws.numel()), nat.ptr(nmap), nat.ptr(nmap_bwd), nat.ptr(gray), nat.ptr(binary),
                 nat.stream()))
         return nmap, nmap_bwd, gray, binary
-    table = int(spconv.HASHMAP_RATIO * m)
+    table = int(ratio * m)
     if m > 0 and table < m:
-        raise ValueError(f"hashmap ratio {spconv.HASHMAP_RATIO} gives a table smaller than the input")
+        raise ValueError(f"hashmap ratio {ratio} gives a table smaller than the input")
     keys = vals = None
     key_bits = 32
     with torch.cuda.device(dev):
@@ -141,6 +143,7 @@ class SparseConv3dFunction(Function):
         stride: Tuple[int, int, int],
         padding: Tuple[int, int, int],
         dilation: Tuple[int, int, int],
+        serialization_mode: Optional[int] = None,
     ) -> torch.Tensor:
         """int32 [L, 4] output coordinates (reference: sparse_conv3d.py:60-94), sorted by (b, x, y, z) under
         SerializationMode.BXYZ, along the z-order or Hilbert curve under the other two modes.
@@ -148,14 +151,15 @@ class SparseConv3dFunction(Function):
         Both of the reference's OUT_COORD_ALGO values name the same result; on gfx950 one streaming pass (candidate
         keys, radix sort, unique) serves both.  The curve modes re-sort the unique coordinates by their code; the bits
         per axis come from the INPUT grid, as in the reference (sparse_neighbor_map.cu:157-160), which fixes the
-        orientation of the Hilbert curve."""
+        orientation of the Hilbert curve.  serialization_mode overrides spconv.SERIALIZATION_MODE for this call."""
+        mode = spconv.SERIALIZATION_MODE if serialization_mode is None else serialization_mode
         assert coords.is_contiguous(), "Coords should be contiguous"
         assert coords.dtype in [torch.int32], "Unsupported coords dtype. Expect int32"
         if not coords.is_cuda:
             raise NotImplementedError("CPU version is not implemented")
         if spconv.OUT_COORD_ALGO not in (SparseConv3dOutCoordAlgorithm.HASHMAP, SparseConv3dOutCoordAlgorithm.EXPAND_UNIQUE):
             raise ValueError(f"Unsupported output-coordinate algorithm {spconv.OUT_COORD_ALGO}")
-        if spconv.SERIALIZATION_MODE not in (SerializationMode.BXYZ, SerializationMode.Z_ORDER, SerializationMode.HILBERT):
+        if mode not in (SerializationMode.BXYZ, SerializationMode.Z_ORDER, SerializationMode.HILBERT):
             raise ValueError("Unsupported serialize mode.")
         B, _, W, H, D = [int(s) for s in shape]
         ks, st, pd, dl = _triple(kernel_size), _triple(stride), _triple(padding), _triple(dilation)
@@ -182,11 +186,11 @@ class SparseConv3dFunction(Function):
             out = torch.empty((total, 4), dtype=torch.int32, device=dev)
             nat.check(L.fgx_spconv_out_coords_decode(nat.ptr(ws), C.c_int(key_bits), nat.sz(total), C.c_int(wo), C.c_int(ho),
                                                      C.c_int(do), nat.ptr(out), nat.stream()))
-        if spconv.SERIALIZATION_MODE != SerializationMode.BXYZ:
+        if mode != SerializationMode.BXYZ:
             bit_length = (max(W, H, D) - 1).bit_length()
             if max(wo, ho, do) > (1 << bit_length):
                 raise ValueError("output grid exceeds the bits per axis of the input grid: curve codes would collide")
-            out = serialize.reorder_coords(out, bit_length, (B - 1).bit_length(), int(spconv.SERIALIZATION_MODE))
+            out = serialize.reorder_coords(out, bit_length, (B - 1).bit_length(), int(mode))
         return out
 
     @staticmethod
