@@ -17,6 +17,7 @@ _lib: Optional[C.CDLL] = None
 
 FGX_F16, FGX_BF16, FGX_F32 = 0, 1, 2
 DTYPE_CODE = {torch.float16: FGX_F16, torch.bfloat16: FGX_BF16, torch.float32: FGX_F32}
+ACT_NONE, ACT_RELU = 0, 1          # FGX_ACT_* of the public header
 PASS_FWD, PASS_DGRAD, PASS_WGRAD = 0, 1, 2
 
 # every symbol the header declares; the CPU-side test checks that the library exports each of them
@@ -29,8 +30,8 @@ EXPORTS = [
     "fgx_pair_workspace_bytes", "fgx_pair_count", "fgx_pair_fill",
     "fgx_tile_workspace_bytes", "fgx_tile_codes", "fgx_tile_fill",
     "fgx_table_lookup", "fgx_weight_panel_bytes", "fgx_pack_weight",
-    "fgx_conv_scratch_bytes", "fgx_conv_gather_gemm",
-    "fgx_gather_plan_count", "fgx_gather_plan_fill", "fgx_conv_gather_gemm_stream",
+    "fgx_conv_scratch_bytes", "fgx_conv_gather_gemm", "fgx_conv_gather_gemm_act",
+    "fgx_gather_plan_count", "fgx_gather_plan_fill", "fgx_conv_gather_gemm_stream", "fgx_conv_gather_gemm_stream_act",
     "fgx_conv_gather_gemm_stream_groups", "fgx_gather_item_order_workspace_bytes", "fgx_gather_item_order",
     "fgx_wgrad_scratch_bytes", "fgx_wgrad_block_bounds_count", "fgx_wgrad_block_bounds", "fgx_conv_wgrad",
     "fgx_colsum_scratch_bytes", "fgx_colsum",

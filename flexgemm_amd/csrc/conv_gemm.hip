@@ -152,7 +152,7 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
                    const typename Tag::type* __restrict__ bias, const uint32_t* __restrict__ map,
                    const int64_t* __restrict__ sorted_idx, const int32_t* __restrict__ tile_code, uint32_t n, int K,
                    int cols, int cols_pad, int V, int splitk, unsigned row_tiles, unsigned col_tiles,
-                   float* __restrict__ partial, typename Tag::type* __restrict__ out) {
+                   float* __restrict__ partial, int act, typename Tag::type* __restrict__ out) {
     using C = GemmCfg<Tag, BM, BN, WAVES_M, WAVES_N, S, CH>;
     using T = typename Tag::type;
     constexpr int NT = C::NT;
@@ -412,7 +412,7 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int r = (e >> 2) * 8 + g * 4 + (e & 3);
-                *(T*)(band + r * C::OUT_PITCH + (j * 32 + l32) * C::ES) = from_float<T>(acc[i][j][e] + bv[j]);
+                *(T*)(band + r * C::OUT_PITCH + (j * 32 + l32) * C::ES) = from_float<T>(activate(acc[i][j][e] + bv[j], act));
             }
         // same wavefront wrote and reads: program order inside the wavefront suffices for LDS
 #pragma unroll
@@ -433,14 +433,14 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
     }
 }
 
-// out[i] = sum_s partial[s][i]
+// out[i] = act(sum_s partial[s][i])   (slice 0 carries the bias)
 template <typename T>
 __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restrict__ partial, int splitk, size_t numel,
-                                                            T* __restrict__ out) {
+                                                            int act, T* __restrict__ out) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < numel; i += (size_t)gridDim.x * 256) {
         float s = 0.f;
         for (int k = 0; k < splitk; ++k) s += partial[(size_t)k * numel + i];
-        out[i] = from_float<T>(s);
+        out[i] = from_float<T>(activate(s, act));
     }
 }
 
@@ -543,7 +543,7 @@ bool dtype_ok(int dtype) { return dtype == FGX_F16 || dtype == FGX_BF16 || dtype
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int S, int CH>
 int launch_gemm(const void* src, const void* panel, const void* bias, const uint32_t* map, const int64_t* sorted_idx,
                 const int32_t* tile_code, size_t n, int K, int cols, int cols_pad, int V, int splitk, void* scratch,
-                void* out, hipStream_t s) {
+                int act, void* out, hipStream_t s) {
     using C = GemmCfg<Tag, BM, BN, WAVES_M, WAVES_N, S, CH>;
     using T = typename Tag::type;
     auto kern = gather_gemm_kernel<Tag, BM, BN, WAVES_M, WAVES_N, S, CH>;
@@ -559,13 +559,13 @@ int launch_gemm(const void* src, const void* panel, const void* bias, const uint
     const unsigned grid_x = cdiv(total, kXcds) * kXcds;
     dim3 grid(grid_x, splitk, 1);
     kern<<<grid, C::NT, lds, s>>>((const T*)src, (const T*)panel, (const T*)bias, map, sorted_idx, tile_code, (uint32_t)n, K,
-                                  cols, cols_pad, V, splitk, row_tiles, col_tiles, (float*)scratch, (T*)out);
+                                  cols, cols_pad, V, splitk, row_tiles, col_tiles, (float*)scratch, act, (T*)out);
     FGX_CHECK_LAUNCH("fgx_conv_gather_gemm");
     if (splitk > 1) {
         size_t numel = n * (size_t)cols;
         unsigned g = cdiv(numel, 256);
         if (g > 65536u) g = 65536u;
-        splitk_reduce_kernel<T><<<g, 256, 0, s>>>((const float*)scratch, splitk, numel, (T*)out);
+        splitk_reduce_kernel<T><<<g, 256, 0, s>>>((const float*)scratch, splitk, numel, act, (T*)out);
         FGX_CHECK_LAUNCH("fgx_conv_gather_gemm(reduce)");
     }
     return FGX_OK;
@@ -574,11 +574,11 @@ int launch_gemm(const void* src, const void* panel, const void* bias, const uint
 template <typename Tag>
 int dispatch_tile(int tile_rows, int tile_cols, int slab_bytes, const void* src, const void* panel, const void* bias,
                   const uint32_t* map, const int64_t* sorted_idx, const int32_t* tile_code, size_t n, int K, int cols,
-                  int cols_pad, int V, int splitk, void* scratch, void* out, hipStream_t s) {
+                  int cols_pad, int V, int splitk, void* scratch, int act, void* out, hipStream_t s) {
 #define FGX_TILE(BM, BN, WMv, WNv, Sv, CHv)                                                                        \
     if (tile_rows == BM && tile_cols == BN && slab_bytes == CHv * 16)                                              \
         return launch_gemm<Tag, BM, BN, WMv, WNv, Sv, CHv>(src, panel, bias, map, sorted_idx, tile_code, n, K, cols, \
-                                                           cols_pad, V, splitk, scratch, out, s);
+                                                           cols_pad, V, splitk, scratch, act, out, s);
     FGX_TILE(256, 128, 2, 2, 3, 4)
     FGX_TILE(256, 128, 4, 2, 3, 8)
     FGX_TILE(128, 128, 2, 2, 3, 4)
@@ -655,6 +655,16 @@ int fgx_conv_gather_gemm(int dtype, const void* src, const void* panel, const vo
                          const int64_t* sorted_idx, const int32_t* tile_code, size_t n, int K, int cols, int V,
                          int tile_rows, int tile_cols, int slab_bytes, int splitk, void* scratch, void* out,
                          fgx_stream_t stream) {
+    return fgx_conv_gather_gemm_act(dtype, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, V, tile_rows, tile_cols,
+                                    slab_bytes, splitk, scratch, FGX_ACT_NONE, out, stream);
+}
+
+int fgx_conv_gather_gemm_act(int dtype, const void* src, const void* panel, const void* bias, const uint32_t* map,
+                             const int64_t* sorted_idx, const int32_t* tile_code, size_t n, int K, int cols, int V,
+                             int tile_rows, int tile_cols, int slab_bytes, int splitk, void* scratch, int activation,
+                             void* out, fgx_stream_t stream) {
+    FGX_CHECK_ARG(activation == FGX_ACT_NONE || activation == FGX_ACT_RELU, "fgx_conv_gather_gemm: unknown activation %d", activation);
+    const int act = activation;
     FGX_CHECK_ARG(dtype_ok(dtype), "fgx_conv_gather_gemm: unknown dtype %d", dtype);
     FGX_CHECK_ARG(K > 0 && cols > 0 && V >= 1 && V <= 32, "fgx_conv_gather_gemm: bad shape K=%d cols=%d V=%d", K, cols, V);
     FGX_CHECK_ARG(splitk >= 1 && splitk <= 1024, "fgx_conv_gather_gemm: splitk %d out of range", splitk);
@@ -669,9 +679,9 @@ int fgx_conv_gather_gemm(int dtype, const void* src, const void* panel, const vo
     const int cols_pad = (int)align_up((size_t)cols, (size_t)tile_cols);
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
-        case FGX_F16: return dispatch_tile<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, out, s);
-        case FGX_BF16: return dispatch_tile<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, out, s);
-        default: return dispatch_tile<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, out, s);
+        case FGX_F16: return dispatch_tile<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, act, out, s);
+        case FGX_BF16: return dispatch_tile<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, act, out, s);
+        default: return dispatch_tile<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, act, out, s);
     }
 }
 

@@ -107,7 +107,7 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
                           const uint32_t* __restrict__ plan_idx, const uint32_t* __restrict__ plan_band, uint32_t n, int K,
                           int cols, int cols_pad,
                           unsigned row_tiles, unsigned col_tiles, uint32_t src_bytes, uint32_t panel_bytes,
-                          uint32_t plan_bytes, const uint32_t* __restrict__ item_at,
+                          uint32_t plan_bytes, const uint32_t* __restrict__ item_at, int act,
                           typename Tag::type* __restrict__ out) {
     using C = StreamCfg<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
     using T = typename Tag::type;
@@ -449,10 +449,10 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
                         const int c = j * 32 + q * 8 + g * 4;                   // first of four columns
                         const f32x4 bv = *(const f32x4*)(bias_lds + col0 + c);
                         T pk[4];
-                        pk[0] = from_float<T>(acc[i][j][q * 4 + 0] + bv.x);
-                        pk[1] = from_float<T>(acc[i][j][q * 4 + 1] + bv.y);
-                        pk[2] = from_float<T>(acc[i][j][q * 4 + 2] + bv.z);
-                        pk[3] = from_float<T>(acc[i][j][q * 4 + 3] + bv.w);
+                        pk[0] = from_float<T>(activate(acc[i][j][q * 4 + 0] + bv.x, act));
+                        pk[1] = from_float<T>(activate(acc[i][j][q * 4 + 1] + bv.y, act));
+                        pk[2] = from_float<T>(activate(acc[i][j][q * 4 + 2] + bv.z, act));
+                        pk[3] = from_float<T>(activate(acc[i][j][q * 4 + 3] + bv.w, act));
                         unsigned char* dstp = band + r * C::OUT_PITCH + c * C::ES;
                         if constexpr (C::ES == 2) *(uint64_t*)dstp = __builtin_bit_cast(uint64_t, pk);
                         else *(u32x4*)dstp = __builtin_bit_cast(u32x4, pk);
@@ -510,7 +510,7 @@ template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int CH>
 int launch_stream(const void* src, const void* panel, const void* bias, const int64_t* order, const int32_t* plan_seg,
                   const int32_t* tile_code, const uint32_t* plan_idx, const uint32_t* plan_band, size_t plan_rows, size_t n,
                   size_t n_src, int K, int cols, int cols_pad, size_t panel_bytes, const uint32_t* item_at, int max_groups,
-                  void* out, hipStream_t s) {
+                  int act, void* out, hipStream_t s) {
     using C = StreamCfg<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
     using T = typename Tag::type;
     auto kern = gather_gemm_stream_kernel<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
@@ -534,7 +534,7 @@ int launch_stream(const void* src, const void* panel, const void* bias, const in
     kern<<<groups, C::NT, lds, s>>>((const T*)src, (const T*)panel, (const T*)bias, order, plan_seg, tile_code, plan_idx,
                                     plan_band, (uint32_t)n, K, cols, cols_pad, row_tiles, col_tiles,
                                     (uint32_t)(n_src * (size_t)K * sizeof(T)), (uint32_t)panel_bytes,
-                                    (uint32_t)(plan_rows * BM * 4), item_at, (T*)out);
+                                    (uint32_t)(plan_rows * BM * 4), item_at, act, (T*)out);
     FGX_CHECK_LAUNCH("fgx_conv_gather_gemm_stream");
     return FGX_OK;
 }
@@ -543,11 +543,11 @@ template <typename Tag>
 int dispatch_stream(int tile_rows, int tile_cols, int slab_bytes, const void* src, const void* panel, const void* bias,
                     const int64_t* order, const int32_t* plan_seg, const int32_t* tile_code, const uint32_t* plan_idx,
                     const uint32_t* plan_band, size_t plan_rows, size_t n, size_t n_src, int K, int cols, int cols_pad,
-                    size_t panel_bytes, const uint32_t* item_at, int max_groups, void* out, hipStream_t s) {
+                    size_t panel_bytes, const uint32_t* item_at, int max_groups, int act, void* out, hipStream_t s) {
 #define FGX_STREAM_TILE(BM, BN, WMv, WNv, CHv)                                                                          \
     if (tile_rows == BM && tile_cols == BN && slab_bytes == CHv * 16)                                                   \
         return launch_stream<Tag, BM, BN, WMv, WNv, CHv>(src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band,  \
-                                                         plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, out, s);
+                                                         plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, act, out, s);
     FGX_STREAM_TILE(256, 128, 4, 2, 8)
     FGX_STREAM_TILE(256, 64, 4, 2, 8)
     FGX_STREAM_TILE(256, 128, 4, 2, 4)      // 64-byte K-slabs: rows shorter than 128 bytes
@@ -569,6 +569,19 @@ extern "C" int fgx_conv_gather_gemm_stream(int dtype, const void* src, const voi
                                            size_t n_src, int K, int cols, int V,
                                            int tile_rows, int tile_cols, int slab_bytes, const uint32_t* item_at,
                                            int max_groups, void* out, fgx_stream_t stream) {
+    return fgx_conv_gather_gemm_stream_act(dtype, src, panel, bias, order, tile_code, plan_seg, plan_idx, plan_band, plan_rows,
+                                           n, n_src, K, cols, V, tile_rows, tile_cols, slab_bytes, item_at, max_groups,
+                                           FGX_ACT_NONE, out, stream);
+}
+
+extern "C" int fgx_conv_gather_gemm_stream_act(int dtype, const void* src, const void* panel, const void* bias,
+                                               const int64_t* order, const int32_t* tile_code, const int32_t* plan_seg,
+                                               const uint32_t* plan_idx, const uint32_t* plan_band, size_t plan_rows,
+                                               size_t n, size_t n_src, int K, int cols, int V,
+                                               int tile_rows, int tile_cols, int slab_bytes, const uint32_t* item_at,
+                                               int max_groups, int activation, void* out, fgx_stream_t stream) {
+    FGX_CHECK_ARG(activation == FGX_ACT_NONE || activation == FGX_ACT_RELU, "fgx_conv_gather_gemm_stream: unknown activation %d", activation);
+    const int act = activation;
     FGX_CHECK_ARG(dtype == FGX_F16 || dtype == FGX_BF16 || dtype == FGX_F32, "fgx_conv_gather_gemm_stream: unknown dtype %d", dtype);
     FGX_CHECK_ARG(K > 0 && cols > 0 && V >= 1 && V <= 32, "fgx_conv_gather_gemm_stream: bad shape K=%d cols=%d V=%d", K, cols, V);
     if (n == 0) return FGX_OK;
@@ -590,9 +603,9 @@ extern "C" int fgx_conv_gather_gemm_stream(int dtype, const void* src, const voi
     }
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
-        case FGX_F16: return dispatch_stream<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, out, s);
-        case FGX_BF16: return dispatch_stream<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, out, s);
-        default: return dispatch_stream<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, out, s);
+        case FGX_F16: return dispatch_stream<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, act, out, s);
+        case FGX_BF16: return dispatch_stream<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, act, out, s);
+        default: return dispatch_stream<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, act, out, s);
     }
 }
 

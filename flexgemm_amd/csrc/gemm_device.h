@@ -45,6 +45,9 @@ template <> __device__ __forceinline__ void mma<F32>(f32x16& acc, const u32x4& a
     acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af.w, bf.w, acc, 0, 0, 0);
 }
 
+// activation of the GEMM epilogues (FGX_ACT_* of the public header), applied to the fp32 sum before it is rounded
+__device__ __forceinline__ float activate(float x, int act) { return act == FGX_ACT_RELU ? fmaxf(x, 0.f) : x; }
+
 template <typename T> __device__ __forceinline__ T from_float(float x);
 template <> __device__ __forceinline__ _Float16 from_float<_Float16>(float x) { return (_Float16)x; }
 template <> __device__ __forceinline__ float from_float<float>(float x) { return x; }

@@ -91,5 +91,6 @@ def set_hashmap_ratio(ratio: float):
     HASHMAP_RATIO = ratio
 
 
-from .submanifold_conv3d import SubMConv3dFunction, SubMConv3dNeighborCache, sparse_submanifold_conv3d  # noqa: E402
+from .submanifold_conv3d import (SubMConv3dFunction, SubMConv3dNeighborCache, sparse_submanifold_conv3d,  # noqa: E402
+                                 sparse_submanifold_conv3d_relu)
 from .sparse_conv3d import SparseConv3dFunction, SparseConv3dNeighborCache, sparse_conv3d  # noqa: E402

@@ -386,12 +386,14 @@ def _weight_panel(owner: Optional[torch.Tensor], weight_cvk: torch.Tensor, code:
 
 
 def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[torch.Tensor], cache, mode: int,
-                 allow_splitk: bool, masked: bool = True, weight_owner: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 allow_splitk: bool, masked: bool = True, weight_owner: Optional[torch.Tensor] = None,
+                 activation: int = nat.ACT_NONE) -> torch.Tensor:
     """mode 0: out = conv(src) with weight [Co, V, Ci] (+bias); mode 1: grad_input from src = grad_output through the
     same map with the offsets mirrored (submanifold); mode 2: grad_input through a map of its own, offsets as they
     are (generic sparse convolution).  The result has one row per row of cache["neighbor_map"]; src may have a
     different number of rows.  masked=False: the non-masked schedule (natural row order, all offsets per tile).
-    weight_owner: the tensor the caller's weight lives in, for the optional panel cache (see _weight_panel)."""
+    weight_owner: the tensor the caller's weight lives in, for the optional panel cache (see _weight_panel).
+    activation: nat.ACT_RELU clamps (sum + bias) at zero in the kernel's epilogue."""
     co, v, ci = weight_cvk.shape
     n = cache["neighbor_map"].shape[0]
     n_src = src.shape[0]
@@ -404,7 +406,8 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
     dev = src.device
     if n_src == 0:      # nothing to gather: the bias alone
         out = torch.zeros((n, cols), dtype=dt, device=dev)
-        return out if bias is None else out + bias
+        out = out if bias is None else out + bias
+        return torch.relu(out) if activation == nat.ACT_RELU else out
     # rows must be whole 16-byte chunks: zero-pad the contraction dimension when they are not
     align = 16 // src.element_size()
     if k_true % align:
@@ -440,12 +443,12 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
             item_at = cache._item_order(plan_key, tile_code, -(-cols // sched.tile_cols), groups.value,
                                         -(-(k * src.element_size()) // sched.slab_bytes))
             nat.mark(name, "start")
-            nat.check(L.fgx_conv_gather_gemm_stream(
+            nat.check(L.fgx_conv_gather_gemm_stream_act(
                 C.c_int(code), nat.ptr(src), nat.ptr(panel), nat.ptr(bias), nat.ptr(order), nat.ptr(tile_code),
                 nat.ptr(plan_seg), nat.ptr(plan_idx), nat.ptr(plan_band), nat.sz(plan_idx.shape[0]), nat.sz(n), nat.sz(n_src),
                 C.c_int(k), C.c_int(cols), C.c_int(v),
                 C.c_int(sched.tile_rows), C.c_int(sched.tile_cols), C.c_int(sched.slab_bytes), nat.ptr(item_at),
-                C.c_int(groups.value), nat.ptr(out), nat.stream()))
+                C.c_int(groups.value), C.c_int(activation), nat.ptr(out), nat.stream()))
             nat.mark(name, "stop")
             return out
         if masked:
@@ -456,11 +459,11 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
         if splitk > 1:
             scratch = nat.workspace(L.fgx_conv_scratch_bytes(nat.sz(n), C.c_int(cols), C.c_int(splitk)), dev)
         nat.mark(name, "start")
-        nat.check(L.fgx_conv_gather_gemm(
+        nat.check(L.fgx_conv_gather_gemm_act(
             C.c_int(code), nat.ptr(src), nat.ptr(panel), nat.ptr(bias), nat.ptr(cache["neighbor_map"]),
             nat.ptr(order), nat.ptr(tile_code), nat.sz(n), C.c_int(k), C.c_int(cols), C.c_int(v),
             C.c_int(sched.tile_rows), C.c_int(sched.tile_cols), C.c_int(sched.slab_bytes), C.c_int(splitk),
-            nat.ptr(scratch), nat.ptr(out), nat.stream()))
+            nat.ptr(scratch), C.c_int(activation), nat.ptr(out), nat.stream()))
         nat.mark(name, "stop")
     return out
 
@@ -611,7 +614,9 @@ class SubMConv3dFunction(Function):
         neighbor_cache: SubMConv3dNeighborCache,
         weight: torch.Tensor,
         bias: Optional[torch.Tensor] = None,
+        relu: bool = False,
     ) -> torch.Tensor:
+        """relu (not in the reference): clamp the result at zero, in the GEMM's epilogue for the implicit algorithms."""
         assert feats.is_contiguous(), "Input features should be contiguous"
         co, kw, kh, kd, ci = weight.shape
         v = kw * kh * kd
@@ -619,11 +624,13 @@ class SubMConv3dFunction(Function):
         if algo == Algorithm.EXPLICIT_GEMM:
             col = _gathered_rows(feats, neighbor_cache["neighbor_map"])
             w = weight.reshape(co, v * ci).t()
-            return torch.addmm(bias, col, w) if bias is not None else torch.mm(col, w)
+            out = torch.addmm(bias, col, w) if bias is not None else torch.mm(col, w)
+            return torch.relu(out) if relu else out
         if algo in _IMPLICIT:
             _require_cuda(feats, "sparse_submanifold_conv3d")
             return _gather_gemm(feats, weight.reshape(co, v, ci), bias, neighbor_cache, 0, algo not in _NO_SPLITK,
-                                masked=algo in _MASKED, weight_owner=weight)
+                                masked=algo in _MASKED, weight_owner=weight,
+                                activation=nat.ACT_RELU if relu else nat.ACT_NONE)
         raise ValueError(f"Unsupported algorithm {algo}")
 
     @staticmethod
@@ -681,21 +688,30 @@ class SubMConv3dFunction(Function):
         weight: torch.Tensor,
         bias: Optional[torch.Tensor] = None,
         dilation: Tuple[int, int, int] = (1, 1, 1),
+        relu: bool = False,
     ) -> Tuple[torch.Tensor, SubMConv3dNeighborCache]:
         co, kw, kh, kd, ci = weight.shape
         assert feats.shape[-1] == ci, f"Input channels ({feats.shape[-1]}) should match weight channels ({ci})"
         need_grad = any(ctx.needs_input_grad)
         if neighbor_cache is None:
             neighbor_cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (kw, kh, kd), dilation, need_grad)
-        output = SubMConv3dFunction._sparse_submanifold_conv_forward(feats, neighbor_cache, weight, bias)
-        ctx.save_for_backward(feats, weight, bias)
+        output = SubMConv3dFunction._sparse_submanifold_conv_forward(feats, neighbor_cache, weight, bias, relu=relu)
+        if relu:
+            ctx.save_for_backward(feats, weight, bias, output)      # the output's sign is the activation's derivative
+        else:
+            ctx.save_for_backward(feats, weight, bias)
+        ctx.relu = relu
         ctx.neighbor_cache = neighbor_cache
         ctx.weight_owner = weakref.ref(weight)      # the caller's tensor object: kept weight panels hang on it
         return output, neighbor_cache
 
     @staticmethod
     def backward(ctx, grad_output: torch.Tensor, _):
-        feats, weight, bias = ctx.saved_tensors
+        if ctx.relu:
+            feats, weight, bias, output = ctx.saved_tensors
+            grad_output = torch.where(output > 0, grad_output, torch.zeros((), dtype=grad_output.dtype, device=grad_output.device))
+        else:
+            feats, weight, bias = ctx.saved_tensors
         need_f, need_w, need_b = ctx.needs_input_grad[0], ctx.needs_input_grad[4], ctx.needs_input_grad[5]
         # the helper decides what to compute from requires_grad, as the reference does
         f = feats.detach().requires_grad_(need_f)
@@ -703,7 +719,7 @@ class SubMConv3dFunction(Function):
         b = None if bias is None else bias.detach().requires_grad_(need_b)
         grad_input, grad_weight, grad_bias = SubMConv3dFunction._sparse_submanifold_conv_backward(
             grad_output, f, ctx.neighbor_cache, w, b, weight_owner=ctx.weight_owner())
-        return grad_input, None, None, None, grad_weight, grad_bias, None
+        return grad_input, None, None, None, grad_weight, grad_bias, None, None
 
 
 def sparse_submanifold_conv3d(
@@ -732,3 +748,18 @@ def sparse_submanifold_conv3d(
         (output [N, Co], neighbor_cache)
     """
     return SubMConv3dFunction.apply(feats, coords, shape, neighbor_cache, weight, bias, dilation)
+
+
+def sparse_submanifold_conv3d_relu(
+    feats: torch.Tensor,
+    coords: torch.Tensor,
+    shape: torch.Size,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    neighbor_cache: Optional[SubMConv3dNeighborCache] = None,
+    dilation: Tuple[int, int, int] = (1, 1, 1),
+) -> Tuple[torch.Tensor, SubMConv3dNeighborCache]:
+    """relu(sparse_submanifold_conv3d(...)) with the clamp done in the GEMM's epilogue: the output is written once,
+    already activated (no counterpart in the reference; same arguments and return values as sparse_submanifold_conv3d).
+    Differentiable: backward masks the incoming gradient with the sign of the saved output and runs the usual passes."""
+    return SubMConv3dFunction.apply(feats, coords, shape, neighbor_cache, weight, bias, dilation, True)

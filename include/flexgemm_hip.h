@@ -36,6 +36,10 @@ extern "C" {
 #define FGX_BF16 1
 #define FGX_F32 2
 
+/* epilogue of the gather GEMMs: what is applied to (sum + bias) before it is rounded and stored */
+#define FGX_ACT_NONE 0
+#define FGX_ACT_RELU 1
+
 typedef void* fgx_stream_t;
 
 /* Library identity and error text. */
@@ -194,6 +198,15 @@ int fgx_conv_gather_gemm(int dtype, const void* src, const void* panel, const vo
                          size_t n, int K, int cols, int V, int tile_rows, int tile_cols, int slab_bytes, int splitk,
                          void* scratch, void* out, fgx_stream_t stream);
 
+/* fgx_conv_gather_gemm with an activation (FGX_ACT_*) applied to (sum + bias) in the kernel's epilogue -- with split-K, in
+ * the reduction of the partial sums -- so that out = act(conv + bias) costs no pass over the output of its own.
+ * No counterpart in the reference, whose kernels end with the bias add (..._fwd_masked_implicit_gemm.py:97-100); for
+ * inference graphs whose normalisation layers are folded into weight and bias. */
+int fgx_conv_gather_gemm_act(int dtype, const void* src, const void* panel, const void* bias,
+                             const uint32_t* map, const int64_t* sorted_idx, const int32_t* tile_code,
+                             size_t n, int K, int cols, int V, int tile_rows, int tile_cols, int slab_bytes, int splitk,
+                             void* scratch, int activation, void* out, fgx_stream_t stream);
+
 /* Gather plan of a row order for tiles of `tile_rows` rows: for tile t and the k-th offset v present in it
  * (the set bits of tile_code[t], ascending; a tile whose code is 0 gets one row with every neighbor missing),
  *   plan_idx[(plan_seg[t] + k) * tile_rows + r] = map[order[t * tile_rows + r], v]     (0xFFFFFFFF for rows past n),
@@ -232,6 +245,13 @@ int fgx_conv_gather_gemm_stream(int dtype, const void* src, const void* panel, c
                                 size_t n_src, int K, int cols, int V,
                                 int tile_rows, int tile_cols, int slab_bytes, const uint32_t* item_at,
                                 int max_groups, void* out, fgx_stream_t stream);
+/* ... with an activation (FGX_ACT_*) in the epilogue, as fgx_conv_gather_gemm_act; no counterpart in the reference. */
+int fgx_conv_gather_gemm_stream_act(int dtype, const void* src, const void* panel, const void* bias,
+                                    const int64_t* order, const int32_t* tile_code, const int32_t* plan_seg,
+                                    const uint32_t* plan_idx, const uint32_t* plan_band, size_t plan_rows, size_t n,
+                                    size_t n_src, int K, int cols, int V,
+                                    int tile_rows, int tile_cols, int slab_bytes, const uint32_t* item_at,
+                                    int max_groups, int activation, void* out, fgx_stream_t stream);
 int fgx_conv_gather_gemm_stream_groups(int dtype, int cols, int tile_rows, int tile_cols, int slab_bytes, int* groups);
 
 /* item_at for fgx_conv_gather_gemm_stream, made on the device from the tile codes: items sorted by cost (offsets per

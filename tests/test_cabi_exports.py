@@ -89,6 +89,15 @@ def test_argument_errors_map_to_exceptions(library):
         nat.check(L.fgx_conv_gather_gemm_stream(0, None, None, None, None, None, None, None, None, ctypes.c_size_t(0),
                                                 ctypes.c_size_t(10), ctypes.c_size_t(10), 128, 128, 27, 256, 128, 128, None, 0, None, None))
     assert b"null buffer" in L.fgx_last_error()
+    with pytest.raises(ValueError):   # an activation code the kernels do not know
+        nat.check(L.fgx_conv_gather_gemm_stream_act(0, None, None, None, None, None, None, None, None, ctypes.c_size_t(0),
+                                                    ctypes.c_size_t(10), ctypes.c_size_t(10), 128, 128, 27, 256, 128, 128, None, 0,
+                                                    7, None, None))
+    assert b"activation" in L.fgx_last_error()
+    with pytest.raises(ValueError):
+        nat.check(L.fgx_conv_gather_gemm_act(0, None, None, None, None, None, None, ctypes.c_size_t(10), 128, 128, 27, 128, 128, 64, 1,
+                                             None, 7, None, None))
+    assert b"activation" in L.fgx_last_error()
 
 
 def test_host_logic_without_gpu():

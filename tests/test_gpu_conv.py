@@ -614,3 +614,42 @@ def test_forward_replays_from_a_hip_graph(gpu_device, res, c):
             eager = stack(x)                     # the program's own eager work between the replays
             torch.cuda.synchronize()
             assert torch.equal(static_out, eager), f"replay {k} differs from the eager result"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("res,ci,co", [(48, 128, 128), (24, 64, 96), (8, 256, 64), (16, 20, 12)])
+def test_relu_in_the_epilogue_equals_relu_after_the_operator(gpu_device, dtype, res, ci, co):
+    """sparse_submanifold_conv3d_relu against torch.relu(sparse_submanifold_conv3d): rounding is monotonic and keeps
+    the sign, so the fused output equals the composed one bit for bit, and so do all gradients (the mask is the same).
+    Shapes cover the streaming kernel, the tiled kernel, its split-K reduction and zero-padded channel counts; one
+    comparison against the float64 oracle guards the pair against a common mistake."""
+    from flex_gemm.ops.spconv import sparse_submanifold_conv3d_relu
+    coords_np = reference_test_shell(res)
+    shape = torch.Size([1, ci, res, res, res])
+    feats, weight, bias, grad = _case(coords_np, ci, co, dtype, seed=res + ci)
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+    results = []
+    for fused in (False, True):
+        f = feats.to(gpu_device).requires_grad_(True)
+        w = weight.to(gpu_device).requires_grad_(True)
+        b = bias.to(gpu_device).requires_grad_(True)
+        if fused:
+            out, _ = sparse_submanifold_conv3d_relu(f, coords, shape, w, b, neighbor_cache=cache)
+        else:
+            out = torch.relu(sparse_submanifold_conv3d(f, coords, shape, w, b, neighbor_cache=cache)[0])
+        out.backward(grad.to(gpu_device))
+        torch.cuda.synchronize()
+        results.append((out.detach(), f.grad, w.grad, b.grad))
+    _say(f"fused relu res={res} ci={ci} co={co} {dtype}")
+    for name, a, b_ in zip(("output", "dgrad", "wgrad", "dbias"), results[0], results[1]):
+        assert torch.equal(a, b_), f"{name}: fused and composed results differ"
+    assert (results[1][0] >= 0).all() and (results[1][0] == 0).any() and (results[1][0] > 0).any()
+    nmap = torch.from_numpy(nb.neighbor_map(coords_np, tuple(shape), (3, 3, 3), (1, 1, 1)).view(np.int32))
+    ref = torch.relu(eg.forward(feats.double(), nmap, weight.double(), bias.double()))
+    _assert_close(results[1][0], ref, dtype, "fused relu forward")
+    # without a bias, and without gradients
+    with torch.no_grad():
+        a = sparse_submanifold_conv3d_relu(feats.to(gpu_device), coords, shape, weight.to(gpu_device), None, cache)[0]
+        b_ = torch.relu(sparse_submanifold_conv3d(feats.to(gpu_device), coords, shape, weight.to(gpu_device), None, cache)[0])
+    assert torch.equal(a, b_)
