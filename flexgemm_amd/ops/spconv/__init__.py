@@ -93,4 +93,4 @@ def set_hashmap_ratio(ratio: float):
 
 from .submanifold_conv3d import (SubMConv3dFunction, SubMConv3dNeighborCache, sparse_submanifold_conv3d,  # noqa: E402
                                  sparse_submanifold_conv3d_relu)
-from .sparse_conv3d import SparseConv3dFunction, SparseConv3dNeighborCache, sparse_conv3d  # noqa: E402
+from .sparse_conv3d import SparseConv3dFunction, SparseConv3dNeighborCache, sparse_conv3d, sparse_conv3d_relu  # noqa: E402

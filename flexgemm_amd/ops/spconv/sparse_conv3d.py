@@ -314,7 +314,9 @@ class SparseConv3dFunction(Function):
         neighbor_cache: SparseConv3dNeighborCache,
         weight: torch.Tensor,
         bias: Optional[torch.Tensor] = None,
+        relu: bool = False,
     ) -> torch.Tensor:
+        """relu (not in the reference): clamp the result at zero, in the GEMM's epilogue for the implicit algorithms."""
         assert feats.is_contiguous(), "Input features should be contiguous"
         co, kw, kh, kd, ci = weight.shape
         v = kw * kh * kd
@@ -322,11 +324,13 @@ class SparseConv3dFunction(Function):
         if algo == Algorithm.EXPLICIT_GEMM:
             col = _gathered_rows(feats, neighbor_cache["neighbor_map"])
             w = weight.reshape(co, v * ci).t()
-            return torch.addmm(bias, col, w) if bias is not None else torch.mm(col, w)
+            out = torch.addmm(bias, col, w) if bias is not None else torch.mm(col, w)
+            return torch.relu(out) if relu else out
         if algo in _IMPLICIT:
             _require_cuda(feats, "sparse_conv3d")
             return _gather_gemm(feats, weight.reshape(co, v, ci), bias, neighbor_cache, 0, algo not in _NO_SPLITK,
-                                masked=algo in _MASKED, weight_owner=weight)
+                                masked=algo in _MASKED, weight_owner=weight,
+                                activation=nat.ACT_RELU if relu else nat.ACT_NONE)
         raise ValueError(f"Unsupported algorithm {algo}")
 
     @staticmethod
@@ -383,6 +387,7 @@ class SparseConv3dFunction(Function):
         stride: Tuple[int, int, int] = (1, 1, 1),
         padding: Tuple[int, int, int] = (0, 0, 0),
         dilation: Tuple[int, int, int] = (1, 1, 1),
+        relu: bool = False,
     ):
         co, kw, kh, kd, ci = weight.shape
         assert feats.shape[-1] == ci, f"Input channels ({feats.shape[-1]}) should match weight channels ({ci})"
@@ -393,8 +398,12 @@ class SparseConv3dFunction(Function):
         if neighbor_cache is None:
             neighbor_cache = SparseConv3dFunction._compute_neighbor_cache(coords, out_coords, shape, (kw, kh, kd), stride,
                                                                           padding, dilation, need_grad, given)
-        output = SparseConv3dFunction._sparse_conv_forward(feats, neighbor_cache, weight, bias)
-        ctx.save_for_backward(feats, weight, bias)
+        output = SparseConv3dFunction._sparse_conv_forward(feats, neighbor_cache, weight, bias, relu=relu)
+        if relu:
+            ctx.save_for_backward(feats, weight, bias, output)      # the output's sign is the activation's derivative
+        else:
+            ctx.save_for_backward(feats, weight, bias)
+        ctx.relu = relu
         ctx.neighbor_cache = neighbor_cache
         ctx.weight_owner = weakref.ref(weight)      # the caller's tensor object: kept weight panels hang on it
         ctx.mark_non_differentiable(out_coords)
@@ -402,14 +411,18 @@ class SparseConv3dFunction(Function):
 
     @staticmethod
     def backward(ctx, grad_output: torch.Tensor, _, __):
-        feats, weight, bias = ctx.saved_tensors
+        if ctx.relu:
+            feats, weight, bias, output = ctx.saved_tensors
+            grad_output = torch.where(output > 0, grad_output, torch.zeros((), dtype=grad_output.dtype, device=grad_output.device))
+        else:
+            feats, weight, bias = ctx.saved_tensors
         need_f, need_w, need_b = ctx.needs_input_grad[0], ctx.needs_input_grad[4], ctx.needs_input_grad[5]
         f = feats.detach().requires_grad_(need_f)
         w = weight.detach().requires_grad_(need_w)
         b = None if bias is None else bias.detach().requires_grad_(need_b)
         grad_input, grad_weight, grad_bias = SparseConv3dFunction._sparse_conv_backward(grad_output, f, ctx.neighbor_cache, w, b,
                                                                                         weight_owner=ctx.weight_owner())
-        return grad_input, None, None, None, grad_weight, grad_bias, None, None, None, None
+        return grad_input, None, None, None, grad_weight, grad_bias, None, None, None, None, None
 
 
 def sparse_conv3d(
@@ -443,3 +456,22 @@ def sparse_conv3d(
         (out_feats [M, Co], out_coords [M, 4], neighbor_cache)
     """
     return SparseConv3dFunction.apply(feats, coords, shape, neighbor_cache, weight, bias, out_coords, stride, padding, dilation)
+
+
+def sparse_conv3d_relu(
+    feats: torch.Tensor,
+    coords: torch.Tensor,
+    shape: torch.Size,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    neighbor_cache: Optional[SparseConv3dNeighborCache] = None,
+    out_coords: Optional[torch.Tensor] = None,
+    stride: Tuple[int, int, int] = (1, 1, 1),
+    padding: Tuple[int, int, int] = (0, 0, 0),
+    dilation: Tuple[int, int, int] = (1, 1, 1),
+) -> Tuple[torch.Tensor, torch.Tensor, SparseConv3dNeighborCache]:
+    """relu(sparse_conv3d(...)) with the clamp done in the GEMM's epilogue (no counterpart in the reference; same
+    arguments and return values as sparse_conv3d).  Differentiable: backward masks the incoming gradient with the sign
+    of the saved output and runs the usual passes."""
+    return SparseConv3dFunction.apply(feats, coords, shape, neighbor_cache, weight, bias, out_coords, stride, padding, dilation,
+                                      True)

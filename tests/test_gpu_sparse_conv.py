@@ -290,3 +290,41 @@ def test_empty_input(gpu_device):
     _say("sparse conv, empty input")
     out, oc, cache = sparse_conv3d(f, none, shape, w, None, padding=(1, 1, 1))
     assert out.shape == (0, 8) and oc.shape == (0, 4) and cache.neighbor_map.shape == (0, 27)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("geom", [GEOMS[0], GEOMS[2], GEOMS[3]])
+def test_relu_in_the_epilogue_equals_relu_after_the_operator(gpu_device, dtype, geom):
+    """sparse_conv3d_relu against torch.relu(sparse_conv3d): same bits in the output and in every gradient."""
+    from flex_gemm.ops.spconv import sparse_conv3d_relu
+    res, ci, co = 24, 64, 96
+    ks, st, pd, dl = geom
+    coords_np = _shell(res, 2, shuffle_seed=7)
+    shape = torch.Size([2, 0, res, res, res])
+    g = torch.Generator().manual_seed(17)
+    m = len(coords_np)
+    v = ks[0] * ks[1] * ks[2]
+    feats = torch.randn(m, ci, generator=g).to(dtype)
+    weight = (torch.randn(co, *ks, ci, generator=g) / math.sqrt(v * ci)).to(dtype)
+    bias = torch.randn(co, generator=g).to(dtype)
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    results = []
+    grad = None
+    _say(f"fused relu, generic conv geom={geom} {dtype}")
+    for fused in (False, True):
+        f = feats.to(gpu_device).requires_grad_(True)
+        w = weight.to(gpu_device).requires_grad_(True)
+        b = bias.to(gpu_device).requires_grad_(True)
+        if fused:
+            out, oc, _ = sparse_conv3d_relu(f, coords, shape, w, b, stride=st, padding=pd, dilation=dl)
+        else:
+            out, oc, _ = sparse_conv3d(f, coords, shape, w, b, stride=st, padding=pd, dilation=dl)
+            out = torch.relu(out)
+        if grad is None:
+            grad = torch.randn(out.shape, generator=g).to(dtype).to(gpu_device)
+        out.backward(grad)
+        torch.cuda.synchronize()
+        results.append((out.detach(), f.grad, w.grad, b.grad, oc))
+    for name, a, b_ in zip(("output", "dgrad", "wgrad", "dbias", "out_coords"), results[0], results[1]):
+        assert torch.equal(a, b_), f"{name}: fused and composed results differ"
+    assert (results[1][0] == 0).any() and (results[1][0] > 0).any()
