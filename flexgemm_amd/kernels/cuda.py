@@ -148,12 +148,19 @@ def hashmap_build_grid_sample_3d_trilinear_neighbor_map_weight(*args, **kwargs):
 
 # ---- convolution tables (flex_gemm/kernels/cuda/spconv/*.h) ---------------------------------------------------------
 
+def _check_map(neighbor_map: torch.Tensor) -> None:
+    assert neighbor_map.dtype == torch.uint32 and neighbor_map.ndim == 2, "neighbor_map must be uint32 [N, V]"
+    assert neighbor_map.shape[1] <= 32, "Currently, the max kernel volume is 32 because kernel mask is encoded as uint32"
+
+
 def hashmap_build_submanifold_conv_neighbour_map(hashmap_keys: torch.Tensor, hashmap_vals: torch.Tensor, coords: torch.Tensor,
                                                  W: int, H: int, D: int, Kw: int, Kh: int, Kd: int, Dw: int, Dh: int,
                                                  Dd: int) -> torch.Tensor:
     """uint32 [N, Kw*Kh*Kd] neighbor map; fills the caller's (initialised) table with the voxels on the way
     (subm_neighbor_map.h:40-47, .cu:104-162)."""
     dev = _on_gpu(hashmap_keys, hashmap_vals, coords)
+    assert hashmap_vals.dtype == torch.uint32, "the neighbor-map builder keeps row numbers: hashmap values must be uint32"
+    assert hashmap_keys.shape[0] == hashmap_vals.shape[0], "key and value tables must have one length"
     hashmap_insert_3d_idx_as_val(hashmap_keys, hashmap_vals, coords, W, H, D)
     coords = coords.contiguous()
     n = coords.shape[0]
@@ -170,6 +177,7 @@ def neighbor_map_post_process_for_masked_implicit_gemm_1_no_bwd(neighbor_map: to
     """(gray_code int32 [N], sorted_idx int64 [N])   (migemm_neighmap_pp.h:33-44)."""
     from ..ops.spconv.submanifold_conv3d import _codes_and_order
     _on_gpu(neighbor_map)
+    _check_map(neighbor_map)
     gray, _, order = _codes_and_order(neighbor_map.contiguous(), None, None)
     return gray, order
 
@@ -178,6 +186,7 @@ def neighbor_map_post_process_for_masked_implicit_gemm_1(neighbor_map: torch.Ten
     """(gray_code, sorted_idx, valid_signal_i, valid_signal_o, valid_signal_seg)   (migemm_neighmap_pp.h:46-58)."""
     from ..ops.spconv.submanifold_conv3d import _codes_and_order, _pair_lists
     _on_gpu(neighbor_map)
+    _check_map(neighbor_map)
     nmap = neighbor_map.contiguous()
     gray, _, order = _codes_and_order(nmap, None, None)
     sig_i, sig_o, seg, _ = _pair_lists(nmap, gray)
@@ -188,6 +197,10 @@ def neighbor_map_post_process_for_masked_implicit_gemm_2(gray_code: torch.Tensor
                                                          block_size: int) -> Tuple[torch.Tensor, torch.Tensor]:
     """(valid_kernel int32 [sum], valid_kernel_seg int32 [ceil(N / block_size) + 1])   (migemm_neighmap_pp.h:60-70)."""
     dev = _on_gpu(gray_code, sorted_idx)
+    assert gray_code.dtype == torch.int32 and gray_code.ndim == 1, "gray_code must be int32 [N]"
+    assert sorted_idx.dtype == torch.int64 and sorted_idx.shape == gray_code.shape, "sorted_idx must be int64 [N]"
+    if int(block_size) < 1:
+        raise ValueError(f"block_size must be positive, got {block_size}")
     n = gray_code.shape[0]
     block_size = int(block_size)
     nb = (n + block_size - 1) // block_size

@@ -52,7 +52,19 @@ def _tables_of(neighbor: torch.Tensor, **given) -> SubMConv3dNeighborCache:
     the last four combinations seen with this map are kept)."""
     _require_cuda(neighbor, "flex_gemm.kernels.triton")
     assert neighbor.is_contiguous(), "Matrix neighbor must be contiguous"
+    assert neighbor.dtype == torch.uint32 and neighbor.ndim == 2 and neighbor.shape[1] <= 32, "neighbor must be uint32 [N, V <= 32]"
     given = {k: v for k, v in given.items() if v is not None}
+    n, v = neighbor.shape
+    for k, t in given.items():
+        assert t.is_cuda and t.device == neighbor.device, f"{k} must live on the device of neighbor"
+        if k == "sorted_idx":
+            assert t.dtype == torch.int64 and tuple(t.shape) == (n,), "sorted_idx must be int64 [N]"
+        else:
+            assert t.dtype == torch.uint32 and t.ndim == 1, f"{k} must be a uint32 vector"
+    if "valid_signal_seg" in given:
+        assert given["valid_signal_seg"].shape[0] == v + 1, "valid_signal_seg must have V + 1 entries"
+    if "valid_signal_i" in given and "valid_signal_o" in given:
+        assert given["valid_signal_i"].shape == given["valid_signal_o"].shape, "valid_signal_i / _o must have one length"
     kept = neighbor.__dict__.setdefault("_fgx_kernel_tables", [])
     tables = next((t for t in kept if _fits(t, given)), None)
     if tables is None:
@@ -75,6 +87,7 @@ def _tables_of(neighbor: torch.Tensor, **given) -> SubMConv3dNeighborCache:
 
 
 def _check_fwd(input: torch.Tensor, weight: torch.Tensor, neighbor: torch.Tensor, transposed: bool = False) -> None:
+    assert weight.ndim == 3 and weight.shape[1] == neighbor.shape[1], "weight must be [Co, V, Ci] with V = neighbor.shape[1]"
     assert input.shape[1] == (weight.shape[0] if transposed else weight.shape[2]), "Incompatible dimensions"
     assert input.is_contiguous(), "Matrix input must be contiguous"
     assert weight.is_contiguous(), "Matrix weight must be contiguous"

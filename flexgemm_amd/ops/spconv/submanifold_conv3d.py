@@ -488,6 +488,8 @@ def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int, with_b
     cip, cop = f.shape[1], g.shape[1]
     cache._ensure_pairs()
     seg_host = cache._seg_host()
+    if len(seg_host) != v + 1 or seg_host[-1] > min(cache["valid_signal_i"].numel(), cache["valid_signal_o"].numel()):
+        raise ValueError("valid_signal_seg does not fit the pair lists (V + 1 entries, the last one their length)")
     seg_arr = (C.c_uint32 * (v + 1))(*seg_host)
     sched = nat.table_lookup(nat.PASS_WGRAD, dt, n, cip, cop, v)
     gw = torch.empty((cop, v, cip), dtype=dt, device=dev)

@@ -187,3 +187,34 @@ def test_generic_kernel_calls(gpu_device, dtype, geom):
         gi = kernels.triton.sparse_conv_fwd_masked_implicit_gemm_splitk(go, w.detach(), None, nmap_bwd, cache["sorted_idx_bwd"],
                                                                         None, None, TRANSPOSE_WEIGHT=True)
         _close(gi, ref_gi, dtype, "masked dgrad through TRANSPOSE_WEIGHT")
+
+
+@pytest.mark.gpu
+def test_wrong_dtypes_and_shapes_are_refused_before_any_launch(gpu_device):
+    """Tables of the wrong element type would be read out of bounds by the kernels: the wrappers refuse them on the host."""
+    res, c = 8, 32
+    coords = torch.from_numpy(reference_test_shell(res)).to(gpu_device)
+    shape = torch.Size([1, c, res, res, res])
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+    n = coords.shape[0]
+    x = torch.randn(n, c, device=gpu_device).half()
+    w = torch.randn(c, 27, c, device=gpu_device).half()
+    nmap = cache["neighbor_map"]
+    with pytest.raises(AssertionError):     # sorted_idx must be int64
+        kernels.triton.sparse_submanifold_conv_fwd_masked_implicit_gemm(x, w, None, nmap, cache["sorted_idx"].int())
+    with pytest.raises(AssertionError):     # neighbor must be uint32
+        kernels.triton.sparse_submanifold_conv_fwd_implicit_gemm(x, w, None, nmap.view(torch.int32))
+    with pytest.raises(AssertionError):     # weight [Co, V, Ci] with the map's V
+        kernels.triton.sparse_submanifold_conv_fwd_implicit_gemm(x, w[:, :8].contiguous(), None, nmap)
+    with pytest.raises(AssertionError):     # pair lists must be uint32
+        kernels.triton.sparse_submanifold_conv_bwd_masked_implicit_gemm(
+            x, x.clone().requires_grad_(True), w.requires_grad_(True), None, nmap, cache["sorted_idx"], None, None,
+            cache["valid_signal_i"].view(torch.int32), cache["valid_signal_o"], cache["valid_signal_seg"])
+    with pytest.raises(ValueError):         # a segment table that names more pairs than the lists hold
+        kernels.triton.sparse_submanifold_conv_bwd_masked_implicit_gemm(
+            x, x.clone().requires_grad_(True), w.requires_grad_(True), None, nmap.clone(), cache["sorted_idx"], None, None,
+            cache["valid_signal_i"][:10].contiguous(), cache["valid_signal_o"][:10].contiguous(), cache["valid_signal_seg"])
+    with pytest.raises(AssertionError):
+        kernels.cuda.neighbor_map_post_process_for_masked_implicit_gemm_2(cache["gray_code"], cache["sorted_idx"].int(), 64)
+    with pytest.raises(AssertionError):
+        kernels.cuda.neighbor_map_post_process_for_masked_implicit_gemm_1(nmap.view(torch.int32))
