@@ -98,6 +98,7 @@ def _check_fwd(input: torch.Tensor, weight: torch.Tensor, neighbor: torch.Tensor
 
 def _subm_fwd(input, weight, bias, neighbor, splitk: bool, sorted_idx=None) -> torch.Tensor:
     _check_fwd(input, weight, neighbor)
+    assert input.shape[0] == neighbor.shape[0], "input and neighbor must have one row per voxel"
     tables = _tables_of(neighbor, sorted_idx=sorted_idx)
     return _gather_gemm(input, weight, bias, tables, 0, splitk, masked=sorted_idx is not None)
 
@@ -105,6 +106,8 @@ def _subm_fwd(input, weight, bias, neighbor, splitk: bool, sorted_idx=None) -> t
 def _subm_bwd(grad_output, input, weight, bias, neighbor, splitk: bool, sorted_idx=None, pairs=(None, None, None)):
     assert grad_output.is_contiguous(), "Matrix grad_output must be contiguous"
     _check_fwd(input, weight, neighbor)
+    assert input.shape[0] == neighbor.shape[0] and grad_output.shape[0] == neighbor.shape[0], \
+        "input, grad_output and neighbor must have one row per voxel"
     tables = _tables_of(neighbor, sorted_idx=sorted_idx, valid_signal_i=pairs[0], valid_signal_o=pairs[1],
                         valid_signal_seg=pairs[2])
     v = weight.shape[1]
@@ -202,6 +205,8 @@ def _conv_bwd(grad_output, input, weight, bias, neighbor, neighbor_bwd, splitk: 
     assert grad_output.is_contiguous(), "Matrix grad_output must be contiguous"
     _check_fwd(input, weight, neighbor)
     assert neighbor_bwd.is_contiguous(), "Matrix neighbor_bwd must be contiguous"
+    assert input.shape[0] == neighbor_bwd.shape[0] and grad_output.shape[0] == neighbor.shape[0], \
+        "input needs one row per row of neighbor_bwd, grad_output one per row of neighbor"
     grad_input = grad_weight = grad_bias = None
     if input.requires_grad:
         tables_bwd = _tables_of(neighbor_bwd, sorted_idx=sorted_idx_bwd)

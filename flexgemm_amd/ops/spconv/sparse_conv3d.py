@@ -246,11 +246,12 @@ class SparseConv3dFunction(Function):
         v = ks[0] * ks[1] * ks[2]
         if algo not in _MASKED:
             nmap, nmap_bwd, _, _ = _build_maps(coords, out_coords, shape, ks, st, pd, dl, needs_grad, with_codes=False)
-            return SparseConv3dNeighborCache(neighbor_map=nmap, neighbor_map_bwd=nmap_bwd)
+            return SparseConv3dNeighborCache(neighbor_map=nmap, neighbor_map_bwd=nmap_bwd, _n_in=coords.shape[0])
         assert v <= 32, "Currently, the max kernel volume is 32 because kernel mask is encoded as uint32"
         nmap, nmap_bwd, gray, binary = _build_maps(coords, out_coords, shape, ks, st, pd, dl, needs_grad, with_codes=True)
         gray, binary, order = _codes_and_order(nmap, gray, binary)
-        cache = SparseConv3dNeighborCache(neighbor_map=nmap, neighbor_map_bwd=nmap_bwd, gray_code=gray, sorted_idx=order)
+        cache = SparseConv3dNeighborCache(neighbor_map=nmap, neighbor_map_bwd=nmap_bwd, gray_code=gray, sorted_idx=order,
+                                          _n_in=coords.shape[0])
         if needs_grad:
             sig_i, sig_o, seg, seg_host = _pair_lists(nmap, gray)
             cache["valid_signal_seg"] = seg
@@ -318,6 +319,10 @@ class SparseConv3dFunction(Function):
     ) -> torch.Tensor:
         """relu (not in the reference): clamp the result at zero, in the GEMM's epilogue for the implicit algorithms."""
         assert feats.is_contiguous(), "Input features should be contiguous"
+        n_in = neighbor_cache["_n_in"]          # input voxels the maps were built for (absent on a hand-made cache)
+        if n_in is None and neighbor_cache["neighbor_map_bwd"] is not None:
+            n_in = neighbor_cache["neighbor_map_bwd"].shape[0]
+        assert n_in is None or feats.shape[0] == n_in, f"{feats.shape[0]} feature rows for a neighbor cache of {n_in} input voxels"
         co, kw, kh, kd, ci = weight.shape
         v = kw * kh * kd
         algo = spconv.ALGORITHM
@@ -345,6 +350,11 @@ class SparseConv3dFunction(Function):
         co, kw, kh, kd, ci = weight.shape
         v = kw * kh * kd
         algo = spconv.ALGORITHM
+        assert grad_output.shape[0] == neighbor_cache["neighbor_map"].shape[0], \
+            f"{grad_output.shape[0]} gradient rows for a neighbor cache of {neighbor_cache['neighbor_map'].shape[0]} output voxels"
+        if neighbor_cache["neighbor_map_bwd"] is not None:
+            assert feats.shape[0] == neighbor_cache["neighbor_map_bwd"].shape[0], \
+                f"{feats.shape[0]} feature rows for a neighbor cache of {neighbor_cache['neighbor_map_bwd'].shape[0]} input voxels"
         grad_input = grad_weight = grad_bias = None
         if algo == Algorithm.EXPLICIT_GEMM:
             if feats.requires_grad:

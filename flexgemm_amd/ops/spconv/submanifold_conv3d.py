@@ -620,6 +620,8 @@ class SubMConv3dFunction(Function):
     ) -> torch.Tensor:
         """relu (not in the reference): clamp the result at zero, in the GEMM's epilogue for the implicit algorithms."""
         assert feats.is_contiguous(), "Input features should be contiguous"
+        assert feats.shape[0] == neighbor_cache["neighbor_map"].shape[0], \
+            f"{feats.shape[0]} feature rows for a neighbor cache of {neighbor_cache['neighbor_map'].shape[0]} voxels"
         co, kw, kh, kd, ci = weight.shape
         v = kw * kh * kd
         algo = spconv.ALGORITHM
@@ -647,6 +649,9 @@ class SubMConv3dFunction(Function):
         co, kw, kh, kd, ci = weight.shape
         v = kw * kh * kd
         algo = spconv.ALGORITHM
+        n_rows = neighbor_cache["neighbor_map"].shape[0]
+        assert feats.shape[0] == n_rows and grad_output.shape[0] == n_rows, \
+            f"{feats.shape[0]} feature rows and {grad_output.shape[0]} gradient rows for a neighbor cache of {n_rows} voxels"
         grad_input = grad_weight = grad_bias = None
         if algo == Algorithm.EXPLICIT_GEMM:
             nmap = neighbor_cache["neighbor_map"]
