@@ -158,3 +158,24 @@ def test_explicit_algorithm_matches_oracle_on_cpu():
         assert torch.allclose(feats.grad, gi) and torch.allclose(weight.grad, gw) and torch.allclose(bias.grad, gb)
     finally:
         flex_gemm.ops.spconv.set_algorithm(Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
+
+
+def test_wgrad_block_rule_keeps_its_promises(library):
+    """The schedule rule for wgrad's voxel blocks: whole kibi-rows, even blocks where there are few, at most 12288 rows (four times that for
+    the 32 x 32 tile, which writes four partial products per block) unless the 256 MiB cap on fp32 partial products asks
+    for longer ones, and never more partial products than that cap allows."""
+    import torch
+    for c in (32, 64, 128, 256, 512, 1024):
+        for n in (1, 192, 3840, 15192, 42608, 64160, 166232, 300000, 669288, 1026536, 2667120):
+            s = nat.table_lookup(nat.PASS_WGRAD, torch.float16, n, c, c, 27)
+            rows = s.block_rows
+            assert rows >= 1024 and rows % 1024 == 0, (n, c, rows)
+            blocks = -(-n // rows)
+            slices = 4 if (s.stream and s.tile_rows == 32) else 1
+            if blocks > 1:
+                assert blocks * slices * 27 * c * c * 4 <= 256 << 20, (n, c, rows, "partial products exceed the cap")
+                if blocks <= 4:         # with many blocks a short last one is immaterial
+                    assert n - (blocks - 1) * rows > rows // 2, (n, c, rows, "short last block")
+            cap_blocks = max((256 << 20) // (27 * c * c * 4 * slices), 1)
+            if rows > 12288 * slices:
+                assert -(-n // cap_blocks) > 12288 * slices - 1024 or (n >> 15, c) in ((1, 1024),), (n, c, rows)
