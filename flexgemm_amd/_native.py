@@ -113,8 +113,19 @@ def workspace(nbytes: int, device) -> torch.Tensor:
     return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
 
 
+_schedules: dict = {}        # (pass, dtype, n, ci, co, v) -> bytes of the library's answer (a pure function of the key)
+
+
 def table_lookup(pass_kind: int, dtype: torch.dtype, n: int, ci: int, co: int, v: int) -> Schedule:
-    s = Schedule()
-    check(lib().fgx_table_lookup(C.c_int(pass_kind), C.c_int(DTYPE_CODE[dtype]), sz(n), C.c_int(ci), C.c_int(co),
-                                 C.c_int(v), C.byref(s)))
-    return s
+    """The library's schedule for a pass and shape.  Answers are remembered per key (the hot path asks on every call);
+    every caller gets a Schedule of its own, so changing its fields changes nothing for the next one."""
+    key = (pass_kind, dtype, int(n), int(ci), int(co), int(v))
+    raw = _schedules.get(key)
+    if raw is None:
+        s = Schedule()
+        check(lib().fgx_table_lookup(C.c_int(pass_kind), C.c_int(DTYPE_CODE[dtype]), sz(n), C.c_int(ci), C.c_int(co),
+                                     C.c_int(v), C.byref(s)))
+        if len(_schedules) > 4096:
+            _schedules.clear()
+        raw = _schedules[key] = bytes(s)
+    return Schedule.from_buffer_copy(raw)

@@ -342,6 +342,25 @@ def _pad_cols(t: torch.Tensor, mult: int) -> torch.Tensor:
 
 
 _panel_bytes_kept = 0       # bytes of weight panels kept with their weights (all devices)
+_pure_answers: dict = {}    # answers of the library's size / occupancy queries, which depend on their arguments alone
+
+
+def _panel_nbytes(code: int, mode: int, ci: int, co: int, v: int, slab_bytes: int, tile_cols: int) -> int:
+    key = ("panel", code, mode, ci, co, v, slab_bytes, tile_cols)
+    if key not in _pure_answers:
+        _pure_answers[key] = int(nat.lib().fgx_weight_panel_bytes(C.c_int(code), C.c_int(mode), C.c_int(ci), C.c_int(co), C.c_int(v),
+                                                                   C.c_int(slab_bytes), C.c_int(tile_cols)))
+    return _pure_answers[key]
+
+
+def _stream_groups(code: int, cols: int, tile_rows: int, tile_cols: int, slab_bytes: int, dev: torch.device) -> int:
+    key = ("groups", code, cols, tile_rows, tile_cols, slab_bytes, dev.index)
+    if key not in _pure_answers:
+        groups = C.c_int(0)
+        nat.check(nat.lib().fgx_conv_gather_gemm_stream_groups(C.c_int(code), C.c_int(cols), C.c_int(tile_rows), C.c_int(tile_cols),
+                                                               C.c_int(slab_bytes), C.byref(groups)))
+        _pure_answers[key] = groups.value
+    return _pure_answers[key]
 
 
 def _release_panel_bytes(nbytes: int) -> None:
@@ -356,8 +375,7 @@ def _weight_panel(owner: Optional[torch.Tensor], weight_cvk: torch.Tensor, code:
     global _panel_bytes_kept
     co, v, ci = weight_cvk.shape
     L = nat.lib()
-    nbytes = L.fgx_weight_panel_bytes(C.c_int(code), C.c_int(mode), C.c_int(ci), C.c_int(co), C.c_int(v),
-                                      C.c_int(sched.slab_bytes), C.c_int(sched.tile_cols))
+    nbytes = _panel_nbytes(code, mode, ci, co, v, int(sched.slab_bytes), int(sched.tile_cols))
 
     def pack(panel):
         nat.check(L.fgx_pack_weight(C.c_int(code), C.c_int(mode), nat.ptr(weight_cvk), C.c_int(ci), C.c_int(co), C.c_int(v),
@@ -437,10 +455,8 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
         if sched.stream and _stream_fits(n, n_src, k * src.element_size()):
             order, tile_code, plan_seg, plan_idx, plan_band, plan_key = cache._gather_plan(sched.tile_rows, private,
                                                                                            dense=not masked)
-            groups = C.c_int(0)
-            nat.check(L.fgx_conv_gather_gemm_stream_groups(C.c_int(code), C.c_int(cols), C.c_int(sched.tile_rows),
-                                                           C.c_int(sched.tile_cols), C.c_int(sched.slab_bytes), C.byref(groups)))
-            item_at = cache._item_order(plan_key, tile_code, -(-cols // sched.tile_cols), groups.value,
+            groups = _stream_groups(code, cols, int(sched.tile_rows), int(sched.tile_cols), int(sched.slab_bytes), dev)
+            item_at = cache._item_order(plan_key, tile_code, -(-cols // sched.tile_cols), groups,
                                         -(-(k * src.element_size()) // sched.slab_bytes))
             nat.mark(name, "start")
             nat.check(L.fgx_conv_gather_gemm_stream_act(
@@ -448,7 +464,7 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
                 nat.ptr(plan_seg), nat.ptr(plan_idx), nat.ptr(plan_band), nat.sz(plan_idx.shape[0]), nat.sz(n), nat.sz(n_src),
                 C.c_int(k), C.c_int(cols), C.c_int(v),
                 C.c_int(sched.tile_rows), C.c_int(sched.tile_cols), C.c_int(sched.slab_bytes), nat.ptr(item_at),
-                C.c_int(groups.value), C.c_int(activation), nat.ptr(out), nat.stream()))
+                C.c_int(groups), C.c_int(activation), nat.ptr(out), nat.stream()))
             nat.mark(name, "stop")
             return out
         if masked:
