@@ -653,3 +653,61 @@ def test_relu_in_the_epilogue_equals_relu_after_the_operator(gpu_device, dtype, 
         a = sparse_submanifold_conv3d_relu(feats.to(gpu_device), coords, shape, weight.to(gpu_device), None, cache)[0]
         b_ = torch.relu(sparse_submanifold_conv3d(feats.to(gpu_device), coords, shape, weight.to(gpu_device), None, cache)[0])
     assert torch.equal(a, b_)
+
+
+def test_training_step_replays_from_a_hip_graph(gpu_device):
+    """Forward and backward of two stacked layers captured once (whole-step capture: static input, gradients allocated
+    by the captured backward) and replayed with new inputs; every replay equals the eager step bit for bit, with eager
+    steps of the same layers running between the replays."""
+    res, c = 48, 128
+    coords_np = reference_test_shell(res)
+    shape = torch.Size([1, c, res, res, res])
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    n = len(coords_np)
+    g = torch.Generator().manual_seed(5)
+    ws = [torch.nn.Parameter((torch.randn(c, 3, 3, 3, c, generator=g) / math.sqrt(27 * c)).half().to(gpu_device)) for _ in range(2)]
+    bs = [torch.nn.Parameter(torch.randn(c, generator=g).half().to(gpu_device)) for _ in range(2)]
+    params = ws + bs
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+    upstream = torch.randn(n, c, generator=g).half().to(gpu_device)
+
+    def step(x):
+        h = x
+        for w, b in zip(ws, bs):
+            h = sparse_submanifold_conv3d(h, coords, shape, w, b, cache)[0]
+        h.backward(upstream)
+        return h
+
+    static_in = torch.randn(n, c, generator=g).half().to(gpu_device)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            for p in params:
+                p.grad = None
+            step(static_in)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for p in params:
+        p.grad = None                      # the captured backward allocates the gradients in the graph's pool
+    _say("graph capture of a training step")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = step(static_in)
+    static_grads = [p.grad for p in params]
+    assert all(sg is not None for sg in static_grads)
+    for k in range(3):
+        x = torch.randn(n, c, generator=g).half().to(gpu_device)
+        static_in.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [static_out.clone()] + [sg.clone() for sg in static_grads]
+        for p in params:
+            p.grad = None
+        want_out = step(x)                 # eager step between the replays
+        torch.cuda.synchronize()
+        want = [want_out.detach()] + [p.grad for p in params]
+        for i, (a, b_) in enumerate(zip(got, want)):
+            assert torch.equal(a, b_), f"replay {k}, tensor {i} differs from the eager step"
+        for p, sg in zip(params, static_grads):
+            p.grad = sg                    # hand the static gradient tensors back for the next replay
