@@ -48,8 +48,9 @@ def main():
     p.add_argument("--max-res", type=int, default=512, help="skip configurations above this resolution")
     p.add_argument("--mode", choices=("train", "inference"), default="train")
     p.add_argument("--graph", action="store_true",
-                   help="inference only: the L forward passes are captured once into a HIP graph and replayed (the "
-                        "neighbor cache is built once, outside the timed loop: a graph is tied to its cache's tables)")
+                   help="the L forward passes (and, in train mode, the backward pass) are captured once into a HIP graph "
+                        "and replayed (the neighbor cache is built once, outside the timed loop: a graph is tied to its "
+                        "cache's tables)")
     p.add_argument("--panel-cache", action="store_true",
                    help="keep the repacked weight panels with the weights (flex_gemm.ops.spconv.set_weight_panel_cache): "
                         "the loop never updates its weights, so every pack after the second iteration is saved")
@@ -61,8 +62,6 @@ def main():
     from flexgemm_amd.workloads import reference_test_shell
 
     assert torch.cuda.is_available(), "needs a GPU"
-    if args.graph and args.mode != "inference":
-        p.error("--graph goes with --mode inference")
     nat.lib()
     dev = torch.device("cuda:0")
     flex_gemm.ops.spconv.set_algorithm(Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
@@ -95,25 +94,34 @@ def main():
             SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), train)
 
         if args.graph:
-            fixed = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), False)
+            fixed = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), train)
+            ones = torch.ones((n, c), dtype=feats.dtype, device=dev)
 
-            def forward_stack():
+            def whole_step():
                 h = feats
                 for w, b in params:
                     h = sparse_submanifold_conv3d(h, coords, shape, w, b, fixed)[0]
+                if train:
+                    h.backward(ones)
                 return h
 
-            with torch.no_grad():
+            with torch.set_grad_enabled(train):
                 side = torch.cuda.Stream()
                 side.wait_stream(torch.cuda.current_stream())
                 with torch.cuda.stream(side):
                     for _ in range(3):
-                        forward_stack()
+                        for w, b in params:
+                            w.grad = None
+                            b.grad = None
+                        whole_step()
                 torch.cuda.current_stream().wait_stream(side)
                 torch.cuda.synchronize()
+                for w, b in params:
+                    w.grad = None              # the captured backward allocates the gradients in the graph's pool
+                    b.grad = None
                 graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(graph):
-                    forward_stack()
+                    whole_step()
             iteration = graph.replay
         ms = _median_ms(iteration, args.warmup, args.iters)
         ms_build = _median_ms(build_only, 1, args.iters)
