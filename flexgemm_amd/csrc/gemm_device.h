@@ -64,11 +64,14 @@ template <> __device__ __forceinline__ float to_float<__bf16>(__bf16 x) {
     return __builtin_bit_cast(float, (uint32_t)__builtin_bit_cast(uint16_t, x) << 16);
 }
 
-// Physical position of logical chunk `chunk` of slab row `row` (CH chunks per row).  The XOR key makes rows that
-// read the same logical chunk in one LDS pass hit distinct 16-byte bank groups: with 128-byte rows any 8 consecutive
-// rows (and the even / odd rows of any 16), with 64-byte rows (two per bank line) any 8 and any 16 consecutive rows.
+// Physical position of logical chunk `chunk` of slab row `row` (CH chunks per row).  The gfx950 LDS has 64 banks of
+// 4 bytes: a 256-byte bank line holds two 128-byte rows (four 64-byte rows), and a 128-bit read serves 16 lanes --
+// 16 consecutive slab rows at one logical chunk -- per pass.  The XOR key below gives the rows that share a half
+// (quarter) of the bank line distinct chunk positions within any 16 consecutive rows, so a fragment read takes the
+// same 4.9 cycles as a linear one (measured; a key with period 8 in the row, e.g. row & 7, takes 8.2: two rows of
+// every pass then meet in one bank group).
 template <int CH> __device__ __forceinline__ int swz_key(int row) {
-    return CH == 8 ? ((row + (row >> 3)) & 7) : (((row >> 1) + (row >> 3)) & 3);
+    return CH == 8 ? ((row >> 1) & 7) : ((row >> 2) & 3);
 }
 template <int CH> __device__ __forceinline__ int swz(int row, int chunk) {
     return row * (CH * 16) + ((chunk ^ swz_key<CH>(row)) << 4);
