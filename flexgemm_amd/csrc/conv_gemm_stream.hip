@@ -609,6 +609,23 @@ extern "C" int fgx_conv_gather_gemm_stream_act(int dtype, const void* src, const
     }
 }
 
+namespace fgx {
+bool stream_lds_fits(int tile_rows, int tile_cols, int slab_bytes, int cols) {
+    if (cols <= 0 || tile_cols <= 0) return false;
+    const size_t bias_bytes = align_up((size_t)cols, (size_t)tile_cols) * sizeof(float);
+    size_t fixed = 0;       // (the ring sizes do not depend on the element type)
+#define FGX_STREAM_TILE(BM, BN, WMv, WNv, CHv) \
+    if (tile_rows == BM && tile_cols == BN && slab_bytes == CHv * 16) fixed = StreamCfg<F16, BM, BN, WMv, WNv, CHv>::fixed_lds;
+    FGX_STREAM_TILE(256, 128, 4, 2, 8)
+    FGX_STREAM_TILE(256, 64, 4, 2, 8)
+    FGX_STREAM_TILE(256, 128, 4, 2, 4)
+    FGX_STREAM_TILE(256, 64, 4, 2, 4)
+    FGX_STREAM_TILE(256, 32, 8, 1, 4)
+#undef FGX_STREAM_TILE
+    return fixed != 0 && fixed + bias_bytes <= 160 * 1024;
+}
+}  // namespace fgx
+
 extern "C" int fgx_conv_gather_gemm_stream_groups(int dtype, int cols, int tile_rows, int tile_cols, int slab_bytes,
                                                   int* groups) {
     FGX_CHECK_ARG(dtype == FGX_F16 || dtype == FGX_BF16 || dtype == FGX_F32, "fgx_conv_gather_gemm_stream_groups: unknown dtype %d", dtype);

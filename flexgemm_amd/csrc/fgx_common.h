@@ -40,6 +40,14 @@ inline int fail_hip(hipError_t e, const char* what) {
         if (e_ != hipSuccess) return ::fgx::fail_hip(e_, #expr); \
     } while (0)
 
+// Names the phase whose kernels are enqueued next on `s` to the profiling hook (fgx_set_phase_hook), if one is set;
+// an empty name closes the last phase of a call.
+void phase_mark(const char* name, hipStream_t s);
+
+// Whether the persistent gather GEMM of this tile shape has room in a CU's 160 KiB of LDS for `cols` output columns
+// (it stages the bias of every column tile next to its rings); defined in conv_gemm_stream.hip.
+bool stream_lds_fits(int tile_rows, int tile_cols, int slab_bytes, int cols);
+
 inline unsigned cdiv(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
 
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }

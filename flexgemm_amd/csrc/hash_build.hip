@@ -26,6 +26,12 @@ void set_error(const char* fmt, ...) {
     va_end(ap);
 }
 
+static fgx_phase_hook_t g_phase_hook = nullptr;
+
+void phase_mark(const char* name, hipStream_t s) {
+    if (g_phase_hook) g_phase_hook(name, (fgx_stream_t)s);
+}
+
 namespace {
 
 constexpr int kBlock = 256;
@@ -181,6 +187,8 @@ using namespace fgx;
 extern "C" {
 
 int fgx_abi_version(void) { return 1; }
+
+void fgx_set_phase_hook(fgx_phase_hook_t hook) { fgx::g_phase_hook = hook; }
 
 const char* fgx_last_error(void) { return fgx::g_error; }
 

@@ -113,6 +113,17 @@ __device__ __forceinline__ void search_staged(const K* wkeys, const uint32_t* wr
                 const unsigned at = pos < wn ? pos : wn - 1;
                 if (wkeys[at] < tk && pos < wn) ++pos;
             }
+            // Only a window with repeated keys (the same voxel given twice) can still be short of the target:
+            // finish with a search over the rest.
+            if (pos < wn && wkeys[pos] < tk) {
+                unsigned lo = pos + 1, hi = wn;
+                while (lo < hi) {
+                    const unsigned mid = (lo + hi) >> 1;
+                    if (wkeys[mid] < tk) lo = mid + 1;
+                    else hi = mid;
+                }
+                pos = lo;
+            }
         }
         const unsigned at = pos < wn ? pos : wn - 1;
         const int z2 = z_first + kz * Dd;
@@ -238,8 +249,9 @@ __global__ void __launch_bounds__(kGroup) merge_neighbor_kernel(const K* __restr
                                               : out_map + (size_t)me * g.V + (size_t)r * g.Kd;
                 const long long first = (long long)key + off - (long long)(g.Kd / 2) * g.Dd;
                 auto emit = [&](int kz, uint32_t value) {
-                    out_row[kz] = value;
                     const int v = r * g.Kd + kz;
+                    if (v == g.V / 2) value = me;       // the middle entry is the voxel itself, found or not (subm_neighbor_map.cu:64-66)
+                    out_row[kz] = value;
                     if (v < 32 && value != FGX_EMPTY32) mask |= 1u << v;
                 };
                 if (staged && w > 0) search_staged<K>(wkeys, wrows, (unsigned)w, first, row_in, z_first, g.Kd, g.Dd, g.D, emit);

@@ -102,7 +102,8 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
     const int slab = row_bytes >= 128 ? 128 : 64;
     const int scols = cols > 64 ? 128 : ((cols > 32 || slab == 128) ? 64 : 32);
     const size_t enough = slab == 128 ? (size_t)kCUs * 7 / 16 : 2 * (size_t)kCUs;
-    if (row_bytes >= 64 && (slab == 64 || cols >= 64) && (size_t)cdiv(n, 256) * cdiv(cols, scols) >= enough) {
+    if (row_bytes >= 64 && (slab == 64 || cols >= 64) && (size_t)cdiv(n, 256) * cdiv(cols, scols) >= enough &&
+        stream_lds_fits(256, scols, slab, cols)) {      // (from ~1900 output columns on the staged bias no longer fits)
         out->tile_rows = 256;
         out->tile_cols = scols;
         out->slab_bytes = slab;
@@ -126,6 +127,8 @@ extern "C" int fgx_table_lookup(int pass_kind, int dtype, size_t n, int Ci, int 
     for (const Entry& e : kTable) {
         if (e.pass_kind == pass_kind && (e.dtype_bytes == 0 || e.dtype_bytes == es) && e.log2n == l2 && e.ci == Ci && e.co == Co) {
             *out = e.s;
+            if (pass_kind != 2 && out->stream && !stream_lds_fits(out->tile_rows, out->tile_cols, out->slab_bytes, pass_kind == 0 ? Co : Ci))
+                break;      // (cannot happen for the shapes listed; the rule decides then)
             return FGX_OK;
         }
     }

@@ -29,53 +29,16 @@
 // kernel over sig_o.
 #include <type_traits>
 
-#include "fgx_common.h"
+#include "wgrad_device.h"
 
 namespace fgx {
 namespace {
 
-using f16x8 = _Float16 __attribute__((ext_vector_type(8)));
-using bf16x8 = __bf16 __attribute__((ext_vector_type(8)));
-using f32x16 = float __attribute__((ext_vector_type(16)));
-using u32x4 = uint32_t __attribute__((ext_vector_type(4)));
-using i16x4 = short __attribute__((ext_vector_type(4)));
-using i16x8 = short __attribute__((ext_vector_type(8)));
-
-struct F16 { using type = _Float16; };
-struct BF16 { using type = __bf16; };
-struct F32 { using type = float; };
-
-template <typename T> __device__ __forceinline__ T from_float(float x);
-template <> __device__ __forceinline__ _Float16 from_float<_Float16>(float x) { return (_Float16)x; }
-template <> __device__ __forceinline__ float from_float<float>(float x) { return x; }
-template <> __device__ __forceinline__ __bf16 from_float<__bf16>(float x) {
-    uint32_t u = __builtin_bit_cast(uint32_t, x);
-    uint16_t h;
-    if ((u & 0x7FFFFFFFu) > 0x7F800000u) h = (uint16_t)((u >> 16) | 0x0040u);
-    else h = (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
-    return __builtin_bit_cast(__bf16, h);
-}
-
-constexpr int kMaxV = 32;
-constexpr int kXcds = 8;
 constexpr int kStages = 4;      // row ring depth
 constexpr int kIdxSlots = 8;    // index ring depth (>= kStages, power of two)
 
 // 16 zero bytes every lane may read: pairs past the end of an item, columns past the tensor width
 __device__ __attribute__((aligned(256))) unsigned char g_zero_block_w[256];
-
-#define FGX_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
-#define FGX_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
-}
-
-struct SegTable {
-    uint32_t seg[kMaxV + 1];   // pair offsets per kernel offset
-};
 
 // bounds[v * (nb + 1) + b] = first pair of offset v whose output row is >= b * block_rows
 __global__ void __launch_bounds__(256) block_bounds_kernel(const uint32_t* __restrict__ sig_o, SegTable tab, int V,
@@ -121,39 +84,6 @@ struct WgradCfg {
     static constexpr int key_a(int row) { return ES == 2 && CH_A >= 8 ? 2 * (row & 3) : 0; }
     static constexpr int key_b(int row) { return ES == 2 && CH_B >= 8 ? 2 * (row & 3) : 0; }
 };
-
-// Transposing LDS read, issued as inline assembly: through the compiler builtin every such read is preceded by a
-// conservative s_waitcnt vmcnt(0) (the compiler cannot tell it apart from the LDS areas the in-flight direct-to-LDS
-// loads are filling), which would drain the whole ring each step.  The price is that the result must be waited
-// for by hand: lds_wait_all() below ties the fragment registers to an s_waitcnt lgkmcnt(0).
-__device__ __forceinline__ i16x4 lds_read_tr16(const unsigned char* p) {
-    const uint32_t addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const unsigned char*)p;
-    i16x4 r;
-    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(r) : "v"(addr));
-    return r;
-}
-template <int N>
-__device__ __forceinline__ void lds_wait_all(i16x4 (&r)[N]) {
-    static_assert(N % 4 == 0, "fragments come in groups of four registers pairs");
-#pragma unroll
-    for (int i = 0; i < N; i += 4)
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[i]), "+v"(r[i + 1]), "+v"(r[i + 2]), "+v"(r[i + 3]));
-}
-
-template <typename Tag> __device__ __forceinline__ void mma16(f32x16& acc, const i16x8& a, const i16x8& b);
-template <> __device__ __forceinline__ void mma16<F16>(f32x16& acc, const i16x8& a, const i16x8& b) {
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), acc, 0, 0, 0);
-}
-template <> __device__ __forceinline__ void mma16<BF16>(f32x16& acc, const i16x8& a, const i16x8& b) {
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
-}
-template <> __device__ __forceinline__ void mma16<F32>(f32x16&, const i16x8&, const i16x8&) {}
-
-// eight ones in the 16-bit type, as a fragment
-template <typename Tag> __device__ __forceinline__ i16x8 ones16() {
-    constexpr short one = sizeof(typename Tag::type) == 2 && __is_same(typename Tag::type, _Float16) ? (short)0x3C00 : (short)0x3F80;
-    return i16x8{one, one, one, one, one, one, one, one};
-}
 
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N>
 __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N)
@@ -394,13 +324,6 @@ constexpr int kWsIdxSlots = 8;
 constexpr int kWsIdxAhead = 4;       // index loads run this many steps ahead of the row loads (> kWsStages - 1)
 constexpr int kWsLoaders = 4;
 constexpr int kWsPairs = 64;         // pairs per step
-constexpr uint32_t kOobOffset = 0xFF000000u;
-
-using rsrc_t = __amdgpu_buffer_rsrc_t;
-__device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint32_t bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), (short)0, (int)bytes, 0x00020000);
-}
-
 template <typename Tag, int BM, int BN>
 struct WStreamCfg {
     using T = typename Tag::type;
@@ -430,18 +353,6 @@ struct WStreamCfg {
     static constexpr int key_a(int row) { return CH_A >= 8 ? 2 * (row & 3) : 0; }
     static constexpr int key_b(int row) { return CH_B >= 8 ? 2 * (row & 3) : 0; }
 };
-
-// wait until the LDS reads before the newest N have returned; the registers are tied to the wait so that the
-// compiler cannot move their first use above it
-template <int N, int R>
-__device__ __forceinline__ void lds_wait_but(i16x4 (&r)[R]) {
-    static_assert(N >= 0 && N < 16 && R % 4 == 0, "lgkmcnt is a 4-bit counter");
-#if defined(__HIP_DEVICE_COMPILE__)   // (the host pass only needs the kernel's signature; it has no such registers)
-#pragma unroll
-    for (int i = 0; i < R; i += 4)
-        asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(r[i]), "+v"(r[i + 1]), "+v"(r[i + 2]), "+v"(r[i + 3]) : "n"(N));
-#endif
-}
 
 template <typename Tag, int BM, int BN>
 __global__ void __launch_bounds__(64 * (4 + kWsLoaders))
@@ -1159,6 +1070,9 @@ bool stream_ok(int tile_rows, int tile_cols, size_t n, size_t n_in, int Ci, int 
     if (sizeof(typename Tag::type) != 2) return false;
     if (!((tile_rows == 128 && tile_cols == 128) || (tile_rows == 64 && tile_cols == 64) || (tile_rows == 32 && tile_cols == 32)))
         return false;
+    // the 32 x 32 tile writes four partial products per voxel block; fgx_wgrad_scratch_bytes leaves room for them only
+    // where the table picks that tile (at most 32 channels on a side): anything wider runs the tiled kernel
+    if (tile_rows == 32 && (Ci < Co ? Ci : Co) > 32) return false;
     return (double)n * Co * 2 <= (double)kOobOffset && (double)n_in * Ci * 2 <= (double)kOobOffset &&
            (double)n_pairs * 4 + 256 <= (double)kOobOffset;
 }

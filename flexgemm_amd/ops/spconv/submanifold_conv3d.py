@@ -382,7 +382,9 @@ def _weight_panel(owner: Optional[torch.Tensor], weight_cvk: torch.Tensor, code:
                                     C.c_int(sched.slab_bytes), C.c_int(sched.tile_cols), nat.ptr(panel), nat.stream()))
         return panel
 
-    if owner is None or not spconv.WEIGHT_PANEL_CACHE:
+    # Under graph capture the pack kernel must be part of the graph: a kept panel read by the captured GEMMs would pin
+    # the weights of the day of the capture, whatever the optimizer does to them between replays.
+    if owner is None or not spconv.WEIGHT_PANEL_CACHE or torch.cuda.is_current_stream_capturing():
         return pack(nat.workspace(nbytes, dev))
     kept = owner.__dict__.setdefault("_fgx_weight_panels", {})
     key = (code, mode, ci, co, v, int(sched.slab_bytes), int(sched.tile_cols), str(dev))

@@ -46,6 +46,14 @@ typedef void* fgx_stream_t;
 int fgx_abi_version(void);
 const char* fgx_last_error(void);
 
+/* Profiling aid (no counterpart in the reference, which is timed from outside with CUDA events, tests/utils.py:35-65):
+ * calls that enqueue several kernels name their phases.  With a hook set, the calling thread invokes
+ * hook(phase_name, stream) right before the kernels of each phase are enqueued and hook("", stream) after the last
+ * one; a caller records an event on `stream` in it and reads the time per phase.  NULL (the default) switches it off.
+ * Process-wide; set it only while no other thread is inside the library. */
+typedef void (*fgx_phase_hook_t)(const char* phase_name, fgx_stream_t stream);
+void fgx_set_phase_hook(fgx_phase_hook_t hook);
+
 /* ---------------------------------------------------------------------------------------------
  * Hash table (open addressing, linear probing, Murmur3 finaliser, all-ones key = empty slot).
  * key_bits / val_bits are 32 or 64.
@@ -273,7 +281,8 @@ int fgx_gather_item_order(const int32_t* tile_code, size_t num_tiles, int col_ti
  * convolution.  `block_bounds` (optional): the table fgx_wgrad_block_bounds makes from the same pair lists and
  * block_rows -- block_bounds[v * (nb + 1) + b] = first pair of offset v whose grad_out row is >= b * block_rows,
  * nb = ceil(n / block_rows) -- for callers that keep it with their neighbor cache; NULL = computed here, per call.
- * The 32x32 streaming tile writes four partial products per block (the scratch size accounts for it).
+ * The 32x32 streaming tile writes four partial products per block; the scratch size accounts for it where that tile
+ * may stream, i.e. with at most 32 channels on a side -- a 32x32 tile with wider channels runs the tiled kernel.
  * `grad_bias` (optional, Co elements of the tensors' type): the column sums of grad_out over its n rows, the bias
  * gradient.  `bias_offset` names an offset whose pairs hold every grad_out row exactly once (the centre offset of a
  * submanifold convolution; -1 when there is none): the streaming kernel then sums the grad_out rows it loads for that

@@ -84,6 +84,20 @@ def backward(grad_output: torch.Tensor, feats: torch.Tensor, neighbor_map: torch
     return grad_input, grad_weight, grad_bias
 
 
+def weight_grad_offset(grad_output: torch.Tensor, feats: torch.Tensor, neighbor_map: torch.Tensor, v: int,
+                       chunk_rows: int = 262144) -> torch.Tensor:
+    """grad_weight[:, v, :] alone, [Co, Ci]: column v of the im2col product of submanifold_conv3d.py:246-253, i.e. the
+    sum over the rows n with a neighbor at offset v of grad_output[n]^T feats[neighbor_map[n, v]].  For full-size
+    workloads, where the whole [V*Ci, Co] product is too slow; tests/test_oracle_gemm.py pins it to backward()."""
+    idx = _as_index(neighbor_map)[:, v]
+    rows = torch.nonzero(idx >= 0).reshape(-1)
+    acc = torch.zeros((grad_output.shape[1], feats.shape[1]), dtype=feats.dtype)
+    for s in range(0, rows.numel(), chunk_rows):
+        r = rows[s:s + chunk_rows]
+        acc += torch.mm(grad_output[r].t(), feats[idx[r]])
+    return acc
+
+
 def calc_err(src: torch.Tensor, ref: torch.Tensor) -> Tuple[float, float]:
     """max / mean over elements of min(abs err, rel err), rel clamp 1e-6 (reference tests/utils.py:28-32)."""
     abs_err = (src.double() - ref.double()).abs()

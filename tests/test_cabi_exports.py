@@ -74,6 +74,20 @@ def test_host_only_entry_points(library):
     assert L.fgx_wgrad_scratch_bytes(ctypes.c_size_t(1000), 3, 8, 16, 256) == 256 + 4 * 4 * 3 * 8 * 16 * 4 + 4 * 4 * 16 * 4 + colsum
 
 
+def test_table_leaves_very_wide_layers_to_the_tiled_kernel(library):
+    # the persistent gather GEMM stages the bias of all output columns in LDS beside its rings: from about 1900 columns
+    # on that no longer fits, and the table must not pick it (any channel count has to run)
+    import torch
+    for c in (2048, 4096):
+        for p in (nat.PASS_FWD, nat.PASS_DGRAD):
+            s = nat.table_lookup(p, torch.float16, 100000, c, c, 27)
+            assert s.stream == 0 and s.tile_cols == 128 and s.splitk >= 1, (c, p)
+    assert nat.table_lookup(nat.PASS_FWD, torch.float16, 100000, 1024, 1920, 27).stream == 1
+    assert nat.table_lookup(nat.PASS_FWD, torch.float16, 100000, 1024, 1921, 27).stream == 0
+    assert nat.table_lookup(nat.PASS_DGRAD, torch.float16, 100000, 2048, 1024, 27).stream == 0   # dgrad: columns = Ci
+    assert nat.table_lookup(nat.PASS_DGRAD, torch.float16, 100000, 1024, 2048, 27).stream == 1
+
+
 def test_argument_errors_map_to_exceptions(library):
     L = nat.lib()
     with pytest.raises(ValueError):

@@ -450,14 +450,16 @@ def test_cfg5_fp32_variant(gpu_device):
     assert max(e[1] for e in errs) <= 1e-4
 
 
-def test_full_size_properties_cfg3(gpu_device):
-    """Configuration 3 at full size (669 288 voxels, C = 128, fp16): the float64 oracle is evaluated on a random
-    sample of output rows (forward, dgrad) and the closed-form identities <conv(f), g> = <f, dgrad(g)> = <W, wgrad>
-    tie the three passes together."""
-    _say("conv cfg3 full size")
-    wl = make_workload("cfg3")
-    dev = gpu_device
-    dt = torch.float16
+WGRAD_OFFSETS = (0, 4, 13, 22, 26, 17)
+
+
+def _full_size_check(wl, dt, sample, dev, seed):
+    """A benchmark configuration at full size through the public operator: a random sample of output rows against the
+    float64 oracle (forward and input gradient); the weight gradient of six offsets (the corners 0 and 26, the face
+    neighbors 4 and 22, the centre 13 and offset 17), every element of their [Co, Ci] slices, against the float64
+    oracle; the inner-product identities <conv(f), g> = <f, dgrad(g)> = <W, wgrad> over the whole tensors; and the
+    bias gradient against the column sums."""
+    c = wl.feats.shape[1]
     f = wl.feats.to(dt).to(dev).requires_grad_(True)
     w = wl.weight.to(dt).to(dev).requires_grad_(True)
     b = wl.bias.to(dt).to(dev).requires_grad_(True)
@@ -467,12 +469,16 @@ def test_full_size_properties_cfg3(gpu_device):
     out.backward(g.to(dev))
     torch.cuda.synchronize()
     nmap = cache.neighbor_map.cpu().view(torch.int32)
-    rows = torch.randperm(wl.n, generator=torch.Generator().manual_seed(0))[:4096]
+    rows = torch.randperm(wl.n, generator=torch.Generator().manual_seed(seed))[:sample]
     f64, w64, b64, g64 = f.detach().cpu().double(), w.detach().cpu().double(), b.detach().cpu().double(), g.double()
     ref_rows = eg.forward(f64, nmap[rows], w64, b64)
     _assert_close(out[rows.to(dev)], ref_rows, dt, "forward sample")
-    ref_gi = torch.mm(eg._im2col(g64, torch.flip(nmap[rows].long(), [1])), w64.reshape(128, 27, 128).transpose(0, 1).reshape(27 * 128, 128))
+    ref_gi = torch.mm(eg._im2col(g64, torch.flip(nmap[rows].long(), [1])), w64.reshape(c, 27, c).transpose(0, 1).reshape(27 * c, c))
     _assert_close(f.grad[rows.to(dev)], ref_gi, dt, "dgrad sample")
+    gw = w.grad.detach().cpu().reshape(c, 27, c)
+    for v in WGRAD_OFFSETS:
+        _say(f"  wgrad slice of offset {v}")
+        _assert_close(gw[:, v], eg.weight_grad_offset(g64, f64, nmap, v), dt, f"wgrad offset {v}")
     # inner-product identities in float64 from the GPU results (bias-free part)
     conv_nobias = out.detach().cpu().double() - b64
     lhs = (conv_nobias * g64).sum()
@@ -480,41 +486,65 @@ def test_full_size_properties_cfg3(gpu_device):
     rhs = (w64 * w.grad.cpu().double()).sum()
     scale = float((conv_nobias.abs() * g64.abs()).sum())
     assert abs(lhs - mid) / scale < 1e-3 and abs(lhs - rhs) / scale < 1e-3
-    assert eg.max_rel_err(b.grad.cpu(), g64.sum(0)) <= 1e-2
+    _assert_close(b.grad, g64.sum(0), dt, "dbias")
 
 
-@pytest.mark.parametrize("name,sample", [("cfg2", 2048), ("cfg4", 4096), ("cfg5", 512)])
-def test_full_size_properties_other_configurations(gpu_device, name, sample):
-    """Configurations 2, 4 and 5 at full size, in their own dtypes: a random sample of output rows against the float64
-    oracle (forward and input gradient), the inner-product identities <conv(f), g> = <f, dgrad(g)> = <W, wgrad> over the
-    whole tensors, and the bias gradient against the column sums."""
+@pytest.mark.parametrize("name,sample", [("cfg3", 4096), ("cfg2", 2048), ("cfg4", 4096), ("cfg5", 512)])
+def test_full_size_properties(gpu_device, name, sample):
+    """Configurations 2, 3, 4 and 5 at full size, in their own dtypes (cfg3: 669 288 voxels, C = 128, fp16)."""
     wl = make_workload(name)
-    dt = wl.dtype
-    c = wl.feats.shape[1]
-    _say(f"conv {name} full size, n={wl.n} C={c} {dt}")
+    _say(f"conv {name} full size, n={wl.n} C={wl.feats.shape[1]} {wl.dtype}")
+    _full_size_check(wl, wl.dtype, sample, gpu_device, seed=1)
+
+
+def test_full_size_cfg5_fp32_variant(gpu_device):
+    """Configuration 5's fp32-input variant (fp32 accumulation) at full size: 42 608 voxels, C = 1024, tolerance 1e-4."""
+    wl = make_workload("cfg5")
+    _say(f"conv cfg5 fp32 variant full size, n={wl.n}")
+    _full_size_check(wl, torch.float32, 256, gpu_device, seed=2)
+
+
+def test_cfg1_whole_tensors(gpu_device):
+    """Configuration 1 (res-64 shell, 10 208 voxels, Ci = Co = 64, fp32) on the HIP path: forward with the workload's
+    own values against the float64 oracle over the whole tensor, and the backward pass as well."""
+    wl = make_workload("cfg1")
+    _say(f"conv cfg1, n={wl.n}")
+    assert wl.n == 10208 and wl.dtype == torch.float32
     dev = gpu_device
-    f = wl.feats.to(dt).to(dev).requires_grad_(True)
-    w = wl.weight.to(dt).to(dev).requires_grad_(True)
-    b = wl.bias.to(dt).to(dev).requires_grad_(True)
-    g = wl.grad.to(dt)
-    coords = wl.coords.to(dev)
-    out, cache = sparse_submanifold_conv3d(f, coords, wl.shape, w, b)
-    out.backward(g.to(dev))
+    f = wl.feats.to(dev).requires_grad_(True)
+    w = wl.weight.to(dev).requires_grad_(True)
+    b = wl.bias.to(dev).requires_grad_(True)
+    out, cache = sparse_submanifold_conv3d(f, wl.coords.to(dev), wl.shape, w, b)
+    out.backward(wl.grad.to(dev))
     torch.cuda.synchronize()
-    nmap = cache.neighbor_map.cpu().view(torch.int32)
-    rows = torch.randperm(wl.n, generator=torch.Generator().manual_seed(1))[:sample]
-    f64, w64, b64, g64 = f.detach().cpu().double(), w.detach().cpu().double(), b.detach().cpu().double(), g.double()
-    ref_rows = eg.forward(f64, nmap[rows], w64, b64)
-    _assert_close(out[rows.to(dev)], ref_rows, dt, "forward sample")
-    ref_gi = torch.mm(eg._im2col(g64, torch.flip(nmap[rows].long(), [1])), w64.reshape(c, 27, c).transpose(0, 1).reshape(27 * c, c))
-    _assert_close(f.grad[rows.to(dev)], ref_gi, dt, "dgrad sample")
-    conv_nobias = out.detach().cpu().double() - b64
-    lhs = (conv_nobias * g64).sum()
-    mid = (f64 * f.grad.cpu().double()).sum()
-    rhs = (w64 * w.grad.cpu().double()).sum()
-    scale = float((conv_nobias.abs() * g64.abs()).sum())
-    assert abs(lhs - mid) / scale < 1e-3 and abs(lhs - rhs) / scale < 1e-3
-    assert eg.max_rel_err(b.grad.cpu(), g64.sum(0)) <= 1e-2
+    nmap = torch.from_numpy(nb.neighbor_map(wl.coords.numpy(), tuple(wl.shape)).view(np.int32))
+    assert torch.equal(cache.neighbor_map.cpu().view(torch.int32), nmap)
+    f64, w64, b64, g64 = wl.feats.double(), wl.weight.double(), wl.bias.double(), wl.grad.double()
+    _assert_close(out, eg.forward(f64, nmap, w64, b64), torch.float32, "forward")
+    ref_gi, ref_gw, ref_gb = eg.backward(g64, f64, nmap, w64)
+    _assert_close(f.grad, ref_gi, torch.float32, "dgrad")
+    _assert_close(w.grad, ref_gw, torch.float32, "wgrad")
+    _assert_close(b.grad, ref_gb, torch.float32, "dbias")
+
+
+def test_very_wide_output_runs_the_tiled_kernel(gpu_device):
+    """2048 output columns: the persistent kernel's staged bias no longer fits a CU's LDS, the table leaves the layer
+    to the tiled kernel (forward: Co columns; dgrad: Ci columns)."""
+    res = 20
+    coords_np = reference_test_shell(res)
+    _say(f"conv Co=2048 / Ci=2048, n={len(coords_np)}")
+    _run_and_check(coords_np, torch.Size([1, 64, res, res, res]), 64, 2048, torch.float16, gpu_device, seed=3)
+    _run_and_check(coords_np, torch.Size([1, 2048, res, res, res]), 2048, 64, torch.float16, gpu_device, seed=4)
+
+
+def test_wide_channels_with_a_32x32_streaming_wgrad_tile_fall_back(gpu_device):
+    """A caller that asks for the 32 x 32 streaming wgrad tile with more than 32 channels on both sides gets the tiled
+    kernel: the scratch size the library quotes has no room for that tile's four partial products per block there."""
+    res, c = 24, 64
+    coords_np = reference_test_shell(res)
+    _say(f"wgrad tile 32 stream=1 at C={c}")
+    with _force_schedule(wgrad=True, tile_rows=32, tile_cols=32, block_rows=512, stream=1):
+        _run_and_check(coords_np, torch.Size([1, c, res, res, res]), c, c, torch.float16, gpu_device, seed=29)
 
 
 def test_weight_panel_cache_keeps_results_and_follows_weight_updates(gpu_device):
@@ -614,6 +644,45 @@ def test_forward_replays_from_a_hip_graph(gpu_device, res, c):
             eager = stack(x)                     # the program's own eager work between the replays
             torch.cuda.synchronize()
             assert torch.equal(static_out, eager), f"replay {k} differs from the eager result"
+
+
+def test_graph_captured_with_the_panel_cache_on_follows_weight_updates(gpu_device):
+    """With the weight panel cache on and panels already kept, a captured forward still packs its panels inside the
+    graph: after an in-place weight update every replay equals the eager result of the updated weights."""
+    from flexgemm_amd.ops import spconv as cfg
+    res, c = 24, 64
+    coords_np = reference_test_shell(res)
+    shape = torch.Size([1, c, res, res, res])
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    n = len(coords_np)
+    g = torch.Generator().manual_seed(77)
+    w = (torch.randn(c, 3, 3, 3, c, generator=g) / math.sqrt(27 * c)).half().to(gpu_device)
+    b = torch.randn(c, generator=g).half().to(gpu_device)
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), False)
+    static_in = torch.randn(n, c, generator=g).half().to(gpu_device)
+    cfg.set_weight_panel_cache(True)
+    try:
+        with torch.no_grad():
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(3):          # the second and third call keep and reuse a panel
+                    sparse_submanifold_conv3d(static_in, coords, shape, w, b, cache)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            assert any(e[1] is not None for e in w.__dict__["_fgx_weight_panels"].values())
+            _say("graph capture with kept weight panels")
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                static_out = sparse_submanifold_conv3d(static_in, coords, shape, w, b, cache)[0]
+            for k in range(3):
+                w.mul_(-0.5).add_(0.01)     # an optimizer step's in-place update
+                graph.replay()
+                eager = sparse_submanifold_conv3d(static_in, coords, shape, w, b, cache)[0]
+                torch.cuda.synchronize()
+                assert torch.equal(static_out, eager), f"replay {k} used stale weights"
+    finally:
+        cfg.set_weight_panel_cache(False)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])

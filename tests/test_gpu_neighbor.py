@@ -82,6 +82,41 @@ def test_cache_matches_oracle_reference_geometry(gpu_device, res, needs_grad):
         flex_gemm.ops.spconv.set_algorithm(Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
 
 
+@pytest.mark.parametrize("res", [128, 256, 512])
+def test_cache_matches_oracle_reference_geometry_large(gpu_device, res):
+    # the upper part of the reference's sweep (tests/submconv/neighbor_cache.py:54 runs its shell up to res 512)
+    _say(f"neighbor cache reference shell res={res}")
+    coords_np = reference_test_shell(res)
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    shape = torch.Size([1, 0, res, res, res])
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+    _check_cache(cache, coords_np, shape, True, blocks=(128,))
+
+
+def test_repeated_voxels_give_the_same_map_with_both_builders(gpu_device, neighbor_map_builder):
+    """A coordinate list that names some voxels twice: which of the equal rows a neighbor entry names is not fixed
+    (the reference's hash insert lets the last writer win), but every entry must name a row with the right
+    coordinates, exist exactly when such a row exists, and the middle entry must be the row itself."""
+    rng = np.random.default_rng(5)
+    res = 24
+    base = reference_test_shell(res)
+    coords_np = np.concatenate([base, base[rng.choice(len(base), 300, replace=False)], base[:7], base[:7]])
+    coords_np = coords_np[rng.permutation(len(coords_np))]
+    _say(f"neighbor map with repeated voxels, n={len(coords_np)} builder={neighbor_map_builder}")
+    shape = torch.Size([1, 0, res, res, res])
+    cache = SubMConv3dFunction._compute_neighbor_cache(torch.from_numpy(coords_np).to(gpu_device), shape, (3, 3, 3), (1, 1, 1), False)
+    nmap = _np(cache.neighbor_map)
+    n = len(coords_np)
+    assert np.array_equal(nmap[:, 13], np.arange(n, dtype=np.uint32))
+    present = {tuple(c) for c in coords_np.tolist()}
+    offs = np.array([(0, dx, dy, dz) for dx in (-1, 0, 1) for dy in (-1, 0, 1) for dz in (-1, 0, 1)], dtype=np.int32)
+    for v in range(27):
+        want = coords_np + offs[v]
+        found = nmap[:, v] != EMPTY
+        assert np.array_equal(found, np.array([tuple(c) in present for c in want.tolist()]))
+        assert np.array_equal(coords_np[nmap[found, v]], want[found])
+
+
 def test_cache_shuffled_batched_dilated(gpu_device):
     rng = np.random.default_rng(7)
     res = 20

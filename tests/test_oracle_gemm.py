@@ -87,6 +87,17 @@ def test_closed_forms_and_invariants():
     assert torch.allclose(lhs, (weight * g1[1]).sum())
 
 
+def test_single_offset_weight_gradient_is_a_slice_of_backward():
+    res, ci, co = 9, 5, 7
+    coords, feats, weight, bias, grad, nmap = _random_case(res, ci, co, 5)
+    gw = eg.backward(grad, feats, nmap, weight, need_input=False, need_bias=False)[1].reshape(co, 27, ci)
+    for v in range(27):
+        for chunk in (3, 10 ** 6):
+            assert torch.allclose(eg.weight_grad_offset(grad, feats, nmap, v, chunk_rows=chunk), gw[:, v], rtol=1e-12, atol=1e-12)
+    # the centre offset pairs every row with itself
+    assert torch.allclose(eg.weight_grad_offset(grad, feats, nmap, 13), grad.t() @ feats, rtol=1e-12, atol=1e-12)
+
+
 def test_map_forms_accepted():
     res, ci, co = 6, 3, 3
     coords, feats, weight, bias, grad, nmap = _random_case(res, ci, co, 9)
