@@ -10,7 +10,12 @@ Headline workload (N = 1): configuration 3 -- res 512 shell (669 288 voxels), Ci
 `value` = effective TFLOP/s = useful FLOP / time with useful FLOP = 6 * L * Ci * Co per step
 (L = valid neighbor pairs; the reference's accounting: tests/submconv/fwd.py:247-249, bwd.py:288-290).
 
-Prints ONE JSON line.  `--workload cfg2|cfg3|cfg4|cfg5` selects another configuration (cfg2 is forward only).
+Prints ONE JSON line.  `--workload cfg2|cfg3|cfg4|cfg5` selects another configuration (cfg2 is forward only),
+`--dtype f32` the fp32-input variant of a configuration (configuration 5 names one).
+
+Timing follows the reference's protocol (tests/utils.py:35-65: events around every call, peak memory): besides the
+wall-clock mean over the timed steps, the line carries median and minimum per step and per pass from HIP events,
+the peak of allocated device memory over the timed region, and the neighbor-cache build split into its phases.
 """
 from __future__ import annotations
 
@@ -27,10 +32,25 @@ if ROOT not in sys.path:
 
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}   # MI355X dense MFMA peaks
 HBM_PEAK_GBS = 8000.0
-# HBM-side bytes per launch of the dominant kernel, from two rocprofv3 counter runs of this script (FETCH_SIZE, then
-# WRITE_SIZE, each scaled by what the same counter reads for the plain copy of --calibrate-copy: x2.0 and x1.0).
-# The counters cannot be read from inside the process, so the measured figure is kept here per workload.
-MEASURED_TRAFFIC_BYTES = {"cfg3": 1.755e9}
+# HBM-side bytes per launch of the dominant kernel come from two rocprofv3 counter runs of this script (FETCH_SIZE, then
+# WRITE_SIZE, each scaled by what the same counter reads for the plain copy of --calibrate-copy).  The counters cannot
+# be read from inside the process: `python -m flexgemm_amd.profile_traffic` turns the two counter files into an entry of
+# this file, stamped with a digest of the kernel's source files, and the summary under profiles/ quotes the same entry.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def measured_traffic(workload: str, dname: str):
+    """Bytes per launch of the dominant kernel from profiles/traffic.json, or None when there is no entry for this
+    workload and dtype or the kernel's sources have changed since it was measured."""
+    from flexgemm_amd.profile_traffic import source_digest
+    try:
+        with open(TRAFFIC_FILE) as f:
+            entry = json.load(f).get(f"{workload}_{dname}")
+    except (OSError, ValueError):
+        return None
+    if not entry or entry.get("source_digest") != source_digest(entry.get("sources", [])):
+        return None
+    return entry.get("traffic_bytes")
 
 
 def parse():
@@ -39,6 +59,7 @@ def parse():
     p.add_argument("--steps", type=int, default=50)
     p.add_argument("--warmup", type=int, default=5)
     p.add_argument("--workload", default="cfg3", choices=["cfg2", "cfg3", "cfg4", "cfg5"])
+    p.add_argument("--dtype", default=None, choices=["f16", "bf16", "f32"], help="override the configuration's dtype")
     p.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (used under rocprofv3)")
     p.add_argument("--cpu-rows", type=int, default=0, help="rows in the CPU baseline sample (0 = auto)")
     p.add_argument("--build-only", action="store_true", help="time only the neighbor-cache build")
@@ -107,9 +128,10 @@ def main():
     torch.cuda.set_device(dev)
     flex_gemm.ops.spconv.set_algorithm(Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
 
-    wl = make_workload(args.workload)
+    names = {torch.float16: "f16", torch.bfloat16: "bf16", torch.float32: "f32"}
+    wl = make_workload(args.workload, dtype={v: k for k, v in names.items()}.get(args.dtype))
     dt = wl.dtype
-    dname = {torch.float16: "f16", torch.bfloat16: "bf16", torch.float32: "f32"}[dt]
+    dname = names[dt]
     c = wl.channels
     passes = 1 if args.workload == "cfg2" else 3
     coords = wl.coords.to(dev)
@@ -133,6 +155,36 @@ def main():
         torch.cuda.synchronize()
         build_ms.append(ev0.elapsed_time(ev1))
     build_ms.sort()
+
+    # the build split into its phases: the library names them to a hook, which records an event on their stream; the
+    # first forward of a fresh cache adds the tables made on first use (tile masks, gather plan)
+    def build_phases(reps=5):
+        marks = []
+
+        def hook(name, stream):
+            e = torch.cuda.Event(enable_timing=True)
+            e.record(torch.cuda.current_stream())
+            marks.append((name, e))
+
+        gap = "between calls (host: allocations, read-backs)"
+        runs = []
+        nat.set_phase_hook(hook)
+        try:
+            for _ in range(reps):
+                del marks[:]
+                fresh = build_cache()
+                with torch.no_grad():
+                    SubMConv3dFunction._sparse_submanifold_conv_forward(feats, fresh, weight, bias)
+                torch.cuda.synchronize()
+                once = {}
+                for (name, e0), (_, e1) in zip(marks[:-1], marks[1:]):
+                    once[name or gap] = once.get(name or gap, 0.0) + e0.elapsed_time(e1)
+                runs.append(once)
+        finally:
+            nat.set_phase_hook(None)
+        return {k: sorted(r.get(k, 0.0) for r in runs)[len(runs) // 2] for k in runs[-1]}
+
+    phases_ms = build_phases()
     pairs = int(cache.valid_signal_seg.view(torch.int32)[-1].item()) if passes == 3 else \
         int((cache.neighbor_map.view(torch.int32) != -1).sum().item())
     n = wl.n
@@ -140,7 +192,8 @@ def main():
     if args.build_only:
         print(json.dumps({"metric": "neighbor-cache build", "workload": args.workload, "n": n, "pairs": pairs,
                           "build_ms_median": build_ms[len(build_ms) // 2], "build_ms_min": build_ms[0],
-                          "algorithmic_GBps": build_bytes / (build_ms[len(build_ms) // 2] * 1e-3) / 1e9}))
+                          "algorithmic_GBps": build_bytes / (build_ms[len(build_ms) // 2] * 1e-3) / 1e9,
+                          "phases_ms_median": phases_ms}))
         return
 
     # ---- the step ----
@@ -171,29 +224,41 @@ def main():
         events.setdefault(name, []).append(e)
 
     nat.EVENT_HOOK = hook
+    step_events = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats(dev)
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for i in range(args.steps):
+        step_events[i].record()
         step()
+    step_events[args.steps].record()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     nat.EVENT_HOOK = None
+    peak_bytes = torch.cuda.max_memory_allocated(dev)
 
     ms_per_step = elapsed * 1e3 / args.steps
+    step_ms = sorted(step_events[i].elapsed_time(step_events[i + 1]) for i in range(args.steps))
     flop_pass = 2.0 * pairs * c * c
     value = flop_pass * passes / (ms_per_step * 1e-3) / 1e12
 
-    def avg_ms(names):
-        tot, cnt = 0.0, 0
+    def pass_ms(names):
+        """(mean, median, min, count) of the event-timed calls of these names"""
+        ts = []
         for nm in names:
             ev = events.get(nm, [])
-            for i in range(0, len(ev) - 1, 2):
-                tot += ev[i].elapsed_time(ev[i + 1])
-                cnt += 1
-        return (tot / cnt if cnt else float("nan")), cnt
+            ts += [ev[i].elapsed_time(ev[i + 1]) for i in range(0, len(ev) - 1, 2)]
+        ts.sort()
+        if not ts:
+            return float("nan"), float("nan"), float("nan"), 0
+        return sum(ts) / len(ts), ts[len(ts) // 2], ts[0], len(ts)
 
-    gemm_ms, gemm_launches = avg_ms(["gather_gemm_fwd", "gather_gemm_dgrad"])
-    wgrad_ms, _ = avg_ms(["wgrad"])
+    def stats(names):
+        mean, med, lo, cnt = pass_ms(names)
+        return {"mean": mean, "median": med, "min": lo, "calls": cnt} if cnt else None
+
+    gemm_ms, _, _, gemm_launches = pass_ms(["gather_gemm_fwd", "gather_gemm_dgrad"])
+    wgrad_ms = pass_ms(["wgrad"])[0]
     es = 2 if dname != "f32" else 4
     gemm_bytes = es * n * (c + c) + es * 27 * c * c + 108.0 * n + 8.0 * n
     roof = {
@@ -204,9 +269,9 @@ def main():
         "algorithmic_flop_per_launch": flop_pass,
         "algorithmic_bytes_per_launch": gemm_bytes,
         "algorithmic_hbm_GBps": gemm_bytes / (gemm_ms * 1e-3) / 1e9,
-        "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+        "traffic": measured_traffic(args.workload, dname),
     }
-    if args.workload == "cfg4":   # C = 32: every pass is HBM bound
+    if c * es <= 64:   # rows of 64 bytes (configuration 4, C = 32): every pass is HBM bound
         roof.update({"bound": "hbm", "achieved": gemm_bytes / (gemm_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gemm_bytes / (gemm_ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
 
@@ -220,11 +285,15 @@ def main():
                                + ("fwd+dgrad+wgrad+dbias, neighbor cache prebuilt and reused" if passes == 3 else "forward"),
                    "n_voxels": n, "valid_pairs": pairs, "useful_gflop_per_step": flop_pass * passes / 1e9},
         "frac_of_mfma_peak": value / PEAK_TFLOPS[dname],
-        "pass_ms": {"gather_gemm_avg": gemm_ms, "wgrad_incl_reduce": wgrad_ms},
+        "pass_ms": {"gather_gemm_avg": gemm_ms, "wgrad_incl_reduce": wgrad_ms,
+                    "forward": stats(["gather_gemm_fwd"]), "dgrad": stats(["gather_gemm_dgrad"]), "wgrad": stats(["wgrad"])},
+        "step_ms": {"wall_mean": ms_per_step, "median": step_ms[len(step_ms) // 2], "min": step_ms[0]},
+        "peak_memory_bytes": peak_bytes,
         "neighbor_cache_build": {"ms_median": build_ms[len(build_ms) // 2], "ms_min": build_ms[0],
                                  "algorithmic_bytes": build_bytes,
                                  "algorithmic_GBps": build_bytes / (build_ms[len(build_ms) // 2] * 1e-3) / 1e9,
-                                 "frac_of_hbm_peak": build_bytes / (build_ms[len(build_ms) // 2] * 1e-3) / 1e9 / HBM_PEAK_GBS},
+                                 "frac_of_hbm_peak": build_bytes / (build_ms[len(build_ms) // 2] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                 "phases_ms_median": phases_ms},
         "roofline": roof,
     }
     if not args.no_cpu_baseline:

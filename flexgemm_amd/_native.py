@@ -22,7 +22,7 @@ PASS_FWD, PASS_DGRAD, PASS_WGRAD = 0, 1, 2
 
 # every symbol the header declares; the CPU-side test checks that the library exports each of them
 EXPORTS = [
-    "fgx_abi_version", "fgx_last_error",
+    "fgx_abi_version", "fgx_last_error", "fgx_set_phase_hook",
     "fgx_hash_init", "fgx_hash_insert_3d_idx_as_val", "fgx_hash_insert", "fgx_hash_lookup",
     "fgx_hash_insert_3d", "fgx_hash_lookup_3d",
     "fgx_subm_neighbor_map", "fgx_subm_neighbor_map_sorted_workspace_bytes", "fgx_subm_neighbor_map_sorted", "fgx_mask_codes",
@@ -51,6 +51,23 @@ EVENT_HOOK = None
 def mark(name: str, phase: str) -> None:
     if EVENT_HOOK is not None:
         EVENT_HOOK(name, phase)
+
+
+PHASE_HOOK_T = C.CFUNCTYPE(None, C.c_char_p, C.c_void_p)
+_phase_hook_ref = None      # keeps the ctypes trampoline alive while the library holds its address
+
+
+def set_phase_hook(fn) -> None:
+    """fn(phase_name: str, stream: int) is called by the library's multi-kernel calls right before each of their phases
+    is enqueued ("" after the last one); None switches it off (fgx_set_phase_hook)."""
+    global _phase_hook_ref
+    if fn is None:
+        lib().fgx_set_phase_hook(PHASE_HOOK_T(0))
+        _phase_hook_ref = None
+        return
+    cb = PHASE_HOOK_T(lambda name, stream: fn(name.decode() if name else "", stream))
+    lib().fgx_set_phase_hook(cb)
+    _phase_hook_ref = cb
 
 
 class Schedule(C.Structure):

@@ -43,6 +43,11 @@ inline int fail_hip(hipError_t e, const char* what) {
 // Names the phase whose kernels are enqueued next on `s` to the profiling hook (fgx_set_phase_hook), if one is set;
 // an empty name closes the last phase of a call.
 void phase_mark(const char* name, hipStream_t s);
+// closes the last phase when the call returns, by whichever path
+struct PhaseEnd {
+    hipStream_t s;
+    ~PhaseEnd() { phase_mark("", s); }
+};
 
 // Whether the persistent gather GEMM of this tile shape has room in a CU's 160 KiB of LDS for `cols` output columns
 // (it stages the bias of every column tile next to its rings); defined in conv_gemm_stream.hip.

@@ -306,8 +306,11 @@ int fgx_subm_neighbor_map(void* keys, int key_bits, uint32_t* vals, size_t table
     FGX_CHECK_ARG(keys && vals && coords && out_map, "fgx_subm_neighbor_map: null buffer");
     FGX_CHECK_ARG(((uintptr_t)coords & 15) == 0, "fgx_subm_neighbor_map: coords must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
+    PhaseEnd phases{s};
+    phase_mark("hash insert", s);
     int rc = fgx_hash_insert_3d_idx_as_val(keys, key_bits, vals, 32, table_size, coords, n, W, H, D, stream);
     if (rc != FGX_OK) return rc;
+    phase_mark("hash probe", s);
     if (V <= 32) {
         unsigned grid = cdiv(n * 32, kBlock);
         if (key_bits == 32)

@@ -491,6 +491,8 @@ int fgx_sort_by_code(const int32_t* binary, size_t n, int V, int64_t* sorted_idx
     int32_t* keys_out = (int32_t*)(ws + L.keys_out);
     uint32_t* vals_in = (uint32_t*)(ws + L.vals_in);
     uint32_t* vals_out = (uint32_t*)(ws + L.vals_out);
+    PhaseEnd phases{s};
+    phase_mark("mask sort", s);
     iota_u32_kernel<<<cdiv(n, kBlock), kBlock, 0, s>>>(vals_in, n);
     FGX_CHECK_LAUNCH("fgx_sort_by_code(iota)");
     size_t temp_bytes = L.temp_bytes;
@@ -553,6 +555,8 @@ int fgx_pair_count(const int32_t* gray, size_t n, int V, uint32_t* seg, void* wo
     char* ws = (char*)workspace;
     uint32_t* counts = n ? (uint32_t*)(ws + L.counts) : nullptr;
     uint32_t* offsets = n ? (uint32_t*)(ws + L.offsets) : nullptr;
+    PhaseEnd phases{s};
+    phase_mark("pair count", s);
     if (n > 0) {
         pair_count_kernel<<<L.nblk, kPairThreads, 0, s>>>(gray, n, V, L.nblk, counts);
         FGX_CHECK_LAUNCH("fgx_pair_count(count)");
@@ -573,6 +577,8 @@ int fgx_pair_fill(const uint32_t* map, const int32_t* gray, size_t n, int V, con
     PairLayout L = pair_layout(n, V);
     const uint32_t* offsets = (const uint32_t*)((const char*)workspace + L.offsets);
     size_t lds = ((size_t)kPairThreads * V + 2 * (kPairThreads / 64) * 32 + 32) * sizeof(uint32_t);
+    PhaseEnd phases{(hipStream_t)stream};
+    phase_mark("pair fill", (hipStream_t)stream);
     pair_fill_kernel<<<L.nblk, kPairThreads, lds, (hipStream_t)stream>>>(map, gray, n, V, L.nblk, offsets, sig_i, sig_o);
     FGX_CHECK_LAUNCH("fgx_pair_fill");
     return FGX_OK;
@@ -596,6 +602,8 @@ int fgx_tile_codes(const int32_t* gray, const int64_t* sorted_idx, size_t n, int
     FGX_CHECK_ARG(((uintptr_t)workspace & 255) == 0, "fgx_tile_codes: workspace must be 256-byte aligned");
     char* ws = (char*)workspace;
     uint32_t* popc = (uint32_t*)(ws + L.popc);
+    PhaseEnd phases{s};
+    phase_mark("tile masks", s);
     tile_or_kernel<<<cdiv(L.num_tiles * 64, kBlock), kBlock, 0, s>>>(gray, sorted_idx, n, block, L.num_tiles, tile_code, popc);
     FGX_CHECK_LAUNCH("fgx_tile_codes(or)");
     size_t temp_bytes = L.temp_bytes;
@@ -630,6 +638,8 @@ int fgx_gather_plan_count(const int32_t* tile_code, size_t num_tiles, int32_t* p
     FGX_CHECK_ARG(((uintptr_t)workspace & 255) == 0, "fgx_gather_plan_count: workspace must be 256-byte aligned");
     unsigned char* ws = (unsigned char*)workspace;
     uint32_t* cnt = (uint32_t*)(ws + L.popc);
+    PhaseEnd phases{s};
+    phase_mark("gather plan count", s);
     plan_count_kernel<<<cdiv(num_tiles, kBlock), kBlock, 0, s>>>(tile_code, num_tiles, cnt);
     FGX_CHECK_LAUNCH("fgx_gather_plan_count(count)");
     size_t temp_bytes = L.temp_bytes;
@@ -648,6 +658,8 @@ int fgx_gather_plan_fill(const uint32_t* map, const int64_t* order, const int32_
     const size_t num_tiles = (n + tile_rows - 1) / tile_rows;
     FGX_CHECK_ARG(num_tiles <= 0x7FFFFFFFu, "fgx_gather_plan_fill: too many tiles");
     FGX_CHECK_ARG(plan_band == nullptr || tile_rows <= 1024, "fgx_gather_plan_fill: band masks need tile_rows <= 1024");
+    PhaseEnd phases{(hipStream_t)stream};
+    phase_mark("gather plan fill", (hipStream_t)stream);
     plan_fill_kernel<<<(unsigned)num_tiles, kBlock, 0, (hipStream_t)stream>>>(map, order, tile_code, plan_seg, n, V, tile_rows,
                                                                               plan_idx, plan_band);
     FGX_CHECK_LAUNCH("fgx_gather_plan_fill");

@@ -322,6 +322,8 @@ int build_sorted(const int32_t* coords, size_t n, uint64_t vol, const SubmGeom& 
     K* keys_out = (K*)(ws + L.keys_out);
     uint32_t* rows_in = (uint32_t*)(ws + L.rows_in);
     uint32_t* rows_out = (uint32_t*)(ws + L.rows_out);
+    PhaseEnd phases{s};
+    phase_mark("key sort", s);
     flat_keys_kernel<K><<<cdiv(n, 256), 256, 0, s>>>(coords, n, g.W, g.H, g.D, keys_in, rows_in);
     FGX_CHECK_LAUNCH("fgx_subm_neighbor_map_sorted(keys)");
     size_t temp_bytes = L.temp_bytes;
@@ -331,8 +333,10 @@ int build_sorted(const int32_t* coords, size_t n, uint64_t vol, const SubmGeom& 
                                             n, 0u, end_bit, s));
     const unsigned groups = cdiv(n, kGroup);
     uint32_t* bounds = (uint32_t*)(ws + L.bounds);
+    phase_mark("window bounds", s);
     window_bounds_kernel<K><<<cdiv((size_t)groups * g.Kw * g.Kh * 2, 256), 256, 0, s>>>(keys_out, n, (unsigned long long)vol, g, groups, bounds);
     FGX_CHECK_LAUNCH("fgx_subm_neighbor_map_sorted(bounds)");
+    phase_mark("merge", s);
     merge_neighbor_kernel<K><<<groups, kGroup, 0, s>>>(keys_out, rows_out, bounds, n, g, out_map, gray, binary);
     FGX_CHECK_LAUNCH("fgx_subm_neighbor_map_sorted");
     return FGX_OK;
