@@ -28,6 +28,8 @@
 //
 // dgrad is the same kernel: src = grad_output and a panel packed with the mirrored, transposed
 // weight (fgx_pack_weight mode 1).
+#include <atomic>
+
 #include "gemm_device.h"
 
 namespace fgx {
@@ -592,8 +594,37 @@ int dispatch_tile(int tile_rows, int tile_cols, int slab_bytes, const void* src,
     return FGX_ERR_UNSUPPORTED;
 }
 
+// both column-sum kernels on `s`, partial sums in `scratch` (kColsumSlices x cols floats)
+int colsum_launch(int dtype, const void* x, size_t n, int cols, float* scratch, void* out, hipStream_t s) {
+    unsigned slices = n ? (unsigned)((n + 255) / 256) : 0u;     // at least 256 rows per slice
+    if (slices > (unsigned)kColsumSlices) slices = kColsumSlices;
+    const unsigned gfin = cdiv(cols, 16);
+    const int es = elem_size(dtype);
+    const bool vec = ((size_t)cols * es) % 16 == 0 && ((uintptr_t)x & 15) == 0;
+#define FGX_COLSUM(T, VEC)                                                                                  \
+    do {                                                                                                    \
+        if (slices) colsum_partial_kernel<T, VEC><<<slices, 256, 0, s>>>((const T*)x, n, cols, scratch);    \
+        colsum_final_kernel<T><<<gfin, 256, 0, s>>>((const float*)scratch, slices, cols, (T*)out);          \
+    } while (0)
+    if (dtype == FGX_F16) { if (vec) FGX_COLSUM(_Float16, 8); else FGX_COLSUM(_Float16, 1); }
+    else if (dtype == FGX_BF16) { if (vec) FGX_COLSUM(__bf16, 8); else FGX_COLSUM(__bf16, 1); }
+    else { if (vec) FGX_COLSUM(float, 4); else FGX_COLSUM(float, 1); }
+#undef FGX_COLSUM
+    FGX_CHECK_LAUNCH("fgx_colsum");
+    return FGX_OK;
+}
+
+constexpr int kStaticColsumCols = 2048;     // widest tensor fgx_colsum_static serves
+constexpr int kMaxDevices = 64;
+
 }  // namespace
 }  // namespace fgx
+
+// Scratch of fgx_colsum_static: the partial sums of the column sum for up to kStaticColsumCols columns (8 MiB), held
+// by every GPU the library runs on until the process ends.  In host code this name is only a handle for
+// hipGetSymbolAddress: kernels and copies are given the device address found there (one per device), never the name.
+static __device__ __align__(256) float g_static_colsum_scratch[(size_t)fgx::kColsumSlices * fgx::kStaticColsumCols];
+static std::atomic<float*> g_static_colsum_ptr[fgx::kMaxDevices];
 
 using namespace fgx;
 
@@ -694,23 +725,31 @@ int fgx_colsum(int dtype, const void* x, size_t n, int cols, void* scratch, void
     FGX_CHECK_ARG(dtype_ok(dtype), "fgx_colsum: unknown dtype %d", dtype);
     FGX_CHECK_ARG(cols > 0 && out != nullptr, "fgx_colsum: bad shape or null output");
     FGX_CHECK_ARG(scratch != nullptr && (n == 0 || x != nullptr), "fgx_colsum: null buffer");
-    hipStream_t s = (hipStream_t)stream;
-    unsigned slices = n ? (unsigned)((n + 255) / 256) : 0u;     // at least 256 rows per slice
-    if (slices > (unsigned)kColsumSlices) slices = kColsumSlices;
-    const unsigned gfin = cdiv(cols, 16);
-    const int es = elem_size(dtype);
-    const bool vec = ((size_t)cols * es) % 16 == 0 && ((uintptr_t)x & 15) == 0;
-#define FGX_COLSUM(T, VEC)                                                                                        \
-    do {                                                                                                          \
-        if (slices) colsum_partial_kernel<T, VEC><<<slices, 256, 0, s>>>((const T*)x, n, cols, (float*)scratch);   \
-        colsum_final_kernel<T><<<gfin, 256, 0, s>>>((const float*)scratch, slices, cols, (T*)out);                \
-    } while (0)
-    if (dtype == FGX_F16) { if (vec) FGX_COLSUM(_Float16, 8); else FGX_COLSUM(_Float16, 1); }
-    else if (dtype == FGX_BF16) { if (vec) FGX_COLSUM(__bf16, 8); else FGX_COLSUM(__bf16, 1); }
-    else { if (vec) FGX_COLSUM(float, 4); else FGX_COLSUM(float, 1); }
-#undef FGX_COLSUM
-    FGX_CHECK_LAUNCH("fgx_colsum");
-    return FGX_OK;
+    return colsum_launch(dtype, x, n, cols, (float*)scratch, out, (hipStream_t)stream);
+}
+
+int fgx_colsum_static_max_cols(void) { return kStaticColsumCols; }
+
+int fgx_colsum_static(int dtype, const void* x, size_t n, int cols, void* out, fgx_stream_t stream) {
+    FGX_CHECK_ARG(dtype_ok(dtype), "fgx_colsum_static: unknown dtype %d", dtype);
+    FGX_CHECK_ARG(cols > 0 && out != nullptr, "fgx_colsum_static: bad shape or null output");
+    FGX_CHECK_ARG(n == 0 || x != nullptr, "fgx_colsum_static: null buffer");
+    FGX_CHECK_ARG(cols <= kStaticColsumCols,
+                  "fgx_colsum_static: %d columns exceed the %d the library's own scratch holds; use fgx_colsum with caller-owned scratch",
+                  cols, kStaticColsumCols);
+    // The device address of this GPU's copy of the array, looked up once per device with that device current.
+    int dev = 0;
+    FGX_CHECK_HIP(hipGetDevice(&dev));
+    FGX_CHECK_ARG(dev >= 0 && dev < kMaxDevices, "fgx_colsum_static: device ordinal %d out of range", dev);
+    float* ptr = g_static_colsum_ptr[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        void* found = nullptr;
+        FGX_CHECK_HIP(hipGetSymbolAddress(&found, HIP_SYMBOL(g_static_colsum_scratch)));
+        FGX_CHECK_ARG(found != nullptr, "fgx_colsum_static: the scratch array has no address on device %d", dev);
+        ptr = (float*)found;
+        g_static_colsum_ptr[dev].store(ptr, std::memory_order_release);     // (two first callers find the same address)
+    }
+    return colsum_launch(dtype, x, n, cols, ptr, out, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -308,6 +308,16 @@ size_t fgx_colsum_scratch_bytes(size_t n, int cols);
 int fgx_colsum(int dtype, const void* grad_out, size_t n, int cols, void* scratch, void* out,
                fgx_stream_t stream);
 
+/* fgx_colsum without a scratch argument, for callers that cannot allocate (code under HIP graph capture, serving loops
+ * with a fixed memory plan, harnesses that forbid hipMalloc): the fp32 partial sums go to an array the library itself
+ * holds on every GPU it runs on (8 MiB, for up to fgx_colsum_static_max_cols() = 2048 columns; wider tensors are
+ * refused with FGX_ERR_ARG).  Allocates nothing, same kernels and same bits as fgx_colsum.  All calls on one GPU share
+ * that array: calls that may overlap there (different streams, different threads) race -- serialise them.  Every
+ * call overwrites the part it reads, so nothing has to be cleared between calls.
+ * No counterpart in the reference (torch allocates its reduction buffers itself). */
+int fgx_colsum_static_max_cols(void);
+int fgx_colsum_static(int dtype, const void* grad_out, size_t n, int cols, void* out, fgx_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Generic sparse convolution (stride / padding / dilation): output coordinates and neighbor maps.
  * The GEMM passes are the ones above: forward gathers feats through map_fwd (n = output rows, n_src = input
