@@ -96,6 +96,22 @@ __device__ __forceinline__ void lds_wait_but(i16x4 (&r)[R]) {
 #endif
 }
 
+// bounds[v * (nb + 1) + b] = first pair of offset v whose output row is >= b * block_rows
+__global__ void __launch_bounds__(256) block_bounds_kernel(const uint32_t* __restrict__ sig_o, SegTable tab, int V,
+                                                           unsigned nb, unsigned block_rows,
+                                                           uint32_t* __restrict__ bounds) {
+    const unsigned t = blockIdx.x * 256 + threadIdx.x;
+    if (t >= (unsigned)V * (nb + 1)) return;
+    const unsigned v = t / (nb + 1), b = t % (nb + 1);
+    uint32_t lo = tab.seg[v], hi = tab.seg[v + 1];
+    const uint64_t target = (uint64_t)b * block_rows;
+    while (lo < hi) {
+        uint32_t mid = lo + ((hi - lo) >> 1);
+        if ((uint64_t)sig_o[mid] < target) lo = mid + 1;
+        else hi = mid;
+    }
+    bounds[t] = lo;
+}
 
 }  // namespace
 }  // namespace fgx

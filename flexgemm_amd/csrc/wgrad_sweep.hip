@@ -1,0 +1,928 @@
+// Weight gradient of the masked implicit GEMM as a paced sweep over the voxels, for gfx950 (16-bit types, a single
+// Co x Ci tile of 128 x 128 or 64 x 64, many voxels).
+//
+// grad_weight[:, v, :] = sum over the pairs (n -> m at offset v) of grad_out[n]^T feats[m]
+// (reference: flex_gemm/kernels/triton/spconv/sparse_submanifold_conv_bwd_masked_implicit_gemm_splitk.py:108-182,
+// 278-317, which cuts the pairs of every offset into SPLITK slices with a partial product each).
+//
+// The block-major kernel of wgrad_gemm.hip cuts the voxels into blocks of ~12K rows and writes an fp32 partial product
+// per (block, offset): the 27 offset items of a block share its rows through an XCD's L2, but the block's rows (4.7 MB
+// at 128 channels) overflow the 4 MiB L2 while smaller blocks multiply the partial products.  Here
+//
+//   * XCD x owns one contiguous eighth of the voxels (pair lists ascend in the output row inside every offset, so that
+//     is one contiguous pair range per offset);
+//   * the pairs of an XCD's range are cut into 2 x (workgroups per XCD) parts of nearly equal size -- an offset with
+//     many pairs is split into several parts that take its 64-pair steps in turn -- and every workgroup gets two parts,
+//     a large and a small one, and KEEPS BOTH ACCUMULATORS IN REGISTERS for the whole range: 512 partial products in
+//     all instead of one per (block, offset);
+//   * a workgroup takes the steps of its two parts in the order of the sub-block (1024 voxels) their pairs lie in, and
+//     the workgroups of an XCD pace each other: nobody starts a sub-block more than `lead` sub-blocks ahead of the
+//     slowest, so the rows the 32 workgroups gather at any time span a few thousand voxels and are fetched into the
+//     XCD's L2 once for all offsets.  The wait is bounded: after max_polls polls a workgroup goes on regardless, so the
+//     kernel ends whatever the progress words say.
+//
+// The step sequence of every workgroup is a function of the pair lists alone: fgx_wgrad_sweep_plan builds it once per
+// neighbor cache.  Sums are taken in a fixed order (steps in list order, parts in ascending order), so results are the
+// same on every run; they differ from the block-major kernels' in the order of the fp32 additions.
+#include <type_traits>
+
+#include "wgrad_device.h"
+
+namespace fgx {
+namespace {
+
+constexpr int kSwStages = 4;         // row ring depth
+constexpr int kSwIdxSlots = 8;       // index ring depth
+constexpr int kSwIdxAhead = 4;       // index loads run this many steps ahead of the row loads
+constexpr int kSwLoaders = 4;
+constexpr int kSwPairs = 64;         // pairs per step
+constexpr int kSwStepRing = 256;     // step-list entries held in LDS (four chunks of 64)
+constexpr int kSwMergeShift = 1;     // a workgroup changes units every 2^this sub-blocks (a change swaps the accumulators)
+constexpr int kSwMaxSlots = 64;      // workgroups per XCD the pacing poll can look at (one lane each)
+constexpr int kSwMaxGroups = kXcds * kSwMaxSlots;
+
+// ------------------------------------------------------------------------------------------------
+// Plan: fine bounds, units (parts), per-workgroup step lists
+// ------------------------------------------------------------------------------------------------
+struct SweepUnit {
+    uint32_t v, p, P;       // offset, part index, parts of this offset in this XCD
+    uint32_t lo, hi;        // pair range of the offset inside the XCD's voxels
+    uint32_t nsteps;
+};
+struct SweepGroup {         // one workgroup
+    uint32_t step_off, nsteps;
+    uint32_t sb0;           // first sub-block of its XCD
+    uint32_t active;        // workgroups of its XCD that have steps
+};
+
+struct SweepLayout {
+    unsigned nsb, groups, spx;
+    size_t fine, units, wg, vcount, vlist, steps_k, steps_m, step_cap, total;
+};
+
+SweepLayout sweep_layout(size_t n, size_t n_pairs, int V, int sub_rows, int groups) {
+    SweepLayout L{};
+    L.nsb = n ? cdiv(n, (size_t)sub_rows) : 0u;
+    L.groups = (unsigned)groups;
+    L.spx = (unsigned)groups / kXcds;
+    size_t off = 0;
+    L.fine = off;
+    off = align_up(off + (size_t)V * (L.nsb + 1) * 4, 256);
+    L.units = off;
+    off = align_up(off + (size_t)groups * 2 * sizeof(SweepUnit), 256);
+    L.wg = off;
+    off = align_up(off + (size_t)groups * sizeof(SweepGroup), 256);
+    L.vcount = off;
+    off = align_up(off + (size_t)kMaxV * 4, 256);
+    L.vlist = off;
+    off = align_up(off + (size_t)kMaxV * groups * 2 * 2, 256);
+    // every unit's steps: at most pairs / 64 whole steps in all plus one ragged step per unit
+    L.step_cap = n_pairs / kSwPairs + (size_t)groups * 2 + 64;
+    L.steps_k = off;
+    off = align_up(off + L.step_cap * 4, 256);
+    L.steps_m = off;
+    off = align_up(off + L.step_cap * 4, 256);
+    L.total = off;
+    return L;
+}
+
+__device__ __forceinline__ uint32_t unit_steps(uint32_t cnt, uint32_t p, uint32_t P) {
+    const uint64_t first = (uint64_t)p * kSwPairs;
+    if (P == 0 || cnt <= first) return 0;
+    return (uint32_t)((cnt - first + (uint64_t)P * kSwPairs - 1) / ((uint64_t)P * kSwPairs));
+}
+
+// One thread per XCD cuts its pair ranges into 2 * spx parts and pairs them up; thread 0 then lays out the step lists
+// and the per-offset lists of partial products.  A few thousand scalar operations in all.
+__global__ void __launch_bounds__(64) sweep_units_kernel(const uint32_t* __restrict__ fine, int V, unsigned nsb, unsigned spx,
+                                                         SweepUnit* __restrict__ units, SweepGroup* __restrict__ wg,
+                                                         uint32_t* __restrict__ vcount, uint16_t* __restrict__ vlist) {
+    const unsigned x = threadIdx.x;
+    const unsigned slots = 2 * spx;
+    if (x < (unsigned)kXcds) {
+        // XCD x takes the sub-blocks [sbA, sbB): boundaries where the running pair count (all offsets) passes x / 8 of
+        // the total, so that the XCDs get equal work rather than equal voxel counts
+        auto pairs_before = [&](unsigned sb) {
+            uint64_t c = 0;
+            for (int v = 0; v < V; ++v) c += fine[(size_t)v * (nsb + 1) + sb] - fine[(size_t)v * (nsb + 1)];
+            return c;
+        };
+        auto boundary = [&](unsigned xc) -> unsigned {
+            if (xc == 0) return 0u;
+            if (xc >= (unsigned)kXcds) return nsb;
+            const uint64_t want = pairs_before(nsb) * xc / kXcds;
+            unsigned lo_sb = 0, hi_sb = nsb;            // first sub-block boundary with at least `want` pairs before it
+            while (lo_sb < hi_sb) {
+                const unsigned mid = (lo_sb + hi_sb) >> 1;
+                if (pairs_before(mid) < want) lo_sb = mid + 1;
+                else hi_sb = mid;
+            }
+            return lo_sb;
+        };
+        const unsigned sbA = boundary(x), sbB = boundary(x + 1);
+        uint32_t lo[kMaxV], cnt[kMaxV], P[kMaxV];
+        unsigned parts = 0;
+        for (int v = 0; v < V; ++v) {
+            lo[v] = fine[(size_t)v * (nsb + 1) + sbA];
+            cnt[v] = fine[(size_t)v * (nsb + 1) + sbB] - lo[v];
+            P[v] = cnt[v] ? 1u : 0u;
+            parts += P[v];
+        }
+        // split the offset with the largest parts until every slot has one (never below one step per part)
+        while (parts > 0 && parts < slots) {
+            int best = -1;
+            float best_size = 0.f;
+            for (int v = 0; v < V; ++v) {
+                if (!P[v]) continue;
+                const float size = (float)cnt[v] / (float)P[v];
+                if (size > best_size) {
+                    best_size = size;
+                    best = v;
+                }
+            }
+            if (best < 0 || best_size <= (float)kSwPairs) break;
+            ++P[best];
+            ++parts;
+        }
+        // parts by descending size (insertion sort, stable in (offset, part) order)
+        uint16_t order_v[2 * kSwMaxSlots], order_p[2 * kSwMaxSlots];
+        float order_s[2 * kSwMaxSlots];
+        unsigned m = 0;
+        for (int v = 0; v < V; ++v)
+            for (uint32_t p = 0; p < P[v]; ++p) {
+                const float size = (float)cnt[v] / (float)P[v];
+                unsigned at = m;
+                while (at > 0 && order_s[at - 1] < size) {
+                    order_s[at] = order_s[at - 1];
+                    order_v[at] = order_v[at - 1];
+                    order_p[at] = order_p[at - 1];
+                    --at;
+                }
+                order_s[at] = size;
+                order_v[at] = (uint16_t)v;
+                order_p[at] = (uint16_t)p;
+                ++m;
+            }
+        // workgroup s: the s-th largest part and the s-th smallest
+        for (unsigned s = 0; s < spx; ++s) {
+            for (int u = 0; u < 2; ++u) {
+                const unsigned at = u == 0 ? s : slots - 1 - s;
+                SweepUnit un{};
+                if (at < m) {
+                    const unsigned v = order_v[at];
+                    un.v = v;
+                    un.p = order_p[at];
+                    un.P = P[v];
+                    un.lo = lo[v];
+                    un.hi = lo[v] + cnt[v];
+                    un.nsteps = unit_steps(cnt[v], un.p, un.P);
+                }
+                units[((size_t)x * spx + s) * 2 + u] = un;
+            }
+            wg[(size_t)x * spx + s].sb0 = sbA;
+        }
+    }
+    __syncthreads();
+    if (x == 0) {
+        uint32_t off = 0;
+        for (unsigned xc = 0; xc < (unsigned)kXcds; ++xc) {
+            uint32_t active = 0;
+            for (unsigned s = 0; s < spx; ++s) {
+                const size_t g = (size_t)xc * spx + s;
+                const uint32_t ns = units[g * 2].nsteps + units[g * 2 + 1].nsteps;
+                wg[g].step_off = off;
+                wg[g].nsteps = ns;
+                off += ns;
+                active += ns ? 1u : 0u;
+            }
+            for (unsigned s = 0; s < spx; ++s) wg[(size_t)xc * spx + s].active = active;
+        }
+        for (int v = 0; v < V; ++v) vcount[v] = 0;
+        const unsigned total_units = kXcds * spx * 2;
+        for (unsigned q = 0; q < total_units; ++q) {
+            if (!units[q].nsteps) continue;
+            const uint32_t v = units[q].v;
+            vlist[(size_t)v * total_units + vcount[v]] = (uint16_t)q;
+            ++vcount[v];
+        }
+    }
+}
+
+// number of steps of unit u whose first pair lies below `bound`
+__device__ __forceinline__ uint32_t steps_below(const SweepUnit& u, uint32_t bound) {
+    const uint64_t first = (uint64_t)u.lo + (uint64_t)u.p * kSwPairs;
+    if (u.nsteps == 0 || (uint64_t)bound <= first) return 0;
+    const uint64_t c = ((uint64_t)bound - first + (uint64_t)u.P * kSwPairs - 1) / ((uint64_t)u.P * kSwPairs);
+    return c < u.nsteps ? (uint32_t)c : u.nsteps;
+}
+
+// The merged step list of one workgroup per block: its two units' steps ordered by the group of sub-blocks their first
+// pair lies in, unit 0 first inside a group.  Entry: first pair | pairs in the step (7 bits), unit (1 bit), sub-block relative to
+// the XCD's first (24 bits).
+__global__ void __launch_bounds__(256) sweep_steps_kernel(const uint32_t* __restrict__ fine, unsigned nsb,
+                                                          const SweepUnit* __restrict__ units,
+                                                          const SweepGroup* __restrict__ wg, uint32_t* __restrict__ steps_k,
+                                                          uint32_t* __restrict__ steps_m, size_t step_cap) {
+    const unsigned g = blockIdx.x;
+    const SweepGroup grp = wg[g];
+    const SweepUnit u0 = units[(size_t)g * 2], u1 = units[(size_t)g * 2 + 1];
+    const unsigned sbA = grp.sb0;
+    for (int u = 0; u < 2; ++u) {
+        const SweepUnit& me = u == 0 ? u0 : u1;
+        const SweepUnit& other = u == 0 ? u1 : u0;
+        const uint32_t* mine = fine + (size_t)me.v * (nsb + 1);
+        const uint32_t* theirs = fine + (size_t)other.v * (nsb + 1);
+        for (uint32_t j = threadIdx.x; j < me.nsteps; j += 256) {
+            const uint32_t k = me.lo + (me.p + j * me.P) * kSwPairs;
+            const uint32_t left = me.hi - k;
+            // sub-block of pair k: the last s with mine[s] <= k (pairs of the XCD start at sub-block sbA)
+            unsigned lo = sbA, hi = nsb;            // invariant: mine[lo] <= k, answer in [lo, hi)
+            while (hi - lo > 1) {
+                const unsigned mid = (lo + hi) >> 1;
+                if (mine[mid] <= k) lo = mid;
+                else hi = mid;
+            }
+            const unsigned sb = lo;
+            // the two units take turns by groups of 2^kSwMergeShift sub-blocks: the other unit's steps in earlier groups
+            // and, for unit 1, in this one (unit 0 goes first)
+            const unsigned grp_first = sbA + (((sb - sbA) >> kSwMergeShift) << kSwMergeShift);
+            const unsigned grp_end = grp_first + (1u << kSwMergeShift) < nsb ? grp_first + (1u << kSwMergeShift) : nsb;
+            const uint32_t before = u == 0 ? steps_below(other, theirs[grp_first]) : steps_below(other, theirs[grp_end]);
+            const size_t at = (size_t)grp.step_off + j + before;
+            if (at < step_cap) {
+                steps_k[at] = k;
+                steps_m[at] = (left < (uint32_t)kSwPairs ? left : (uint32_t)kSwPairs) | ((uint32_t)u << 7) | ((sb - sbA) << 8);
+            }
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256) sweep_clear_kernel(uint32_t* __restrict__ prog, unsigned n) {
+    const unsigned i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) prog[i] = 0u;
+}
+
+// ------------------------------------------------------------------------------------------------
+// The kernel
+// ------------------------------------------------------------------------------------------------
+// Exchange two accumulator tiles in place.  Written as register swaps by hand: left to the compiler, "whose sums are
+// in the working registers" becomes a copy of a whole tile into a third set of registers before every step and back
+// after it.
+__device__ __forceinline__ void swap_tiles(f32x16& a, f32x16& b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        float x = a[e], y = b[e];
+        asm volatile("v_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+        a[e] = x;
+        b[e] = y;
+    }
+#endif
+}
+
+// sum of the eight 16-bit values of a fragment, in fp32
+template <typename Tag> __device__ __forceinline__ float sum8(const i16x8& f);
+template <> __device__ __forceinline__ float sum8<F16>(const i16x8& f) {
+    const f16x8 h = __builtin_bit_cast(f16x8, f);
+    return (((float)h[0] + (float)h[1]) + ((float)h[2] + (float)h[3])) + (((float)h[4] + (float)h[5]) + ((float)h[6] + (float)h[7]));
+}
+template <> __device__ __forceinline__ float sum8<BF16>(const i16x8& f) {
+    const u32x4 w = __builtin_bit_cast(u32x4, f);
+    float s = 0.f;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+        s += __builtin_bit_cast(float, w[q] << 16) + __builtin_bit_cast(float, w[q] & 0xFFFF0000u);
+    return s;
+}
+
+template <typename Tag, int BM, int BN>
+struct SweepCfg {
+    using T = typename Tag::type;
+    static constexpr int ES = (int)sizeof(T);
+    static constexpr int P = kSwPairs, S = kSwStages;
+    static constexpr int NW = 4, NL = kSwLoaders, NT = 64 * (NW + NL);
+    static constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+    static constexpr int ROWB_A = BM * ES, ROWB_B = BN * ES;
+    static constexpr int CH_A = ROWB_A / 16, CH_B = ROWB_B / 16;
+    static constexpr int RPI_A = 64 / CH_A, RPI_B = 64 / CH_B;
+    static constexpr int A_PER = P / RPI_A / NL, B_PER = P / RPI_B / NL;
+    static constexpr int LPS = A_PER + B_PER;
+    static constexpr int A_BYTES = P * ROWB_A, B_BYTES = P * ROWB_B, STAGE_BYTES = A_BYTES + B_BYTES;
+    static constexpr int IDX_SLOT_BYTES = 2 * P * 4;               // sig_o x P | sig_i x P
+    static constexpr size_t lds_bytes = (size_t)S * STAGE_BYTES + (size_t)kSwIdxSlots * IDX_SLOT_BYTES + (size_t)kSwStepRing * 8;
+    static_assert(ES == 2, "16-bit types");
+    static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
+    static_assert(P % (RPI_A * NL) == 0 && P % (RPI_B * NL) == 0, "every loader issues the same row loads");
+    static_assert(2 * (LPS + 3) < 64, "outstanding loads exceed the vmcnt range");
+    static constexpr int key_a(int row) { return CH_A >= 8 ? 2 * (row & 3) : 0; }
+    static constexpr int key_b(int row) { return CH_B >= 8 ? 2 * (row & 3) : 0; }
+};
+
+template <typename Tag, int BM, int BN>
+__global__ void __launch_bounds__(64 * (4 + kSwLoaders))
+wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename Tag::type* __restrict__ feats,
+                   const uint32_t* __restrict__ sig_i, const uint32_t* __restrict__ sig_o,
+                   const SweepUnit* __restrict__ units, const SweepGroup* __restrict__ groups_tab,
+                   const uint32_t* __restrict__ steps_k, const uint32_t* __restrict__ steps_m, unsigned spx, int V, int Ci,
+                   int Co, uint32_t n_pairs, uint32_t gout_bytes, uint32_t feats_bytes, float* __restrict__ partial,
+                   float* __restrict__ bias_partial, int bias_offset, uint32_t* __restrict__ prog, unsigned lead,
+                   unsigned max_polls) {
+    using C = SweepCfg<Tag, BM, BN>;
+    constexpr int ES = C::ES, S = C::S, P = C::P;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    unsigned char* ring = lds_raw;                                              // [S][A rows | B rows]
+    uint32_t* idx_ring = (uint32_t*)(ring + S * C::STAGE_BYTES);                // [kSwIdxSlots][o x P | i x P]
+    uint32_t* step_k = idx_ring + kSwIdxSlots * 2 * P;                          // [kSwStepRing] first pair of a step
+    uint32_t* step_m = step_k + kSwStepRing;                                    // [kSwStepRing] count | unit | sub-block
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool loader = wave >= C::NW;
+    const int lw = loader ? wave - C::NW : 0, mw = loader ? 0 : wave;
+    const int wave_m = mw >> 1, wave_n = mw & 1;
+    const int g = lane >> 5, l32 = lane & 31;
+
+    // workgroup ids are dealt round-robin to the XCDs
+    const unsigned xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
+    const unsigned gid = xcd * spx + slot;
+    const SweepGroup grp = groups_tab[gid];
+    const unsigned nsteps = grp.nsteps;
+    uint32_t* my_prog = prog + gid;
+    if (nsteps == 0) {                               // nothing to do: nobody has to wait for this workgroup
+        if (tid == 0) __hip_atomic_store(my_prog, 0xFFFFFFFFu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+    }
+
+    const rsrc_t gout_rs = make_rsrc(gout, gout_bytes);
+    const rsrc_t feats_rs = make_rsrc(feats, feats_bytes);
+    const rsrc_t sigo_rs = make_rsrc(sig_o, n_pairs * 4u);
+    const rsrc_t sigi_rs = make_rsrc(sig_i, n_pairs * 4u);
+    const rsrc_t stepk_rs = make_rsrc(steps_k + grp.step_off, nsteps * 4u);     // reads past the list give zeros
+    const rsrc_t stepm_rs = make_rsrc(steps_m + grp.step_off, nsteps * 4u);
+    const uint32_t rowb_o = (uint32_t)Co * ES, rowb_i = (uint32_t)Ci * ES;
+
+    // 64 entries of the step list into LDS (chunk c -> ring quarter c & 3)
+    auto load_chunk = [&](unsigned c) {
+        uint32_t* dk = step_k + (c & 3) * 64;
+        uint32_t* dm = step_m + (c & 3) * 64;
+        const uint32_t vo = (c * 64 + (uint32_t)lane) * 4u;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(stepk_rs, FGX_LDS_PTR(dk), 4, vo, 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(stepm_rs, FGX_LDS_PTR(dm), 4, vo, 0, 0, 0);
+    };
+
+    if (loader) {
+        // =============================================================================================
+        // loaders
+        // =============================================================================================
+        if (lw == 0) {
+            load_chunk(0);
+            load_chunk(1);
+            wait_vmcnt<0>();
+        }
+        __syncthreads();                            // (1) the first two chunks of the step list are in LDS
+        int a_row[C::A_PER], b_row[C::B_PER];
+        uint32_t a_chb[C::A_PER], b_chb[C::B_PER];          // byte column inside the tile, swizzle applied
+#pragma unroll
+        for (int i = 0; i < C::A_PER; ++i) {
+            a_row[i] = (i * C::NL + lw) * C::RPI_A + lane / C::CH_A;
+            a_chb[i] = (uint32_t)(((lane % C::CH_A) ^ C::key_a(a_row[i])) * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < C::B_PER; ++i) {
+            b_row[i] = (i * C::NL + lw) * C::RPI_B + lane / C::CH_B;
+            b_chb[i] = (uint32_t)(((lane % C::CH_B) ^ C::key_b(b_row[i])) * 16);
+        }
+        unsigned f_step = 0, r_step = 0;            // index stream, row stream: steps handed out so far
+        // The list entries of the two streams' next steps are read one round early (right after the previous ones were
+        // used), so that their LDS latency passes while this wavefront waits at the barrier instead of before its loads.
+        uint32_t f_k = step_k[0], r_left = step_m[0] & 127u;
+        auto issue_idx = [&]() -> int {             // index loads of the index stream's next step (+ step-list prefetch)
+            if (f_step >= nsteps) return 0;
+            int ops = 0;
+            const uint32_t k = f_k;
+            uint32_t* dst = idx_ring + (f_step & (kSwIdxSlots - 1)) * (2 * P);
+            if (lw == 0) {
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(sigo_rs, FGX_LDS_PTR(dst), 4, (k + (uint32_t)lane) * 4u, 0, 0, 0);
+                ops = 1;
+                if ((f_step & 63) == 0) {           // the chunk after next; its quarter of the ring was read 128+ steps ago
+                    load_chunk(f_step / 64 + 2);
+                    ops += 2;
+                }
+            } else if (lw == 1) {
+                uint32_t* dst_i = dst + P;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(sigi_rs, FGX_LDS_PTR(dst_i), 4, (k + (uint32_t)lane) * 4u, 0, 0, 0);
+                ops = 1;
+            }
+            ++f_step;
+            f_k = step_k[f_step & (kSwStepRing - 1)];
+            return ops;
+        };
+        bool pr_live = false;
+        unsigned pr_stage = 0;
+        uint32_t va[C::A_PER], vb[C::B_PER];
+        auto prep_rows = [&]() {
+            pr_live = r_step < nsteps;
+            if (!pr_live) return;
+            pr_stage = r_step & (S - 1);
+            const uint32_t* slot_p = idx_ring + (r_step & (kSwIdxSlots - 1)) * (2 * P);
+            const uint32_t left = r_left;                                             // pairs in this step
+            const bool ragged = left < (uint32_t)P || (uint32_t)(BM * ES) > rowb_o || (uint32_t)(BN * ES) > rowb_i;   // uniform
+#pragma unroll
+            for (int i = 0; i < C::A_PER; ++i) va[i] = slot_p[a_row[i]] * rowb_o + a_chb[i];
+#pragma unroll
+            for (int i = 0; i < C::B_PER; ++i) vb[i] = slot_p[P + b_row[i]] * rowb_i + b_chb[i];
+            if (ragged) {
+#pragma unroll
+                for (int i = 0; i < C::A_PER; ++i)
+                    va[i] = ((uint32_t)a_row[i] < left && a_chb[i] < rowb_o) ? va[i] : kOobOffset;
+#pragma unroll
+                for (int i = 0; i < C::B_PER; ++i)
+                    vb[i] = ((uint32_t)b_row[i] < left && b_chb[i] < rowb_i) ? vb[i] : kOobOffset;
+            }
+            ++r_step;
+            r_left = step_m[r_step & (kSwStepRing - 1)] & 127u;
+        };
+        auto fire_rows = [&]() -> int {             // 0 when the stream is over
+            if (!pr_live) return 0;
+            unsigned char* stage = ring + pr_stage * C::STAGE_BYTES;
+#pragma unroll
+            for (int i = 0; i < C::A_PER; ++i) {
+                const uint32_t vo = va[i];
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(gout_rs, FGX_LDS_PTR(stage + (i * C::NL + lw) * 1024), 16, vo, 0, 0, 0);
+            }
+            unsigned char* stage_b = stage + C::A_BYTES;
+#pragma unroll
+            for (int i = 0; i < C::B_PER; ++i) {
+                const uint32_t vo = vb[i];
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(feats_rs, FGX_LDS_PTR(stage_b + (i * C::NL + lw) * 1024), 16, vo, 0, 0, 0);
+            }
+            return C::LPS;
+        };
+        // at most `n` of this loader's loads may be outstanding; n is the sum of the loads of the last two rounds, each
+        // 0 ... LPS + 3 (rounded down to the next value handled here, which is merely stricter)
+        auto wait_loads = [&](int n) {
+            if (n >= 2 * C::LPS + 2) wait_vmcnt<2 * C::LPS + 2>();
+            else if (n == 2 * C::LPS + 1) wait_vmcnt<2 * C::LPS + 1>();
+            else if (n == 2 * C::LPS) wait_vmcnt<2 * C::LPS>();
+            else if (n > C::LPS) wait_vmcnt<C::LPS + 1>();
+            else if (n == C::LPS) wait_vmcnt<C::LPS>();
+            else wait_vmcnt<0>();
+        };
+
+        // prologue: indices of the first kSwIdxAhead steps, then S-1 row rounds
+#pragma unroll
+        for (int j = 0; j < kSwIdxAhead; ++j) (void)issue_idx();
+        wait_vmcnt<0>();
+        __syncthreads();                            // (2)
+        prep_rows();
+        int drained = 0, ops1 = 0, ops2 = 0;        // ops1: loads issued in the previous round, ops2: the one before
+#pragma unroll
+        for (int j = 0; j < S - 1; ++j) {
+            int ops = fire_rows();
+            if (ops == 0) ++drained;
+            prep_rows();                            // indices of steps 1 .. S-1 came with the first batch
+            ops += issue_idx();
+            ops2 = ops1;
+            ops1 = ops;
+        }
+        while (true) {
+            wait_loads(ops1 + ops2);               // everything issued before the last two rounds has landed
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();          // ... everybody's; the stage multiplied in the previous step is free
+            asm volatile("" ::: "memory");
+            int ops = fire_rows();
+            if (ops == 0) ++drained;
+            if (drained >= S - 1) break;           // that was the barrier of the stream's last step
+            prep_rows();
+            ops += issue_idx();
+            ops2 = ops1;
+            ops1 = ops;
+        }
+        wait_vmcnt<0>();
+        return;
+    }
+
+    // =================================================================================================
+    // multipliers
+    // =================================================================================================
+    __syncthreads();                                // (1)
+    __syncthreads();                                // (2) the loaders' prologue barriers
+    const SweepUnit un0 = units[(size_t)gid * 2], un1 = units[(size_t)gid * 2 + 1];
+    const int s16 = lane & 15, mb = (lane >> 4) & 1;
+    int a_off[C::TM][2], b_off[C::TN][2];
+    {
+        const int prow = g * 8 + (s16 >> 2);
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i) {
+            const int byte = (wave_m * C::WM + i * 32 + mb * 16 + (s16 & 3) * 4) * 2;
+            const int c = byte >> 4, w = byte & 15;
+            a_off[i][0] = prow * C::ROWB_A + ((c ^ C::key_a(prow)) << 4) + w;
+            a_off[i][1] = (prow + 4) * C::ROWB_A + ((c ^ C::key_a(prow + 4)) << 4) + w;
+        }
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) {
+            const int byte = (wave_n * C::WN + j * 32 + mb * 16 + (s16 & 3) * 4) * 2;
+            const int c = byte >> 4, w = byte & 15;
+            b_off[j][0] = C::A_BYTES + prow * C::ROWB_B + ((c ^ C::key_b(prow)) << 4) + w;
+            b_off[j][1] = C::A_BYTES + (prow + 4) * C::ROWB_B + ((c ^ C::key_b(prow + 4)) << 4) + w;
+        }
+    }
+    constexpr int NK = P / 16;                      // k-blocks (16 pair rows) per step
+    constexpr int RK = 2 * (C::TM + C::TN);         // LDS reads per k-block
+
+    // `acc` is the accumulator of the unit whose steps are being multiplied, `rest` that of the other one: the two
+    // change places when the step list changes units (a handful of times per sub-block), so that the multiply code
+    // exists once and the register allocator sees one set of MFMA destinations.
+    f32x16 acc[C::TM][C::TN], rest[C::TM][C::TN];
+    float bsum[C::TM];
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                acc[i][j][e] = 0.f;
+                rest[i][j][e] = 0.f;
+            }
+        bsum[i] = 0.f;
+    }
+    unsigned acc_unit = 0;                          // whose sums `acc` holds
+    // Column sums of grad_out (the bias gradient) ride along with the offset whose pairs hold every output row once:
+    // a lane's grad_out fragment is eight pair values of one output channel, which it adds up on the side (a second
+    // accumulator tile of ones-products, as in the block-major kernel, does not fit beside two accumulators).  Both
+    // units of a workgroup add to the same sums; only the wavefronts of the first column of wave tiles do it.
+    const bool bias0 = bias_partial != nullptr && un0.nsteps && (int)un0.v == bias_offset && wave_n == 0;
+    const bool bias1 = bias_partial != nullptr && un1.nsteps && (int)un1.v == bias_offset && wave_n == 0;
+
+    auto multiply_step = [&](const unsigned char* cur, auto with_bias, const bool count_bias) {
+        i16x4 fr[2][RK];
+        auto read_block = [&](int kk, i16x4 (&dst)[RK]) {
+            const unsigned char* base = cur + kk * 16 * C::ROWB_A;
+#pragma unroll
+            for (int i = 0; i < C::TM; ++i) {
+                dst[i * 2] = lds_read_tr16(base + a_off[i][0]);
+                dst[i * 2 + 1] = lds_read_tr16(base + a_off[i][1]);
+            }
+            const unsigned char* base_b = cur + kk * 16 * C::ROWB_B;
+#pragma unroll
+            for (int j = 0; j < C::TN; ++j) {
+                dst[(C::TM + j) * 2] = lds_read_tr16(base_b + b_off[j][0]);
+                dst[(C::TM + j) * 2 + 1] = lds_read_tr16(base_b + b_off[j][1]);
+            }
+        };
+        read_block(0, fr[0]);
+#pragma unroll
+        for (int kk = 0; kk < NK; ++kk) {
+            if (kk + 1 < NK) {
+                read_block(kk + 1, fr[(kk + 1) & 1]);
+                lds_wait_but<RK>(fr[kk & 1]);
+            } else {
+                lds_wait_but<0>(fr[kk & 1]);
+            }
+#pragma unroll
+            for (int i = 0; i < C::TM; ++i) {
+                const i16x8 af = __builtin_shufflevector(fr[kk & 1][i * 2], fr[kk & 1][i * 2 + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                if constexpr (decltype(with_bias)::value) {
+                    const float s8 = sum8<Tag>(af);     // (a select, not a branch: the step stays one basic block)
+                    bsum[i] += count_bias ? s8 : 0.f;
+                }
+#pragma unroll
+                for (int j = 0; j < C::TN; ++j) {
+                    const i16x8 bf = __builtin_shufflevector(fr[kk & 1][(C::TM + j) * 2], fr[kk & 1][(C::TM + j) * 2 + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                    mma16<Tag>(acc[i][j], af, bf);
+                }
+            }
+        }
+    };
+
+    // pacing state of the first multiplier (values in `prog`: sub-block + 1; 0 = not started, all ones = finished)
+    uint32_t cur_sb = step_m[0] >> 8, known_min = 0;
+    bool pacing = mw == 0 && max_polls > 0 && grp.active > 1;
+    if (mw == 0 && lane == 0) __hip_atomic_store(my_prog, cur_sb + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t* xcd_prog = prog + xcd * spx;
+
+    // The step loop in two compiled forms, chosen per workgroup: the one that also adds up the grad_out fragments runs
+    // in the workgroups that hold a unit of the bias offset (a per-step choice between two forms would keep both
+    // forms' address registers alive next to two accumulators).
+    auto run_steps = [&](auto with_bias) {
+        uint32_t next_meta = step_m[0];
+        for (unsigned step = 0; step < nsteps; ++step) {
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();               // the loaders saw this step's rows land
+            asm volatile("" ::: "memory");
+            const unsigned char* cur = ring + (step & (S - 1)) * C::STAGE_BYTES;
+            const uint32_t meta = next_meta;            // (read during the previous step: no LDS round trip after the barrier)
+            const unsigned unit = (meta >> 7) & 1u;
+            if (unit != acc_unit) {
+                acc_unit = unit;
+#pragma unroll
+                for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < C::TN; ++j) swap_tiles(acc[i][j], rest[i][j]);
+            }
+            next_meta = step_m[(step + 1) & (kSwStepRing - 1)];
+            multiply_step(cur, with_bias, unit ? bias1 : bias0);
+            // Pacing, by the first multiplier before it joins the next step's barrier (which holds the whole workgroup
+            // back with it): tell the XCD which sub-block this workgroup is entering, and do not enter one more than
+            // `lead` ahead of the slowest workgroup.  Bounded: after max_polls looks the workgroup stops pacing.
+            if (mw == 0 && step + 1 < nsteps) {
+                const uint32_t next_sb = next_meta >> 8;
+                if (next_sb != cur_sb) {
+                    cur_sb = next_sb;
+                    if (lane == 0) __hip_atomic_store(my_prog, cur_sb + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (pacing && cur_sb > known_min + lead) {
+                        unsigned polls = 0;
+                        while (true) {
+                            uint32_t seen = 0xFFFFFFFFu;
+                            if ((unsigned)lane < spx) seen = __hip_atomic_load(xcd_prog + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                            for (int sh = 32; sh > 0; sh >>= 1) {
+                                const uint32_t o = (uint32_t)__shfl_xor((int)seen, sh, 64);
+                                seen = o < seen ? o : seen;
+                            }
+                            known_min = seen ? seen - 1u : 0u;
+                            if (cur_sb <= known_min + lead) break;
+                            if (++polls >= max_polls) {
+                                pacing = false;         // give up for good: the kernel must end whatever the others do
+                                break;
+                            }
+                            __builtin_amdgcn_s_sleep(32);
+                        }
+                    }
+                }
+            }
+        }
+    };
+    if (bias0 || bias1) run_steps(std::true_type{});
+    else run_steps(std::false_type{});
+    if (mw == 0 && lane == 0) __hip_atomic_store(my_prog, 0xFFFFFFFFu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+    // partial[unit][co][ci], fp32
+    auto store_acc = [&](f32x16 (&a)[C::TM][C::TN], unsigned q) {
+        float* dst = partial + (size_t)q * ((size_t)Co * Ci);
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) {
+            const int ci = wave_n * C::WN + j * 32 + l32;
+            if (ci >= Ci) continue;
+#pragma unroll
+            for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int co = wave_m * C::WM + i * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
+                    if (co < Co) dst[(size_t)co * Ci + ci] = a[i][j][e];
+                }
+        }
+    };
+    if (acc_unit == 0) {
+        if (un0.nsteps) store_acc(acc, gid * 2);
+        if (un1.nsteps) store_acc(rest, gid * 2 + 1);
+    } else {
+        if (un0.nsteps) store_acc(rest, gid * 2);
+        if (un1.nsteps) store_acc(acc, gid * 2 + 1);
+    }
+    if (bias0 || bias1) {                           // bias_partial[workgroup][co]; the two wave halves hold half the pairs each
+        float* bdst = bias_partial + (size_t)gid * Co;
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i) {
+            const float both = bsum[i] + __shfl_xor(bsum[i], 32, 64);
+            const int co = wave_m * C::WM + i * 32 + l32;
+            if (g == 0 && co < Co) bdst[co] = both;
+        }
+    }
+}
+
+// grad_weight[co][v][ci] = sum of the partial products of offset v's units, in ascending unit order.  One thread per
+// four adjacent ci; eight loads in flight.
+template <typename T>
+__global__ void __launch_bounds__(256) sweep_reduce_kernel(const float* __restrict__ partial,
+                                                           const uint32_t* __restrict__ vcount,
+                                                           const uint16_t* __restrict__ vlist, unsigned total_units, int V,
+                                                           int Ci, int Co, T* __restrict__ gw) {
+    const size_t quads = (size_t)Co * V * (Ci / 4);
+    const size_t per = (size_t)Co * Ci;
+    for (size_t t = (size_t)blockIdx.x * 256 + threadIdx.x; t < quads; t += (size_t)gridDim.x * 256) {
+        const int cq = (int)(t % (Ci / 4));
+        const size_t r = t / (Ci / 4);
+        const int v = (int)(r % V), co = (int)(r / V);
+        const unsigned cnt = vcount[v];
+        const uint16_t* list = vlist + (size_t)v * total_units;
+        const float* src = partial + (size_t)co * Ci + cq * 4;
+        float4 s = {0.f, 0.f, 0.f, 0.f};
+        unsigned i = 0;
+        for (; i + 8 <= cnt; i += 8) {
+            float4 x[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) x[q] = *(const float4*)(src + (size_t)list[i + q] * per);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                s.x += x[q].x;
+                s.y += x[q].y;
+                s.z += x[q].z;
+                s.w += x[q].w;
+            }
+        }
+        for (; i < cnt; ++i) {
+            const float4 x = *(const float4*)(src + (size_t)list[i] * per);
+            s.x += x.x;
+            s.y += x.y;
+            s.z += x.z;
+            s.w += x.w;
+        }
+        T* dst = gw + ((size_t)co * V + v) * Ci + cq * 4;
+        dst[0] = from_float<T>(s.x);
+        dst[1] = from_float<T>(s.y);
+        dst[2] = from_float<T>(s.z);
+        dst[3] = from_float<T>(s.w);
+    }
+}
+
+// grad_bias[co] = sum over the workgroups that held a unit of the bias offset.  One block per column, one thread per
+// workgroup, then a tree over LDS: a fixed order of additions.
+template <typename T>
+__global__ void __launch_bounds__(kSwMaxGroups) sweep_bias_reduce_kernel(const float* __restrict__ bias_partial,
+                                                                         const SweepUnit* __restrict__ units, unsigned groups,
+                                                                         int bias_offset, int Co, T* __restrict__ out) {
+    __shared__ float sums[kSwMaxGroups];
+    const int co = blockIdx.x;
+    const unsigned gidx = threadIdx.x;
+    float s = 0.f;
+    if (gidx < groups) {
+        const SweepUnit a = units[(size_t)gidx * 2], b = units[(size_t)gidx * 2 + 1];
+        const bool has = (a.nsteps && (int)a.v == bias_offset) || (b.nsteps && (int)b.v == bias_offset);
+        if (has) s = bias_partial[(size_t)gidx * Co + co];
+    }
+    sums[gidx] = s;
+    __syncthreads();
+    for (unsigned half = kSwMaxGroups / 2; half > 0; half >>= 1) {
+        if (gidx < half) sums[gidx] += sums[gidx + half];
+        __syncthreads();
+    }
+    if (gidx == 0) out[co] = from_float<T>(sums[0]);
+}
+
+struct SweepScratch {
+    size_t prog, partial, bias, colsum, total;
+};
+SweepScratch sweep_scratch(int Ci, int Co, int groups) {
+    SweepScratch S{};
+    size_t off = 0;
+    S.prog = off;
+    off = align_up(off + (size_t)groups * 4, 256);
+    S.partial = off;
+    off = align_up(off + (size_t)groups * 2 * Co * Ci * sizeof(float), 256);
+    S.bias = off;
+    off = align_up(off + (size_t)groups * Co * sizeof(float), 256);
+    S.colsum = off;
+    off += fgx_colsum_scratch_bytes(0, Co);
+    S.total = off;
+    return S;
+}
+
+int sweep_groups() {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    int g = cus / kXcds * kXcds;
+    if (g > kSwMaxGroups) g = kSwMaxGroups;
+    return g;
+}
+
+bool tile_ok(int tile, int Ci, int Co) { return (tile == 128 || tile == 64) && Ci <= tile && Co <= tile; }
+
+template <typename Tag, int BM, int BN>
+int launch_sweep(const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o, const char* plan,
+                 const SweepLayout& L, size_t n, size_t n_in, uint32_t n_pairs, int V, int Ci, int Co, char* scratch,
+                 const SweepScratch& S, void* gw, void* gbias, int bias_offset, int lead, int max_polls, hipStream_t s) {
+    using C = SweepCfg<Tag, BM, BN>;
+    using T = typename Tag::type;
+    auto kern = wgrad_sweep_kernel<Tag, BM, BN>;
+    static thread_local bool lds_raised = false;
+    if (C::lds_bytes > 64 * 1024 && !lds_raised) {
+        FGX_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::lds_bytes));
+        lds_raised = true;
+    }
+    uint32_t* prog = (uint32_t*)(scratch + S.prog);
+    float* partial = (float*)(scratch + S.partial);
+    float* bias_partial = gbias ? (float*)(scratch + S.bias) : nullptr;
+    const SweepUnit* units = (const SweepUnit*)(plan + L.units);
+    sweep_clear_kernel<<<cdiv(L.groups, 256), 256, 0, s>>>(prog, L.groups);
+    FGX_CHECK_LAUNCH("fgx_conv_wgrad_sweep(clear)");
+    kern<<<L.groups, C::NT, C::lds_bytes, s>>>((const T*)gout, (const T*)feats, sig_i, sig_o, units,
+                                               (const SweepGroup*)(plan + L.wg), (const uint32_t*)(plan + L.steps_k),
+                                               (const uint32_t*)(plan + L.steps_m), L.spx, V, Ci, Co, n_pairs,
+                                               (uint32_t)(n * (size_t)Co * sizeof(T)), (uint32_t)(n_in * (size_t)Ci * sizeof(T)),
+                                               partial, bias_partial, bias_offset, prog, (unsigned)lead, (unsigned)max_polls);
+    FGX_CHECK_LAUNCH("fgx_conv_wgrad_sweep");
+    const size_t quads = (size_t)Co * V * (Ci / 4);
+    unsigned grid = cdiv(quads, 256);
+    sweep_reduce_kernel<T><<<grid, 256, 0, s>>>(partial, (const uint32_t*)(plan + L.vcount), (const uint16_t*)(plan + L.vlist),
+                                                L.groups * 2, V, Ci, Co, (T*)gw);
+    FGX_CHECK_LAUNCH("fgx_conv_wgrad_sweep(reduce)");
+    if (bias_partial) {
+        sweep_bias_reduce_kernel<T><<<(unsigned)Co, kSwMaxGroups, 0, s>>>(bias_partial, units, L.groups, bias_offset, Co, (T*)gbias);
+        FGX_CHECK_LAUNCH("fgx_conv_wgrad_sweep(bias reduce)");
+    }
+    return FGX_OK;
+}
+
+}  // namespace
+}  // namespace fgx
+
+using namespace fgx;
+
+extern "C" {
+
+size_t fgx_wgrad_sweep_plan_bytes(size_t n, size_t n_pairs, int V, int sub_rows) {
+    const int groups = sweep_groups();
+    if (V < 1 || V > kMaxV || sub_rows < 1 || groups < kXcds) return 0;
+    return sweep_layout(n, n_pairs, V, sub_rows, groups).total;
+}
+
+int fgx_wgrad_sweep_plan(const uint32_t* sig_o, const uint32_t* seg_host, size_t n, int V, int sub_rows, void* plan,
+                         size_t plan_bytes, fgx_stream_t stream) {
+    FGX_CHECK_ARG(V >= 1 && V <= kMaxV, "fgx_wgrad_sweep_plan: bad kernel volume %d", V);
+    FGX_CHECK_ARG(sub_rows >= 64, "fgx_wgrad_sweep_plan: sub_rows must be at least 64, got %d", sub_rows);
+    FGX_CHECK_ARG(seg_host && plan, "fgx_wgrad_sweep_plan: null buffer");
+    FGX_CHECK_ARG(n > 0 && n < 0xFFFFFFFFull, "fgx_wgrad_sweep_plan: row count out of range");
+    FGX_CHECK_ARG(((uintptr_t)plan & 255) == 0, "fgx_wgrad_sweep_plan: plan must be 256-byte aligned");
+    SegTable tab;
+    for (int v = 0; v <= V; ++v) {
+        FGX_CHECK_ARG(v == 0 || seg_host[v] >= seg_host[v - 1], "fgx_wgrad_sweep_plan: segment table is not monotone");
+        tab.seg[v] = seg_host[v];
+    }
+    for (int v = V + 1; v <= kMaxV; ++v) tab.seg[v] = seg_host[V];
+    const size_t n_pairs = seg_host[V];
+    FGX_CHECK_ARG(n_pairs == seg_host[0] || sig_o != nullptr, "fgx_wgrad_sweep_plan: null pair list");
+    FGX_CHECK_ARG(seg_host[0] == 0, "fgx_wgrad_sweep_plan: the segment table must start at 0");
+    const int groups = sweep_groups();
+    FGX_CHECK_ARG(groups >= kXcds && groups / kXcds * 2 >= V, "fgx_wgrad_sweep_plan: too few compute units for %d offsets", V);
+    const SweepLayout L = sweep_layout(n, n_pairs, V, sub_rows, groups);
+    FGX_CHECK_ARG((size_t)L.nsb + 1 < (1u << 24), "fgx_wgrad_sweep_plan: too many sub-blocks; use larger sub_rows");
+    FGX_CHECK_ARG(plan_bytes >= L.total, "fgx_wgrad_sweep_plan: plan of %zu bytes, need %zu", plan_bytes, L.total);
+    hipStream_t s = (hipStream_t)stream;
+    char* p = (char*)plan;
+    uint32_t* fine = (uint32_t*)(p + L.fine);
+    PhaseEnd phases{s};
+    phase_mark("wgrad sweep plan", s);
+    block_bounds_kernel<<<cdiv((size_t)V * (L.nsb + 1), 256), 256, 0, s>>>(sig_o, tab, V, L.nsb, (unsigned)sub_rows, fine);
+    FGX_CHECK_LAUNCH("fgx_wgrad_sweep_plan(bounds)");
+    sweep_units_kernel<<<1, 64, 0, s>>>(fine, V, L.nsb, L.spx, (SweepUnit*)(p + L.units), (SweepGroup*)(p + L.wg),
+                                        (uint32_t*)(p + L.vcount), (uint16_t*)(p + L.vlist));
+    FGX_CHECK_LAUNCH("fgx_wgrad_sweep_plan(units)");
+    sweep_steps_kernel<<<L.groups, 256, 0, s>>>(fine, L.nsb, (const SweepUnit*)(p + L.units), (const SweepGroup*)(p + L.wg),
+                                                (uint32_t*)(p + L.steps_k), (uint32_t*)(p + L.steps_m), L.step_cap);
+    FGX_CHECK_LAUNCH("fgx_wgrad_sweep_plan(steps)");
+    return FGX_OK;
+}
+
+size_t fgx_wgrad_sweep_scratch_bytes(int Ci, int Co) {
+    const int groups = sweep_groups();
+    if (Ci <= 0 || Co <= 0 || groups < kXcds) return 0;
+    return sweep_scratch(Ci, Co, groups).total;
+}
+
+int fgx_conv_wgrad_sweep(int dtype, const void* grad_out, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
+                         const uint32_t* seg_host, const void* plan, size_t n, size_t n_in, int Ci, int Co, int V, int tile,
+                         int sub_rows, int lead, int max_polls, void* scratch, void* grad_weight, void* grad_bias,
+                         int bias_offset, fgx_stream_t stream) {
+    FGX_CHECK_ARG(dtype == FGX_F16 || dtype == FGX_BF16, "fgx_conv_wgrad_sweep: 16-bit types only (dtype %d)", dtype);
+    FGX_CHECK_ARG(Ci > 0 && Co > 0 && V >= 1 && V <= kMaxV, "fgx_conv_wgrad_sweep: bad shape Ci=%d Co=%d V=%d", Ci, Co, V);
+    FGX_CHECK_ARG(tile_ok(tile, Ci, Co), "fgx_conv_wgrad_sweep: a single %dx%d tile does not hold Co=%d x Ci=%d", tile, tile, Co, Ci);
+    FGX_CHECK_ARG(Ci % 8 == 0 && Co % 8 == 0, "fgx_conv_wgrad_sweep: rows of %d / %d elements are not multiples of 16 bytes", Ci, Co);
+    FGX_CHECK_ARG(sub_rows >= 64 && lead >= 0 && max_polls >= 0, "fgx_conv_wgrad_sweep: bad pacing arguments");
+    FGX_CHECK_ARG(seg_host && plan && scratch && grad_weight, "fgx_conv_wgrad_sweep: null buffer");
+    FGX_CHECK_ARG(n > 0 && n < 0xFFFFFFFFull && n_in < 0xFFFFFFFFull, "fgx_conv_wgrad_sweep: row count out of range");
+    FGX_CHECK_ARG(((uintptr_t)scratch & 255) == 0 && ((uintptr_t)plan & 255) == 0, "fgx_conv_wgrad_sweep: scratch and plan must be 256-byte aligned");
+    const size_t n_pairs = seg_host[V];
+    FGX_CHECK_ARG(n_pairs > 0 && grad_out && feats && sig_i && sig_o, "fgx_conv_wgrad_sweep: empty pair lists or null buffer");
+    FGX_CHECK_ARG((((uintptr_t)grad_out | (uintptr_t)feats) & 15) == 0, "fgx_conv_wgrad_sweep: grad_out and feats must be 16-byte aligned");
+    FGX_CHECK_ARG((double)n * Co * 2 <= (double)kOobOffset && (double)n_in * Ci * 2 <= (double)kOobOffset &&
+                      (double)n_pairs * 4 + 256 <= (double)kOobOffset,
+                  "fgx_conv_wgrad_sweep: an operand exceeds the 32-bit offset range; use fgx_conv_wgrad");
+    const int groups = sweep_groups();
+    FGX_CHECK_ARG(groups >= kXcds && groups / kXcds * 2 >= V, "fgx_conv_wgrad_sweep: too few compute units for %d offsets", V);
+    const SweepLayout L = sweep_layout(n, n_pairs, V, sub_rows, groups);
+    const SweepScratch S = sweep_scratch(Ci, Co, groups);
+    hipStream_t s = (hipStream_t)stream;
+    void* fused_bias = nullptr;
+    if (grad_bias != nullptr) {
+        const bool fuse = bias_offset >= 0 && bias_offset < V && (size_t)(seg_host[bias_offset + 1] - seg_host[bias_offset]) == n;
+        if (fuse) fused_bias = grad_bias;
+        else {
+            int rc = fgx_colsum(dtype, grad_out, n, Co, (char*)scratch + S.colsum, grad_bias, stream);
+            if (rc != FGX_OK) return rc;
+        }
+    }
+#define FGX_SWEEP(TAG, T_)                                                                                                      \
+    if (tile == T_)                                                                                                             \
+        return launch_sweep<TAG, T_, T_>(grad_out, feats, sig_i, sig_o, (const char*)plan, L, n, n_in, (uint32_t)n_pairs, V, Ci, Co, \
+                                         (char*)scratch, S, grad_weight, fused_bias, bias_offset, lead, max_polls, s);
+    if (dtype == FGX_F16) { FGX_SWEEP(F16, 128) FGX_SWEEP(F16, 64) }
+    else { FGX_SWEEP(BF16, 128) FGX_SWEEP(BF16, 64) }
+#undef FGX_SWEEP
+    set_error("fgx_conv_wgrad_sweep: no kernel for tile %d", tile);
+    return FGX_ERR_UNSUPPORTED;
+}
+
+}  // extern "C"

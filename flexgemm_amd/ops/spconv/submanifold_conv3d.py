@@ -232,6 +232,23 @@ class SubMConv3dNeighborCache:
             setattr(self, key, bounds)
         return getattr(self, key)
 
+    def _wgrad_sweep_plan(self, sub_rows: int):
+        """Step lists of the paced wgrad sweep (fgx_wgrad_sweep_plan): a function of the pair lists and the sub-block
+        size alone, made once and kept."""
+        key = f"_wgrad_sweep_plan_{sub_rows}"
+        if not hasattr(self, key):
+            sig_o = self["valid_signal_o"]
+            n, v = self["neighbor_map"].shape
+            seg_host = self._seg_host()
+            L = nat.lib()
+            with torch.cuda.device(sig_o.device):
+                nbytes = L.fgx_wgrad_sweep_plan_bytes(nat.sz(n), nat.sz(seg_host[-1]), C.c_int(v), C.c_int(sub_rows))
+                plan = nat.workspace(nbytes, sig_o.device)
+                nat.check(L.fgx_wgrad_sweep_plan(nat.ptr(sig_o), (C.c_uint32 * (v + 1))(*seg_host), nat.sz(n), C.c_int(v),
+                                                 C.c_int(sub_rows), nat.ptr(plan), nat.sz(plan.numel()), nat.stream()))
+            setattr(self, key, plan)
+        return getattr(self, key)
+
     def _seg_host(self):
         if not hasattr(self, "_valid_signal_seg_host"):
             seg = self["valid_signal_seg"]
@@ -491,6 +508,12 @@ def _stream_fits(n: int, n_src: int, row_bytes: int) -> bool:
     return n_src * row_bytes <= 0xFF000000 and n * 8 <= 0xFF000000 and n * 27 * 4 * 2 <= 0xFF000000
 
 
+# pacing of the wgrad sweep: sub-blocks a workgroup may run ahead of the slowest one of its XCD, and the looks at the
+# others' progress after which it stops waiting (0 = no pacing)
+WGRAD_SWEEP_LEAD = 3
+WGRAD_SWEEP_MAX_POLLS = 2000
+
+
 def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int, with_bias: bool = False, bias_offset: int = -1):
     """[Co, V, Ci] weight gradient from the pair lists of cache["neighbor_map"]: grad_output has one row per row of
     that map, feats one per row the map points at.  with_bias: also the bias gradient (column sums of grad_output),
@@ -514,6 +537,21 @@ def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int, with_b
     gb = torch.empty((cop,), dtype=dt, device=dev) if with_bias else None
     L = nat.lib()
     code = nat.DTYPE_CODE[dt]
+    if sched.stream == 2 and seg_host[-1] > 0 and n > 0:
+        plan = cache._wgrad_sweep_plan(sched.block_rows)
+        with torch.cuda.device(dev):
+            scratch = nat.workspace(L.fgx_wgrad_sweep_scratch_bytes(C.c_int(cip), C.c_int(cop)), dev)
+            nat.mark("wgrad", "start")
+            nat.check(L.fgx_conv_wgrad_sweep(
+                C.c_int(code), nat.ptr(g), nat.ptr(f), nat.ptr(cache["valid_signal_i"]), nat.ptr(cache["valid_signal_o"]),
+                seg_arr, nat.ptr(plan), nat.sz(n), nat.sz(n_in), C.c_int(cip), C.c_int(cop), C.c_int(v), C.c_int(sched.tile_rows),
+                C.c_int(sched.block_rows), C.c_int(WGRAD_SWEEP_LEAD), C.c_int(WGRAD_SWEEP_MAX_POLLS), nat.ptr(scratch), nat.ptr(gw),
+                nat.ptr(gb), C.c_int(bias_offset), nat.stream()))
+            nat.mark("wgrad", "stop")
+        if cip != ci or cop != co:
+            gw = gw[:co, :, :ci].contiguous()
+            gb = gb[:co].contiguous() if with_bias else None
+        return (gw, gb) if with_bias else gw
     bounds = cache._wgrad_bounds(sched.block_rows)
     with torch.cuda.device(dev):
         scratch = nat.workspace(L.fgx_wgrad_scratch_bytes(nat.sz(n), C.c_int(v), C.c_int(cip), C.c_int(cop),

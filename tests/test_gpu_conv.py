@@ -417,6 +417,50 @@ def test_streaming_wgrad_matches_oracle(gpu_device, dtype, res, ci, co, tile, bl
         _run_and_check(coords_np, shape, ci, co, dtype, gpu_device, seed=23)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("res,ci,co,tile,sub_rows,lead,max_polls", [
+    (32, 128, 128, 128, 256, 3, 2000), (48, 128, 128, 128, 128, 1, 2000), (24, 64, 64, 64, 64, 3, 2000),
+    (32, 96, 40, 128, 512, 0, 3), (40, 48, 64, 64, 100000, 3, 2000), (64, 128, 128, 128, 1024, 2, 0),
+    (16, 128, 64, 128, 64, 3, 2000)])
+def test_sweep_wgrad_matches_oracle(gpu_device, dtype, res, ci, co, tile, sub_rows, lead, max_polls):
+    """wgrad as the paced sweep, forced on small shells: sub-blocks far smaller than in production (most parts a step or
+    two long, ragged steps everywhere), one sub-block for everything, channel counts below the tile, pacing with no
+    lead and a poll limit that runs out (the workgroups then go on unpaced), and pacing switched off."""
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    _say(f"sweep wgrad res={res} ci={ci} co={co} tile={tile} sub_rows={sub_rows} lead={lead} polls={max_polls} {dtype}")
+    coords_np = reference_test_shell(res)
+    shape = torch.Size([1, ci, res, res, res])
+    old = impl.WGRAD_SWEEP_LEAD, impl.WGRAD_SWEEP_MAX_POLLS
+    impl.WGRAD_SWEEP_LEAD, impl.WGRAD_SWEEP_MAX_POLLS = lead, max_polls
+    try:
+        with _force_schedule(wgrad=True, tile_rows=tile, tile_cols=tile, block_rows=sub_rows, stream=2):
+            cache, _ = _run_and_check(coords_np, shape, ci, co, dtype, gpu_device, seed=31)
+        assert any(k.startswith("_wgrad_sweep_plan_") for k in vars(cache))
+    finally:
+        impl.WGRAD_SWEEP_LEAD, impl.WGRAD_SWEEP_MAX_POLLS = old
+
+
+def test_sweep_wgrad_is_reproducible_and_close_to_the_block_major_kernel(gpu_device):
+    """Two runs of the sweep give the same bits (fixed summation order); against the block-major streaming kernel the
+    difference is fp32 rounding of a different order of additions."""
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    _say("sweep wgrad vs streaming wgrad")
+    res, c = 64, 128
+    coords_np = reference_test_shell(res)
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    shape = torch.Size([1, c, res, res, res])
+    f, _, _, g = _case(coords_np, c, c, torch.float16, 35)
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+    outs = []
+    for stream, rows in ((2, 512), (2, 512), (1, 4096)):
+        with _force_schedule(wgrad=True, tile_rows=128, tile_cols=128, block_rows=rows, stream=stream):
+            gw, gb = impl._wgrad(g.to(gpu_device), f.to(gpu_device), cache, 27, with_bias=True, bias_offset=13)
+            outs.append((gw.cpu(), gb.cpu()))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    assert eg.max_rel_err(outs[0][0], outs[2][0].double()) <= 2e-3
+    assert eg.max_rel_err(outs[0][1], outs[2][1].double()) <= 2e-3
+
+
 def test_streaming_wgrad_equals_tiled_wgrad_bitwise(gpu_device):
     """Same 16-pair MFMA blocks in the same order inside every (voxel block, offset) item, same block-ordered
     reduction: the two wgrad kernels agree bit for bit."""
