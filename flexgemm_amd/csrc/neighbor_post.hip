@@ -14,6 +14,7 @@
 #include <rocprim/rocprim.hpp>
 
 #include "fgx_common.h"
+#include "radix_sort.h"
 
 namespace fgx {
 namespace {
@@ -87,6 +88,12 @@ int bits_for(size_t x) {   // smallest b with 2^b > x
     while (b < 63 && ((size_t)1 << b) <= x) ++b;
     return b;
 }
+
+
+// The mask sort: between these sizes the radix sort of radix_sort.h is ahead of the library's (measured, 27-bit keys:
+// 0.095 against 0.154 ms at 669 288 items; 0.077 against 0.068 ms at 166 232, where the library sorts blocks and merges
+// them; 0.189 against 0.182 ms at 2 667 120, where it runs onesweep passes with tiles sorted in LDS first).
+constexpr size_t kOwnSortMin = 393216, kOwnSortMax = 2097152;
 
 struct SortLayout {
     size_t keys_out, vals_in, vals_out, temp, temp_bytes, total;
@@ -475,29 +482,39 @@ using namespace fgx;
 
 extern "C" {
 
-size_t fgx_sort_workspace_bytes(size_t n) { return sort_layout(n).total; }
+size_t fgx_sort_workspace_bytes(size_t n) {
+    return n >= kOwnSortMin && n <= kOwnSortMax ? radix_layout(n).total : sort_layout(n).total;
+}
 
 int fgx_sort_by_code(const int32_t* binary, size_t n, int V, int64_t* sorted_idx, void* workspace,
                      size_t workspace_bytes, fgx_stream_t stream) {
     FGX_CHECK_ARG(V >= 1 && V <= 32, "fgx_sort_by_code: kernel volume must be in [1, 32], got %d", V);
     FGX_CHECK_ARG(n < 0xFFFFFFFFull, "fgx_sort_by_code: too many rows");
     if (n == 0) return FGX_OK;
-    SortLayout L = sort_layout(n);
+    const bool own = n >= kOwnSortMin && n <= kOwnSortMax;
+    const size_t need = fgx_sort_workspace_bytes(n);
     FGX_CHECK_ARG(binary && sorted_idx && workspace, "fgx_sort_by_code: null buffer");
-    FGX_CHECK_ARG(workspace_bytes >= L.total, "fgx_sort_by_code: workspace of %zu bytes, need %zu", workspace_bytes, L.total);
+    FGX_CHECK_ARG(workspace_bytes >= need, "fgx_sort_by_code: workspace of %zu bytes, need %zu", workspace_bytes, need);
     FGX_CHECK_ARG(((uintptr_t)workspace & 255) == 0, "fgx_sort_by_code: workspace must be 256-byte aligned");
     hipStream_t s = (hipStream_t)stream;
     char* ws = (char*)workspace;
+    PhaseEnd phases{s};
+    phase_mark("mask sort", s);
+    // With V < 32 every key is non-negative and only bits [0, V) can differ.
+    const unsigned end_bit = V < 32 ? (unsigned)V : 32u;
+    if (own && V < 32) {
+        // (as unsigned numbers the keys then order like the int32 codes); the first pass numbers the rows itself and the
+        // last one writes the 64-bit indices
+        return radix_sort_pairs_u32((const uint32_t*)binary, nullptr, n, end_bit, ws, radix_layout(n), nullptr, nullptr, sorted_idx, s,
+                                    "fgx_sort_by_code");
+    }
+    const SortLayout L = sort_layout(n);
     int32_t* keys_out = (int32_t*)(ws + L.keys_out);
     uint32_t* vals_in = (uint32_t*)(ws + L.vals_in);
     uint32_t* vals_out = (uint32_t*)(ws + L.vals_out);
-    PhaseEnd phases{s};
-    phase_mark("mask sort", s);
     iota_u32_kernel<<<cdiv(n, kBlock), kBlock, 0, s>>>(vals_in, n);
     FGX_CHECK_LAUNCH("fgx_sort_by_code(iota)");
     size_t temp_bytes = L.temp_bytes;
-    // With V < 32 every key is non-negative and only bits [0, V) can differ.
-    unsigned end_bit = V < 32 ? (unsigned)V : 32u;
     FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp_bytes, binary, keys_out, vals_in, vals_out, n, 0u, end_bit, s));
     widen_u32_i64_kernel<<<cdiv(n, kBlock), kBlock, 0, s>>>(vals_out, sorted_idx, n);
     FGX_CHECK_LAUNCH("fgx_sort_by_code(widen)");

@@ -44,6 +44,17 @@ __global__ void __launch_bounds__(256) flat_keys_kernel(const int32_t* __restric
     rows[i] = (uint32_t)i;
 }
 
+// descents[0] = 1 when some voxel's flattened key is smaller than its predecessor's (the caller clears the word first)
+__global__ void __launch_bounds__(256) key_order_kernel(const int32_t* __restrict__ coords, size_t n, int W, int H, int D,
+                                                        uint32_t* __restrict__ descents) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i == 0 || i >= n) return;
+    const int4 a = reinterpret_cast<const int4*>(coords)[i - 1], c = reinterpret_cast<const int4*>(coords)[i];
+    const uint64_t ka = (((uint64_t)(uint32_t)a.x * (uint64_t)W + (uint64_t)a.y) * (uint64_t)H + (uint64_t)a.z) * (uint64_t)D + (uint64_t)a.w;
+    const uint64_t kc = (((uint64_t)(uint32_t)c.x * (uint64_t)W + (uint64_t)c.y) * (uint64_t)H + (uint64_t)c.z) * (uint64_t)D + (uint64_t)c.w;
+    if (kc < ka) descents[0] = 1u;      // (every writer stores the same value)
+}
+
 // first position in a[lo, hi) whose key is >= t (hi if none)
 template <typename K>
 __device__ __forceinline__ size_t lower_bound_at(const K* a, size_t lo, size_t hi, K t) {
@@ -316,21 +327,27 @@ unsigned bit_length(uint64_t x) {
 }
 
 template <typename K>
-int build_sorted(const int32_t* coords, size_t n, uint64_t vol, const SubmGeom& g, char* ws, const SortedLayout& L,
+int build_sorted(const int32_t* coords, size_t n, uint64_t vol, const SubmGeom& g, bool presorted, char* ws, const SortedLayout& L,
                  uint32_t* out_map, int32_t* gray, int32_t* binary, hipStream_t s) {
     K* keys_in = (K*)(ws + L.keys_in);
     K* keys_out = (K*)(ws + L.keys_out);
     uint32_t* rows_in = (uint32_t*)(ws + L.rows_in);
     uint32_t* rows_out = (uint32_t*)(ws + L.rows_out);
     PhaseEnd phases{s};
-    phase_mark("key sort", s);
-    flat_keys_kernel<K><<<cdiv(n, 256), 256, 0, s>>>(coords, n, g.W, g.H, g.D, keys_in, rows_in);
-    FGX_CHECK_LAUNCH("fgx_subm_neighbor_map_sorted(keys)");
-    size_t temp_bytes = L.temp_bytes;
-    unsigned end_bit = bit_length(vol - 1);
-    if (end_bit == 0) end_bit = 1;
-    FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp_bytes, (const K*)keys_in, keys_out, (const uint32_t*)rows_in, rows_out,
-                                            n, 0u, end_bit, s));
+    if (presorted) {        // keys ascend as the voxels come: the sorted arrays are the keys and 0, 1, 2, ... themselves
+        phase_mark("keys", s);
+        flat_keys_kernel<K><<<cdiv(n, 256), 256, 0, s>>>(coords, n, g.W, g.H, g.D, keys_out, rows_out);
+        FGX_CHECK_LAUNCH("fgx_subm_neighbor_map_sorted(keys)");
+    } else {
+        phase_mark("key sort", s);
+        flat_keys_kernel<K><<<cdiv(n, 256), 256, 0, s>>>(coords, n, g.W, g.H, g.D, keys_in, rows_in);
+        FGX_CHECK_LAUNCH("fgx_subm_neighbor_map_sorted(keys)");
+        size_t temp_bytes = L.temp_bytes;
+        unsigned end_bit = bit_length(vol - 1);
+        if (end_bit == 0) end_bit = 1;
+        FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp_bytes, (const K*)keys_in, keys_out, (const uint32_t*)rows_in, rows_out,
+                                                n, 0u, end_bit, s));
+    }
     const unsigned groups = cdiv(n, kGroup);
     uint32_t* bounds = (uint32_t*)(ws + L.bounds);
     phase_mark("window bounds", s);
@@ -598,9 +615,22 @@ size_t fgx_subm_neighbor_map_sorted_workspace_bytes(size_t n, int key_bits, int 
     return sorted_layout(n, key_bits, Kw * Kh).total;
 }
 
+int fgx_coords_key_order(const int32_t* coords, size_t n, int W, int H, int D, uint32_t* descents, fgx_stream_t stream) {
+    FGX_CHECK_ARG(W > 0 && H > 0 && D > 0, "fgx_coords_key_order: grid extents must be positive");
+    FGX_CHECK_ARG(descents != nullptr && (n == 0 || coords != nullptr), "fgx_coords_key_order: null buffer");
+    FGX_CHECK_ARG(((uintptr_t)coords & 15) == 0, "fgx_coords_key_order: coords must be 16-byte aligned");
+    if (n < 2) return FGX_OK;
+    hipStream_t s = (hipStream_t)stream;
+    PhaseEnd phases{s};
+    phase_mark("key order check", s);
+    key_order_kernel<<<cdiv(n, 256), 256, 0, s>>>(coords, n, W, H, D, descents);
+    FGX_CHECK_LAUNCH("fgx_coords_key_order");
+    return FGX_OK;
+}
+
 int fgx_subm_neighbor_map_sorted(const int32_t* coords, size_t n, int B, int W, int H, int D, int Kw, int Kh, int Kd, int Dw,
-                                 int Dh, int Dd, int key_bits, void* workspace, size_t workspace_bytes, uint32_t* out_map,
-                                 int32_t* gray, int32_t* binary, fgx_stream_t stream) {
+                                 int Dh, int Dd, int key_bits, int presorted, void* workspace, size_t workspace_bytes,
+                                 uint32_t* out_map, int32_t* gray, int32_t* binary, fgx_stream_t stream) {
     FGX_CHECK_ARG(key_bits == 32 || key_bits == 64, "fgx_subm_neighbor_map_sorted: key_bits must be 32 or 64, got %d", key_bits);
     FGX_CHECK_ARG(Kw > 0 && Kh > 0 && Kd > 0 && (Kw & 1) && (Kh & 1) && (Kd & 1),
                   "fgx_subm_neighbor_map_sorted: kernel sizes must be odd and positive, got (%d,%d,%d)", Kw, Kh, Kd);
@@ -624,8 +654,8 @@ int fgx_subm_neighbor_map_sorted(const int32_t* coords, size_t n, int B, int W, 
     SubmGeom g{W, H, D, Kw, Kh, Kd, V, Dw, Dh, Dd};
     hipStream_t s = (hipStream_t)stream;
     char* ws = (char*)workspace;
-    return key_bits == 32 ? build_sorted<uint32_t>(coords, n, vol, g, ws, L, out_map, gray, binary, s)
-                          : build_sorted<uint64_t>(coords, n, vol, g, ws, L, out_map, gray, binary, s);
+    return key_bits == 32 ? build_sorted<uint32_t>(coords, n, vol, g, presorted != 0, ws, L, out_map, gray, binary, s)
+                          : build_sorted<uint64_t>(coords, n, vol, g, presorted != 0, ws, L, out_map, gray, binary, s);
 }
 
 size_t fgx_spconv_neighbor_map_sorted_workspace_bytes(size_t n_in, size_t n_out, int key_bits, int Kw, int Kh) {
