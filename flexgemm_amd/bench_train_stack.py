@@ -54,10 +54,18 @@ def main():
     p.add_argument("--panel-cache", action="store_true",
                    help="keep the repacked weight panels with the weights (flex_gemm.ops.spconv.set_weight_panel_cache): "
                         "the loop never updates its weights, so every pack after the second iteration is saved")
+    p.add_argument("--relu", choices=("none", "fused", "separate"), default="none",
+                   help="a ReLU after every layer: in the GEMM's epilogue (sparse_submanifold_conv3d_relu) or as torch.relu")
     args = p.parse_args()
 
     import flex_gemm
-    from flex_gemm.ops.spconv import Algorithm, SubMConv3dFunction, sparse_submanifold_conv3d
+    from flex_gemm.ops.spconv import Algorithm, SubMConv3dFunction, sparse_submanifold_conv3d, sparse_submanifold_conv3d_relu
+
+    def layer(h, coords, shape, w, b, cache):
+        if args.relu == "fused":
+            return sparse_submanifold_conv3d_relu(h, coords, shape, w, b, cache)[0]
+        h = sparse_submanifold_conv3d(h, coords, shape, w, b, cache)[0]
+        return torch.relu(h) if args.relu == "separate" else h
     from flexgemm_amd import _native as nat
     from flexgemm_amd.workloads import reference_test_shell
 
@@ -86,7 +94,7 @@ def main():
             cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), train)
             h = feats
             for w, b in params:
-                h = sparse_submanifold_conv3d(h, coords, shape, w, b, cache)[0]
+                h = layer(h, coords, shape, w, b, cache)
             if train:
                 h.backward(torch.ones_like(h))
 
@@ -100,7 +108,7 @@ def main():
             def whole_step():
                 h = feats
                 for w, b in params:
-                    h = sparse_submanifold_conv3d(h, coords, shape, w, b, fixed)[0]
+                    h = layer(h, coords, shape, w, b, fixed)
                 if train:
                     h.backward(ones)
                 return h
@@ -133,7 +141,7 @@ def main():
         print(json.dumps({
             "benchmark": "L stacked submanifold 3x3x3 convolutions, " + ("forward + backward" if train else "forward only")
                          + (", replayed from a HIP graph, cache built once" if args.graph else ", cache built per iteration"),
-            "weight_panel_cache": bool(args.panel_cache), "res": res, "channels": c, "layers": layers, "voxels": n, "pairs": pairs, "dtype": "f16",
+            "weight_panel_cache": bool(args.panel_cache), "relu": args.relu, "res": res, "channels": c, "layers": layers, "voxels": n, "pairs": pairs, "dtype": "f16",
             "ms_per_iteration": round(ms, 4), "cache_build_ms": round(ms_build, 4), "gemm_passes": passes,
             "tflops": round(flop / (ms * 1e-3) / 1e12, 1),
         }), flush=True)
