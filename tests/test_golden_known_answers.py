@@ -42,6 +42,11 @@ def test_curve_codes():
     walk = np.array([[0] + p for p in KA["hilbert_first_order"]["walk_xyz"]], dtype=np.int32)
     assert oz.encode(walk, 1, "hilbert").tolist() == list(range(8))
     assert np.array_equal(oz.decode(np.arange(8, dtype=np.int64), 1, "hilbert"), walk)
+    # second order: the orientation of the sub-cubes below the first level, worked by hand from Skilling's steps
+    second = KA["hilbert_second_order"]
+    pts = np.array([[0] + p for p in second["coords_xyz"]], dtype=np.int32)
+    assert oz.encode(pts, second["bit_length"], "hilbert").tolist() == second["codes"]
+    assert np.array_equal(oz.decode(np.array(second["codes"], dtype=np.int64), second["bit_length"], "hilbert"), pts)
 
 
 def test_gray_decode_and_output_extent():
@@ -85,3 +90,6 @@ def test_hip_curve_codes(gpu_device):
     assert codes.cpu().tolist() == z["codes"]
     walk = torch.tensor([[0] + p for p in KA["hilbert_first_order"]["walk_xyz"]], dtype=torch.int32, device=gpu_device)
     assert ops.serialize.encode_seq(walk, torch.Size([1, 0, 2, 2, 2]), mode="hilbert").cpu().tolist() == list(range(8))
+    second = KA["hilbert_second_order"]
+    pts = torch.tensor([[0] + p for p in second["coords_xyz"]], dtype=torch.int32, device=gpu_device)
+    assert ops.serialize.encode_seq(pts, torch.Size([1, 0, 4, 4, 4]), mode="hilbert").cpu().tolist() == second["codes"]
