@@ -94,27 +94,35 @@ __device__ __forceinline__ uint32_t unit_steps(uint32_t cnt, uint32_t p, uint32_
 
 // One thread per XCD cuts its pair ranges into 2 * spx parts and pairs them up; thread 0 then lays out the step lists
 // and the per-offset lists of partial products.  A few thousand scalar operations in all.
-__global__ void __launch_bounds__(64) sweep_units_kernel(const uint32_t* __restrict__ fine, int V, unsigned nsb, unsigned spx,
+constexpr unsigned kSwCumMax = 4096;     // sub-blocks whose running pair counts fit the units kernel's LDS
+__global__ void __launch_bounds__(256) sweep_units_kernel(const uint32_t* __restrict__ fine, int V, unsigned nsb, unsigned spx,
                                                          SweepUnit* __restrict__ units, SweepGroup* __restrict__ wg,
                                                          uint32_t* __restrict__ vcount, uint16_t* __restrict__ vlist) {
     const unsigned x = threadIdx.x;
     const unsigned slots = 2 * spx;
+    // pairs (all offsets) before every sub-block boundary, by all threads: the XCDs' ranges are cut from it
+    __shared__ uint32_t cum[kSwCumMax + 1];
+    const bool by_pairs = nsb <= kSwCumMax;
+    if (by_pairs) {
+        for (unsigned sb = x; sb <= nsb; sb += blockDim.x) {
+            uint32_t c = 0;
+            for (int v = 0; v < V; ++v) c += fine[(size_t)v * (nsb + 1) + sb] - fine[(size_t)v * (nsb + 1)];
+            cum[sb] = c;
+        }
+    }
+    __syncthreads();
     if (x < (unsigned)kXcds) {
         // XCD x takes the sub-blocks [sbA, sbB): boundaries where the running pair count (all offsets) passes x / 8 of
         // the total, so that the XCDs get equal work rather than equal voxel counts
-        auto pairs_before = [&](unsigned sb) {
-            uint64_t c = 0;
-            for (int v = 0; v < V; ++v) c += fine[(size_t)v * (nsb + 1) + sb] - fine[(size_t)v * (nsb + 1)];
-            return c;
-        };
         auto boundary = [&](unsigned xc) -> unsigned {
             if (xc == 0) return 0u;
             if (xc >= (unsigned)kXcds) return nsb;
-            const uint64_t want = pairs_before(nsb) * xc / kXcds;
+            if (!by_pairs) return (unsigned)((uint64_t)xc * nsb / kXcds);      // (very many sub-blocks: equal voxel counts)
+            const uint64_t want = (uint64_t)cum[nsb] * xc / kXcds;
             unsigned lo_sb = 0, hi_sb = nsb;            // first sub-block boundary with at least `want` pairs before it
             while (lo_sb < hi_sb) {
                 const unsigned mid = (lo_sb + hi_sb) >> 1;
-                if (pairs_before(mid) < want) lo_sb = mid + 1;
+                if (cum[mid] < want) lo_sb = mid + 1;
                 else hi_sb = mid;
             }
             return lo_sb;
@@ -867,7 +875,7 @@ int fgx_wgrad_sweep_plan(const uint32_t* sig_o, const uint32_t* seg_host, size_t
     phase_mark("wgrad sweep plan", s);
     block_bounds_kernel<<<cdiv((size_t)V * (L.nsb + 1), 256), 256, 0, s>>>(sig_o, tab, V, L.nsb, (unsigned)sub_rows, fine);
     FGX_CHECK_LAUNCH("fgx_wgrad_sweep_plan(bounds)");
-    sweep_units_kernel<<<1, 64, 0, s>>>(fine, V, L.nsb, L.spx, (SweepUnit*)(p + L.units), (SweepGroup*)(p + L.wg),
+    sweep_units_kernel<<<1, 256, 0, s>>>(fine, V, L.nsb, L.spx, (SweepUnit*)(p + L.units), (SweepGroup*)(p + L.wg),
                                         (uint32_t*)(p + L.vcount), (uint16_t*)(p + L.vlist));
     FGX_CHECK_LAUNCH("fgx_wgrad_sweep_plan(units)");
     sweep_steps_kernel<<<L.groups, 256, 0, s>>>(fine, L.nsb, (const SweepUnit*)(p + L.units), (const SweepGroup*)(p + L.wg),
