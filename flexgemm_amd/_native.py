@@ -12,7 +12,8 @@ from typing import Optional
 
 import torch
 
-_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "libflexgemm_hip.so")
+# (FGX_LIB_PATH: another build of the same library, e.g. one compiled with different kernel parameters)
+_LIB_PATH = os.environ.get("FGX_LIB_PATH") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "libflexgemm_hip.so")
 _lib: Optional[C.CDLL] = None
 
 FGX_F16, FGX_BF16, FGX_F32 = 0, 1, 2
