@@ -4,11 +4,11 @@ The counters FETCH_SIZE and WRITE_SIZE (KiB per dispatch, collected in a run of 
 the same counter reads for the plain copy that `bench.py --calibrate-copy` adds (1 GiB read, 1 GiB written per
 launch).  Usage, after the two runs
 
-    rocprofv3 --pmc FETCH_SIZE --output-format csv -d gpurun_out/pmc_fetch -- python3 bench.py --steps 5 --warmup 2 --no-cpu-baseline --calibrate-copy
-    rocprofv3 --pmc WRITE_SIZE --output-format csv -d gpurun_out/pmc_write -- python3 bench.py --steps 5 --warmup 2 --no-cpu-baseline --calibrate-copy
+    rocprofv3 --pmc FETCH_SIZE --output-format csv -d /tmp/pmc_fetch -- python3 bench.py --steps 5 --warmup 2 --no-cpu-baseline --calibrate-copy
+    rocprofv3 --pmc WRITE_SIZE --output-format csv -d /tmp/pmc_write -- python3 bench.py --steps 5 --warmup 2 --no-cpu-baseline --calibrate-copy
 
     python -m flexgemm_amd.profile_traffic --workload cfg3 --dtype f16 --kernel gather_gemm_stream_kernel \
-        --fetch gpurun_out/pmc_fetch --write gpurun_out/pmc_write
+        --fetch /tmp/pmc_fetch --write /tmp/pmc_write
 
 writes the entry "cfg3_f16" of profiles/traffic.json (and prints a table of every kernel of the run for the summary
 under profiles/).  The entry carries a digest of the kernel's source files; bench.py reports the traffic only while
