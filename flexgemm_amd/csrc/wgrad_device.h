@@ -54,6 +54,14 @@ __device__ __forceinline__ i16x4 lds_read_tr16(const unsigned char* p) {
     asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(r) : "v"(addr));
     return r;
 }
+// the same with the address given as an LDS byte address plus a constant that goes into the instruction's offset field
+template <int OFFSET>
+__device__ __forceinline__ i16x4 lds_read_tr16_at(uint32_t addr) {
+    static_assert(OFFSET >= 0 && OFFSET < 65536, "the offset field is 16 bits wide");
+    i16x4 r;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFFSET));
+    return r;
+}
 template <int N>
 __device__ __forceinline__ void lds_wait_all(i16x4 (&r)[N]) {
     static_assert(N % 4 == 0, "fragments come in groups of four registers pairs");

@@ -32,14 +32,56 @@ namespace fgx {
 namespace {
 
 constexpr int kSwStages = 4;         // row ring depth
-constexpr int kSwIdxSlots = 8;       // index ring depth
-constexpr int kSwIdxAhead = 4;       // index loads run this many steps ahead of the row loads
+constexpr int kSwIdxSlots = 8;       // index ring: two slots per loader
 constexpr int kSwLoaders = 4;
 constexpr int kSwPairs = 64;         // pairs per step
 constexpr int kSwStepRing = 256;     // step-list entries held in LDS (four chunks of 64)
 constexpr int kSwMergeShift = 1;     // a workgroup changes units every 2^this sub-blocks (a change swaps the accumulators)
 constexpr int kSwMaxSlots = 64;      // workgroups per XCD the pacing poll can look at (one lane each)
 constexpr int kSwMaxGroups = kXcds * kSwMaxSlots;
+constexpr unsigned kSwSpinMax = 1u << 20;   // looks at a progress word before a wavefront goes on regardless
+
+// Progress words in LDS replace a barrier per step.  Loader w owns ring stage w and counts the steps it has landed
+// there (step k is landed[k % S] > k / S); every multiplier counts the steps whose fragments it has read, and a
+// loader refills its stage with step k once all four have read step k - S.  A wavefront writes only its own word.
+// The LDS executes one wavefront's operations in order and a word is written after the wait for what it announces,
+// so whoever sees the count also sees the data.  The roles run up to S - 1 steps apart and nobody waits for a
+// wavefront of its own role.
+__device__ __forceinline__ void progress_store(uint32_t* word, uint32_t v) {
+    const uint32_t addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)word;
+    asm volatile("ds_write_b32 %0, %1" ::"v"(addr), "v"(v) : "memory");
+}
+__device__ __forceinline__ uint32_t progress_load(const uint32_t* word) {
+    const uint32_t addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint32_t*)word;
+    uint32_t w;
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(w) : "v"(addr) : "memory");
+    return (uint32_t)__builtin_amdgcn_readfirstlane((int)w);
+}
+__device__ __forceinline__ uint32_t progress_min4(const uint32_t* words) {
+    const uint32_t addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint32_t*)words;
+    u32x4 w;
+    asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(w) : "v"(addr) : "memory");
+    const uint32_t a = w[0] < w[1] ? w[0] : w[1], b = w[2] < w[3] ? w[2] : w[3];
+    return (uint32_t)__builtin_amdgcn_readfirstlane((int)(a < b ? a : b));
+}
+// a 32-bit LDS read that is not waited for here: the value may be used after a later wait for LDS reads (they return
+// in order) and lds_arrived(), which keeps the compiler from using it earlier
+__device__ __forceinline__ uint32_t lds_read_word(const uint32_t* word) {
+    const uint32_t addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint32_t*)word;
+    uint32_t w;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(w) : "v"(addr) : "memory");
+    return w;
+}
+__device__ __forceinline__ void lds_arrived(uint32_t& a, uint32_t& b) { asm volatile("" : "+v"(a), "+v"(b)); }
+// spins until the minimum of the four words reaches `need`; `known` caches the last minimum seen
+__device__ __forceinline__ void progress_wait(const uint32_t* words, uint32_t need, uint32_t& known) {
+    if (known >= need) return;
+    for (unsigned spins = 0; spins < kSwSpinMax; ++spins) {
+        known = progress_min4(words);
+        if (known >= need) return;
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
 
 // ------------------------------------------------------------------------------------------------
 // Plan: fine bounds, units (parts), per-workgroup step lists
@@ -288,19 +330,35 @@ __device__ __forceinline__ void swap_tiles(f32x16& a, f32x16& b) {
 #endif
 }
 
-// sum of the eight 16-bit values of a fragment, in fp32
-template <typename Tag> __device__ __forceinline__ float sum8(const i16x8& f);
-template <> __device__ __forceinline__ float sum8<F16>(const i16x8& f) {
-    const f16x8 h = __builtin_bit_cast(f16x8, f);
-    return (((float)h[0] + (float)h[1]) + ((float)h[2] + (float)h[3])) + (((float)h[4] + (float)h[5]) + ((float)h[6] + (float)h[7]));
+// acc + the eight 16-bit values of a fragment, each times the 16-bit value `w` (given twice, as a packed pair: ones to
+// count the fragment, zeros to leave the sum as it is), in fp32: four two-element dot products
+using f16x2 = _Float16 __attribute__((ext_vector_type(2)));
+using bf16x2 = __bf16 __attribute__((ext_vector_type(2)));
+template <typename Tag> __device__ __forceinline__ float add8(float acc, const i16x8& f, uint32_t w);
+template <> __device__ __forceinline__ float add8<F16>(float acc, const i16x8& f, uint32_t w) {
+    // (the four pairs are taken out of a vector of pairs: a bit cast of an indexed 32-bit element inside an unrolled loop
+    // has been seen to read element 0 four times)
+    struct Pairs { f16x2 p0, p1, p2, p3; };
+    const Pairs d = __builtin_bit_cast(Pairs, f);
+    const f16x2 ww = __builtin_bit_cast(f16x2, w);
+    acc = __builtin_amdgcn_fdot2(d.p0, ww, acc, false);
+    acc = __builtin_amdgcn_fdot2(d.p1, ww, acc, false);
+    acc = __builtin_amdgcn_fdot2(d.p2, ww, acc, false);
+    acc = __builtin_amdgcn_fdot2(d.p3, ww, acc, false);
+    return acc;
 }
-template <> __device__ __forceinline__ float sum8<BF16>(const i16x8& f) {
-    const u32x4 w = __builtin_bit_cast(u32x4, f);
-    float s = 0.f;
-#pragma unroll
-    for (int q = 0; q < 4; ++q)
-        s += __builtin_bit_cast(float, w[q] << 16) + __builtin_bit_cast(float, w[q] & 0xFFFF0000u);
-    return s;
+template <> __device__ __forceinline__ float add8<BF16>(float acc, const i16x8& f, uint32_t w) {
+    struct Pairs { bf16x2 p0, p1, p2, p3; };
+    const Pairs d = __builtin_bit_cast(Pairs, f);
+    const bf16x2 ww = __builtin_bit_cast(bf16x2, w);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(d.p0, ww, acc, false);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(d.p1, ww, acc, false);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(d.p2, ww, acc, false);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(d.p3, ww, acc, false);
+    return acc;
+}
+template <typename Tag> __device__ __forceinline__ uint32_t packed_ones() {
+    return __is_same(typename Tag::type, _Float16) ? 0x3C003C00u : 0x3F803F80u;
 }
 
 template <typename Tag, int BM, int BN>
@@ -317,11 +375,11 @@ struct SweepCfg {
     static constexpr int LPS = A_PER + B_PER;
     static constexpr int A_BYTES = P * ROWB_A, B_BYTES = P * ROWB_B, STAGE_BYTES = A_BYTES + B_BYTES;
     static constexpr int IDX_SLOT_BYTES = 2 * P * 4;               // sig_o x P | sig_i x P
-    static constexpr size_t lds_bytes = (size_t)S * STAGE_BYTES + (size_t)kSwIdxSlots * IDX_SLOT_BYTES + (size_t)kSwStepRing * 8;
+    static constexpr size_t lds_bytes = (size_t)S * STAGE_BYTES + (size_t)kSwIdxSlots * IDX_SLOT_BYTES + (size_t)kSwStepRing * 8 + 32;
+    static_assert(NW == 4 && NL == S, "one loader per ring stage; the multipliers' progress words are read four at a time");
     static_assert(ES == 2, "16-bit types");
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
     static_assert(P % (RPI_A * NL) == 0 && P % (RPI_B * NL) == 0, "every loader issues the same row loads");
-    static_assert(2 * (LPS + 3) < 64, "outstanding loads exceed the vmcnt range");
     static constexpr int key_a(int row) { return CH_A >= 8 ? 2 * (row & 3) : 0; }
     static constexpr int key_b(int row) { return CH_B >= 8 ? 2 * (row & 3) : 0; }
 };
@@ -343,6 +401,8 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
     uint32_t* idx_ring = (uint32_t*)(ring + S * C::STAGE_BYTES);                // [kSwIdxSlots][o x P | i x P]
     uint32_t* step_k = idx_ring + kSwIdxSlots * 2 * P;                          // [kSwStepRing] first pair of a step
     uint32_t* step_m = step_k + kSwStepRing;                                    // [kSwStepRing] count | unit | sub-block
+    uint32_t* landed = step_m + kSwStepRing;                                    // [NL] steps whose rows have landed, per loader
+    uint32_t* consumed = landed + 4;                                            // [NW] steps read, per multiplier
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -387,125 +447,78 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
             load_chunk(0);
             load_chunk(1);
             wait_vmcnt<0>();
+        } else if (lw == 1 && lane < 8) {
+            landed[lane] = 0u;                      // (landed and consumed are adjacent)
         }
-        __syncthreads();                            // (1) the first two chunks of the step list are in LDS
-        int a_row[C::A_PER], b_row[C::B_PER];
-        uint32_t a_chb[C::A_PER], b_chb[C::B_PER];          // byte column inside the tile, swizzle applied
-#pragma unroll
-        for (int i = 0; i < C::A_PER; ++i) {
-            a_row[i] = (i * C::NL + lw) * C::RPI_A + lane / C::CH_A;
-            a_chb[i] = (uint32_t)(((lane % C::CH_A) ^ C::key_a(a_row[i])) * 16);
-        }
-#pragma unroll
-        for (int i = 0; i < C::B_PER; ++i) {
-            b_row[i] = (i * C::NL + lw) * C::RPI_B + lane / C::CH_B;
-            b_chb[i] = (uint32_t)(((lane % C::CH_B) ^ C::key_b(b_row[i])) * 16);
-        }
-        unsigned f_step = 0, r_step = 0;            // index stream, row stream: steps handed out so far
-        // The list entries of the two streams' next steps are read one round early (right after the previous ones were
-        // used), so that their LDS latency passes while this wavefront waits at the barrier instead of before its loads.
-        uint32_t f_k = step_k[0], r_left = step_m[0] & 127u;
-        auto issue_idx = [&]() -> int {             // index loads of the index stream's next step (+ step-list prefetch)
-            if (f_step >= nsteps) return 0;
-            int ops = 0;
-            const uint32_t k = f_k;
-            uint32_t* dst = idx_ring + (f_step & (kSwIdxSlots - 1)) * (2 * P);
-            if (lw == 0) {
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(sigo_rs, FGX_LDS_PTR(dst), 4, (k + (uint32_t)lane) * 4u, 0, 0, 0);
-                ops = 1;
-                if ((f_step & 63) == 0) {           // the chunk after next; its quarter of the ring was read 128+ steps ago
-                    load_chunk(f_step / 64 + 2);
-                    ops += 2;
-                }
-            } else if (lw == 1) {
-                uint32_t* dst_i = dst + P;
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(sigi_rs, FGX_LDS_PTR(dst_i), 4, (k + (uint32_t)lane) * 4u, 0, 0, 0);
-                ops = 1;
-            }
-            ++f_step;
-            f_k = step_k[f_step & (kSwStepRing - 1)];
-            return ops;
+        __syncthreads();                            // (1) the first two chunks of the step list are in LDS, progress words zero
+        // Loader lw owns ring stage lw and the steps lw, lw + S, lw + 2S, ...: it enqueues all of a step's rows, prepares
+        // the next step's addresses while they are on their way, and announces the step when they have landed.  The
+        // four loaders take turns on the address path, and the per-step scalar work and LDS round trips of the
+        // preparation happen once per step and loader beside the load latency instead of in front of it.
+        constexpr int NA = P / C::RPI_A, NB = P / C::RPI_B;     // load instructions per operand and step
+        static_assert(NA + NB + 6 < 64, "outstanding loads exceed the vmcnt range");
+        const int a_sub = lane / C::CH_A, b_sub = lane / C::CH_B;          // row inside a load instruction
+        // byte column inside the tile, swizzle applied (the key depends on row & 3 alone, an instruction covers 4 or 8 rows)
+        const uint32_t a_chb = (uint32_t)(((lane % C::CH_A) ^ C::key_a(a_sub)) * 16);
+        const uint32_t b_chb = (uint32_t)(((lane % C::CH_B) ^ C::key_b(b_sub)) * 16);
+        unsigned char* stage = ring + lw * C::STAGE_BYTES;
+        uint32_t* my_idx = idx_ring + lw * 2 * (2 * P);                    // two index slots per loader
+        auto issue_idx = [&](unsigned k) {         // index columns of step k into slot (k / S) & 1
+            if (k >= nsteps) return;
+            const uint32_t first = step_k[k & (kSwStepRing - 1)];
+            uint32_t* dst = my_idx + ((k / S) & 1) * (2 * P);
+            uint32_t* dst_i = dst + P;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(sigo_rs, FGX_LDS_PTR(dst), 4, (first + (uint32_t)lane) * 4u, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(sigi_rs, FGX_LDS_PTR(dst_i), 4, (first + (uint32_t)lane) * 4u, 0, 0, 0);
         };
-        bool pr_live = false;
-        unsigned pr_stage = 0;
-        uint32_t va[C::A_PER], vb[C::B_PER];
-        auto prep_rows = [&]() {
-            pr_live = r_step < nsteps;
-            if (!pr_live) return;
-            pr_stage = r_step & (S - 1);
-            const uint32_t* slot_p = idx_ring + (r_step & (kSwIdxSlots - 1)) * (2 * P);
-            const uint32_t left = r_left;                                             // pairs in this step
+        uint32_t va[NA], vb[NB];
+        auto prep_rows = [&](unsigned k) {         // buffer offsets of step k's rows (rows and row sizes fit 24 bits)
+            if (k >= nsteps) return;
+            const uint32_t* slot_p = my_idx + ((k / S) & 1) * (2 * P);
+            const uint32_t left = step_m[k & (kSwStepRing - 1)] & 127u;                // pairs in this step
             const bool ragged = left < (uint32_t)P || (uint32_t)(BM * ES) > rowb_o || (uint32_t)(BN * ES) > rowb_i;   // uniform
 #pragma unroll
-            for (int i = 0; i < C::A_PER; ++i) va[i] = slot_p[a_row[i]] * rowb_o + a_chb[i];
+            for (int i = 0; i < NA; ++i) va[i] = __umul24(slot_p[i * C::RPI_A + a_sub], rowb_o) + a_chb;
 #pragma unroll
-            for (int i = 0; i < C::B_PER; ++i) vb[i] = slot_p[P + b_row[i]] * rowb_i + b_chb[i];
+            for (int i = 0; i < NB; ++i) vb[i] = __umul24(slot_p[P + i * C::RPI_B + b_sub], rowb_i) + b_chb;
             if (ragged) {
 #pragma unroll
-                for (int i = 0; i < C::A_PER; ++i)
-                    va[i] = ((uint32_t)a_row[i] < left && a_chb[i] < rowb_o) ? va[i] : kOobOffset;
+                for (int i = 0; i < NA; ++i)
+                    va[i] = ((uint32_t)(i * C::RPI_A + a_sub) < left && a_chb < rowb_o) ? va[i] : kOobOffset;
 #pragma unroll
-                for (int i = 0; i < C::B_PER; ++i)
-                    vb[i] = ((uint32_t)b_row[i] < left && b_chb[i] < rowb_i) ? vb[i] : kOobOffset;
+                for (int i = 0; i < NB; ++i)
+                    vb[i] = ((uint32_t)(i * C::RPI_B + b_sub) < left && b_chb < rowb_i) ? vb[i] : kOobOffset;
             }
-            ++r_step;
-            r_left = step_m[r_step & (kSwStepRing - 1)] & 127u;
         };
-        auto fire_rows = [&]() -> int {             // 0 when the stream is over
-            if (!pr_live) return 0;
-            unsigned char* stage = ring + pr_stage * C::STAGE_BYTES;
+        auto fire_rows = [&]() {
 #pragma unroll
-            for (int i = 0; i < C::A_PER; ++i) {
+            for (int i = 0; i < NA; ++i) {
                 const uint32_t vo = va[i];
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(gout_rs, FGX_LDS_PTR(stage + (i * C::NL + lw) * 1024), 16, vo, 0, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(gout_rs, FGX_LDS_PTR(stage + i * 1024), 16, vo, 0, 0, 0);
             }
             unsigned char* stage_b = stage + C::A_BYTES;
 #pragma unroll
-            for (int i = 0; i < C::B_PER; ++i) {
+            for (int i = 0; i < NB; ++i) {
                 const uint32_t vo = vb[i];
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(feats_rs, FGX_LDS_PTR(stage_b + (i * C::NL + lw) * 1024), 16, vo, 0, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(feats_rs, FGX_LDS_PTR(stage_b + i * 1024), 16, vo, 0, 0, 0);
             }
-            return C::LPS;
-        };
-        // at most `n` of this loader's loads may be outstanding; n is the sum of the loads of the last two rounds, each
-        // 0 ... LPS + 3 (rounded down to the next value handled here, which is merely stricter)
-        auto wait_loads = [&](int n) {
-            if (n >= 2 * C::LPS + 2) wait_vmcnt<2 * C::LPS + 2>();
-            else if (n == 2 * C::LPS + 1) wait_vmcnt<2 * C::LPS + 1>();
-            else if (n == 2 * C::LPS) wait_vmcnt<2 * C::LPS>();
-            else if (n > C::LPS) wait_vmcnt<C::LPS + 1>();
-            else if (n == C::LPS) wait_vmcnt<C::LPS>();
-            else wait_vmcnt<0>();
         };
 
-        // prologue: indices of the first kSwIdxAhead steps, then S-1 row rounds
-#pragma unroll
-        for (int j = 0; j < kSwIdxAhead; ++j) (void)issue_idx();
+        issue_idx((unsigned)lw);
+        issue_idx((unsigned)lw + S);
         wait_vmcnt<0>();
         __syncthreads();                            // (2)
-        prep_rows();
-        int drained = 0, ops1 = 0, ops2 = 0;        // ops1: loads issued in the previous round, ops2: the one before
-#pragma unroll
-        for (int j = 0; j < S - 1; ++j) {
-            int ops = fire_rows();
-            if (ops == 0) ++drained;
-            prep_rows();                            // indices of steps 1 .. S-1 came with the first batch
-            ops += issue_idx();
-            ops2 = ops1;
-            ops1 = ops;
-        }
-        while (true) {
-            wait_loads(ops1 + ops2);               // everything issued before the last two rounds has landed
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_s_barrier();          // ... everybody's; the stage multiplied in the previous step is free
-            asm volatile("" ::: "memory");
-            int ops = fire_rows();
-            if (ops == 0) ++drained;
-            if (drained >= S - 1) break;           // that was the barrier of the stream's last step
-            prep_rows();
-            ops += issue_idx();
-            ops2 = ops1;
-            ops1 = ops;
+        prep_rows((unsigned)lw);
+        uint32_t known_consumed = 0;
+        for (unsigned k = (unsigned)lw; k < nsteps; k += S) {
+            if (k >= (unsigned)S) progress_wait(consumed, k - S + 1u, known_consumed);   // every multiplier has read step k - S
+            fire_rows();
+            // loader 0 also keeps the step list: the chunk after next, whose quarter of the ring was read 128+ steps ago
+            if (lw == 0 && (k & 63u) == 0u) load_chunk(k / 64 + 2);
+            issue_idx(k + 2 * S);
+            prep_rows(k + S);                       // its index columns landed a round ago
+            wait_vmcnt<0>();
+            progress_store(landed + lw, k / S + 1u);
         }
         wait_vmcnt<0>();
         return;
@@ -518,22 +531,23 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
     __syncthreads();                                // (2) the loaders' prologue barriers
     const SweepUnit un0 = units[(size_t)gid * 2], un1 = units[(size_t)gid * 2 + 1];
     const int s16 = lane & 15, mb = (lane >> 4) & 1;
-    int a_off[C::TM][2], b_off[C::TN][2];
+    // Per-lane byte offsets of the transposing reads inside a stage, for k-block 0 and the first of a lane's two pair
+    // rows; the second pair row (4 rows on: same swizzle key) and the k-block go into the instruction's offset field.
+    uint32_t a_off[C::TM], b_off[C::TN];
     {
         const int prow = g * 8 + (s16 >> 2);
+        static_assert(C::key_a(0) == C::key_a(4) && C::key_b(1) == C::key_b(5), "pair rows 4 apart share a swizzle key");
 #pragma unroll
         for (int i = 0; i < C::TM; ++i) {
             const int byte = (wave_m * C::WM + i * 32 + mb * 16 + (s16 & 3) * 4) * 2;
             const int c = byte >> 4, w = byte & 15;
-            a_off[i][0] = prow * C::ROWB_A + ((c ^ C::key_a(prow)) << 4) + w;
-            a_off[i][1] = (prow + 4) * C::ROWB_A + ((c ^ C::key_a(prow + 4)) << 4) + w;
+            a_off[i] = (uint32_t)(prow * C::ROWB_A + ((c ^ C::key_a(prow)) << 4) + w);
         }
 #pragma unroll
         for (int j = 0; j < C::TN; ++j) {
             const int byte = (wave_n * C::WN + j * 32 + mb * 16 + (s16 & 3) * 4) * 2;
             const int c = byte >> 4, w = byte & 15;
-            b_off[j][0] = C::A_BYTES + prow * C::ROWB_B + ((c ^ C::key_b(prow)) << 4) + w;
-            b_off[j][1] = C::A_BYTES + (prow + 4) * C::ROWB_B + ((c ^ C::key_b(prow + 4)) << 4) + w;
+            b_off[j] = (uint32_t)(C::A_BYTES + prow * C::ROWB_B + ((c ^ C::key_b(prow)) << 4) + w);
         }
     }
     constexpr int NK = P / 16;                      // k-blocks (16 pair rows) per step
@@ -557,49 +571,46 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
     }
     unsigned acc_unit = 0;                          // whose sums `acc` holds
     // Column sums of grad_out (the bias gradient) ride along with the offset whose pairs hold every output row once:
-    // a lane's grad_out fragment is eight pair values of one output channel, which it adds up on the side (a second
-    // accumulator tile of ones-products, as in the block-major kernel, does not fit beside two accumulators).  Both
+    // a lane's grad_out fragment is eight pair values of one output channel, which it adds up on the side with four
+    // two-element dot products against ones (a second accumulator tile of ones-products, as in the block-major
+    // kernel, does not fit beside two accumulators; converting and adding the eight values one by one took as many
+    // issue slots as the step's MFMAs and made the workgroups of this offset the last to finish).  Both
     // units of a workgroup add to the same sums; only the wavefronts of the first column of wave tiles do it.
     const bool bias0 = bias_partial != nullptr && un0.nsteps && (int)un0.v == bias_offset && wave_n == 0;
     const bool bias1 = bias_partial != nullptr && un1.nsteps && (int)un1.v == bias_offset && wave_n == 0;
 
-    auto multiply_step = [&](const unsigned char* cur, auto with_bias, const bool count_bias) {
-        i16x4 fr[2][RK];
-        auto read_block = [&](int kk, i16x4 (&dst)[RK]) {
-            const unsigned char* base = cur + kk * 16 * C::ROWB_A;
+    // Fragments of one k-block (16 pair rows): TM x 2 reads of the grad_out tile, TN x 2 of the feats tile.
+    i16x4 fr[2][RK];
+    // (the k-block is a compile-time constant: it is part of the instructions' offset fields)
+    auto read_block = [&](const uint32_t stage_addr, auto kk_c, i16x4 (&dst)[RK]) {
+        constexpr int kk = decltype(kk_c)::value;
 #pragma unroll
-            for (int i = 0; i < C::TM; ++i) {
-                dst[i * 2] = lds_read_tr16(base + a_off[i][0]);
-                dst[i * 2 + 1] = lds_read_tr16(base + a_off[i][1]);
-            }
-            const unsigned char* base_b = cur + kk * 16 * C::ROWB_B;
+        for (int i = 0; i < C::TM; ++i) {
+            dst[i * 2] = lds_read_tr16_at<kk * 16 * C::ROWB_A>(stage_addr + a_off[i]);
+            dst[i * 2 + 1] = lds_read_tr16_at<kk * 16 * C::ROWB_A + 4 * C::ROWB_A>(stage_addr + a_off[i]);
+        }
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) {
+            dst[(C::TM + j) * 2] = lds_read_tr16_at<kk * 16 * C::ROWB_B>(stage_addr + b_off[j]);
+            dst[(C::TM + j) * 2 + 1] = lds_read_tr16_at<kk * 16 * C::ROWB_B + 4 * C::ROWB_B>(stage_addr + b_off[j]);
+        }
+    };
+    using K0 = std::integral_constant<int, 0>;
+    using K1 = std::integral_constant<int, 1>;
+    using K2 = std::integral_constant<int, 2>;
+    using K3 = std::integral_constant<int, 3>;
+    const uint32_t ring_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const unsigned char*)ring;
+    // the products of one k-block; `bias_w`: packed ones to count the grad_out fragments into the bias sums, zeros not to
+    // (a weight, not a branch: the step stays straight-line code)
+    auto multiply_block = [&](i16x4 (&f)[RK], auto with_bias, const uint32_t bias_w) {
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i) {
+            const i16x8 af = __builtin_shufflevector(f[i * 2], f[i * 2 + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+            if constexpr (decltype(with_bias)::value) bsum[i] = add8<Tag>(bsum[i], af, bias_w);
 #pragma unroll
             for (int j = 0; j < C::TN; ++j) {
-                dst[(C::TM + j) * 2] = lds_read_tr16(base_b + b_off[j][0]);
-                dst[(C::TM + j) * 2 + 1] = lds_read_tr16(base_b + b_off[j][1]);
-            }
-        };
-        read_block(0, fr[0]);
-#pragma unroll
-        for (int kk = 0; kk < NK; ++kk) {
-            if (kk + 1 < NK) {
-                read_block(kk + 1, fr[(kk + 1) & 1]);
-                lds_wait_but<RK>(fr[kk & 1]);
-            } else {
-                lds_wait_but<0>(fr[kk & 1]);
-            }
-#pragma unroll
-            for (int i = 0; i < C::TM; ++i) {
-                const i16x8 af = __builtin_shufflevector(fr[kk & 1][i * 2], fr[kk & 1][i * 2 + 1], 0, 1, 2, 3, 4, 5, 6, 7);
-                if constexpr (decltype(with_bias)::value) {
-                    const float s8 = sum8<Tag>(af);     // (a select, not a branch: the step stays one basic block)
-                    bsum[i] += count_bias ? s8 : 0.f;
-                }
-#pragma unroll
-                for (int j = 0; j < C::TN; ++j) {
-                    const i16x8 bf = __builtin_shufflevector(fr[kk & 1][(C::TM + j) * 2], fr[kk & 1][(C::TM + j) * 2 + 1], 0, 1, 2, 3, 4, 5, 6, 7);
-                    mma16<Tag>(acc[i][j], af, bf);
-                }
+                const i16x8 bf = __builtin_shufflevector(f[(C::TM + j) * 2], f[(C::TM + j) * 2 + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                mma16<Tag>(acc[i][j], af, bf);
             }
         }
     };
@@ -614,26 +625,59 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
     // in the workgroups that hold a unit of the bias offset (a per-step choice between two forms would keep both
     // forms' address registers alive next to two accumulators).
     auto run_steps = [&](auto with_bias) {
-        uint32_t next_meta = step_m[0];
+        static_assert(NK == 4, "the step below is written out for four k-blocks");
+        // The fragment reads run one k-block ahead of the products and do not stop at the end of a step: while the last
+        // k-block of a step is multiplied the first one of the next step arrives.
+        uint32_t meta = step_m[0];
+        for (unsigned spins = 0; spins < kSwSpinMax && progress_load(landed) < 1u; ++spins) __builtin_amdgcn_s_sleep(1);
+        read_block(ring_addr, K0{}, fr[0]);
+        lds_wait_but<0>(fr[0]);
         for (unsigned step = 0; step < nsteps; ++step) {
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_s_barrier();               // the loaders saw this step's rows land
-            asm volatile("" ::: "memory");
-            const unsigned char* cur = ring + (step & (S - 1)) * C::STAGE_BYTES;
-            const uint32_t meta = next_meta;            // (read during the previous step: no LDS round trip after the barrier)
+            const uint32_t cur = ring_addr + (step & (S - 1)) * (uint32_t)C::STAGE_BYTES;
+            const uint32_t nxt = ring_addr + ((step + 1) & (S - 1)) * (uint32_t)C::STAGE_BYTES;
+            const bool more = step + 1 < nsteps;
             const unsigned unit = (meta >> 7) & 1u;
             if (unit != acc_unit) {
                 acc_unit = unit;
+                // (the swaps are assembly the compiler does not see into: let the last products leave the pipe first)
+#pragma unroll
+                for (int q = 0; q < 3; ++q) asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
                 for (int i = 0; i < C::TM; ++i)
 #pragma unroll
                     for (int j = 0; j < C::TN; ++j) swap_tiles(acc[i][j], rest[i][j]);
             }
-            next_meta = step_m[(step + 1) & (kSwStepRing - 1)];
-            multiply_step(cur, with_bias, unit ? bias1 : bias0);
-            // Pacing, by the first multiplier before it joins the next step's barrier (which holds the whole workgroup
-            // back with it): tell the XCD which sub-block this workgroup is entering, and do not enter one more than
-            // `lead` ahead of the slowest workgroup.  Bounded: after max_polls looks the workgroup stops pacing.
+            const uint32_t bias_w = (unit ? bias1 : bias0) ? packed_ones<Tag>() : 0u;
+            read_block(cur, K1{}, fr[1]);
+            multiply_block(fr[0], with_bias, bias_w);       // (landed before the loop came round)
+            // the next step's list entry and its stage's progress word travel with the fragments of the third k-block
+            uint32_t next_meta = lds_read_word(step_m + ((step + 1) & (kSwStepRing - 1)));
+            uint32_t seen = lds_read_word(landed + ((step + 1) & (S - 1)));
+            read_block(cur, K2{}, fr[0]);
+            lds_wait_but<RK>(fr[1]);
+            lds_arrived(next_meta, seen);
+            multiply_block(fr[1], with_bias, bias_w);
+            read_block(cur, K3{}, fr[1]);
+            lds_wait_but<RK>(fr[0]);
+            multiply_block(fr[0], with_bias, bias_w);
+            if (more && (uint32_t)__builtin_amdgcn_readfirstlane((int)seen) < (step + 1) / S + 1u) {     // the loaders are behind: wait here
+                for (unsigned spins = 0; spins < kSwSpinMax && progress_load(landed + ((step + 1) & (S - 1))) < (step + 1) / S + 1u; ++spins)
+                    __builtin_amdgcn_s_sleep(1);
+            }
+            read_block(nxt, K0{}, fr[0]);                      // (after the last step: read and never used)
+            lds_wait_but<RK>(fr[1]);
+            progress_store(consumed + mw, step + 1u);       // the stage has been read: its loader may refill it
+            multiply_block(fr[1], with_bias, bias_w);
+            // The prefetched fragments land while these products run.  They are waited for before the loop goes round:
+            // registers with a read in flight must not cross the loop edge, where the compiler may copy them.
+            lds_wait_but<0>(fr[0]);
+            meta = (uint32_t)__builtin_amdgcn_readfirstlane((int)next_meta);
+            next_meta = meta;
+            // Pacing, by the first multiplier before its next step (while it waits its progress word stands still, the
+            // loaders run out of free stages after S - 1 steps and the other multipliers out of landed ones, so the
+            // whole workgroup is held back with it): tell the XCD which sub-block this workgroup is entering, and do
+            // not enter one more than `lead` ahead of the slowest workgroup.  Bounded: after max_polls looks the
+            // workgroup stops pacing.
             if (mw == 0 && step + 1 < nsteps) {
                 const uint32_t next_sb = next_meta >> 8;
                 if (next_sb != cur_sb) {
@@ -900,7 +944,8 @@ int fgx_conv_wgrad_sweep(int dtype, const void* grad_out, const void* feats, con
     FGX_CHECK_ARG(Ci % 8 == 0 && Co % 8 == 0, "fgx_conv_wgrad_sweep: rows of %d / %d elements are not multiples of 16 bytes", Ci, Co);
     FGX_CHECK_ARG(sub_rows >= 64 && lead >= 0 && max_polls >= 0, "fgx_conv_wgrad_sweep: bad pacing arguments");
     FGX_CHECK_ARG(seg_host && plan && scratch && grad_weight, "fgx_conv_wgrad_sweep: null buffer");
-    FGX_CHECK_ARG(n > 0 && n < 0xFFFFFFFFull && n_in < 0xFFFFFFFFull, "fgx_conv_wgrad_sweep: row count out of range");
+    // (the loaders multiply row numbers with 24-bit multiplies)
+    FGX_CHECK_ARG(n > 0 && n <= (1ull << 24) && n_in <= (1ull << 24), "fgx_conv_wgrad_sweep: at most 2^24 rows per operand (n=%zu, n_in=%zu)", n, n_in);
     FGX_CHECK_ARG(((uintptr_t)scratch & 255) == 0 && ((uintptr_t)plan & 255) == 0, "fgx_conv_wgrad_sweep: scratch and plan must be 256-byte aligned");
     const size_t n_pairs = seg_host[V];
     FGX_CHECK_ARG(n_pairs > 0 && grad_out && feats && sig_i && sig_o, "fgx_conv_wgrad_sweep: empty pair lists or null buffer");
