@@ -61,9 +61,11 @@ def parse():
     p.add_argument("--workload", default="cfg3", choices=["cfg2", "cfg3", "cfg4", "cfg5"])
     p.add_argument("--dtype", default=None, choices=["f16", "bf16", "f32"], help="override the configuration's dtype")
     p.add_argument("--wgrad-sweep", type=int, default=0, metavar="SUB_ROWS",
-                   help="run wgrad as the paced sweep (fgx_conv_wgrad_sweep) with sub-blocks of SUB_ROWS voxels instead of the table's schedule")
-    p.add_argument("--wgrad-sweep-lead", type=int, default=3, help="sub-blocks a workgroup may run ahead (with --wgrad-sweep)")
-    p.add_argument("--wgrad-sweep-polls", type=int, default=2000, help="poll limit of the pacing, 0 = unpaced (with --wgrad-sweep)")
+                   help="run wgrad as the sweep (fgx_conv_wgrad_sweep) with sub-blocks of SUB_ROWS voxels instead of the table's schedule")
+    p.add_argument("--wgrad-sweep-lead", type=int, default=3, help="sub-blocks a workgroup may run ahead when paced")
+    p.add_argument("--wgrad-sweep-polls", type=int, default=0, help="poll limit of the sweep's pacing, 0 = unpaced")
+    p.add_argument("--wgrad-block-major", type=int, default=0, metavar="BLOCK_ROWS",
+                   help="run wgrad with the block-major streaming kernel (fgx_conv_wgrad) on voxel blocks of BLOCK_ROWS rows instead of the table's schedule")
     p.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (used under rocprofv3)")
     p.add_argument("--cpu-rows", type=int, default=0, help="rows in the CPU baseline sample (0 = auto)")
     p.add_argument("--build-only", action="store_true", help="time only the neighbor-cache build")
@@ -133,17 +135,20 @@ def main():
     flex_gemm.ops.spconv.set_algorithm(Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
 
     names = {torch.float16: "f16", torch.bfloat16: "bf16", torch.float32: "f32"}
-    if args.wgrad_sweep:
-        from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    impl.WGRAD_SWEEP_LEAD, impl.WGRAD_SWEEP_MAX_POLLS = args.wgrad_sweep_lead, args.wgrad_sweep_polls
+    if args.wgrad_sweep or args.wgrad_block_major:
         table = nat.table_lookup
 
-        def with_sweep(pass_kind, *a):
+        def with_wgrad_kernel(pass_kind, *a):
             sc = table(pass_kind, *a)
             if pass_kind == nat.PASS_WGRAD:
-                sc.stream, sc.block_rows = 2, args.wgrad_sweep
+                if args.wgrad_sweep:
+                    sc.stream, sc.block_rows = 2, args.wgrad_sweep
+                else:
+                    sc.stream, sc.block_rows = 1, args.wgrad_block_major
             return sc
-        nat.table_lookup = with_sweep
-        impl.WGRAD_SWEEP_LEAD, impl.WGRAD_SWEEP_MAX_POLLS = args.wgrad_sweep_lead, args.wgrad_sweep_polls
+        nat.table_lookup = with_wgrad_kernel
     wl = make_workload(args.workload, dtype={v: k for k, v in names.items()}.get(args.dtype))
     dt = wl.dtype
     dname = names[dt]

@@ -22,7 +22,7 @@ const Entry kTable[] = {
     // pass dtype log2n  Ci    Co    {rows, cols, slab_bytes, splitk, block_rows, stream}
     {0, 2, 19, 128, 128, {256, 128, 128, 1, 0, 1}},
     {1, 2, 19, 128, 128, {256, 128, 128, 1, 0, 1}},
-    {2, 2, 19, 128, 128, {128, 128, 64, 1, 12288, 1}},
+    {2, 2, 19, 128, 128, {128, 128, 64, 1, 2048, 2}},
     {0, 2, 17, 256, 256, {256, 128, 128, 1, 0, 1}},
     {1, 2, 17, 256, 256, {256, 128, 128, 1, 0, 1}},
     {2, 2, 17, 256, 256, {128, 128, 64, 1, 12288, 1}},
@@ -61,6 +61,15 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
         // writes four partial products per voxel block (one per multiplying wavefront), so its blocks are four times
         // as long.
         out->stream = (es == 2 && n >= 2048) ? 1 : 0;
+        // A weight of one 64 x 64 or 128 x 128 tile (33 ... 128 channels on both sides): the sweep (stream = 2) --
+        // every workgroup keeps two accumulators over an eighth of the voxels, block_rows is its sub-block size.
+        // Measured 20 % to 30 % ahead of the block-major kernel from ten thousand voxels (C = 128: 0.051 against
+        // 0.067 ms) to 2.7 million (1.32 against 1.70 ms), for C = 64, 96, 128, coordinates in scan order or shuffled.
+        if (es == 2 && n >= 8192 && n <= ((size_t)1 << 24) && t >= 64 && Ci <= t && Co <= t && V <= 2 * (kCUs / 8)) {
+            out->stream = 2;
+            out->block_rows = 2048;
+            return;
+        }
         const int slices = (out->stream && t == 32) ? 4 : 1;
         const double per_block = 4.0 * V * (double)Co * (double)Ci * slices;
         size_t max_blocks = (size_t)(268435456.0 / per_block);

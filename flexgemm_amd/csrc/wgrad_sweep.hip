@@ -36,7 +36,7 @@ constexpr int kSwIdxSlots = 8;       // index ring: two slots per loader
 constexpr int kSwLoaders = 4;
 constexpr int kSwPairs = 64;         // pairs per step
 constexpr int kSwStepRing = 256;     // step-list entries held in LDS (four chunks of 64)
-constexpr int kSwMergeShift = 1;     // a workgroup changes units every 2^this sub-blocks (a change swaps the accumulators)
+constexpr int kSwTurnRows = 16384;   // a workgroup changes units about every so many voxels (a change swaps the accumulators)
 constexpr int kSwMaxSlots = 64;      // workgroups per XCD the pacing poll can look at (one lane each)
 constexpr int kSwMaxGroups = kXcds * kSwMaxSlots;
 constexpr unsigned kSwSpinMax = 1u << 20;   // looks at a progress word before a wavefront goes on regardless
@@ -87,9 +87,14 @@ __device__ __forceinline__ void progress_wait(const uint32_t* words, uint32_t ne
 // Plan: fine bounds, units (parts), per-workgroup step lists
 // ------------------------------------------------------------------------------------------------
 struct SweepUnit {
-    uint32_t v, p, P;       // offset, part index, parts of this offset in this XCD
+    // The 64-pair steps of offset v inside the XCD's voxels are numbered 0, 1, 2, ...; the offset is cut into P slices
+    // that take the steps in turn (step j belongs to slice j % P, P <= 64), and a unit owns the slices in `mask`.
+    // Units of one offset can so have any sizes, which is what evens out the workgroups' loads.
+    uint32_t v, P;
     uint32_t lo, hi;        // pair range of the offset inside the XCD's voxels
     uint32_t nsteps;
+    uint32_t mask_lo, mask_hi;
+    uint32_t pad;
 };
 struct SweepGroup {         // one workgroup
     uint32_t step_off, nsteps;
@@ -128,11 +133,24 @@ SweepLayout sweep_layout(size_t n, size_t n_pairs, int V, int sub_rows, int grou
     return L;
 }
 
-__device__ __forceinline__ uint32_t unit_steps(uint32_t cnt, uint32_t p, uint32_t P) {
-    const uint64_t first = (uint64_t)p * kSwPairs;
-    if (P == 0 || cnt <= first) return 0;
-    return (uint32_t)((cnt - first + (uint64_t)P * kSwPairs - 1) / ((uint64_t)P * kSwPairs));
+__device__ __forceinline__ uint64_t unit_mask(const SweepUnit& u) { return ((uint64_t)u.mask_hi << 32) | u.mask_lo; }
+// how many of the offset's steps 0 .. J-1 belong to the unit
+__device__ __forceinline__ uint32_t unit_count_below(const SweepUnit& u, uint32_t J) {
+    if (u.P == 0) return 0;
+    const uint32_t full = J / u.P, rem = J % u.P;
+    const uint64_t m = unit_mask(u);
+    const uint64_t low = rem ? (m & (~0ull >> (64 - rem))) : 0ull;
+    return full * (uint32_t)__popcll(m) + (uint32_t)__popcll(low);
 }
+// the offset-wide number of the unit's t-th step
+__device__ __forceinline__ uint32_t unit_step_at(const SweepUnit& u, uint32_t t) {
+    uint64_t m = unit_mask(u);
+    const uint32_t pc = (uint32_t)__popcll(m);
+    const uint32_t cycle = t / pc;
+    for (uint32_t r = t % pc; r > 0; --r) m &= m - 1;       // drop the r lowest slices
+    return cycle * u.P + (uint32_t)(__ffsll((long long)m) - 1);
+}
+__device__ __forceinline__ uint32_t offset_steps(uint32_t cnt) { return (cnt + kSwPairs - 1) / kSwPairs; }
 
 // One thread per XCD cuts its pair ranges into 2 * spx parts and pairs them up; thread 0 then lays out the step lists
 // and the per-offset lists of partial products.  A few thousand scalar operations in all.
@@ -141,7 +159,6 @@ __global__ void __launch_bounds__(256) sweep_units_kernel(const uint32_t* __rest
                                                          SweepUnit* __restrict__ units, SweepGroup* __restrict__ wg,
                                                          uint32_t* __restrict__ vcount, uint16_t* __restrict__ vlist) {
     const unsigned x = threadIdx.x;
-    const unsigned slots = 2 * spx;
     // pairs (all offsets) before every sub-block boundary, by all threads: the XCDs' ranges are cut from it
     __shared__ uint32_t cum[kSwCumMax + 1];
     const bool by_pairs = nsb <= kSwCumMax;
@@ -170,65 +187,94 @@ __global__ void __launch_bounds__(256) sweep_units_kernel(const uint32_t* __rest
             return lo_sb;
         };
         const unsigned sbA = boundary(x), sbB = boundary(x + 1);
-        uint32_t lo[kMaxV], cnt[kMaxV], P[kMaxV];
-        unsigned parts = 0;
+        // Every offset is cut into up to 64 slices that take its steps in turn.  The workgroups are filled one after
+        // the other to the average of what is left: the smallest remaining offset whole, topped up with slices of the
+        // largest one (or, when the smallest is larger than the average, a share of it alone) -- at most two units per
+        // workgroup, loads equal up to a slice.  A workgroup must retire offsets for good when as many remain as the
+        // workgroups after it can still take (two each): that keeps the scheme from running out of unit slots.
+        uint32_t lo[kMaxV], cnt[kMaxV], N[kMaxV], P[kMaxV];
+        uint64_t left[kMaxV];                       // slices not yet given out
+        float total = 0.f;
         for (int v = 0; v < V; ++v) {
             lo[v] = fine[(size_t)v * (nsb + 1) + sbA];
             cnt[v] = fine[(size_t)v * (nsb + 1) + sbB] - lo[v];
-            P[v] = cnt[v] ? 1u : 0u;
-            parts += P[v];
+            N[v] = offset_steps(cnt[v]);
+            P[v] = N[v] < 64u ? N[v] : 64u;
+            left[v] = P[v] ? (~0ull >> (64 - P[v])) : 0ull;
+            total += (float)N[v];
         }
-        // split the offset with the largest parts until every slot has one (never below one step per part)
-        while (parts > 0 && parts < slots) {
-            int best = -1;
-            float best_size = 0.f;
-            for (int v = 0; v < V; ++v) {
-                if (!P[v]) continue;
-                const float size = (float)cnt[v] / (float)P[v];
-                if (size > best_size) {
-                    best_size = size;
-                    best = v;
+        auto remaining = [&](int v) -> float { return (float)N[v] * (float)__popcll(left[v]) / (float)P[v]; };
+        // k of the remaining slices of offset v, evenly spread over them
+        auto take = [&](int v, unsigned k) -> uint64_t {
+            const unsigned have = (unsigned)__popcll(left[v]);
+            if (k >= have) {
+                const uint64_t all = left[v];
+                left[v] = 0;
+                return all;
+            }
+            uint64_t got = 0, m = left[v];
+            unsigned seen = 0, given = 0;
+            while (m) {
+                const uint64_t bit = m & (~m + 1);
+                m &= m - 1;
+                ++seen;
+                if ((uint64_t)seen * k / have > given) {       // the slices where k * seen / have steps up
+                    got |= bit;
+                    ++given;
                 }
             }
-            if (best < 0 || best_size <= (float)kSwPairs) break;
-            ++P[best];
-            ++parts;
-        }
-        // parts by descending size (insertion sort, stable in (offset, part) order)
-        uint16_t order_v[2 * kSwMaxSlots], order_p[2 * kSwMaxSlots];
-        float order_s[2 * kSwMaxSlots];
-        unsigned m = 0;
-        for (int v = 0; v < V; ++v)
-            for (uint32_t p = 0; p < P[v]; ++p) {
-                const float size = (float)cnt[v] / (float)P[v];
-                unsigned at = m;
-                while (at > 0 && order_s[at - 1] < size) {
-                    order_s[at] = order_s[at - 1];
-                    order_v[at] = order_v[at - 1];
-                    order_p[at] = order_p[at - 1];
-                    --at;
-                }
-                order_s[at] = size;
-                order_v[at] = (uint16_t)v;
-                order_p[at] = (uint16_t)p;
-                ++m;
-            }
-        // workgroup s: the s-th largest part and the s-th smallest
+            left[v] &= ~got;
+            return got;
+        };
+        auto make_unit = [&](int v, uint64_t mask) -> SweepUnit {
+            SweepUnit un{};
+            if (v < 0 || mask == 0) return un;
+            un.v = (uint32_t)v;
+            un.P = P[v];
+            un.lo = lo[v];
+            un.hi = lo[v] + cnt[v];
+            un.mask_lo = (uint32_t)mask;
+            un.mask_hi = (uint32_t)(mask >> 32);
+            un.nsteps = unit_count_below(un, N[v]);
+            return un;
+        };
         for (unsigned s = 0; s < spx; ++s) {
-            for (int u = 0; u < 2; ++u) {
-                const unsigned at = u == 0 ? s : slots - 1 - s;
-                SweepUnit un{};
-                if (at < m) {
-                    const unsigned v = order_v[at];
-                    un.v = v;
-                    un.p = order_p[at];
-                    un.P = P[v];
-                    un.lo = lo[v];
-                    un.hi = lo[v] + cnt[v];
-                    un.nsteps = unit_steps(cnt[v], un.p, un.P);
+            const unsigned after = spx - 1 - s;                 // workgroups after this one
+            const float want = total / (float)(spx - s);
+            int items = 0;                                      // offsets that still have slices
+            for (int v = 0; v < V; ++v) items += left[v] ? 1 : 0;
+            const int must_retire = items - 2 * (int)after;
+            int a = -1, b = -1;
+            for (int v = 0; v < V; ++v)
+                if (left[v] && (a < 0 || remaining(v) < remaining(a))) a = v;
+            uint64_t mask_a = 0, mask_b = 0;
+            if (a >= 0) {
+                const float rem_a = remaining(a);
+                if (rem_a > want && must_retire < 1) {          // a share of the smallest offset fills the workgroup
+                    const float per = (float)N[a] / (float)P[a];
+                    unsigned k = (unsigned)(want / per + 0.5f);
+                    mask_a = take(a, k ? k : 1u);
+                } else {
+                    mask_a = take(a, 64u);
+                    // top up: from the largest other offset, or (when offsets must go) the smallest one whole
+                    for (int v = 0; v < V; ++v) {
+                        if (!left[v] || v == a) continue;
+                        if (b < 0 || (must_retire >= 2 ? remaining(v) < remaining(b) : remaining(v) > remaining(b))) b = v;
+                    }
+                    if (b >= 0) {
+                        const float need = want - rem_a, per = (float)N[b] / (float)P[b];
+                        if (must_retire >= 2) {
+                            mask_b = take(b, 64u);
+                        } else if (need > 0.5f * per) {
+                            mask_b = take(b, (unsigned)(need / per + 0.5f));
+                        }
+                    }
                 }
-                units[((size_t)x * spx + s) * 2 + u] = un;
             }
+            const SweepUnit u0 = make_unit(a, mask_a), u1 = make_unit(b, mask_b);
+            total -= (float)(u0.nsteps + u1.nsteps);
+            units[((size_t)x * spx + s) * 2] = u0;
+            units[((size_t)x * spx + s) * 2 + 1] = u1;
             wg[(size_t)x * spx + s].sb0 = sbA;
         }
     }
@@ -260,10 +306,11 @@ __global__ void __launch_bounds__(256) sweep_units_kernel(const uint32_t* __rest
 
 // number of steps of unit u whose first pair lies below `bound`
 __device__ __forceinline__ uint32_t steps_below(const SweepUnit& u, uint32_t bound) {
-    const uint64_t first = (uint64_t)u.lo + (uint64_t)u.p * kSwPairs;
-    if (u.nsteps == 0 || (uint64_t)bound <= first) return 0;
-    const uint64_t c = ((uint64_t)bound - first + (uint64_t)u.P * kSwPairs - 1) / ((uint64_t)u.P * kSwPairs);
-    return c < u.nsteps ? (uint32_t)c : u.nsteps;
+    if (u.nsteps == 0 || bound <= u.lo) return 0;
+    const uint32_t all = offset_steps(u.hi - u.lo);
+    uint32_t J = (bound - u.lo + kSwPairs - 1) / kSwPairs;       // steps of the offset that start below the bound
+    if (J > all) J = all;
+    return unit_count_below(u, J);
 }
 
 // The merged step list of one workgroup per block: its two units' steps ordered by the group of sub-blocks their first
@@ -272,7 +319,7 @@ __device__ __forceinline__ uint32_t steps_below(const SweepUnit& u, uint32_t bou
 __global__ void __launch_bounds__(256) sweep_steps_kernel(const uint32_t* __restrict__ fine, unsigned nsb,
                                                           const SweepUnit* __restrict__ units,
                                                           const SweepGroup* __restrict__ wg, uint32_t* __restrict__ steps_k,
-                                                          uint32_t* __restrict__ steps_m, size_t step_cap) {
+                                                          uint32_t* __restrict__ steps_m, size_t step_cap, unsigned turn_shift) {
     const unsigned g = blockIdx.x;
     const SweepGroup grp = wg[g];
     const SweepUnit u0 = units[(size_t)g * 2], u1 = units[(size_t)g * 2 + 1];
@@ -283,7 +330,7 @@ __global__ void __launch_bounds__(256) sweep_steps_kernel(const uint32_t* __rest
         const uint32_t* mine = fine + (size_t)me.v * (nsb + 1);
         const uint32_t* theirs = fine + (size_t)other.v * (nsb + 1);
         for (uint32_t j = threadIdx.x; j < me.nsteps; j += 256) {
-            const uint32_t k = me.lo + (me.p + j * me.P) * kSwPairs;
+            const uint32_t k = me.lo + unit_step_at(me, j) * kSwPairs;
             const uint32_t left = me.hi - k;
             // sub-block of pair k: the last s with mine[s] <= k (pairs of the XCD start at sub-block sbA)
             unsigned lo = sbA, hi = nsb;            // invariant: mine[lo] <= k, answer in [lo, hi)
@@ -293,10 +340,10 @@ __global__ void __launch_bounds__(256) sweep_steps_kernel(const uint32_t* __rest
                 else hi = mid;
             }
             const unsigned sb = lo;
-            // the two units take turns by groups of 2^kSwMergeShift sub-blocks: the other unit's steps in earlier groups
+            // the two units take turns by groups of 2^turn_shift sub-blocks: the other unit's steps in earlier groups
             // and, for unit 1, in this one (unit 0 goes first)
-            const unsigned grp_first = sbA + (((sb - sbA) >> kSwMergeShift) << kSwMergeShift);
-            const unsigned grp_end = grp_first + (1u << kSwMergeShift) < nsb ? grp_first + (1u << kSwMergeShift) : nsb;
+            const unsigned grp_first = sbA + (((sb - sbA) >> turn_shift) << turn_shift);
+            const unsigned grp_end = grp_first + (1u << turn_shift) < nsb ? grp_first + (1u << turn_shift) : nsb;
             const uint32_t before = u == 0 ? steps_below(other, theirs[grp_first]) : steps_below(other, theirs[grp_end]);
             const size_t at = (size_t)grp.step_off + j + before;
             if (at < step_cap) {
@@ -451,43 +498,61 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
             landed[lane] = 0u;                      // (landed and consumed are adjacent)
         }
         __syncthreads();                            // (1) the first two chunks of the step list are in LDS, progress words zero
-        // Loader lw owns ring stage lw and the steps lw, lw + S, lw + 2S, ...: it enqueues all of a step's rows, prepares
-        // the next step's addresses while they are on their way, and announces the step when they have landed.  The
-        // four loaders take turns on the address path, and the per-step scalar work and LDS round trips of the
-        // preparation happen once per step and loader beside the load latency instead of in front of it.
+        // Loader lw owns ring stage lw and the steps lw, lw + S, lw + 2S, ...: it enqueues all of a step's rows, turns
+        // the next step's indices into addresses while they are on their way, and announces the step when they have
+        // landed.  The four loaders take turns on the address path, and the per-step scalar work happens once per step
+        // and loader, beside the load latency instead of in front of it.
+        //
+        // Which pair goes to which of a stage's P row slots is free as long as both operands agree (the products are
+        // summed over the slots).  Slot i * RPI + sub (load instruction i, row `sub` of its RPI rows) takes pair
+        // sub * NA + i of the step: a lane then needs NA consecutive entries of each pair list, which it fetches
+        // straight into registers with 16-byte loads, a round ahead -- no index ring in LDS, no LDS round trip.
         constexpr int NA = P / C::RPI_A, NB = P / C::RPI_B;     // load instructions per operand and step
-        static_assert(NA + NB + 6 < 64, "outstanding loads exceed the vmcnt range");
-        const int a_sub = lane / C::CH_A, b_sub = lane / C::CH_B;          // row inside a load instruction
+        static_assert(NA == NB && NA % 4 == 0, "one slot order for both operands, indices in 16-byte pieces");
+        static_assert(NA + NB + NA / 2 + 4 < 64, "outstanding loads exceed the vmcnt range");
+        const int sub = lane / C::CH_A;                                    // row inside a load instruction
         // byte column inside the tile, swizzle applied (the key depends on row & 3 alone, an instruction covers 4 or 8 rows)
-        const uint32_t a_chb = (uint32_t)(((lane % C::CH_A) ^ C::key_a(a_sub)) * 16);
-        const uint32_t b_chb = (uint32_t)(((lane % C::CH_B) ^ C::key_b(b_sub)) * 16);
+        const uint32_t a_chb = (uint32_t)(((lane % C::CH_A) ^ C::key_a(sub)) * 16);
+        const uint32_t b_chb = (uint32_t)(((lane % C::CH_B) ^ C::key_b(sub)) * 16);
         unsigned char* stage = ring + lw * C::STAGE_BYTES;
-        uint32_t* my_idx = idx_ring + lw * 2 * (2 * P);                    // two index slots per loader
-        auto issue_idx = [&](unsigned k) {         // index columns of step k into slot (k / S) & 1
-            if (k >= nsteps) return;
-            const uint32_t first = step_k[k & (kSwStepRing - 1)];
-            uint32_t* dst = my_idx + ((k / S) & 1) * (2 * P);
-            uint32_t* dst_i = dst + P;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(sigo_rs, FGX_LDS_PTR(dst), 4, (first + (uint32_t)lane) * 4u, 0, 0, 0);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(sigi_rs, FGX_LDS_PTR(dst_i), 4, (first + (uint32_t)lane) * 4u, 0, 0, 0);
+        struct Indices {
+            u32x4 o[NA / 4], i[NA / 4];
+        };
+        auto fetch_idx = [&](unsigned k, Indices& ix) {     // this lane's pair-list entries of step k (zeros past the lists)
+            const uint32_t first = k < nsteps ? step_k[k & (kSwStepRing - 1)] : n_pairs;
+            const uint32_t at = (first + (uint32_t)(sub * NA)) * 4u;
+#pragma unroll
+            for (int q = 0; q < NA / 4; ++q) {
+                ix.o[q] = __builtin_amdgcn_raw_buffer_load_b128(sigo_rs, (int)(at + q * 16u), 0, 0);
+                ix.i[q] = __builtin_amdgcn_raw_buffer_load_b128(sigi_rs, (int)(at + q * 16u), 0, 0);
+            }
         };
         uint32_t va[NA], vb[NB];
-        auto prep_rows = [&](unsigned k) {         // buffer offsets of step k's rows (rows and row sizes fit 24 bits)
+        auto prep_rows = [&](unsigned k, const Indices& ix) {     // buffer offsets of step k's rows (rows and row sizes fit 24 bits)
             if (k >= nsteps) return;
-            const uint32_t* slot_p = my_idx + ((k / S) & 1) * (2 * P);
             const uint32_t left = step_m[k & (kSwStepRing - 1)] & 127u;                // pairs in this step
             const bool ragged = left < (uint32_t)P || (uint32_t)(BM * ES) > rowb_o || (uint32_t)(BN * ES) > rowb_i;   // uniform
 #pragma unroll
-            for (int i = 0; i < NA; ++i) va[i] = __umul24(slot_p[i * C::RPI_A + a_sub], rowb_o) + a_chb;
-#pragma unroll
-            for (int i = 0; i < NB; ++i) vb[i] = __umul24(slot_p[P + i * C::RPI_B + b_sub], rowb_i) + b_chb;
+            for (int q = 0; q < NA / 4; ++q) {
+                // (whole vectors into scalars first: indexing a vector element inside a cast has been miscompiled)
+                const uint32_t o0 = ix.o[q][0], o1 = ix.o[q][1], o2 = ix.o[q][2], o3 = ix.o[q][3];
+                const uint32_t i0 = ix.i[q][0], i1 = ix.i[q][1], i2 = ix.i[q][2], i3 = ix.i[q][3];
+                va[q * 4 + 0] = __umul24(o0, rowb_o) + a_chb;
+                va[q * 4 + 1] = __umul24(o1, rowb_o) + a_chb;
+                va[q * 4 + 2] = __umul24(o2, rowb_o) + a_chb;
+                va[q * 4 + 3] = __umul24(o3, rowb_o) + a_chb;
+                vb[q * 4 + 0] = __umul24(i0, rowb_i) + b_chb;
+                vb[q * 4 + 1] = __umul24(i1, rowb_i) + b_chb;
+                vb[q * 4 + 2] = __umul24(i2, rowb_i) + b_chb;
+                vb[q * 4 + 3] = __umul24(i3, rowb_i) + b_chb;
+            }
             if (ragged) {
 #pragma unroll
-                for (int i = 0; i < NA; ++i)
-                    va[i] = ((uint32_t)(i * C::RPI_A + a_sub) < left && a_chb < rowb_o) ? va[i] : kOobOffset;
-#pragma unroll
-                for (int i = 0; i < NB; ++i)
-                    vb[i] = ((uint32_t)(i * C::RPI_B + b_sub) < left && b_chb < rowb_i) ? vb[i] : kOobOffset;
+                for (int i = 0; i < NA; ++i) {
+                    const bool live = (uint32_t)(sub * NA + i) < left;
+                    va[i] = (live && a_chb < rowb_o) ? va[i] : kOobOffset;
+                    vb[i] = (live && b_chb < rowb_i) ? vb[i] : kOobOffset;
+                }
             }
         };
         auto fire_rows = [&]() {
@@ -503,22 +568,28 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(feats_rs, FGX_LDS_PTR(stage_b + i * 1024), 16, vo, 0, 0, 0);
             }
         };
-
-        issue_idx((unsigned)lw);
-        issue_idx((unsigned)lw + S);
-        wait_vmcnt<0>();
-        __syncthreads();                            // (2)
-        prep_rows((unsigned)lw);
+        // one round: step k's rows are enqueued, the entries of step k + 2S requested, step k + S prepared from the
+        // entries requested a round ago, and step k announced
         uint32_t known_consumed = 0;
-        for (unsigned k = (unsigned)lw; k < nsteps; k += S) {
+        auto round = [&](unsigned k, const Indices& ready, Indices& coming) {
             if (k >= (unsigned)S) progress_wait(consumed, k - S + 1u, known_consumed);   // every multiplier has read step k - S
             fire_rows();
             // loader 0 also keeps the step list: the chunk after next, whose quarter of the ring was read 128+ steps ago
             if (lw == 0 && (k & 63u) == 0u) load_chunk(k / 64 + 2);
-            issue_idx(k + 2 * S);
-            prep_rows(k + S);                       // its index columns landed a round ago
+            fetch_idx(k + 2 * S, coming);
+            prep_rows(k + S, ready);
             wait_vmcnt<0>();
             progress_store(landed + lw, k / S + 1u);
+        };
+
+        __syncthreads();                            // (2)
+        Indices ix0, ix1;
+        fetch_idx((unsigned)lw, ix0);
+        fetch_idx((unsigned)lw + S, ix1);
+        prep_rows((unsigned)lw, ix0);
+        for (unsigned k = (unsigned)lw; k < nsteps; k += 2 * S) {
+            round(k, ix1, ix0);
+            if (k + S < nsteps) round(k + S, ix0, ix1);
         }
         wait_vmcnt<0>();
         return;
@@ -922,8 +993,10 @@ int fgx_wgrad_sweep_plan(const uint32_t* sig_o, const uint32_t* seg_host, size_t
     sweep_units_kernel<<<1, 256, 0, s>>>(fine, V, L.nsb, L.spx, (SweepUnit*)(p + L.units), (SweepGroup*)(p + L.wg),
                                         (uint32_t*)(p + L.vcount), (uint16_t*)(p + L.vlist));
     FGX_CHECK_LAUNCH("fgx_wgrad_sweep_plan(units)");
+    unsigned turn_shift = 0;
+    while (turn_shift < 16 && ((size_t)sub_rows << turn_shift) < (size_t)kSwTurnRows) ++turn_shift;
     sweep_steps_kernel<<<L.groups, 256, 0, s>>>(fine, L.nsb, (const SweepUnit*)(p + L.units), (const SweepGroup*)(p + L.wg),
-                                                (uint32_t*)(p + L.steps_k), (uint32_t*)(p + L.steps_m), L.step_cap);
+                                                (uint32_t*)(p + L.steps_k), (uint32_t*)(p + L.steps_m), L.step_cap, turn_shift);
     FGX_CHECK_LAUNCH("fgx_wgrad_sweep_plan(steps)");
     return FGX_OK;
 }

@@ -515,9 +515,10 @@ def _stream_fits(n: int, n_src: int, row_bytes: int) -> bool:
 
 
 # pacing of the wgrad sweep: sub-blocks a workgroup may run ahead of the slowest one of its XCD, and the looks at the
-# others' progress after which it stops waiting (0 = no pacing)
+# others' progress after which it stops waiting (0 = no pacing, the default: the workgroups of an XCD stay close enough
+# together by themselves, and waiting costs more time than the L2 misses it saves)
 WGRAD_SWEEP_LEAD = 3
-WGRAD_SWEEP_MAX_POLLS = 2000
+WGRAD_SWEEP_MAX_POLLS = 0
 
 
 def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int, with_bias: bool = False, bias_offset: int = -1):
@@ -543,6 +544,9 @@ def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int, with_b
     gb = torch.empty((cop,), dtype=dt, device=dev) if with_bias else None
     L = nat.lib()
     code = nat.DTYPE_CODE[dt]
+    if sched.stream == 2 and (n > (1 << 24) or n_in > (1 << 24)):
+        # the sweep multiplies row numbers with 24-bit multiplies: very long operands take the block-major kernel
+        sched.stream, sched.block_rows = 1, 12288
     if sched.stream == 2 and seg_host[-1] > 0 and n > 0:
         plan = cache._wgrad_sweep_plan(sched.block_rows)
         with torch.cuda.device(dev):

@@ -43,8 +43,17 @@ def test_host_only_entry_points(library):
     assert s.tile_rows in (128, 256) and s.tile_cols == 128 and s.splitk == 1 and s.slab_bytes in (64, 128)
     # the persistent streaming kernel walks 256-row tiles; rows of 128 bytes or more use 128-byte K-slabs
     assert (s.stream, s.tile_rows, s.slab_bytes) in ((1, 256, 128), (0, s.tile_rows, s.slab_bytes))
+    # a weight of one 128 x 128 tile: the sweep (stream 2, block_rows = its sub-block size)
     s = nat.table_lookup(nat.PASS_WGRAD, torch.float16, 669288, 128, 128, 27)
-    assert s.block_rows >= 1024 and s.stream in (0, 1)
+    assert s.block_rows >= 1024 and s.stream == 2 and (s.tile_rows, s.tile_cols) == (128, 128)
+    s = nat.table_lookup(nat.PASS_WGRAD, torch.bfloat16, 40000, 48, 64, 27)
+    assert s.stream == 2 and (s.tile_rows, s.tile_cols) == (64, 64)
+    # ... not for several tiles, 32 x 32 tiles, few voxels, more than 2^24 of them, or fp32
+    assert nat.table_lookup(nat.PASS_WGRAD, torch.float16, 669288, 256, 128, 27).stream == 1
+    assert nat.table_lookup(nat.PASS_WGRAD, torch.float16, 669288, 32, 32, 27).stream == 1
+    assert nat.table_lookup(nat.PASS_WGRAD, torch.float16, 4000, 128, 128, 27).stream == 1
+    assert nat.table_lookup(nat.PASS_WGRAD, torch.float16, (1 << 24) + 1, 128, 128, 27).stream == 1
+    assert nat.table_lookup(nat.PASS_WGRAD, torch.float32, 669288, 128, 128, 27).stream == 0
     s = nat.table_lookup(nat.PASS_FWD, torch.float32, 100, 16, 16, 27)
     assert s.tile_rows in (32, 64, 128) and s.tile_cols == 32 and s.splitk >= 1 and s.stream == 0
     # rule (no table entry): big problems stream, small ones and rows below 64 bytes do not
@@ -184,6 +193,9 @@ def test_wgrad_block_rule_keeps_its_promises(library):
             s = nat.table_lookup(nat.PASS_WGRAD, torch.float16, n, c, c, 27)
             rows = s.block_rows
             assert rows >= 1024 and rows % 1024 == 0, (n, c, rows)
+            if s.stream == 2:           # the sweep: block_rows is its sub-block size, it has no voxel blocks
+                assert c in (64, 128) and n >= 8192, (n, c)
+                continue
             blocks = -(-n // rows)
             slices = 4 if (s.stream and s.tile_rows == 32) else 1
             if blocks > 1:
