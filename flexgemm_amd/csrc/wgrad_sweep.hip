@@ -152,15 +152,43 @@ __device__ __forceinline__ uint32_t unit_step_at(const SweepUnit& u, uint32_t t)
 }
 __device__ __forceinline__ uint32_t offset_steps(uint32_t cnt) { return (cnt + kSwPairs - 1) / kSwPairs; }
 
-// One thread per XCD cuts its pair ranges into 2 * spx parts and pairs them up; thread 0 then lays out the step lists
-// and the per-offset lists of partial products.  A few thousand scalar operations in all.
+// One wavefront per XCD cuts its pair ranges into units, lane v keeping the state of offset v; then the step-list
+// offsets and the per-offset lists of partial products are laid out.
 constexpr unsigned kSwCumMax = 4096;     // sub-blocks whose running pair counts fit the units kernel's LDS
-__global__ void __launch_bounds__(256) sweep_units_kernel(const uint32_t* __restrict__ fine, int V, unsigned nsb, unsigned spx,
-                                                         SweepUnit* __restrict__ units, SweepGroup* __restrict__ wg,
-                                                         uint32_t* __restrict__ vcount, uint16_t* __restrict__ vlist) {
+
+// k of the slices in `have_mask`, evenly spread over them (all lanes: lane i decides slice i)
+__device__ __forceinline__ uint64_t spread_take(uint64_t have_mask, unsigned k, unsigned lane) {
+    const unsigned have = (unsigned)__popcll(have_mask);
+    if (k >= have) return have_mask;
+    const bool mine = (have_mask >> lane) & 1ull;
+    const unsigned rank = (unsigned)__popcll(have_mask & ((1ull << lane) - 1ull));      // slices of the mask below this one
+    const bool taken = mine && ((rank + 1u) * k / have > rank * k / have);              // where k * rank / have steps up
+    return __ballot(taken);
+}
+// lane holding the smallest (largest) key among the lanes with `live`, lowest lane on ties; -1 if none
+__device__ __forceinline__ int wave_arg(bool live, float key, unsigned lane, bool want_max) {
+    const uint32_t bits = __builtin_bit_cast(uint32_t, key);                              // keys are >= 0: bits order like values
+    unsigned long long k = want_max ? (((unsigned long long)bits << 8) | (255u - lane))
+                                    : (((unsigned long long)(~bits) << 8) | (255u - lane));
+    if (!live) k = 0ull;
+#pragma unroll
+    for (int sh = 32; sh > 0; sh >>= 1) {
+        const unsigned long long o = __shfl_xor(k, sh, 64);
+        k = o > k ? o : k;
+    }
+    return k == 0ull ? -1 : (int)(255u - (unsigned)(k & 255u));
+}
+
+__global__ void __launch_bounds__(64 * kXcds) sweep_units_kernel(const uint32_t* __restrict__ fine, int V, unsigned nsb, unsigned spx,
+                                                                SweepUnit* __restrict__ units, SweepGroup* __restrict__ wg,
+                                                                uint32_t* __restrict__ vcount, uint16_t* __restrict__ vlist) {
     const unsigned x = threadIdx.x;
     // pairs (all offsets) before every sub-block boundary, by all threads: the XCDs' ranges are cut from it
     __shared__ uint32_t cum[kSwCumMax + 1];
+    // what the layout pass below needs of every unit (steps, offset), kept out of global memory
+    __shared__ uint32_t sh_steps[kSwMaxGroups * 2];
+    __shared__ uint8_t sh_v[kSwMaxGroups * 2];
+    __shared__ uint32_t sh_vcount[kMaxV];
     const bool by_pairs = nsb <= kSwCumMax;
     if (by_pairs) {
         for (unsigned sb = x; sb <= nsb; sb += blockDim.x) {
@@ -170,14 +198,15 @@ __global__ void __launch_bounds__(256) sweep_units_kernel(const uint32_t* __rest
         }
     }
     __syncthreads();
-    if (x < (unsigned)kXcds) {
-        // XCD x takes the sub-blocks [sbA, sbB): boundaries where the running pair count (all offsets) passes x / 8 of
-        // the total, so that the XCDs get equal work rather than equal voxel counts
-        auto boundary = [&](unsigned xc) -> unsigned {
-            if (xc == 0) return 0u;
-            if (xc >= (unsigned)kXcds) return nsb;
-            if (!by_pairs) return (unsigned)((uint64_t)xc * nsb / kXcds);      // (very many sub-blocks: equal voxel counts)
-            const uint64_t want = (uint64_t)cum[nsb] * xc / kXcds;
+    {
+        const unsigned xc = x >> 6, lane = x & 63u;         // wavefront xc plans XCD xc
+        // XCD xc takes the sub-blocks [sbA, sbB): boundaries where the running pair count (all offsets) passes xc / 8
+        // of the total, so that the XCDs get equal work rather than equal voxel counts
+        auto boundary = [&](unsigned q) -> unsigned {
+            if (q == 0) return 0u;
+            if (q >= (unsigned)kXcds) return nsb;
+            if (!by_pairs) return (unsigned)((uint64_t)q * nsb / kXcds);      // (very many sub-blocks: equal voxel counts)
+            const uint64_t want = (uint64_t)cum[nsb] * q / kXcds;
             unsigned lo_sb = 0, hi_sb = nsb;            // first sub-block boundary with at least `want` pairs before it
             while (lo_sb < hi_sb) {
                 const unsigned mid = (lo_sb + hi_sb) >> 1;
@@ -186,121 +215,117 @@ __global__ void __launch_bounds__(256) sweep_units_kernel(const uint32_t* __rest
             }
             return lo_sb;
         };
-        const unsigned sbA = boundary(x), sbB = boundary(x + 1);
+        const unsigned sbA = boundary(xc), sbB = boundary(xc + 1);
         // Every offset is cut into up to 64 slices that take its steps in turn.  The workgroups are filled one after
         // the other to the average of what is left: the smallest remaining offset whole, topped up with slices of the
         // largest one (or, when the smallest is larger than the average, a share of it alone) -- at most two units per
         // workgroup, loads equal up to a slice.  A workgroup must retire offsets for good when as many remain as the
         // workgroups after it can still take (two each): that keeps the scheme from running out of unit slots.
-        uint32_t lo[kMaxV], cnt[kMaxV], N[kMaxV], P[kMaxV];
-        uint64_t left[kMaxV];                       // slices not yet given out
-        float total = 0.f;
-        for (int v = 0; v < V; ++v) {
-            lo[v] = fine[(size_t)v * (nsb + 1) + sbA];
-            cnt[v] = fine[(size_t)v * (nsb + 1) + sbB] - lo[v];
-            N[v] = offset_steps(cnt[v]);
-            P[v] = N[v] < 64u ? N[v] : 64u;
-            left[v] = P[v] ? (~0ull >> (64 - P[v])) : 0ull;
-            total += (float)N[v];
+        uint32_t lo = 0, cnt = 0, N = 0, P = 0;             // this lane's offset
+        uint64_t left = 0;                                  // its slices not yet given out
+        float per = 0.f;                                    // steps per slice
+        if (lane < (unsigned)V) {
+            lo = fine[(size_t)lane * (nsb + 1) + sbA];
+            cnt = fine[(size_t)lane * (nsb + 1) + sbB] - lo;
+            N = offset_steps(cnt);
+            P = N < 64u ? N : 64u;
+            left = P ? (~0ull >> (64 - P)) : 0ull;
+            per = P ? (float)N / (float)P : 0.f;
         }
-        auto remaining = [&](int v) -> float { return (float)N[v] * (float)__popcll(left[v]) / (float)P[v]; };
-        // k of the remaining slices of offset v, evenly spread over them
-        auto take = [&](int v, unsigned k) -> uint64_t {
-            const unsigned have = (unsigned)__popcll(left[v]);
-            if (k >= have) {
-                const uint64_t all = left[v];
-                left[v] = 0;
-                return all;
-            }
-            uint64_t got = 0, m = left[v];
-            unsigned seen = 0, given = 0;
-            while (m) {
-                const uint64_t bit = m & (~m + 1);
-                m &= m - 1;
-                ++seen;
-                if ((uint64_t)seen * k / have > given) {       // the slices where k * seen / have steps up
-                    got |= bit;
-                    ++given;
-                }
-            }
-            left[v] &= ~got;
-            return got;
-        };
-        auto make_unit = [&](int v, uint64_t mask) -> SweepUnit {
-            SweepUnit un{};
-            if (v < 0 || mask == 0) return un;
-            un.v = (uint32_t)v;
-            un.P = P[v];
-            un.lo = lo[v];
-            un.hi = lo[v] + cnt[v];
-            un.mask_lo = (uint32_t)mask;
-            un.mask_hi = (uint32_t)(mask >> 32);
-            un.nsteps = unit_count_below(un, N[v]);
-            return un;
-        };
+        float total = (float)N;
+#pragma unroll
+        for (int sh = 32; sh > 0; sh >>= 1) total += __shfl_xor(total, sh, 64);
         for (unsigned s = 0; s < spx; ++s) {
-            const unsigned after = spx - 1 - s;                 // workgroups after this one
+            const int after = (int)(spx - 1 - s);               // workgroups after this one
             const float want = total / (float)(spx - s);
-            int items = 0;                                      // offsets that still have slices
-            for (int v = 0; v < V; ++v) items += left[v] ? 1 : 0;
-            const int must_retire = items - 2 * (int)after;
-            int a = -1, b = -1;
-            for (int v = 0; v < V; ++v)
-                if (left[v] && (a < 0 || remaining(v) < remaining(a))) a = v;
+            const int items = (int)__popcll(__ballot(left != 0));
+            const int must_retire = items - 2 * after;
+            const float rem = per * (float)__popcll(left);
+            const int a = wave_arg(left != 0, rem, lane, false);
+            int b = -1;
             uint64_t mask_a = 0, mask_b = 0;
-            if (a >= 0) {
-                const float rem_a = remaining(a);
-                if (rem_a > want && must_retire < 1) {          // a share of the smallest offset fills the workgroup
-                    const float per = (float)N[a] / (float)P[a];
-                    unsigned k = (unsigned)(want / per + 0.5f);
-                    mask_a = take(a, k ? k : 1u);
+            if (a >= 0) {                                       // (uniform)
+                const float rem_a = __shfl(rem, a, 64), per_a = __shfl(per, a, 64);
+                const uint64_t left_a = __shfl((unsigned long long)left, a, 64);
+                const bool share = rem_a > want && must_retire < 1;     // a share of the smallest offset fills the workgroup
+                if (share) {
+                    const unsigned k = (unsigned)(want / per_a + 0.5f);
+                    mask_a = spread_take(left_a, k ? k : 1u, lane);
                 } else {
-                    mask_a = take(a, 64u);
+                    mask_a = left_a;
+                }
+                if ((int)lane == a) left &= ~mask_a;
+                if (!share) {
                     // top up: from the largest other offset, or (when offsets must go) the smallest one whole
-                    for (int v = 0; v < V; ++v) {
-                        if (!left[v] || v == a) continue;
-                        if (b < 0 || (must_retire >= 2 ? remaining(v) < remaining(b) : remaining(v) > remaining(b))) b = v;
-                    }
+                    b = wave_arg(left != 0 && (int)lane != a, rem, lane, must_retire < 2);
                     if (b >= 0) {
-                        const float need = want - rem_a, per = (float)N[b] / (float)P[b];
-                        if (must_retire >= 2) {
-                            mask_b = take(b, 64u);
-                        } else if (need > 0.5f * per) {
-                            mask_b = take(b, (unsigned)(need / per + 0.5f));
-                        }
+                        const float per_b = __shfl(per, b, 64), need = want - rem_a;
+                        const uint64_t left_b = __shfl((unsigned long long)left, b, 64);
+                        if (must_retire >= 2) mask_b = left_b;
+                        else if (need > 0.5f * per_b) mask_b = spread_take(left_b, (unsigned)(need / per_b + 0.5f), lane);
+                        if ((int)lane == b) left &= ~mask_b;
                     }
                 }
             }
-            const SweepUnit u0 = make_unit(a, mask_a), u1 = make_unit(b, mask_b);
-            total -= (float)(u0.nsteps + u1.nsteps);
-            units[((size_t)x * spx + s) * 2] = u0;
-            units[((size_t)x * spx + s) * 2 + 1] = u1;
-            wg[(size_t)x * spx + s].sb0 = sbA;
+            // lane a writes the first unit, lane b the second (lane 0 an empty one where there is none)
+            uint32_t my_steps = 0;
+            for (int u = 0; u < 2; ++u) {
+                const int who = u == 0 ? a : b;
+                const uint64_t mask = u == 0 ? mask_a : mask_b;
+                const bool have = who >= 0 && mask != 0;
+                if ((int)lane == (have ? who : 0)) {
+                    SweepUnit un{};
+                    if (have) {
+                        un.v = lane;
+                        un.P = P;
+                        un.lo = lo;
+                        un.hi = lo + cnt;
+                        un.mask_lo = (uint32_t)mask;
+                        un.mask_hi = (uint32_t)(mask >> 32);
+                        un.nsteps = unit_count_below(un, N);
+                        my_steps += un.nsteps;
+                    }
+                    const unsigned q = (xc * spx + s) * 2 + (unsigned)u;
+                    units[q] = un;
+                    sh_steps[q] = un.nsteps;
+                    sh_v[q] = (uint8_t)un.v;
+                }
+            }
+            float given = (float)my_steps;
+#pragma unroll
+            for (int sh = 32; sh > 0; sh >>= 1) given += __shfl_xor(given, sh, 64);
+            total -= given;
+            if (lane == 0) wg[(size_t)xc * spx + s].sb0 = sbA;
         }
     }
     __syncthreads();
+    // step-list offsets: a running sum over the workgroups (thread 0, from LDS); the rest in parallel
+    __shared__ uint32_t sh_off[kSwMaxGroups + 1];
     if (x == 0) {
         uint32_t off = 0;
-        for (unsigned xc = 0; xc < (unsigned)kXcds; ++xc) {
-            uint32_t active = 0;
-            for (unsigned s = 0; s < spx; ++s) {
-                const size_t g = (size_t)xc * spx + s;
-                const uint32_t ns = units[g * 2].nsteps + units[g * 2 + 1].nsteps;
-                wg[g].step_off = off;
-                wg[g].nsteps = ns;
-                off += ns;
-                active += ns ? 1u : 0u;
-            }
-            for (unsigned s = 0; s < spx; ++s) wg[(size_t)xc * spx + s].active = active;
+        for (unsigned g = 0; g < (unsigned)kXcds * spx; ++g) {
+            sh_off[g] = off;
+            off += sh_steps[g * 2] + sh_steps[g * 2 + 1];
         }
-        for (int v = 0; v < V; ++v) vcount[v] = 0;
-        const unsigned total_units = kXcds * spx * 2;
-        for (unsigned q = 0; q < total_units; ++q) {
-            if (!units[q].nsteps) continue;
-            const uint32_t v = units[q].v;
-            vlist[(size_t)v * total_units + vcount[v]] = (uint16_t)q;
-            ++vcount[v];
-        }
+    }
+    if (x < (unsigned)kMaxV) sh_vcount[x] = 0;
+    __syncthreads();
+    for (unsigned g = x; g < (unsigned)kXcds * spx; g += blockDim.x) {
+        const unsigned xc = g / spx;
+        uint32_t active = 0;
+        for (unsigned s = 0; s < spx; ++s) active += (sh_steps[(xc * spx + s) * 2] + sh_steps[(xc * spx + s) * 2 + 1]) ? 1u : 0u;
+        wg[g].step_off = sh_off[g];
+        wg[g].nsteps = sh_steps[g * 2] + sh_steps[g * 2 + 1];
+        wg[g].active = active;
+    }
+    // the partial products of every offset, in ascending unit order (the reduction adds them in this order): thread v
+    // collects offset v's
+    const unsigned total_units = kXcds * spx * 2;
+    if (x < (unsigned)V) {
+        uint32_t c = 0;
+        for (unsigned q = 0; q < total_units; ++q)
+            if (sh_steps[q] && sh_v[q] == x) vlist[(size_t)x * total_units + c++] = (uint16_t)q;
+        vcount[x] = c;
     }
 }
 
@@ -990,7 +1015,7 @@ int fgx_wgrad_sweep_plan(const uint32_t* sig_o, const uint32_t* seg_host, size_t
     phase_mark("wgrad sweep plan", s);
     block_bounds_kernel<<<cdiv((size_t)V * (L.nsb + 1), 256), 256, 0, s>>>(sig_o, tab, V, L.nsb, (unsigned)sub_rows, fine);
     FGX_CHECK_LAUNCH("fgx_wgrad_sweep_plan(bounds)");
-    sweep_units_kernel<<<1, 256, 0, s>>>(fine, V, L.nsb, L.spx, (SweepUnit*)(p + L.units), (SweepGroup*)(p + L.wg),
+    sweep_units_kernel<<<1, 64 * kXcds, 0, s>>>(fine, V, L.nsb, L.spx, (SweepUnit*)(p + L.units), (SweepGroup*)(p + L.wg),
                                         (uint32_t*)(p + L.vcount), (uint16_t*)(p + L.vlist));
     FGX_CHECK_LAUNCH("fgx_wgrad_sweep_plan(units)");
     unsigned turn_shift = 0;
