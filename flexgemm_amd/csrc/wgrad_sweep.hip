@@ -1,28 +1,28 @@
-// Weight gradient of the masked implicit GEMM as a paced sweep over the voxels, for gfx950 (16-bit types, a single
-// Co x Ci tile of 128 x 128 or 64 x 64, many voxels).
+// Weight gradient of the masked implicit GEMM as a sweep over the voxels, for gfx950 (16-bit types, a single Co x Ci
+// tile of 128 x 128 or 64 x 64, up to 2^24 voxels).
 //
 // grad_weight[:, v, :] = sum over the pairs (n -> m at offset v) of grad_out[n]^T feats[m]
 // (reference: flex_gemm/kernels/triton/spconv/sparse_submanifold_conv_bwd_masked_implicit_gemm_splitk.py:108-182,
 // 278-317, which cuts the pairs of every offset into SPLITK slices with a partial product each).
 //
 // The block-major kernel of wgrad_gemm.hip cuts the voxels into blocks of ~12K rows and writes an fp32 partial product
-// per (block, offset): the 27 offset items of a block share its rows through an XCD's L2, but the block's rows (4.7 MB
-// at 128 channels) overflow the 4 MiB L2 while smaller blocks multiply the partial products.  Here
+// per (block, offset).  Here
 //
-//   * XCD x owns one contiguous eighth of the voxels (pair lists ascend in the output row inside every offset, so that
-//     is one contiguous pair range per offset);
-//   * the pairs of an XCD's range are cut into 2 x (workgroups per XCD) parts of nearly equal size -- an offset with
-//     many pairs is split into several parts that take its 64-pair steps in turn -- and every workgroup gets two parts,
-//     a large and a small one, and KEEPS BOTH ACCUMULATORS IN REGISTERS for the whole range: 512 partial products in
-//     all instead of one per (block, offset);
-//   * a workgroup takes the steps of its two parts in the order of the sub-block (1024 voxels) their pairs lie in, and
-//     the workgroups of an XCD pace each other: nobody starts a sub-block more than `lead` sub-blocks ahead of the
-//     slowest, so the rows the 32 workgroups gather at any time span a few thousand voxels and are fetched into the
-//     XCD's L2 once for all offsets.  The wait is bounded: after max_polls polls a workgroup goes on regardless, so the
-//     kernel ends whatever the progress words say.
+//   * XCD x owns a contiguous range of sub-blocks holding an eighth of the pairs (pair lists ascend in the output row
+//     inside every offset, so that is one contiguous pair range per offset);
+//   * every offset is cut into up to 64 slices that take its 64-pair steps in turn, a unit is a set of slices of one
+//     offset, and every workgroup gets at most two units of together (nearly) the same number of steps and KEEPS BOTH
+//     ACCUMULATORS IN REGISTERS for the whole range: 512 partial products in all instead of one per (block, offset);
+//   * a workgroup takes the steps of its two units in the order of the sub-blocks their pairs lie in, changing units
+//     every ~16K voxels.  Loaders and multipliers meet through progress words in LDS, not at a barrier per step: a
+//     loader owns a ring stage and whole steps, a multiplier's fragment reads run on across the end of a step;
+//   * optionally the workgroups of an XCD pace each other: nobody starts a sub-block more than `lead` sub-blocks ahead
+//     of the slowest, so the rows the 32 workgroups gather at any time span a few thousand voxels and are fetched into
+//     the XCD's L2 once for all offsets.  The wait is bounded: after max_polls polls a workgroup goes on regardless, so
+//     the kernel ends whatever the progress words say.  Pacing saves traffic and costs time; max_polls = 0 is the default.
 //
 // The step sequence of every workgroup is a function of the pair lists alone: fgx_wgrad_sweep_plan builds it once per
-// neighbor cache.  Sums are taken in a fixed order (steps in list order, parts in ascending order), so results are the
+// neighbor cache.  Sums are taken in a fixed order (steps in list order, units in ascending order), so results are the
 // same on every run; they differ from the block-major kernels' in the order of the fp32 additions.
 #include <type_traits>
 

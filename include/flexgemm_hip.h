@@ -176,7 +176,7 @@ typedef struct fgx_schedule {
     int splitk;         /* fwd/dgrad: number of K splits (1 = none) */
     int block_rows;     /* wgrad: voxel rows per partial-sum block */
     int stream;         /* 1 = persistent streaming kernel (fwd/dgrad: fgx_conv_gather_gemm_stream; wgrad: the
-                         * `streaming` argument of fgx_conv_wgrad), 0 = tiled kernel; wgrad only: 2 = the paced sweep
+                         * `streaming` argument of fgx_conv_wgrad), 0 = tiled kernel; wgrad only: 2 = the sweep
                          * fgx_conv_wgrad_sweep with tile = tile_rows and sub_rows = block_rows */
 } fgx_schedule;
 int fgx_table_lookup(int pass_kind, int dtype, size_t n, int Ci, int Co, int V, fgx_schedule* out);
@@ -306,17 +306,18 @@ int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats,
                    int streaming, void* scratch, void* grad_weight, void* grad_bias, int bias_offset,
                    fgx_stream_t stream);
 
-/* The same weight gradient as a paced sweep, for 16-bit types, a single Co x Ci tile (`tile` = 128 or 64 >= Co, Ci) and
- * many voxels: each XCD takes a contiguous eighth of the voxels, every workgroup keeps the accumulators of two "parts"
- * (an offset, or a share of the 64-pair steps of an offset with many pairs) over that whole range -- 2 x (compute units)
- * partial products in all -- and the workgroups of an XCD walk the sub-blocks of `sub_rows` voxels together (nobody starts
- * a sub-block more than `lead` ahead of the slowest; after `max_polls` looks at the others' progress a workgroup stops
- * waiting, so the kernel ends whatever happens; max_polls = 0 switches the pacing off), which keeps the gathered rows in
- * the XCD's L2.  fgx_wgrad_sweep_plan builds the per-workgroup step lists from the pair lists alone (once per neighbor
- * cache and sub_rows; fgx_wgrad_sweep_plan_bytes bytes, 256-byte aligned); fgx_conv_wgrad_sweep needs
- * fgx_wgrad_sweep_scratch_bytes of scratch.  Sums are taken in a fixed order: same bits on every run, fp32 rounding
- * differences against fgx_conv_wgrad.  grad_bias / bias_offset as for fgx_conv_wgrad.
- * Replaces: the same Triton kernels as fgx_conv_wgrad (its SPLITK slices become the parts). */
+/* The same weight gradient as a sweep over the voxels, for 16-bit types, a single Co x Ci tile (`tile` = 128 or 64 >= Co,
+ * Ci) and at most 2^24 rows per operand: each XCD takes a contiguous range of sub-blocks of `sub_rows` voxels holding an
+ * eighth of the pairs, and every workgroup keeps the accumulators of two "units" (an offset, or a share of the 64-pair
+ * steps of an offset) over that whole range -- 2 x (compute units) partial products in all.  The table's schedule for such
+ * weights (fgx_schedule.stream = 2).  Optional pacing: nobody starts a sub-block more than `lead` ahead of the slowest
+ * workgroup of its XCD; after `max_polls` looks at the others' progress a workgroup stops waiting, so the kernel ends
+ * whatever happens; max_polls = 0 switches the pacing off (faster; pacing keeps the gathered rows in the XCD's L2).
+ * fgx_wgrad_sweep_plan builds the units and the per-workgroup step lists from the pair lists alone, which must ascend in
+ * the output row inside every offset (once per neighbor cache and sub_rows; fgx_wgrad_sweep_plan_bytes bytes, 256-byte
+ * aligned); fgx_conv_wgrad_sweep needs fgx_wgrad_sweep_scratch_bytes of scratch.  Sums are taken in a fixed order: same
+ * bits on every run, fp32 rounding differences against fgx_conv_wgrad.  grad_bias / bias_offset as for fgx_conv_wgrad.
+ * Replaces: the same Triton kernels as fgx_conv_wgrad (its SPLITK slices become the units). */
 size_t fgx_wgrad_sweep_plan_bytes(size_t n, size_t n_pairs, int V, int sub_rows);
 int fgx_wgrad_sweep_plan(const uint32_t* sig_o, const uint32_t* seg_host, size_t n, int V, int sub_rows, void* plan,
                          size_t plan_bytes, fgx_stream_t stream);
