@@ -1,6 +1,8 @@
 // Device-side pieces shared by the weight-gradient kernels (wgrad_gemm.hip, wgrad_sweep.hip): vector types, the
 // transposing LDS read with its hand-placed waits, the MFMA wrappers, buffer resources.
 #pragma once
+#include <type_traits>
+
 #include "fgx_common.h"
 
 namespace fgx {
@@ -90,6 +92,15 @@ constexpr uint32_t kOobOffset = 0xFF000000u;
 using rsrc_t = __amdgpu_buffer_rsrc_t;
 __device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), (short)0, (int)bytes, 0x00020000);
+}
+
+// f(integral_constant<int, 0>), ..., f(integral_constant<int, N - 1>): a loop whose counter is a compile-time constant
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, I + 1>(f);
+    }
 }
 
 // wait until the LDS reads before the newest N have returned; the registers are tied to the wait so that the

@@ -550,27 +550,29 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
     // =================================================================================================
     __syncthreads();                                // the loaders' prologue barrier
     const int s16 = lane & 15, mb = (lane >> 4) & 1;
-    // per-lane byte offsets of the transposing reads inside a stage, for k-block 0 (a k-block is 16 pair rows)
-    int a_off[C::TM][2], b_off[C::TN][2];
+    constexpr int NK = P / 16 / C::SLICES;          // k-blocks (16 pair rows) this wavefront multiplies per step
+    const int kk0 = C::KSPLIT ? mw * NK : 0;        // ... starting at this one
+    // Per-lane byte offsets of the transposing reads inside a stage, for this wavefront's first k-block (a k-block is
+    // 16 pair rows) and the first of a lane's two pair rows; the second pair row (4 rows on: same swizzle key) and the
+    // k-block go into the instruction's offset field, so a step costs one address add per fragment tile.
+    uint32_t a_off[C::TM], b_off[C::TN];
     {
         const int prow = g * 8 + (s16 >> 2);
+        static_assert(C::key_a(0) == C::key_a(4) && C::key_b(1) == C::key_b(5), "pair rows 4 apart share a swizzle key");
 #pragma unroll
         for (int i = 0; i < C::TM; ++i) {
             const int byte = (wave_m * C::WM + i * 32 + mb * 16 + (s16 & 3) * 4) * 2;
             const int c = byte >> 4, w = byte & 15;
-            a_off[i][0] = prow * C::ROWB_A + ((c ^ C::key_a(prow)) << 4) + w;
-            a_off[i][1] = (prow + 4) * C::ROWB_A + ((c ^ C::key_a(prow + 4)) << 4) + w;
+            a_off[i] = (uint32_t)((kk0 * 16 + prow) * C::ROWB_A + ((c ^ C::key_a(prow)) << 4) + w);
         }
 #pragma unroll
         for (int j = 0; j < C::TN; ++j) {
             const int byte = (wave_n * C::WN + j * 32 + mb * 16 + (s16 & 3) * 4) * 2;
             const int c = byte >> 4, w = byte & 15;
-            b_off[j][0] = C::A_BYTES + prow * C::ROWB_B + ((c ^ C::key_b(prow)) << 4) + w;
-            b_off[j][1] = C::A_BYTES + (prow + 4) * C::ROWB_B + ((c ^ C::key_b(prow + 4)) << 4) + w;
+            b_off[j] = (uint32_t)(C::A_BYTES + (kk0 * 16 + prow) * C::ROWB_B + ((c ^ C::key_b(prow)) << 4) + w);
         }
     }
-    constexpr int NK = P / 16 / C::SLICES;          // k-blocks (16 pair rows) this wavefront multiplies per step
-    const int kk0 = C::KSPLIT ? mw * NK : 0;        // ... starting at this one
+    const uint32_t ring_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const unsigned char*)ring;
     constexpr int RK = 2 * (C::TM + C::TN);         // LDS reads per k-block
     Walk m = first;
     unsigned step = 0;
@@ -600,33 +602,36 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
                 asm volatile("" ::: "memory");
                 __builtin_amdgcn_s_barrier();           // the loaders saw this step's rows land
                 asm volatile("" ::: "memory");
-                const unsigned char* cur = ring + (step & (S - 1)) * C::STAGE_BYTES;
+                const uint32_t cur = ring_addr + (step & (S - 1)) * (uint32_t)C::STAGE_BYTES;
                 ++step;
                 // Transposing read: in a 16-lane group, lane s supplies the address of 4 adjacent channels of pair row
                 // (s / 4) and receives the 4 pair values of channel (group base + s).  Lanes 0-15 / 16-31 cover fragment
                 // rows 0-15 / 16-31, the two wave halves take pair rows [0, 8) / [8, 16) of the k-block.  The reads of
                 // k-block kk+1 are in flight while k-block kk is multiplied.
                 i16x4 fr[2][RK];
-                auto read_block = [&](int kl, i16x4 (&dst)[RK]) {
-                    const int kk = kk0 + kl;
-                    const unsigned char* base = cur + kk * 16 * C::ROWB_A;      // ROWB_A == ROWB_B is not assumed below
+                uint32_t a_at[C::TM], b_at[C::TN];
+    #pragma unroll
+                for (int i = 0; i < C::TM; ++i) a_at[i] = cur + a_off[i];
+    #pragma unroll
+                for (int j = 0; j < C::TN; ++j) b_at[j] = cur + b_off[j];
+                auto read_block = [&](auto kl_c, i16x4 (&dst)[RK]) {        // (the k-block is a compile-time constant)
+                    constexpr int kl = decltype(kl_c)::value;
     #pragma unroll
                     for (int i = 0; i < C::TM; ++i) {
-                        dst[i * 2] = lds_read_tr16(base + a_off[i][0]);
-                        dst[i * 2 + 1] = lds_read_tr16(base + a_off[i][1]);
+                        dst[i * 2] = lds_read_tr16_at<kl * 16 * C::ROWB_A>(a_at[i]);
+                        dst[i * 2 + 1] = lds_read_tr16_at<kl * 16 * C::ROWB_A + 4 * C::ROWB_A>(a_at[i]);
                     }
-                    const unsigned char* base_b = cur + kk * 16 * C::ROWB_B;
     #pragma unroll
                     for (int j = 0; j < C::TN; ++j) {
-                        dst[(C::TM + j) * 2] = lds_read_tr16(base_b + b_off[j][0]);
-                        dst[(C::TM + j) * 2 + 1] = lds_read_tr16(base_b + b_off[j][1]);
+                        dst[(C::TM + j) * 2] = lds_read_tr16_at<kl * 16 * C::ROWB_B>(b_at[j]);
+                        dst[(C::TM + j) * 2 + 1] = lds_read_tr16_at<kl * 16 * C::ROWB_B + 4 * C::ROWB_B>(b_at[j]);
                     }
                 };
-                read_block(0, fr[0]);
-    #pragma unroll
-                for (int kk = 0; kk < NK; ++kk) {
-                    if (kk + 1 < NK) {
-                        read_block(kk + 1, fr[(kk + 1) & 1]);
+                read_block(std::integral_constant<int, 0>{}, fr[0]);
+                static_for<NK>([&](auto kk_c) {
+                    constexpr int kk = decltype(kk_c)::value;
+                    if constexpr (kk + 1 < NK) {
+                        read_block(std::integral_constant<int, kk + 1>{}, fr[(kk + 1) & 1]);
                         lds_wait_but<RK>(fr[kk & 1]);
                     } else {
                         lds_wait_but<0>(fr[kk & 1]);
@@ -641,7 +646,7 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
                             mma16<Tag>(acc[i][j], af, bf);
                         }
                     }
-                }
+                });
             }
         };
         if (do_bias) run_steps(std::true_type{});
