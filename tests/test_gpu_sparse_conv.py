@@ -282,6 +282,20 @@ def test_streaming_kernels_with_distinct_row_counts(gpu_device, geom):
         _run_and_check(coords_np, shape, geom, 128, 128, torch.float16, gpu_device, seed=13)
 
 
+@pytest.mark.parametrize("geom", [GEOMS[0], GEOMS[2], GEOMS[3]])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_weight_gradient_sweep_with_distinct_row_counts(gpu_device, geom, dtype):
+    """The wgrad sweep (a weight of one tile) forced on maps whose output rows and input rows differ in number, from
+    shuffled coordinates: its plan only needs pair lists that ascend in the output row inside every offset."""
+    res = 40
+    coords_np = _shell(res, 1, shuffle_seed=8)
+    shape = torch.Size([1, 0, res, res, res])
+    for ci, co, tile, sub_rows in ((128, 128, 128, 256), (48, 64, 64, 2048)):
+        _say(f"sparse conv wgrad sweep geom={geom} ci={ci} co={co} sub_rows={sub_rows} {dtype}")
+        with _force_schedule(wgrad=True, tile_rows=tile, tile_cols=tile, block_rows=sub_rows, stream=2):
+            _run_and_check(coords_np, shape, geom, ci, co, dtype, gpu_device, seed=17)
+
+
 def test_empty_input(gpu_device):
     shape = torch.Size([1, 0, 8, 8, 8])
     none = torch.empty((0, 4), dtype=torch.int32, device=gpu_device)
