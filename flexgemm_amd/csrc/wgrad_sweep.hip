@@ -841,15 +841,44 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
 }
 
 // grad_weight[co][v][ci] = sum of the partial products of offset v's units, in ascending unit order.  One thread per
-// four adjacent ci; eight loads in flight.
+// four adjacent ci; eight loads in flight.  The blocks from `weight_blocks` on (present when a bias gradient is asked
+// for) take one column of grad_bias each: the sum over the workgroups that held a unit of the bias offset, two
+// workgroups per thread, then a tree over LDS -- a fixed order of additions.
 template <typename T>
 __global__ void __launch_bounds__(256) sweep_reduce_kernel(const float* __restrict__ partial,
                                                            const uint32_t* __restrict__ vcount,
                                                            const uint16_t* __restrict__ vlist, unsigned total_units, int V,
-                                                           int Ci, int Co, T* __restrict__ gw) {
+                                                           int Ci, int Co, T* __restrict__ gw, unsigned weight_blocks,
+                                                           const float* __restrict__ bias_partial,
+                                                           const SweepUnit* __restrict__ units, unsigned groups,
+                                                           int bias_offset, T* __restrict__ gbias) {
+    static_assert(kSwMaxGroups == 512, "two workgroups per thread");
+    if (blockIdx.x >= weight_blocks) {
+        __shared__ float sums[256];
+        const int co = (int)(blockIdx.x - weight_blocks);
+        float pair[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const unsigned gidx = threadIdx.x + h * 256;
+            pair[h] = 0.f;
+            if (gidx < groups) {
+                const SweepUnit a = units[(size_t)gidx * 2], b = units[(size_t)gidx * 2 + 1];
+                const bool has = (a.nsteps && (int)a.v == bias_offset) || (b.nsteps && (int)b.v == bias_offset);
+                if (has) pair[h] = bias_partial[(size_t)gidx * Co + co];
+            }
+        }
+        sums[threadIdx.x] = pair[0] + pair[1];
+        __syncthreads();
+        for (unsigned half = 128; half > 0; half >>= 1) {
+            if (threadIdx.x < half) sums[threadIdx.x] += sums[threadIdx.x + half];
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) gbias[co] = from_float<T>(sums[0]);
+        return;
+    }
     const size_t quads = (size_t)Co * V * (Ci / 4);
     const size_t per = (size_t)Co * Ci;
-    for (size_t t = (size_t)blockIdx.x * 256 + threadIdx.x; t < quads; t += (size_t)gridDim.x * 256) {
+    for (size_t t = (size_t)blockIdx.x * 256 + threadIdx.x; t < quads; t += (size_t)weight_blocks * 256) {
         const int cq = (int)(t % (Ci / 4));
         const size_t r = t / (Ci / 4);
         const int v = (int)(r % V), co = (int)(r / V);
@@ -883,30 +912,6 @@ __global__ void __launch_bounds__(256) sweep_reduce_kernel(const float* __restri
         dst[2] = from_float<T>(s.z);
         dst[3] = from_float<T>(s.w);
     }
-}
-
-// grad_bias[co] = sum over the workgroups that held a unit of the bias offset.  One block per column, one thread per
-// workgroup, then a tree over LDS: a fixed order of additions.
-template <typename T>
-__global__ void __launch_bounds__(kSwMaxGroups) sweep_bias_reduce_kernel(const float* __restrict__ bias_partial,
-                                                                         const SweepUnit* __restrict__ units, unsigned groups,
-                                                                         int bias_offset, int Co, T* __restrict__ out) {
-    __shared__ float sums[kSwMaxGroups];
-    const int co = blockIdx.x;
-    const unsigned gidx = threadIdx.x;
-    float s = 0.f;
-    if (gidx < groups) {
-        const SweepUnit a = units[(size_t)gidx * 2], b = units[(size_t)gidx * 2 + 1];
-        const bool has = (a.nsteps && (int)a.v == bias_offset) || (b.nsteps && (int)b.v == bias_offset);
-        if (has) s = bias_partial[(size_t)gidx * Co + co];
-    }
-    sums[gidx] = s;
-    __syncthreads();
-    for (unsigned half = kSwMaxGroups / 2; half > 0; half >>= 1) {
-        if (gidx < half) sums[gidx] += sums[gidx + half];
-        __syncthreads();
-    }
-    if (gidx == 0) out[co] = from_float<T>(sums[0]);
 }
 
 struct SweepScratch {
@@ -954,8 +959,10 @@ int launch_sweep(const void* gout, const void* feats, const uint32_t* sig_i, con
     float* partial = (float*)(scratch + S.partial);
     float* bias_partial = gbias ? (float*)(scratch + S.bias) : nullptr;
     const SweepUnit* units = (const SweepUnit*)(plan + L.units);
-    sweep_clear_kernel<<<cdiv(L.groups, 256), 256, 0, s>>>(prog, L.groups);
-    FGX_CHECK_LAUNCH("fgx_conv_wgrad_sweep(clear)");
+    if (max_polls > 0) {       // the pacing words; nobody looks at them otherwise
+        sweep_clear_kernel<<<cdiv(L.groups, 256), 256, 0, s>>>(prog, L.groups);
+        FGX_CHECK_LAUNCH("fgx_conv_wgrad_sweep(clear)");
+    }
     kern<<<L.groups, C::NT, C::lds_bytes, s>>>((const T*)gout, (const T*)feats, sig_i, sig_o, units,
                                                (const SweepGroup*)(plan + L.wg), (const uint32_t*)(plan + L.steps_k),
                                                (const uint32_t*)(plan + L.steps_m), L.spx, V, Ci, Co, n_pairs,
@@ -964,13 +971,10 @@ int launch_sweep(const void* gout, const void* feats, const uint32_t* sig_i, con
     FGX_CHECK_LAUNCH("fgx_conv_wgrad_sweep");
     const size_t quads = (size_t)Co * V * (Ci / 4);
     unsigned grid = cdiv(quads, 256);
-    sweep_reduce_kernel<T><<<grid, 256, 0, s>>>(partial, (const uint32_t*)(plan + L.vcount), (const uint16_t*)(plan + L.vlist),
-                                                L.groups * 2, V, Ci, Co, (T*)gw);
+    sweep_reduce_kernel<T><<<grid + (bias_partial ? (unsigned)Co : 0u), 256, 0, s>>>(
+        partial, (const uint32_t*)(plan + L.vcount), (const uint16_t*)(plan + L.vlist), L.groups * 2, V, Ci, Co, (T*)gw, grid,
+        bias_partial, units, L.groups, bias_offset, (T*)gbias);
     FGX_CHECK_LAUNCH("fgx_conv_wgrad_sweep(reduce)");
-    if (bias_partial) {
-        sweep_bias_reduce_kernel<T><<<(unsigned)Co, kSwMaxGroups, 0, s>>>(bias_partial, units, L.groups, bias_offset, Co, (T*)gbias);
-        FGX_CHECK_LAUNCH("fgx_conv_wgrad_sweep(bias reduce)");
-    }
     return FGX_OK;
 }
 
