@@ -692,10 +692,10 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
 // kReduceSlices contiguous ranges, one per group of threads; a slice adds its blocks in ascending order (eight loads in
 // flight) and the slice sums are added in ascending order as well, so the result depends on nb alone, not on which
 // kernel wrote the partial products.
-constexpr int kReduceElems = 32, kReduceSlices = 8;
+constexpr int kReduceElems = 32, kReduceSlices = 32;
 
 template <typename T>
-__global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restrict__ partial,
+__global__ void __launch_bounds__(kReduceElems * kReduceSlices) wgrad_reduce_kernel(const float* __restrict__ partial,
                                                            const uint32_t* __restrict__ bounds, int V, int Ci, int Co,
                                                            unsigned nb, unsigned per_block, T* __restrict__ gw) {
     // `per_block` partial products per voxel block (consecutive in `partial`); nb counts the partial products
@@ -858,7 +858,7 @@ int launch_reduce(const float* partial, const uint32_t* bounds, int V, int Ci, i
     if (few_groups) {
         unsigned g = cdiv(total, kReduceElems);
         if (g > 65536u) g = 65536u;
-        wgrad_reduce_kernel<T><<<g, 256, 0, s>>>(partial, bounds, V, Ci, Co, nb, per_block, gw);
+        wgrad_reduce_kernel<T><<<g, kReduceElems * kReduceSlices, 0, s>>>(partial, bounds, V, Ci, Co, nb, per_block, gw);
     } else {
         unsigned g = cdiv(total, 256);
         if (g > 65536u) g = 65536u;
@@ -869,7 +869,7 @@ int launch_reduce(const float* partial, const uint32_t* bounds, int V, int Ci, i
 }
 
 // grad_bias[co] = sum over the voxel blocks (and slices) of their column sums.  A workgroup owns 32 columns; its 32
-// groups of 32 threads each add every 32nd slot (four independent loads in flight), then the group sums are added in
+// groups of 32 threads each add every 32nd slot (eight independent loads in flight), then the group sums are added in
 // group order: a fixed order, the same on every run.  `live` is the block table row of the offset the sums were made
 // from: a block without a pair there was skipped by the kernel and its slots hold nothing.
 template <typename T>
@@ -879,22 +879,25 @@ __global__ void __launch_bounds__(1024) bias_reduce_kernel(const float* __restri
     __shared__ float sums[32][33];
     const int c = threadIdx.x & 31, grp = threadIdx.x >> 5;
     const int co = blockIdx.x * 32 + c;
-    auto term = [&](unsigned q) -> float {
-        const unsigned blk = q / slices;
-        return live[blk] < live[blk + 1] ? bias_partial[(size_t)q * Co + co] : 0.f;
-    };
-    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if (co < Co) {
-        unsigned q = grp;
-        for (; q + 96 < slots; q += 128) {
-            s0 += term(q);
-            s1 += term(q + 32);
-            s2 += term(q + 64);
-            s3 += term(q + 96);
+        for (unsigned base = grp; base < slots; base += 256) {
+            // eight slots at a time, no serial tail: first which of them were written, then their sums
+            bool ok[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const unsigned q = base + 32 * k;
+                const unsigned blk = (q < slots ? q : base) / slices;
+                ok[k] = q < slots && live[blk] < live[blk + 1];
+            }
+            float t[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) t[k] = ok[k] ? bias_partial[(size_t)(base + 32 * k) * Co + co] : 0.f;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) acc[k] += t[k];
         }
-        for (; q < slots; q += 32) s0 += term(q);
     }
-    sums[grp][c] = (s0 + s1) + (s2 + s3);
+    sums[grp][c] = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
     __syncthreads();
     if (grp == 0 && co < Co) {
         float s = 0.f;

@@ -840,8 +840,8 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
     }
 }
 
-// grad_weight[co][v][ci] = sum of the partial products of offset v's units, in ascending unit order.  One thread per
-// four adjacent ci; eight loads in flight.  The blocks from `weight_blocks` on (present when a bias gradient is asked
+// grad_weight[co][v][ci] = sum of the partial products of offset v's units, in a fixed order.  Four lanes per four
+// adjacent ci, four loads in flight each.  The blocks from `weight_blocks` on (present when a bias gradient is asked
 // for) take one column of grad_bias each: the sum over the workgroups that held a unit of the bias offset, two
 // workgroups per thread, then a tree over LDS -- a fixed order of additions.
 template <typename T>
@@ -878,7 +878,10 @@ __global__ void __launch_bounds__(256) sweep_reduce_kernel(const float* __restri
     }
     const size_t quads = (size_t)Co * V * (Ci / 4);
     const size_t per = (size_t)Co * Ci;
-    for (size_t t = (size_t)blockIdx.x * 256 + threadIdx.x; t < quads; t += (size_t)weight_blocks * 256) {
+    // four adjacent lanes share a quad: lane j adds the units j, j + 4, ... of the list, the four sums are then added as
+    // (0 + 1) + (2 + 3)
+    const unsigned part = threadIdx.x & 3u;
+    for (size_t t = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 2; t < quads; t += (size_t)weight_blocks * 64) {
         const int cq = (int)(t % (Ci / 4));
         const size_t r = t / (Ci / 4);
         const int v = (int)(r % V), co = (int)(r / V);
@@ -886,31 +889,40 @@ __global__ void __launch_bounds__(256) sweep_reduce_kernel(const float* __restri
         const uint16_t* list = vlist + (size_t)v * total_units;
         const float* src = partial + (size_t)co * Ci + cq * 4;
         float4 s = {0.f, 0.f, 0.f, 0.f};
-        unsigned i = 0;
-        for (; i + 8 <= cnt; i += 8) {
-            float4 x[8];
+        unsigned i = part;
+        for (; i + 12 < cnt; i += 16) {
+            float4 x[4];
 #pragma unroll
-            for (int q = 0; q < 8; ++q) x[q] = *(const float4*)(src + (size_t)list[i + q] * per);
+            for (int q = 0; q < 4; ++q) x[q] = *(const float4*)(src + (size_t)list[i + 4 * q] * per);
 #pragma unroll
-            for (int q = 0; q < 8; ++q) {
+            for (int q = 0; q < 4; ++q) {
                 s.x += x[q].x;
                 s.y += x[q].y;
                 s.z += x[q].z;
                 s.w += x[q].w;
             }
         }
-        for (; i < cnt; ++i) {
+        for (; i < cnt; i += 4) {
             const float4 x = *(const float4*)(src + (size_t)list[i] * per);
             s.x += x.x;
             s.y += x.y;
             s.z += x.z;
             s.w += x.w;
         }
-        T* dst = gw + ((size_t)co * V + v) * Ci + cq * 4;
-        dst[0] = from_float<T>(s.x);
-        dst[1] = from_float<T>(s.y);
-        dst[2] = from_float<T>(s.z);
-        dst[3] = from_float<T>(s.w);
+#pragma unroll
+        for (int sh = 1; sh <= 2; sh <<= 1) {
+            s.x += __shfl_xor(s.x, sh, 64);
+            s.y += __shfl_xor(s.y, sh, 64);
+            s.z += __shfl_xor(s.z, sh, 64);
+            s.w += __shfl_xor(s.w, sh, 64);
+        }
+        if (part == 0) {
+            T* dst = gw + ((size_t)co * V + v) * Ci + cq * 4;
+            dst[0] = from_float<T>(s.x);
+            dst[1] = from_float<T>(s.y);
+            dst[2] = from_float<T>(s.z);
+            dst[3] = from_float<T>(s.w);
+        }
     }
 }
 
@@ -970,7 +982,7 @@ int launch_sweep(const void* gout, const void* feats, const uint32_t* sig_i, con
                                                partial, bias_partial, bias_offset, prog, (unsigned)lead, (unsigned)max_polls);
     FGX_CHECK_LAUNCH("fgx_conv_wgrad_sweep");
     const size_t quads = (size_t)Co * V * (Ci / 4);
-    unsigned grid = cdiv(quads, 256);
+    unsigned grid = cdiv(quads * 4, 256);      // four lanes per quad of weights
     sweep_reduce_kernel<T><<<grid + (bias_partial ? (unsigned)Co : 0u), 256, 0, s>>>(
         partial, (const uint32_t*)(plan + L.vcount), (const uint16_t*)(plan + L.vlist), L.groups * 2, V, Ci, Co, (T*)gw, grid,
         bias_partial, units, L.groups, bias_offset, (T*)gbias);
