@@ -16,6 +16,8 @@
 //   * a workgroup takes the steps of its two units in the order of the sub-blocks their pairs lie in, changing units
 //     every ~16K voxels.  Loaders and multipliers meet through progress words in LDS, not at a barrier per step: a
 //     loader owns a ring stage and whole steps, a multiplier's fragment reads run on across the end of a step;
+//   * the bias gradient (column sums of grad_out over the offset whose pairs hold every output row once) is added up
+//     by the loaders from what they deposited in their stages;
 //   * optionally the workgroups of an XCD pace each other: nobody starts a sub-block more than `lead` sub-blocks ahead
 //     of the slowest, so the rows the 32 workgroups gather at any time span a few thousand voxels and are fetched into
 //     the XCD's L2 once for all offsets.  The wait is bounded: after max_polls polls a workgroup goes on regardless, so
@@ -402,36 +404,13 @@ __device__ __forceinline__ void swap_tiles(f32x16& a, f32x16& b) {
 #endif
 }
 
-// acc + the eight 16-bit values of a fragment, each times the 16-bit value `w` (given twice, as a packed pair: ones to
-// count the fragment, zeros to leave the sum as it is), in fp32: four two-element dot products
-using f16x2 = _Float16 __attribute__((ext_vector_type(2)));
-using bf16x2 = __bf16 __attribute__((ext_vector_type(2)));
-template <typename Tag> __device__ __forceinline__ float add8(float acc, const i16x8& f, uint32_t w);
-template <> __device__ __forceinline__ float add8<F16>(float acc, const i16x8& f, uint32_t w) {
-    // (the four pairs are taken out of a vector of pairs: a bit cast of an indexed 32-bit element inside an unrolled loop
-    // has been seen to read element 0 four times)
-    struct Pairs { f16x2 p0, p1, p2, p3; };
-    const Pairs d = __builtin_bit_cast(Pairs, f);
-    const f16x2 ww = __builtin_bit_cast(f16x2, w);
-    acc = __builtin_amdgcn_fdot2(d.p0, ww, acc, false);
-    acc = __builtin_amdgcn_fdot2(d.p1, ww, acc, false);
-    acc = __builtin_amdgcn_fdot2(d.p2, ww, acc, false);
-    acc = __builtin_amdgcn_fdot2(d.p3, ww, acc, false);
-    return acc;
+// a 16-bit value (the low half of `bits`) as fp32
+template <typename Tag> __device__ __forceinline__ float half_to_float(uint32_t bits);
+template <> __device__ __forceinline__ float half_to_float<F16>(uint32_t bits) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)bits);
 }
-template <> __device__ __forceinline__ float add8<BF16>(float acc, const i16x8& f, uint32_t w) {
-    struct Pairs { bf16x2 p0, p1, p2, p3; };
-    const Pairs d = __builtin_bit_cast(Pairs, f);
-    const bf16x2 ww = __builtin_bit_cast(bf16x2, w);
-    acc = __builtin_amdgcn_fdot2_f32_bf16(d.p0, ww, acc, false);
-    acc = __builtin_amdgcn_fdot2_f32_bf16(d.p1, ww, acc, false);
-    acc = __builtin_amdgcn_fdot2_f32_bf16(d.p2, ww, acc, false);
-    acc = __builtin_amdgcn_fdot2_f32_bf16(d.p3, ww, acc, false);
-    return acc;
-}
-template <typename Tag> __device__ __forceinline__ uint32_t packed_ones() {
-    return __is_same(typename Tag::type, _Float16) ? 0x3C003C00u : 0x3F803F80u;
-}
+template <> __device__ __forceinline__ float half_to_float<BF16>(uint32_t bits) { return __builtin_bit_cast(float, bits << 16); }
+template <> __device__ __forceinline__ float half_to_float<F32>(uint32_t) { return 0.f; }
 
 template <typename Tag, int BM, int BN>
 struct SweepCfg {
@@ -533,7 +512,7 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
         // sub * NA + i of the step: a lane then needs NA consecutive entries of each pair list, which it fetches
         // straight into registers with 16-byte loads, a round ahead -- no index ring in LDS, no LDS round trip.
         constexpr int NA = P / C::RPI_A, NB = P / C::RPI_B;     // load instructions per operand and step
-        static_assert(NA == NB && NA % 4 == 0, "one slot order for both operands, indices in 16-byte pieces");
+        static_assert(NA == NB && NA % 8 == 0, "one slot order for both operands, indices in 16-byte pieces, column sums eight rows at a time");
         static_assert(NA + NB + NA / 2 + 4 < 64, "outstanding loads exceed the vmcnt range");
         const int sub = lane / C::CH_A;                                    // row inside a load instruction
         // byte column inside the tile, swizzle applied (the key depends on row & 3 alone, an instruction covers 4 or 8 rows)
@@ -595,6 +574,40 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
         };
         // one round: step k's rows are enqueued, the entries of step k + 2S requested, step k + S prepared from the
         // entries requested a round ago, and step k announced
+        // Column sums of grad_out (the bias gradient) ride along with the offset whose pairs hold every output row once.
+        // The loaders add them up, not the multipliers: a loader has time to spare between its rounds, a multiplier
+        // none (with the sums in the multipliers, the workgroups that held a unit of this offset were the last to
+        // finish by a tenth of the kernel).  After announcing a step of that offset the loader reads back what its own
+        // loads deposited -- lane l of load instruction i wrote 16 bytes at i * 1024 + 16 * l, the same eight channels
+        // for every i -- and adds the NA pairs into eight fp32 sums.  Rows past the end of a step and channels past Co
+        // arrived as zeros.  The stage is this loader's own: nobody refills it before its next round.
+        const SweepUnit lu0 = units[(size_t)gid * 2], lu1 = units[(size_t)gid * 2 + 1];
+        const bool lbias0 = bias_partial != nullptr && lu0.nsteps && (int)lu0.v == bias_offset;
+        const bool lbias1 = bias_partial != nullptr && lu1.nsteps && (int)lu1.v == bias_offset;
+        float bsum[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) bsum[e] = 0.f;
+        auto add_columns = [&]() {
+            const unsigned char* mine = stage + lane * 16;
+#pragma unroll
+            for (int i0 = 0; i0 < NA; i0 += 8) {
+                u32x4 piece[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) piece[i] = *(const u32x4*)(mine + (i0 + i) * 1024);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint32_t w0 = piece[i][0], w1 = piece[i][1], w2 = piece[i][2], w3 = piece[i][3];
+                    bsum[0] += half_to_float<Tag>(w0 & 0xFFFFu);
+                    bsum[1] += half_to_float<Tag>(w0 >> 16);
+                    bsum[2] += half_to_float<Tag>(w1 & 0xFFFFu);
+                    bsum[3] += half_to_float<Tag>(w1 >> 16);
+                    bsum[4] += half_to_float<Tag>(w2 & 0xFFFFu);
+                    bsum[5] += half_to_float<Tag>(w2 >> 16);
+                    bsum[6] += half_to_float<Tag>(w3 & 0xFFFFu);
+                    bsum[7] += half_to_float<Tag>(w3 >> 16);
+                }
+            }
+        };
         uint32_t known_consumed = 0;
         auto round = [&](unsigned k, const Indices& ready, Indices& coming) {
             if (k >= (unsigned)S) progress_wait(consumed, k - S + 1u, known_consumed);   // every multiplier has read step k - S
@@ -602,9 +615,11 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
             // loader 0 also keeps the step list: the chunk after next, whose quarter of the ring was read 128+ steps ago
             if (lw == 0 && (k & 63u) == 0u) load_chunk(k / 64 + 2);
             fetch_idx(k + 2 * S, coming);
+            const bool sums = ((step_m[k & (kSwStepRing - 1)] >> 7) & 1u) ? lbias1 : lbias0;       // (uniform)
             prep_rows(k + S, ready);
             wait_vmcnt<0>();
             progress_store(landed + lw, k / S + 1u);
+            if (sums) add_columns();
         };
 
         __syncthreads();                            // (2)
@@ -617,6 +632,29 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
             if (k + S < nsteps) round(k + S, ix0, ix1);
         }
         wait_vmcnt<0>();
+        if (lbias0 || lbias1) {
+            // bias_partial[workgroup][loader][co].  Row r of a load instruction holds channel piece c in lane
+            // r * CH_A + (c ^ key(r)): every lane collects its own piece from all rows, the lanes of row 0 write.
+            const int piece = (int)(a_chb >> 4);
+            float total[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) total[e] = 0.f;
+#pragma unroll
+            for (int r = 0; r < C::RPI_A; ++r) {
+                const int from = r * C::CH_A + (piece ^ C::key_a(r));
+#pragma unroll
+                for (int e = 0; e < 8; ++e) total[e] += __shfl(bsum[e], from, 64);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) bsum[e] = total[e];
+            float* bdst = bias_partial + ((size_t)gid * kSwLoaders + lw) * Co;
+            const int co0 = (int)(a_chb / ES);
+            if (sub == 0) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (co0 + e < Co) bdst[co0 + e] = bsum[e];
+            }
+        }
         return;
     }
 
@@ -653,7 +691,6 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
     // change places when the step list changes units (a handful of times per sub-block), so that the multiply code
     // exists once and the register allocator sees one set of MFMA destinations.
     f32x16 acc[C::TM][C::TN], rest[C::TM][C::TN];
-    float bsum[C::TM];
 #pragma unroll
     for (int i = 0; i < C::TM; ++i) {
 #pragma unroll
@@ -663,17 +700,8 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
                 acc[i][j][e] = 0.f;
                 rest[i][j][e] = 0.f;
             }
-        bsum[i] = 0.f;
     }
     unsigned acc_unit = 0;                          // whose sums `acc` holds
-    // Column sums of grad_out (the bias gradient) ride along with the offset whose pairs hold every output row once:
-    // a lane's grad_out fragment is eight pair values of one output channel, which it adds up on the side with four
-    // two-element dot products against ones (a second accumulator tile of ones-products, as in the block-major
-    // kernel, does not fit beside two accumulators; converting and adding the eight values one by one took as many
-    // issue slots as the step's MFMAs and made the workgroups of this offset the last to finish).  Both
-    // units of a workgroup add to the same sums; only the wavefronts of the first column of wave tiles do it.
-    const bool bias0 = bias_partial != nullptr && un0.nsteps && (int)un0.v == bias_offset && wave_n == 0;
-    const bool bias1 = bias_partial != nullptr && un1.nsteps && (int)un1.v == bias_offset && wave_n == 0;
 
     // Fragments of one k-block (16 pair rows): TM x 2 reads of the grad_out tile, TN x 2 of the feats tile.
     i16x4 fr[2][RK];
@@ -696,13 +724,11 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
     using K2 = std::integral_constant<int, 2>;
     using K3 = std::integral_constant<int, 3>;
     const uint32_t ring_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const unsigned char*)ring;
-    // the products of one k-block; `bias_w`: packed ones to count the grad_out fragments into the bias sums, zeros not to
-    // (a weight, not a branch: the step stays straight-line code)
-    auto multiply_block = [&](i16x4 (&f)[RK], auto with_bias, const uint32_t bias_w) {
+    // the products of one k-block
+    auto multiply_block = [&](i16x4 (&f)[RK]) {
 #pragma unroll
         for (int i = 0; i < C::TM; ++i) {
             const i16x8 af = __builtin_shufflevector(f[i * 2], f[i * 2 + 1], 0, 1, 2, 3, 4, 5, 6, 7);
-            if constexpr (decltype(with_bias)::value) bsum[i] = add8<Tag>(bsum[i], af, bias_w);
 #pragma unroll
             for (int j = 0; j < C::TN; ++j) {
                 const i16x8 bf = __builtin_shufflevector(f[(C::TM + j) * 2], f[(C::TM + j) * 2 + 1], 0, 1, 2, 3, 4, 5, 6, 7);
@@ -717,10 +743,7 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
     if (mw == 0 && lane == 0) __hip_atomic_store(my_prog, cur_sb + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const uint32_t* xcd_prog = prog + xcd * spx;
 
-    // The step loop in two compiled forms, chosen per workgroup: the one that also adds up the grad_out fragments runs
-    // in the workgroups that hold a unit of the bias offset (a per-step choice between two forms would keep both
-    // forms' address registers alive next to two accumulators).
-    auto run_steps = [&](auto with_bias) {
+    auto run_steps = [&]() {
         static_assert(NK == 4, "the step below is written out for four k-blocks");
         // The fragment reads run one k-block ahead of the products and do not stop at the end of a step: while the last
         // k-block of a step is multiplied the first one of the next step arrives.
@@ -743,19 +766,18 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
 #pragma unroll
                     for (int j = 0; j < C::TN; ++j) swap_tiles(acc[i][j], rest[i][j]);
             }
-            const uint32_t bias_w = (unit ? bias1 : bias0) ? packed_ones<Tag>() : 0u;
             read_block(cur, K1{}, fr[1]);
-            multiply_block(fr[0], with_bias, bias_w);       // (landed before the loop came round)
+            multiply_block(fr[0]);       // (landed before the loop came round)
             // the next step's list entry and its stage's progress word travel with the fragments of the third k-block
             uint32_t next_meta = lds_read_word(step_m + ((step + 1) & (kSwStepRing - 1)));
             uint32_t seen = lds_read_word(landed + ((step + 1) & (S - 1)));
             read_block(cur, K2{}, fr[0]);
             lds_wait_but<RK>(fr[1]);
             lds_arrived(next_meta, seen);
-            multiply_block(fr[1], with_bias, bias_w);
+            multiply_block(fr[1]);
             read_block(cur, K3{}, fr[1]);
             lds_wait_but<RK>(fr[0]);
-            multiply_block(fr[0], with_bias, bias_w);
+            multiply_block(fr[0]);
             if (more && (uint32_t)__builtin_amdgcn_readfirstlane((int)seen) < (step + 1) / S + 1u) {     // the loaders are behind: wait here
                 for (unsigned spins = 0; spins < kSwSpinMax && progress_load(landed + ((step + 1) & (S - 1))) < (step + 1) / S + 1u; ++spins)
                     __builtin_amdgcn_s_sleep(1);
@@ -763,7 +785,7 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
             read_block(nxt, K0{}, fr[0]);                      // (after the last step: read and never used)
             lds_wait_but<RK>(fr[1]);
             progress_store(consumed + mw, step + 1u);       // the stage has been read: its loader may refill it
-            multiply_block(fr[1], with_bias, bias_w);
+            multiply_block(fr[1]);
             // The prefetched fragments land while these products run.  They are waited for before the loop goes round:
             // registers with a read in flight must not cross the loop edge, where the compiler may copy them.
             lds_wait_but<0>(fr[0]);
@@ -802,8 +824,7 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
             }
         }
     };
-    if (bias0 || bias1) run_steps(std::true_type{});
-    else run_steps(std::false_type{});
+    run_steps();
     if (mw == 0 && lane == 0) __hip_atomic_store(my_prog, 0xFFFFFFFFu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
     // partial[unit][co][ci], fp32
@@ -829,21 +850,12 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
         if (un0.nsteps) store_acc(rest, gid * 2);
         if (un1.nsteps) store_acc(acc, gid * 2 + 1);
     }
-    if (bias0 || bias1) {                           // bias_partial[workgroup][co]; the two wave halves hold half the pairs each
-        float* bdst = bias_partial + (size_t)gid * Co;
-#pragma unroll
-        for (int i = 0; i < C::TM; ++i) {
-            const float both = bsum[i] + __shfl_xor(bsum[i], 32, 64);
-            const int co = wave_m * C::WM + i * 32 + l32;
-            if (g == 0 && co < Co) bdst[co] = both;
-        }
-    }
 }
 
 // grad_weight[co][v][ci] = sum of the partial products of offset v's units, in a fixed order.  Four lanes per four
 // adjacent ci, four loads in flight each.  The blocks from `weight_blocks` on (present when a bias gradient is asked
-// for) take one column of grad_bias each: the sum over the workgroups that held a unit of the bias offset, two
-// workgroups per thread, then a tree over LDS -- a fixed order of additions.
+// for) take one column of grad_bias each: the sum over the workgroups that held a unit of the bias offset (four
+// loaders' sums each), two workgroups per thread, then a tree over LDS -- a fixed order of additions.
 template <typename T>
 __global__ void __launch_bounds__(256) sweep_reduce_kernel(const float* __restrict__ partial,
                                                            const uint32_t* __restrict__ vcount,
@@ -852,7 +864,7 @@ __global__ void __launch_bounds__(256) sweep_reduce_kernel(const float* __restri
                                                            const float* __restrict__ bias_partial,
                                                            const SweepUnit* __restrict__ units, unsigned groups,
                                                            int bias_offset, T* __restrict__ gbias) {
-    static_assert(kSwMaxGroups == 512, "two workgroups per thread");
+    static_assert(kSwMaxGroups == 512 && kSwLoaders == 4, "two workgroups per thread, four sums per workgroup");
     if (blockIdx.x >= weight_blocks) {
         __shared__ float sums[256];
         const int co = (int)(blockIdx.x - weight_blocks);
@@ -864,7 +876,10 @@ __global__ void __launch_bounds__(256) sweep_reduce_kernel(const float* __restri
             if (gidx < groups) {
                 const SweepUnit a = units[(size_t)gidx * 2], b = units[(size_t)gidx * 2 + 1];
                 const bool has = (a.nsteps && (int)a.v == bias_offset) || (b.nsteps && (int)b.v == bias_offset);
-                if (has) pair[h] = bias_partial[(size_t)gidx * Co + co];
+                if (has) {
+                    const float* p = bias_partial + (size_t)gidx * kSwLoaders * Co + co;        // one sum per loader
+                    pair[h] = (p[0] + p[Co]) + (p[2 * (size_t)Co] + p[3 * (size_t)Co]);
+                }
             }
         }
         sums[threadIdx.x] = pair[0] + pair[1];
@@ -937,7 +952,7 @@ SweepScratch sweep_scratch(int Ci, int Co, int groups) {
     S.partial = off;
     off = align_up(off + (size_t)groups * 2 * Co * Ci * sizeof(float), 256);
     S.bias = off;
-    off = align_up(off + (size_t)groups * Co * sizeof(float), 256);
+    off = align_up(off + (size_t)groups * kSwLoaders * Co * sizeof(float), 256);
     S.colsum = off;
     off += fgx_colsum_scratch_bytes(0, Co);
     S.total = off;
