@@ -471,7 +471,8 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
                 const unsigned char* sp = band + r * C::OUT_PITCH + piece * 16;
                 T* dp = out + (size_t)orow * cols + col;
                 if (vec_ok && col + 16 / C::ES <= cols) {
-                    *(u32x4*)dp = *(const u32x4*)sp;
+                    // (streaming store: the output is not read again by this launch and should not push source rows out of L2)
+                    __builtin_nontemporal_store(*(const u32x4*)sp, (u32x4*)dp);
                 } else {
                     for (int t = 0; t < 16 / C::ES && col + t < cols; ++t) dp[t] = ((const T*)sp)[t];
                 }
