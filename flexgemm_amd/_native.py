@@ -34,7 +34,6 @@ EXPORTS = [
     "fgx_conv_scratch_bytes", "fgx_conv_gather_gemm", "fgx_conv_gather_gemm_act",
     "fgx_gather_plan_count", "fgx_gather_plan_fill", "fgx_conv_gather_gemm_stream", "fgx_conv_gather_gemm_stream_act",
     "fgx_conv_gather_gemm_stream_groups", "fgx_gather_item_order_workspace_bytes", "fgx_gather_item_order",
-    "fgx_conv_gather_gemm_chunk_supported", "fgx_conv_gather_gemm_chunk",
     "fgx_wgrad_scratch_bytes", "fgx_wgrad_block_bounds_count", "fgx_wgrad_block_bounds", "fgx_conv_wgrad",
     "fgx_wgrad_sweep_plan_bytes", "fgx_wgrad_sweep_plan", "fgx_wgrad_sweep_scratch_bytes", "fgx_conv_wgrad_sweep",
     "fgx_colsum_scratch_bytes", "fgx_colsum", "fgx_colsum_static_max_cols", "fgx_colsum_static",

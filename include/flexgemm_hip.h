@@ -267,32 +267,6 @@ int fgx_conv_gather_gemm_stream_act(int dtype, const void* src, const void* pane
                                     int max_groups, int activation, void* out, fgx_stream_t stream);
 int fgx_conv_gather_gemm_stream_groups(int dtype, int cols, int tile_rows, int tile_cols, int slab_bytes, int* groups);
 
-/* Chunk-resident gather GEMM (16-bit element types): the same sums as fgx_conv_gather_gemm, with the gather done in
- * LDS.  A chunk is FGX_CHUNK_ROWS output rows that are neighbors in space; every source row a chunk's neighbors name
- * (the chunk itself and a thin halo: "local rows", at most FGX_CHUNK_SRC_MAX of them, local row 0 = the empty row)
- * is loaded once per 64-byte K-slab, and the MFMA operands are read from LDS through the plan's local row indices.
- * Position p of a chunk = wave * 64 + band * 16 + row (8 wavefronts x 4 bands x 16 rows).  Plan arrays (device):
- *   chunk_src  uint32 [nchunks][FGX_CHUNK_SRC_MAX]   source row of each local row, 0xFFFFFFFF = empty
- *   chunk_nsrc int32  [nchunks]                      local rows in use, the empty row included
- *   chunk_idx  uint16 [nchunks][V][8][16][4]         local row of neighbor v of position (wave, row, band)
- *   chunk_out  uint32 [nchunks][FGX_CHUNK_ROWS]      output row at each position, 0xFFFFFFFF = none
- *   chunk_band uint32 [nchunks][32]                  bit v of entry wave * 4 + band: some row of the band has offset v
- * `panel`: fgx_pack_weight(..., slab_bytes 64, col_pad 128) of mode 0 (forward), 1 (submanifold dgrad) or 2.
- * Needs K * 2 a multiple of 64 bytes, cols a multiple of 8, 12 <= V <= 32, operands below ~4 GB
- * (fgx_conv_gather_gemm_chunk_supported tells; otherwise FGX_ERR_UNSUPPORTED and callers use the other kernels).
- * `max_groups` <= 0: one workgroup per CU.  The result does not depend on how rows are dealt to chunks; sums run
- * over K-slabs outermost and offsets ascending inside, so they differ from the other kernels' in fp32 rounding only.
- * Replaces: the same reference kernels as fgx_conv_gather_gemm (..._fwd_masked_implicit_gemm.py:20-100,
- *           ..._bwd_masked_implicit_gemm.py:19-91). */
-#define FGX_CHUNK_ROWS 512
-#define FGX_CHUNK_SRC_MAX 912
-int fgx_conv_gather_gemm_chunk_supported(int dtype, size_t n_src, int K, int cols, int V);
-int fgx_conv_gather_gemm_chunk(int dtype, const void* src, const void* panel, const void* bias,
-                               const uint32_t* chunk_src, const int32_t* chunk_nsrc, const uint16_t* chunk_idx,
-                               const uint32_t* chunk_out, const uint32_t* chunk_band, size_t nchunks,
-                               size_t n_src, int K, int cols, int V, int max_groups, int activation, void* out,
-                               fgx_stream_t stream);
-
 /* item_at for fgx_conv_gather_gemm_stream, made on the device from the tile codes: items sorted by cost (offsets per
  * row tile x `slabs` K-slabs + an epilogue), the incomplete last round of `groups` positions filled with the cheapest,
  * every full round dealt most-expensive-item to least-loaded-slot.  One workgroup, deterministic, no read-back;
