@@ -36,7 +36,8 @@ EXPORTS = [
     "fgx_conv_gather_gemm_stream_groups", "fgx_gather_item_order_workspace_bytes", "fgx_gather_item_order",
     "fgx_wgrad_scratch_bytes", "fgx_wgrad_block_bounds_count", "fgx_wgrad_block_bounds", "fgx_conv_wgrad",
     "fgx_wgrad_sweep_plan_bytes", "fgx_wgrad_sweep_plan", "fgx_wgrad_sweep_scratch_bytes", "fgx_conv_wgrad_sweep",
-    "fgx_colsum_scratch_bytes", "fgx_colsum", "fgx_colsum_static_max_cols", "fgx_colsum_static",
+    "fgx_wgrad_sweep_giveup_words", "fgx_wgrad_sweep_reduce",
+    "fgx_colsum_scratch_bytes", "fgx_colsum", "fgx_colsum_static_prepare", "fgx_colsum_static_max_cols", "fgx_colsum_static",
     "fgx_spconv_out_dims", "fgx_spconv_out_coords_workspace_bytes", "fgx_spconv_out_coords_keys",
     "fgx_spconv_out_coords_decode", "fgx_spconv_neighbor_map",
     "fgx_spconv_neighbor_map_sorted_workspace_bytes", "fgx_spconv_neighbor_map_sorted",
@@ -100,7 +101,7 @@ def lib() -> C.CDLL:
                      "fgx_colsum_scratch_bytes", "fgx_spconv_out_coords_workspace_bytes",
                      "fgx_subm_neighbor_map_sorted_workspace_bytes", "fgx_wgrad_block_bounds_count",
                      "fgx_spconv_neighbor_map_sorted_workspace_bytes", "fgx_serialize_reorder_workspace_bytes",
-                     "fgx_gather_item_order_workspace_bytes", "fgx_wgrad_sweep_plan_bytes", "fgx_wgrad_sweep_scratch_bytes"):
+                     "fgx_gather_item_order_workspace_bytes", "fgx_wgrad_sweep_plan_bytes", "fgx_wgrad_sweep_scratch_bytes", "fgx_wgrad_sweep_giveup_words"):
             getattr(L, name).restype = C.c_size_t
         _lib = L
     return _lib

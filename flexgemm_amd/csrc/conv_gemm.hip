@@ -730,6 +730,35 @@ int fgx_colsum(int dtype, const void* x, size_t n, int cols, void* scratch, void
 
 int fgx_colsum_static_max_cols(void) { return kStaticColsumCols; }
 
+// The device address of the current GPU's copy of the scratch array, looked up once per device with that device current.
+// The lookup may load the code object and is no stream operation: it must not happen while a stream is being captured.
+static int static_colsum_ptr(const char* who, hipStream_t s, float** out) {
+    int dev = 0;
+    FGX_CHECK_HIP(hipGetDevice(&dev));
+    FGX_CHECK_ARG(dev >= 0 && dev < kMaxDevices, "%s: device ordinal %d out of range", who, dev);
+    float* ptr = g_static_colsum_ptr[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &capturing) == hipSuccess && capturing != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            set_error("%s: first use on device %d while its stream is being captured; call fgx_colsum_static_prepare() on this device before the capture", who, dev);
+            return FGX_ERR_ARG;
+        }
+        void* found = nullptr;
+        FGX_CHECK_HIP(hipGetSymbolAddress(&found, HIP_SYMBOL(g_static_colsum_scratch)));
+        FGX_CHECK_ARG(found != nullptr, "%s: the scratch array has no address on device %d", who, dev);
+        ptr = (float*)found;
+        g_static_colsum_ptr[dev].store(ptr, std::memory_order_release);     // (two first callers find the same address)
+    }
+    *out = ptr;
+    return FGX_OK;
+}
+
+int fgx_colsum_static_prepare(void) {
+    float* ptr = nullptr;
+    return static_colsum_ptr("fgx_colsum_static_prepare", nullptr, &ptr);
+}
+
 int fgx_colsum_static(int dtype, const void* x, size_t n, int cols, void* out, fgx_stream_t stream) {
     FGX_CHECK_ARG(dtype_ok(dtype), "fgx_colsum_static: unknown dtype %d", dtype);
     FGX_CHECK_ARG(cols > 0 && out != nullptr, "fgx_colsum_static: bad shape or null output");
@@ -737,18 +766,9 @@ int fgx_colsum_static(int dtype, const void* x, size_t n, int cols, void* out, f
     FGX_CHECK_ARG(cols <= kStaticColsumCols,
                   "fgx_colsum_static: %d columns exceed the %d the library's own scratch holds; use fgx_colsum with caller-owned scratch",
                   cols, kStaticColsumCols);
-    // The device address of this GPU's copy of the array, looked up once per device with that device current.
-    int dev = 0;
-    FGX_CHECK_HIP(hipGetDevice(&dev));
-    FGX_CHECK_ARG(dev >= 0 && dev < kMaxDevices, "fgx_colsum_static: device ordinal %d out of range", dev);
-    float* ptr = g_static_colsum_ptr[dev].load(std::memory_order_acquire);
-    if (ptr == nullptr) {
-        void* found = nullptr;
-        FGX_CHECK_HIP(hipGetSymbolAddress(&found, HIP_SYMBOL(g_static_colsum_scratch)));
-        FGX_CHECK_ARG(found != nullptr, "fgx_colsum_static: the scratch array has no address on device %d", dev);
-        ptr = (float*)found;
-        g_static_colsum_ptr[dev].store(ptr, std::memory_order_release);     // (two first callers find the same address)
-    }
+    float* ptr = nullptr;
+    const int rc = static_colsum_ptr("fgx_colsum_static", (hipStream_t)stream, &ptr);
+    if (rc != FGX_OK) return rc;
     return colsum_launch(dtype, x, n, cols, ptr, out, (hipStream_t)stream);
 }
 

@@ -186,7 +186,7 @@ using namespace fgx;
 
 extern "C" {
 
-int fgx_abi_version(void) { return 1; }
+int fgx_abi_version(void) { return 2; }
 
 void fgx_set_phase_hook(fgx_phase_hook_t hook) { fgx::g_phase_hook = hook; }
 

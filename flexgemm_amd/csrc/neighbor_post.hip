@@ -483,7 +483,11 @@ using namespace fgx;
 extern "C" {
 
 size_t fgx_sort_workspace_bytes(size_t n) {
-    return n >= kOwnSortMin && n <= kOwnSortMax ? radix_layout(n).total : sort_layout(n).total;
+    // (in the radix sort's range a call with a full 32-bit code still takes the library sort: room for either)
+    const size_t lib_sort = sort_layout(n).total;
+    if (n < kOwnSortMin || n > kOwnSortMax) return lib_sort;
+    const size_t own = radix_layout(n).total;
+    return own > lib_sort ? own : lib_sort;
 }
 
 int fgx_sort_by_code(const int32_t* binary, size_t n, int V, int64_t* sorted_idx, void* workspace,

@@ -1142,6 +1142,8 @@ int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uin
     FGX_CHECK_ARG(dtype_ok(dtype), "fgx_conv_wgrad: unknown dtype %d", dtype);
     FGX_CHECK_ARG(Ci > 0 && Co > 0 && V >= 1 && V <= kMaxV, "fgx_conv_wgrad: bad shape Ci=%d Co=%d V=%d", Ci, Co, V);
     FGX_CHECK_ARG(block_rows >= 1, "fgx_conv_wgrad: block_rows must be positive, got %d", block_rows);
+    FGX_CHECK_ARG(streaming == 0 || streaming == 1,
+                  "fgx_conv_wgrad: streaming must be 0 or 1, got %d (a schedule with stream = 2 is for fgx_conv_wgrad_sweep)", streaming);
     FGX_CHECK_ARG(seg_host && scratch && grad_weight, "fgx_conv_wgrad: null buffer");
     FGX_CHECK_ARG(n < 0xFFFFFFFFull && n_in < 0xFFFFFFFFull, "fgx_conv_wgrad: too many rows");
     const int es = dtype == FGX_F32 ? 4 : 2;

@@ -41,6 +41,7 @@ constexpr int kSwStepRing = 256;     // step-list entries held in LDS (four chun
 constexpr int kSwTurnRows = 16384;   // a workgroup changes units about every so many voxels (a change swaps the accumulators)
 constexpr int kSwMaxSlots = 64;      // workgroups per XCD the pacing poll can look at (one lane each)
 constexpr int kSwMaxGroups = kXcds * kSwMaxSlots;
+constexpr int kSwWaves = 4 + kSwLoaders;     // wavefronts of a sweep workgroup: four multipliers and the loaders
 constexpr unsigned kSwSpinMax = 1u << 20;   // looks at a progress word before a wavefront goes on regardless
 
 // Progress words in LDS replace a barrier per step.  Loader w owns ring stage w and counts the steps it has landed
@@ -75,14 +76,17 @@ __device__ __forceinline__ uint32_t lds_read_word(const uint32_t* word) {
     return w;
 }
 __device__ __forceinline__ void lds_arrived(uint32_t& a, uint32_t& b) { asm volatile("" : "+v"(a), "+v"(b)); }
-// spins until the minimum of the four words reaches `need`; `known` caches the last minimum seen
-__device__ __forceinline__ void progress_wait(const uint32_t* words, uint32_t need, uint32_t& known) {
+// spins until the minimum of the four words reaches `need`; `known` caches the last minimum seen.  After kSwSpinMax looks
+// the wavefront goes on regardless, so that the kernel ends whatever happens, and `gave_up` is set: data it works with from
+// then on may be stale, and the reduction turns the whole result into NaN
+__device__ __forceinline__ void progress_wait(const uint32_t* words, uint32_t need, uint32_t& known, uint32_t& gave_up) {
     if (known >= need) return;
     for (unsigned spins = 0; spins < kSwSpinMax; ++spins) {
         known = progress_min4(words);
         if (known >= need) return;
         __builtin_amdgcn_s_sleep(1);
     }
+    gave_up = 1u;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -443,7 +447,7 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
                    const uint32_t* __restrict__ steps_k, const uint32_t* __restrict__ steps_m, unsigned spx, int V, int Ci,
                    int Co, uint32_t n_pairs, uint32_t gout_bytes, uint32_t feats_bytes, float* __restrict__ partial,
                    float* __restrict__ bias_partial, int bias_offset, uint32_t* __restrict__ prog, unsigned lead,
-                   unsigned max_polls) {
+                   unsigned max_polls, uint32_t* __restrict__ giveup) {
     using C = SweepCfg<Tag, BM, BN>;
     constexpr int ES = C::ES, S = C::S, P = C::P;
 
@@ -468,8 +472,13 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
     const SweepGroup grp = groups_tab[gid];
     const unsigned nsteps = grp.nsteps;
     uint32_t* my_prog = prog + gid;
+    // giveup[workgroup][wavefront]: every wavefront writes its word once, at its end -- 1 if one of its waits for data ran
+    // out of looks, else 0 -- so the words need no clearing between calls
+    uint32_t* my_giveup = giveup + (size_t)gid * kSwWaves + wave;
+    uint32_t gave_up = 0u;
     if (nsteps == 0) {                               // nothing to do: nobody has to wait for this workgroup
         if (tid == 0) __hip_atomic_store(my_prog, 0xFFFFFFFFu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) *my_giveup = 0u;
         return;
     }
 
@@ -610,7 +619,7 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
         };
         uint32_t known_consumed = 0;
         auto round = [&](unsigned k, const Indices& ready, Indices& coming) {
-            if (k >= (unsigned)S) progress_wait(consumed, k - S + 1u, known_consumed);   // every multiplier has read step k - S
+            if (k >= (unsigned)S) progress_wait(consumed, k - S + 1u, known_consumed, gave_up);   // every multiplier has read step k - S
             fire_rows();
             // loader 0 also keeps the step list: the chunk after next, whose quarter of the ring was read 128+ steps ago
             if (lw == 0 && (k & 63u) == 0u) load_chunk(k / 64 + 2);
@@ -655,6 +664,7 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
                     if (co0 + e < Co) bdst[co0 + e] = bsum[e];
             }
         }
+        if (lane == 0) *my_giveup = gave_up;
         return;
     }
 
@@ -748,7 +758,11 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
         // The fragment reads run one k-block ahead of the products and do not stop at the end of a step: while the last
         // k-block of a step is multiplied the first one of the next step arrives.
         uint32_t meta = step_m[0];
-        for (unsigned spins = 0; spins < kSwSpinMax && progress_load(landed) < 1u; ++spins) __builtin_amdgcn_s_sleep(1);
+        {
+            unsigned spins = 0;
+            for (; spins < kSwSpinMax && progress_load(landed) < 1u; ++spins) __builtin_amdgcn_s_sleep(1);
+            if (spins == kSwSpinMax) gave_up = 1u;      // went on without the first step's rows
+        }
         read_block(ring_addr, K0{}, fr[0]);
         lds_wait_but<0>(fr[0]);
         for (unsigned step = 0; step < nsteps; ++step) {
@@ -779,8 +793,10 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
             lds_wait_but<RK>(fr[0]);
             multiply_block(fr[0]);
             if (more && (uint32_t)__builtin_amdgcn_readfirstlane((int)seen) < (step + 1) / S + 1u) {     // the loaders are behind: wait here
-                for (unsigned spins = 0; spins < kSwSpinMax && progress_load(landed + ((step + 1) & (S - 1))) < (step + 1) / S + 1u; ++spins)
+                unsigned spins = 0;
+                for (; spins < kSwSpinMax && progress_load(landed + ((step + 1) & (S - 1))) < (step + 1) / S + 1u; ++spins)
                     __builtin_amdgcn_s_sleep(1);
+                if (spins == kSwSpinMax) gave_up = 1u;      // goes on with whatever the stage holds
             }
             read_block(nxt, K0{}, fr[0]);                      // (after the last step: read and never used)
             lds_wait_but<RK>(fr[1]);
@@ -850,12 +866,15 @@ wgrad_sweep_kernel(const typename Tag::type* __restrict__ gout, const typename T
         if (un0.nsteps) store_acc(rest, gid * 2);
         if (un1.nsteps) store_acc(acc, gid * 2 + 1);
     }
+    if (lane == 0) *my_giveup = gave_up;
 }
 
 // grad_weight[co][v][ci] = sum of the partial products of offset v's units, in a fixed order.  Four lanes per four
 // adjacent ci, four loads in flight each.  The blocks from `weight_blocks` on (present when a bias gradient is asked
 // for) take one column of grad_bias each: the sum over the workgroups that held a unit of the bias offset (four
 // loaders' sums each), two workgroups per thread, then a tree over LDS -- a fixed order of additions.
+// Every block first looks at the sweep's give-up words (one per wavefront): if any is set, a wavefront went on without the
+// data it waited for, and every weight and bias gradient is written as NaN instead of a sum that may be wrong.
 template <typename T>
 __global__ void __launch_bounds__(256) sweep_reduce_kernel(const float* __restrict__ partial,
                                                            const uint32_t* __restrict__ vcount,
@@ -863,8 +882,13 @@ __global__ void __launch_bounds__(256) sweep_reduce_kernel(const float* __restri
                                                            int Ci, int Co, T* __restrict__ gw, unsigned weight_blocks,
                                                            const float* __restrict__ bias_partial,
                                                            const SweepUnit* __restrict__ units, unsigned groups,
-                                                           int bias_offset, T* __restrict__ gbias) {
+                                                           int bias_offset, T* __restrict__ gbias,
+                                                           const uint32_t* __restrict__ giveup) {
     static_assert(kSwMaxGroups == 512 && kSwLoaders == 4, "two workgroups per thread, four sums per workgroup");
+    uint32_t flags = 0u;
+    for (unsigned i = threadIdx.x; i < groups * kSwWaves; i += 256) flags |= giveup[i];
+    const bool poisoned = __syncthreads_or(flags != 0u) != 0;
+    const float poison = __builtin_nanf("");
     if (blockIdx.x >= weight_blocks) {
         __shared__ float sums[256];
         const int co = (int)(blockIdx.x - weight_blocks);
@@ -888,7 +912,7 @@ __global__ void __launch_bounds__(256) sweep_reduce_kernel(const float* __restri
             if (threadIdx.x < half) sums[threadIdx.x] += sums[threadIdx.x + half];
             __syncthreads();
         }
-        if (threadIdx.x == 0) gbias[co] = from_float<T>(sums[0]);
+        if (threadIdx.x == 0) gbias[co] = from_float<T>(poisoned ? poison : sums[0]);
         return;
     }
     const size_t quads = (size_t)Co * V * (Ci / 4);
@@ -931,6 +955,7 @@ __global__ void __launch_bounds__(256) sweep_reduce_kernel(const float* __restri
             s.z += __shfl_xor(s.z, sh, 64);
             s.w += __shfl_xor(s.w, sh, 64);
         }
+        if (poisoned) s.x = s.y = s.z = s.w = poison;
         if (part == 0) {
             T* dst = gw + ((size_t)co * V + v) * Ci + cq * 4;
             dst[0] = from_float<T>(s.x);
@@ -942,13 +967,15 @@ __global__ void __launch_bounds__(256) sweep_reduce_kernel(const float* __restri
 }
 
 struct SweepScratch {
-    size_t prog, partial, bias, colsum, total;
+    size_t prog, giveup, partial, bias, colsum, total;
 };
 SweepScratch sweep_scratch(int Ci, int Co, int groups) {
     SweepScratch S{};
     size_t off = 0;
     S.prog = off;
     off = align_up(off + (size_t)groups * 4, 256);
+    S.giveup = off;
+    off = align_up(off + (size_t)groups * kSwWaves * 4, 256);
     S.partial = off;
     off = align_up(off + (size_t)groups * 2 * Co * Ci * sizeof(float), 256);
     S.bias = off;
@@ -969,6 +996,22 @@ int sweep_groups() {
 }
 
 bool tile_ok(int tile, int Ci, int Co) { return (tile == 128 || tile == 64) && Ci <= tile && Co <= tile; }
+
+// the second half of a sweep: the units' partial products (and the loaders' column sums, if `gbias`) in `scratch` -> gradients
+template <typename T>
+int launch_sweep_reduce(const char* plan, const SweepLayout& L, int V, int Ci, int Co, char* scratch, const SweepScratch& S,
+                        void* gw, void* gbias, int bias_offset, hipStream_t s) {
+    const float* partial = (const float*)(scratch + S.partial);
+    const float* bias_partial = gbias ? (const float*)(scratch + S.bias) : nullptr;
+    const size_t quads = (size_t)Co * V * (Ci / 4);
+    unsigned grid = cdiv(quads * 4, 256);      // four lanes per quad of weights
+    sweep_reduce_kernel<T><<<grid + (bias_partial ? (unsigned)Co : 0u), 256, 0, s>>>(
+        partial, (const uint32_t*)(plan + L.vcount), (const uint16_t*)(plan + L.vlist), L.groups * 2, V, Ci, Co, (T*)gw, grid,
+        bias_partial, (const SweepUnit*)(plan + L.units), L.groups, bias_offset, (T*)gbias,
+        (const uint32_t*)(scratch + S.giveup));
+    FGX_CHECK_LAUNCH("fgx_conv_wgrad_sweep(reduce)");
+    return FGX_OK;
+}
 
 template <typename Tag, int BM, int BN>
 int launch_sweep(const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o, const char* plan,
@@ -994,15 +1037,10 @@ int launch_sweep(const void* gout, const void* feats, const uint32_t* sig_i, con
                                                (const SweepGroup*)(plan + L.wg), (const uint32_t*)(plan + L.steps_k),
                                                (const uint32_t*)(plan + L.steps_m), L.spx, V, Ci, Co, n_pairs,
                                                (uint32_t)(n * (size_t)Co * sizeof(T)), (uint32_t)(n_in * (size_t)Ci * sizeof(T)),
-                                               partial, bias_partial, bias_offset, prog, (unsigned)lead, (unsigned)max_polls);
+                                               partial, bias_partial, bias_offset, prog, (unsigned)lead, (unsigned)max_polls,
+                                               (uint32_t*)(scratch + S.giveup));
     FGX_CHECK_LAUNCH("fgx_conv_wgrad_sweep");
-    const size_t quads = (size_t)Co * V * (Ci / 4);
-    unsigned grid = cdiv(quads * 4, 256);      // four lanes per quad of weights
-    sweep_reduce_kernel<T><<<grid + (bias_partial ? (unsigned)Co : 0u), 256, 0, s>>>(
-        partial, (const uint32_t*)(plan + L.vcount), (const uint16_t*)(plan + L.vlist), L.groups * 2, V, Ci, Co, (T*)gw, grid,
-        bias_partial, units, L.groups, bias_offset, (T*)gbias);
-    FGX_CHECK_LAUNCH("fgx_conv_wgrad_sweep(reduce)");
-    return FGX_OK;
+    return launch_sweep_reduce<T>(plan, L, V, Ci, Co, scratch, S, gw, gbias, bias_offset, s);
 }
 
 }  // namespace
@@ -1105,6 +1143,30 @@ int fgx_conv_wgrad_sweep(int dtype, const void* grad_out, const void* feats, con
 #undef FGX_SWEEP
     set_error("fgx_conv_wgrad_sweep: no kernel for tile %d", tile);
     return FGX_ERR_UNSUPPORTED;
+}
+
+size_t fgx_wgrad_sweep_giveup_words(int Ci, int Co, size_t* byte_offset) {
+    const int groups = sweep_groups();
+    if (Ci <= 0 || Co <= 0 || groups < kXcds) return 0;
+    if (byte_offset) *byte_offset = sweep_scratch(Ci, Co, groups).giveup;
+    return (size_t)groups * kSwWaves;
+}
+
+int fgx_wgrad_sweep_reduce(int dtype, const void* plan, size_t n, size_t n_pairs, int Ci, int Co, int V, int sub_rows,
+                           void* scratch, void* grad_weight, void* grad_bias, int bias_offset, fgx_stream_t stream) {
+    FGX_CHECK_ARG(dtype == FGX_F16 || dtype == FGX_BF16, "fgx_wgrad_sweep_reduce: 16-bit types only (dtype %d)", dtype);
+    FGX_CHECK_ARG(Ci > 0 && Co > 0 && Ci % 8 == 0 && Co % 8 == 0 && V >= 1 && V <= kMaxV, "fgx_wgrad_sweep_reduce: bad shape Ci=%d Co=%d V=%d", Ci, Co, V);
+    FGX_CHECK_ARG(sub_rows >= 64 && n > 0 && n_pairs > 0, "fgx_wgrad_sweep_reduce: bad sizes");
+    FGX_CHECK_ARG(plan && scratch && grad_weight, "fgx_wgrad_sweep_reduce: null buffer");
+    FGX_CHECK_ARG(((uintptr_t)scratch & 255) == 0 && ((uintptr_t)plan & 255) == 0, "fgx_wgrad_sweep_reduce: scratch and plan must be 256-byte aligned");
+    const int groups = sweep_groups();
+    FGX_CHECK_ARG(groups >= kXcds && groups / kXcds * 2 >= V, "fgx_wgrad_sweep_reduce: too few compute units for %d offsets", V);
+    const SweepLayout L = sweep_layout(n, n_pairs, V, sub_rows, groups);
+    const SweepScratch S = sweep_scratch(Ci, Co, groups);
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == FGX_F16)
+        return launch_sweep_reduce<F16::type>((const char*)plan, L, V, Ci, Co, (char*)scratch, S, grad_weight, grad_bias, bias_offset, s);
+    return launch_sweep_reduce<BF16::type>((const char*)plan, L, V, Ci, Co, (char*)scratch, S, grad_weight, grad_bias, bias_offset, s);
 }
 
 }  // extern "C"

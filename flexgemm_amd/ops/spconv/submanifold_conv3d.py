@@ -514,6 +514,14 @@ def _stream_fits(n: int, n_src: int, row_bytes: int) -> bool:
     return n_src * row_bytes <= 0xFF000000 and n * 8 <= 0xFF000000 and n * 27 * 4 * 2 <= 0xFF000000
 
 
+def _sweep_fits(n: int, n_in: int, ci: int, co: int, elem_bytes: int, n_pairs: int) -> bool:
+    """What fgx_conv_wgrad_sweep accepts: it multiplies row numbers with 24-bit multiplies and addresses both operands
+    and the pair lists with 32-bit byte offsets below 0xFF000000 (the checks of the C entry point, restated)."""
+    return (0 < n <= (1 << 24) and n_in <= (1 << 24) and n_pairs > 0
+            and n * co * elem_bytes <= 0xFF000000 and n_in * ci * elem_bytes <= 0xFF000000
+            and n_pairs * 4 + 256 <= 0xFF000000)
+
+
 # pacing of the wgrad sweep: sub-blocks a workgroup may run ahead of the slowest one of its XCD, and the looks at the
 # others' progress after which it stops waiting (0 = no pacing, the default: the workgroups of an XCD stay close enough
 # together by themselves, and waiting costs more time than the L2 misses it saves)
@@ -544,10 +552,10 @@ def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int, with_b
     gb = torch.empty((cop,), dtype=dt, device=dev) if with_bias else None
     L = nat.lib()
     code = nat.DTYPE_CODE[dt]
-    if sched.stream == 2 and (n > (1 << 24) or n_in > (1 << 24)):
-        # the sweep multiplies row numbers with 24-bit multiplies: very long operands take the block-major kernel
+    if sched.stream == 2 and not _sweep_fits(n, n_in, cip, cop, f.element_size(), seg_host[-1]):
+        # very long operands (and empty pair lists) take the block-major kernel
         sched.stream, sched.block_rows = 1, 12288
-    if sched.stream == 2 and seg_host[-1] > 0 and n > 0:
+    if sched.stream == 2:
         plan = cache._wgrad_sweep_plan(sched.block_rows)
         with torch.cuda.device(dev):
             scratch = nat.workspace(L.fgx_wgrad_sweep_scratch_bytes(C.c_int(cip), C.c_int(cop)), dev)

@@ -42,7 +42,10 @@ extern "C" {
 
 typedef void* fgx_stream_t;
 
-/* Library identity and error text. */
+/* Library identity and error text.  fgx_abi_version() is 2 for this header.  Against version 1:
+ * fgx_subm_neighbor_map_sorted has a `presorted` argument before its workspace, fgx_schedule.stream may be 2 for the
+ * weight gradient (call fgx_conv_wgrad_sweep then; fgx_conv_wgrad refuses `streaming` values other than 0 and 1), and the
+ * sweep entry points exist.  A caller checks the version once after loading the library. */
 int fgx_abi_version(void);
 const char* fgx_last_error(void);
 
@@ -327,6 +330,18 @@ int fgx_conv_wgrad_sweep(int dtype, const void* grad_out, const void* feats, con
                          int sub_rows, int lead, int max_polls, void* scratch, void* grad_weight, void* grad_bias,
                          int bias_offset, fgx_stream_t stream);
 
+/* A wavefront of the sweep that waits for data (rows that have not landed, a ring stage that has not been read) looks at
+ * the progress word a bounded number of times and then goes on, so that the kernel ends whatever happens; it then sets its
+ * give-up word in the scratch, and the sweep's reduction writes NaN into all of grad_weight and grad_bias instead of sums
+ * that may be wrong.  (The optional pacing wait is not data: giving up on it costs speed only and sets nothing.)
+ * fgx_wgrad_sweep_giveup_words returns the number of 32-bit give-up words and their byte offset inside the scratch;
+ * fgx_wgrad_sweep_reduce runs the reduction alone over a scratch that a fgx_conv_wgrad_sweep call with the same plan and
+ * shapes has filled (grad_bias non-null: that call made the bias gradient inside the sweep).  Both exist for tests of the
+ * NaN path and for diagnosis; no counterpart in the reference. */
+size_t fgx_wgrad_sweep_giveup_words(int Ci, int Co, size_t* byte_offset);
+int fgx_wgrad_sweep_reduce(int dtype, const void* plan, size_t n, size_t n_pairs, int Ci, int Co, int V, int sub_rows,
+                           void* scratch, void* grad_weight, void* grad_bias, int bias_offset, fgx_stream_t stream);
+
 /* grad_bias[co] = sum over rows of grad_out[:, co], accumulated in fp32.
  * `scratch`: fgx_colsum_scratch_bytes bytes of fp32 partial sums.
  * Replaces: grad_output.sum(0), ..._bwd_masked_implicit_gemm_splitk.py:365-366. */
@@ -340,7 +355,13 @@ int fgx_colsum(int dtype, const void* grad_out, size_t n, int cols, void* scratc
  * refused with FGX_ERR_ARG).  Allocates nothing, same kernels and same bits as fgx_colsum.  All calls on one GPU share
  * that array: calls that may overlap there (different streams, different threads) race -- serialise them.  Every
  * call overwrites the part it reads, so nothing has to be cleared between calls.
+ * The first use on a device looks up that device's address of the array, which may load the code object and is no
+ * stream operation: it cannot happen under capture.  Call fgx_colsum_static_prepare() once per device, with that device
+ * current, before capturing (any earlier fgx_colsum_static call on the device does the same); a first use on a stream
+ * that is being captured is refused with FGX_ERR_ARG.  A caller that also wants the kernels loaded before the capture
+ * makes one ordinary call of the same dtype first.
  * No counterpart in the reference (torch allocates its reduction buffers itself). */
+int fgx_colsum_static_prepare(void);
 int fgx_colsum_static_max_cols(void);
 int fgx_colsum_static(int dtype, const void* grad_out, size_t n, int cols, void* out, fgx_stream_t stream);
 

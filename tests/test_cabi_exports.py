@@ -36,7 +36,7 @@ def test_every_declared_symbol_is_exported(library):
 
 def test_host_only_entry_points(library):
     # these touch no device: identity, sizing and the schedule table
-    assert library.fgx_abi_version() == 1
+    assert library.fgx_abi_version() == 2
     L = nat.lib()
     import torch
     s = nat.table_lookup(nat.PASS_FWD, torch.float16, 669288, 128, 128, 27)
@@ -53,6 +53,17 @@ def test_host_only_entry_points(library):
     assert nat.table_lookup(nat.PASS_WGRAD, torch.float16, 669288, 32, 32, 27).stream == 1
     assert nat.table_lookup(nat.PASS_WGRAD, torch.float16, 4000, 128, 128, 27).stream == 1
     assert nat.table_lookup(nat.PASS_WGRAD, torch.float16, (1 << 24) + 1, 128, 128, 27).stream == 1
+    # the table answers stream = 2 up to 2^24 rows; the host falls back to the block-major kernel where the sweep's own
+    # limits (operands and pair lists below 0xFF000000 bytes) are tighter than that
+    from flexgemm_amd.ops.spconv.submanifold_conv3d import _sweep_fits
+    n_big = 16_711_681                                     # x 128 channels x 2 bytes: just past 0xFF000000
+    assert nat.table_lookup(nat.PASS_WGRAD, torch.float16, n_big, 128, 128, 27).stream == 2
+    assert not _sweep_fits(n_big, n_big, 128, 128, 2, 27 * 1000)
+    assert _sweep_fits(n_big - 1, n_big - 1, 128, 128, 2, 27 * 1000)
+    assert _sweep_fits(669288, 669288, 128, 128, 2, 7082928)
+    assert not _sweep_fits(669288, 669288, 128, 128, 2, 0)                    # no pairs: nothing to sweep
+    assert not _sweep_fits((1 << 24) + 1, 100, 64, 64, 2, 1000)                # 24-bit row numbers
+    assert not _sweep_fits(1 << 24, 1 << 24, 64, 64, 2, (0xFF000000 - 256) // 4 + 1)   # pair lists past the offset range
     assert nat.table_lookup(nat.PASS_WGRAD, torch.float32, 669288, 128, 128, 27).stream == 0
     s = nat.table_lookup(nat.PASS_FWD, torch.float32, 100, 16, 16, 27)
     assert s.tile_rows in (32, 64, 128) and s.tile_cols == 32 and s.splitk >= 1 and s.stream == 0

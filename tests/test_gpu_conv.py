@@ -461,6 +461,67 @@ def test_sweep_wgrad_is_reproducible_and_close_to_the_block_major_kernel(gpu_dev
     assert eg.max_rel_err(outs[0][1], outs[2][1].double()) <= 2e-3
 
 
+def test_sweep_wgrad_give_up_word_turns_the_result_into_nan(gpu_device):
+    """A sweep wavefront whose wait for data runs out of looks goes on and sets its give-up word; the reduction then
+    writes NaN everywhere.  Checked on the reduction alone: a normal sweep fills the scratch (all give-up words 0, result
+    as usual), then one word is set by hand and only the reduction is run again -- no kernel is made to wait."""
+    import ctypes as C
+    from flexgemm_amd import _native as nat
+    _say("sweep wgrad: give-up word -> NaN")
+    L = nat.lib()
+    res, ci, co, v, sub_rows, tile = 32, 128, 64, 27, 256, 128
+    dtype = torch.float16
+    code = nat.DTYPE_CODE[dtype]
+    coords_np = reference_test_shell(res)
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    shape = torch.Size([1, ci, res, res, res])
+    f, _, _, g = _case(coords_np, ci, co, dtype, 37)
+    f, g = f.to(gpu_device), g.to(gpu_device)
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+    cache._ensure_pairs()
+    seg_host = cache._seg_host()
+    n = f.shape[0]
+    plan = cache._wgrad_sweep_plan(sub_rows)
+    seg_arr = (C.c_uint32 * (v + 1))(*seg_host)
+    with torch.cuda.device(gpu_device):
+        scratch = nat.workspace(L.fgx_wgrad_sweep_scratch_bytes(C.c_int(ci), C.c_int(co)), gpu_device)
+        scratch.fill_(0xFF)                          # stale give-up words from "an earlier call": the sweep overwrites them
+        offset = C.c_size_t(0)
+        words = L.fgx_wgrad_sweep_giveup_words(C.c_int(ci), C.c_int(co), C.byref(offset))
+        assert words > 0 and offset.value % 256 == 0 and offset.value + words * 4 <= scratch.numel()
+        flags = scratch[offset.value:offset.value + words * 4].view(torch.int32)
+        gw = torch.empty((co, v, ci), dtype=dtype, device=gpu_device)
+        gb = torch.empty((co,), dtype=dtype, device=gpu_device)
+        nat.check(L.fgx_conv_wgrad_sweep(
+            C.c_int(code), nat.ptr(g), nat.ptr(f), nat.ptr(cache["valid_signal_i"]), nat.ptr(cache["valid_signal_o"]),
+            seg_arr, nat.ptr(plan), nat.sz(n), nat.sz(n), C.c_int(ci), C.c_int(co), C.c_int(v), C.c_int(tile),
+            C.c_int(sub_rows), C.c_int(3), C.c_int(0), nat.ptr(scratch), nat.ptr(gw), nat.ptr(gb), C.c_int(13), nat.stream()))
+        torch.cuda.synchronize()
+        assert int(flags.abs().max()) == 0, "a sweep wavefront gave up waiting on a healthy run"
+        assert bool(torch.isfinite(gw.float()).all()) and bool(torch.isfinite(gb.float()).all())
+
+        def reduce_again():
+            gw2 = torch.zeros_like(gw)
+            gb2 = torch.zeros_like(gb)
+            nat.check(L.fgx_wgrad_sweep_reduce(
+                C.c_int(code), nat.ptr(plan), nat.sz(n), nat.sz(seg_host[-1]), C.c_int(ci), C.c_int(co), C.c_int(v),
+                C.c_int(sub_rows), nat.ptr(scratch), nat.ptr(gw2), nat.ptr(gb2), C.c_int(13), nat.stream()))
+            torch.cuda.synchronize()
+            return gw2, gb2
+
+        gw2, gb2 = reduce_again()                    # untouched scratch: the reduction alone gives the same bits
+        assert torch.equal(gw2, gw) and torch.equal(gb2, gb)
+        for word in (0, words // 2 + 3, words - 1):  # any wavefront's word poisons everything
+            flags.zero_()
+            flags[word] = 1
+            gw2, gb2 = reduce_again()
+            assert bool(torch.isnan(gw2.float()).all()), f"give-up word {word} set, grad_weight not all NaN"
+            assert bool(torch.isnan(gb2.float()).all()), f"give-up word {word} set, grad_bias not all NaN"
+        flags.zero_()
+        gw2, gb2 = reduce_again()
+        assert torch.equal(gw2, gw) and torch.equal(gb2, gb)
+
+
 def test_streaming_wgrad_equals_tiled_wgrad_bitwise(gpu_device):
     """Same 16-pair MFMA blocks in the same order inside every (voxel block, offset) item, same block-ordered
     reduction: the two wgrad kernels agree bit for bit."""

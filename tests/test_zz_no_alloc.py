@@ -57,3 +57,45 @@ def test_static_scratch_colsum_rejects_what_does_not_fit(gpu_device):
     with pytest.raises(ValueError):
         nat.check(L.fgx_colsum_static(C.c_int(nat.DTYPE_CODE[x.dtype]), nat.ptr(x), nat.sz(4), C.c_int(2056), nat.ptr(out), nat.stream()))
     assert b"2048" in L.fgx_last_error()
+
+
+def test_static_scratch_colsum_allocates_nothing_and_replays_in_a_graph(gpu_device):
+    """After the per-device preparation a call leaves the allocator and the device's free memory alone, and it can be
+    captured: every replay, with eager work and synchronisations in between, gives fgx_colsum's bits for the input the
+    captured buffer holds at that moment."""
+    L = nat.lib()
+    dtype = torch.float16
+    code = nat.DTYPE_CODE[dtype]
+    g = torch.Generator().manual_seed(11)
+    n, cols = 40000, 256
+    x = torch.randn(n, cols, generator=g).to(dtype).to(gpu_device)
+    out = torch.empty((cols,), dtype=dtype, device=gpu_device)
+    with torch.cuda.device(gpu_device):
+        nat.check(L.fgx_colsum_static_prepare())
+        # one ordinary call first: the kernels are loaded, and the array holds old partial sums
+        nat.check(L.fgx_colsum_static(C.c_int(code), nat.ptr(x), nat.sz(n), C.c_int(cols), nat.ptr(out), nat.stream()))
+        torch.cuda.synchronize()
+        _say("colsum static: allocation check")
+        allocated, reserved = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+        free_before, _ = torch.cuda.mem_get_info()
+        nat.check(L.fgx_colsum_static(C.c_int(code), nat.ptr(x), nat.sz(n), C.c_int(cols), nat.ptr(out), nat.stream()))
+        torch.cuda.synchronize()
+        free_after, _ = torch.cuda.mem_get_info()
+        assert (torch.cuda.memory_allocated(), torch.cuda.memory_reserved()) == (allocated, reserved)
+        assert free_after == free_before, "device memory changed across a call that must allocate nothing"
+
+        _say("colsum static: capture")
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            nat.check(L.fgx_colsum_static(C.c_int(code), nat.ptr(x), nat.sz(n), C.c_int(cols), nat.ptr(out), nat.stream()))
+        for replay in range(4):
+            _say(f"colsum static: replay {replay}")
+            fresh = torch.randn(n, cols, generator=g).to(dtype).to(gpu_device)
+            x.copy_(fresh)
+            out.fill_(float("nan"))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            want, eager = _colsum_pair(fresh)           # eager work between the replays
+            assert torch.equal(out, want), f"replay {replay} differs from the eager result"
+            assert torch.equal(eager, want)
