@@ -69,6 +69,8 @@ def parse():
     p.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (used under rocprofv3)")
     p.add_argument("--cpu-rows", type=int, default=0, help="rows in the CPU baseline sample (0 = auto)")
     p.add_argument("--build-only", action="store_true", help="time only the neighbor-cache build")
+    p.add_argument("--no-others", action="store_true", help="skip the other configurations that follow the headline one")
+    p.add_argument("--other-steps", type=int, default=10, help="timed steps of each of the other configurations")
     p.add_argument("--calibrate-copy", action="store_true",
                    help="also run a plain 1 GiB device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     return p.parse_args()
@@ -149,173 +151,213 @@ def main():
                     sc.stream, sc.block_rows = 1, args.wgrad_block_major
             return sc
         nat.table_lookup = with_wgrad_kernel
-    wl = make_workload(args.workload, dtype={v: k for k, v in names.items()}.get(args.dtype))
-    dt = wl.dtype
-    dname = names[dt]
-    c = wl.channels
-    passes = 1 if args.workload == "cfg2" else 3
-    coords = wl.coords.to(dev)
-    feats = wl.feats.to(dt).to(dev).requires_grad_(passes == 3)
-    weight = wl.weight.to(dt).to(dev).requires_grad_(passes == 3)
-    bias = wl.bias.to(dt).to(dev).requires_grad_(passes == 3)
-    grad = wl.grad.to(dt).to(dev)
 
-    # ---- neighbor cache: built once, timed separately ----
-    def build_cache():
-        return SubMConv3dFunction._compute_neighbor_cache(coords, wl.shape, (3, 3, 3), (1, 1, 1), passes == 3)
+    def measure(workload, dtype_name, steps, warmup, full, time_hash_builder=False):
+        """One configuration: cache build (timed), warm-up, `steps` timed steps.  full: also the build's phases."""
+        wl = make_workload(workload, dtype={v: k for k, v in names.items()}.get(dtype_name))
+        dt = wl.dtype
+        dname = names[dt]
+        c = wl.channels
+        passes = 1 if workload == "cfg2" else 3
+        coords = wl.coords.to(dev)
+        feats = wl.feats.to(dt).to(dev).requires_grad_(passes == 3)
+        weight = wl.weight.to(dt).to(dev).requires_grad_(passes == 3)
+        bias = wl.bias.to(dt).to(dev).requires_grad_(passes == 3)
+        grad = wl.grad.to(dt).to(dev)
 
-    cache = build_cache()
-    torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    build_ms = []
-    for _ in range(5):
-        ev0.record()
+        # ---- neighbor cache: built once, timed separately ----
+        def build_cache():
+            return SubMConv3dFunction._compute_neighbor_cache(coords, wl.shape, (3, 3, 3), (1, 1, 1), passes == 3)
+
         cache = build_cache()
-        ev1.record()
         torch.cuda.synchronize()
-        build_ms.append(ev0.elapsed_time(ev1))
-    build_ms.sort()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        build_ms = []
+        for _ in range(5):
+            ev0.record()
+            cache = build_cache()
+            ev1.record()
+            torch.cuda.synchronize()
+            build_ms.append(ev0.elapsed_time(ev1))
+        build_ms.sort()
+        hash_build_ms = None
+        if time_hash_builder:
+            flex_gemm.ops.spconv.set_neighbor_map_builder("hash")
+            try:
+                hash_build_ms = []
+                for _ in range(4):          # (the first one also warms the allocator up for the hash table)
+                    ev0.record()
+                    build_cache()
+                    ev1.record()
+                    torch.cuda.synchronize()
+                    hash_build_ms.append(ev0.elapsed_time(ev1))
+                hash_build_ms = sorted(hash_build_ms[1:])
+            finally:
+                flex_gemm.ops.spconv.set_neighbor_map_builder("auto")
 
-    # the build split into its phases: the library names them to a hook, which records an event on their stream; the
-    # first forward of a fresh cache adds the tables made on first use (tile masks, gather plan)
-    def build_phases(reps=5):
-        marks = []
+        # the build split into its phases: the library names them to a hook, which records an event on their stream; the
+        # first forward of a fresh cache adds the tables made on first use (tile masks, gather plan)
+        def build_phases(reps=5):
+            marks = []
 
-        def hook(name, stream):
+            def hook(name, stream):
+                e = torch.cuda.Event(enable_timing=True)
+                e.record(torch.cuda.current_stream())
+                marks.append((name, e))
+
+            gap = "between calls (host: allocations, read-backs)"
+            runs = []
+            nat.set_phase_hook(hook)
+            try:
+                for _ in range(reps):
+                    del marks[:]
+                    fresh = build_cache()
+                    with torch.no_grad():
+                        SubMConv3dFunction._sparse_submanifold_conv_forward(feats, fresh, weight, bias)
+                    torch.cuda.synchronize()
+                    once = {}
+                    for (name, e0), (_, e1) in zip(marks[:-1], marks[1:]):
+                        once[name or gap] = once.get(name or gap, 0.0) + e0.elapsed_time(e1)
+                    runs.append(once)
+            finally:
+                nat.set_phase_hook(None)
+            return {k: sorted(r.get(k, 0.0) for r in runs)[len(runs) // 2] for k in runs[-1]}
+
+        phases_ms = build_phases() if full else None
+        pairs = int(cache.valid_signal_seg.view(torch.int32)[-1].item()) if passes == 3 else \
+            int((cache.neighbor_map.view(torch.int32) != -1).sum().item())
+        n = wl.n
+        build_bytes = 152.0 * n + (8.0 * pairs + 4 * 28 if passes == 3 else 0.0)
+        if args.build_only:
+            return {"metric": "neighbor-cache build", "workload": workload, "n": n, "pairs": pairs,
+                    "build_ms_median": build_ms[len(build_ms) // 2], "build_ms_min": build_ms[0],
+                    "algorithmic_GBps": build_bytes / (build_ms[len(build_ms) // 2] * 1e-3) / 1e9,
+                    "phases_ms_median": phases_ms}, None, None, None
+
+        # ---- the step ----
+        def step():
+            out = SubMConv3dFunction._sparse_submanifold_conv_forward(feats, cache, weight, bias)
+            if passes == 3:
+                return out, SubMConv3dFunction._sparse_submanifold_conv_backward(grad, feats, cache, weight, bias)
+            return out, None
+
+        for _ in range(max(warmup, 1)):
+            step()
+        torch.cuda.synchronize()
+        if args.calibrate_copy and full:
+            # a plain copy kernel of known size: reads 1 GiB, writes 1 GiB per launch
+            a = torch.empty(1 << 29, dtype=torch.float16, device=dev).fill_(1.0)
+            b = torch.empty_like(a)
+            for _ in range(3):
+                torch.neg(a, out=b)
+            torch.cuda.synchronize()
+            del a, b
+
+        # HIP events around the dominant kernel's launches, on the stream they are launched on
+        events = {}
+
+        def hook(name, phase):
             e = torch.cuda.Event(enable_timing=True)
             e.record(torch.cuda.current_stream())
-            marks.append((name, e))
+            events.setdefault(name, []).append(e)
 
-        gap = "between calls (host: allocations, read-backs)"
-        runs = []
-        nat.set_phase_hook(hook)
-        try:
-            for _ in range(reps):
-                del marks[:]
-                fresh = build_cache()
-                with torch.no_grad():
-                    SubMConv3dFunction._sparse_submanifold_conv_forward(feats, fresh, weight, bias)
-                torch.cuda.synchronize()
-                once = {}
-                for (name, e0), (_, e1) in zip(marks[:-1], marks[1:]):
-                    once[name or gap] = once.get(name or gap, 0.0) + e0.elapsed_time(e1)
-                runs.append(once)
-        finally:
-            nat.set_phase_hook(None)
-        return {k: sorted(r.get(k, 0.0) for r in runs)[len(runs) // 2] for k in runs[-1]}
-
-    phases_ms = build_phases()
-    pairs = int(cache.valid_signal_seg.view(torch.int32)[-1].item()) if passes == 3 else \
-        int((cache.neighbor_map.view(torch.int32) != -1).sum().item())
-    n = wl.n
-    build_bytes = 152.0 * n + (8.0 * pairs + 4 * 28 if passes == 3 else 0.0)
-    if args.build_only:
-        print(json.dumps({"metric": "neighbor-cache build", "workload": args.workload, "n": n, "pairs": pairs,
-                          "build_ms_median": build_ms[len(build_ms) // 2], "build_ms_min": build_ms[0],
-                          "algorithmic_GBps": build_bytes / (build_ms[len(build_ms) // 2] * 1e-3) / 1e9,
-                          "phases_ms_median": phases_ms}))
-        return
-
-    # ---- the step ----
-    def step():
-        out = SubMConv3dFunction._sparse_submanifold_conv_forward(feats, cache, weight, bias)
-        if passes == 3:
-            return out, SubMConv3dFunction._sparse_submanifold_conv_backward(grad, feats, cache, weight, bias)
-        return out, None
-
-    for _ in range(max(args.warmup, 1)):
-        step()
-    torch.cuda.synchronize()
-    if args.calibrate_copy:
-        # a plain copy kernel of known size: reads 1 GiB, writes 1 GiB per launch
-        a = torch.empty(1 << 29, dtype=torch.float16, device=dev).fill_(1.0)
-        b = torch.empty_like(a)
-        for _ in range(3):
-            torch.neg(a, out=b)
+        nat.EVENT_HOOK = hook
+        step_events = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
         torch.cuda.synchronize()
-        del a, b
+        torch.cuda.reset_peak_memory_stats(dev)
+        t0 = time.perf_counter()
+        for i in range(steps):
+            step_events[i].record()
+            step()
+        step_events[steps].record()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        nat.EVENT_HOOK = None
+        peak_bytes = torch.cuda.max_memory_allocated(dev)
 
-    # HIP events around the dominant kernel's launches, on the stream they are launched on
-    events = {}
+        ms_per_step = elapsed * 1e3 / steps
+        step_ms = sorted(step_events[i].elapsed_time(step_events[i + 1]) for i in range(steps))
+        flop_pass = 2.0 * pairs * c * c
+        value = flop_pass * passes / (ms_per_step * 1e-3) / 1e12
 
-    def hook(name, phase):
-        e = torch.cuda.Event(enable_timing=True)
-        e.record(torch.cuda.current_stream())
-        events.setdefault(name, []).append(e)
+        def pass_ms(names):
+            """(mean, median, min, count) of the event-timed calls of these names"""
+            ts = []
+            for nm in names:
+                ev = events.get(nm, [])
+                ts += [ev[i].elapsed_time(ev[i + 1]) for i in range(0, len(ev) - 1, 2)]
+            ts.sort()
+            if not ts:
+                return float("nan"), float("nan"), float("nan"), 0
+            return sum(ts) / len(ts), ts[len(ts) // 2], ts[0], len(ts)
 
-    nat.EVENT_HOOK = hook
-    step_events = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
-    torch.cuda.synchronize()
-    torch.cuda.reset_peak_memory_stats(dev)
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step_events[i].record()
-        step()
-    step_events[args.steps].record()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    nat.EVENT_HOOK = None
-    peak_bytes = torch.cuda.max_memory_allocated(dev)
+        def stats(names):
+            mean, med, lo, cnt = pass_ms(names)
+            return {"mean": mean, "median": med, "min": lo, "calls": cnt} if cnt else None
 
-    ms_per_step = elapsed * 1e3 / args.steps
-    step_ms = sorted(step_events[i].elapsed_time(step_events[i + 1]) for i in range(args.steps))
-    flop_pass = 2.0 * pairs * c * c
-    value = flop_pass * passes / (ms_per_step * 1e-3) / 1e12
+        gemm_ms, _, _, gemm_launches = pass_ms(["gather_gemm_fwd", "gather_gemm_dgrad"])
+        wgrad_ms = pass_ms(["wgrad"])[0]
+        es = 2 if dname != "f32" else 4
+        gemm_bytes = es * n * (c + c) + es * 27 * c * c + 108.0 * n + 8.0 * n
+        roof = {
+            "bound": "mfma", "kernel": "gather GEMM (gather_gemm_stream_kernel or gather_gemm_kernel; forward and dgrad launches)",
+            "achieved": flop_pass / (gemm_ms * 1e-3) / 1e12, "peak": PEAK_TFLOPS[dname], "unit": "TFLOP/s",
+            "frac": flop_pass / (gemm_ms * 1e-3) / 1e12 / PEAK_TFLOPS[dname],
+            "avg_launch_ms": gemm_ms, "launches_timed": gemm_launches,
+            "algorithmic_flop_per_launch": flop_pass,
+            "algorithmic_bytes_per_launch": gemm_bytes,
+            "algorithmic_hbm_GBps": gemm_bytes / (gemm_ms * 1e-3) / 1e9,
+            "traffic": measured_traffic(workload, dname),
+        }
+        if c * es <= 64:   # rows of 64 bytes (configuration 4, C = 32): every pass is HBM bound
+            roof.update({"bound": "hbm", "achieved": gemm_bytes / (gemm_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": gemm_bytes / (gemm_ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
 
-    def pass_ms(names):
-        """(mean, median, min, count) of the event-timed calls of these names"""
-        ts = []
-        for nm in names:
-            ev = events.get(nm, [])
-            ts += [ev[i].elapsed_time(ev[i + 1]) for i in range(0, len(ev) - 1, 2)]
-        ts.sort()
-        if not ts:
-            return float("nan"), float("nan"), float("nan"), 0
-        return sum(ts) / len(ts), ts[len(ts) // 2], ts[0], len(ts)
+        result = {
+            "metric": "effective TFLOPS (useful MACs over valid neighbor pairs), submconv3d 3^3 "
+                      + ("fwd+dgrad+wgrad" if passes == 3 else "fwd") + f", res{wl.res} C={c}",
+            "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": dname, "data": "synthetic",
+            "config": {"workload": f"{workload}: res {wl.res} shell, N={n}, L={pairs}, Ci=Co={c}, {dname}, "
+                                   + ("fwd+dgrad+wgrad+dbias, neighbor cache prebuilt and reused" if passes == 3 else "forward"),
+                       "n_voxels": n, "valid_pairs": pairs, "useful_gflop_per_step": flop_pass * passes / 1e9},
+            "frac_of_mfma_peak": value / PEAK_TFLOPS[dname],
+            "pass_ms": {"gather_gemm_avg": gemm_ms, "wgrad_incl_reduce": wgrad_ms,
+                        "forward": stats(["gather_gemm_fwd"]), "dgrad": stats(["gather_gemm_dgrad"]), "wgrad": stats(["wgrad"])},
+            "step_ms": {"wall_mean": ms_per_step, "median": step_ms[len(step_ms) // 2], "min": step_ms[0]},
+            "peak_memory_bytes": peak_bytes,
+            "neighbor_cache_build": {"ms_median": build_ms[len(build_ms) // 2], "ms_min": build_ms[0],
+                                     "algorithmic_bytes": build_bytes,
+                                     "algorithmic_GBps": build_bytes / (build_ms[len(build_ms) // 2] * 1e-3) / 1e9,
+                                     "frac_of_hbm_peak": build_bytes / (build_ms[len(build_ms) // 2] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                     "phases_ms_median": phases_ms},
+            "roofline": roof,
+        }
+        if hash_build_ms:
+            med = hash_build_ms[len(hash_build_ms) // 2]
+            result["neighbor_cache_build"]["hash_builder"] = {
+                "ms_median": med, "ms_min": hash_build_ms[0], "algorithmic_GBps": build_bytes / (med * 1e-3) / 1e9,
+                "frac_of_hbm_peak": build_bytes / (med * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        return result, wl, cache, passes
 
-    def stats(names):
-        mean, med, lo, cnt = pass_ms(names)
-        return {"mean": mean, "median": med, "min": lo, "calls": cnt} if cnt else None
-
-    gemm_ms, _, _, gemm_launches = pass_ms(["gather_gemm_fwd", "gather_gemm_dgrad"])
-    wgrad_ms = pass_ms(["wgrad"])[0]
-    es = 2 if dname != "f32" else 4
-    gemm_bytes = es * n * (c + c) + es * 27 * c * c + 108.0 * n + 8.0 * n
-    roof = {
-        "bound": "mfma", "kernel": "gather GEMM (gather_gemm_stream_kernel or gather_gemm_kernel; forward and dgrad launches)",
-        "achieved": flop_pass / (gemm_ms * 1e-3) / 1e12, "peak": PEAK_TFLOPS[dname], "unit": "TFLOP/s",
-        "frac": flop_pass / (gemm_ms * 1e-3) / 1e12 / PEAK_TFLOPS[dname],
-        "avg_launch_ms": gemm_ms, "launches_timed": gemm_launches,
-        "algorithmic_flop_per_launch": flop_pass,
-        "algorithmic_bytes_per_launch": gemm_bytes,
-        "algorithmic_hbm_GBps": gemm_bytes / (gemm_ms * 1e-3) / 1e9,
-        "traffic": measured_traffic(args.workload, dname),
-    }
-    if c * es <= 64:   # rows of 64 bytes (configuration 4, C = 32): every pass is HBM bound
-        roof.update({"bound": "hbm", "achieved": gemm_bytes / (gemm_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": gemm_bytes / (gemm_ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
-
-    result = {
-        "metric": "effective TFLOPS (useful MACs over valid neighbor pairs), submconv3d 3^3 "
-                  + ("fwd+dgrad+wgrad" if passes == 3 else "fwd") + f", res{wl.res} C={c}",
-        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": dname, "data": "synthetic",
-        "config": {"workload": f"{args.workload}: res {wl.res} shell, N={n}, L={pairs}, Ci=Co={c}, {dname}, "
-                               + ("fwd+dgrad+wgrad+dbias, neighbor cache prebuilt and reused" if passes == 3 else "forward"),
-                   "n_voxels": n, "valid_pairs": pairs, "useful_gflop_per_step": flop_pass * passes / 1e9},
-        "frac_of_mfma_peak": value / PEAK_TFLOPS[dname],
-        "pass_ms": {"gather_gemm_avg": gemm_ms, "wgrad_incl_reduce": wgrad_ms,
-                    "forward": stats(["gather_gemm_fwd"]), "dgrad": stats(["gather_gemm_dgrad"]), "wgrad": stats(["wgrad"])},
-        "step_ms": {"wall_mean": ms_per_step, "median": step_ms[len(step_ms) // 2], "min": step_ms[0]},
-        "peak_memory_bytes": peak_bytes,
-        "neighbor_cache_build": {"ms_median": build_ms[len(build_ms) // 2], "ms_min": build_ms[0],
-                                 "algorithmic_bytes": build_bytes,
-                                 "algorithmic_GBps": build_bytes / (build_ms[len(build_ms) // 2] * 1e-3) / 1e9,
-                                 "frac_of_hbm_peak": build_bytes / (build_ms[len(build_ms) // 2] * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                                 "phases_ms_median": phases_ms},
-        "roofline": roof,
-    }
+    result, wl, cache, passes = measure(args.workload, args.dtype, args.steps, args.warmup, True)
+    if args.build_only:
+        print(json.dumps(result))
+        return
+    if not args.no_others and args.workload == "cfg3" and args.dtype is None:
+        # the other configurations, a few steps each (no CPU leg, no phase split); configuration 4 also with the hash builder
+        others = []
+        for wname, dn in (("cfg2", None), ("cfg4", None), ("cfg5", None), ("cfg5", "f32")):
+            r, _, _, _ = measure(wname, dn, args.other_steps, 3, False, time_hash_builder=(wname == "cfg4"))
+            others.append({"workload": wname, "dtype": r["dtype"], "ms_per_step": r["ms_per_step"], "value": r["value"],
+                           "unit": r["unit"], "steps": args.other_steps, "config": r["config"]["workload"],
+                           "frac_of_mfma_peak": r["frac_of_mfma_peak"],
+                           "roofline": {k: r["roofline"][k] for k in ("bound", "achieved", "peak", "unit", "frac", "avg_launch_ms")},
+                           "pass_ms": r["pass_ms"], "step_ms": r["step_ms"],
+                           "neighbor_cache_build": {k: v for k, v in r["neighbor_cache_build"].items() if k != "phases_ms_median"}})
+            torch.cuda.empty_cache()
+        result["other_workloads"] = others
     if not args.no_cpu_baseline:
         nmap_cpu = cache.neighbor_map.cpu().view(torch.int32)
         result["cpu_baseline"] = cpu_baseline(wl, nmap_cpu, passes, args.cpu_rows)

@@ -189,8 +189,8 @@ def neighbor_map_post_process_for_masked_implicit_gemm_1(neighbor_map: torch.Ten
     _check_map(neighbor_map)
     nmap = neighbor_map.contiguous()
     gray, _, order = _codes_and_order(nmap, None, None)
-    sig_i, sig_o, seg, _ = _pair_lists(nmap, gray)
-    return gray, order, sig_i, sig_o, seg
+    pairs = _pair_lists(nmap, gray, exact=True)
+    return gray, order, pairs["sig_i"], pairs["sig_o"], pairs["seg"]
 
 
 def neighbor_map_post_process_for_masked_implicit_gemm_2(gray_code: torch.Tensor, sorted_idx: torch.Tensor,

@@ -253,11 +253,7 @@ class SparseConv3dFunction(Function):
         cache = SparseConv3dNeighborCache(neighbor_map=nmap, neighbor_map_bwd=nmap_bwd, gray_code=gray, sorted_idx=order,
                                           _n_in=coords.shape[0])
         if needs_grad:
-            sig_i, sig_o, seg, seg_host = _pair_lists(nmap, gray)
-            cache["valid_signal_seg"] = seg
-            cache["valid_signal_i"] = sig_i
-            cache["valid_signal_o"] = sig_o
-            cache["_valid_signal_seg_host"] = seg_host
+            cache._attach_pairs(_pair_lists(nmap, gray))
             if any(s != 1 for s in st) or is_out_coords_given:
                 # irregular backward masks: sort the input rows by theirs, as the reference does (:191-207); otherwise
                 # nearly every input reaches every kernel position and the input gradient runs unsorted

@@ -55,6 +55,34 @@ class SubMConv3dNeighborCache:
     def __contains__(self, key):
         return hasattr(self, key)
 
+    # The pair lists are filled while their length L is still on its way to the host: they are allocated at their bound
+    # (one entry per slot of the map) and cut to L when somebody first reads them or the host copy of the segment
+    # table, which by then has long arrived.  (__getattr__ is only asked for names that are not there yet.)
+    _PENDING = ("valid_signal_i", "valid_signal_o", "_valid_signal_seg_host")
+
+    def __getattr__(self, name):
+        if name in SubMConv3dNeighborCache._PENDING and "_pending_pairs" in self.__dict__:
+            self._finish_pairs()
+            return self.__dict__[name]
+        raise AttributeError(name)
+
+    def _attach_pairs(self, pairs):
+        """Take the result of _pair_lists: finished lists, or buffers whose length is still in flight."""
+        self["valid_signal_seg"] = pairs["seg"]
+        if "pending" in pairs:
+            self.__dict__["_pending_pairs"] = pairs["pending"]
+        else:
+            self["valid_signal_i"], self["valid_signal_o"] = pairs["sig_i"], pairs["sig_o"]
+            self["_valid_signal_seg_host"] = pairs["seg_host"]
+
+    def _finish_pairs(self):
+        buf_i, buf_o, seg_pinned, arrived = self.__dict__.pop("_pending_pairs")
+        arrived.synchronize()
+        seg_host = [x & 0xFFFFFFFF for x in seg_pinned.tolist()]
+        total = seg_host[-1]
+        self["valid_signal_i"], self["valid_signal_o"] = buf_i[:total], buf_o[:total]
+        self["_valid_signal_seg_host"] = seg_host
+
     # -- per-tile offset lists -------------------------------------------------------------------
     def _tile_tables(self, block_size: int, private: bool):
         """(order int64 [N], tile_code int32 [nb], seg int32 [nb+1]) for tiles of `block_size` rows; no host sync.
@@ -103,8 +131,8 @@ class SubMConv3dNeighborCache:
     def _gather_plan(self, block_size: int, private: bool, dense: bool = False):
         """(order, tile_code int32 [nb], plan_seg int32 [nb+1], plan_idx uint32 [P, block_size], plan_band uint32 [P])
         for the streaming GEMM: per tile and offset present in it, the tile's source rows as one contiguous run and the
-        mask of its 32-row bands that hold any.  Built once per tile size (one 4-byte read-back sizes it) and kept with
-        the cache."""
+        mask of its 32-row bands that hold any.  Built once per tile size and kept with the cache; the lists are
+        allocated at their bound (every offset present in every tile), plan_seg[-1] rows of them are used."""
         if dense:
             order, code = self._dense_tile_tables(block_size)
             key = f"_plan_d_{block_size}"
@@ -123,7 +151,7 @@ class SubMConv3dNeighborCache:
                 ws = nat.workspace(L.fgx_tile_workspace_bytes(nat.sz(nb), C.c_int(1)), dev)
                 nat.check(L.fgx_gather_plan_count(nat.ptr(code), nat.sz(nb), nat.ptr(seg), nat.ptr(ws), nat.sz(ws.numel()),
                                                   nat.stream()))
-                rows = int(seg[-1].item())
+                rows = nb * min(v, 32)       # the bound (every offset in every tile): no wait for the exact count
                 plan_idx = torch.empty((rows, block_size), dtype=torch.uint32, device=dev)
                 plan_band = torch.empty((rows,), dtype=torch.uint32, device=dev)
                 nat.check(L.fgx_gather_plan_fill(nat.ptr(nmap), nat.ptr(order), nat.ptr(code), nat.ptr(seg), nat.sz(n),
@@ -211,9 +239,7 @@ class SubMConv3dNeighborCache:
         if hasattr(self, "valid_signal_i") and hasattr(self, "valid_signal_o") and hasattr(self, "valid_signal_seg"):
             return
         self._ensure_sorted()
-        sig_i, sig_o, seg, seg_host = _pair_lists(self["neighbor_map"], self["gray_code"])
-        self["valid_signal_i"], self["valid_signal_o"], self["valid_signal_seg"] = sig_i, sig_o, seg
-        self["_valid_signal_seg_host"] = seg_host
+        self._attach_pairs(_pair_lists(self["neighbor_map"], self["gray_code"]))
 
     def _wgrad_bounds(self, block_rows: int):
         """First pair of every (offset, voxel block) for wgrad's blocks of `block_rows` rows: a function of the pair lists
@@ -295,7 +321,16 @@ def _locality_order(coords: torch.Tensor, binary: torch.Tensor, v: int) -> torch
     return order
 
 
-def _pair_lists(nmap: torch.Tensor, gray: torch.Tensor):
+# pair lists up to this many bytes (both together, at their bound of one entry per slot of the map) are allocated before
+# their length is known, which saves the build its wait for the host; larger ones wait and are allocated exactly
+PAIR_LISTS_UNSIZED_MAX_BYTES = 2 << 30
+
+
+def _pair_lists(nmap: torch.Tensor, gray: torch.Tensor, exact: bool = False):
+    """The (input row, output row) lists per offset and their segment table (reference: migemm_neighmap_pp.cu:180-260).
+    Returns {"seg", "sig_i", "sig_o", "seg_host"}, or {"seg", "pending"} when the lists were filled into buffers of the
+    bound's size without waiting for their length (SubMConv3dNeighborCache._attach_pairs takes either); exact=True
+    always waits and returns the finished lists."""
     n, v = nmap.shape
     dev = nmap.device
     L = nat.lib()
@@ -304,14 +339,25 @@ def _pair_lists(nmap: torch.Tensor, gray: torch.Tensor):
         ws = nat.workspace(L.fgx_pair_workspace_bytes(nat.sz(n), C.c_int(v)), dev)
         nat.check(L.fgx_pair_count(nat.ptr(gray), nat.sz(n), C.c_int(v), nat.ptr(seg), nat.ptr(ws), nat.sz(ws.numel()),
                                    nat.stream()))
-        seg_host = [x & 0xFFFFFFFF for x in seg.view(torch.int32).cpu().tolist()]   # the one host sync: sizes L
+        bound = n * v
+        if not exact and 0 < bound * 8 <= PAIR_LISTS_UNSIZED_MAX_BYTES:
+            seg_pinned = torch.empty((v + 1,), dtype=torch.int32, pin_memory=True)
+            seg_pinned.copy_(seg.view(torch.int32), non_blocking=True)
+            arrived = torch.cuda.Event()
+            arrived.record()
+            buf_i = torch.empty((bound,), dtype=torch.uint32, device=dev)
+            buf_o = torch.empty((bound,), dtype=torch.uint32, device=dev)
+            nat.check(L.fgx_pair_fill(nat.ptr(nmap), nat.ptr(gray), nat.sz(n), C.c_int(v), nat.ptr(ws), nat.ptr(buf_i),
+                                      nat.ptr(buf_o), nat.stream()))
+            return {"seg": seg, "pending": (buf_i, buf_o, seg_pinned, arrived)}
+        seg_host = [x & 0xFFFFFFFF for x in seg.view(torch.int32).cpu().tolist()]   # a host sync: sizes L
         total = seg_host[-1]
         sig_i = torch.empty((total,), dtype=torch.uint32, device=dev)
         sig_o = torch.empty((total,), dtype=torch.uint32, device=dev)
         if total:
             nat.check(L.fgx_pair_fill(nat.ptr(nmap), nat.ptr(gray), nat.sz(n), C.c_int(v), nat.ptr(ws), nat.ptr(sig_i),
                                       nat.ptr(sig_o), nat.stream()))
-    return sig_i, sig_o, seg, seg_host
+    return {"seg": seg, "sig_i": sig_i, "sig_o": sig_o, "seg_host": seg_host}
 
 
 def _build_neighbor_map(coords: torch.Tensor, shape, kernel_size, dilation, with_codes: bool):
@@ -641,11 +687,7 @@ class SubMConv3dFunction(Function):
         cache["_coords"] = coords           # for the private row order, built on first use by a short-row layer
         cache["_binary_code"] = binary
         if needs_grad:
-            sig_i, sig_o, seg, seg_host = _pair_lists(nmap, gray)
-            cache["valid_signal_seg"] = seg
-            cache["valid_signal_i"] = sig_i
-            cache["valid_signal_o"] = sig_o
-            cache["_valid_signal_seg_host"] = seg_host
+            cache._attach_pairs(_pair_lists(nmap, gray))
         return cache
 
     @staticmethod
