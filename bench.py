@@ -32,25 +32,29 @@ if ROOT not in sys.path:
 
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}   # MI355X dense MFMA peaks
 HBM_PEAK_GBS = 8000.0
-# HBM-side bytes per launch of the dominant kernel come from two rocprofv3 counter runs of this script (FETCH_SIZE, then
-# WRITE_SIZE, each scaled by what the same counter reads for the plain copy of --calibrate-copy).  The counters cannot
-# be read from inside the process: `python -m flexgemm_amd.profile_traffic` turns the two counter files into an entry of
-# this file, stamped with a digest of the kernel's source files, and the summary under profiles/ quotes the same entry.
+# HBM-side bytes per launch of the dominant kernels come from two rocprofv3 counter runs of this script (FETCH_SIZE, then
+# WRITE_SIZE, each scaled by what the same counter reads for the plain copy of --calibrate-copy), MFMA-busy share, clock and
+# L2 hit rate from two more.  The counters cannot be read from inside the process: `python -m flexgemm_amd.profile_traffic`
+# turns the counter files into an entry of this file, stamped with a digest of each kernel's source files, and the summary
+# under profiles/ quotes the same entry.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
 
 
-def measured_traffic(workload: str, dname: str):
-    """Bytes per launch of the dominant kernel from profiles/traffic.json, or None when there is no entry for this
-    workload and dtype or the kernel's sources have changed since it was measured."""
+def measured_counters(workload: str, dname: str, role: str):
+    """{traffic_bytes, mfma_busy_frac, l2_hit, clock_ghz} per launch of a role's kernel ("gemm": the gather GEMM, "wgrad":
+    the weight gradient) from profiles/traffic.json; every value is None when there is no entry for this workload and
+    dtype or the kernel's sources have changed since it was measured."""
     from flexgemm_amd.profile_traffic import source_digest
+    keys = ("traffic_bytes", "mfma_busy_frac", "l2_hit", "clock_ghz")
+    none = {k: None for k in keys}
     try:
         with open(TRAFFIC_FILE) as f:
-            entry = json.load(f).get(f"{workload}_{dname}")
+            entry = json.load(f).get(f"{workload}_{dname}", {}).get(role)
     except (OSError, ValueError):
-        return None
+        return none
     if not entry or entry.get("source_digest") != source_digest(entry.get("sources", [])):
-        return None
-    return entry.get("traffic_bytes")
+        return none
+    return {k: entry.get(k) for k in keys}
 
 
 def parse():
@@ -307,11 +311,28 @@ def main():
             "algorithmic_flop_per_launch": flop_pass,
             "algorithmic_bytes_per_launch": gemm_bytes,
             "algorithmic_hbm_GBps": gemm_bytes / (gemm_ms * 1e-3) / 1e9,
-            "traffic": measured_traffic(workload, dname),
         }
+        seen = measured_counters(workload, dname, "gemm")
+        roof.update({"traffic": seen["traffic_bytes"], "mfma_busy_frac": seen["mfma_busy_frac"], "l2_hit": seen["l2_hit"],
+                     "clock_ghz": seen["clock_ghz"]})
         if c * es <= 64:   # rows of 64 bytes (configuration 4, C = 32): every pass is HBM bound
             roof.update({"bound": "hbm", "achieved": gemm_bytes / (gemm_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": gemm_bytes / (gemm_ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
+
+        wgrad_roof = None
+        if passes == 3 and wgrad_ms == wgrad_ms:
+            wgrad_bytes = es * n * (c + c) + 8.0 * pairs + es * 27 * c * c
+            seen = measured_counters(workload, dname, "wgrad")
+            wgrad_roof = {
+                "bound": "mfma", "kernel": "weight gradient (wgrad_sweep_kernel + its reduction, or the block-major kernels)",
+                "achieved": flop_pass / (wgrad_ms * 1e-3) / 1e12, "peak": PEAK_TFLOPS[dname], "unit": "TFLOP/s",
+                "frac": flop_pass / (wgrad_ms * 1e-3) / 1e12 / PEAK_TFLOPS[dname], "avg_launch_ms": wgrad_ms,
+                "algorithmic_flop_per_launch": flop_pass, "algorithmic_bytes_per_launch": wgrad_bytes,
+                "traffic": seen["traffic_bytes"], "mfma_busy_frac": seen["mfma_busy_frac"], "l2_hit": seen["l2_hit"],
+                "clock_ghz": seen["clock_ghz"]}
+            if c * es <= 64:
+                wgrad_roof.update({"bound": "hbm", "achieved": wgrad_bytes / (wgrad_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
+                                   "unit": "GB/s", "frac": wgrad_bytes / (wgrad_ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
 
         result = {
             "metric": "effective TFLOPS (useful MACs over valid neighbor pairs), submconv3d 3^3 "
@@ -333,6 +354,7 @@ def main():
                                      "frac_of_hbm_peak": build_bytes / (build_ms[len(build_ms) // 2] * 1e-3) / 1e9 / HBM_PEAK_GBS,
                                      "phases_ms_median": phases_ms},
             "roofline": roof,
+            "wgrad_roofline": wgrad_roof,
         }
         if hash_build_ms:
             med = hash_build_ms[len(hash_build_ms) // 2]
@@ -354,6 +376,8 @@ def main():
                            "unit": r["unit"], "steps": args.other_steps, "config": r["config"]["workload"],
                            "frac_of_mfma_peak": r["frac_of_mfma_peak"],
                            "roofline": {k: r["roofline"][k] for k in ("bound", "achieved", "peak", "unit", "frac", "avg_launch_ms")},
+                           "wgrad_roofline": None if r["wgrad_roofline"] is None else
+                           {k: r["wgrad_roofline"][k] for k in ("bound", "achieved", "peak", "unit", "frac", "avg_launch_ms")},
                            "pass_ms": r["pass_ms"], "step_ms": r["step_ms"],
                            "neighbor_cache_build": {k: v for k, v in r["neighbor_cache_build"].items() if k != "phases_ms_median"}})
             torch.cuda.empty_cache()

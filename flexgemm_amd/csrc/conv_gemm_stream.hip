@@ -43,6 +43,13 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), (short)0, (int)bytes, 0x00020000);
 }
 
+// multiplier wavefronts along the rows of the 256 x 128 tile with 128-byte slabs: 4 (x 2 along the columns: eight
+// multipliers with 64 x 64 wave tiles), or 2 (four multipliers with 128 x 64 wave tiles: 6 instead of 8 fragment reads
+// per 8 products)
+#ifndef FGX_BIG_WAVES_M
+#define FGX_BIG_WAVES_M 4
+#endif
+
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int CH>
 struct StreamCfg {
     using T = typename Tag::type;
@@ -549,7 +556,7 @@ int dispatch_stream(int tile_rows, int tile_cols, int slab_bytes, const void* sr
     if (tile_rows == BM && tile_cols == BN && slab_bytes == CHv * 16)                                                   \
         return launch_stream<Tag, BM, BN, WMv, WNv, CHv>(src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band,  \
                                                          plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, act, out, s);
-    FGX_STREAM_TILE(256, 128, 4, 2, 8)
+    FGX_STREAM_TILE(256, 128, FGX_BIG_WAVES_M, 2, 8)
     FGX_STREAM_TILE(256, 64, 4, 2, 8)
     FGX_STREAM_TILE(256, 128, 4, 2, 4)      // 64-byte K-slabs: rows shorter than 128 bytes
     FGX_STREAM_TILE(256, 64, 4, 2, 4)
@@ -617,7 +624,7 @@ bool stream_lds_fits(int tile_rows, int tile_cols, int slab_bytes, int cols) {
     size_t fixed = 0;       // (the ring sizes do not depend on the element type)
 #define FGX_STREAM_TILE(BM, BN, WMv, WNv, CHv) \
     if (tile_rows == BM && tile_cols == BN && slab_bytes == CHv * 16) fixed = StreamCfg<F16, BM, BN, WMv, WNv, CHv>::fixed_lds;
-    FGX_STREAM_TILE(256, 128, 4, 2, 8)
+    FGX_STREAM_TILE(256, 128, FGX_BIG_WAVES_M, 2, 8)
     FGX_STREAM_TILE(256, 64, 4, 2, 8)
     FGX_STREAM_TILE(256, 128, 4, 2, 4)
     FGX_STREAM_TILE(256, 64, 4, 2, 4)
@@ -636,7 +643,7 @@ extern "C" int fgx_conv_gather_gemm_stream_groups(int dtype, int cols, int tile_
     if (tile_rows == BM && tile_cols == BN && slab_bytes == CHv * 16)                            \
         return resident_groups<TAG, BM, BN, WMv, WNv, CHv>(StreamCfg<TAG, BM, BN, WMv, WNv, CHv>::fixed_lds + bias_bytes, groups);
 #define FGX_STREAM_TILES(TAG)            \
-    FGX_STREAM_TILE(TAG, 256, 128, 4, 2, 8) \
+    FGX_STREAM_TILE(TAG, 256, 128, FGX_BIG_WAVES_M, 2, 8) \
     FGX_STREAM_TILE(TAG, 256, 64, 4, 2, 8)  \
     FGX_STREAM_TILE(TAG, 256, 128, 4, 2, 4) \
     FGX_STREAM_TILE(TAG, 256, 64, 4, 2, 4)  \
