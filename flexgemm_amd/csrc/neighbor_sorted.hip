@@ -19,6 +19,7 @@
 #include <rocprim/rocprim.hpp>
 
 #include "fgx_common.h"
+#include "radix_sort.h"
 
 namespace fgx {
 namespace {
@@ -42,6 +43,25 @@ __global__ void __launch_bounds__(256) flat_keys_kernel(const int32_t* __restric
     const int4 c = reinterpret_cast<const int4*>(coords)[i];
     keys[i] = (K)((((uint64_t)(uint32_t)c.x * (uint64_t)W + (uint64_t)c.y) * (uint64_t)H + (uint64_t)c.z) * (uint64_t)D + (uint64_t)c.w);
     rows[i] = (uint32_t)i;
+}
+
+// flat_keys_kernel that also tells whether the keys ascend as the voxels come: descents[0] = 1 when some voxel's key is
+// smaller than its predecessor's (the word is cleared by a kernel before this one)
+template <typename K>
+__global__ void __launch_bounds__(256) flat_keys_check_kernel(const int32_t* __restrict__ coords, size_t n, int W, int H, int D,
+                                                              K* __restrict__ keys, uint32_t* __restrict__ rows,
+                                                              uint32_t* __restrict__ descents) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int4 c = reinterpret_cast<const int4*>(coords)[i];
+    const uint64_t kc = (((uint64_t)(uint32_t)c.x * (uint64_t)W + (uint64_t)c.y) * (uint64_t)H + (uint64_t)c.z) * (uint64_t)D + (uint64_t)c.w;
+    keys[i] = (K)kc;
+    rows[i] = (uint32_t)i;
+    if (i > 0) {
+        const int4 a = reinterpret_cast<const int4*>(coords)[i - 1];
+        const uint64_t ka = (((uint64_t)(uint32_t)a.x * (uint64_t)W + (uint64_t)a.y) * (uint64_t)H + (uint64_t)a.z) * (uint64_t)D + (uint64_t)a.w;
+        if (kc < ka) descents[0] = 1u;      // (every writer stores the same value)
+    }
 }
 
 // descents[0] = 1 when some voxel's flattened key is smaller than its predecessor's (the caller clears the word first)
@@ -78,9 +98,13 @@ __device__ __forceinline__ uint32_t gray_decode(uint32_t g) {
 // bounds[(group * R + r) * 2 + {0, 1}] = [first, one past last) position of the window of sorted keys in which the
 // (dx, dy) = r neighbors of the group's voxels lie: the group's own key range shifted by the row's constant and
 // widened by the reach along z.  One thread per bound: the searches of all groups overlap.
+// (`pick` != nullptr: the sorted keys are `skeys` when that word is non-zero and `skeys_if_not` when it is zero -- the
+// key sort ahead of this kernel was conditional on the same word)
 template <typename K>
 __global__ void __launch_bounds__(256) window_bounds_kernel(const K* __restrict__ skeys, size_t n, unsigned long long vol,
-                                                            SubmGeom g, unsigned groups, uint32_t* __restrict__ bounds) {
+                                                            SubmGeom g, unsigned groups, uint32_t* __restrict__ bounds,
+                                                            const uint32_t* __restrict__ pick, const K* __restrict__ skeys_if_not) {
+    if (pick != nullptr && *pick == 0u) skeys = skeys_if_not;
     const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
     const int R = g.Kw * g.Kh;
     if (t >= (size_t)groups * R * 2) return;
@@ -164,7 +188,13 @@ template <typename K>
 __global__ void __launch_bounds__(kGroup) merge_neighbor_kernel(const K* __restrict__ skeys, const uint32_t* __restrict__ srows,
                                                                 const uint32_t* __restrict__ bounds, size_t n, SubmGeom g,
                                                                 uint32_t* __restrict__ out_map,
-                                                                int32_t* __restrict__ gray, int32_t* __restrict__ binary) {
+                                                                int32_t* __restrict__ gray, int32_t* __restrict__ binary,
+                                                                const uint32_t* __restrict__ pick, const K* __restrict__ skeys_if_not,
+                                                                const uint32_t* __restrict__ srows_if_not) {
+    if (pick != nullptr && *pick == 0u) {       // (as in window_bounds_kernel)
+        skeys = skeys_if_not;
+        srows = srows_if_not;
+    }
     constexpr int kPer = kWindow / kGroup;      // window entries a lane carries from memory to LDS
     __shared__ K wkeys[kWindow];
     __shared__ uint32_t wrows[kWindow];
@@ -285,9 +315,18 @@ __global__ void __launch_bounds__(kGroup) merge_neighbor_kernel(const K* __restr
     }
 }
 
+__global__ void __launch_bounds__(256) fill_words_kernel(uint32_t* p, size_t count, uint32_t value) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (; i < count; i += stride) p[i] = value;
+}
+
 struct SortedLayout {
-    size_t keys_in, keys_out, rows_in, rows_out, bounds, temp, temp_bytes, total;
+    size_t keys_in, keys_out, rows_in, rows_out, bounds, temp, temp_bytes, radix, flag, total;
 };
+
+// up to this many voxels with 32-bit keys the key sort can be left to the device (radix_sort.h with its run_if word)
+constexpr size_t kDeviceDecidesMax = 2097152;
 
 template <typename K>
 size_t pair_sort_temp_bytes(size_t n) {
@@ -313,7 +352,12 @@ SortedLayout sorted_layout(size_t n, int key_bits, int rows_xy) {
     off = align_up(off + (size_t)cdiv(nn, kGroup) * rows_xy * 2 * sizeof(uint32_t), 256);
     L.temp = off;
     L.temp_bytes = key_bits == 32 ? pair_sort_temp_bytes<uint32_t>(n) : pair_sort_temp_bytes<uint64_t>(n);
-    L.total = off + align_up(L.temp_bytes, 256);
+    off += align_up(L.temp_bytes, 256);
+    L.flag = off;
+    off += 256;
+    L.radix = off;
+    if (key_bits == 32 && n <= kDeviceDecidesMax) off += radix_layout(n).total;
+    L.total = off;
     return L;
 }
 
@@ -326,35 +370,59 @@ unsigned bit_length(uint64_t x) {
     return b;
 }
 
+// presorted: 0 = sort the keys, 1 = the caller knows that they ascend as the voxels come, 2 = find out on the device
 template <typename K>
-int build_sorted(const int32_t* coords, size_t n, uint64_t vol, const SubmGeom& g, bool presorted, char* ws, const SortedLayout& L,
+int build_sorted(const int32_t* coords, size_t n, uint64_t vol, const SubmGeom& g, int presorted, char* ws, const SortedLayout& L,
                  uint32_t* out_map, int32_t* gray, int32_t* binary, hipStream_t s) {
     K* keys_in = (K*)(ws + L.keys_in);
     K* keys_out = (K*)(ws + L.keys_out);
     uint32_t* rows_in = (uint32_t*)(ws + L.rows_in);
     uint32_t* rows_out = (uint32_t*)(ws + L.rows_out);
+    const K* skeys = keys_out;
+    const uint32_t* srows = rows_out;
+    const uint32_t* pick = nullptr;         // device word: 0 = the voxels came in key order and nothing was sorted
     PhaseEnd phases{s};
-    if (presorted) {        // keys ascend as the voxels come: the sorted arrays are the keys and 0, 1, 2, ... themselves
+    unsigned end_bit = bit_length(vol - 1);
+    if (end_bit == 0) end_bit = 1;
+    if (presorted == 1) {   // keys ascend as the voxels come: the sorted arrays are the keys and 0, 1, 2, ... themselves
         phase_mark("keys", s);
         flat_keys_kernel<K><<<cdiv(n, 256), 256, 0, s>>>(coords, n, g.W, g.H, g.D, keys_out, rows_out);
         FGX_CHECK_LAUNCH("fgx_subm_neighbor_map_sorted(keys)");
+    } else if (presorted == 2 && sizeof(K) == 4 && n <= kDeviceDecidesMax) {
+        // Voxels that already come in scan order (a dense grid's nonzero(), a sorted voxelizer) need no key sort.  Whether
+        // they do is found while the keys are made; the sort's kernels return at once when they do, and the kernels after
+        // it take the unsorted arrays then -- no answer has to travel to the host.
+        uint32_t* flag = (uint32_t*)(ws + L.flag);
+        phase_mark("keys", s);
+        fill_words_kernel<<<1, 64, 0, s>>>(flag, 1, 0u);
+        FGX_CHECK_LAUNCH("fgx_subm_neighbor_map_sorted(flag)");
+        flat_keys_check_kernel<K><<<cdiv(n, 256), 256, 0, s>>>(coords, n, g.W, g.H, g.D, keys_in, rows_in, flag);
+        FGX_CHECK_LAUNCH("fgx_subm_neighbor_map_sorted(keys)");
+        phase_mark("key sort", s);
+        const uint32_t *ks = nullptr, *vs = nullptr;
+        int rc = radix_sort_pairs_u32((const uint32_t*)keys_in, nullptr, n, end_bit, ws + L.radix, radix_layout(n), &ks, &vs, nullptr,
+                                      s, "fgx_subm_neighbor_map_sorted(key sort)", flag);
+        if (rc != FGX_OK) return rc;
+        skeys = (const K*)ks;
+        srows = vs;
+        pick = flag;
     } else {
         phase_mark("key sort", s);
         flat_keys_kernel<K><<<cdiv(n, 256), 256, 0, s>>>(coords, n, g.W, g.H, g.D, keys_in, rows_in);
         FGX_CHECK_LAUNCH("fgx_subm_neighbor_map_sorted(keys)");
         size_t temp_bytes = L.temp_bytes;
-        unsigned end_bit = bit_length(vol - 1);
-        if (end_bit == 0) end_bit = 1;
         FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp_bytes, (const K*)keys_in, keys_out, (const uint32_t*)rows_in, rows_out,
                                                 n, 0u, end_bit, s));
     }
     const unsigned groups = cdiv(n, kGroup);
     uint32_t* bounds = (uint32_t*)(ws + L.bounds);
     phase_mark("window bounds", s);
-    window_bounds_kernel<K><<<cdiv((size_t)groups * g.Kw * g.Kh * 2, 256), 256, 0, s>>>(keys_out, n, (unsigned long long)vol, g, groups, bounds);
+    window_bounds_kernel<K><<<cdiv((size_t)groups * g.Kw * g.Kh * 2, 256), 256, 0, s>>>(skeys, n, (unsigned long long)vol, g, groups, bounds,
+                                                                                        pick, (const K*)keys_in);
     FGX_CHECK_LAUNCH("fgx_subm_neighbor_map_sorted(bounds)");
     phase_mark("merge", s);
-    merge_neighbor_kernel<K><<<groups, kGroup, 0, s>>>(keys_out, rows_out, bounds, n, g, out_map, gray, binary);
+    merge_neighbor_kernel<K><<<groups, kGroup, 0, s>>>(skeys, srows, bounds, n, g, out_map, gray, binary, pick, (const K*)keys_in,
+                                                       (const uint32_t*)rows_in);
     FGX_CHECK_LAUNCH("fgx_subm_neighbor_map_sorted");
     return FGX_OK;
 }
@@ -532,11 +600,6 @@ __global__ void __launch_bounds__(kGroup) merge_query_kernel(const K* __restrict
     }
 }
 
-__global__ void __launch_bounds__(256) fill_words_kernel(uint32_t* p, size_t count, uint32_t value) {
-    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    const size_t stride = (size_t)gridDim.x * 256;
-    for (; i < count; i += stride) p[i] = value;
-}
 
 struct QueryLayout {
     SortedLayout in;            // the input voxels' sort (bounds sized for the query groups)
@@ -632,6 +695,7 @@ int fgx_subm_neighbor_map_sorted(const int32_t* coords, size_t n, int B, int W, 
                                  int Dh, int Dd, int key_bits, int presorted, void* workspace, size_t workspace_bytes,
                                  uint32_t* out_map, int32_t* gray, int32_t* binary, fgx_stream_t stream) {
     FGX_CHECK_ARG(key_bits == 32 || key_bits == 64, "fgx_subm_neighbor_map_sorted: key_bits must be 32 or 64, got %d", key_bits);
+    FGX_CHECK_ARG(presorted >= 0 && presorted <= 2, "fgx_subm_neighbor_map_sorted: presorted must be 0, 1 or 2, got %d", presorted);
     FGX_CHECK_ARG(Kw > 0 && Kh > 0 && Kd > 0 && (Kw & 1) && (Kh & 1) && (Kd & 1),
                   "fgx_subm_neighbor_map_sorted: kernel sizes must be odd and positive, got (%d,%d,%d)", Kw, Kh, Kd);
     FGX_CHECK_ARG(B > 0 && W > 0 && H > 0 && D > 0, "fgx_subm_neighbor_map_sorted: grid extents must be positive");
@@ -654,8 +718,8 @@ int fgx_subm_neighbor_map_sorted(const int32_t* coords, size_t n, int B, int W, 
     SubmGeom g{W, H, D, Kw, Kh, Kd, V, Dw, Dh, Dd};
     hipStream_t s = (hipStream_t)stream;
     char* ws = (char*)workspace;
-    return key_bits == 32 ? build_sorted<uint32_t>(coords, n, vol, g, presorted != 0, ws, L, out_map, gray, binary, s)
-                          : build_sorted<uint64_t>(coords, n, vol, g, presorted != 0, ws, L, out_map, gray, binary, s);
+    return key_bits == 32 ? build_sorted<uint32_t>(coords, n, vol, g, presorted, ws, L, out_map, gray, binary, s)
+                          : build_sorted<uint64_t>(coords, n, vol, g, presorted, ws, L, out_map, gray, binary, s);
 }
 
 size_t fgx_spconv_neighbor_map_sorted_workspace_bytes(size_t n_in, size_t n_out, int key_bits, int Kw, int Kh) {

@@ -51,9 +51,12 @@ inline RadixLayout radix_layout(size_t n) {
     return L;
 }
 
-// hist[digit * tiles + tile] = items of the tile with that digit
+// hist[digit * tiles + tile] = items of the tile with that digit.  run_if != nullptr: the whole sort is conditional on that
+// word, which an earlier kernel of the stream has written -- every wavefront returns at once when it is zero.
 __global__ void __launch_bounds__(64) radix_hist_kernel(const uint32_t* __restrict__ keys, size_t n, unsigned shift, unsigned bits,
-                                                        unsigned tiles, uint32_t* __restrict__ hist) {
+                                                        unsigned tiles, uint32_t* __restrict__ hist,
+                                                        const uint32_t* __restrict__ run_if) {
+    if (run_if != nullptr && *run_if == 0u) return;
     __shared__ uint32_t count[1 << kRsMaxBits];
     const unsigned bins = 1u << bits, mask = bins - 1u;
     for (unsigned b = threadIdx.x; b < bins; b += 64) count[b] = 0u;
@@ -80,7 +83,9 @@ __global__ void __launch_bounds__(64) radix_hist_kernel(const uint32_t* __restri
 __global__ void __launch_bounds__(64) radix_scatter_kernel(const uint32_t* __restrict__ keys, const uint32_t* __restrict__ vals_in,
                                                            size_t n, unsigned shift, unsigned bits, unsigned tiles,
                                                            const uint32_t* __restrict__ offs, uint32_t* __restrict__ keys_out,
-                                                           uint32_t* __restrict__ vals_out, int64_t* __restrict__ out64) {
+                                                           uint32_t* __restrict__ vals_out, int64_t* __restrict__ out64,
+                                                           const uint32_t* __restrict__ run_if) {
+    if (run_if != nullptr && *run_if == 0u) return;
     __shared__ uint32_t next[1 << kRsMaxBits];        // where the next item of each digit goes
     const unsigned bins = 1u << bits, mask = bins - 1u;
     for (unsigned b = threadIdx.x; b < bins; b += 64) next[b] = offs[(size_t)b * tiles + blockIdx.x];
@@ -129,9 +134,11 @@ __global__ void __launch_bounds__(64) radix_scatter_kernel(const uint32_t* __res
 
 // Sorts (keys[i], vals[i] or i) by the low `end_bit` bits of the keys, stable.  `ws`: radix_layout(n).total bytes, 256-byte
 // aligned.  The result ends in (*keys_sorted, *vals_sorted), which point into the workspace, or, with out64, in out64 alone.
+// run_if (a device word, or nullptr): when it reads zero the histogram and scatter kernels do nothing, the scans in between
+// run over whatever the tables hold, and the buffers the result would have ended in are left as they were.
 inline int radix_sort_pairs_u32(const uint32_t* keys, const uint32_t* vals, size_t n, unsigned end_bit, char* ws, const RadixLayout& L,
                                 const uint32_t** keys_sorted, const uint32_t** vals_sorted, int64_t* out64, hipStream_t s,
-                                const char* what) {
+                                const char* what, const uint32_t* run_if = nullptr) {
     if (end_bit < 1) end_bit = 1;
     if (end_bit > 32) end_bit = 32;
     const unsigned passes = (end_bit + kRsMaxBits - 1) / kRsMaxBits;
@@ -145,13 +152,13 @@ inline int radix_sort_pairs_u32(const uint32_t* keys, const uint32_t* vals, size
     for (unsigned p = 0; p < passes; ++p) {
         const unsigned shift = p * bits;
         const bool last = p + 1 == passes;
-        radix_hist_kernel<<<L.tiles, 64, 0, s>>>(kin, n, shift, bits, L.tiles, hist);
+        radix_hist_kernel<<<L.tiles, 64, 0, s>>>(kin, n, shift, bits, L.tiles, hist, run_if);
         FGX_CHECK_LAUNCH(what);
         size_t tb = L.temp_bytes;
         FGX_CHECK_HIP(rocprim::exclusive_scan(ws + L.temp, tb, (const uint32_t*)hist, offs, 0u, ((size_t)1 << bits) * L.tiles,
                                               rocprim::plus<uint32_t>(), s));
         radix_scatter_kernel<<<L.tiles, 64, 0, s>>>(kin, vin, n, shift, bits, L.tiles, offs, kbuf[p & 1], vbuf[p & 1],
-                                                    last ? out64 : nullptr);
+                                                    last ? out64 : nullptr, run_if);
         FGX_CHECK_LAUNCH(what);
         kin = kbuf[p & 1];
         vin = vbuf[p & 1];

@@ -379,16 +379,13 @@ def _build_neighbor_map(coords: torch.Tensor, shape, kernel_size, dilation, with
         key_bits = 32 if vol <= 2 ** 32 else 64
         with torch.cuda.device(dev):
             L = nat.lib()
-            # voxels that already come in scan order (a dense grid's nonzero(), a sorted voxelizer) need no key sort: one
-            # pass over the coordinates and a 4-byte read-back tell, and save the sort's ~0.13 ms
-            descents = torch.zeros((1,), dtype=torch.int32, device=dev)
-            nat.check(L.fgx_coords_key_order(nat.ptr(coords), nat.sz(n), C.c_int(W), C.c_int(H), C.c_int(D), nat.ptr(descents), nat.stream()))
-            presorted = int(descents.item()) == 0
+            # voxels that already come in scan order (a dense grid's nonzero(), a sorted voxelizer) need no key sort; the
+            # library finds out on the device (presorted = 2), so nothing is read back here
             ws = nat.workspace(L.fgx_subm_neighbor_map_sorted_workspace_bytes(nat.sz(n), C.c_int(key_bits), C.c_int(kw), C.c_int(kh)), dev)
             nat.check(L.fgx_subm_neighbor_map_sorted(
                 nat.ptr(coords), nat.sz(n), C.c_int(B), C.c_int(W), C.c_int(H), C.c_int(D), C.c_int(kw), C.c_int(kh), C.c_int(kd),
                 C.c_int(int(dilation[0])), C.c_int(int(dilation[1])), C.c_int(int(dilation[2])), C.c_int(key_bits),
-                C.c_int(1 if presorted else 0),
+                C.c_int(2),
                 nat.ptr(ws), nat.sz(ws.numel()), nat.ptr(nmap), nat.ptr(gray), nat.ptr(binary), nat.stream()))
         return nmap, gray, binary
     table = int(spconv.HASHMAP_RATIO * n)

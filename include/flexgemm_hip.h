@@ -108,10 +108,13 @@ int fgx_subm_neighbor_map(void* keys, int key_bits, uint32_t* vals, size_t table
  * the sorted array (two binary searches, one coalesced read into LDS, per-lane searches there).  Meant for large or
  * shuffled coordinate sets, where hash probes are cache-line fetches at random addresses.  key_bits: 32 when
  * B*W*H*D <= 2^32, else 64 (grids up to 2^63 cells).  workspace: fgx_subm_neighbor_map_sorted_workspace_bytes bytes,
- * 256-byte aligned.  gray / binary as above.  presorted != 0 promises that the flattened keys ((b*W + x)*H + y)*D + z
- * never descend from one voxel to the next (voxels listed in scan order): the radix sort is skipped.
- * fgx_coords_key_order tells: it sets descents[0] (device, cleared by the caller beforehand) to 1 when some key is
- * smaller than its predecessor's; the caller reads the word back before it decides.
+ * 256-byte aligned.  gray / binary as above.  presorted = 1 promises that the flattened keys ((b*W + x)*H + y)*D + z
+ * never descend from one voxel to the next (voxels listed in scan order): the radix sort is skipped.  presorted = 2
+ * leaves the question to the device: the kernel that makes the keys also notes whether one descends, the sort's kernels
+ * return at once when none does, and the search takes the unsorted arrays then -- nothing is read back (32-bit keys and up
+ * to 2^21 voxels; otherwise 2 means 0: the keys are sorted without asking).  presorted = 0 always sorts.
+ * fgx_coords_key_order answers the question for a caller that wants to know: it sets descents[0] (device, cleared by the
+ * caller beforehand) to 1 when some key is smaller than its predecessor's.
  * Replaces: the same reference function as fgx_subm_neighbor_map (the result is identical; only the search differs). */
 size_t fgx_subm_neighbor_map_sorted_workspace_bytes(size_t n, int key_bits, int Kw, int Kh);
 int fgx_coords_key_order(const int32_t* coords, size_t n, int W, int H, int D, uint32_t* descents, fgx_stream_t stream);

@@ -301,3 +301,53 @@ def test_private_tile_order(gpu_device, res, batch, shuffle):
     vk, seg = nb.tile_masks(_np(cache.gray_code), _np(cache.sorted_idx), 128)
     assert np.array_equal(_np(cache.valid_kernel_callback(128)), vk)
     assert np.array_equal(_np(cache.valid_kernel_seg_callback(128)), seg)
+
+
+def test_sorted_builder_decides_the_key_sort_on_the_device(gpu_device, neighbor_map_builder):
+    """fgx_subm_neighbor_map_sorted with presorted = 2 (what the cache builder passes) against presorted = 0 (always
+    sort) and, where it applies, presorted = 1: coordinates in scan order, shuffled, in scan order but for the last two
+    voxels, a single voxel, and more voxels than the device-side decision covers (it then sorts without asking)."""
+    if neighbor_map_builder != "sort":
+        pytest.skip("the sorted builder's own entry point")
+    L = nat.lib()
+    rng = np.random.default_rng(5)
+    cases = []
+    shell = reference_test_shell(96)
+    cases.append(("scan order", shell, 96, True))
+    cases.append(("shuffled", shell[rng.permutation(len(shell))], 96, False))
+    swapped = shell.copy()
+    swapped[[-1, -2]] = swapped[[-2, -1]]
+    cases.append(("last two swapped", swapped, 96, False))
+    cases.append(("one voxel", shell[:1].copy(), 96, True))
+    big = shell_coords(1024)
+    assert len(big) > (1 << 21)
+    cases.append(("2.6 M voxels in scan order", big, 1024, True))
+    for name, coords_np, res, ascending in cases:
+        _say(f"sorted builder, key sort decided on the device: {name} (n={len(coords_np)})")
+        coords = torch.from_numpy(np.ascontiguousarray(coords_np, dtype=np.int32)).to(gpu_device)
+        n = coords.shape[0]
+        maps = {}
+        for mode in (0, 2) + ((1,) if ascending else ()):
+            nmap = torch.full((n, 27), 0x7FFFFFFF, dtype=torch.int32, device=gpu_device)
+            gray = torch.empty((n,), dtype=torch.int32, device=gpu_device)
+            binary = torch.empty((n,), dtype=torch.int32, device=gpu_device)
+            with torch.cuda.device(gpu_device):
+                ws = nat.workspace(L.fgx_subm_neighbor_map_sorted_workspace_bytes(nat.sz(n), C.c_int(32), C.c_int(3), C.c_int(3)), gpu_device)
+                ws.fill_(0xA5)          # stale flag words and tables must not matter
+                nat.check(L.fgx_subm_neighbor_map_sorted(
+                    nat.ptr(coords), nat.sz(n), C.c_int(1), C.c_int(res), C.c_int(res), C.c_int(res), C.c_int(3), C.c_int(3), C.c_int(3),
+                    C.c_int(1), C.c_int(1), C.c_int(1), C.c_int(32), C.c_int(mode), nat.ptr(ws), nat.sz(ws.numel()),
+                    nat.ptr(nmap), nat.ptr(gray), nat.ptr(binary), nat.stream()))
+            torch.cuda.synchronize()
+            maps[mode] = (nmap.cpu(), gray.cpu(), binary.cpu())
+        for mode in maps:
+            for got, want in zip(maps[mode], maps[0]):
+                assert torch.equal(got, want), f"{name}: presorted={mode} differs from the always-sorting call"
+        if n <= 200000:
+            ref = nb.neighbor_cache(coords_np, (1, 8, res, res, res), (3, 3, 3), (1, 1, 1), needs_grad=False, blocks=())
+            assert np.array_equal(maps[2][0].numpy().view(np.uint32), ref["neighbor_map"])
+    with pytest.raises(ValueError):
+        nat.check(L.fgx_subm_neighbor_map_sorted(
+            nat.ptr(coords), nat.sz(n), C.c_int(1), C.c_int(res), C.c_int(res), C.c_int(res), C.c_int(3), C.c_int(3), C.c_int(3),
+            C.c_int(1), C.c_int(1), C.c_int(1), C.c_int(32), C.c_int(3), nat.ptr(ws), nat.sz(ws.numel()),
+            nat.ptr(nmap), nat.ptr(gray), nat.ptr(binary), nat.stream()))
