@@ -31,7 +31,8 @@ EXPORTS = [
     "fgx_pair_workspace_bytes", "fgx_pair_count", "fgx_pair_fill",
     "fgx_tile_workspace_bytes", "fgx_tile_codes", "fgx_tile_fill",
     "fgx_table_lookup", "fgx_weight_panel_bytes", "fgx_pack_weight",
-    "fgx_conv_scratch_bytes", "fgx_conv_gather_gemm", "fgx_conv_gather_gemm_act",
+    "fgx_conv_scratch_bytes", "fgx_conv_gather_gemm", "fgx_conv_gather_gemm_act", "fgx_conv_gather_gemm_act_mask",
+    "fgx_relu_mask_apply", "fgx_conv_gather_gemm_stream_act_mask",
     "fgx_gather_plan_count", "fgx_gather_plan_fill", "fgx_conv_gather_gemm_stream", "fgx_conv_gather_gemm_stream_act",
     "fgx_conv_gather_gemm_stream_groups", "fgx_gather_item_order_workspace_bytes", "fgx_gather_item_order",
     "fgx_wgrad_scratch_bytes", "fgx_wgrad_block_bounds_count", "fgx_wgrad_block_bounds", "fgx_conv_wgrad",

@@ -54,15 +54,18 @@ def main():
     p.add_argument("--panel-cache", action="store_true",
                    help="keep the repacked weight panels with the weights (flex_gemm.ops.spconv.set_weight_panel_cache): "
                         "the loop never updates its weights, so every pack after the second iteration is saved")
-    p.add_argument("--relu", choices=("none", "fused", "separate"), default="none",
-                   help="a ReLU after every layer: in the GEMM's epilogue (sparse_submanifold_conv3d_relu) or as torch.relu")
+    p.add_argument("--relu", choices=("none", "fused", "fused-no-bits", "separate"), default="none",
+                   help="a ReLU after every layer: in the GEMM's epilogue (sparse_submanifold_conv3d_relu; fused-no-bits: "
+                        "its backward tests the saved output instead of the epilogue's bit mask) or as torch.relu")
     args = p.parse_args()
 
     import flex_gemm
     from flex_gemm.ops.spconv import Algorithm, SubMConv3dFunction, sparse_submanifold_conv3d, sparse_submanifold_conv3d_relu
+    from flexgemm_amd.ops import spconv as spconv_config
+    spconv_config.RELU_BIT_MASK = args.relu != "fused-no-bits"
 
     def layer(h, coords, shape, w, b, cache):
-        if args.relu == "fused":
+        if args.relu in ("fused", "fused-no-bits"):
             return sparse_submanifold_conv3d_relu(h, coords, shape, w, b, cache)[0]
         h = sparse_submanifold_conv3d(h, coords, shape, w, b, cache)[0]
         return torch.relu(h) if args.relu == "separate" else h

@@ -154,7 +154,8 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
                    const typename Tag::type* __restrict__ bias, const uint32_t* __restrict__ map,
                    const int64_t* __restrict__ sorted_idx, const int32_t* __restrict__ tile_code, uint32_t n, int K,
                    int cols, int cols_pad, int V, int splitk, unsigned row_tiles, unsigned col_tiles,
-                   float* __restrict__ partial, int act, typename Tag::type* __restrict__ out) {
+                   float* __restrict__ partial, int act, typename Tag::type* __restrict__ out,
+                   uint8_t* __restrict__ relu_mask) {
     using C = GemmCfg<Tag, BM, BN, WAVES_M, WAVES_N, S, CH>;
     using T = typename Tag::type;
     constexpr int NT = C::NT;
@@ -427,7 +428,12 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
             const unsigned char* sp = band + r * C::OUT_PITCH + piece * 16;
             T* dp = out + (size_t)orow * cols + col;
             if (vec_ok && col + 16 / C::ES <= cols) {
-                *(u32x4*)dp = *(const u32x4*)sp;
+                const u32x4 piece16 = *(const u32x4*)sp;
+                *(u32x4*)dp = piece16;
+                // one bit per output for the activation's derivative (16-bit types, whole pieces only: the host passes a
+                // mask for such shapes alone)
+                if (C::ES == 2 && relu_mask != nullptr)
+                    relu_mask[((size_t)orow * cols + col) >> 3] = (uint8_t)positive_bits16<PositiveLimit<T>::value>(piece16);
             } else {
                 for (int t = 0; t < 16 / C::ES && col + t < cols; ++t) dp[t] = ((const T*)sp)[t];
             }
@@ -435,14 +441,36 @@ gather_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
     }
 }
 
-// out[i] = act(sum_s partial[s][i])   (slice 0 carries the bias)
+// out[i] = act(sum_s partial[s][i])   (slice 0 carries the bias).  relu_mask != nullptr (numel a multiple of 8): bit i says
+// whether out[i] > 0 -- a wavefront holds 64 consecutive i, one ballot gives their bits and every eighth lane writes a byte.
 template <typename T>
 __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restrict__ partial, int splitk, size_t numel,
-                                                            int act, T* __restrict__ out) {
+                                                            int act, T* __restrict__ out, uint8_t* __restrict__ relu_mask) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < numel; i += (size_t)gridDim.x * 256) {
         float s = 0.f;
         for (int k = 0; k < splitk; ++k) s += partial[(size_t)k * numel + i];
-        out[i] = from_float<T>(activate(s, act));
+        const T rounded = from_float<T>(activate(s, act));
+        out[i] = rounded;
+        if (relu_mask != nullptr) {
+            const unsigned long long positive = __ballot(to_float<T>(rounded) > 0.f);
+            const unsigned lane = threadIdx.x & 63u;
+            if ((lane & 7u) == 0u) relu_mask[i >> 3] = (uint8_t)(positive >> lane);
+        }
+    }
+}
+
+// out[8 i .. 8 i + 7] = grad[...] where bit t of mask[i] is set, else 0 (16-bit elements: one 16-byte piece per lane)
+__global__ void __launch_bounds__(256) relu_mask_apply_kernel(const u32x4* __restrict__ grad, const uint8_t* __restrict__ mask,
+                                                              size_t pieces, u32x4* __restrict__ out) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < pieces; i += (size_t)gridDim.x * 256) {
+        const uint32_t m = mask[i];
+        u32x4 v = __builtin_nontemporal_load(grad + i);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const uint32_t keep = ((m >> (2 * w)) & 1u ? 0x0000FFFFu : 0u) | ((m >> (2 * w + 1)) & 1u ? 0xFFFF0000u : 0u);
+            v[w] &= keep;
+        }
+        __builtin_nontemporal_store(v, out + i);
     }
 }
 
@@ -545,7 +573,7 @@ bool dtype_ok(int dtype) { return dtype == FGX_F16 || dtype == FGX_BF16 || dtype
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int S, int CH>
 int launch_gemm(const void* src, const void* panel, const void* bias, const uint32_t* map, const int64_t* sorted_idx,
                 const int32_t* tile_code, size_t n, int K, int cols, int cols_pad, int V, int splitk, void* scratch,
-                int act, void* out, hipStream_t s) {
+                int act, void* out, uint8_t* relu_mask, hipStream_t s) {
     using C = GemmCfg<Tag, BM, BN, WAVES_M, WAVES_N, S, CH>;
     using T = typename Tag::type;
     auto kern = gather_gemm_kernel<Tag, BM, BN, WAVES_M, WAVES_N, S, CH>;
@@ -561,13 +589,14 @@ int launch_gemm(const void* src, const void* panel, const void* bias, const uint
     const unsigned grid_x = cdiv(total, kXcds) * kXcds;
     dim3 grid(grid_x, splitk, 1);
     kern<<<grid, C::NT, lds, s>>>((const T*)src, (const T*)panel, (const T*)bias, map, sorted_idx, tile_code, (uint32_t)n, K,
-                                  cols, cols_pad, V, splitk, row_tiles, col_tiles, (float*)scratch, act, (T*)out);
+                                  cols, cols_pad, V, splitk, row_tiles, col_tiles, (float*)scratch, act, (T*)out,
+                                  splitk > 1 ? nullptr : relu_mask);
     FGX_CHECK_LAUNCH("fgx_conv_gather_gemm");
     if (splitk > 1) {
         size_t numel = n * (size_t)cols;
         unsigned g = cdiv(numel, 256);
         if (g > 65536u) g = 65536u;
-        splitk_reduce_kernel<T><<<g, 256, 0, s>>>((const float*)scratch, splitk, numel, act, (T*)out);
+        splitk_reduce_kernel<T><<<g, 256, 0, s>>>((const float*)scratch, splitk, numel, act, (T*)out, relu_mask);
         FGX_CHECK_LAUNCH("fgx_conv_gather_gemm(reduce)");
     }
     return FGX_OK;
@@ -576,11 +605,11 @@ int launch_gemm(const void* src, const void* panel, const void* bias, const uint
 template <typename Tag>
 int dispatch_tile(int tile_rows, int tile_cols, int slab_bytes, const void* src, const void* panel, const void* bias,
                   const uint32_t* map, const int64_t* sorted_idx, const int32_t* tile_code, size_t n, int K, int cols,
-                  int cols_pad, int V, int splitk, void* scratch, int act, void* out, hipStream_t s) {
+                  int cols_pad, int V, int splitk, void* scratch, int act, void* out, uint8_t* relu_mask, hipStream_t s) {
 #define FGX_TILE(BM, BN, WMv, WNv, Sv, CHv)                                                                        \
     if (tile_rows == BM && tile_cols == BN && slab_bytes == CHv * 16)                                              \
         return launch_gemm<Tag, BM, BN, WMv, WNv, Sv, CHv>(src, panel, bias, map, sorted_idx, tile_code, n, K, cols, \
-                                                           cols_pad, V, splitk, scratch, act, out, s);
+                                                           cols_pad, V, splitk, scratch, act, out, relu_mask, s);
     FGX_TILE(256, 128, 2, 2, 3, 4)
     FGX_TILE(256, 128, 4, 2, 3, 8)
     FGX_TILE(128, 128, 2, 2, 3, 4)
@@ -694,7 +723,17 @@ int fgx_conv_gather_gemm_act(int dtype, const void* src, const void* panel, cons
                              const int64_t* sorted_idx, const int32_t* tile_code, size_t n, int K, int cols, int V,
                              int tile_rows, int tile_cols, int slab_bytes, int splitk, void* scratch, int activation,
                              void* out, fgx_stream_t stream) {
+    return fgx_conv_gather_gemm_act_mask(dtype, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, V, tile_rows, tile_cols,
+                                         slab_bytes, splitk, scratch, activation, out, nullptr, stream);
+}
+
+int fgx_conv_gather_gemm_act_mask(int dtype, const void* src, const void* panel, const void* bias, const uint32_t* map,
+                                  const int64_t* sorted_idx, const int32_t* tile_code, size_t n, int K, int cols, int V,
+                                  int tile_rows, int tile_cols, int slab_bytes, int splitk, void* scratch, int activation,
+                                  void* out, uint8_t* relu_mask, fgx_stream_t stream) {
     FGX_CHECK_ARG(activation == FGX_ACT_NONE || activation == FGX_ACT_RELU, "fgx_conv_gather_gemm: unknown activation %d", activation);
+    FGX_CHECK_ARG(relu_mask == nullptr || (activation == FGX_ACT_RELU && dtype != FGX_F32 && cols % 8 == 0),
+                  "fgx_conv_gather_gemm: a ReLU mask needs the ReLU epilogue, a 16-bit type and a multiple of 8 columns (got %d)", cols);
     const int act = activation;
     FGX_CHECK_ARG(dtype_ok(dtype), "fgx_conv_gather_gemm: unknown dtype %d", dtype);
     FGX_CHECK_ARG(K > 0 && cols > 0 && V >= 1 && V <= 32, "fgx_conv_gather_gemm: bad shape K=%d cols=%d V=%d", K, cols, V);
@@ -710,10 +749,24 @@ int fgx_conv_gather_gemm_act(int dtype, const void* src, const void* panel, cons
     const int cols_pad = (int)align_up((size_t)cols, (size_t)tile_cols);
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
-        case FGX_F16: return dispatch_tile<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, act, out, s);
-        case FGX_BF16: return dispatch_tile<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, act, out, s);
-        default: return dispatch_tile<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, act, out, s);
+        case FGX_F16: return dispatch_tile<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, act, out, relu_mask, s);
+        case FGX_BF16: return dispatch_tile<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, act, out, relu_mask, s);
+        default: return dispatch_tile<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, map, sorted_idx, tile_code, n, K, cols, cols_pad, V, splitk, scratch, act, out, nullptr, s);
     }
+}
+
+int fgx_relu_mask_apply(int dtype, const void* grad, const uint8_t* relu_mask, size_t numel, void* out, fgx_stream_t stream) {
+    FGX_CHECK_ARG(dtype == FGX_F16 || dtype == FGX_BF16, "fgx_relu_mask_apply: 16-bit types only (dtype %d)", dtype);
+    FGX_CHECK_ARG(numel % 8 == 0, "fgx_relu_mask_apply: %zu elements are not a multiple of 8", numel);
+    if (numel == 0) return FGX_OK;
+    FGX_CHECK_ARG(grad && relu_mask && out, "fgx_relu_mask_apply: null buffer");
+    FGX_CHECK_ARG((((uintptr_t)grad | (uintptr_t)out) & 15) == 0, "fgx_relu_mask_apply: grad and out must be 16-byte aligned");
+    const size_t pieces = numel / 8;
+    unsigned grid = cdiv(pieces, 256);
+    if (grid > 16384u) grid = 16384u;
+    relu_mask_apply_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const u32x4*)grad, relu_mask, pieces, (u32x4*)out);
+    FGX_CHECK_LAUNCH("fgx_relu_mask_apply");
+    return FGX_OK;
 }
 
 size_t fgx_colsum_scratch_bytes(size_t n, int cols) {

@@ -115,7 +115,7 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
                           int cols, int cols_pad,
                           unsigned row_tiles, unsigned col_tiles, uint32_t src_bytes, uint32_t panel_bytes,
                           uint32_t plan_bytes, const uint32_t* __restrict__ item_at, int act,
-                          typename Tag::type* __restrict__ out) {
+                          typename Tag::type* __restrict__ out, uint8_t* __restrict__ relu_mask) {
     using C = StreamCfg<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
     using T = typename Tag::type;
     constexpr int S = C::S, kSlabBytes = C::SLAB, kChunks = CH;
@@ -479,7 +479,12 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
                 T* dp = out + (size_t)orow * cols + col;
                 if (vec_ok && col + 16 / C::ES <= cols) {
                     // (streaming store: the output is not read again by this launch and should not push source rows out of L2)
-                    __builtin_nontemporal_store(*(const u32x4*)sp, (u32x4*)dp);
+                    const u32x4 piece16 = *(const u32x4*)sp;
+                    __builtin_nontemporal_store(piece16, (u32x4*)dp);
+                    // one bit per output for the activation's derivative (16-bit types, whole pieces only: the host
+                    // passes a mask for such shapes alone)
+                    if (C::ES == 2 && relu_mask != nullptr)
+                        relu_mask[((size_t)orow * cols + col) >> 3] = (uint8_t)positive_bits16<PositiveLimit<T>::value>(piece16);
                 } else {
                     for (int t = 0; t < 16 / C::ES && col + t < cols; ++t) dp[t] = ((const T*)sp)[t];
                 }
@@ -518,7 +523,7 @@ template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N, int CH>
 int launch_stream(const void* src, const void* panel, const void* bias, const int64_t* order, const int32_t* plan_seg,
                   const int32_t* tile_code, const uint32_t* plan_idx, const uint32_t* plan_band, size_t plan_rows, size_t n,
                   size_t n_src, int K, int cols, int cols_pad, size_t panel_bytes, const uint32_t* item_at, int max_groups,
-                  int act, void* out, hipStream_t s) {
+                  int act, void* out, uint8_t* relu_mask, hipStream_t s) {
     using C = StreamCfg<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
     using T = typename Tag::type;
     auto kern = gather_gemm_stream_kernel<Tag, BM, BN, WAVES_M, WAVES_N, CH>;
@@ -542,7 +547,7 @@ int launch_stream(const void* src, const void* panel, const void* bias, const in
     kern<<<groups, C::NT, lds, s>>>((const T*)src, (const T*)panel, (const T*)bias, order, plan_seg, tile_code, plan_idx,
                                     plan_band, (uint32_t)n, K, cols, cols_pad, row_tiles, col_tiles,
                                     (uint32_t)(n_src * (size_t)K * sizeof(T)), (uint32_t)panel_bytes,
-                                    (uint32_t)(plan_rows * BM * 4), item_at, act, (T*)out);
+                                    (uint32_t)(plan_rows * BM * 4), item_at, act, (T*)out, relu_mask);
     FGX_CHECK_LAUNCH("fgx_conv_gather_gemm_stream");
     return FGX_OK;
 }
@@ -551,11 +556,12 @@ template <typename Tag>
 int dispatch_stream(int tile_rows, int tile_cols, int slab_bytes, const void* src, const void* panel, const void* bias,
                     const int64_t* order, const int32_t* plan_seg, const int32_t* tile_code, const uint32_t* plan_idx,
                     const uint32_t* plan_band, size_t plan_rows, size_t n, size_t n_src, int K, int cols, int cols_pad,
-                    size_t panel_bytes, const uint32_t* item_at, int max_groups, int act, void* out, hipStream_t s) {
+                    size_t panel_bytes, const uint32_t* item_at, int max_groups, int act, void* out, uint8_t* relu_mask,
+                    hipStream_t s) {
 #define FGX_STREAM_TILE(BM, BN, WMv, WNv, CHv)                                                                          \
     if (tile_rows == BM && tile_cols == BN && slab_bytes == CHv * 16)                                                   \
         return launch_stream<Tag, BM, BN, WMv, WNv, CHv>(src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band,  \
-                                                         plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, act, out, s);
+                                                         plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, act, out, relu_mask, s);
     FGX_STREAM_TILE(256, 128, FGX_BIG_WAVES_M, 2, 8)
     FGX_STREAM_TILE(256, 64, 4, 2, 8)
     FGX_STREAM_TILE(256, 128, 4, 2, 4)      // 64-byte K-slabs: rows shorter than 128 bytes
@@ -588,7 +594,21 @@ extern "C" int fgx_conv_gather_gemm_stream_act(int dtype, const void* src, const
                                                size_t n, size_t n_src, int K, int cols, int V,
                                                int tile_rows, int tile_cols, int slab_bytes, const uint32_t* item_at,
                                                int max_groups, int activation, void* out, fgx_stream_t stream) {
+    return fgx_conv_gather_gemm_stream_act_mask(dtype, src, panel, bias, order, tile_code, plan_seg, plan_idx, plan_band, plan_rows,
+                                                n, n_src, K, cols, V, tile_rows, tile_cols, slab_bytes, item_at, max_groups,
+                                                activation, out, nullptr, stream);
+}
+
+extern "C" int fgx_conv_gather_gemm_stream_act_mask(int dtype, const void* src, const void* panel, const void* bias,
+                                                    const int64_t* order, const int32_t* tile_code, const int32_t* plan_seg,
+                                                    const uint32_t* plan_idx, const uint32_t* plan_band, size_t plan_rows,
+                                                    size_t n, size_t n_src, int K, int cols, int V,
+                                                    int tile_rows, int tile_cols, int slab_bytes, const uint32_t* item_at,
+                                                    int max_groups, int activation, void* out, uint8_t* relu_mask,
+                                                    fgx_stream_t stream) {
     FGX_CHECK_ARG(activation == FGX_ACT_NONE || activation == FGX_ACT_RELU, "fgx_conv_gather_gemm_stream: unknown activation %d", activation);
+    FGX_CHECK_ARG(relu_mask == nullptr || (activation == FGX_ACT_RELU && dtype != FGX_F32 && cols % 8 == 0),
+                  "fgx_conv_gather_gemm_stream: a ReLU mask needs the ReLU epilogue, a 16-bit type and a multiple of 8 columns (got %d)", cols);
     const int act = activation;
     FGX_CHECK_ARG(dtype == FGX_F16 || dtype == FGX_BF16 || dtype == FGX_F32, "fgx_conv_gather_gemm_stream: unknown dtype %d", dtype);
     FGX_CHECK_ARG(K > 0 && cols > 0 && V >= 1 && V <= 32, "fgx_conv_gather_gemm_stream: bad shape K=%d cols=%d V=%d", K, cols, V);
@@ -611,9 +631,9 @@ extern "C" int fgx_conv_gather_gemm_stream_act(int dtype, const void* src, const
     }
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
-        case FGX_F16: return dispatch_stream<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, act, out, s);
-        case FGX_BF16: return dispatch_stream<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, act, out, s);
-        default: return dispatch_stream<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, act, out, s);
+        case FGX_F16: return dispatch_stream<F16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, act, out, relu_mask, s);
+        case FGX_BF16: return dispatch_stream<BF16>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, act, out, relu_mask, s);
+        default: return dispatch_stream<F32>(tile_rows, tile_cols, slab_bytes, src, panel, bias, order, plan_seg, tile_code, plan_idx, plan_band, plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, act, out, nullptr, s);
     }
 }
 

@@ -48,6 +48,23 @@ template <> __device__ __forceinline__ void mma<F32>(f32x16& acc, const u32x4& a
 // activation of the GEMM epilogues (FGX_ACT_* of the public header), applied to the fp32 sum before it is rounded
 __device__ __forceinline__ float activate(float x, int act) { return act == FGX_ACT_RELU ? fmaxf(x, 0.f) : x; }
 
+// ReLU mask of a 16-byte piece of eight 16-bit outputs: bit t is set when element t is greater than zero (not zero, not
+// negative, not NaN) -- as unsigned numbers those are the patterns 1 ... the encoding of +infinity (LIMIT).
+template <uint32_t LIMIT>
+__device__ __forceinline__ uint32_t positive_bits16(const u32x4& v) {
+    uint32_t bits = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const uint32_t x = v[w];
+        bits |= (uint32_t)(((x & 0xFFFFu) - 1u) < LIMIT) << (2 * w);
+        bits |= (uint32_t)(((x >> 16) - 1u) < LIMIT) << (2 * w + 1);
+    }
+    return bits;
+}
+template <typename T> struct PositiveLimit { static constexpr uint32_t value = 0u; };        // fp32: no mask
+template <> struct PositiveLimit<_Float16> { static constexpr uint32_t value = 0x7C00u; };
+template <> struct PositiveLimit<__bf16> { static constexpr uint32_t value = 0x7F80u; };
+
 template <typename T> __device__ __forceinline__ T from_float(float x);
 template <> __device__ __forceinline__ _Float16 from_float<_Float16>(float x) { return (_Float16)x; }
 template <> __device__ __forceinline__ float from_float<float>(float x) { return x; }

@@ -54,6 +54,10 @@ GEMM_ITEM_ORDER = "auto"
 # The bias gradient of a submanifold layer comes out of the streaming wgrad kernel (which loads every grad_output row for
 # the centre offset anyway) instead of a column-sum pass of its own.  False: always the separate pass.
 FUSE_DBIAS = True
+# The fused-ReLU forward (sparse_submanifold_conv3d_relu) leaves the activation's derivative as one bit per output and
+# backward masks the gradient with it (fgx_relu_mask_apply).  False: backward tests the saved output instead
+# (torch.where), which reads the output again.
+RELU_BIT_MASK = True
 
 
 # Keep the repacked weight panels of the gather GEMMs with the weight tensor and reuse them while the weight is unchanged

@@ -473,13 +473,15 @@ def _weight_panel(owner: Optional[torch.Tensor], weight_cvk: torch.Tensor, code:
 
 def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[torch.Tensor], cache, mode: int,
                  allow_splitk: bool, masked: bool = True, weight_owner: Optional[torch.Tensor] = None,
-                 activation: int = nat.ACT_NONE) -> torch.Tensor:
+                 activation: int = nat.ACT_NONE, relu_mask_out: Optional[list] = None) -> torch.Tensor:
     """mode 0: out = conv(src) with weight [Co, V, Ci] (+bias); mode 1: grad_input from src = grad_output through the
     same map with the offsets mirrored (submanifold); mode 2: grad_input through a map of its own, offsets as they
     are (generic sparse convolution).  The result has one row per row of cache["neighbor_map"]; src may have a
     different number of rows.  masked=False: the non-masked schedule (natural row order, all offsets per tile).
     weight_owner: the tensor the caller's weight lives in, for the optional panel cache (see _weight_panel).
-    activation: nat.ACT_RELU clamps (sum + bias) at zero in the kernel's epilogue."""
+    activation: nat.ACT_RELU clamps (sum + bias) at zero in the kernel's epilogue.  relu_mask_out: a list; where the kernels
+    can (ReLU, 16-bit type, a multiple of 8 output columns) they also write one bit per output, "greater than zero", and
+    the uint8 tensor [n * cols / 8] holding them is appended to the list."""
     co, v, ci = weight_cvk.shape
     n = cache["neighbor_map"].shape[0]
     n_src = src.shape[0]
@@ -518,6 +520,10 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
     L = nat.lib()
     code = nat.DTYPE_CODE[dt]
     name = "gather_gemm_fwd" if mode == 0 else "gather_gemm_dgrad"
+    mask = None
+    if relu_mask_out is not None and activation == nat.ACT_RELU and src.element_size() == 2 and cols % 8 == 0:
+        mask = torch.empty((n * cols // 8,), dtype=torch.uint8, device=dev)
+        relu_mask_out.append(mask)
     with torch.cuda.device(dev):
         panel = _weight_panel(weight_owner, weight_cvk, code, mode, sched, dev)
         if sched.stream and _stream_fits(n, n_src, k * src.element_size()):
@@ -527,12 +533,12 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
             item_at = cache._item_order(plan_key, tile_code, -(-cols // sched.tile_cols), groups,
                                         -(-(k * src.element_size()) // sched.slab_bytes))
             nat.mark(name, "start")
-            nat.check(L.fgx_conv_gather_gemm_stream_act(
+            nat.check(L.fgx_conv_gather_gemm_stream_act_mask(
                 C.c_int(code), nat.ptr(src), nat.ptr(panel), nat.ptr(bias), nat.ptr(order), nat.ptr(tile_code),
                 nat.ptr(plan_seg), nat.ptr(plan_idx), nat.ptr(plan_band), nat.sz(plan_idx.shape[0]), nat.sz(n), nat.sz(n_src),
                 C.c_int(k), C.c_int(cols), C.c_int(v),
                 C.c_int(sched.tile_rows), C.c_int(sched.tile_cols), C.c_int(sched.slab_bytes), nat.ptr(item_at),
-                C.c_int(groups), C.c_int(activation), nat.ptr(out), nat.stream()))
+                C.c_int(groups), C.c_int(activation), nat.ptr(out), nat.ptr(mask), nat.stream()))
             nat.mark(name, "stop")
             return out
         if masked:
@@ -543,12 +549,23 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
         if splitk > 1:
             scratch = nat.workspace(L.fgx_conv_scratch_bytes(nat.sz(n), C.c_int(cols), C.c_int(splitk)), dev)
         nat.mark(name, "start")
-        nat.check(L.fgx_conv_gather_gemm_act(
+        nat.check(L.fgx_conv_gather_gemm_act_mask(
             C.c_int(code), nat.ptr(src), nat.ptr(panel), nat.ptr(bias), nat.ptr(cache["neighbor_map"]),
             nat.ptr(order), nat.ptr(tile_code), nat.sz(n), C.c_int(k), C.c_int(cols), C.c_int(v),
             C.c_int(sched.tile_rows), C.c_int(sched.tile_cols), C.c_int(sched.slab_bytes), C.c_int(splitk),
-            nat.ptr(scratch), C.c_int(activation), nat.ptr(out), nat.stream()))
+            nat.ptr(scratch), C.c_int(activation), nat.ptr(out), nat.ptr(mask), nat.stream()))
         nat.mark(name, "stop")
+    return out
+
+
+def _relu_mask_apply(grad_output: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
+    """grad_output where the forward pass's bit mask says the activated output was positive, zero elsewhere
+    (fgx_relu_mask_apply: one pass that reads an eighth of a byte per element beside the gradient)."""
+    g = grad_output.contiguous()
+    out = torch.empty_like(g)
+    with torch.cuda.device(g.device):
+        nat.check(nat.lib().fgx_relu_mask_apply(C.c_int(nat.DTYPE_CODE[g.dtype]), nat.ptr(g), nat.ptr(mask), nat.sz(g.numel()),
+                                                nat.ptr(out), nat.stream()))
     return out
 
 
@@ -730,8 +747,10 @@ class SubMConv3dFunction(Function):
         weight: torch.Tensor,
         bias: Optional[torch.Tensor] = None,
         relu: bool = False,
+        relu_mask_out: Optional[list] = None,
     ) -> torch.Tensor:
-        """relu (not in the reference): clamp the result at zero, in the GEMM's epilogue for the implicit algorithms."""
+        """relu (not in the reference): clamp the result at zero, in the GEMM's epilogue for the implicit algorithms.
+        relu_mask_out: a list that receives the bit mask "output > 0" when the kernels wrote one (see _gather_gemm)."""
         assert feats.is_contiguous(), "Input features should be contiguous"
         assert feats.shape[0] == neighbor_cache["neighbor_map"].shape[0], \
             f"{feats.shape[0]} feature rows for a neighbor cache of {neighbor_cache['neighbor_map'].shape[0]} voxels"
@@ -747,7 +766,7 @@ class SubMConv3dFunction(Function):
             _require_cuda(feats, "sparse_submanifold_conv3d")
             return _gather_gemm(feats, weight.reshape(co, v, ci), bias, neighbor_cache, 0, algo not in _NO_SPLITK,
                                 masked=algo in _MASKED, weight_owner=weight,
-                                activation=nat.ACT_RELU if relu else nat.ACT_NONE)
+                                activation=nat.ACT_RELU if relu else nat.ACT_NONE, relu_mask_out=relu_mask_out)
         raise ValueError(f"Unsupported algorithm {algo}")
 
     @staticmethod
@@ -815,19 +834,27 @@ class SubMConv3dFunction(Function):
         need_grad = any(ctx.needs_input_grad)
         if neighbor_cache is None:
             neighbor_cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (kw, kh, kd), dilation, need_grad)
-        output = SubMConv3dFunction._sparse_submanifold_conv_forward(feats, neighbor_cache, weight, bias, relu=relu)
-        if relu:
-            ctx.save_for_backward(feats, weight, bias, output)      # the output's sign is the activation's derivative
+        masks = [] if (relu and need_grad and spconv.RELU_BIT_MASK) else None
+        output = SubMConv3dFunction._sparse_submanifold_conv_forward(feats, neighbor_cache, weight, bias, relu=relu,
+                                                                     relu_mask_out=masks)
+        if relu and masks:
+            ctx.save_for_backward(feats, weight, bias, masks[0])    # one bit per output: the activation's derivative
+        elif relu:
+            ctx.save_for_backward(feats, weight, bias, output)      # ... or the output itself, whose sign tells
         else:
             ctx.save_for_backward(feats, weight, bias)
         ctx.relu = relu
+        ctx.relu_bits = bool(relu and masks)
         ctx.neighbor_cache = neighbor_cache
         ctx.weight_owner = weakref.ref(weight)      # the caller's tensor object: kept weight panels hang on it
         return output, neighbor_cache
 
     @staticmethod
     def backward(ctx, grad_output: torch.Tensor, _):
-        if ctx.relu:
+        if ctx.relu and ctx.relu_bits:
+            feats, weight, bias, mask = ctx.saved_tensors
+            grad_output = _relu_mask_apply(grad_output, mask)
+        elif ctx.relu:
             feats, weight, bias, output = ctx.saved_tensors
             grad_output = torch.where(output > 0, grad_output, torch.zeros((), dtype=grad_output.dtype, device=grad_output.device))
         else:

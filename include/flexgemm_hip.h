@@ -226,6 +226,19 @@ int fgx_conv_gather_gemm_act(int dtype, const void* src, const void* panel, cons
                              size_t n, int K, int cols, int V, int tile_rows, int tile_cols, int slab_bytes, int splitk,
                              void* scratch, int activation, void* out, fgx_stream_t stream);
 
+/* ... which also leaves the activation's derivative as one bit per output: bit (c mod 8) of relu_mask[(r * cols + c) / 8]
+ * is set when out[r][c] > 0.  For the backward pass of a fused ReLU, which then reads n * cols / 8 bytes instead of the
+ * output again (fgx_relu_mask_apply).  relu_mask may be NULL (no mask); otherwise activation must be FGX_ACT_RELU, the type
+ * 16-bit and cols a multiple of 8.  No counterpart in the reference. */
+int fgx_conv_gather_gemm_act_mask(int dtype, const void* src, const void* panel, const void* bias,
+                                  const uint32_t* map, const int64_t* sorted_idx, const int32_t* tile_code,
+                                  size_t n, int K, int cols, int V, int tile_rows, int tile_cols, int slab_bytes, int splitk,
+                                  void* scratch, int activation, void* out, uint8_t* relu_mask, fgx_stream_t stream);
+/* out[i] = bit i of relu_mask ? grad[i] : 0 for i < numel (a multiple of 8; 16-bit types; grad and out 16-byte aligned,
+ * out may be grad): the gradient of a fused ReLU from the mask its forward pass wrote.  One pass, numel / 8 bytes of mask
+ * read beside the gradient.  No counterpart in the reference. */
+int fgx_relu_mask_apply(int dtype, const void* grad, const uint8_t* relu_mask, size_t numel, void* out, fgx_stream_t stream);
+
 /* Gather plan of a row order for tiles of `tile_rows` rows: for tile t and the k-th offset v present in it
  * (the set bits of tile_code[t], ascending; a tile whose code is 0 gets one row with every neighbor missing),
  *   plan_idx[(plan_seg[t] + k) * tile_rows + r] = map[order[t * tile_rows + r], v]     (0xFFFFFFFF for rows past n),
@@ -271,6 +284,13 @@ int fgx_conv_gather_gemm_stream_act(int dtype, const void* src, const void* pane
                                     size_t n_src, int K, int cols, int V,
                                     int tile_rows, int tile_cols, int slab_bytes, const uint32_t* item_at,
                                     int max_groups, int activation, void* out, fgx_stream_t stream);
+/* ... and with the ReLU mask of fgx_conv_gather_gemm_act_mask. */
+int fgx_conv_gather_gemm_stream_act_mask(int dtype, const void* src, const void* panel, const void* bias,
+                                         const int64_t* order, const int32_t* tile_code, const int32_t* plan_seg,
+                                         const uint32_t* plan_idx, const uint32_t* plan_band, size_t plan_rows, size_t n,
+                                         size_t n_src, int K, int cols, int V,
+                                         int tile_rows, int tile_cols, int slab_bytes, const uint32_t* item_at,
+                                         int max_groups, int activation, void* out, uint8_t* relu_mask, fgx_stream_t stream);
 int fgx_conv_gather_gemm_stream_groups(int dtype, int cols, int tile_rows, int tile_cols, int slab_bytes, int* groups);
 
 /* item_at for fgx_conv_gather_gemm_stream, made on the device from the tile codes: items sorted by cost (offsets per

@@ -831,6 +831,51 @@ def test_relu_in_the_epilogue_equals_relu_after_the_operator(gpu_device, dtype, 
     assert torch.equal(a, b_)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("res,ci,co", [(48, 128, 128), (24, 64, 96), (8, 256, 64), (40, 32, 32)])
+def test_relu_bit_mask_of_the_epilogue_and_its_use_in_backward(gpu_device, dtype, res, ci, co):
+    """The fused-ReLU forward also writes one bit per output, "greater than zero" (streaming kernel, tiled kernel, split-K
+    reduction); backward masks the gradient with those bits in one pass.  The bits must equal (output > 0) exactly, and
+    fgx_relu_mask_apply must equal torch.where on gradients that hold NaN, infinities and negative zero."""
+    import ctypes as C
+    from flexgemm_amd import _native as nat
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    _say(f"relu bit mask res={res} ci={ci} co={co} {dtype}")
+    coords_np = reference_test_shell(res)
+    shape = torch.Size([1, ci, res, res, res])
+    feats, weight, bias, grad = _case(coords_np, ci, co, dtype, seed=res + co)
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+    masks = []
+    out = SubMConv3dFunction._sparse_submanifold_conv_forward(feats.to(gpu_device), cache, weight.to(gpu_device),
+                                                              bias.to(gpu_device), relu=True, relu_mask_out=masks)
+    torch.cuda.synchronize()
+    assert len(masks) == 1 and masks[0].dtype == torch.uint8 and masks[0].numel() == out.numel() // 8
+    want = np.packbits((out.float().cpu().numpy() > 0).reshape(-1), bitorder="little")
+    assert np.array_equal(masks[0].cpu().numpy(), want), "mask bits differ from (output > 0)"
+    assert 0 < int(want.sum()) and (want != 0xFF).any()
+    g = grad.to(gpu_device).clone()
+    flat = g.view(-1)
+    flat[0], flat[1], flat[2], flat[3] = float("nan"), float("inf"), float("-inf"), -0.0
+    flat[-1] = float("nan")
+    got = impl._relu_mask_apply(g, masks[0])
+    torch.cuda.synchronize()
+    ref = torch.where(out > 0, g, torch.zeros((), dtype=dtype, device=gpu_device))
+    assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), "masked gradient differs from torch.where"
+    # in place, as the header allows
+    nat.check(nat.lib().fgx_relu_mask_apply(C.c_int(nat.DTYPE_CODE[dtype]), nat.ptr(g), nat.ptr(masks[0]), nat.sz(g.numel()),
+                                            nat.ptr(g), nat.stream()))
+    torch.cuda.synchronize()
+    assert torch.equal(g.view(torch.int16), ref.view(torch.int16))
+    # what the kernels refuse
+    with pytest.raises(ValueError):
+        nat.check(nat.lib().fgx_relu_mask_apply(C.c_int(nat.FGX_F32), nat.ptr(g), nat.ptr(masks[0]), nat.sz(g.numel()),
+                                                nat.ptr(g), nat.stream()))
+    with pytest.raises(ValueError):
+        nat.check(nat.lib().fgx_relu_mask_apply(C.c_int(nat.DTYPE_CODE[dtype]), nat.ptr(g), nat.ptr(masks[0]), nat.sz(12),
+                                                nat.ptr(g), nat.stream()))
+
+
 def test_training_step_replays_from_a_hip_graph(gpu_device):
     """Forward and backward of two stacked layers captured once (whole-step capture: static input, gradients allocated
     by the captured backward) and replayed with new inputs; every replay equals the eager step bit for bit, with eager
