@@ -344,7 +344,7 @@ def main():
                                    + ("fwd+dgrad+wgrad+dbias, neighbor cache prebuilt and reused" if passes == 3 else "forward"),
                        "n_voxels": n, "valid_pairs": pairs, "useful_gflop_per_step": flop_pass * passes / 1e9},
             "frac_of_mfma_peak": value / PEAK_TFLOPS[dname],
-            "pass_ms": {"gather_gemm_avg": gemm_ms, "wgrad_incl_reduce": wgrad_ms,
+            "pass_ms": {"gather_gemm_avg": gemm_ms, "wgrad_incl_reduce": wgrad_ms if wgrad_ms == wgrad_ms else None,
                         "forward": stats(["gather_gemm_fwd"]), "dgrad": stats(["gather_gemm_dgrad"]), "wgrad": stats(["wgrad"])},
             "step_ms": {"wall_mean": ms_per_step, "median": step_ms[len(step_ms) // 2], "min": step_ms[0]},
             "peak_memory_bytes": peak_bytes,
@@ -387,7 +387,7 @@ def main():
         result["cpu_baseline"] = cpu_baseline(wl, nmap_cpu, passes, args.cpu_rows)
     else:
         result["cpu_baseline"] = None
-    print(json.dumps(result))
+    print(json.dumps(result, allow_nan=False))
 
 
 if __name__ == "__main__":

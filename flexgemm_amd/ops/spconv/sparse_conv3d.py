@@ -20,7 +20,7 @@ from .. import spconv, utils
 from .. import serialize
 from . import Algorithm, SerializationMode, SparseConv3dOutCoordAlgorithm
 from .submanifold_conv3d import (EMPTY, _IMPLICIT, _MASKED, _NO_SPLITK, SubMConv3dNeighborCache, _codes_and_order, _colsum,
-                                 _gather_gemm, _gathered_rows, _pair_lists, _require_cuda, _wgrad)
+                                 _gather_gemm, _gathered_rows, _pair_lists, _relu_mask_apply, _require_cuda, _wgrad)
 
 
 def _triple(x) -> Tuple[int, int, int]:
@@ -312,8 +312,10 @@ class SparseConv3dFunction(Function):
         weight: torch.Tensor,
         bias: Optional[torch.Tensor] = None,
         relu: bool = False,
+        relu_mask_out: Optional[list] = None,
     ) -> torch.Tensor:
-        """relu (not in the reference): clamp the result at zero, in the GEMM's epilogue for the implicit algorithms."""
+        """relu (not in the reference): clamp the result at zero, in the GEMM's epilogue for the implicit algorithms.
+        relu_mask_out: a list that receives the bit mask "output > 0" when the kernels wrote one (see _gather_gemm)."""
         assert feats.is_contiguous(), "Input features should be contiguous"
         n_in = neighbor_cache["_n_in"]          # input voxels the maps were built for (absent on a hand-made cache)
         if n_in is None and neighbor_cache["neighbor_map_bwd"] is not None:
@@ -331,7 +333,7 @@ class SparseConv3dFunction(Function):
             _require_cuda(feats, "sparse_conv3d")
             return _gather_gemm(feats, weight.reshape(co, v, ci), bias, neighbor_cache, 0, algo not in _NO_SPLITK,
                                 masked=algo in _MASKED, weight_owner=weight,
-                                activation=nat.ACT_RELU if relu else nat.ACT_NONE)
+                                activation=nat.ACT_RELU if relu else nat.ACT_NONE, relu_mask_out=relu_mask_out)
         raise ValueError(f"Unsupported algorithm {algo}")
 
     @staticmethod
@@ -404,12 +406,16 @@ class SparseConv3dFunction(Function):
         if neighbor_cache is None:
             neighbor_cache = SparseConv3dFunction._compute_neighbor_cache(coords, out_coords, shape, (kw, kh, kd), stride,
                                                                           padding, dilation, need_grad, given)
-        output = SparseConv3dFunction._sparse_conv_forward(feats, neighbor_cache, weight, bias, relu=relu)
-        if relu:
-            ctx.save_for_backward(feats, weight, bias, output)      # the output's sign is the activation's derivative
+        masks = [] if (relu and need_grad and spconv.RELU_BIT_MASK) else None
+        output = SparseConv3dFunction._sparse_conv_forward(feats, neighbor_cache, weight, bias, relu=relu, relu_mask_out=masks)
+        if relu and masks:
+            ctx.save_for_backward(feats, weight, bias, masks[0])    # one bit per output: the activation's derivative
+        elif relu:
+            ctx.save_for_backward(feats, weight, bias, output)      # ... or the output itself, whose sign tells
         else:
             ctx.save_for_backward(feats, weight, bias)
         ctx.relu = relu
+        ctx.relu_bits = bool(relu and masks)
         ctx.neighbor_cache = neighbor_cache
         ctx.weight_owner = weakref.ref(weight)      # the caller's tensor object: kept weight panels hang on it
         ctx.mark_non_differentiable(out_coords)
@@ -417,7 +423,10 @@ class SparseConv3dFunction(Function):
 
     @staticmethod
     def backward(ctx, grad_output: torch.Tensor, _, __):
-        if ctx.relu:
+        if ctx.relu and ctx.relu_bits:
+            feats, weight, bias, mask = ctx.saved_tensors
+            grad_output = _relu_mask_apply(grad_output, mask)
+        elif ctx.relu:
             feats, weight, bias, output = ctx.saved_tensors
             grad_output = torch.where(output > 0, grad_output, torch.zeros((), dtype=grad_output.dtype, device=grad_output.device))
         else:

@@ -323,7 +323,7 @@ def _locality_order(coords: torch.Tensor, binary: torch.Tensor, v: int) -> torch
 
 # pair lists up to this many bytes (both together, at their bound of one entry per slot of the map) are allocated before
 # their length is known, which saves the build its wait for the host; larger ones wait and are allocated exactly
-PAIR_LISTS_UNSIZED_MAX_BYTES = 2 << 30
+PAIR_LISTS_UNSIZED_MAX_BYTES = 1 << 30
 
 
 def _pair_lists(nmap: torch.Tensor, gray: torch.Tensor, exact: bool = False):
@@ -360,6 +360,9 @@ def _pair_lists(nmap: torch.Tensor, gray: torch.Tensor, exact: bool = False):
     return {"seg": seg, "sig_i": sig_i, "sig_o": sig_o, "seg_host": seg_host}
 
 
+SORT_DECIDED_ON_DEVICE_MAX = 1 << 21     # fgx_subm_neighbor_map_sorted honours presorted = 2 up to this many voxels
+
+
 def _build_neighbor_map(coords: torch.Tensor, shape, kernel_size, dilation, with_codes: bool):
     n = coords.shape[0]
     B, _, W, H, D = [int(s) for s in shape]
@@ -379,13 +382,19 @@ def _build_neighbor_map(coords: torch.Tensor, shape, kernel_size, dilation, with
         key_bits = 32 if vol <= 2 ** 32 else 64
         with torch.cuda.device(dev):
             L = nat.lib()
-            # voxels that already come in scan order (a dense grid's nonzero(), a sorted voxelizer) need no key sort; the
-            # library finds out on the device (presorted = 2), so nothing is read back here
+            # voxels that already come in scan order (a dense grid's nonzero(), a sorted voxelizer) need no key sort.  Up to
+            # 2^21 voxels with 32-bit keys the library finds out on the device (presorted = 2) and nothing is read back;
+            # beyond that a skipped sort is worth more than the wait: one pass over the coordinates and a 4-byte read-back
+            presorted = 2
+            if n > SORT_DECIDED_ON_DEVICE_MAX or key_bits != 32:
+                descents = torch.zeros((1,), dtype=torch.int32, device=dev)
+                nat.check(L.fgx_coords_key_order(nat.ptr(coords), nat.sz(n), C.c_int(W), C.c_int(H), C.c_int(D), nat.ptr(descents), nat.stream()))
+                presorted = 1 if int(descents.item()) == 0 else 0
             ws = nat.workspace(L.fgx_subm_neighbor_map_sorted_workspace_bytes(nat.sz(n), C.c_int(key_bits), C.c_int(kw), C.c_int(kh)), dev)
             nat.check(L.fgx_subm_neighbor_map_sorted(
                 nat.ptr(coords), nat.sz(n), C.c_int(B), C.c_int(W), C.c_int(H), C.c_int(D), C.c_int(kw), C.c_int(kh), C.c_int(kd),
                 C.c_int(int(dilation[0])), C.c_int(int(dilation[1])), C.c_int(int(dilation[2])), C.c_int(key_bits),
-                C.c_int(2),
+                C.c_int(presorted),
                 nat.ptr(ws), nat.sz(ws.numel()), nat.ptr(nmap), nat.ptr(gray), nat.ptr(binary), nat.stream()))
         return nmap, gray, binary
     table = int(spconv.HASHMAP_RATIO * n)
