@@ -25,13 +25,13 @@ const Entry kTable[] = {
     {2, 2, 19, 128, 128, {128, 128, 64, 1, 2048, 2}},
     {0, 2, 17, 256, 256, {256, 128, 128, 1, 0, 1}},
     {1, 2, 17, 256, 256, {256, 128, 128, 1, 0, 1}},
-    {2, 2, 17, 256, 256, {128, 128, 64, 1, 12288, 1}},
+    {2, 2, 17, 256, 256, {256, 128, 64, 1, 16384, 1}},
     {0, 2, 21, 32, 32, {256, 32, 64, 1, 0, 1}},
     {1, 2, 21, 32, 32, {256, 32, 64, 1, 0, 1}},
     {2, 2, 21, 32, 32, {32, 32, 64, 1, 16384, 1}},
     {0, 2, 15, 1024, 1024, {256, 128, 128, 1, 0, 1}},
     {1, 2, 15, 1024, 1024, {256, 128, 128, 1, 0, 1}},
-    {2, 2, 15, 1024, 1024, {128, 128, 64, 1, 65536, 1}},
+    {2, 2, 15, 1024, 1024, {256, 128, 64, 1, 65536, 1}},
 };
 
 int floor_log2(size_t n) {
@@ -70,16 +70,24 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
             out->block_rows = 2048;
             return;
         }
+        // Wide weights on the streaming kernel: tiles of 256 (Co) x 128 (Ci) where they pad no more than 128 x 128 ones do.
+        // A step then loads 48 KiB of rows for twice the products (24 instead of 32 KiB per 512 MFMA cycles), and these
+        // shapes are bound by what the CUs can pull out of L2: C = 1024, 42 608 voxels 1.54 -> 1.34 ms; C = 512, 64 160
+        // voxels 0.70 -> 0.58; C = 256, 252 392 voxels 0.71 -> 0.54 (with blocks of 16 384 rows, which suit the longer
+        // tile better than 12 288: 0.58).
+        const bool tall = out->stream == 1 && t == 128 && Co > 128 && cdiv(Co, 256) * 256 == cdiv(Co, 128) * 128;
+        if (tall) out->tile_rows = 256;
         const int slices = (out->stream && t == 32) ? 4 : 1;
         const double per_block = 4.0 * V * (double)Co * (double)Ci * slices;
         size_t max_blocks = (size_t)(268435456.0 / per_block);
         if (max_blocks < 1) max_blocks = 1;
-        const size_t tiles = (size_t)cdiv(Co, t) * cdiv(Ci, t);
+        const size_t tiles = (size_t)cdiv(Co, out->tile_rows) * cdiv(Ci, out->tile_cols);
         size_t blocks_wanted = cdiv((size_t)4 * kCUs, (size_t)V * tiles);
         if (blocks_wanted < 1) blocks_wanted = 1;
         size_t rows = round_up(cdiv(n ? n : 1, blocks_wanted), 1024);
         if (rows < (size_t)4096 * slices) rows = (size_t)4096 * slices;
-        if (rows > (size_t)12288 * slices) rows = (size_t)12288 * slices;
+        const size_t longest = tall ? 16384 : (size_t)12288 * slices;
+        if (rows > longest) rows = longest;
         const size_t rows_mem = round_up((n + max_blocks - 1) / max_blocks, 1024);
         if (rows < rows_mem) rows = rows_mem;
         // even blocks: with a handful of them a short last block leaves its workgroups idle (two blocks of 12288 + 2904

@@ -316,7 +316,8 @@ struct WStreamCfg {
     // carries four times the pairs so that its loads are as many bytes as a wide tile's.
     static constexpr bool KSPLIT = BM == 32 && BN == 32;
     static constexpr int SLICES = KSPLIT ? 4 : 1;                  // partial products per (voxel block, offset, tile)
-    static constexpr int P = KSPLIT ? 4 * kWsPairs : kWsPairs, S = kWsStages;
+    // (a 256 x 128 tile's stages are 48 KiB: three of them fit, with the same 64-pair steps)
+    static constexpr int P = KSPLIT ? 4 * kWsPairs : kWsPairs, S = BM * BN > 128 * 128 ? 3 : kWsStages;
     static constexpr int NW = 4, NL = kWsLoaders, NT = 64 * (NW + NL);
     static constexpr int WM = KSPLIT ? BM : BM / 2, WN = KSPLIT ? BN : BN / 2, TM = WM / 32, TN = WN / 32;
     static constexpr int IDX_PER = P / 64;                         // wave-wide index loads per operand and step
@@ -329,6 +330,8 @@ struct WStreamCfg {
     static constexpr int IDX_SLOT_BYTES = 2 * P * 4;               // sig_o x P | sig_i x P
     static constexpr size_t lds_bytes = (size_t)S * STAGE_BYTES + (size_t)kWsIdxSlots * IDX_SLOT_BYTES;
     static_assert(ES == 2, "the streaming kernel handles 16-bit types");
+    static_assert(S == 3 || S == 4, "the loaders' wait is written for rings of three or four stages");
+    static_assert(kWsIdxAhead > S - 1 && lds_bytes <= 160 * 1024, "index loads run ahead of the row loads; the ring fits LDS");
     static_assert(IDX_PER == 1 || IDX_PER == NL, "index loads: one loader per operand, or every loader a quarter of both");
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
     static_assert(P % (RPI_A * NL) == 0 && P % (RPI_B * NL) == 0, "every loader issues the same row loads");
@@ -462,7 +465,7 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
         auto prep_rows = [&]() {
             pr_live = r.live;
             if (!r.live) return;
-            pr_stage = r_step & (S - 1);
+            pr_stage = r_step % S;
             const uint32_t* slot_p = idx_ring + (r_step & (kWsIdxSlots - 1)) * (2 * P);
             const unsigned co_tile = r.tile % co_tiles, ci_tile = r.tile / co_tiles;
             const uint32_t m0b = co_tile * (uint32_t)(BM * ES), n0b = ci_tile * (uint32_t)(BN * ES);
@@ -529,7 +532,8 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
             ops1 = ops;
         }
         while (true) {
-            wait_loads(ops1 + ops2);               // everything issued before the last two rounds has landed
+            // everything issued before the last S - 2 rounds has landed: the rows of the step the barrier opens
+            wait_loads(S == 4 ? ops1 + ops2 : ops1);
             asm volatile("" ::: "memory");
             __builtin_amdgcn_s_barrier();          // ... everybody's; the stage multiplied in the previous step is free
             asm volatile("" ::: "memory");
@@ -589,7 +593,8 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
         // Column sums of grad_out (the bias gradient) ride along with the offset whose pairs hold every output row once:
         // the grad_out fragments are multiplied by a fragment of ones as well, so every column of bacc is the sum.  Only
         // the wavefronts of the first column of wave tiles do it, for the first Ci-tile.
-        const bool do_bias = bias_partial != nullptr && (int)v == bias_offset && wave_n == 0 && tile < co_tiles;
+        // (not with 128-row wave tiles: the extra accumulators do not fit the register budget; the host then sums apart)
+        const bool do_bias = C::TM <= 2 && bias_partial != nullptr && (int)v == bias_offset && wave_n == 0 && tile < co_tiles;
         f32x16 bacc[C::TM];
 #pragma unroll
         for (int i = 0; i < C::TM; ++i)
@@ -602,7 +607,7 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
                 asm volatile("" ::: "memory");
                 __builtin_amdgcn_s_barrier();           // the loaders saw this step's rows land
                 asm volatile("" ::: "memory");
-                const uint32_t cur = ring_addr + (step & (S - 1)) * (uint32_t)C::STAGE_BYTES;
+                const uint32_t cur = ring_addr + (step % S) * (uint32_t)C::STAGE_BYTES;
                 ++step;
                 // Transposing read: in a 16-lane group, lane s supplies the address of 4 adjacent channels of pair row
                 // (s / 4) and receives the 4 pair values of channel (group base + s).  Lanes 0-15 / 16-31 cover fragment
@@ -649,8 +654,12 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
                 });
             }
         };
-        if (do_bias) run_steps(std::true_type{});
-        else run_steps(std::false_type{});
+        if constexpr (C::TM <= 2) {
+            if (do_bias) run_steps(std::true_type{});
+            else run_steps(std::false_type{});
+        } else {
+            run_steps(std::false_type{});
+        }
         // partial[b][v][co][ci], fp32
         const unsigned co_tile = tile % co_tiles, ci_tile = tile / co_tiles;
         const int m0 = (int)co_tile * BM, n0 = (int)ci_tile * BN;
@@ -1059,7 +1068,8 @@ int launch_wgrad_stream(const void* gout, const void* feats, const uint32_t* sig
 template <typename Tag>
 bool stream_ok(int tile_rows, int tile_cols, size_t n, size_t n_in, int Ci, int Co, uint32_t n_pairs) {
     if (sizeof(typename Tag::type) != 2) return false;
-    if (!((tile_rows == 128 && tile_cols == 128) || (tile_rows == 64 && tile_cols == 64) || (tile_rows == 32 && tile_cols == 32)))
+    if (!((tile_rows == 128 && tile_cols == 128) || (tile_rows == 64 && tile_cols == 64) || (tile_rows == 32 && tile_cols == 32) ||
+          (tile_rows == 256 && tile_cols == 128)))
         return false;
     // the 32 x 32 tile writes four partial products per voxel block; fgx_wgrad_scratch_bytes leaves room for them only
     // where the table picks that tile (at most 32 channels on a side): anything wider runs the tiled kernel
@@ -1073,6 +1083,7 @@ int dispatch_wgrad_stream(int tile_rows, const void* gout, const void* feats, co
                           const uint32_t* given_bounds, const SegTable& tab, const Layout& L, size_t n, size_t n_in, int V, int Ci, int Co, int block_rows,
                           void* scratch, void* gw, BiasOut bias, hipStream_t s) {
     if constexpr (sizeof(typename Tag::type) == 2) {
+        if (tile_rows == 256) return launch_wgrad_stream<Tag, 256, 128>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, s);
         if (tile_rows == 128) return launch_wgrad_stream<Tag, 128, 128>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, s);
         if (tile_rows == 64) return launch_wgrad_stream<Tag, 64, 64>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, s);
         return launch_wgrad_stream<Tag, 32, 32>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, s);
@@ -1171,7 +1182,7 @@ int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uin
     // hold every output row exactly once (the caller says which); every other path runs the stand-alone column sum.
     BiasOut bias;
     if (grad_bias != nullptr) {
-        const bool fuse = (stream_f16 || stream_bf16) && bias_offset >= 0 && bias_offset < V &&
+        const bool fuse = (stream_f16 || stream_bf16) && tile_rows <= 128 && bias_offset >= 0 && bias_offset < V &&
                           (size_t)(tab.seg[bias_offset + 1] - tab.seg[bias_offset]) == n;
         if (fuse) {
             bias.out = grad_bias;

@@ -196,7 +196,7 @@ def test_explicit_algorithm_matches_oracle_on_cpu():
 
 def test_wgrad_block_rule_keeps_its_promises(library):
     """The schedule rule for wgrad's voxel blocks: whole kibi-rows, even blocks where there are few, at most 12288 rows (four times that for
-    the 32 x 32 tile, which writes four partial products per block) unless the 256 MiB cap on fp32 partial products asks
+    the 32 x 32 tile, which writes four partial products per block; 16384 for 256 x 128 tiles) unless the 256 MiB cap on fp32 partial products asks
     for longer ones, and never more partial products than that cap allows."""
     import torch
     for c in (32, 64, 128, 256, 512, 1024):
@@ -214,5 +214,8 @@ def test_wgrad_block_rule_keeps_its_promises(library):
                 if blocks <= 4:         # with many blocks a short last one is immaterial
                     assert n - (blocks - 1) * rows > rows // 2, (n, c, rows, "short last block")
             cap_blocks = max((256 << 20) // (27 * c * c * 4 * slices), 1)
-            if rows > 12288 * slices:
-                assert -(-n // cap_blocks) > 12288 * slices - 1024 or (n >> 15, c) in ((1, 1024),), (n, c, rows)
+            longest = 16384 if s.tile_rows == 256 else 12288 * slices      # (256 x 128 tiles take longer blocks)
+            if rows > longest:
+                assert -(-n // cap_blocks) > longest - 1024 or (n >> 15, c) in ((1, 1024),), (n, c, rows)
+            # tiles of 256 x 128 for wide weights on the streaming kernel, where they pad no more than 128 x 128 ones
+            assert (s.tile_rows, s.tile_cols) == ((256, 128) if (s.stream == 1 and c >= 256) else (s.tile_cols, s.tile_cols)), (n, c)
