@@ -75,8 +75,11 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
         // shapes are bound by what the CUs can pull out of L2: C = 1024, 42 608 voxels 1.54 -> 1.34 ms; C = 512, 64 160
         // voxels 0.70 -> 0.58; C = 256, 252 392 voxels 0.71 -> 0.54 (with blocks of 16 384 rows, which suit the longer
         // tile better than 12 288: 0.58).
+        // The same with the long side along Ci (128 x 256 tiles) where only the input side is wide.
         const bool tall = out->stream == 1 && t == 128 && Co > 128 && cdiv(Co, 256) * 256 == cdiv(Co, 128) * 128;
+        const bool wide = out->stream == 1 && t == 128 && !tall && Ci > 128 && cdiv(Ci, 256) * 256 == cdiv(Ci, 128) * 128;
         if (tall) out->tile_rows = 256;
+        if (wide) out->tile_cols = 256;
         const int slices = (out->stream && t == 32) ? 4 : 1;
         const double per_block = 4.0 * V * (double)Co * (double)Ci * slices;
         size_t max_blocks = (size_t)(268435456.0 / per_block);
@@ -86,7 +89,7 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
         if (blocks_wanted < 1) blocks_wanted = 1;
         size_t rows = round_up(cdiv(n ? n : 1, blocks_wanted), 1024);
         if (rows < (size_t)4096 * slices) rows = (size_t)4096 * slices;
-        const size_t longest = tall ? 16384 : (size_t)12288 * slices;
+        const size_t longest = (tall || wide) ? 16384 : (size_t)12288 * slices;
         if (rows > longest) rows = longest;
         const size_t rows_mem = round_up((n + max_blocks - 1) / max_blocks, 1024);
         if (rows < rows_mem) rows = rows_mem;

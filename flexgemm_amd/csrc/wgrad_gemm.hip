@@ -593,8 +593,8 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
         // Column sums of grad_out (the bias gradient) ride along with the offset whose pairs hold every output row once:
         // the grad_out fragments are multiplied by a fragment of ones as well, so every column of bacc is the sum.  Only
         // the wavefronts of the first column of wave tiles do it, for the first Ci-tile.
-        // (not with 128-row wave tiles: the extra accumulators do not fit the register budget; the host then sums apart)
-        const bool do_bias = C::TM <= 2 && bias_partial != nullptr && (int)v == bias_offset && wave_n == 0 && tile < co_tiles;
+        // (not with 128 x 64 or 64 x 128 wave tiles: the extra accumulators do not fit the register budget; the host then sums apart)
+        const bool do_bias = C::TM * C::TN <= 4 && bias_partial != nullptr && (int)v == bias_offset && wave_n == 0 && tile < co_tiles;
         f32x16 bacc[C::TM];
 #pragma unroll
         for (int i = 0; i < C::TM; ++i)
@@ -654,7 +654,7 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
                 });
             }
         };
-        if constexpr (C::TM <= 2) {
+        if constexpr (C::TM * C::TN <= 4) {
             if (do_bias) run_steps(std::true_type{});
             else run_steps(std::false_type{});
         } else {
@@ -1069,7 +1069,7 @@ template <typename Tag>
 bool stream_ok(int tile_rows, int tile_cols, size_t n, size_t n_in, int Ci, int Co, uint32_t n_pairs) {
     if (sizeof(typename Tag::type) != 2) return false;
     if (!((tile_rows == 128 && tile_cols == 128) || (tile_rows == 64 && tile_cols == 64) || (tile_rows == 32 && tile_cols == 32) ||
-          (tile_rows == 256 && tile_cols == 128)))
+          (tile_rows == 256 && tile_cols == 128) || (tile_rows == 128 && tile_cols == 256)))
         return false;
     // the 32 x 32 tile writes four partial products per voxel block; fgx_wgrad_scratch_bytes leaves room for them only
     // where the table picks that tile (at most 32 channels on a side): anything wider runs the tiled kernel
@@ -1079,10 +1079,11 @@ bool stream_ok(int tile_rows, int tile_cols, size_t n, size_t n_in, int Ci, int 
 }
 
 template <typename Tag>
-int dispatch_wgrad_stream(int tile_rows, const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
+int dispatch_wgrad_stream(int tile_rows, int tile_cols, const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
                           const uint32_t* given_bounds, const SegTable& tab, const Layout& L, size_t n, size_t n_in, int V, int Ci, int Co, int block_rows,
                           void* scratch, void* gw, BiasOut bias, hipStream_t s) {
     if constexpr (sizeof(typename Tag::type) == 2) {
+        if (tile_cols == 256) return launch_wgrad_stream<Tag, 128, 256>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, s);
         if (tile_rows == 256) return launch_wgrad_stream<Tag, 256, 128>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, s);
         if (tile_rows == 128) return launch_wgrad_stream<Tag, 128, 128>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, s);
         if (tile_rows == 64) return launch_wgrad_stream<Tag, 64, 64>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, s);
@@ -1182,7 +1183,7 @@ int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uin
     // hold every output row exactly once (the caller says which); every other path runs the stand-alone column sum.
     BiasOut bias;
     if (grad_bias != nullptr) {
-        const bool fuse = (stream_f16 || stream_bf16) && tile_rows <= 128 && bias_offset >= 0 && bias_offset < V &&
+        const bool fuse = (stream_f16 || stream_bf16) && tile_rows <= 128 && tile_cols <= 128 && bias_offset >= 0 && bias_offset < V &&
                           (size_t)(tab.seg[bias_offset + 1] - tab.seg[bias_offset]) == n;
         if (fuse) {
             bias.out = grad_bias;
@@ -1194,9 +1195,9 @@ int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uin
     }
     // (outside the streaming kernel's range the tiled kernel runs)
     if (stream_f16)
-        return dispatch_wgrad_stream<F16>(tile_rows, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, bias, s);
+        return dispatch_wgrad_stream<F16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, bias, s);
     if (stream_bf16)
-        return dispatch_wgrad_stream<BF16>(tile_rows, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, bias, s);
+        return dispatch_wgrad_stream<BF16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, bias, s);
     switch (dtype) {
         case FGX_F16: return dispatch_wgrad<F16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);
         case FGX_BF16: return dispatch_wgrad<BF16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);

@@ -49,7 +49,10 @@ def test_host_only_entry_points(library):
     s = nat.table_lookup(nat.PASS_WGRAD, torch.bfloat16, 40000, 48, 64, 27)
     assert s.stream == 2 and (s.tile_rows, s.tile_cols) == (64, 64)
     # ... not for several tiles, 32 x 32 tiles, few voxels, more than 2^24 of them, or fp32
-    assert nat.table_lookup(nat.PASS_WGRAD, torch.float16, 669288, 256, 128, 27).stream == 1
+    s = nat.table_lookup(nat.PASS_WGRAD, torch.float16, 669288, 256, 128, 27)
+    assert s.stream == 1 and (s.tile_rows, s.tile_cols) == (128, 256)          # wide on the input side only
+    s = nat.table_lookup(nat.PASS_WGRAD, torch.float16, 669288, 128, 384, 27)
+    assert s.stream == 1 and (s.tile_rows, s.tile_cols) == (128, 128)          # 384 rows: 256-row tiles would pad more
     assert nat.table_lookup(nat.PASS_WGRAD, torch.float16, 669288, 32, 32, 27).stream == 1
     assert nat.table_lookup(nat.PASS_WGRAD, torch.float16, 4000, 128, 128, 27).stream == 1
     assert nat.table_lookup(nat.PASS_WGRAD, torch.float16, (1 << 24) + 1, 128, 128, 27).stream == 1
@@ -214,7 +217,7 @@ def test_wgrad_block_rule_keeps_its_promises(library):
                 if blocks <= 4:         # with many blocks a short last one is immaterial
                     assert n - (blocks - 1) * rows > rows // 2, (n, c, rows, "short last block")
             cap_blocks = max((256 << 20) // (27 * c * c * 4 * slices), 1)
-            longest = 16384 if s.tile_rows == 256 else 12288 * slices      # (256 x 128 tiles take longer blocks)
+            longest = 16384 if 256 in (s.tile_rows, s.tile_cols) else 12288 * slices      # (256 x 128 tiles take longer blocks)
             if rows > longest:
                 assert -(-n // cap_blocks) > longest - 1024 or (n >> 15, c) in ((1, 1024),), (n, c, rows)
             # tiles of 256 x 128 for wide weights on the streaming kernel, where they pad no more than 128 x 128 ones

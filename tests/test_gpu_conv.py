@@ -420,26 +420,27 @@ def test_streaming_wgrad_matches_oracle(gpu_device, dtype, res, ci, co, tile, bl
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("tile", [(256, 128), (128, 256)])
 @pytest.mark.parametrize("res,ci,co,block_rows", [(24, 128, 512, 1024), (16, 384, 256, 100000), (16, 256, 136, 300),
-                                                  (32, 200, 264, 37)])
-def test_streaming_wgrad_with_256x128_tiles_matches_oracle(gpu_device, dtype, res, ci, co, block_rows):
-    """The block-major streaming wgrad kernel on 256 x 128 tiles of the weight (three ring stages of 48 KiB, wave tiles
-    of 128 x 64): several tiles on both sides, ragged edge tiles, one voxel block and blocks shorter than a step; with a
+                                                  (32, 200, 264, 37), (24, 512, 96, 2048)])
+def test_streaming_wgrad_with_256x128_tiles_matches_oracle(gpu_device, dtype, res, ci, co, block_rows, tile):
+    """The block-major streaming wgrad kernel on 256 x 128 (Co x Ci) and 128 x 256 tiles of the weight (three ring stages of
+    48 KiB, wave tiles of 128 x 64 or 64 x 128): several tiles on both sides, ragged edge tiles, one voxel block and blocks shorter than a step; with a
     bias gradient, which this tile leaves to the column-sum kernel.  Against the 128 x 128 tile the sums per element run
     over the same pairs in the same order: bit-identical."""
     from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
-    _say(f"stream wgrad 256x128 res={res} ci={ci} co={co} block_rows={block_rows} {dtype}")
+    _say(f"stream wgrad {tile[0]}x{tile[1]} res={res} ci={ci} co={co} block_rows={block_rows} {dtype}")
     coords_np = reference_test_shell(res)
     shape = torch.Size([1, ci, res, res, res])
-    with _force_schedule(wgrad=True, tile_rows=256, tile_cols=128, block_rows=block_rows, stream=1):
+    with _force_schedule(wgrad=True, tile_rows=tile[0], tile_cols=tile[1], block_rows=block_rows, stream=1):
         cache, _ = _run_and_check(coords_np, shape, ci, co, dtype, gpu_device, seed=41)
     f, _, _, g = _case(coords_np, ci, co, dtype, 43)
     outs = []
-    for tr, tc in ((256, 128), (128, 128)):
+    for tr, tc in (tile, (128, 128)):
         with _force_schedule(wgrad=True, tile_rows=tr, tile_cols=tc, block_rows=block_rows, stream=1):
             gw, gb = impl._wgrad(g.to(gpu_device), f.to(gpu_device), cache, 27, with_bias=True, bias_offset=13)
             outs.append((gw.cpu(), gb.cpu()))
-    assert torch.equal(outs[0][0], outs[1][0]), "256 x 128 and 128 x 128 tiles differ"
+    assert torch.equal(outs[0][0], outs[1][0]), f"{tile[0]} x {tile[1]} and 128 x 128 tiles differ"
     assert eg.max_rel_err(outs[0][1], outs[1][1].double()) <= 2e-3
 
 
