@@ -564,6 +564,7 @@ int dispatch_stream(int tile_rows, int tile_cols, int slab_bytes, const void* sr
                                                          plan_rows, n, n_src, K, cols, cols_pad, panel_bytes, item_at, max_groups, act, out, relu_mask, s);
     FGX_STREAM_TILE(256, 128, FGX_BIG_WAVES_M, 2, 8)
     FGX_STREAM_TILE(256, 64, 4, 2, 8)
+    FGX_STREAM_TILE(128, 256, 2, 4, 8)      // few voxels, wide outputs: half the rows per tile pad less
     FGX_STREAM_TILE(256, 128, 4, 2, 4)      // 64-byte K-slabs: rows shorter than 128 bytes
     FGX_STREAM_TILE(256, 64, 4, 2, 4)
     FGX_STREAM_TILE(256, 32, 8, 1, 4)
@@ -646,6 +647,7 @@ bool stream_lds_fits(int tile_rows, int tile_cols, int slab_bytes, int cols) {
     if (tile_rows == BM && tile_cols == BN && slab_bytes == CHv * 16) fixed = StreamCfg<F16, BM, BN, WMv, WNv, CHv>::fixed_lds;
     FGX_STREAM_TILE(256, 128, FGX_BIG_WAVES_M, 2, 8)
     FGX_STREAM_TILE(256, 64, 4, 2, 8)
+    FGX_STREAM_TILE(128, 256, 2, 4, 8)      // few voxels, wide outputs: half the rows per tile pad less
     FGX_STREAM_TILE(256, 128, 4, 2, 4)
     FGX_STREAM_TILE(256, 64, 4, 2, 4)
     FGX_STREAM_TILE(256, 32, 8, 1, 4)
@@ -665,6 +667,7 @@ extern "C" int fgx_conv_gather_gemm_stream_groups(int dtype, int cols, int tile_
 #define FGX_STREAM_TILES(TAG)            \
     FGX_STREAM_TILE(TAG, 256, 128, FGX_BIG_WAVES_M, 2, 8) \
     FGX_STREAM_TILE(TAG, 256, 64, 4, 2, 8)  \
+    FGX_STREAM_TILE(TAG, 128, 256, 2, 4, 8) \
     FGX_STREAM_TILE(TAG, 256, 128, 4, 2, 4) \
     FGX_STREAM_TILE(TAG, 256, 64, 4, 2, 4)  \
     FGX_STREAM_TILE(TAG, 256, 32, 8, 1, 4)

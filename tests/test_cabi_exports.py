@@ -71,8 +71,12 @@ def test_host_only_entry_points(library):
     s = nat.table_lookup(nat.PASS_FWD, torch.float32, 100, 16, 16, 27)
     assert s.tile_rows in (32, 64, 128) and s.tile_cols == 32 and s.splitk >= 1 and s.stream == 0
     # rule (no table entry): big problems stream, small ones and rows below 64 bytes do not
-    s = nat.table_lookup(nat.PASS_DGRAD, torch.bfloat16, 300000, 192, 160, 27)
+    s = nat.table_lookup(nat.PASS_DGRAD, torch.bfloat16, 300000, 192, 160, 27)      # 192 input-gradient columns: one wide tile
+    assert (s.stream, s.tile_rows, s.tile_cols, s.slab_bytes, s.splitk) == (1, 128, 256, 128, 1)
+    s = nat.table_lookup(nat.PASS_FWD, torch.bfloat16, 300000, 192, 320, 27)        # beyond 256 columns: 256-row tiles
     assert (s.stream, s.tile_rows, s.tile_cols, s.slab_bytes, s.splitk) == (1, 256, 128, 128, 1)
+    s = nat.table_lookup(nat.PASS_FWD, torch.float16, 166232, 256, 256, 27)         # (a table entry)
+    assert (s.stream, s.tile_rows, s.tile_cols, s.slab_bytes, s.splitk) == (1, 128, 256, 128, 1)
     s = nat.table_lookup(nat.PASS_FWD, torch.bfloat16, 300000, 32, 32, 27)      # 64-byte rows: 64-byte slabs, 32-column tiles
     assert (s.stream, s.tile_rows, s.tile_cols, s.slab_bytes, s.splitk) == (1, 256, 32, 64, 1)
     s = nat.table_lookup(nat.PASS_DGRAD, torch.bfloat16, 300000, 96, 32, 27)    # K = Co = 32, 96 input-gradient columns

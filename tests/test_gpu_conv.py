@@ -240,6 +240,10 @@ def test_streaming_kernel_matches_oracle(gpu_device, dtype, res, ci, co):
     if co <= 136:   # the narrow-tile variant of the streaming kernel (64 columns per tile)
         with _force_schedule(tile_rows=256, tile_cols=64, slab_bytes=128, splitk=1, stream=1):
             _run_and_check(coords_np, shape, ci, co, dtype, gpu_device, seed=22)
+    # the wide-tile variant (128 rows x 256 columns: 2 x 4 multipliers), also where most of its columns are padding
+    with _force_schedule(tile_rows=128, tile_cols=256, slab_bytes=128, splitk=1, stream=1):
+        cache, _ = _run_and_check(coords_np, shape, ci, co, dtype, gpu_device, seed=24)
+    assert any(k.startswith("_plan_") and k.endswith("_128") for k in vars(cache)), "the 128-row gather plan was not used"
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
