@@ -57,6 +57,17 @@ def measured_counters(workload: str, dname: str, role: str):
     return {k: entry.get(k) for k in keys}
 
 
+def _finite(obj):
+    """The same structure with NaN and infinities replaced by None (they are not JSON)."""
+    if isinstance(obj, float):
+        return obj if math.isfinite(obj) else None
+    if isinstance(obj, dict):
+        return {k: _finite(v) for k, v in obj.items()}
+    if isinstance(obj, (list, tuple)):
+        return [_finite(v) for v in obj]
+    return obj
+
+
 def parse():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
@@ -365,13 +376,18 @@ def main():
 
     result, wl, cache, passes = measure(args.workload, args.dtype, args.steps, args.warmup, True)
     if args.build_only:
-        print(json.dumps(result))
+        print(json.dumps(_finite(result), allow_nan=False))
         return
     if not args.no_others and args.workload == "cfg3" and args.dtype is None:
         # the other configurations, a few steps each (no CPU leg, no phase split); configuration 4 also with the hash builder
         others = []
         for wname, dn in (("cfg2", None), ("cfg4", None), ("cfg5", None), ("cfg5", "f32")):
-            r, _, _, _ = measure(wname, dn, args.other_steps, 3, False, time_hash_builder=(wname == "cfg4"))
+            try:
+                r, _, _, _ = measure(wname, dn, args.other_steps, 3, False, time_hash_builder=(wname == "cfg4"))
+            except Exception as exc:       # the headline line must come out whatever happens to a side measurement
+                others.append({"workload": wname, "dtype": dn, "error": f"{type(exc).__name__}: {exc}"})
+                torch.cuda.empty_cache()
+                continue
             others.append({"workload": wname, "dtype": r["dtype"], "ms_per_step": r["ms_per_step"], "value": r["value"],
                            "unit": r["unit"], "steps": args.other_steps, "config": r["config"]["workload"],
                            "frac_of_mfma_peak": r["frac_of_mfma_peak"],
@@ -384,10 +400,13 @@ def main():
         result["other_workloads"] = others
     if not args.no_cpu_baseline:
         nmap_cpu = cache.neighbor_map.cpu().view(torch.int32)
-        result["cpu_baseline"] = cpu_baseline(wl, nmap_cpu, passes, args.cpu_rows)
+        try:
+            result["cpu_baseline"] = cpu_baseline(wl, nmap_cpu, passes, args.cpu_rows)
+        except Exception as exc:           # (as above: never at the price of the line itself)
+            result["cpu_baseline"] = {"error": f"{type(exc).__name__}: {exc}"}
     else:
         result["cpu_baseline"] = None
-    print(json.dumps(result, allow_nan=False))
+    print(json.dumps(_finite(result), allow_nan=False))
 
 
 if __name__ == "__main__":
