@@ -60,7 +60,9 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
         // on (both walk the same item list).  Its 32 x 32 tile
         // writes four partial products per voxel block (one per multiplying wavefront), so its blocks are four times
         // as long.
-        out->stream = (es == 2 && n >= 2048) ? 1 : 0;
+        // Under a weight of 512 x 512 channels and more it is ahead from the smallest layers on (C = 1024: 192 voxels 0.053 ->
+        // 0.048 ms, 848 voxels 0.084 -> 0.072, 1 976 voxels 0.134 -> 0.115; C = 512: 1 976 voxels 0.055 -> 0.043).
+        out->stream = (es == 2 && (n >= 2048 || (n >= 128 && (size_t)Ci * Co >= (size_t)512 * 512))) ? 1 : 0;
         // A weight of one 64 x 64 or 128 x 128 tile (33 ... 128 channels on both sides): the sweep (stream = 2) --
         // every workgroup keeps two accumulators over an eighth of the voxels, block_rows is its sub-block size.
         // Measured 20 % to 30 % ahead of the block-major kernel from ten thousand voxels (C = 128: 0.051 against
@@ -76,8 +78,9 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
         // voxels 0.70 -> 0.58; C = 256, 252 392 voxels 0.71 -> 0.54 (with blocks of 16 384 rows, which suit the longer
         // tile better than 12 288: 0.58).
         // The same with the long side along Ci (128 x 256 tiles) where only the input side is wide.
-        const bool tall = out->stream == 1 && t == 128 && Co > 128 && cdiv(Co, 256) * 256 == cdiv(Co, 128) * 128;
-        const bool wide = out->stream == 1 && t == 128 && !tall && Ci > 128 && cdiv(Ci, 256) * 256 == cdiv(Ci, 128) * 128;
+        // (from about three thousand voxels on: below, the square tile's larger number of items counts for more)
+        const bool tall = out->stream == 1 && n >= 3072 && t == 128 && Co > 128 && cdiv(Co, 256) * 256 == cdiv(Co, 128) * 128;
+        const bool wide = out->stream == 1 && n >= 3072 && t == 128 && !tall && Ci > 128 && cdiv(Ci, 256) * 256 == cdiv(Ci, 128) * 128;
         if (tall) out->tile_rows = 256;
         if (wide) out->tile_cols = 256;
         const int slices = (out->stream && t == 32) ? 4 : 1;
@@ -137,6 +140,20 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
             out->tile_rows = 128;
             out->tile_cols = 256;
         }
+    } else if (es == 2 && row_bytes >= 1024 && cols >= 128) {
+        // Too few tiles to stream and rows of 1 KiB or more (512 channels of a 16-bit type): a few hundred or thousand voxels
+        // under a weight of tens of megabytes.  The tiled kernel on 256 x 128 tiles and 128-byte slabs, with as many K
+        // splits as give every CU one workgroup, keeps more of the weight in flight than 128 x 128 tiles on 64-byte slabs
+        // (measured forward, C = 1024: 192 voxels 0.048 -> 0.042 ms, 848 voxels 0.090 -> 0.084, 1 976 voxels 0.227 -> 0.138;
+        // C = 512: 1 976 voxels 0.073 -> 0.054, 3 840 voxels 0.094 -> 0.085, 5 816 voxels 0.145 -> 0.133; at C = 256 the
+        // smaller tiles are level).
+        out->tile_rows = 256;
+        out->tile_cols = 128;
+        out->slab_bytes = 128;
+        const size_t wide_items = (size_t)cdiv(n ? n : 1, 256) * cdiv(cols, 128);
+        int sk = 1;
+        while (wide_items * (size_t)sk * 2 <= (size_t)kCUs && sk < 32) sk *= 2;
+        out->splitk = sk;
     }
 }
 

@@ -225,4 +225,7 @@ def test_wgrad_block_rule_keeps_its_promises(library):
             if rows > longest:
                 assert -(-n // cap_blocks) > longest - 1024 or (n >> 15, c) in ((1, 1024),), (n, c, rows)
             # tiles of 256 x 128 for wide weights on the streaming kernel, where they pad no more than 128 x 128 ones
-            assert (s.tile_rows, s.tile_cols) == ((256, 128) if (s.stream == 1 and c >= 256) else (s.tile_cols, s.tile_cols)), (n, c)
+            # (from about three thousand voxels on; smaller layers keep the square tile's larger number of items)
+            assert (s.tile_rows, s.tile_cols) == ((256, 128) if (s.stream == 1 and c >= 256 and n >= 3072) else (s.tile_cols, s.tile_cols)), (n, c)
+            # under weights of 512 x 512 and more the streaming kernel runs from 128 voxels on, otherwise from 2048
+            assert s.stream == (1 if (n >= 2048 or (n >= 128 and c >= 512)) else 0), (n, c)
