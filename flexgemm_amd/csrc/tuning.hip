@@ -108,6 +108,9 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
     out->tile_rows = n >= 4096 ? 128 : (n >= 1024 ? 64 : 32);
     if (out->tile_rows == 64 && out->tile_cols == 128) out->tile_rows = 128;
     if (out->tile_rows == 32 && out->tile_cols != 32) out->tile_rows = out->tile_cols == 64 ? 64 : 128;
+    // narrow outputs with fewer 128-row tiles than CUs: 64-row tiles before any split of K (15 192 voxels, C = 64: 0.036 ->
+    // 0.030 ms)
+    if (out->tile_rows == 128 && out->tile_cols == 64 && (size_t)cdiv(n, 128) * cdiv(cols, 64) < (size_t)kCUs) out->tile_rows = 64;
     out->block_rows = 0;
     out->stream = 0;
     out->slab_bytes = 64;
@@ -122,9 +125,17 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
     // behind); the short-row form, two workgroups per CU, keeps the bar of two items per CU.
     const int K = pass_kind == 0 ? Ci : Co;
     const size_t row_bytes = (size_t)K * es;
-    const int slab = row_bytes >= 128 ? 128 : 64;
-    const int scols = cols > 64 ? 128 : ((cols > 32 || slab == 128) ? 64 : 32);
-    const size_t enough = slab == 128 ? (size_t)kCUs * 7 / 16 : 2 * (size_t)kCUs;
+    // 16-bit rows of 128 ... 255 bytes (64 ... 127 channels) also take the 64-byte slabs: their rings leave room for two
+    // workgroups per CU, which is worth more than the longer pieces (measured forward, C = 64: 143 616 / 252 392 / 577 592 /
+    // 1 026 536 voxels -5 / -22 / -7 / -12 %; C = 80 and 96: -2 ... -5 %; from 256 bytes on the 128-byte slabs are ahead,
+    // C = 128: 0.049 against 0.056 ms at 64 160 voxels)
+    // ... given two items per CU to keep both workgroups busy (64 160 voxels, 251 items: 0.028 ms on 128-byte slabs, 0.031 on
+    // 64-byte ones)
+    const bool short_slabs = es == 2 && row_bytes >= 128 && row_bytes < 256 &&
+                             (size_t)cdiv(n, 256) * cdiv(cols, cols > 64 ? 128 : 64) >= 2 * (size_t)kCUs;
+    const int slab = (row_bytes >= 128 && !short_slabs) ? 128 : 64;
+    int scols = cols > 64 ? 128 : ((cols > 32 || row_bytes >= 128) ? 64 : 32);
+    const size_t enough = row_bytes >= 128 ? (size_t)kCUs * 7 / 16 : 2 * (size_t)kCUs;
     if (row_bytes >= 64 && (slab == 64 || cols >= 64) && (size_t)cdiv(n, 256) * cdiv(cols, scols) >= enough &&
         stream_lds_fits(256, scols, slab, cols)) {      // (from ~1900 output columns on the staged bias no longer fits)
         out->tile_rows = 256;
@@ -139,6 +150,14 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
         if (slab == 128 && cols > 128 && cols <= 256 && stream_lds_fits(128, 256, slab, cols)) {
             out->tile_rows = 128;
             out->tile_cols = 256;
+        }
+        // Half a chip's worth of items or fewer: tiles of 64 columns make twice as many, and a gathered row read twice
+        // from L2 costs less than idle CUs (measured forward: 15 192 voxels C = 256, 119 items, 0.074 -> 0.064 ms; 3 840
+        // voxels C = 1024, 120 items, 0.270 -> 0.223 ms).
+        if (slab == 128 && out->tile_cols >= 128 &&
+            (size_t)cdiv(n, out->tile_rows) * cdiv(cols, out->tile_cols) <= (size_t)kCUs / 2 && stream_lds_fits(256, 64, slab, cols)) {
+            out->tile_rows = 256;
+            out->tile_cols = 64;
         }
     } else if (es == 2 && row_bytes >= 1024 && cols >= 128) {
         // Too few tiles to stream and rows of 1 KiB or more (512 channels of a 16-bit type): a few hundred or thousand voxels

@@ -83,8 +83,14 @@ def test_host_only_entry_points(library):
     assert (s.stream, s.tile_rows, s.tile_cols, s.slab_bytes) == (1, 256, 128, 64)
     assert nat.table_lookup(nat.PASS_FWD, torch.float16, 300000, 16, 64, 27).stream == 0
     assert nat.table_lookup(nat.PASS_FWD, torch.float16, 300000, 128, 32, 27).stream == 0   # no 32-column tile for long rows
-    s = nat.table_lookup(nat.PASS_FWD, torch.float16, 300000, 64, 64, 27)
+    s = nat.table_lookup(nat.PASS_FWD, torch.float16, 300000, 64, 64, 27)       # 128-byte rows of a 16-bit type: 64-byte slabs
+    assert (s.stream, s.tile_rows, s.tile_cols, s.slab_bytes) == (1, 256, 64, 64)
+    s = nat.table_lookup(nat.PASS_FWD, torch.float32, 300000, 32, 64, 27)       # ... of fp32: 128-byte slabs as before
     assert (s.stream, s.tile_rows, s.tile_cols, s.slab_bytes) == (1, 256, 64, 128)
+    s = nat.table_lookup(nat.PASS_FWD, torch.float16, 15192, 256, 256, 27)      # 119 tiles of 128 x 256: 64-column tiles instead
+    assert (s.stream, s.tile_rows, s.tile_cols, s.slab_bytes) == (1, 256, 64, 128)
+    s = nat.table_lookup(nat.PASS_FWD, torch.float16, 64160, 256, 256, 27)
+    assert (s.stream, s.tile_rows, s.tile_cols, s.slab_bytes) == (1, 128, 256, 128)
     assert nat.table_lookup(nat.PASS_FWD, torch.float16, 5000, 192, 160, 27).stream == 0
     assert nat.table_lookup(nat.PASS_WGRAD, torch.float32, 300000, 192, 160, 27).stream == 0
     assert L.fgx_weight_panel_bytes(0, 0, 128, 128, 27, 64, 128) == 27 * 2 * 128 * 128
