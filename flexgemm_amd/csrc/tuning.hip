@@ -25,13 +25,10 @@ const Entry kTable[] = {
     {2, 2, 19, 128, 128, {128, 128, 64, 1, 2048, 2}},
     {0, 2, 17, 256, 256, {128, 256, 128, 1, 0, 1}},
     {1, 2, 17, 256, 256, {128, 256, 128, 1, 0, 1}},
-    {2, 2, 17, 256, 256, {256, 128, 64, 1, 16384, 1}},
     {0, 2, 21, 32, 32, {256, 32, 64, 1, 0, 1}},
     {1, 2, 21, 32, 32, {256, 32, 64, 1, 0, 1}},
-    {2, 2, 21, 32, 32, {32, 32, 64, 1, 16384, 1}},
     {0, 2, 15, 1024, 1024, {256, 128, 128, 1, 0, 1}},
     {1, 2, 15, 1024, 1024, {256, 128, 128, 1, 0, 1}},
-    {2, 2, 15, 1024, 1024, {256, 128, 64, 1, 65536, 1}},
 };
 
 int floor_log2(size_t n) {
@@ -46,23 +43,18 @@ size_t round_up(size_t x, size_t m) { return (x + m - 1) / m * m; }
 
 void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* out) {
     if (pass_kind == 2) {
-        // wgrad: square tiles over (Co, Ci); voxel blocks of 4096 to 12288 rows -- as long as that still leaves about
-        // four items (block, offset, tile) per CU: every item costs an exposed epilogue and a partial product, while
-        // blocks beyond ~12K rows overflow an XCD's L2 (measured at C = 128 ... 512: 12288 rows are 4 % to 11 % ahead of
-        // 4096 once there are enough voxels) -- enlarged further until the fp32 partial products (blocks x V x Co x Ci)
-        // stay below 256 MiB.
+        // wgrad: tiles over (Co, Ci) and voxel blocks; an item is (block, offset, tile), every item costs an exposed
+        // epilogue and a partial product, and the fp32 partial products (blocks x V x Co x Ci) stay below 256 MiB.
         int t = pick_cols(Ci < Co ? Ci : Co);
         out->tile_rows = t;
         out->tile_cols = t;
         out->slab_bytes = 64;
         out->splitk = 1;
-        // persistent streaming kernel: 16-bit types; measured ahead of the tiled kernel from about two thousand voxels
-        // on (both walk the same item list).  Its 32 x 32 tile
-        // writes four partial products per voxel block (one per multiplying wavefront), so its blocks are four times
-        // as long.
+        // persistent streaming kernel: 16-bit types; measured ahead of the tiled kernel from a few hundred voxels on
+        // (848 voxels: C = 32 0.024 -> 0.020 ms, C = 64 0.023 -> 0.020, C = 128 0.031 -> 0.020, C = 256 0.033 -> 0.023).
         // Under a weight of 512 x 512 channels and more it is ahead from the smallest layers on (C = 1024: 192 voxels 0.053 ->
         // 0.048 ms, 848 voxels 0.084 -> 0.072, 1 976 voxels 0.134 -> 0.115; C = 512: 1 976 voxels 0.055 -> 0.043).
-        out->stream = (es == 2 && (n >= 2048 || (n >= 128 && (size_t)Ci * Co >= (size_t)512 * 512))) ? 1 : 0;
+        out->stream = (es == 2 && (n >= 512 || (n >= 128 && (size_t)Ci * Co >= (size_t)512 * 512))) ? 1 : 0;
         // A weight of one 64 x 64 or 128 x 128 tile (33 ... 128 channels on both sides): the sweep (stream = 2) --
         // every workgroup keeps two accumulators over an eighth of the voxels, block_rows is its sub-block size.
         // Measured 20 % to 30 % ahead of the block-major kernel from ten thousand voxels (C = 128: 0.051 against
@@ -72,18 +64,67 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
             out->block_rows = 2048;
             return;
         }
-        // Wide weights on the streaming kernel: tiles of 256 (Co) x 128 (Ci) where they pad no more than 128 x 128 ones do.
-        // A step then loads 48 KiB of rows for twice the products (24 instead of 32 KiB per 512 MFMA cycles), and these
-        // shapes are bound by what the CUs can pull out of L2: C = 1024, 42 608 voxels 1.54 -> 1.34 ms; C = 512, 64 160
-        // voxels 0.70 -> 0.58; C = 256, 252 392 voxels 0.71 -> 0.54 (with blocks of 16 384 rows, which suit the longer
-        // tile better than 12 288: 0.58).
-        // The same with the long side along Ci (128 x 256 tiles) where only the input side is wide.
-        // (from about three thousand voxels on: below, the square tile's larger number of items counts for more)
-        const bool tall = out->stream == 1 && n >= 3072 && t == 128 && Co > 128 && cdiv(Co, 256) * 256 == cdiv(Co, 128) * 128;
-        const bool wide = out->stream == 1 && n >= 3072 && t == 128 && !tall && Ci > 128 && cdiv(Ci, 256) * 256 == cdiv(Ci, 128) * 128;
-        if (tall) out->tile_rows = 256;
-        if (wide) out->tile_cols = 256;
-        const int slices = (out->stream && t == 32) ? 4 : 1;
+        // Streaming kernel with balanced work lists (fgx_wgrad_item_lists): a launch takes as long as its most loaded
+        // workgroup, and the lists even the loads out as far as the items allow -- the largest item is the centre
+        // offset of a voxel block (one pair per row), the mean load is about 0.45 V pairs per voxel x tiles / CUs.
+        // So: the largest tile shape whose items still fill the chip one and a half times with blocks of 4096 rows or
+        // more, and as few blocks as keep a block's centre item below the mean load (CUs / (0.45 V x tiles) blocks).
+        // Measured on shells with the lists (ms, best of the swept tile shapes and block counts):
+        //   C = 256:  848 voxels 64 x 64 tiles 1 block 0.023 (tiled kernel 0.033);  3 840: 64 x 64, 1 block 0.035
+        //             (256 x 128: 0.063);  15 192: 128 x 128, 4 blocks 0.059 (256 x 128, 4: 0.077);  64 160: 256 x 128,
+        //             8 blocks 0.156, 11: 0.169 (16: 0.176);  166 232: 256 x 128, 11 blocks 0.295 (8: 0.337, 24: 0.329)
+        //   C = 512:  3 840: 128 x 128, 1 block 0.054 (256 x 128: 0.072);  15 192: 256 x 128, 2 blocks 0.144, 3: 0.150
+        //             (4: 0.162);  64 160: 256 x 128, 3 blocks 0.484 (5: 0.503, 8: 0.520)
+        //   C = 1024: 3 840 ... 64 160 voxels: 256 x 128, 1 block (42 608 voxels: 0.957, 2 blocks 1.02, 4: 1.12)
+        //   C = 32:   15 192: 8 blocks 0.026 (1: 0.040);  64 160: 11 blocks 0.030 (4: 0.046, 32: 0.040)
+        // Tiles of 256 x 128 (or 128 x 256 where only Ci is wide) where they pad no more than 128 x 128 ones do: a step
+        // then loads 48 KiB of rows for twice the products, and these shapes are bound by what the CUs can pull out
+        // of L2.  Below about three thousand voxels the square tile's larger number of items counts for more.
+        if (out->stream == 1) {
+            struct Shape { int rows, cols; };
+            Shape shapes[3];
+            int ns = 0;
+            if (t == 128) {
+                if (n >= 3072 && Co > 128 && cdiv(Co, 256) * 256 == cdiv(Co, 128) * 128) shapes[ns++] = {256, 128};
+                else if (n >= 3072 && Ci > 128 && cdiv(Ci, 256) * 256 == cdiv(Ci, 128) * 128) shapes[ns++] = {128, 256};
+                shapes[ns++] = {128, 128};
+                shapes[ns++] = {64, 64};
+            } else {
+                shapes[ns++] = {t, t};
+            }
+            size_t nb = 1, tiles = 1;
+            int slices = 1;
+            for (int i = 0; i < ns; ++i) {
+                const bool last = i == ns - 1;
+                slices = shapes[i].rows == 32 ? 4 : 1;           // the 32 x 32 tile splits a step's pairs over its four wavefronts
+                tiles = (size_t)cdiv(Co, shapes[i].rows) * cdiv(Ci, shapes[i].cols);
+                const size_t per_voxel = (size_t)V * 4 / 9 * (slices == 4 ? 2 : 1);
+                const size_t wanted = cdiv((size_t)kCUs, (per_voxel ? per_voxel : 1) * tiles);
+                const size_t shortest = slices == 4 ? 2048 : 4096;
+                const size_t most = n > shortest ? cdiv(n, shortest) : 1;
+                nb = wanted < most ? wanted : most;
+                out->tile_rows = shapes[i].rows;
+                out->tile_cols = shapes[i].cols;
+                const bool fills = 2 * (size_t)V * tiles * nb >= 3 * (size_t)kCUs;
+                if (last && !fills) {                           // nothing fills the chip: blocks down to 2048 rows
+                    const size_t most_short = n > 2048 ? cdiv(n, (size_t)2048) : 1;
+                    nb = wanted < most_short ? wanted : most_short;
+                }
+                if (last || fills) break;
+            }
+            // long blocks overflow an XCD's L2 when few tiles share their rows; partial products stay below 256 MiB
+            const size_t longest = tiles <= 4 ? 16384 : (tiles <= 8 ? 24576 : 65536);
+            if (nb < cdiv(n, longest)) nb = cdiv(n, longest);
+            size_t max_blocks = (size_t)(268435456.0 / (4.0 * V * (double)Co * (double)Ci * slices));
+            if (max_blocks < 1) max_blocks = 1;
+            if (nb > max_blocks) nb = max_blocks;
+            size_t rows = round_up(cdiv(n, nb), 1024);
+            if (rows > 0x40000000) rows = 0x40000000;
+            out->block_rows = (int)rows;
+            return;
+        }
+        // tiled kernel (fp32, or too few voxels for the streaming one)
+        const int slices = 1;
         const double per_block = 4.0 * V * (double)Co * (double)Ci * slices;
         size_t max_blocks = (size_t)(268435456.0 / per_block);
         if (max_blocks < 1) max_blocks = 1;
@@ -92,7 +133,7 @@ void rule(int pass_kind, int es, size_t n, int Ci, int Co, int V, fgx_schedule* 
         if (blocks_wanted < 1) blocks_wanted = 1;
         size_t rows = round_up(cdiv(n ? n : 1, blocks_wanted), 1024);
         if (rows < (size_t)4096 * slices) rows = (size_t)4096 * slices;
-        const size_t longest = (tall || wide) ? 16384 : (size_t)12288 * slices;
+        const size_t longest = (size_t)12288 * slices;
         if (rows > longest) rows = longest;
         const size_t rows_mem = round_up((n + max_blocks - 1) / max_blocks, 1024);
         if (rows < rows_mem) rows = rows_mem;

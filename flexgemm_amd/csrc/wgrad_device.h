@@ -32,6 +32,10 @@ template <> __device__ __forceinline__ __bf16 from_float<__bf16>(float x) {
 
 constexpr int kMaxV = 32;
 constexpr int kXcds = 8;
+// Balanced item lists of the streaming weight gradient: words [0..3] = {workgroups, items, tiles per (block, offset),
+// kItemListMagic}, then head[workgroups], then next[items]; kItemListEnd closes a chain.
+constexpr uint32_t kItemListEnd = 0xFFFFFFFFu, kItemListMagic = 0x4C495354u;
+constexpr int kItemListHeader = 4;
 
 #define FGX_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 #define FGX_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))

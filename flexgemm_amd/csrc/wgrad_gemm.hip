@@ -347,7 +347,7 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
                     const uint32_t* __restrict__ bounds, int V, int Ci, int Co, unsigned nb, unsigned co_tiles,
                     unsigned ci_tiles, uint32_t n_pairs, uint32_t gout_bytes, uint32_t feats_bytes,
                     float* __restrict__ partial, typename Tag::type* __restrict__ direct,
-                    float* __restrict__ bias_partial, int bias_offset) {
+                    float* __restrict__ bias_partial, int bias_offset, const uint32_t* __restrict__ lists) {
     using C = WStreamCfg<Tag, BM, BN>;
     constexpr int ES = C::ES, S = C::S, P = C::P;
 
@@ -363,12 +363,20 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
     const int g = lane >> 5, l32 = lane & 31;
 
     // ---- item list: block-major (block, offset, tile); XCD x owns the x-th eighth, its workgroups interleave ----
+    // With `lists` (head[workgroups] | next[items], kItemListEnd closes a chain) a workgroup walks the chain that the
+    // balancing pass made for it instead.
     const unsigned tiles = co_tiles * ci_tiles;
     const unsigned per_block = (unsigned)V * tiles;
     const unsigned total_items = nb * per_block;
     const unsigned per_xcd = (total_items + kXcds - 1) / kXcds;
     const unsigned xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds, stride = gridDim.x / kXcds;
-    const unsigned range_end = (xcd + 1) * per_xcd < total_items ? (xcd + 1) * per_xcd : total_items;
+    // (lists made for another launch shape are ignored: every partition of the items gives the same result, a list of
+    // the wrong size does not)
+    if (lists && !(lists[0] == gridDim.x && lists[1] == total_items && lists[2] == tiles && lists[3] == kItemListMagic)) lists = nullptr;
+    if (lists) lists += kItemListHeader;
+    const unsigned range_end = lists ? total_items : ((xcd + 1) * per_xcd < total_items ? (xcd + 1) * per_xcd : total_items);
+    const uint32_t* chain = lists ? lists + gridDim.x : nullptr;
+    auto after = [&](unsigned item) -> unsigned { return chain ? chain[item] : item + stride; };
 
     struct Walk {
         unsigned item;
@@ -391,18 +399,18 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
                 w.live = true;
                 return;
             }
-            w.item += stride;
+            w.item = after(w.item);
         }
     };
     auto advance = [&](Walk& w) {                   // one step further
         w.k += P;
         if (w.k >= w.k_hi) {
-            w.item += stride;
+            w.item = after(w.item);
             seek(w);
         }
     };
     Walk first;
-    first.item = xcd * per_xcd + slot;
+    first.item = lists ? lists[blockIdx.x] : xcd * per_xcd + slot;
     seek(first);
     if (!first.live) return;                        // whole workgroup: nothing to do
 
@@ -691,7 +699,7 @@ wgrad_stream_kernel(const typename Tag::type* __restrict__ gout, const typename 
                 }
         }
         m.k = m.k_hi;                               // on to the next non-empty item
-        m.item += stride;
+        m.item = after(m.item);
         seek(m);
     }
 }
@@ -1012,10 +1020,141 @@ int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, con
     return launch_reduce<T>(partial, bounds, V, Ci, Co, L.nb, 1u, (T*)gw, s);
 }
 
+// ------------------------------------------------------------------------------------------------
+// Balanced item lists for the streaming kernel.  Its items (voxel block, offset, tile) cost what their pair count says:
+// the centre offset pairs every row of a block, a corner offset a fraction, and dealt out in a fixed interleave the
+// workgroup with the most pairs sets the launch's time (measured on shells: the mean workgroup has 0.4 to 0.85 of the
+// largest one's pairs when there are 1 to 16 items per workgroup).  One workgroup builds the lists, longest processing
+// time first on two levels so that tiles of one (block, offset) -- which share the rows they gather through an XCD's
+// L2 -- stay on one XCD:
+//   1. chunks = up to 32 tiles of one (block, offset), cost = tiles x (pairs + kItemFixedCost); sorted by falling cost;
+//   2. each chunk goes to the XCD with the least cost so far (one thread, in sorted order);
+//   3. per XCD (one wavefront each): the chunks' items go, in the same order, to the workgroup of that XCD with the
+//      least cost so far; a workgroup's chain links its items in the order they arrived.
+// Items without pairs cost nothing and are linked too, so the chains cover every item whatever the pair lists hold.
+// ------------------------------------------------------------------------------------------------
+constexpr int kItemListMaxChunks = 8192;        // chunks the builder sorts in LDS
+constexpr unsigned kItemListMaxItems = 16384;   // beyond: the fixed interleave is balanced enough (>= 64 items per workgroup)
+constexpr unsigned kItemListMaxGroups = 512;    // 64 workgroups per XCD: one lane each
+constexpr uint32_t kItemFixedCost = 1280;       // an item's prologue, epilogue and share of the reduction, in pairs
+
+__global__ void __launch_bounds__(1024) wgrad_item_lists_kernel(const uint32_t* __restrict__ bounds, int V, unsigned nb,
+                                                                unsigned tiles, unsigned groups, uint32_t* __restrict__ out) {
+    __shared__ uint32_t key[kItemListMaxChunks];
+    __shared__ uint16_t sorted[kItemListMaxChunks];
+    __shared__ uint8_t xcd_of[kItemListMaxChunks];
+    const unsigned units = nb * (unsigned)V, per_unit = (tiles + 31) / 32, chunks = units * per_unit;
+    const unsigned items = units * tiles, per_xcd = groups / kXcds;
+    const int tid = threadIdx.x;
+    uint32_t* head = out + kItemListHeader;
+    uint32_t* next = head + groups;
+    auto unit_cost = [&](unsigned u) -> uint32_t {          // per item of unit u = b * V + v
+        const unsigned b = u / (unsigned)V, v = u % (unsigned)V;
+        const uint32_t cnt = bounds[v * (nb + 1) + b + 1] - bounds[v * (nb + 1) + b];
+        return cnt ? cnt + kItemFixedCost : 0u;
+    };
+    auto chunk_items = [&](unsigned m) -> unsigned {
+        const unsigned j = m % per_unit;
+        return tiles - 32 * j < 32 ? tiles - 32 * j : 32;
+    };
+    if (tid == 0) {
+        out[0] = groups;
+        out[1] = items;
+        out[2] = tiles;
+        out[3] = kItemListMagic;
+    }
+    for (unsigned m = tid; m < chunks; m += 1024) key[m] = unit_cost(m / per_unit) * chunk_items(m);
+    __syncthreads();
+    for (unsigned m = tid; m < chunks; m += 1024) {         // rank by counting: falling cost, ties by index
+        const uint32_t mine = key[m];
+        unsigned rank = 0;
+        for (unsigned j = 0; j < chunks; ++j) {
+            const uint32_t other = key[j];
+            rank += (other > mine || (other == mine && j < m)) ? 1u : 0u;
+        }
+        sorted[rank] = (uint16_t)m;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t load[kXcds];
+        for (int x = 0; x < kXcds; ++x) load[x] = 0;
+        for (unsigned r = 0; r < chunks; ++r) {
+            const unsigned m = sorted[r];
+            int best = 0;
+            for (int x = 1; x < kXcds; ++x)
+                if (load[x] < load[best]) best = x;
+            load[best] += key[m];
+            xcd_of[m] = (uint8_t)best;
+        }
+    }
+    __syncthreads();
+    const int wave = tid >> 6, lane = tid & 63;
+    if (wave >= kXcds) return;
+    // lane l < per_xcd is workgroup l * kXcds + wave (blockIdx % kXcds is the XCD a workgroup lands on)
+    uint32_t load = (unsigned)lane < per_xcd ? 0u : 0xFFFFFFFFu;
+    uint32_t tail = kItemListEnd;
+    bool any = false;
+    for (unsigned r = 0; r < chunks; ++r) {
+        const unsigned m = sorted[r];
+        if (xcd_of[m] != wave) continue;
+        const unsigned u = m / per_unit, k = chunk_items(m);
+        const uint32_t per = key[m] / k;
+        const unsigned first_item = u * tiles + 32 * (m % per_unit);
+        for (unsigned i = 0; i < k; ++i) {
+            // least loaded lane: minimum over (load, lane), loads stay below 2^26
+            uint32_t best = (load << 6) | (uint32_t)lane;
+            if (load == 0xFFFFFFFFu) best = 0xFFFFFFFFu;
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) {
+                const uint32_t o = (uint32_t)__shfl_xor((int)best, d, 64);
+                best = o < best ? o : best;
+            }
+            if ((best & 63u) == (uint32_t)lane) {
+                const uint32_t item = first_item + i;
+                if (any) next[tail] = item;
+                else head[(unsigned)lane * kXcds + wave] = item;
+                any = true;
+                tail = item;
+                load += per;
+            }
+        }
+    }
+    if ((unsigned)lane < per_xcd) {
+        if (any) next[tail] = kItemListEnd;
+        else head[(unsigned)lane * kXcds + wave] = kItemListEnd;
+    }
+}
+
+// workgroups of a streaming launch on the current device
+int stream_groups(unsigned* out) {
+    int dev = 0, cus = 0;
+    FGX_CHECK_HIP(hipGetDevice(&dev));
+    FGX_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    unsigned groups = (unsigned)(cus > 0 ? cus : 256);
+    groups = groups / kXcds * kXcds;                      // whole rounds over the XCDs
+    if (groups < (unsigned)kXcds) groups = kXcds;
+    *out = groups;
+    return FGX_OK;
+}
+
+// 0 where the lists do not apply (too many items for them to matter, or for the builder)
+size_t item_lists_words(size_t n, int V, int Ci, int Co, int tile_rows, int tile_cols, int block_rows, unsigned groups,
+                        unsigned* tiles_out, unsigned* nb_out) {
+    const size_t nb = cdiv(n, (size_t)block_rows);
+    const size_t tiles = (size_t)cdiv(Co, tile_rows) * cdiv(Ci, tile_cols);
+    const size_t items = nb * V * tiles, chunks = nb * V * cdiv(tiles, (size_t)32);
+    if (tiles_out) *tiles_out = (unsigned)tiles;
+    if (nb_out) *nb_out = (unsigned)nb;
+    if (items == 0 || items > kItemListMaxItems || chunks > (size_t)kItemListMaxChunks || groups > kItemListMaxGroups) return 0;
+    // loads are compared as 26-bit numbers
+    if ((double)items / (groups / kXcds) * ((double)block_rows + kItemFixedCost) * 4.0 >= 67108864.0) return 0;
+    return (size_t)kItemListHeader + groups + items;
+}
+
 template <typename Tag, int BM, int BN>
 int launch_wgrad_stream(const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
                         const uint32_t* given_bounds, const SegTable& tab, const Layout& L, size_t n, size_t n_in, int V, int Ci, int Co, int block_rows,
-                        void* scratch, void* gw, BiasOut bias, hipStream_t s) {
+                        void* scratch, void* gw, BiasOut bias, const uint32_t* lists, hipStream_t s) {
     using C = WStreamCfg<Tag, BM, BN>;
     using T = typename Tag::type;
     // the block table depends on the pair lists and block_rows alone: callers that keep it pass it in
@@ -1030,12 +1169,9 @@ int launch_wgrad_stream(const void* gout, const void* feats, const uint32_t* sig
         const unsigned co_tiles = cdiv(Co, BM), ci_tiles = cdiv(Ci, BN);
         const size_t items = (size_t)L.nb * V * co_tiles * ci_tiles;
         FGX_CHECK_ARG(items < 0x7FFFFFFFull, "fgx_conv_wgrad: too many work items (%zu); use larger voxel blocks", items);
-        int dev = 0, cus = 0;
-        FGX_CHECK_HIP(hipGetDevice(&dev));
-        FGX_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-        unsigned groups = (unsigned)(cus > 0 ? cus : 256);
-        groups = groups / kXcds * kXcds;                      // whole rounds over the XCDs
-        if (groups < (unsigned)kXcds) groups = kXcds;
+        unsigned groups = 0;
+        int grc = stream_groups(&groups);
+        if (grc != FGX_OK) return grc;
         auto kern = wgrad_stream_kernel<Tag, BM, BN>;
         static thread_local bool lds_raised = false;
         if (C::lds_bytes > 64 * 1024 && !lds_raised) {
@@ -1052,7 +1188,7 @@ int launch_wgrad_stream(const void* gout, const void* feats, const uint32_t* sig
         kern<<<groups, C::NT, C::lds_bytes, s>>>((const T*)gout, (const T*)feats, sig_i, sig_o, bounds, V, Ci, Co, L.nb, co_tiles,
                                                  ci_tiles, tab.seg[V], (uint32_t)(n * (size_t)Co * sizeof(T)),
                                                  (uint32_t)(n_in * (size_t)Ci * sizeof(T)), partial, direct ? (T*)gw : nullptr,
-                                                 bias_partial, bias.offset);
+                                                 bias_partial, bias.offset, lists);
         FGX_CHECK_LAUNCH("fgx_conv_wgrad(stream)");
         if (bias_partial) {
             bias_reduce_kernel<T><<<cdiv((size_t)Co, 32), 1024, 0, s>>>(bias_partial, bounds + (size_t)bias.offset * (L.nb + 1),
@@ -1081,13 +1217,13 @@ bool stream_ok(int tile_rows, int tile_cols, size_t n, size_t n_in, int Ci, int 
 template <typename Tag>
 int dispatch_wgrad_stream(int tile_rows, int tile_cols, const void* gout, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
                           const uint32_t* given_bounds, const SegTable& tab, const Layout& L, size_t n, size_t n_in, int V, int Ci, int Co, int block_rows,
-                          void* scratch, void* gw, BiasOut bias, hipStream_t s) {
+                          void* scratch, void* gw, BiasOut bias, const uint32_t* lists, hipStream_t s) {
     if constexpr (sizeof(typename Tag::type) == 2) {
-        if (tile_cols == 256) return launch_wgrad_stream<Tag, 128, 256>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, s);
-        if (tile_rows == 256) return launch_wgrad_stream<Tag, 256, 128>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, s);
-        if (tile_rows == 128) return launch_wgrad_stream<Tag, 128, 128>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, s);
-        if (tile_rows == 64) return launch_wgrad_stream<Tag, 64, 64>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, s);
-        return launch_wgrad_stream<Tag, 32, 32>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, s);
+        if (tile_cols == 256) return launch_wgrad_stream<Tag, 128, 256>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, lists, s);
+        if (tile_rows == 256) return launch_wgrad_stream<Tag, 256, 128>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, lists, s);
+        if (tile_rows == 128) return launch_wgrad_stream<Tag, 128, 128>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, lists, s);
+        if (tile_rows == 64) return launch_wgrad_stream<Tag, 64, 64>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, lists, s);
+        return launch_wgrad_stream<Tag, 32, 32>(gout, feats, sig_i, sig_o, given_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, gw, bias, lists, s);
     } else {
         set_error("fgx_conv_wgrad: the streaming kernel handles 16-bit types only");
         return FGX_ERR_UNSUPPORTED;
@@ -1147,10 +1283,42 @@ int fgx_wgrad_block_bounds(const uint32_t* sig_o, const uint32_t* seg_host, size
     return FGX_OK;
 }
 
+size_t fgx_wgrad_item_lists_count(size_t n, int V, int Ci, int Co, int tile_rows, int tile_cols, int block_rows) {
+    if (V < 1 || V > kMaxV || Ci <= 0 || Co <= 0 || tile_rows <= 0 || tile_cols <= 0 || block_rows <= 0) return 0;
+    unsigned groups = 0;
+    if (stream_groups(&groups) != FGX_OK) return 0;
+    return item_lists_words(n, V, Ci, Co, tile_rows, tile_cols, block_rows, groups, nullptr, nullptr);
+}
+
+int fgx_wgrad_item_lists(const uint32_t* block_bounds, size_t n, int V, int Ci, int Co, int tile_rows, int tile_cols,
+                         int block_rows, uint32_t* item_lists, fgx_stream_t stream) {
+    FGX_CHECK_ARG(V >= 1 && V <= kMaxV && Ci > 0 && Co > 0, "fgx_wgrad_item_lists: bad shape Ci=%d Co=%d V=%d", Ci, Co, V);
+    FGX_CHECK_ARG(tile_rows > 0 && tile_cols > 0 && block_rows > 0, "fgx_wgrad_item_lists: bad tile %d x %d or block_rows %d", tile_rows,
+                  tile_cols, block_rows);
+    FGX_CHECK_ARG(block_bounds && item_lists, "fgx_wgrad_item_lists: null buffer");
+    unsigned groups = 0, tiles = 0, nb = 0;
+    int rc = stream_groups(&groups);
+    if (rc != FGX_OK) return rc;
+    const size_t words = item_lists_words(n, V, Ci, Co, tile_rows, tile_cols, block_rows, groups, &tiles, &nb);
+    FGX_CHECK_ARG(words > 0, "fgx_wgrad_item_lists: no lists for this shape (fgx_wgrad_item_lists_count says 0)");
+    wgrad_item_lists_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(block_bounds, V, nb, tiles, groups, item_lists);
+    FGX_CHECK_LAUNCH("fgx_wgrad_item_lists");
+    return FGX_OK;
+}
+
 int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
                    const uint32_t* seg_host, const uint32_t* block_bounds, size_t n, size_t n_in, int Ci, int Co, int V,
                    int tile_rows, int tile_cols, int block_rows, int streaming, void* scratch, void* grad_weight,
                    void* grad_bias, int bias_offset, fgx_stream_t stream) {
+    return fgx_conv_wgrad_lists(dtype, grad_out, feats, sig_i, sig_o, seg_host, block_bounds, nullptr, n, n_in, Ci, Co, V, tile_rows,
+                                tile_cols, block_rows, streaming, scratch, grad_weight, grad_bias, bias_offset, stream);
+}
+
+int fgx_conv_wgrad_lists(int dtype, const void* grad_out, const void* feats, const uint32_t* sig_i, const uint32_t* sig_o,
+                         const uint32_t* seg_host, const uint32_t* block_bounds, const uint32_t* item_lists, size_t n, size_t n_in,
+                         int Ci, int Co, int V, int tile_rows, int tile_cols, int block_rows, int streaming, void* scratch,
+                         void* grad_weight, void* grad_bias, int bias_offset, fgx_stream_t stream) {
+    FGX_CHECK_ARG(item_lists == nullptr || block_bounds != nullptr, "fgx_conv_wgrad_lists: item lists go with the block table they were made from");
     FGX_CHECK_ARG(dtype_ok(dtype), "fgx_conv_wgrad: unknown dtype %d", dtype);
     FGX_CHECK_ARG(Ci > 0 && Co > 0 && V >= 1 && V <= kMaxV, "fgx_conv_wgrad: bad shape Ci=%d Co=%d V=%d", Ci, Co, V);
     FGX_CHECK_ARG(block_rows >= 1, "fgx_conv_wgrad: block_rows must be positive, got %d", block_rows);
@@ -1195,9 +1363,9 @@ int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats, const uin
     }
     // (outside the streaming kernel's range the tiled kernel runs)
     if (stream_f16)
-        return dispatch_wgrad_stream<F16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, bias, s);
+        return dispatch_wgrad_stream<F16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, bias, item_lists, s);
     if (stream_bf16)
-        return dispatch_wgrad_stream<BF16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, bias, s);
+        return dispatch_wgrad_stream<BF16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, n, n_in, V, Ci, Co, block_rows, scratch, grad_weight, bias, item_lists, s);
     switch (dtype) {
         case FGX_F16: return dispatch_wgrad<F16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);
         case FGX_BF16: return dispatch_wgrad<BF16>(tile_rows, tile_cols, grad_out, feats, sig_i, sig_o, block_bounds, tab, L, small, V, Ci, Co, block_rows, scratch, grad_weight, s);

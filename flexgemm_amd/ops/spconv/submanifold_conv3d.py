@@ -258,6 +258,25 @@ class SubMConv3dNeighborCache:
             setattr(self, key, bounds)
         return getattr(self, key)
 
+    def _wgrad_item_lists(self, block_rows: int, tile_rows: int, tile_cols: int, ci: int, co: int):
+        """Balanced work lists of the streaming weight gradient (fgx_wgrad_item_lists) for one block size, tile shape and
+        channel counts, made on the device from the block table and kept; None where the library has none for the shape."""
+        key = f"_wgrad_lists_{block_rows}_{tile_rows}_{tile_cols}_{ci}_{co}"
+        if not hasattr(self, key):
+            bounds = self._wgrad_bounds(block_rows)
+            n, v = self["neighbor_map"].shape
+            L = nat.lib()
+            lists = None
+            with torch.cuda.device(bounds.device):
+                words = int(L.fgx_wgrad_item_lists_count(nat.sz(n), C.c_int(v), C.c_int(ci), C.c_int(co), C.c_int(tile_rows),
+                                                         C.c_int(tile_cols), C.c_int(block_rows)))
+                if words > 0:
+                    lists = torch.empty((words,), dtype=torch.uint32, device=bounds.device)
+                    nat.check(L.fgx_wgrad_item_lists(nat.ptr(bounds), nat.sz(n), C.c_int(v), C.c_int(ci), C.c_int(co), C.c_int(tile_rows),
+                                                     C.c_int(tile_cols), C.c_int(block_rows), nat.ptr(lists), nat.stream()))
+            setattr(self, key, lists)
+        return getattr(self, key)
+
     def _wgrad_sweep_plan(self, sub_rows: int):
         """Step lists of the paced wgrad sweep (fgx_wgrad_sweep_plan): a function of the pair lists and the sub-block
         size alone, made once and kept."""
@@ -594,6 +613,9 @@ def _sweep_fits(n: int, n_in: int, ci: int, co: int, elem_bytes: int, n_pairs: i
 # pacing of the wgrad sweep: sub-blocks a workgroup may run ahead of the slowest one of its XCD, and the looks at the
 # others' progress after which it stops waiting (0 = no pacing, the default: the workgroups of an XCD stay close enough
 # together by themselves, and waiting costs more time than the L2 misses it saves)
+# The streaming weight gradient walks per-workgroup work lists balanced by pair count (fgx_wgrad_item_lists) where the
+# library has them for the shape; False = the kernel's fixed interleave.  Same result bit for bit.
+WGRAD_BALANCED_LISTS = True
 WGRAD_SWEEP_LEAD = 3
 WGRAD_SWEEP_MAX_POLLS = 0
 
@@ -640,13 +662,16 @@ def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int, with_b
             gb = gb[:co].contiguous() if with_bias else None
         return (gw, gb) if with_bias else gw
     bounds = cache._wgrad_bounds(sched.block_rows)
+    lists = None
+    if sched.stream == 1 and WGRAD_BALANCED_LISTS:
+        lists = cache._wgrad_item_lists(sched.block_rows, sched.tile_rows, sched.tile_cols, cip, cop)
     with torch.cuda.device(dev):
         scratch = nat.workspace(L.fgx_wgrad_scratch_bytes(nat.sz(n), C.c_int(v), C.c_int(cip), C.c_int(cop),
                                                           C.c_int(sched.block_rows)), dev)
         nat.mark("wgrad", "start")
-        nat.check(L.fgx_conv_wgrad(
+        nat.check(L.fgx_conv_wgrad_lists(
             C.c_int(code), nat.ptr(g), nat.ptr(f), nat.ptr(cache["valid_signal_i"]), nat.ptr(cache["valid_signal_o"]),
-            seg_arr, nat.ptr(bounds), nat.sz(n), nat.sz(n_in), C.c_int(cip), C.c_int(cop), C.c_int(v), C.c_int(sched.tile_rows), C.c_int(sched.tile_cols),
+            seg_arr, nat.ptr(bounds), nat.ptr(lists), nat.sz(n), nat.sz(n_in), C.c_int(cip), C.c_int(cop), C.c_int(v), C.c_int(sched.tile_rows), C.c_int(sched.tile_cols),
             C.c_int(sched.block_rows), C.c_int(sched.stream), nat.ptr(scratch), nat.ptr(gw), nat.ptr(gb), C.c_int(bias_offset),
             nat.stream()))
         nat.mark("wgrad", "stop")

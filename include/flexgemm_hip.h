@@ -332,6 +332,25 @@ int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats,
                    int streaming, void* scratch, void* grad_weight, void* grad_bias, int bias_offset,
                    fgx_stream_t stream);
 
+/* Balanced work lists for the streaming kernel of fgx_conv_wgrad (streaming = 1).  Its work items are (voxel block, offset,
+ * tile) and cost what their pair count says (the centre offset pairs every row of a block, a corner offset a fraction);
+ * dealt out in a fixed order, the workgroup with the most pairs sets the launch's time.  fgx_wgrad_item_lists reads the
+ * block table and deals the items longest-first to the least loaded XCD and workgroup (on the device, one small kernel:
+ * once per neighbor cache, block_rows and tile shape); fgx_conv_wgrad_lists is fgx_conv_wgrad walking those lists
+ * (item_lists = NULL: the fixed order; lists made for another shape are ignored).  The result is the same bit for bit
+ * either way: every item is still summed by one workgroup in the same order.  fgx_wgrad_item_lists_count gives the
+ * uint32 words of the lists, 0 where they do not apply (more than 16 384 items: the fixed order is balanced then).
+ * No counterpart in the reference, whose Triton launch leaves the order of its programs to the hardware scheduler
+ * (..._bwd_masked_implicit_gemm_splitk.py:278-317). */
+size_t fgx_wgrad_item_lists_count(size_t n, int V, int Ci, int Co, int tile_rows, int tile_cols, int block_rows);
+int fgx_wgrad_item_lists(const uint32_t* block_bounds, size_t n, int V, int Ci, int Co, int tile_rows, int tile_cols,
+                         int block_rows, uint32_t* item_lists, fgx_stream_t stream);
+int fgx_conv_wgrad_lists(int dtype, const void* grad_out, const void* feats,
+                         const uint32_t* sig_i, const uint32_t* sig_o, const uint32_t* seg_host, const uint32_t* block_bounds,
+                         const uint32_t* item_lists, size_t n, size_t n_in, int Ci, int Co, int V, int tile_rows, int tile_cols,
+                         int block_rows, int streaming, void* scratch, void* grad_weight, void* grad_bias, int bias_offset,
+                         fgx_stream_t stream);
+
 /* The same weight gradient as a sweep over the voxels, for 16-bit types, a single Co x Ci tile (`tile` = 128 or 64 >= Co,
  * Ci) and at most 2^24 rows per operand: each XCD takes a contiguous range of sub-blocks of `sub_rows` voxels holding an
  * eighth of the pairs, and every workgroup keeps the accumulators of two "units" (an offset, or a share of the 64-pair

@@ -208,12 +208,12 @@ def test_explicit_algorithm_matches_oracle_on_cpu():
 
 
 def test_wgrad_block_rule_keeps_its_promises(library):
-    """The schedule rule for wgrad's voxel blocks: whole kibi-rows, even blocks where there are few, at most 12288 rows (four times that for
-    the 32 x 32 tile, which writes four partial products per block; 16384 for 256 x 128 tiles) unless the 256 MiB cap on fp32 partial products asks
-    for longer ones, and never more partial products than that cap allows."""
+    """The schedule rule for wgrad's voxel blocks: whole kibi-rows, even blocks, never more fp32 partial products than the
+    256 MiB cap allows; on the streaming kernel, the tile shape and block count that the balanced work lists were measured
+    best with (the largest tile shape whose items fill the chip one and a half times, few blocks under many tiles)."""
     import torch
     for c in (32, 64, 128, 256, 512, 1024):
-        for n in (1, 192, 3840, 15192, 42608, 64160, 166232, 300000, 669288, 1026536, 2667120):
+        for n in (1, 192, 848, 3840, 15192, 42608, 64160, 166232, 300000, 669288, 1026536, 2667120):
             s = nat.table_lookup(nat.PASS_WGRAD, torch.float16, n, c, c, 27)
             rows = s.block_rows
             assert rows >= 1024 and rows % 1024 == 0, (n, c, rows)
@@ -224,14 +224,22 @@ def test_wgrad_block_rule_keeps_its_promises(library):
             slices = 4 if (s.stream and s.tile_rows == 32) else 1
             if blocks > 1:
                 assert blocks * slices * 27 * c * c * 4 <= 256 << 20, (n, c, rows, "partial products exceed the cap")
-                if blocks <= 4:         # with many blocks a short last one is immaterial
-                    assert n - (blocks - 1) * rows > rows // 2, (n, c, rows, "short last block")
-            cap_blocks = max((256 << 20) // (27 * c * c * 4 * slices), 1)
-            longest = 16384 if 256 in (s.tile_rows, s.tile_cols) else 12288 * slices      # (256 x 128 tiles take longer blocks)
-            if rows > longest:
-                assert -(-n // cap_blocks) > longest - 1024 or (n >> 15, c) in ((1, 1024),), (n, c, rows)
-            # tiles of 256 x 128 for wide weights on the streaming kernel, where they pad no more than 128 x 128 ones
-            # (from about three thousand voxels on; smaller layers keep the square tile's larger number of items)
-            assert (s.tile_rows, s.tile_cols) == ((256, 128) if (s.stream == 1 and c >= 256 and n >= 3072) else (s.tile_cols, s.tile_cols)), (n, c)
-            # under weights of 512 x 512 and more the streaming kernel runs from 128 voxels on, otherwise from 2048
-            assert s.stream == (1 if (n >= 2048 or (n >= 128 and c >= 512)) else 0), (n, c)
+                assert n - (blocks - 1) * rows > rows // 2 or blocks > 4, (n, c, rows, "short last block")
+            # 16-bit types stream from 512 voxels on, under weights of 512 x 512 and more from 128 on
+            assert s.stream == (1 if (n >= 512 or (n >= 128 and c >= 512)) else 0), (n, c)
+            if s.stream == 1:
+                tiles = -(-c // s.tile_rows) * -(-c // s.tile_cols)
+                items = 27 * tiles * blocks
+                assert items <= 16384 or n > 1 << 20, (n, c, "more items than the work lists take")
+                # 256 x 128 tiles only from about three thousand voxels on and only where their items fill the chip
+                if s.tile_rows == 256:
+                    assert c >= 256 and n >= 3072 and items >= 384, (n, c, items)
+                # few tiles: blocks of at most 16384 rows (an XCD's L2), unless the cap asks for longer ones
+                if tiles <= 4 and rows > 16384:
+                    assert -(-n // (rows - 1024)) > max((256 << 20) // (27 * c * c * 4 * slices), 1), (n, c, rows)
+    expect = {(848, 256): (64, 64, 1024), (3840, 256): (64, 64, 4096), (15192, 256): (128, 128, 4096), (166232, 256): (256, 128, 15360),
+              (3840, 512): (128, 128, 4096), (64160, 512): (256, 128, 21504), (42608, 1024): (256, 128, 43008), (848, 1024): (128, 128, 1024),
+              (15192, 32): (32, 32, 2048), (64160, 32): (32, 32, 6144), (848, 128): (64, 64, 1024)}
+    for (n, c), want in expect.items():
+        s = nat.table_lookup(nat.PASS_WGRAD, torch.float16, n, c, c, 27)
+        assert (s.tile_rows, s.tile_cols, s.block_rows, s.stream) == want + (1,), (n, c)

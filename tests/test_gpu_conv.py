@@ -448,6 +448,60 @@ def test_streaming_wgrad_with_256x128_tiles_matches_oracle(gpu_device, dtype, re
     assert eg.max_rel_err(outs[0][1], outs[1][1].double()) <= 2e-3
 
 
+@pytest.mark.parametrize("res,ci,co,tile,block_rows", [(32, 256, 256, (256, 128), 1024), (32, 256, 384, (128, 128), 4096), (24, 320, 128, (128, 256), 512),
+                                                       (40, 96, 96, (64, 64), 2048), (40, 32, 24, (32, 32), 1024), (16, 1024, 512, (256, 128), 1024),
+                                                       (24, 64, 64, (64, 64), 37)])
+def test_streaming_wgrad_balanced_lists_change_no_bit(gpu_device, res, ci, co, tile, block_rows):
+    """The streaming wgrad kernel walking the work lists that fgx_wgrad_item_lists balances by pair count against the same
+    kernel on its fixed interleave: every item is summed by one workgroup in the same order and the blocks are reduced in
+    the same order, so the results agree bit for bit.  The lists link every item exactly once (checked on the host), and
+    lists made for another shape are ignored by the kernel."""
+    import ctypes as C
+    from flexgemm_amd import _native as nat
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    _say(f"stream wgrad lists res={res} ci={ci} co={co} tile={tile} block_rows={block_rows}")
+    coords_np = reference_test_shell(res)
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    n = coords_np.shape[0]
+    shape = torch.Size([1, ci, res, res, res])
+    f, _, _, g = _case(coords_np, ci, co, torch.float16, 47)
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+    outs = {}
+    old = impl.WGRAD_BALANCED_LISTS
+    try:
+        for on in (False, True):
+            impl.WGRAD_BALANCED_LISTS = on
+            with _force_schedule(wgrad=True, tile_rows=tile[0], tile_cols=tile[1], block_rows=block_rows, stream=1):
+                gw, gb = impl._wgrad(g.to(gpu_device), f.to(gpu_device), cache, 27, with_bias=True, bias_offset=13)
+                outs[on] = (gw.cpu(), gb.cpu())
+        lists = cache._wgrad_item_lists(block_rows, tile[0], tile[1], ci, co)
+        assert lists is not None, "no lists for a shape of a few thousand items"
+        w = lists.cpu().numpy().astype(np.int64)
+        groups, items, tiles = int(w[0]), int(w[1]), int(w[2])
+        assert tiles == -(-co // tile[0]) * -(-ci // tile[1]) and items == 27 * tiles * -(-n // block_rows) and groups % 8 == 0
+        head, nxt = w[4:4 + groups], w[4 + groups:4 + groups + items]
+        seen = np.zeros(items, bool)
+        for h in head:
+            while h != 0xFFFFFFFF:
+                assert 0 <= h < items and not seen[h], "an item linked twice or out of range"
+                seen[h] = True
+                h = nxt[h]
+        assert seen.all(), "an item is on no list"
+        # lists of another shape in place of this one's: the kernel falls back to its fixed order
+        other = cache._wgrad_item_lists(block_rows + 1024, tile[0], tile[1], ci, co)
+        if other is not None and int(other.cpu().numpy()[1]) != items:
+            setattr(cache, f"_wgrad_lists_{block_rows}_{tile[0]}_{tile[1]}_{ci}_{co}", other)
+            with _force_schedule(wgrad=True, tile_rows=tile[0], tile_cols=tile[1], block_rows=block_rows, stream=1):
+                gw, gb = impl._wgrad(g.to(gpu_device), f.to(gpu_device), cache, 27, with_bias=True, bias_offset=13)
+            assert torch.equal(gw.cpu(), outs[False][0])
+    finally:
+        impl.WGRAD_BALANCED_LISTS = old
+    assert torch.equal(outs[True][0], outs[False][0]) and torch.equal(outs[True][1], outs[False][1])
+    # beyond 16 384 items the library makes no lists
+    L = nat.lib()
+    assert L.fgx_wgrad_item_lists_count(nat.sz(1 << 20), C.c_int(27), C.c_int(256), C.c_int(256), C.c_int(128), C.c_int(128), C.c_int(4096)) == 0
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("res,ci,co,tile,sub_rows,lead,max_polls", [
     (32, 128, 128, 128, 256, 3, 2000), (48, 128, 128, 128, 128, 1, 2000), (24, 64, 64, 64, 64, 3, 2000),
