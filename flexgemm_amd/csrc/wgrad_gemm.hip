@@ -1028,15 +1028,50 @@ int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, con
 // time first on two levels so that tiles of one (block, offset) -- which share the rows they gather through an XCD's
 // L2 -- stay on one XCD:
 //   1. chunks = up to 32 tiles of one (block, offset), cost = tiles x (pairs + kItemFixedCost); sorted by falling cost;
-//   2. each chunk goes to the XCD with the least cost so far (one thread, in sorted order);
+//   2. each chunk goes to the XCD with the least cost so far (one wavefront, in sorted order);
 //   3. per XCD (one wavefront each): the chunks' items go, in the same order, to the workgroup of that XCD with the
 //      least cost so far; a workgroup's chain links its items in the order they arrived.
 // Items without pairs cost nothing and are linked too, so the chains cover every item whatever the pair lists hold.
 // ------------------------------------------------------------------------------------------------
-constexpr int kItemListMaxChunks = 8192;        // chunks the builder sorts in LDS
-constexpr unsigned kItemListMaxItems = 16384;   // beyond: the fixed interleave is balanced enough (>= 64 items per workgroup)
+constexpr int kItemListMaxChunks = 2048;        // chunks the builder sorts in LDS (by counting ranks: quadratic)
+constexpr unsigned kItemListMaxItems = 4096;    // beyond (16 items per workgroup and more) the fixed interleave is balanced
+                                                // to within a few per cent, and the one-workgroup builder takes too long
+constexpr size_t kItemListMinRows = 2048;
+constexpr unsigned kItemListGreedyChunks = 256; // chunks dealt to the XCDs one by one
 constexpr unsigned kItemListMaxGroups = 512;    // 64 workgroups per XCD: one lane each
 constexpr uint32_t kItemFixedCost = 1280;       // an item's prologue, epilogue and share of the reduction, in pairs
+
+// minimum over the 64 lanes, in every lane: four shifts inside the rows of 16 lanes, then the rows' last lanes are
+// passed on (lanes shifted in from outside a row, and rows a step leaves out, take the identity)
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
+#define FGX_MIN_STEP(ctrl, rows)                                                                               \
+    {                                                                                                          \
+        const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)0xFFFFFFFF, (int)v, ctrl, rows, 0xF, false); \
+        v = o < v ? o : v;                                                                                     \
+    }
+    FGX_MIN_STEP(0x111, 0xF)    // row_shr:1
+    FGX_MIN_STEP(0x112, 0xF)    // row_shr:2
+    FGX_MIN_STEP(0x114, 0xF)    // row_shr:4
+    FGX_MIN_STEP(0x118, 0xF)    // row_shr:8: lane 15 of every row holds the row's minimum
+    FGX_MIN_STEP(0x142, 0xA)    // row_bcast:15 into rows 1 and 3
+    FGX_MIN_STEP(0x143, 0xC)    // row_bcast:31 into rows 2 and 3: lane 63 holds the minimum
+#undef FGX_MIN_STEP
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+
+// minimum over lanes 0 ... 7, in every lane
+__device__ __forceinline__ uint32_t first8_min_u32(uint32_t v) {
+#define FGX_MIN_STEP(ctrl)                                                                                    \
+    {                                                                                                         \
+        const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)0xFFFFFFFF, (int)v, ctrl, 0xF, 0xF, false); \
+        v = o < v ? o : v;                                                                                    \
+    }
+    FGX_MIN_STEP(0x111)         // row_shr:1
+    FGX_MIN_STEP(0x112)         // row_shr:2
+    FGX_MIN_STEP(0x114)         // row_shr:4: lane 7 holds the minimum of lanes 0 ... 7
+#undef FGX_MIN_STEP
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 7);
+}
 
 __global__ void __launch_bounds__(1024) wgrad_item_lists_kernel(const uint32_t* __restrict__ bounds, int V, unsigned nb,
                                                                 unsigned tiles, unsigned groups, uint32_t* __restrict__ out) {
@@ -1075,51 +1110,93 @@ __global__ void __launch_bounds__(1024) wgrad_item_lists_kernel(const uint32_t* 
         sorted[rank] = (uint16_t)m;
     }
     __syncthreads();
-    if (tid == 0) {
-        uint32_t load[kXcds];
-        for (int x = 0; x < kXcds; ++x) load[x] = 0;
-        for (unsigned r = 0; r < chunks; ++r) {
-            const unsigned m = sorted[r];
-            int best = 0;
-            for (int x = 1; x < kXcds; ++x)
-                if (load[x] < load[best]) best = x;
-            load[best] += key[m];
-            xcd_of[m] = (uint8_t)best;
+    const int wave = tid >> 6, lane = tid & 63;
+    if (wave == 0) {
+        // Chunks to XCDs: lane x < 8 keeps XCD x's cost so far (in units of 32 pairs).  The first kItemListGreedyChunks
+        // chunks -- the large ones -- go one by one to the least loaded XCD; the tail goes eight at a time, the largest
+        // of a round to the least loaded XCD.
+        const bool bin = lane < kXcds;
+        uint32_t load = 0;
+        const unsigned greedy = chunks < kItemListGreedyChunks ? chunks : kItemListGreedyChunks;
+        for (unsigned r0 = 0; r0 < greedy; r0 += 64) {
+            const unsigned r = r0 + lane;
+            const unsigned m = r < greedy ? sorted[r] : 0u;
+            const uint32_t cost = r < greedy ? key[m] >> 5 : 0u;
+            const unsigned count = greedy - r0 < 64 ? greedy - r0 : 64;
+            int mine = 0;
+            for (unsigned j = 0; j < count; ++j) {
+                const uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)cost, (int)j);
+                const int best = (int)(first8_min_u32((load << 6) | (uint32_t)lane) & 63u);
+                if (lane == best) load += c;
+                if ((unsigned)lane == j) mine = best;
+            }
+            if (r < greedy) xcd_of[m] = (uint8_t)mine;
+        }
+        for (unsigned r0 = greedy; r0 < chunks; r0 += kXcds) {
+            unsigned rank = 0;
+#pragma unroll
+            for (int o = 0; o < kXcds; ++o) {
+                const uint32_t other = (uint32_t)__builtin_amdgcn_readlane((int)load, o);
+                rank += (other < load || (other == load && o < lane)) ? 1u : 0u;
+            }
+            if (bin && r0 + rank < chunks) {
+                const unsigned m = sorted[r0 + rank];
+                xcd_of[m] = (uint8_t)lane;
+                load += key[m] >> 5;
+            }
         }
     }
     __syncthreads();
-    const int wave = tid >> 6, lane = tid & 63;
     if (wave >= kXcds) return;
-    // lane l < per_xcd is workgroup l * kXcds + wave (blockIdx % kXcds is the XCD a workgroup lands on)
-    uint32_t load = (unsigned)lane < per_xcd ? 0u : 0xFFFFFFFFu;
+    // Wavefront x deals the items of XCD x's chunks, in the same order, each to the least loaded workgroup of the XCD;
+    // lane l < per_xcd is workgroup l * kXcds + x (blockIdx % kXcds is the XCD a workgroup lands on).  A workgroup's
+    // chain links its items in the order they arrived.
+    const bool bin = (unsigned)lane < per_xcd;
+    uint32_t load = 0;
     uint32_t tail = kItemListEnd;
     bool any = false;
-    for (unsigned r = 0; r < chunks; ++r) {
-        const unsigned m = sorted[r];
-        if (xcd_of[m] != wave) continue;
-        const unsigned u = m / per_unit, k = chunk_items(m);
-        const uint32_t per = key[m] / k;
-        const unsigned first_item = u * tiles + 32 * (m % per_unit);
-        for (unsigned i = 0; i < k; ++i) {
-            // least loaded lane: minimum over (load, lane), loads stay below 2^26
-            uint32_t best = (load << 6) | (uint32_t)lane;
-            if (load == 0xFFFFFFFFu) best = 0xFFFFFFFFu;
-#pragma unroll
-            for (int d = 32; d >= 1; d >>= 1) {
-                const uint32_t o = (uint32_t)__shfl_xor((int)best, d, 64);
-                best = o < best ? o : best;
-            }
-            if ((best & 63u) == (uint32_t)lane) {
-                const uint32_t item = first_item + i;
-                if (any) next[tail] = item;
-                else head[(unsigned)lane * kXcds + wave] = item;
+    for (unsigned r0 = 0; r0 < chunks; r0 += 64) {
+        const unsigned r = r0 + lane;
+        const unsigned m_l = r < chunks ? sorted[r] : 0u;
+        const bool here = r < chunks && xcd_of[m_l] == wave;
+        const uint32_t key_l = key[m_l];
+        uint64_t todo = __ballot(here);
+        while (todo) {
+            const int j = __builtin_ctzll(todo);
+            todo &= todo - 1;
+            const unsigned m = (unsigned)__builtin_amdgcn_readlane((int)m_l, j);
+            const unsigned u = m / per_unit, k = chunk_items(m);
+            const uint32_t per = (uint32_t)__builtin_amdgcn_readlane((int)key_l, j) / k;
+            const unsigned first_item = u * tiles + 32 * (m % per_unit);
+            auto take = [&](uint32_t it) {
+                if (any) next[tail] = it;
+                else head[(unsigned)lane * kXcds + wave] = it;
                 any = true;
-                tail = item;
+                tail = it;
                 load += per;
+            };
+            if (k < 8) {
+                for (unsigned i = 0; i < k; ++i) {
+                    const int best = (int)(wave_min_u32(bin ? (load << 6) | (uint32_t)lane : 0xFFFFFFFFu) & 63u);
+                    if (lane == best) take(first_item + i);
+                }
+            } else {
+                // many items of one cost: the least loaded workgroups take one each (what dealing them one by one does
+                // unless a single item is smaller than the gaps between the loads), per_xcd at a time
+                for (unsigned done = 0; done < k;) {
+                    const unsigned now = k - done < per_xcd ? k - done : per_xcd;
+                    unsigned rank = 0;
+                    for (unsigned o = 0; o < per_xcd; ++o) {
+                        const uint32_t other = (uint32_t)__builtin_amdgcn_readlane((int)load, (int)o);
+                        rank += (other < load || (other == load && o < (unsigned)lane)) ? 1u : 0u;
+                    }
+                    if (bin && rank < now) take(first_item + done + rank);
+                    done += now;
+                }
             }
         }
     }
-    if ((unsigned)lane < per_xcd) {
+    if (bin) {
         if (any) next[tail] = kItemListEnd;
         else head[(unsigned)lane * kXcds + wave] = kItemListEnd;
     }
@@ -1146,8 +1223,10 @@ size_t item_lists_words(size_t n, int V, int Ci, int Co, int tile_rows, int tile
     if (tiles_out) *tiles_out = (unsigned)tiles;
     if (nb_out) *nb_out = (unsigned)nb;
     if (items == 0 || items > kItemListMaxItems || chunks > (size_t)kItemListMaxChunks || groups > kItemListMaxGroups) return 0;
-    // loads are compared as 26-bit numbers
-    if ((double)items / (groups / kXcds) * ((double)block_rows + kItemFixedCost) * 4.0 >= 67108864.0) return 0;
+    // a launch over fewer voxels is over before the lists have paid for their making
+    if (n < kItemListMinRows) return 0;
+    // a workgroup's load is compared as a 26-bit number: the mean load plus the largest item, with a factor of two to spare
+    if (((double)items / groups + 1.0) * ((double)block_rows + kItemFixedCost) * 2.0 >= 67108864.0) return 0;
     return (size_t)kItemListHeader + groups + items;
 }
 

@@ -230,7 +230,7 @@ def test_wgrad_block_rule_keeps_its_promises(library):
             if s.stream == 1:
                 tiles = -(-c // s.tile_rows) * -(-c // s.tile_cols)
                 items = 27 * tiles * blocks
-                assert items <= 16384 or n > 1 << 20, (n, c, "more items than the work lists take")
+                assert items <= 4096 or n > 1 << 20, (n, c, "more items than the work lists take")
                 # 256 x 128 tiles only from about three thousand voxels on and only where their items fill the chip
                 if s.tile_rows == 256:
                     assert c >= 256 and n >= 3072 and items >= 384, (n, c, items)
