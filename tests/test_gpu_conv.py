@@ -450,7 +450,7 @@ def test_streaming_wgrad_with_256x128_tiles_matches_oracle(gpu_device, dtype, re
 
 @pytest.mark.parametrize("res,ci,co,tile,block_rows", [(32, 256, 256, (256, 128), 1024), (32, 256, 384, (128, 128), 4096), (28, 320, 128, (128, 256), 512),
                                                        (40, 96, 96, (64, 64), 2048), (40, 32, 24, (32, 32), 1024), (32, 1024, 512, (256, 128), 1024),
-                                                       (32, 64, 64, (64, 64), 37)])
+                                                       (32, 64, 64, (64, 64), 64)])
 def test_streaming_wgrad_balanced_lists_change_no_bit(gpu_device, res, ci, co, tile, block_rows):
     """The streaming wgrad kernel walking the work lists that fgx_wgrad_item_lists balances by pair count against the same
     kernel on its fixed interleave: every item is summed by one workgroup in the same order and the blocks are reduced in
