@@ -1036,7 +1036,7 @@ int launch_wgrad(const void* gout, const void* feats, const uint32_t* sig_i, con
 constexpr int kItemListMaxChunks = 2048;        // chunks the builder sorts in LDS (by counting ranks: quadratic)
 constexpr unsigned kItemListMaxItems = 4096;    // beyond (16 items per workgroup and more) the fixed interleave is balanced
                                                 // to within a few per cent, and the one-workgroup builder takes too long
-constexpr size_t kItemListMinRows = 2048;
+constexpr size_t kItemListMinRows = 2048, kItemListMaxBlocks = 12, kItemListMaxBlocksTiled = 16;
 constexpr unsigned kItemListGreedyChunks = 256; // chunks dealt to the XCDs one by one
 constexpr unsigned kItemListMaxGroups = 512;    // 64 workgroups per XCD: one lane each
 constexpr uint32_t kItemFixedCost = 1280;       // an item's prologue, epilogue and share of the reduction, in pairs
@@ -1225,6 +1225,12 @@ size_t item_lists_words(size_t n, int V, int Ci, int Co, int tile_rows, int tile
     if (items == 0 || items > kItemListMaxItems || chunks > (size_t)kItemListMaxChunks || groups > kItemListMaxGroups) return 0;
     // a launch over fewer voxels is over before the lists have paid for their making
     if (n < kItemListMinRows) return 0;
+    // The lists deal by cost alone and scatter the offsets of a voxel block over the XCDs; the fixed order keeps them on
+    // one XCD at one time, where they share the block's rows in L2.  With many blocks the fixed order is balanced well
+    // enough and the sharing counts for more (252 392 voxels, 32 channels, 16 blocks: 0.061 ms fixed, 0.070 with lists;
+    // 1 026 536 voxels, 63 blocks: 0.163 against 0.327; 256 channels, 16 blocks: 0.559 against 0.512).
+    // (up to 12 blocks of single-tile items, 16 of several tiles, which share more per block and XCD)
+    if (nb > (tiles >= 2 ? kItemListMaxBlocksTiled : kItemListMaxBlocks)) return 0;
     // a workgroup's load is compared as a 26-bit number: the mean load plus the largest item, with a factor of two to spare
     if (((double)items / groups + 1.0) * ((double)block_rows + kItemFixedCost) * 2.0 >= 67108864.0) return 0;
     return (size_t)kItemListHeader + groups + items;

@@ -339,7 +339,8 @@ int fgx_conv_wgrad(int dtype, const void* grad_out, const void* feats,
  * once per neighbor cache, block_rows and tile shape); fgx_conv_wgrad_lists is fgx_conv_wgrad walking those lists
  * (item_lists = NULL: the fixed order; lists made for another shape are ignored).  The result is the same bit for bit
  * either way: every item is still summed by one workgroup in the same order.  fgx_wgrad_item_lists_count gives the
- * uint32 words of the lists, 0 where they do not apply (more than 4 096 items: the fixed order is balanced then).
+ * uint32 words of the lists, 0 where they do not apply (fewer than 2 048 voxels; more than 12 voxel blocks (16 with several tiles) or 4 096 items: the fixed order, which
+ * keeps the offsets of a voxel block on one XCD, is balanced well enough then).
  * No counterpart in the reference, whose Triton launch leaves the order of its programs to the hardware scheduler
  * (..._bwd_masked_implicit_gemm_splitk.py:278-317). */
 size_t fgx_wgrad_item_lists_count(size_t n, int V, int Ci, int Co, int tile_rows, int tile_cols, int block_rows);

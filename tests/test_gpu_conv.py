@@ -450,7 +450,7 @@ def test_streaming_wgrad_with_256x128_tiles_matches_oracle(gpu_device, dtype, re
 
 @pytest.mark.parametrize("res,ci,co,tile,block_rows", [(32, 256, 256, (256, 128), 1024), (32, 256, 384, (128, 128), 4096), (28, 320, 128, (128, 256), 512),
                                                        (40, 96, 96, (64, 64), 2048), (40, 32, 24, (32, 32), 1024), (32, 1024, 512, (256, 128), 1024),
-                                                       (32, 64, 64, (64, 64), 64)])
+                                                       (32, 64, 64, (64, 64), 512)])
 def test_streaming_wgrad_balanced_lists_change_no_bit(gpu_device, res, ci, co, tile, block_rows):
     """The streaming wgrad kernel walking the work lists that fgx_wgrad_item_lists balances by pair count against the same
     kernel on its fixed interleave: every item is summed by one workgroup in the same order and the blocks are reduced in
@@ -497,9 +497,11 @@ def test_streaming_wgrad_balanced_lists_change_no_bit(gpu_device, res, ci, co, t
     finally:
         impl.WGRAD_BALANCED_LISTS = old
     assert torch.equal(outs[True][0], outs[False][0]) and torch.equal(outs[True][1], outs[False][1])
-    # beyond 4 096 items and below 2 048 voxels the library makes no lists
+    # beyond 4 096 items or 12 voxel blocks and below 2 048 voxels the library makes no lists
     L = nat.lib()
     assert L.fgx_wgrad_item_lists_count(nat.sz(2047), C.c_int(27), C.c_int(256), C.c_int(256), C.c_int(128), C.c_int(128), C.c_int(1024)) == 0
+    assert L.fgx_wgrad_item_lists_count(nat.sz(13 * 1024), C.c_int(27), C.c_int(32), C.c_int(32), C.c_int(32), C.c_int(32), C.c_int(1024)) == 0
+    assert L.fgx_wgrad_item_lists_count(nat.sz(12 * 1024), C.c_int(27), C.c_int(32), C.c_int(32), C.c_int(32), C.c_int(32), C.c_int(1024)) == 4 + 256 + 27 * 12
     assert L.fgx_wgrad_item_lists_count(nat.sz(2048), C.c_int(27), C.c_int(256), C.c_int(256), C.c_int(128), C.c_int(128), C.c_int(1024)) == 4 + 256 + 27 * 4 * 2
     assert L.fgx_wgrad_item_lists_count(nat.sz(1 << 20), C.c_int(27), C.c_int(256), C.c_int(256), C.c_int(128), C.c_int(128), C.c_int(4096)) == 0
 
