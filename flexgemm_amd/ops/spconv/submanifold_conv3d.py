@@ -164,16 +164,20 @@ class SubMConv3dNeighborCache:
         """uint32 device tensor for fgx_conv_gather_gemm_stream's item_at (or None): the tiles dealt to the persistent
         workgroups by cost, built on the device (no read-back) once per plan and shape and kept with the cache."""
         mode = spconv.GEMM_ITEM_ORDER
+        nb = code.shape[0]
         if mode == "auto":
             # the locality order of short-row layers lives on neighboring tiles sharing an XCD (dealing them by cost
-            # alone: 0.32 -> 0.42 ms per launch at C = 32); with rows of 512 bytes and more balance wins (-6 % per
-            # launch at C = 256, -8 % at C = 1024); in between (-1 % at C = 128) it does not pay for the ordering
-            # kernel, which takes ~3 us per round of items
-            mode = "balanced" if slabs >= 4 and not plan_key.startswith("_plan_t_") else "default"
-        nb = code.shape[0]
-        # with fewer than four rounds of items there is little to even out (and the round-by-round dealing is not
-        # reliably better than the kernel's own order)
-        if mode == "default" or nb * col_tiles < 4 * groups or groups > 1024:
+            # alone: 0.32 -> 0.42 ms per launch at C = 32); with rows of 512 bytes and more balance wins whatever the
+            # number of tiles (-6 % per launch at C = 256, -8 % at C = 1024); with shorter rows it wins while a workgroup
+            # has few tiles (C = 128, forward: 143 616 voxels 0.120 -> 0.101 ms, 252 392 voxels 0.179 -> 0.155, 577 592
+            # voxels 0.342 -> 0.320; 669 288 voxels, 10 rounds of items, and 1 026 536 voxels, 16 rounds: no change), and the ordering kernel takes
+            # ~3 us per round of items and neighbor cache
+            few_rounds = nb * col_tiles <= ITEM_ORDER_ANY_ROW_MAX_ROUNDS * groups
+            mode = "balanced" if (slabs >= 4 or few_rounds) and not plan_key.startswith("_plan_t_") else "default"
+        # with at most one item per workgroup there is nothing to even out; from there on the dealt order pays (forward at
+        # 64 160 voxels: C = 256, two rounds of items, 0.158 -> 0.141 ms; C = 512, four rounds, 0.550 -> 0.512 ms;
+        # 15 192 voxels C = 1024, two rounds, 0.601 -> 0.568 ms)
+        if mode == "default" or nb * col_tiles <= ITEM_ORDER_MIN_ROUNDS * groups or groups > 1024:
             return None
         if mode != "balanced":
             raise ValueError(f"unknown GEMM_ITEM_ORDER {spconv.GEMM_ITEM_ORDER!r}; expected 'auto', 'balanced' or 'default'")
@@ -613,6 +617,11 @@ def _sweep_fits(n: int, n_in: int, ci: int, co: int, elem_bytes: int, n_pairs: i
 # pacing of the wgrad sweep: sub-blocks a workgroup may run ahead of the slowest one of its XCD, and the looks at the
 # others' progress after which it stops waiting (0 = no pacing, the default: the workgroups of an XCD stay close enough
 # together by themselves, and waiting costs more time than the L2 misses it saves)
+# The gather GEMM's tiles are dealt by cost when there are more than this many rounds of items (tiles per persistent
+# workgroup).
+ITEM_ORDER_MIN_ROUNDS = 1
+# ... for rows shorter than 512 bytes only up to this many rounds (beyond, the kernel's own order is even enough).
+ITEM_ORDER_ANY_ROW_MAX_ROUNDS = 9
 # The streaming weight gradient walks per-workgroup work lists balanced by pair count (fgx_wgrad_item_lists) where the
 # library has them for the shape; False = the kernel's fixed interleave.  Same result bit for bit.
 WGRAD_BALANCED_LISTS = True
