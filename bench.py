@@ -85,7 +85,7 @@ def parse():
     p.add_argument("--cpu-rows", type=int, default=0, help="rows in the CPU baseline sample (0 = auto)")
     p.add_argument("--build-only", action="store_true", help="time only the neighbor-cache build")
     p.add_argument("--no-others", action="store_true", help="skip the other configurations that follow the headline one")
-    p.add_argument("--other-steps", type=int, default=10, help="timed steps of each of the other configurations")
+    p.add_argument("--other-steps", type=int, default=30, help="timed steps of each of the other configurations (after 5 warm-up steps)")
     p.add_argument("--calibrate-copy", action="store_true",
                    help="also run a plain 1 GiB device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     return p.parse_args()
@@ -383,7 +383,7 @@ def main():
         others = []
         for wname, dn in (("cfg2", None), ("cfg4", None), ("cfg5", None), ("cfg5", "f32")):
             try:
-                r, _, _, _ = measure(wname, dn, args.other_steps, 3, False, time_hash_builder=(wname == "cfg4"))
+                r, _, _, _ = measure(wname, dn, args.other_steps, 5, False, time_hash_builder=(wname == "cfg4"))
             except Exception as exc:       # the headline line must come out whatever happens to a side measurement
                 others.append({"workload": wname, "dtype": dn, "error": f"{type(exc).__name__}: {exc}"})
                 torch.cuda.empty_cache()
