@@ -549,6 +549,11 @@ int fgx_locality_order(const int32_t* coords, const int32_t* binary, size_t n, i
     FGX_CHECK_LAUNCH("fgx_locality_order(keys)");
     size_t temp_bytes = L.temp_bytes;
     FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp_bytes, keys_a, keys_b, vals_a, vals_b, n, 0u, 64u, s));
+    if (chunk_rows == 1) {              // chunks of one rank: the curve's own order, nothing to sort inside them
+        widen_u32_i64_kernel<<<grid, kBlock, 0, s>>>(vals_b, order, n);
+        FGX_CHECK_LAUNCH("fgx_locality_order(widen)");
+        return FGX_OK;
+    }
     chunk_code_key_kernel<<<grid, kBlock, 0, s>>>(vals_b, binary, n, (uint32_t)chunk_rows, keys_a);
     FGX_CHECK_LAUNCH("fgx_locality_order(chunk keys)");
     const unsigned end_bit = 32u + (unsigned)bits_for((n - 1) / (size_t)chunk_rows);

@@ -230,6 +230,29 @@ class SubMConv3dNeighborCache:
         self["_tile_order"] = _locality_order(self["_coords"], self["_binary_code"], self["neighbor_map"].shape[1])
 
 
+    def _narrow_plan(self):
+        """Plan of the resident-row gather GEMM for narrow layers (fgx_narrow_plan): chunks of 128 rows along a Z-order
+        curve of the coordinates, per chunk the distinct source rows and the LDS slot of every (row, offset).  Needs the
+        coordinates the cache was built from; made once and kept (it depends on the map and the coordinates alone)."""
+        if not hasattr(self, "_narrow_plan_buf"):
+            nmap = self["neighbor_map"]
+            n, v = nmap.shape
+            dev = nmap.device
+            if not hasattr(self, "_binary_code"):
+                _, binary, _ = _codes_and_order(nmap, None, None)
+                self["_binary_code"] = binary
+            L = nat.lib()
+            with torch.cuda.device(dev):
+                order = torch.empty((n,), dtype=torch.int64, device=dev)
+                ws = nat.workspace(L.fgx_locality_workspace_bytes(nat.sz(n)), dev)
+                # chunks of one rank: the plain Z-order of the rows
+                nat.check(L.fgx_locality_order(nat.ptr(self["_coords"]), nat.ptr(self["_binary_code"]), nat.sz(n), C.c_int(v),
+                                               C.c_int(1), nat.ptr(order), nat.ptr(ws), nat.sz(ws.numel()), nat.stream()))
+                plan = torch.empty((int(L.fgx_narrow_plan_bytes(nat.sz(n), C.c_int(v))),), dtype=torch.uint8, device=dev)
+                nat.check(L.fgx_narrow_plan(nat.ptr(nmap), nat.ptr(order), nat.sz(n), C.c_int(v), C.c_int(1), nat.ptr(plan), nat.stream()))
+            self["_narrow_plan_buf"] = plan
+        return self["_narrow_plan_buf"]
+
     def _ensure_sorted(self):
         """gray_code / sorted_idx for a cache that only carries `neighbor_map`."""
         if hasattr(self, "gray_code") and hasattr(self, "sorted_idx"):
@@ -558,6 +581,15 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
         relu_mask_out.append(mask)
     with torch.cuda.device(dev):
         panel = _weight_panel(weight_owner, weight_cvk, code, mode, sched, dev)
+        if _narrow_applies(cache, src, k, cols, v, n, n_src, sched):
+            plan = cache._narrow_plan()
+            nat.mark(name, "start")
+            nat.check(L.fgx_conv_narrow_gemm(
+                C.c_int(code), nat.ptr(src), nat.ptr(panel), nat.ptr(bias), nat.ptr(cache["neighbor_map"]), nat.ptr(plan),
+                nat.sz(n), nat.sz(n_src), C.c_int(k), C.c_int(cols), C.c_int(v), C.c_int(activation), nat.ptr(out), nat.ptr(mask),
+                nat.stream()))
+            nat.mark(name, "stop")
+            return out
         if sched.stream and _stream_fits(n, n_src, k * src.element_size()):
             order, tile_code, plan_seg, plan_idx, plan_band, plan_key = cache._gather_plan(sched.tile_rows, private,
                                                                                            dense=not masked)
@@ -601,6 +633,33 @@ def _relu_mask_apply(grad_output: torch.Tensor, mask: torch.Tensor) -> torch.Ten
     return out
 
 
+def _narrow_applies(cache, src: torch.Tensor, k: int, cols: int, v: int, n: int, n_src: int, sched) -> bool:
+    """Whether the resident-row kernel for narrow layers runs this gather GEMM (spconv.NARROW_RESIDENT): 16-bit rows of
+    8 ... 32 channels on both sides, a panel of one 64-byte slab and 32 columns (what the schedule table picks for such
+    layers), enough rows, coordinates to order the rows by, operands within its 32-bit offsets."""
+    mode = spconv.NARROW_RESIDENT
+    if mode == "off":
+        return False
+    if mode not in ("auto", "on"):
+        raise ValueError(f"unknown NARROW_RESIDENT {mode!r}; expected 'auto', 'on' or 'off'")
+    fits = (src.element_size() == 2 and 8 <= k <= 32 and k % 8 == 0 and 8 <= cols <= 32 and cols % 8 == 0 and v <= 27
+            and int(sched.slab_bytes) == 64 and int(sched.tile_cols) == 32
+            and getattr(cache, "_coords", None) is not None and cache._coords.shape[0] == n and n_src == n
+            and n_src * k * 2 < 0xFF000000 and n * 80 + 10240 < 0xFF000000)
+    if not fits:
+        return False
+    if mode == "on" or hasattr(cache, "_narrow_plan_buf"):
+        return True
+    # "auto": the plan costs about as much as a neighbor-cache build (1.2 ms for 2.7 M voxels) and a call gains 0.1 ms on
+    # it, so a cache gets one once it has served NARROW_RESIDENT_AFTER_CALLS narrow products on the streaming kernel:
+    # whatever happens next, the detour then costs at most what the calls before it did.
+    if n < NARROW_RESIDENT_MIN_ROWS:
+        return False
+    calls = getattr(cache, "_narrow_calls", 0) + 1
+    cache["_narrow_calls"] = calls
+    return calls > NARROW_RESIDENT_AFTER_CALLS
+
+
 def _stream_fits(n: int, n_src: int, row_bytes: int) -> bool:
     """The streaming kernel addresses its operands with 32-bit byte offsets."""
     return n_src * row_bytes <= 0xFF000000 and n * 8 <= 0xFF000000 and n * 27 * 4 * 2 <= 0xFF000000
@@ -617,6 +676,10 @@ def _sweep_fits(n: int, n_in: int, ci: int, co: int, elem_bytes: int, n_pairs: i
 # pacing of the wgrad sweep: sub-blocks a workgroup may run ahead of the slowest one of its XCD, and the looks at the
 # others' progress after which it stops waiting (0 = no pacing, the default: the workgroups of an XCD stay close enough
 # together by themselves, and waiting costs more time than the L2 misses it saves)
+# Fewest rows from which NARROW_RESIDENT = "auto" takes the resident-row kernel.
+NARROW_RESIDENT_MIN_ROWS = 32768
+# ... and narrow products a neighbor cache serves on the streaming kernel before it gets the plan.
+NARROW_RESIDENT_AFTER_CALLS = 8
 # The gather GEMM's tiles are dealt by cost when there are more than this many rounds of items (tiles per persistent
 # workgroup).
 ITEM_ORDER_MIN_ROUNDS = 1

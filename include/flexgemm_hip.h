@@ -293,6 +293,26 @@ int fgx_conv_gather_gemm_stream_act_mask(int dtype, const void* src, const void*
                                          int max_groups, int activation, void* out, uint8_t* relu_mask, fgx_stream_t stream);
 int fgx_conv_gather_gemm_stream_groups(int dtype, int cols, int tile_rows, int tile_cols, int slab_bytes, int* groups);
 
+/* Gather GEMM for narrow layers with the gathered rows resident in LDS: 16-bit types, K and cols of 8, 16, 24 or 32
+ * channels (rows of at most 64 bytes), `panel` from fgx_pack_weight with slab_bytes = 64 and col_pad = 32.  Rows walk in
+ * chunks of 128 along `order` (any permutation; a Z-order curve of the coordinates -- fgx_locality_order with
+ * chunk_rows = 1 -- makes a chunk's rows neighbors in space); fgx_narrow_plan names, once per neighbor map and order, every
+ * chunk's distinct source rows (about 1.7 per output row on a surface, where the streaming kernel requests 10.5) and the
+ * LDS slot of the source of every (row, offset).  Per chunk the kernel loads those rows once and multiplies all V offsets
+ * for all rows (a missing neighbor is a row of zeros): same function as fgx_conv_gather_gemm_stream, sums in offset
+ * order.  A chunk with more than 384 distinct sources (rows ordered without locality) stays correct: the surplus is read
+ * from memory through `map`.  same_rows = 1 when output row i and source row i are the same voxel (submanifold layers,
+ * forward and dgrad): every chunk row then sits in the LDS slot of its own number, which keeps the multipliers' reads of
+ * neighboring rows on different banks.  activation / relu_mask as in fgx_conv_gather_gemm_act_mask.
+ * plan: fgx_narrow_plan_bytes(n, V) bytes, 16-byte aligned.
+ * No counterpart in the reference, whose kernels gather every row per (tile, offset) from memory
+ * (..._fwd_masked_implicit_gemm.py:20-100). */
+size_t fgx_narrow_plan_bytes(size_t n, int V);
+int fgx_narrow_plan(const uint32_t* map, const int64_t* order, size_t n, int V, int same_rows, void* plan, fgx_stream_t stream);
+int fgx_conv_narrow_gemm(int dtype, const void* src, const void* panel, const void* bias, const uint32_t* map, const void* plan,
+                         size_t n, size_t n_src, int K, int cols, int V, int activation, void* out, uint8_t* relu_mask,
+                         fgx_stream_t stream);
+
 /* item_at for fgx_conv_gather_gemm_stream, made on the device from the tile codes: items sorted by cost (offsets per
  * row tile x `slabs` K-slabs + an epilogue), the incomplete last round of `groups` positions filled with the cheapest,
  * every full round dealt most-expensive-item to least-loaded-slot.  One workgroup, deterministic, no read-back;

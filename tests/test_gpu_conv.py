@@ -85,6 +85,74 @@ def test_conv_matches_oracle(gpu_device, dtype, res, ci, co):
     _run_and_check(coords_np, torch.Size([1, ci, res, res, res]), ci, co, dtype, gpu_device, seed=res + ci)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("res,ci,co", [(32, 32, 32), (40, 24, 16), (48, 8, 32), (24, 32, 8), (20, 16, 24)])
+def test_narrow_resident_gemm_matches_oracle(gpu_device, dtype, res, ci, co):
+    """Forward and dgrad of narrow layers through the resident-row kernel (fgx_conv_narrow_gemm, forced on): rows of 16 to
+    64 bytes on either side, a last chunk that is partly empty, against the float64 oracle; wgrad and dbias ride along on
+    their usual kernels."""
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    _say(f"narrow resident res={res} ci={ci} co={co} {dtype}")
+    coords_np = reference_test_shell(res)
+    old = impl.spconv.NARROW_RESIDENT
+    impl.spconv.NARROW_RESIDENT = "on"
+    try:
+        cache, _ = _run_and_check(coords_np, torch.Size([1, ci, res, res, res]), ci, co, dtype, gpu_device, seed=res + ci)
+    finally:
+        impl.spconv.NARROW_RESIDENT = old
+    assert hasattr(cache, "_narrow_plan_buf"), "the resident-row kernel did not run"
+
+
+def test_narrow_resident_gemm_relu_mask_and_overflowing_chunks(gpu_device):
+    """The resident-row kernel with the fused ReLU and its bit mask; and with rows in a random order, where a chunk of 128
+    rows has far more than 384 distinct sources, so that most sources are read from memory by the multipliers: the sums
+    run over the same offsets in the same order, so the result is the same bit for bit as with the rows in Z-order."""
+    import ctypes as C
+    from flexgemm_amd import _native as nat
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    _say("narrow resident relu mask / overflow")
+    res, c = 48, 32
+    coords_np = reference_test_shell(res)
+    n = coords_np.shape[0]
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    shape = torch.Size([1, c, res, res, res])
+    f, w, b, _ = _case(coords_np, c, c, torch.float16, 53)
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), False)
+    fd, wd, bd = f.to(gpu_device), w.to(gpu_device).reshape(c, 27, c), b.to(gpu_device)
+    old = impl.spconv.NARROW_RESIDENT
+    impl.spconv.NARROW_RESIDENT = "on"
+    try:
+        masks = []
+        out = impl._gather_gemm(fd, wd, bd, cache, 0, False, activation=nat.ACT_RELU, relu_mask_out=masks)
+    finally:
+        impl.spconv.NARROW_RESIDENT = old
+    assert hasattr(cache, "_narrow_plan_buf") and len(masks) == 1
+    ref = torch.relu(eg.forward(f.double(), cache.neighbor_map.cpu().view(torch.int32), w.double(), b.double()))
+    assert eg.max_rel_err(out.cpu(), ref) <= 1e-2
+    bits = np.unpackbits(masks[0].cpu().numpy(), bitorder="little").reshape(n, c).astype(bool)
+    assert np.array_equal(bits, (out.cpu().float() > 0).numpy()), "the mask is not 'output greater than zero'"
+    # rows in a random order: chunks whose sources do not fit the slots
+    L = nat.lib()
+    order = torch.from_numpy(np.random.default_rng(5).permutation(n).astype(np.int64)).to(gpu_device)
+    nmap = cache["neighbor_map"]
+    plan = torch.empty((int(L.fgx_narrow_plan_bytes(nat.sz(n), C.c_int(27))),), dtype=torch.uint8, device=gpu_device)
+    sched = nat.table_lookup(nat.PASS_FWD, torch.float16, n, c, c, 27)
+    outs = []
+    with torch.cuda.device(gpu_device):
+        panel = impl._weight_panel(None, wd.contiguous(), nat.DTYPE_CODE[torch.float16], 0, sched, gpu_device)
+        for same_rows in (1, 0):
+            nat.check(L.fgx_narrow_plan(nat.ptr(nmap), nat.ptr(order), nat.sz(n), C.c_int(27), C.c_int(same_rows), nat.ptr(plan), nat.stream()))
+            o = torch.empty((n, c), dtype=torch.float16, device=gpu_device)
+            nat.check(L.fgx_conv_narrow_gemm(C.c_int(nat.DTYPE_CODE[torch.float16]), nat.ptr(fd), nat.ptr(panel), nat.ptr(bd), nat.ptr(nmap),
+                                             nat.ptr(plan), nat.sz(n), nat.sz(n), C.c_int(c), C.c_int(c), C.c_int(27), C.c_int(nat.ACT_RELU),
+                                             nat.ptr(o), nat.ptr(None), nat.stream()))
+            outs.append(o.cpu())
+            chunks = -(-n // 128)
+            table = plan.cpu().numpy().reshape(chunks, 8192 + 1536 + 512)[:, :8192].copy().view(np.uint16).reshape(chunks, 128, 32)
+            assert (table[:, :, 31] != 0).any(), "no chunk overflowed: the test does not reach the path it is for"
+    assert torch.equal(outs[0], out.cpu()) and torch.equal(outs[1], out.cpu())
+
+
 @pytest.mark.parametrize("res", [1, 2, 4])
 def test_degenerate_sizes(gpu_device, res):
     # fewer voxels than one tile; N = 1 at res 1
