@@ -10,19 +10,13 @@
 // all rows -- a missing neighbor is the slot of zeros -- because with K = 32 a product is two MFMAs and skipping would
 // cost more instructions than it saves.  The weight (V x 2 KiB) stays in LDS for the whole launch.
 //
-//   plan, per chunk (kNarrowRows output rows), kPlanStride(V) bytes:
-//     table    uint16 [kNarrowRows][32]   byte offset, in the LDS row buffer, of the source row's first 16-byte piece (its
-//                                         pieces are exchanged, below); the row of zeros when the neighbor is missing;
-//                                         kOverflow when the chunk has more distinct sources than slots (the multiplier
-//                                         then reads that row from memory; rare, any input stays correct); entry 31: whether
-//                                         any entry of the row is kOverflow
-//     sources  uint32 [kNarrowSlots]      source row of every slot, FGX_EMPTY32 beyond the chunk's count
-//     rows     uint32 [kNarrowRows]       output row of every chunk row (the row order), FGX_EMPTY32 beyond n
+// (the plan's layout: narrow_plan.h)
 //
-// Workgroup: 4 multiplying wavefronts (32 chunk rows each, one 32 x 32 accumulator) + 4 loading wavefronts; three LDS
-// buffers (the loads run two chunks ahead), one barrier per chunk.  Persistent: XCD x walks the x-th eighth of the chunks, its workgroups interleave, so
+// Workgroup: 4 multiplying wavefronts (32 chunk rows each, one 32 x 32 accumulator) + 4 loading wavefronts; two LDS
+// buffers (the loads run one chunk ahead), one barrier per chunk.  Persistent: XCD x walks the x-th eighth of the chunks, its workgroups interleave, so
 // that neighboring chunks -- which share their halo rows -- run on one L2 at one time.
 #include "gemm_device.h"
+#include "narrow_plan.h"
 
 namespace fgx {
 namespace {
@@ -33,23 +27,14 @@ __device__ __forceinline__ rsrc_t narrow_rsrc(const void* p, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), (short)0, (int)bytes, 0x00020000);
 }
 
-constexpr int kNarrowRows = 128;                 // output rows per chunk
-constexpr int kNarrowSlots = 384;                // source rows resident per chunk (a multiple of 64)
-constexpr uint32_t kZeroSlot = kNarrowSlots;     // one more slot, all zeros
-constexpr uint32_t kOverflow = 0xFFFFu;
-constexpr uint32_t kNarrowOob = 0xFF000000u;     // buffer offset no tensor reaches: the load returns zeros
 constexpr int kNarrowHash = 1024;                // hash table of the plan builder (a power of two)
-constexpr int kNarrowMaxV = 31;                  // (table entry 31 of a row is its overflow flag)
-
-constexpr int kTableStride = 32;                 // table entries per row (V <= 32): a row's entries are four 16-byte reads
-__host__ __device__ constexpr int narrow_table_bytes(int) { return kNarrowRows * kTableStride * 2; }
-__host__ __device__ constexpr int narrow_table_lds(int V) { return narrow_table_bytes(V); }                 // a multiple of 1024
-__host__ __device__ constexpr int narrow_plan_stride(int V) { return narrow_table_bytes(V) + kNarrowSlots * 4 + kNarrowRows * 4; }
 
 // ------------------------------------------------------------------------------------------------
 // Plan builder: one workgroup per chunk.  The distinct neighbors of the chunk's rows go through a hash table in LDS;
 // slots are numbered in table order, so the plan depends on the chunk's set of sources alone.
 // ------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(64) narrow_plan_header_kernel(uint32_t* __restrict__ header) { header[threadIdx.x] = 0u; }
+
 __global__ void __launch_bounds__(256) narrow_plan_kernel(const uint32_t* __restrict__ nmap, const int64_t* __restrict__ order,
                                                           uint32_t n, int V, int own_rows, unsigned char* __restrict__ plan) {
     __shared__ uint32_t keys[kNarrowHash];
@@ -58,9 +43,9 @@ __global__ void __launch_bounds__(256) narrow_plan_kernel(const uint32_t* __rest
     __shared__ uint32_t row_flags[kNarrowRows / 32];
     const int tid = threadIdx.x;
     const uint32_t chunk = blockIdx.x;
-    unsigned char* mine = plan + (size_t)chunk * narrow_plan_stride(V);
+    unsigned char* mine = plan + kNarrowHeader + (size_t)chunk * kNarrowPlanStride;
     uint16_t* table = (uint16_t*)mine;
-    uint32_t* sources = (uint32_t*)(mine + narrow_table_bytes(V));
+    uint32_t* sources = (uint32_t*)(mine + kNarrowTableBytes);
     uint32_t* rows = sources + kNarrowSlots;
     for (int i = tid; i < kNarrowHash; i += 256) keys[i] = FGX_EMPTY32;
     if (tid < kNarrowRows / 32) row_flags[tid] = 0u;
@@ -86,7 +71,7 @@ __global__ void __launch_bounds__(256) narrow_plan_kernel(const uint32_t* __rest
     // the slot of its chunk row number: the 16 rows of a fragment read then fall on 16 different slots modulo 16 for
     // the centre offset and on nearly as many for the others -- the neighbors of consecutive rows are mostly
     // consecutive rows -- which is what keeps the reads of arbitrary slots off each other's banks.
-    for (int i = tid; i < kNarrowHash; i += 256) slot_of[i] = (uint16_t)kOverflow;
+    for (int i = tid; i < kNarrowHash; i += 256) slot_of[i] = (uint16_t)kNarrowOverflow;
     __syncthreads();
     if (own_rows) {
         for (int r = tid; r < kNarrowRows; r += 256) {
@@ -112,7 +97,7 @@ __global__ void __launch_bounds__(256) narrow_plan_kernel(const uint32_t* __rest
         }
     }
     uint32_t own = 0;
-    for (int j = 0; j < 4; ++j) own += (keys[tid * 4 + j] != FGX_EMPTY32 && slot_of[tid * 4 + j] == kOverflow) ? 1u : 0u;
+    for (int j = 0; j < 4; ++j) own += (keys[tid * 4 + j] != FGX_EMPTY32 && slot_of[tid * 4 + j] == kNarrowOverflow) ? 1u : 0u;
     scan[tid] = own;
     __syncthreads();
     for (int d = 1; d < 256; d <<= 1) {
@@ -124,7 +109,7 @@ __global__ void __launch_bounds__(256) narrow_plan_kernel(const uint32_t* __rest
     uint32_t next = base + scan[tid] - own;
     for (int j = 0; j < 4; ++j) {
         const int pos = tid * 4 + j;
-        if (keys[pos] != FGX_EMPTY32 && slot_of[pos] == kOverflow) {
+        if (keys[pos] != FGX_EMPTY32 && slot_of[pos] == kNarrowOverflow) {
             if (next < (uint32_t)kNarrowSlots) {
                 slot_of[pos] = (uint16_t)next;
                 sources[next] = keys[pos];
@@ -137,9 +122,9 @@ __global__ void __launch_bounds__(256) narrow_plan_kernel(const uint32_t* __rest
     __syncthreads();
     for (int e = tid; e < entries; e += 256) {
         const uint32_t idx = source_of(e);
-        uint16_t out = (uint16_t)kZeroSlot;
+        uint16_t out = (uint16_t)kNarrowZeroSlot;
         if (idx != FGX_EMPTY32) {
-            out = (uint16_t)kOverflow;
+            out = (uint16_t)kNarrowOverflow;
             uint32_t h = hash(idx);
             for (int probe = 0; probe < kNarrowHash; ++probe) {
                 const uint32_t k = keys[h];
@@ -149,12 +134,16 @@ __global__ void __launch_bounds__(256) narrow_plan_kernel(const uint32_t* __rest
             }
         }
         // what the multipliers read: the byte offset of the row's logical piece 0 in the row buffer
-        if (out != (uint16_t)kOverflow) out = (uint16_t)(out * 64u + (((uint32_t)out >> 2) & 3u) * 16u);
-        table[(e / V) * kTableStride + (e % V)] = out;
-        if (out == (uint16_t)kOverflow) atomicOr(&row_flags[(e / V) >> 5], 1u << ((e / V) & 31));
+        if (out != (uint16_t)kNarrowOverflow) out = (uint16_t)(out * 64u + (((uint32_t)out >> 2) & 3u) * 16u);
+        table[(e / V) * kNarrowTableStride + (e % V)] = out;
+        if (out == (uint16_t)kNarrowOverflow) atomicOr(&row_flags[(e / V) >> 5], 1u << ((e / V) & 31));
     }
     __syncthreads();
-    for (int r = tid; r < kNarrowRows; r += 256) table[r * kTableStride + kTableStride - 1] = (uint16_t)((row_flags[r >> 5] >> (r & 31)) & 1u);
+    for (int r = tid; r < kNarrowRows; r += 256) {
+        table[r * kNarrowTableStride + kNarrowTableStride - 1] = (uint16_t)((row_flags[r >> 5] >> (r & 31)) & 1u);
+        for (int v = V; v < kNarrowTableStride - 1; ++v) table[r * kNarrowTableStride + v] = (uint16_t)(kNarrowZeroSlot * 64u);
+    }
+    if (tid == 0 && (row_flags[0] | row_flags[1] | row_flags[2] | row_flags[3]) != 0u) atomicAdd((uint32_t*)plan, 1u);
     for (int r = tid; r < kNarrowRows; r += 256) {
         const uint32_t g = chunk * kNarrowRows + (uint32_t)r;
         rows[r] = g < n ? (order ? (uint32_t)order[g] : g) : FGX_EMPTY32;
@@ -167,11 +156,10 @@ __global__ void __launch_bounds__(256) narrow_plan_kernel(const uint32_t* __rest
 // (slot >> 2) & 3, so that the 32 lanes of a fragment read, which fall on arbitrary slots, spread over the banks.
 // ------------------------------------------------------------------------------------------------
 constexpr int kNarrowMult = 4, kNarrowLoad = 4, kNarrowThreads = 64 * (kNarrowMult + kNarrowLoad);
-constexpr int kNarrowBuffers = 3;                              // chunks in LDS: one multiplied, two on their way
-constexpr int kRowBufBytes = (kNarrowSlots + 1) * 64;          // + the slot of zeros
-constexpr int kRowBufPad = (kRowBufBytes + 1023) / 1024 * 1024;
+constexpr int kNarrowBuffers = 2;                              // chunks in LDS: one multiplied, one on its way (a third, two
+                                                               // chunks ahead, measured the same)
 
-__host__ __device__ constexpr int narrow_buffer_bytes(int V) { return kRowBufPad + narrow_table_lds(V) + 1024; }
+__host__ __device__ constexpr int narrow_buffer_bytes(int V) { return kNarrowRowBufPad + kNarrowTableBytes + 1024; }
 __host__ __device__ constexpr size_t narrow_lds_bytes(int V) {
     return (size_t)V * 2048 + (size_t)kNarrowBuffers * narrow_buffer_bytes(V);
 }
@@ -209,7 +197,7 @@ narrow_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const bool loader = wave >= kNarrowMult;
     const int row_bytes = K * 2, out_row_bytes = cols * 2;
-    const int stride = narrow_plan_stride(V), table_bytes = narrow_table_bytes(V);
+    const int stride = kNarrowPlanStride, table_bytes = kNarrowTableBytes;
 
     // ---- chunks of this workgroup: XCD x owns the x-th eighth, its workgroups interleave ----
     const unsigned G = gridDim.x;
@@ -243,7 +231,7 @@ narrow_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
 #pragma unroll
         for (int j = 0; j < kGroups; ++j) {
             const uint32_t s = (uint32_t)((j * kNarrowLoad + lw) * 16 + (lane >> 2));
-            ids[j] = __builtin_amdgcn_raw_buffer_load_b32(plan_rs, chunk * (uint32_t)stride + (uint32_t)table_bytes + s * 4u, 0, 0);
+            ids[j] = __builtin_amdgcn_raw_buffer_load_b32(plan_rs, (uint32_t)kNarrowHeader + chunk * (uint32_t)stride + (uint32_t)table_bytes + s * 4u, 0, 0);
         }
     };
     auto enqueue = [&](unsigned chunk, int b) {
@@ -257,15 +245,15 @@ narrow_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
             const uint32_t vo = live ? ids[j] * (uint32_t)row_bytes + piece * 16u : kNarrowOob;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(src_rs, FGX_LDS_PTR(buf + group * 1024), 16, vo, 0, 0, 0);
         }
-        const int table_insts = narrow_table_lds(V) / 1024;
+        const int table_insts = kNarrowTableBytes / 1024;
         for (int j = lw; j < table_insts; j += kNarrowLoad)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(plan_rs, FGX_LDS_PTR(buf + kRowBufPad + j * 1024), 16,
-                                                     chunk * (uint32_t)stride + (uint32_t)(j * 1024 + lane * 16), 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(plan_rs, FGX_LDS_PTR(buf + kNarrowRowBufPad + j * 1024), 16,
+                                                     (uint32_t)kNarrowHeader + chunk * (uint32_t)stride + (uint32_t)(j * 1024 + lane * 16), 0, 0, 0);
         if (lw == kNarrowLoad - 1) {
             const uint32_t vo = lane < kNarrowRows * 4 / 16
-                                    ? chunk * (uint32_t)stride + (uint32_t)table_bytes + kNarrowSlots * 4u + (uint32_t)lane * 16u
+                                    ? (uint32_t)kNarrowHeader + chunk * (uint32_t)stride + (uint32_t)table_bytes + kNarrowSlots * 4u + (uint32_t)lane * 16u
                                     : kNarrowOob;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(plan_rs, FGX_LDS_PTR(buf + kRowBufPad + narrow_table_lds(V)), 16, vo, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(plan_rs, FGX_LDS_PTR(buf + kNarrowRowBufPad + kNarrowTableBytes), 16, vo, 0, 0, 0);
         }
     };
 
@@ -279,39 +267,32 @@ narrow_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
         bias_e[e] = (bias != nullptr && col < cols) ? to_float<T>(bias[col]) : 0.f;
     }
 
-    // Two chunks ahead: in the iteration that multiplies chunk i the loaders enqueue chunk i + 2 (its source rows are in
-    // registers since the iteration before) and fetch the source rows of chunk i + 3; at the end of the iteration they
-    // wait until chunk i + 1 has landed -- everything but what this iteration issued (loads return in order).
-    constexpr int kEnqueued = kGroups + kNarrowRows * kTableStride * 2 / 1024 / kNarrowLoad;    // + 1 in the last loader
+    // One chunk ahead: in the iteration that multiplies chunk i the loaders enqueue chunk i + 1 (its source rows are in
+    // registers since the iteration before) and fetch the source rows of chunk i + 2; at the end of the iteration they
+    // wait until chunk i + 1 has landed -- everything but the fetch, which was issued last (loads return in order).
     if (loader) {
         fetch_ids(first);
         enqueue(first, 0);
-        if (first + per_round < range_hi) {
-            fetch_ids(first + per_round);
-            enqueue(first + per_round, 1);
-            if (first + 2 * per_round < range_hi) fetch_ids(first + 2 * per_round);
-        }
+        if (first + per_round < range_hi) fetch_ids(first + per_round);
     }
     __builtin_amdgcn_s_waitcnt(0);                                              // the weight and zero stores, the first loads
     __syncthreads();
 
     int b = 0;
-    for (unsigned chunk = first; chunk < range_hi; chunk += per_round, b = b == kNarrowBuffers - 1 ? 0 : b + 1) {
+    for (unsigned chunk = first; chunk < range_hi; chunk += per_round, b ^= 1) {
         if (loader) {
-            const unsigned ahead = chunk + 2 * per_round;
-            const bool enqueues = ahead < range_hi, fetches = ahead + per_round < range_hi;
+            const unsigned next = chunk + per_round;
+            const bool enqueues = next < range_hi, fetches = next + per_round < range_hi;
             if (enqueues) {
-                enqueue(ahead, b >= 1 ? b - 1 : b + 2);                          // (b + 2) mod 3; its ids are in registers
-                if (fetches) fetch_ids(ahead + per_round);
+                enqueue(next, b ^ 1);
+                if (fetches) fetch_ids(next + per_round);
             }
-            const bool last = lw == kNarrowLoad - 1;
-            if (!enqueues) wait_vmcnt<0>();
-            else if (!fetches) { if (last) wait_vmcnt<kEnqueued + 1>(); else wait_vmcnt<kEnqueued>(); }
-            else { if (last) wait_vmcnt<kEnqueued + 1 + kGroups>(); else wait_vmcnt<kEnqueued + kGroups>(); }
+            if (fetches) wait_vmcnt<kGroups>();
+            else wait_vmcnt<0>();
         } else {
             const unsigned char* buf = buffers + (size_t)b * buffer_bytes;
-            const uint16_t* table = (const uint16_t*)(buf + kRowBufPad);
-            const uint32_t* out_rows = (const uint32_t*)(buf + kRowBufPad + narrow_table_lds(V));
+            const uint16_t* table = (const uint16_t*)(buf + kNarrowRowBufPad);
+            const uint32_t* out_rows = (const uint32_t*)(buf + kNarrowRowBufPad + kNarrowTableBytes);
             const int r = mw * 32 + l32;
             // Products are taken as (weight fragment) x (row fragment): the accumulator then holds, per lane, ONE chunk row
             // (r) and sixteen output columns in four runs of four -- 8 bytes each, stored straight from the registers.
@@ -319,10 +300,10 @@ narrow_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
             f32x16 acc, acc1;
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[e] = acc1[e] = 0.f;
-            // this row's table entries: 32 x uint16 in four 16-byte reads; entry 31 says whether any of them is kOverflow
+            // this row's table entries: 32 x uint16 in four 16-byte reads; entry 31 says whether any of them is kNarrowOverflow
             u32x4 ent[4];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) ent[q] = *reinterpret_cast<const u32x4*>((const unsigned char*)table + r * (kTableStride * 2) + q * 16);
+            for (int q = 0; q < 4; ++q) ent[q] = *reinterpret_cast<const u32x4*>((const unsigned char*)table + r * (kNarrowTableStride * 2) + q * 16);
             auto entry = [&](int v) -> uint32_t {
                 const uint32_t word = ent[v >> 3][(v >> 1) & 3];
                 return (v & 1) ? word >> 16 : word & 0xFFFFu;
@@ -332,14 +313,14 @@ narrow_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
             const unsigned char* wrow0 = weight_lds + l32 * 64 + (((uint32_t)g ^ wkey) << 4);
             const unsigned char* wrow1 = weight_lds + l32 * 64 + (((uint32_t)(g + 2) ^ wkey) << 4);
             // (a table entry is the byte offset of a row's logical piece 0; piece q sits at entry ^ (q << 4))
-            if (__builtin_expect(__any(entry(kTableStride - 1) != 0u), 0)) {
+            if (__builtin_expect(__any(entry(kNarrowTableStride - 1) != 0u), 0)) {
                 // a chunk with more distinct sources than slots: lanes whose source is not resident read it from memory
                 for (int v = 0; v < V; ++v) {
-                    const uint32_t s = table[r * kTableStride + v];
-                    const uint32_t off = s == kOverflow ? kZeroSlot * 64u : s;
+                    const uint32_t s = table[r * kNarrowTableStride + v];
+                    const uint32_t off = s == kNarrowOverflow ? kNarrowZeroSlot * 64u : s;
                     u32x4 a0 = *reinterpret_cast<const u32x4*>(buf + (off ^ ((uint32_t)g << 4)));
                     u32x4 a1 = *reinterpret_cast<const u32x4*>(buf + (off ^ ((uint32_t)g << 4) ^ 32u));
-                    if (s == kOverflow && grow != FGX_EMPTY32) {
+                    if (s == kNarrowOverflow && grow != FGX_EMPTY32) {
                         const uint32_t id = nmap[(size_t)grow * V + v];
                         if (id != FGX_EMPTY32) {
                             const u32x4 zero = {0u, 0u, 0u, 0u};
@@ -377,7 +358,7 @@ narrow_gemm_kernel(const typename Tag::type* __restrict__ src, const typename Ta
             } else {
 #pragma unroll 4
                 for (int v = 0; v < V; ++v) {
-                    const uint32_t at = (uint32_t)table[r * kTableStride + v] ^ ((uint32_t)g << 4);
+                    const uint32_t at = (uint32_t)table[r * kNarrowTableStride + v] ^ ((uint32_t)g << 4);
                     const u32x4 a0 = *reinterpret_cast<const u32x4*>(buf + at);
                     const u32x4 a1 = *reinterpret_cast<const u32x4*>(buf + (at ^ 32u));
                     mma<Tag>(acc, *reinterpret_cast<const u32x4*>(wrow0 + v * 2048), a0);
@@ -433,7 +414,7 @@ int launch_narrow(const void* src, const void* panel, const void* bias, const ui
         raised = true;
     }
     kern<<<groups, kNarrowThreads, lds, s>>>((const T*)src, (const T*)panel, (const T*)bias, nmap, (const unsigned char*)plan, chunks,
-                                             (uint32_t)((size_t)chunks * narrow_plan_stride(V)), (uint32_t)(n_src * (size_t)K * 2), V, K,
+                                             (uint32_t)(kNarrowHeader + (size_t)chunks * kNarrowPlanStride), (uint32_t)(n_src * (size_t)K * 2), V, K,
                                              cols, activation, (T*)out, relu_mask);
     FGX_CHECK_LAUNCH("fgx_conv_narrow_gemm");
     return FGX_OK;
@@ -448,7 +429,7 @@ extern "C" {
 
 size_t fgx_narrow_plan_bytes(size_t n, int V) {
     if (V < 1 || V > kNarrowMaxV) return 0;
-    return ((n + kNarrowRows - 1) / kNarrowRows) * (size_t)narrow_plan_stride(V);
+    return kNarrowHeader + ((n + kNarrowRows - 1) / kNarrowRows) * (size_t)kNarrowPlanStride;
 }
 
 int fgx_narrow_plan(const uint32_t* map, const int64_t* order, size_t n, int V, int same_rows, void* plan, fgx_stream_t stream) {
@@ -459,6 +440,8 @@ int fgx_narrow_plan(const uint32_t* map, const int64_t* order, size_t n, int V, 
     FGX_CHECK_ARG(((uintptr_t)plan & 15) == 0, "fgx_narrow_plan: plan must be 16-byte aligned");
     FGX_CHECK_ARG(fgx_narrow_plan_bytes(n, V) < 0xFF000000ull, "fgx_narrow_plan: plan of %zu rows passes the 32-bit offset range", n);
     const unsigned chunks = (unsigned)((n + kNarrowRows - 1) / kNarrowRows);
+    narrow_plan_header_kernel<<<1, 64, 0, (hipStream_t)stream>>>((uint32_t*)plan);
+    FGX_CHECK_LAUNCH("fgx_narrow_plan(header)");
     narrow_plan_kernel<<<chunks, 256, 0, (hipStream_t)stream>>>(map, order, (uint32_t)n, V, same_rows ? 1 : 0, (unsigned char*)plan);
     FGX_CHECK_LAUNCH("fgx_narrow_plan");
     return FGX_OK;

@@ -645,7 +645,7 @@ def _narrow_applies(cache, src: torch.Tensor, k: int, cols: int, v: int, n: int,
     fits = (src.element_size() == 2 and 8 <= k <= 32 and k % 8 == 0 and 8 <= cols <= 32 and cols % 8 == 0 and v <= 27
             and int(sched.slab_bytes) == 64 and int(sched.tile_cols) == 32
             and getattr(cache, "_coords", None) is not None and cache._coords.shape[0] == n and n_src == n
-            and n_src * k * 2 < 0xFF000000 and n * 80 + 10240 < 0xFF000000)
+            and n_src * k * 2 < 0xFF000000 and n * 82 + 10752 < 0xFF000000)
     if not fits:
         return False
     if mode == "on" or hasattr(cache, "_narrow_plan_buf"):
@@ -658,6 +658,23 @@ def _narrow_applies(cache, src: torch.Tensor, k: int, cols: int, v: int, n: int,
     calls = getattr(cache, "_narrow_calls", 0) + 1
     cache["_narrow_calls"] = calls
     return calls > NARROW_RESIDENT_AFTER_CALLS
+
+
+def _narrow_wgrad_applies(cache, f: torch.Tensor, ci: int, co: int, v: int, n: int, n_in: int) -> bool:
+    """Whether the weight gradient runs on the resident-row kernel: a narrow 16-bit layer on a cache that has (mode "on":
+    or can have) the plan, and no chunk of the plan has more distinct sources than slots (the plan's header says so;
+    read back once per plan)."""
+    mode = spconv.NARROW_RESIDENT
+    if mode == "off":
+        return False
+    fits = (f.element_size() == 2 and 8 <= ci <= 32 and ci % 8 == 0 and 8 <= co <= 32 and co % 8 == 0 and v <= 27
+            and getattr(cache, "_coords", None) is not None and cache._coords.shape[0] == n and n_in == n
+            and n * 64 < 0xFF000000 and n * 82 + 10752 < 0xFF000000)
+    if not fits or not (mode == "on" or hasattr(cache, "_narrow_plan_buf")):
+        return False
+    if not hasattr(cache, "_narrow_overflows"):
+        cache["_narrow_overflows"] = int(cache._narrow_plan()[:4].view(torch.int32).item())
+    return cache["_narrow_overflows"] == 0
 
 
 def _stream_fits(n: int, n_src: int, row_bytes: int) -> bool:
@@ -705,6 +722,22 @@ def _wgrad(grad_output: torch.Tensor, feats: torch.Tensor, cache, v: int, with_b
     f = _pad_cols(feats, align).contiguous()
     g = _pad_cols(grad_output, align).contiguous()
     cip, cop = f.shape[1], g.shape[1]
+    if _narrow_wgrad_applies(cache, f, cip, cop, v, n, n_in):
+        # narrow layers on a cache that has the resident-row plan: the chunk's rows gathered in LDS (fgx_conv_narrow_wgrad)
+        L = nat.lib()
+        gw = torch.empty((cop, v, cip), dtype=dt, device=dev)
+        with torch.cuda.device(dev):
+            scratch = nat.workspace(L.fgx_narrow_wgrad_scratch_bytes(C.c_int(v)), dev)
+            nat.mark("wgrad", "start")
+            nat.check(L.fgx_conv_narrow_wgrad(C.c_int(nat.DTYPE_CODE[dt]), nat.ptr(g), nat.ptr(f), nat.ptr(cache._narrow_plan()),
+                                              nat.sz(n), nat.sz(n_in), C.c_int(cip), C.c_int(cop), C.c_int(v), nat.ptr(scratch),
+                                              nat.ptr(gw), nat.stream()))
+            gb = _colsum(g) if with_bias else None
+            nat.mark("wgrad", "stop")
+        if cip != ci or cop != co:
+            gw = gw[:co, :, :ci].contiguous()
+            gb = gb[:co].contiguous() if with_bias else None
+        return (gw, gb) if with_bias else gw
     cache._ensure_pairs()
     seg_host = cache._seg_host()
     if len(seg_host) != v + 1 or seg_host[-1] > min(cache["valid_signal_i"].numel(), cache["valid_signal_o"].numel()):

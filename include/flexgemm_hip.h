@@ -298,9 +298,10 @@ int fgx_conv_gather_gemm_stream_groups(int dtype, int cols, int tile_rows, int t
  * chunks of 128 along `order` (any permutation; a Z-order curve of the coordinates -- fgx_locality_order with
  * chunk_rows = 1 -- makes a chunk's rows neighbors in space); fgx_narrow_plan names, once per neighbor map and order, every
  * chunk's distinct source rows (about 1.7 per output row on a surface, where the streaming kernel requests 10.5) and the
- * LDS slot of the source of every (row, offset).  Per chunk the kernel loads those rows once and multiplies all V offsets
+ * LDS slot of the source of every (row, offset); its first 256 bytes are a header whose first uint32 counts the chunks
+ * with more distinct sources than slots.  Per chunk the kernel loads those rows once and multiplies all V offsets
  * for all rows (a missing neighbor is a row of zeros): same function as fgx_conv_gather_gemm_stream, sums in offset
- * order.  A chunk with more than 384 distinct sources (rows ordered without locality) stays correct: the surplus is read
+ * order.  A chunk with more than 448 distinct sources (rows ordered without locality) stays correct: the surplus is read
  * from memory through `map`.  same_rows = 1 when output row i and source row i are the same voxel (submanifold layers,
  * forward and dgrad): every chunk row then sits in the LDS slot of its own number, which keeps the multipliers' reads of
  * neighboring rows on different banks.  activation / relu_mask as in fgx_conv_gather_gemm_act_mask.
@@ -312,6 +313,20 @@ int fgx_narrow_plan(const uint32_t* map, const int64_t* order, size_t n, int V, 
 int fgx_conv_narrow_gemm(int dtype, const void* src, const void* panel, const void* bias, const uint32_t* map, const void* plan,
                          size_t n, size_t n_src, int K, int cols, int V, int activation, void* out, uint8_t* relu_mask,
                          fgx_stream_t stream);
+
+/* The weight gradient of such a layer on the same plan: grad_weight[co][v][ci] = sum over rows r with a neighbor at offset
+ * v of grad_out[r][co] * feats[source(r, v)][ci], for 16-bit types and Ci, Co of 8, 16, 24 or 32.  Per chunk of 128 rows
+ * the chunk's own grad_out rows and its distinct source rows are loaded into LDS once (the block-major kernel of
+ * fgx_conv_wgrad fetches two rows per pair), the gather happens in the transposing LDS reads.  Every workgroup keeps the
+ * accumulators of all V offsets over its chunks and writes one partial product; a second kernel adds the partial
+ * products in workgroup order (same bits on every run; against fgx_conv_wgrad the sums differ by fp32 rounding of a
+ * different order).  The plan must have been made with same_rows = 1 and must have NO overflowing chunk: the first
+ * uint32 of the plan counts them -- read it back once per plan and call fgx_conv_wgrad instead when it is not 0.
+ * scratch: fgx_narrow_wgrad_scratch_bytes(V) bytes, 16-byte aligned.  The bias gradient is not made here (fgx_colsum).
+ * No counterpart in the reference (..._bwd_masked_implicit_gemm_splitk.py:108-182 gathers both operands per pair). */
+size_t fgx_narrow_wgrad_scratch_bytes(int V);
+int fgx_conv_narrow_wgrad(int dtype, const void* grad_out, const void* feats, const void* plan, size_t n, size_t n_src, int Ci,
+                          int Co, int V, void* scratch, void* grad_weight, fgx_stream_t stream);
 
 /* item_at for fgx_conv_gather_gemm_stream, made on the device from the tile codes: items sorted by cost (offsets per
  * row tile x `slabs` K-slabs + an epilogue), the incomplete last round of `groups` positions filled with the cheapest,

@@ -101,11 +101,42 @@ def test_narrow_resident_gemm_matches_oracle(gpu_device, dtype, res, ci, co):
     finally:
         impl.spconv.NARROW_RESIDENT = old
     assert hasattr(cache, "_narrow_plan_buf"), "the resident-row kernel did not run"
+    assert getattr(cache, "_narrow_overflows", None) == 0, "the weight gradient did not take the resident-row kernel"
+
+
+def test_narrow_resident_wgrad_is_reproducible_and_falls_back_on_overflow(gpu_device):
+    """fgx_conv_narrow_wgrad twice: same bits (fixed summation order); against the block-major kernel fp32 rounding of a
+    different order.  A plan whose header counts overflowing chunks sends the weight gradient to the block-major kernel."""
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    _say("narrow resident wgrad reproducibility / fallback")
+    res, ci, co = 40, 32, 24
+    coords_np = reference_test_shell(res)
+    coords = torch.from_numpy(coords_np).to(gpu_device)
+    shape = torch.Size([1, ci, res, res, res])
+    f, _, _, g = _case(coords_np, ci, co, torch.bfloat16, 59)
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+    fd, gd = f.to(gpu_device), g.to(gpu_device)
+    old = impl.spconv.NARROW_RESIDENT
+    try:
+        impl.spconv.NARROW_RESIDENT = "on"
+        a = impl._wgrad(gd, fd, cache, 27, with_bias=True, bias_offset=13)
+        b = impl._wgrad(gd, fd, cache, 27, with_bias=True, bias_offset=13)
+        assert cache["_narrow_overflows"] == 0
+        impl.spconv.NARROW_RESIDENT = "off"
+        c = impl._wgrad(gd, fd, cache, 27, with_bias=True, bias_offset=13)
+        impl.spconv.NARROW_RESIDENT = "on"
+        cache["_narrow_overflows"] = 3                # as if three chunks had overflowed
+        d = impl._wgrad(gd, fd, cache, 27, with_bias=True, bias_offset=13)
+    finally:
+        impl.spconv.NARROW_RESIDENT = old
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    assert eg.max_rel_err(a[0].cpu(), c[0].cpu().double()) <= 1e-2 and eg.max_rel_err(a[1].cpu(), c[1].cpu().double()) <= 1e-2
+    assert torch.equal(d[0], c[0]), "with overflowing chunks the block-major kernel runs"
 
 
 def test_narrow_resident_gemm_relu_mask_and_overflowing_chunks(gpu_device):
     """The resident-row kernel with the fused ReLU and its bit mask; and with rows in a random order, where a chunk of 128
-    rows has far more than 384 distinct sources, so that most sources are read from memory by the multipliers: the sums
+    rows has far more than 448 distinct sources, so that most sources are read from memory by the multipliers: the sums
     run over the same offsets in the same order, so the result is the same bit for bit as with the rows in Z-order."""
     import ctypes as C
     from flexgemm_amd import _native as nat
@@ -148,8 +179,10 @@ def test_narrow_resident_gemm_relu_mask_and_overflowing_chunks(gpu_device):
                                              nat.ptr(o), nat.ptr(None), nat.stream()))
             outs.append(o.cpu())
             chunks = -(-n // 128)
-            table = plan.cpu().numpy().reshape(chunks, 8192 + 1536 + 512)[:, :8192].copy().view(np.uint16).reshape(chunks, 128, 32)
+            raw = plan.cpu().numpy()
+            table = raw[256:].reshape(chunks, 8192 + 448 * 4 + 512)[:, :8192].copy().view(np.uint16).reshape(chunks, 128, 32)
             assert (table[:, :, 31] != 0).any(), "no chunk overflowed: the test does not reach the path it is for"
+            assert int(raw[:4].view(np.uint32)[0]) == int((table[:, :, 31] != 0).any(1).sum()), "the header does not count the overflowing chunks"
     assert torch.equal(outs[0], out.cpu()) and torch.equal(outs[1], out.cpu())
 
 
