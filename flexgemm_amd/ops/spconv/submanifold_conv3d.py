@@ -648,7 +648,11 @@ def _narrow_applies(cache, src: torch.Tensor, k: int, cols: int, v: int, n: int,
             and n_src * k * 2 < 0xFF000000 and n * 82 + 10752 < 0xFF000000)
     if not fits:
         return False
-    if mode == "on" or hasattr(cache, "_narrow_plan_buf"):
+    if hasattr(cache, "_narrow_plan_buf"):
+        return True
+    if torch.cuda.is_current_stream_capturing():
+        return False                    # no plan is made inside a graph capture (it would be remade on every replay)
+    if mode == "on":
         return True
     # "auto": the plan costs about as much as a neighbor-cache build (1.2 ms for 2.7 M voxels) and a call gains 0.1 ms on
     # it, so a cache gets one once it has served NARROW_RESIDENT_AFTER_CALLS narrow products on the streaming kernel:
@@ -673,6 +677,8 @@ def _narrow_wgrad_applies(cache, f: torch.Tensor, ci: int, co: int, v: int, n: i
     if not fits or not (mode == "on" or hasattr(cache, "_narrow_plan_buf")):
         return False
     if not hasattr(cache, "_narrow_overflows"):
+        if torch.cuda.is_current_stream_capturing():
+            return False                # the header cannot be read back inside a graph capture
         cache["_narrow_overflows"] = int(cache._narrow_plan()[:4].view(torch.int32).item())
     return cache["_narrow_overflows"] == 0
 

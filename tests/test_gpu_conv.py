@@ -1064,11 +1064,23 @@ def test_relu_bit_mask_of_the_epilogue_and_its_use_in_backward(gpu_device, dtype
                                                 nat.ptr(g), nat.stream()))
 
 
-def test_training_step_replays_from_a_hip_graph(gpu_device):
+@pytest.mark.parametrize("c,narrow", [(128, "auto"), (32, "on")])
+def test_training_step_replays_from_a_hip_graph(gpu_device, c, narrow):
     """Forward and backward of two stacked layers captured once (whole-step capture: static input, gradients allocated
     by the captured backward) and replayed with new inputs; every replay equals the eager step bit for bit, with eager
-    steps of the same layers running between the replays."""
-    res, c = 48, 128
+    steps of the same layers running between the replays.  With 32 channels and the resident-row kernels forced on, the
+    warm-up steps make the plan and read its header; the capture then records those kernels and nothing else."""
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    old_narrow = impl.spconv.NARROW_RESIDENT
+    impl.spconv.NARROW_RESIDENT = narrow
+    try:
+        _graph_training_step(gpu_device, c, narrow == "on")
+    finally:
+        impl.spconv.NARROW_RESIDENT = old_narrow
+
+
+def _graph_training_step(gpu_device, c, expect_narrow):
+    res = 48
     coords_np = reference_test_shell(res)
     shape = torch.Size([1, c, res, res, res])
     coords = torch.from_numpy(coords_np).to(gpu_device)
@@ -1120,3 +1132,4 @@ def test_training_step_replays_from_a_hip_graph(gpu_device):
             assert torch.equal(a, b_), f"replay {k}, tensor {i} differs from the eager step"
         for p, sg in zip(params, static_grads):
             p.grad = sg                    # hand the static gradient tensors back for the next replay
+    assert hasattr(cache, "_narrow_plan_buf") == expect_narrow and (getattr(cache, "_narrow_overflows", None) == 0) == expect_narrow
