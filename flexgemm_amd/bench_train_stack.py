@@ -57,12 +57,20 @@ def main():
     p.add_argument("--relu", choices=("none", "fused", "fused-no-bits", "separate"), default="none",
                    help="a ReLU after every layer: in the GEMM's epilogue (sparse_submanifold_conv3d_relu; fused-no-bits: "
                         "its backward tests the saved output instead of the epilogue's bit mask) or as torch.relu")
+    p.add_argument("--config", default="", help="RES,C,L: one configuration of its own instead of the reference's list")
+    p.add_argument("--narrow", choices=("auto", "on", "off"), default="auto",
+                   help="the resident-row kernels of narrow layers (flexgemm_amd.ops.spconv.NARROW_RESIDENT)")
     args = p.parse_args()
 
     import flex_gemm
     from flex_gemm.ops.spconv import Algorithm, SubMConv3dFunction, sparse_submanifold_conv3d, sparse_submanifold_conv3d_relu
     from flexgemm_amd.ops import spconv as spconv_config
     spconv_config.RELU_BIT_MASK = args.relu != "fused-no-bits"
+    spconv_config.NARROW_RESIDENT = args.narrow
+    configs = CONFIGS
+    if args.config:
+        configs = [tuple(int(x) for x in args.config.split(","))]
+        args.max_res = max(args.max_res, configs[0][0])
 
     def layer(h, coords, shape, w, b, cache):
         if args.relu in ("fused", "fused-no-bits"):
@@ -77,7 +85,7 @@ def main():
     dev = torch.device("cuda:0")
     flex_gemm.ops.spconv.set_algorithm(Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
     flex_gemm.ops.spconv.set_weight_panel_cache(args.panel_cache, max_bytes=16 << 30)
-    for res, c, layers in CONFIGS:
+    for res, c, layers in configs:
         if res > args.max_res:
             continue
         coords = torch.from_numpy(reference_test_shell(res)).to(dev)
