@@ -104,6 +104,25 @@ def test_narrow_resident_gemm_matches_oracle(gpu_device, dtype, res, ci, co):
     assert getattr(cache, "_narrow_overflows", None) == 0, "the weight gradient did not take the resident-row kernel"
 
 
+@pytest.mark.parametrize("res,ksize,dilation", [(4, (3, 3, 3), (1, 1, 1)), (24, (3, 3, 1), (1, 1, 1)), (24, (1, 3, 3), (2, 1, 1)),
+                                                (16, (1, 1, 1), (1, 1, 1))])
+def test_narrow_resident_kernels_other_volumes_and_tiny_inputs(gpu_device, res, ksize, dilation):
+    """The resident-row kernels with fewer voxels than one chunk, and with kernel volumes other than 27 (the offsets' loop
+    is then not unrolled; the weight gradient's multipliers own eight offsets each, so nine offsets leave three of the
+    four nearly idle, one offset three of them entirely)."""
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    _say(f"narrow resident res={res} ksize={ksize} dilation={dilation}")
+    coords_np = reference_test_shell(res)
+    old = impl.spconv.NARROW_RESIDENT
+    impl.spconv.NARROW_RESIDENT = "on"
+    try:
+        cache, _ = _run_and_check(coords_np, torch.Size([1, 32, res, res, res]), 32, 16, torch.float16, gpu_device, seed=res,
+                                  ksize=ksize, dilation=dilation)
+    finally:
+        impl.spconv.NARROW_RESIDENT = old
+    assert hasattr(cache, "_narrow_plan_buf") and getattr(cache, "_narrow_overflows", None) == 0
+
+
 def test_narrow_resident_wgrad_is_reproducible_and_falls_back_on_overflow(gpu_device):
     """fgx_conv_narrow_wgrad twice: same bits (fixed summation order); against the block-major kernel fp32 rounding of a
     different order.  A plan whose header counts overflowing chunks sends the weight gradient to the block-major kernel."""
