@@ -37,7 +37,7 @@ EXPORTS = [
     "fgx_conv_gather_gemm_stream_groups", "fgx_gather_item_order_workspace_bytes", "fgx_gather_item_order",
     "fgx_wgrad_scratch_bytes", "fgx_wgrad_block_bounds_count", "fgx_wgrad_block_bounds", "fgx_conv_wgrad",
     "fgx_wgrad_item_lists_count", "fgx_wgrad_item_lists", "fgx_conv_wgrad_lists",
-    "fgx_narrow_plan_bytes", "fgx_narrow_plan", "fgx_conv_narrow_gemm", "fgx_narrow_wgrad_scratch_bytes", "fgx_conv_narrow_wgrad",
+    "fgx_zorder_rows", "fgx_narrow_plan_bytes", "fgx_narrow_plan", "fgx_conv_narrow_gemm", "fgx_narrow_wgrad_scratch_bytes", "fgx_conv_narrow_wgrad",
     "fgx_wgrad_sweep_plan_bytes", "fgx_wgrad_sweep_plan", "fgx_wgrad_sweep_scratch_bytes", "fgx_conv_wgrad_sweep",
     "fgx_wgrad_sweep_giveup_words", "fgx_wgrad_sweep_reduce",
     "fgx_colsum_scratch_bytes", "fgx_colsum", "fgx_colsum_static_prepare", "fgx_colsum_static_max_cols", "fgx_colsum_static",

@@ -83,9 +83,14 @@ __global__ void __launch_bounds__(256) narrow_plan_kernel(const uint32_t* __rest
         }
         __syncthreads();
     }
-    for (int e = tid; e < entries; e += 256) {
-        const uint32_t idx = source_of(e);
-        if (idx != FGX_EMPTY32) insert(idx);
+    // (a thread's entries stay in registers for the second pass: kNarrowRows * kNarrowMaxV / 256 of them at most)
+    constexpr int kPerThread = (kNarrowRows * 32 + 255) / 256;
+    uint32_t mine_idx[kPerThread];
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j) {
+        const int e = tid + j * 256;
+        mine_idx[j] = e < entries ? source_of(e) : FGX_EMPTY32;
+        if (mine_idx[j] != FGX_EMPTY32) insert(mine_idx[j]);
     }
     __syncthreads();
     // the other sources: slots from `base` on in table order (exclusive scan of their positions, four per thread)
@@ -120,8 +125,11 @@ __global__ void __launch_bounds__(256) narrow_plan_kernel(const uint32_t* __rest
     const uint32_t total = base + scan[255];
     for (uint32_t s = total + tid; s < (uint32_t)kNarrowSlots; s += 256) sources[s] = FGX_EMPTY32;
     __syncthreads();
-    for (int e = tid; e < entries; e += 256) {
-        const uint32_t idx = source_of(e);
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j) {
+        const int e = tid + j * 256;
+        if (e >= entries) break;
+        const uint32_t idx = mine_idx[j];
         uint16_t out = (uint16_t)kNarrowZeroSlot;
         if (idx != FGX_EMPTY32) {
             out = (uint16_t)kNarrowOverflow;

@@ -53,6 +53,17 @@ __global__ void __launch_bounds__(kBlock) morton_key_kernel(const int32_t* __res
     vals[i] = (uint32_t)i;
 }
 
+// the same with the batch index right above the 3 * bits interleaved coordinate bits: only the low bits differ
+__global__ void __launch_bounds__(kBlock) morton_key_packed_kernel(const int32_t* __restrict__ coords, size_t n, int bits,
+                                                                   uint64_t* __restrict__ keys, uint32_t* __restrict__ vals) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    int4 c = reinterpret_cast<const int4*>(coords)[i];
+    const uint64_t m = (spread16((uint32_t)c.y) << 2) | (spread16((uint32_t)c.z) << 1) | spread16((uint32_t)c.w);
+    keys[i] = ((uint64_t)(uint32_t)c.x << (3 * bits)) | (m & ((1ull << (3 * bits)) - 1ull));
+    vals[i] = (uint32_t)i;
+}
+
 // position p of the spatial order -> (chunk of p, mask code of its voxel)
 __global__ void __launch_bounds__(kBlock) chunk_code_key_kernel(const uint32_t* __restrict__ perm,
                                                                 const int32_t* __restrict__ binary, size_t n,
@@ -561,6 +572,34 @@ int fgx_locality_order(const int32_t* coords, const int32_t* binary, size_t n, i
     FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp_bytes, keys_a, keys_b, vals_b, vals_a, n, 0u, end_bit, s));
     widen_u32_i64_kernel<<<grid, kBlock, 0, s>>>(vals_a, order, n);
     FGX_CHECK_LAUNCH("fgx_locality_order(widen)");
+    return FGX_OK;
+}
+
+int fgx_zorder_rows(const int32_t* coords, size_t n, int bits_per_axis, int batch_bits, int64_t* order, void* workspace,
+                    size_t workspace_bytes, fgx_stream_t stream) {
+    FGX_CHECK_ARG(bits_per_axis >= 1 && bits_per_axis <= 16 && batch_bits >= 0 && 3 * bits_per_axis + batch_bits <= 64,
+                  "fgx_zorder_rows: %d bits per axis and %d batch bits do not fit a 64-bit key", bits_per_axis, batch_bits);
+    FGX_CHECK_ARG(n < 0xFFFFFFFFull, "fgx_zorder_rows: too many rows");
+    if (n == 0) return FGX_OK;
+    LocalityLayout L = locality_layout(n);
+    FGX_CHECK_ARG(coords && order && workspace, "fgx_zorder_rows: null buffer");
+    FGX_CHECK_ARG(((uintptr_t)coords & 15) == 0, "fgx_zorder_rows: coords must be 16-byte aligned");
+    FGX_CHECK_ARG(workspace_bytes >= L.total, "fgx_zorder_rows: workspace of %zu bytes, need %zu", workspace_bytes, L.total);
+    FGX_CHECK_ARG(((uintptr_t)workspace & 255) == 0, "fgx_zorder_rows: workspace must be 256-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    char* ws = (char*)workspace;
+    uint64_t* keys_a = (uint64_t*)(ws + L.keys_a);
+    uint64_t* keys_b = (uint64_t*)(ws + L.keys_b);
+    uint32_t* vals_a = (uint32_t*)(ws + L.vals_a);
+    uint32_t* vals_b = (uint32_t*)(ws + L.vals_b);
+    const unsigned grid = cdiv(n, kBlock);
+    morton_key_packed_kernel<<<grid, kBlock, 0, s>>>(coords, n, bits_per_axis, keys_a, vals_a);
+    FGX_CHECK_LAUNCH("fgx_zorder_rows(keys)");
+    size_t temp_bytes = L.temp_bytes;
+    FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp_bytes, keys_a, keys_b, vals_a, vals_b, n, 0u,
+                                            (unsigned)(3 * bits_per_axis + batch_bits), s));
+    widen_u32_i64_kernel<<<grid, kBlock, 0, s>>>(vals_b, order, n);
+    FGX_CHECK_LAUNCH("fgx_zorder_rows(widen)");
     return FGX_OK;
 }
 

@@ -238,16 +238,18 @@ class SubMConv3dNeighborCache:
             nmap = self["neighbor_map"]
             n, v = nmap.shape
             dev = nmap.device
-            if not hasattr(self, "_binary_code"):
-                _, binary, _ = _codes_and_order(nmap, None, None)
-                self["_binary_code"] = binary
             L = nat.lib()
             with torch.cuda.device(dev):
                 order = torch.empty((n,), dtype=torch.int64, device=dev)
                 ws = nat.workspace(L.fgx_locality_workspace_bytes(nat.sz(n)), dev)
-                # chunks of one rank: the plain Z-order of the rows
-                nat.check(L.fgx_locality_order(nat.ptr(self["_coords"]), nat.ptr(self["_binary_code"]), nat.sz(n), C.c_int(v),
-                                               C.c_int(1), nat.ptr(order), nat.ptr(ws), nat.sz(ws.numel()), nat.stream()))
+                # the Z-order of the rows; the grid the cache was built for bounds the key bits that can differ
+                batch, spatial = self["_grid"]
+                bits = max(max(int(d) for d in spatial) - 1, 1).bit_length()
+                batch_bits = max(int(batch) - 1, 0).bit_length()
+                if bits > 16 or 3 * bits + batch_bits > 64:
+                    bits, batch_bits = 16, 16
+                nat.check(L.fgx_zorder_rows(nat.ptr(self["_coords"]), nat.sz(n), C.c_int(bits), C.c_int(batch_bits), nat.ptr(order),
+                                            nat.ptr(ws), nat.sz(ws.numel()), nat.stream()))
                 plan = torch.empty((int(L.fgx_narrow_plan_bytes(nat.sz(n), C.c_int(v))),), dtype=torch.uint8, device=dev)
                 nat.check(L.fgx_narrow_plan(nat.ptr(nmap), nat.ptr(order), nat.sz(n), C.c_int(v), C.c_int(1), nat.ptr(plan), nat.stream()))
             self["_narrow_plan_buf"] = plan
@@ -654,7 +656,7 @@ def _narrow_applies(cache, src: torch.Tensor, k: int, cols: int, v: int, n: int,
         return False                    # no plan is made inside a graph capture (it would be remade on every replay)
     if mode == "on":
         return True
-    # "auto": the plan costs about as much as a neighbor-cache build (1.2 ms for 2.7 M voxels) and a call gains 0.1 ms on
+    # "auto": the plan costs two thirds of a neighbor-cache build (0.66 ms for 2.7 M voxels) and a call gains 0.1 ms on
     # it, so a cache gets one once it has served NARROW_RESIDENT_AFTER_CALLS narrow products on the streaming kernel:
     # whatever happens next, the detour then costs at most what the calls before it did.
     if n < NARROW_RESIDENT_MIN_ROWS:
@@ -852,6 +854,7 @@ class SubMConv3dFunction(Function):
         cache = SubMConv3dNeighborCache(neighbor_map=nmap, gray_code=gray, sorted_idx=order)
         cache["_coords"] = coords           # for the private row order, built on first use by a short-row layer
         cache["_needs_grad"] = bool(needs_grad)
+        cache["_grid"] = (int(shape[0]), tuple(int(d) for d in shape[2:]))
         cache["_binary_code"] = binary
         if needs_grad:
             cache._attach_pairs(_pair_lists(nmap, gray))

@@ -145,6 +145,13 @@ size_t fgx_locality_workspace_bytes(size_t n);
 int fgx_locality_order(const int32_t* coords, const int32_t* binary, size_t n, int V, int chunk_rows, int64_t* order,
                        void* workspace, size_t workspace_bytes, fgx_stream_t stream);
 
+/* The plain Z-order of the rows (what fgx_locality_order gives with chunk_rows = 1) when the grid is known: coordinates
+ * below 2^bits_per_axis, batch indices below 2^batch_bits -- the sort then runs over 3 * bits_per_axis + batch_bits key bits
+ * instead of 64 (2.67 M voxels of a 1024-cube: four passes instead of eight).  Coordinates outside that range are sorted
+ * by their low bits (still a permutation).  Workspace: fgx_locality_workspace_bytes(n).  The row order of fgx_narrow_plan. */
+int fgx_zorder_rows(const int32_t* coords, size_t n, int bits_per_axis, int batch_bits, int64_t* order, void* workspace,
+                    size_t workspace_bytes, fgx_stream_t stream);
+
 /* Pair lists for wgrad: all (v, n) with map[n, v] present, ordered by v then n.
  *   count: seg[V+1] <- exclusive offsets per v (seg[V] = L); caller reads seg[V] back, allocates
  *          sig_i / sig_o of L uint32 each, then calls fill with the same workspace.
