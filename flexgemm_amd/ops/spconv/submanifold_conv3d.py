@@ -657,15 +657,15 @@ def _narrow_applies(cache, src: torch.Tensor, k: int, cols: int, v: int, n: int,
     if mode == "on":
         return True
     # "auto": the plan costs two thirds of a neighbor-cache build (0.66 ms for 2.7 M voxels) and a call gains 0.1 ms on
-    # it, so a cache gets one once it has served NARROW_RESIDENT_AFTER_CALLS narrow products on the streaming kernel:
-    # whatever happens next, the detour then costs at most what the calls before it did.
+    # it, so a cache gets one once it has served NARROW_RESIDENT_AFTER_CALLS narrow products on the streaming kernel (what
+    # the plan costs in passes): whatever happens next, the detour then costs at most what the calls before it did.
     if n < NARROW_RESIDENT_MIN_ROWS:
         return False
     calls = getattr(cache, "_narrow_calls", 0) + 1
     cache["_narrow_calls"] = calls
     # A cache made for training also serves weight gradients, which gain three times what a forward pass does (0.66 ->
-    # 0.26 ms at 2.67 M voxels): with half a million voxels and more its plan pays from the third layer on, so it comes
-    # at the third product.
+    # 0.26 ms at 2.67 M voxels): with half a million voxels and more its plan pays from the second layer on, so it comes
+    # at the second product (a single layer never asks for one).
     eager = getattr(cache, "_needs_grad", False) and n >= NARROW_RESIDENT_TRAINING_MIN_ROWS
     return calls > (NARROW_RESIDENT_AFTER_CALLS_TRAINING if eager else NARROW_RESIDENT_AFTER_CALLS)
 
@@ -702,16 +702,13 @@ def _sweep_fits(n: int, n_in: int, ci: int, co: int, elem_bytes: int, n_pairs: i
             and n_pairs * 4 + 256 <= 0xFF000000)
 
 
-# pacing of the wgrad sweep: sub-blocks a workgroup may run ahead of the slowest one of its XCD, and the looks at the
-# others' progress after which it stops waiting (0 = no pacing, the default: the workgroups of an XCD stay close enough
-# together by themselves, and waiting costs more time than the L2 misses it saves)
 # Fewest rows from which NARROW_RESIDENT = "auto" takes the resident-row kernel.
 NARROW_RESIDENT_MIN_ROWS = 32768
 # ... and narrow products a neighbor cache serves on the streaming kernel before it gets the plan.
-NARROW_RESIDENT_AFTER_CALLS = 8
-# ... a cache made for training (it will serve weight gradients too) of this many rows and more: after two products.
+NARROW_RESIDENT_AFTER_CALLS = 5
+# ... a cache made for training (it will serve weight gradients too) of this many rows and more: after one product.
 NARROW_RESIDENT_TRAINING_MIN_ROWS = 524288
-NARROW_RESIDENT_AFTER_CALLS_TRAINING = 2
+NARROW_RESIDENT_AFTER_CALLS_TRAINING = 1
 # The gather GEMM's tiles are dealt by cost when there are more than this many rounds of items (tiles per persistent
 # workgroup).
 ITEM_ORDER_MIN_ROUNDS = 1
@@ -720,6 +717,9 @@ ITEM_ORDER_ANY_ROW_MAX_ROUNDS = 9
 # The streaming weight gradient walks per-workgroup work lists balanced by pair count (fgx_wgrad_item_lists) where the
 # library has them for the shape; False = the kernel's fixed interleave.  Same result bit for bit.
 WGRAD_BALANCED_LISTS = True
+# pacing of the wgrad sweep: sub-blocks a workgroup may run ahead of the slowest one of its XCD, and the looks at the
+# others' progress after which it stops waiting (0 = no pacing, the default: the workgroups of an XCD stay close enough
+# together by themselves, and waiting costs more time than the L2 misses it saves)
 WGRAD_SWEEP_LEAD = 3
 WGRAD_SWEEP_MAX_POLLS = 0
 
