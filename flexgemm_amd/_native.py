@@ -27,7 +27,7 @@ EXPORTS = [
     "fgx_hash_init", "fgx_hash_insert_3d_idx_as_val", "fgx_hash_insert", "fgx_hash_lookup",
     "fgx_hash_insert_3d", "fgx_hash_lookup_3d",
     "fgx_subm_neighbor_map", "fgx_subm_neighbor_map_sorted_workspace_bytes", "fgx_subm_neighbor_map_sorted", "fgx_coords_key_order", "fgx_mask_codes",
-    "fgx_sort_workspace_bytes", "fgx_sort_by_code", "fgx_locality_workspace_bytes", "fgx_locality_order",
+    "fgx_sort_workspace_bytes", "fgx_sort_by_code", "fgx_locality_workspace_bytes", "fgx_locality_order", "fgx_locality_order_grid",
     "fgx_pair_workspace_bytes", "fgx_pair_count", "fgx_pair_fill",
     "fgx_tile_workspace_bytes", "fgx_tile_codes", "fgx_tile_fill",
     "fgx_table_lookup", "fgx_weight_panel_bytes", "fgx_pack_weight",

@@ -43,34 +43,25 @@ __device__ __forceinline__ uint64_t spread16(uint32_t x) {
     return v;
 }
 
-__global__ void __launch_bounds__(kBlock) morton_key_kernel(const int32_t* __restrict__ coords, size_t n,
-                                                            uint64_t* __restrict__ keys, uint32_t* __restrict__ vals) {
-    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i >= n) return;
-    int4 c = reinterpret_cast<const int4*>(coords)[i];
-    keys[i] = ((uint64_t)((uint32_t)c.x & 0xFFFFu) << 48) | (spread16((uint32_t)c.y) << 2) | (spread16((uint32_t)c.z) << 1) |
-              spread16((uint32_t)c.w);
-    vals[i] = (uint32_t)i;
-}
-
-// the same with the batch index right above the 3 * bits interleaved coordinate bits: only the low bits differ
+// Z-order key: the batch index right above the 3 * bits interleaved coordinate bits (Key: 32 bits when they all fit)
+template <typename Key>
 __global__ void __launch_bounds__(kBlock) morton_key_packed_kernel(const int32_t* __restrict__ coords, size_t n, int bits,
-                                                                   uint64_t* __restrict__ keys, uint32_t* __restrict__ vals) {
+                                                                   Key* __restrict__ keys, uint32_t* __restrict__ vals) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
     int4 c = reinterpret_cast<const int4*>(coords)[i];
     const uint64_t m = (spread16((uint32_t)c.y) << 2) | (spread16((uint32_t)c.z) << 1) | spread16((uint32_t)c.w);
-    keys[i] = ((uint64_t)(uint32_t)c.x << (3 * bits)) | (m & ((1ull << (3 * bits)) - 1ull));
+    keys[i] = (Key)(((uint64_t)(uint32_t)c.x << (3 * bits)) | (m & ((1ull << (3 * bits)) - 1ull)));
     vals[i] = (uint32_t)i;
 }
 
 // position p of the spatial order -> (chunk of p, mask code of its voxel)
 __global__ void __launch_bounds__(kBlock) chunk_code_key_kernel(const uint32_t* __restrict__ perm,
                                                                 const int32_t* __restrict__ binary, size_t n,
-                                                                uint32_t chunk_rows, uint64_t* __restrict__ keys) {
+                                                                uint32_t chunk_rows, int code_bits, uint64_t* __restrict__ keys) {
     size_t p = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (p >= n) return;
-    keys[p] = ((uint64_t)(p / chunk_rows) << 32) | (uint32_t)binary[perm[p]];
+    keys[p] = ((uint64_t)(p / chunk_rows) << code_bits) | (uint32_t)binary[perm[p]];
 }
 
 struct LocalityLayout {
@@ -486,6 +477,30 @@ TileLayout tile_layout(size_t n, int block) {
     return L;
 }
 
+// rows ranked along the Z-order curve (batch index above 3 * bits interleaved coordinate bits) into ranked[]: a radix sort
+// over the key bits a coordinate of the grid can differ in, on 32-bit keys when they fit
+int zorder_rank(const int32_t* coords, size_t n, int bits_per_axis, int batch_bits, const LocalityLayout& L, char* ws,
+                uint32_t* ranked, uint32_t* other, hipStream_t s, const char* what) {
+    const unsigned grid = cdiv(n, kBlock);
+    const unsigned end_bit = (unsigned)(3 * bits_per_axis + batch_bits);
+    size_t temp_bytes = L.temp_bytes;
+    if (end_bit <= 32) {
+        uint32_t* keys_a = (uint32_t*)(ws + L.keys_a);
+        uint32_t* keys_b = (uint32_t*)(ws + L.keys_b);
+        morton_key_packed_kernel<uint32_t><<<grid, kBlock, 0, s>>>(coords, n, bits_per_axis, keys_a, other);
+        FGX_CHECK_LAUNCH(what);
+        FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp_bytes, keys_a, keys_b, other, ranked, n, 0u, end_bit, s));
+    } else {
+        uint64_t* keys_a = (uint64_t*)(ws + L.keys_a);
+        uint64_t* keys_b = (uint64_t*)(ws + L.keys_b);
+        morton_key_packed_kernel<uint64_t><<<grid, kBlock, 0, s>>>(coords, n, bits_per_axis, keys_a, other);
+        FGX_CHECK_LAUNCH(what);
+        FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp_bytes, keys_a, keys_b, other, ranked, n, 0u, end_bit, s));
+    }
+    return FGX_OK;
+}
+
+
 }  // namespace
 }  // namespace fgx
 
@@ -538,10 +553,12 @@ int fgx_sort_by_code(const int32_t* binary, size_t n, int V, int64_t* sorted_idx
 
 size_t fgx_locality_workspace_bytes(size_t n) { return locality_layout(n).total; }
 
-int fgx_locality_order(const int32_t* coords, const int32_t* binary, size_t n, int V, int chunk_rows, int64_t* order,
-                       void* workspace, size_t workspace_bytes, fgx_stream_t stream) {
+int fgx_locality_order_grid(const int32_t* coords, const int32_t* binary, size_t n, int V, int chunk_rows, int bits_per_axis,
+                            int batch_bits, int64_t* order, void* workspace, size_t workspace_bytes, fgx_stream_t stream) {
     FGX_CHECK_ARG(V >= 1 && V <= 32, "fgx_locality_order: kernel volume must be in [1, 32], got %d", V);
     FGX_CHECK_ARG(chunk_rows >= 1, "fgx_locality_order: chunk_rows must be positive, got %d", chunk_rows);
+    FGX_CHECK_ARG(bits_per_axis >= 1 && bits_per_axis <= 16 && batch_bits >= 0 && 3 * bits_per_axis + batch_bits <= 64,
+                  "fgx_locality_order: %d bits per axis and %d batch bits do not fit a 64-bit key", bits_per_axis, batch_bits);
     FGX_CHECK_ARG(n < 0xFFFFFFFFull, "fgx_locality_order: too many rows");
     if (n == 0) return FGX_OK;
     LocalityLayout L = locality_layout(n);
@@ -556,23 +573,28 @@ int fgx_locality_order(const int32_t* coords, const int32_t* binary, size_t n, i
     uint32_t* vals_a = (uint32_t*)(ws + L.vals_a);
     uint32_t* vals_b = (uint32_t*)(ws + L.vals_b);
     const unsigned grid = cdiv(n, kBlock);
-    morton_key_kernel<<<grid, kBlock, 0, s>>>(coords, n, keys_a, vals_a);
-    FGX_CHECK_LAUNCH("fgx_locality_order(keys)");
-    size_t temp_bytes = L.temp_bytes;
-    FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp_bytes, keys_a, keys_b, vals_a, vals_b, n, 0u, 64u, s));
+    int rc = zorder_rank(coords, n, bits_per_axis, batch_bits, L, ws, vals_b, vals_a, s, "fgx_locality_order(keys)");
+    if (rc != FGX_OK) return rc;
     if (chunk_rows == 1) {              // chunks of one rank: the curve's own order, nothing to sort inside them
         widen_u32_i64_kernel<<<grid, kBlock, 0, s>>>(vals_b, order, n);
         FGX_CHECK_LAUNCH("fgx_locality_order(widen)");
         return FGX_OK;
     }
-    chunk_code_key_kernel<<<grid, kBlock, 0, s>>>(vals_b, binary, n, (uint32_t)chunk_rows, keys_a);
+    // (chunk, mask code) keys with the chunk right above the V code bits: the sort runs over the bits in use alone
+    chunk_code_key_kernel<<<grid, kBlock, 0, s>>>(vals_b, binary, n, (uint32_t)chunk_rows, V, keys_a);
     FGX_CHECK_LAUNCH("fgx_locality_order(chunk keys)");
-    const unsigned end_bit = 32u + (unsigned)bits_for((n - 1) / (size_t)chunk_rows);
-    temp_bytes = L.temp_bytes;
+    const unsigned end_bit = (unsigned)V + (unsigned)bits_for((n - 1) / (size_t)chunk_rows);
+    size_t temp_bytes = L.temp_bytes;
     FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp_bytes, keys_a, keys_b, vals_b, vals_a, n, 0u, end_bit, s));
     widen_u32_i64_kernel<<<grid, kBlock, 0, s>>>(vals_a, order, n);
     FGX_CHECK_LAUNCH("fgx_locality_order(widen)");
     return FGX_OK;
+}
+
+int fgx_locality_order(const int32_t* coords, const int32_t* binary, size_t n, int V, int chunk_rows, int64_t* order,
+                       void* workspace, size_t workspace_bytes, fgx_stream_t stream) {
+    // coordinates of any grid: 16 bits per axis and 16 bits of batch index
+    return fgx_locality_order_grid(coords, binary, n, V, chunk_rows, 16, 16, order, workspace, workspace_bytes, stream);
 }
 
 int fgx_zorder_rows(const int32_t* coords, size_t n, int bits_per_axis, int batch_bits, int64_t* order, void* workspace,
@@ -588,17 +610,11 @@ int fgx_zorder_rows(const int32_t* coords, size_t n, int bits_per_axis, int batc
     FGX_CHECK_ARG(((uintptr_t)workspace & 255) == 0, "fgx_zorder_rows: workspace must be 256-byte aligned");
     hipStream_t s = (hipStream_t)stream;
     char* ws = (char*)workspace;
-    uint64_t* keys_a = (uint64_t*)(ws + L.keys_a);
-    uint64_t* keys_b = (uint64_t*)(ws + L.keys_b);
     uint32_t* vals_a = (uint32_t*)(ws + L.vals_a);
     uint32_t* vals_b = (uint32_t*)(ws + L.vals_b);
-    const unsigned grid = cdiv(n, kBlock);
-    morton_key_packed_kernel<<<grid, kBlock, 0, s>>>(coords, n, bits_per_axis, keys_a, vals_a);
-    FGX_CHECK_LAUNCH("fgx_zorder_rows(keys)");
-    size_t temp_bytes = L.temp_bytes;
-    FGX_CHECK_HIP(rocprim::radix_sort_pairs(ws + L.temp, temp_bytes, keys_a, keys_b, vals_a, vals_b, n, 0u,
-                                            (unsigned)(3 * bits_per_axis + batch_bits), s));
-    widen_u32_i64_kernel<<<grid, kBlock, 0, s>>>(vals_b, order, n);
+    int rc = zorder_rank(coords, n, bits_per_axis, batch_bits, L, ws, vals_b, vals_a, s, "fgx_zorder_rows(keys)");
+    if (rc != FGX_OK) return rc;
+    widen_u32_i64_kernel<<<cdiv(n, kBlock), kBlock, 0, s>>>(vals_b, order, n);
     FGX_CHECK_LAUNCH("fgx_zorder_rows(widen)");
     return FGX_OK;
 }

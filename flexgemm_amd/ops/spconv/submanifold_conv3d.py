@@ -227,7 +227,8 @@ class SubMConv3dNeighborCache:
         if not hasattr(self, "_binary_code"):
             _, binary, _ = _codes_and_order(self["neighbor_map"], None, None)
             self["_binary_code"] = binary
-        self["_tile_order"] = _locality_order(self["_coords"], self["_binary_code"], self["neighbor_map"].shape[1])
+        self["_tile_order"] = _locality_order(self["_coords"], self["_binary_code"], self["neighbor_map"].shape[1],
+                                              getattr(self, "_grid", None))
 
 
     def _narrow_plan(self):
@@ -243,11 +244,7 @@ class SubMConv3dNeighborCache:
                 order = torch.empty((n,), dtype=torch.int64, device=dev)
                 ws = nat.workspace(L.fgx_locality_workspace_bytes(nat.sz(n)), dev)
                 # the Z-order of the rows; the grid the cache was built for bounds the key bits that can differ
-                batch, spatial = self["_grid"]
-                bits = max(max(int(d) for d in spatial) - 1, 1).bit_length()
-                batch_bits = max(int(batch) - 1, 0).bit_length()
-                if bits > 16 or 3 * bits + batch_bits > 64:
-                    bits, batch_bits = 16, 16
+                bits, batch_bits = _grid_key_bits(self["_grid"])
                 nat.check(L.fgx_zorder_rows(nat.ptr(self["_coords"]), nat.sz(n), C.c_int(bits), C.c_int(batch_bits), nat.ptr(order),
                                             nat.ptr(ws), nat.sz(ws.numel()), nat.stream()))
                 plan = torch.empty((int(L.fgx_narrow_plan_bytes(nat.sz(n), C.c_int(v))),), dtype=torch.uint8, device=dev)
@@ -351,21 +348,58 @@ def _codes_and_order(nmap: torch.Tensor, gray: Optional[torch.Tensor], binary: O
 
 
 # The kernels' private row order (Z-order chunks, mask-sorted inside a chunk) trades ~12 % more padded MFMA work for
-# gathers that stay inside an XCD's L2.  It pays when rows are short and the pass is bandwidth bound.
+# gathers that stay inside an XCD's L2.  It pays when rows are short, the pass is bandwidth bound and the voxels are many
+# more than an L2 holds -- measured per forward pass at 32 / 64 channels: 4.1 M voxels 0.61 -> 0.54 / 1.07 -> 1.02 ms,
+# 1.03 M 0.169 -> 0.143 / 0.275 -> 0.240, 578 k 0.109 -> 0.103 / 0.172 -> 0.168, 252 k 0.060 -> 0.065 / 0.092 -> 0.090,
+# 64 k 0.049 -> 0.051 / 0.050 -> 0.053 -- and making it (two sorts and the tile tables of the new order) costs what seven to
+# ten passes gain (0.50 ms at 4.1 M voxels, 0.24 at 1.03 M).  So a cache gets it once it has served LOCALITY_AFTER_CALLS
+# short-row passes on the public order: whatever happens next, the detour then costs at most what those passes did.
 LOCALITY_CHUNK_ROWS = 8192      # rows per spatial chunk
 LOCALITY_MAX_ROW_BYTES = 128    # use the private order when a gathered row is at most this long
+LOCALITY_MIN_ROWS = 786432      # ... and the map has this many rows or more
+LOCALITY_AFTER_CALLS = 8        # ... and the cache has served this many such passes on the public order
 
 
-def _locality_order(coords: torch.Tensor, binary: torch.Tensor, v: int) -> torch.Tensor:
-    """Z-order chunks, mask-sorted inside each chunk (int64 permutation)."""
+def _locality_applies(cache, n: int, row_bytes: int) -> bool:
+    """Whether a masked gather GEMM with rows of `row_bytes` walks the private row order of `cache` (see above).  An order
+    that exists is used; none is made during a graph capture (the capture would hold the sorts)."""
+    if row_bytes > LOCALITY_MAX_ROW_BYTES:
+        return False
+    if hasattr(cache, "_tile_order"):
+        return True
+    if n < LOCALITY_MIN_ROWS or not hasattr(cache, "_coords") or torch.cuda.is_current_stream_capturing():
+        return False
+    calls = getattr(cache, "_short_row_calls", 0) + 1
+    cache["_short_row_calls"] = calls
+    return calls > LOCALITY_AFTER_CALLS
+
+
+def _grid_key_bits(grid) -> Tuple[int, int]:
+    """(bits per axis, batch bits) a Z-order key needs for coordinates of `grid` = (batch size, spatial sizes); 16 and 16
+    -- any coordinates -- when the grid is unknown or too large for less."""
+    if grid is None:
+        return 16, 16
+    batch, spatial = grid
+    bits = max(max(int(d) for d in spatial) - 1, 1).bit_length()
+    batch_bits = max(int(batch) - 1, 0).bit_length()
+    if bits > 16 or 3 * bits + batch_bits > 64:
+        return 16, 16
+    return bits, batch_bits
+
+
+def _locality_order(coords: torch.Tensor, binary: torch.Tensor, v: int, grid=None) -> torch.Tensor:
+    """Z-order chunks, mask-sorted inside each chunk (int64 permutation); `grid` = (batch size, spatial sizes) the
+    coordinates lie in, when known: it bounds the key bits the sorts go over."""
     n = coords.shape[0]
     dev = coords.device
     order = torch.empty((n,), dtype=torch.int64, device=dev)
     L = nat.lib()
+    bits, batch_bits = _grid_key_bits(grid)
     with torch.cuda.device(dev):
         ws = nat.workspace(L.fgx_locality_workspace_bytes(nat.sz(n)), dev)
-        nat.check(L.fgx_locality_order(nat.ptr(coords), nat.ptr(binary), nat.sz(n), C.c_int(v), C.c_int(LOCALITY_CHUNK_ROWS),
-                                       nat.ptr(order), nat.ptr(ws), nat.sz(ws.numel()), nat.stream()))
+        nat.check(L.fgx_locality_order_grid(nat.ptr(coords), nat.ptr(binary), nat.sz(n), C.c_int(v), C.c_int(LOCALITY_CHUNK_ROWS),
+                                            C.c_int(bits), C.c_int(batch_bits), nat.ptr(order), nat.ptr(ws), nat.sz(ws.numel()),
+                                            nat.stream()))
     return order
 
 
@@ -570,7 +604,7 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
     splitk = sched.splitk if allow_splitk else 1
     if masked:
         cache._ensure_sorted()
-    private = masked and k * src.element_size() <= LOCALITY_MAX_ROW_BYTES
+    private = masked and _locality_applies(cache, n, k * src.element_size())
     out = torch.empty((n, cols), dtype=dt, device=dev)
     if n == 0:
         return out

@@ -144,6 +144,11 @@ int fgx_sort_by_code(const int32_t* binary, size_t n, int V, int64_t* sorted_idx
 size_t fgx_locality_workspace_bytes(size_t n);
 int fgx_locality_order(const int32_t* coords, const int32_t* binary, size_t n, int V, int chunk_rows, int64_t* order,
                        void* workspace, size_t workspace_bytes, fgx_stream_t stream);
+/* The same order when the grid is known (coordinates below 2^bits_per_axis, batch indices below 2^batch_bits): both sorts
+ * then run over the key bits in use alone, the first on 32-bit keys when 3 * bits_per_axis + batch_bits <= 32 (4.1 M voxels
+ * of a 1024-cube: 9 radix passes instead of 14).  fgx_locality_order is this function with 16 and 16 bits. */
+int fgx_locality_order_grid(const int32_t* coords, const int32_t* binary, size_t n, int V, int chunk_rows, int bits_per_axis,
+                            int batch_bits, int64_t* order, void* workspace, size_t workspace_bytes, fgx_stream_t stream);
 
 /* The plain Z-order of the rows (what fgx_locality_order gives with chunk_rows = 1) when the grid is known: coordinates
  * below 2^bits_per_axis, batch indices below 2^batch_bits -- the sort then runs over 3 * bits_per_axis + batch_bits key bits

@@ -272,29 +272,48 @@ def test_non_masked_schedule(gpu_device, stream):
 
 
 def test_private_row_order_is_used_and_equivalent(gpu_device):
-    """Short rows (<= 128 bytes) run on the Z-order-chunked private row order, long rows on the public mask-sorted one;
-    both give the oracle's result (checked by _run_and_check) and agree with each other."""
+    """Short rows (<= 128 bytes) of a large enough map run on the Z-order-chunked private row order once the cache has
+    served a few passes on the public one, long rows always on the public mask-sorted order; both give the oracle's result
+    (checked by _run_and_check) and agree with each other."""
     from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
     res = 24
     coords_np = reference_test_shell(res)
     coords_np = coords_np[np.random.default_rng(0).permutation(len(coords_np))]
     shape = torch.Size([1, 0, res, res, res])
-    _say("private row order: C=32 fp16 (64-byte rows)")
-    cache, _ = _run_and_check(coords_np, shape, 32, 32, torch.float16, gpu_device, seed=21)
-    assert hasattr(cache, "_tile_order")
-    _say("public row order: C=128 fp16 (256-byte rows)")
-    cache2, _ = _run_and_check(coords_np, shape, 128, 128, torch.float16, gpu_device, seed=22)
-    assert not hasattr(cache2, "_tile_order")
-    f, w, b, _ = _case(coords_np, 32, 32, torch.float16, 23)
-    old = impl.LOCALITY_MAX_ROW_BYTES
-    outs = []
+    old = (impl.LOCALITY_MAX_ROW_BYTES, impl.LOCALITY_MIN_ROWS, impl.LOCALITY_AFTER_CALLS)
     try:
+        _say("private row order: a small map stays on the public order")
+        cache0, _ = _run_and_check(coords_np, shape, 32, 32, torch.float16, gpu_device, seed=20)
+        assert not hasattr(cache0, "_tile_order")
+        impl.LOCALITY_MIN_ROWS, impl.LOCALITY_AFTER_CALLS = 0, 0
+        _say("private row order: C=32 fp16 (64-byte rows)")
+        cache, _ = _run_and_check(coords_np, shape, 32, 32, torch.float16, gpu_device, seed=21)
+        assert hasattr(cache, "_tile_order")
+        _say("public row order: C=128 fp16 (256-byte rows)")
+        cache2, _ = _run_and_check(coords_np, shape, 128, 128, torch.float16, gpu_device, seed=22)
+        assert not hasattr(cache2, "_tile_order")
+        f, w, b, _ = _case(coords_np, 32, 32, torch.float16, 23)
+        f, w, b = f.to(gpu_device), w.to(gpu_device).reshape(32, 27, 32), b.to(gpu_device)
+        outs = []
         for limit in (0, 1 << 20):
             impl.LOCALITY_MAX_ROW_BYTES = limit
-            outs.append(impl._gather_gemm(f.to(gpu_device), w.to(gpu_device).reshape(32, 27, 32), b.to(gpu_device), cache, 0, True).float().cpu())
+            fresh = SubMConv3dFunction._compute_neighbor_cache(torch.from_numpy(coords_np).to(gpu_device), shape, (3, 3, 3), (1, 1, 1), False)
+            outs.append(impl._gather_gemm(f, w, b, fresh, 0, True).float().cpu())
+            assert hasattr(fresh, "_tile_order") == (limit > 0)
+        assert eg.max_rel_err(outs[0], outs[1].double()) <= 2e-3
+        # the order comes when the cache has served LOCALITY_AFTER_CALLS short-row passes on the public one, and changes
+        # no result beyond the rounding of a different tile split
+        _say("private row order: made at the third pass of a cache")
+        impl.LOCALITY_MAX_ROW_BYTES, impl.LOCALITY_AFTER_CALLS = old[0], 2
+        late = SubMConv3dFunction._compute_neighbor_cache(torch.from_numpy(coords_np).to(gpu_device), shape, (3, 3, 3), (1, 1, 1), False)
+        seen = []
+        for call in range(4):
+            seen.append(impl._gather_gemm(f, w, b, late, 0, True).float().cpu())
+            assert hasattr(late, "_tile_order") == (call >= 2), call
+        assert torch.equal(seen[0], seen[1]) and torch.equal(seen[2], seen[3])
+        assert eg.max_rel_err(seen[0], seen[2].double()) <= 2e-3
     finally:
-        impl.LOCALITY_MAX_ROW_BYTES = old
-    assert eg.max_rel_err(outs[0], outs[1].double()) <= 2e-3
+        impl.LOCALITY_MAX_ROW_BYTES, impl.LOCALITY_MIN_ROWS, impl.LOCALITY_AFTER_CALLS = old
 
 
 def test_forced_splitk_matches_unsplit(gpu_device):
