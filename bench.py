@@ -217,8 +217,9 @@ def main():
 
             def hook(name, stream):
                 e = torch.cuda.Event(enable_timing=True)
-                e.record(torch.cuda.current_stream())
-                marks.append((name, e))
+                cur = torch.cuda.current_stream()
+                e.record(cur)
+                marks.append((name, e, cur.cuda_stream))
 
             gap = "between calls (host: allocations, read-backs)"
             runs = []
@@ -231,8 +232,12 @@ def main():
                         SubMConv3dFunction._sparse_submanifold_conv_forward(feats, fresh, weight, bias)
                     torch.cuda.synchronize()
                     once = {}
-                    for (name, e0), (_, e1) in zip(marks[:-1], marks[1:]):
-                        once[name or gap] = once.get(name or gap, 0.0) + e0.elapsed_time(e1)
+                    # a phase lasts until the next mark on its own stream (the pair lists of a training cache are made
+                    # on a second stream, beside the mask sort)
+                    for sid in {m[2] for m in marks}:
+                        mine = [m for m in marks if m[2] == sid]
+                        for (name, e0, _), (_, e1, _) in zip(mine[:-1], mine[1:]):
+                            once[name or gap] = once.get(name or gap, 0.0) + e0.elapsed_time(e1)
                     runs.append(once)
             finally:
                 nat.set_phase_hook(None)
