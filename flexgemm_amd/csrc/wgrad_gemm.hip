@@ -64,8 +64,8 @@ struct WgradCfg {
     static_assert((kStages - 2) * LPS < 64, "outstanding loads exceed the vmcnt range");
     // XOR key on the 16-byte chunk index: the transposing read touches 4 consecutive pair rows x 32 bytes, which
     // must fall into distinct bank groups
-    static constexpr int key_a(int row) { return ES == 2 && CH_A >= 8 ? 2 * (row & 3) : 0; }
-    static constexpr int key_b(int row) { return ES == 2 && CH_B >= 8 ? 2 * (row & 3) : 0; }
+    static constexpr int key_a(int row) { return ES != 2 ? 0 : (CH_A >= 16 ? 4 * (row & 3) : (CH_A >= 8 ? 2 * (row & 3) : 0)); }
+    static constexpr int key_b(int row) { return ES != 2 ? 0 : (CH_B >= 16 ? 4 * (row & 3) : (CH_B >= 8 ? 2 * (row & 3) : 0)); }
 };
 
 template <typename Tag, int BM, int BN, int WAVES_M, int WAVES_N>
@@ -336,8 +336,8 @@ struct WStreamCfg {
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
     static_assert(P % (RPI_A * NL) == 0 && P % (RPI_B * NL) == 0, "every loader issues the same row loads");
     static_assert(2 * (LPS + 1) < 64, "outstanding loads exceed the vmcnt range");
-    static constexpr int key_a(int row) { return CH_A >= 8 ? 2 * (row & 3) : 0; }
-    static constexpr int key_b(int row) { return CH_B >= 8 ? 2 * (row & 3) : 0; }
+    static constexpr int key_a(int row) { return CH_A >= 16 ? 4 * (row & 3) : (CH_A >= 8 ? 2 * (row & 3) : 0); }
+    static constexpr int key_b(int row) { return CH_B >= 16 ? 4 * (row & 3) : (CH_B >= 8 ? 2 * (row & 3) : 0); }
 };
 
 template <typename Tag, int BM, int BN>

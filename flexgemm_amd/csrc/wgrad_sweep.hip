@@ -435,8 +435,8 @@ struct SweepCfg {
     static_assert(ES == 2, "16-bit types");
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
     static_assert(P % (RPI_A * NL) == 0 && P % (RPI_B * NL) == 0, "every loader issues the same row loads");
-    static constexpr int key_a(int row) { return CH_A >= 8 ? 2 * (row & 3) : 0; }
-    static constexpr int key_b(int row) { return CH_B >= 8 ? 2 * (row & 3) : 0; }
+    static constexpr int key_a(int row) { return CH_A >= 16 ? 4 * (row & 3) : (CH_A >= 8 ? 2 * (row & 3) : 0); }
+    static constexpr int key_b(int row) { return CH_B >= 16 ? 4 * (row & 3) : (CH_B >= 8 ? 2 * (row & 3) : 0); }
 };
 
 template <typename Tag, int BM, int BN>
