@@ -303,6 +303,43 @@ def test_private_tile_order(gpu_device, res, batch, shuffle):
     assert np.array_equal(_np(cache.valid_kernel_seg_callback(128)), seg)
 
 
+def test_locality_order_over_the_grid_bits_equals_the_order_over_all_bits(gpu_device):
+    """fgx_locality_order_grid sorts over the key bits a grid can differ in (on 32-bit keys when they fit): the same
+    permutation as fgx_locality_order, which sorts over 16 bits per axis and 16 batch bits -- for a grid whose keys fit 32
+    bits, one that needs 64, chunks of one rank (the curve's own order, also fgx_zorder_rows) and a handful of rows."""
+    L = nat.lib()
+    rng = np.random.default_rng(11)
+    cases = [("32-bit keys", 3, 200, 9000, 8, 2, 512), ("64-bit keys", 5, 3000, 9000, 12, 3, 512),
+             ("chunks of one rank", 2, 100, 5000, 7, 1, 1), ("five rows", 1, 64, 5, 6, 0, 8192)]
+    for name, batch, res, n, bits, batch_bits, chunk in cases:
+        _say(f"locality order over the grid's key bits: {name}")
+        cn = np.concatenate([rng.integers(0, batch, (n, 1)), rng.integers(0, res, (n, 3))], axis=1).astype(np.int32)
+        cn = np.unique(cn, axis=0)[rng.permutation(len(np.unique(cn, axis=0)))]
+        n = len(cn)
+        coords = torch.from_numpy(np.ascontiguousarray(cn)).to(gpu_device)
+        binary = torch.from_numpy(rng.integers(0, 1 << 27, n).astype(np.int32)).to(gpu_device)
+        with torch.cuda.device(gpu_device):
+            ws = nat.workspace(L.fgx_locality_workspace_bytes(nat.sz(n)), gpu_device)
+            wide = torch.empty((n,), dtype=torch.int64, device=gpu_device)
+            tight = torch.empty_like(wide)
+            nat.check(L.fgx_locality_order(nat.ptr(coords), nat.ptr(binary), nat.sz(n), C.c_int(27), C.c_int(chunk), nat.ptr(wide),
+                                           nat.ptr(ws), nat.sz(ws.numel()), nat.stream()))
+            nat.check(L.fgx_locality_order_grid(nat.ptr(coords), nat.ptr(binary), nat.sz(n), C.c_int(27), C.c_int(chunk),
+                                                C.c_int(bits), C.c_int(batch_bits), nat.ptr(tight), nat.ptr(ws), nat.sz(ws.numel()),
+                                                nat.stream()))
+            assert torch.equal(wide, tight), name
+            if chunk == 1:
+                rows = torch.empty_like(wide)
+                nat.check(L.fgx_zorder_rows(nat.ptr(coords), nat.sz(n), C.c_int(bits), C.c_int(batch_bits), nat.ptr(rows), nat.ptr(ws),
+                                            nat.sz(ws.numel()), nat.stream()))
+                assert torch.equal(wide, rows), name
+        order = _np(wide)
+        assert np.array_equal(np.sort(order), np.arange(n))
+        rank_order = np.argsort(_morton_keys(cn), kind="stable")
+        key = (np.arange(n) // chunk).astype(np.int64) << 32 | _np(binary).astype(np.int64)[rank_order]
+        assert np.array_equal(order, rank_order[np.argsort(key, kind="stable")]), name
+
+
 def test_sorted_builder_decides_the_key_sort_on_the_device(gpu_device, neighbor_map_builder):
     """fgx_subm_neighbor_map_sorted with presorted = 2 (what the cache builder passes) against presorted = 0 (always
     sort) and, where it applies, presorted = 1: coordinates in scan order, shuffled, in scan order but for the last two
