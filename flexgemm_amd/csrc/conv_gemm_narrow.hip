@@ -41,20 +41,26 @@ __global__ void __launch_bounds__(256) narrow_plan_kernel(const uint32_t* __rest
     __shared__ uint16_t slot_of[kNarrowHash];
     __shared__ uint32_t scan[256];
     __shared__ uint32_t row_flags[kNarrowRows / 32];
+    __shared__ uint32_t grow_of[kNarrowRows];                                       // the chunk's rows (FGX_EMPTY32 beyond n)
+    __shared__ __attribute__((aligned(16))) uint16_t table_lds[kNarrowRows * kNarrowTableStride];   // leaves as 16-byte stores
     const int tid = threadIdx.x;
     const uint32_t chunk = blockIdx.x;
     unsigned char* mine = plan + kNarrowHeader + (size_t)chunk * kNarrowPlanStride;
-    uint16_t* table = (uint16_t*)mine;
     uint32_t* sources = (uint32_t*)(mine + kNarrowTableBytes);
     uint32_t* rows = sources + kNarrowSlots;
     for (int i = tid; i < kNarrowHash; i += 256) keys[i] = FGX_EMPTY32;
     if (tid < kNarrowRows / 32) row_flags[tid] = 0u;
+    for (int r = tid; r < kNarrowRows; r += 256) {
+        const uint32_t gr = chunk * kNarrowRows + (uint32_t)r;
+        grow_of[r] = gr < n ? (order ? (uint32_t)order[gr] : gr) : FGX_EMPTY32;
+    }
+    // entries from V on: the row of zeros (entry 31, the row's overflow flag, is written at the end)
+    for (int i = tid; i < kNarrowRows * kNarrowTableStride; i += 256) table_lds[i] = (uint16_t)(kNarrowZeroSlot * 64u);
     __syncthreads();
     const int entries = kNarrowRows * V;
     auto source_of = [&](int e) -> uint32_t {
-        const uint32_t r = chunk * kNarrowRows + (uint32_t)(e / V);
-        if (r >= n) return FGX_EMPTY32;
-        const uint32_t grow = order ? (uint32_t)order[r] : r;
+        const uint32_t grow = grow_of[e / V];
+        if (grow == FGX_EMPTY32) return FGX_EMPTY32;
         return nmap[(size_t)grow * V + (e % V)];
     };
     auto hash = [](uint32_t x) -> uint32_t { return (x * 2654435761u) >> 22; };      // 10 bits
@@ -75,31 +81,30 @@ __global__ void __launch_bounds__(256) narrow_plan_kernel(const uint32_t* __rest
     __syncthreads();
     if (own_rows) {
         for (int r = tid; r < kNarrowRows; r += 256) {
-            const uint32_t gr = chunk * kNarrowRows + (uint32_t)r;
-            if (gr < n) {
-                const int pos = insert(order ? (uint32_t)order[gr] : gr);
+            if (grow_of[r] != FGX_EMPTY32) {
+                const int pos = insert(grow_of[r]);
                 if (pos >= 0) slot_of[pos] = (uint16_t)r;
             }
         }
         __syncthreads();
     }
-    // (a thread's entries stay in registers for the second pass: kNarrowRows * kNarrowMaxV / 256 of them at most)
+    // (a thread's entries stay in registers for the second pass: kNarrowRows * kNarrowMaxV / 256 of them at most; all
+    // of them are fetched before the first goes into the table, so that their latencies overlap)
     constexpr int kPerThread = (kNarrowRows * 32 + 255) / 256;
     uint32_t mine_idx[kPerThread];
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j) {
         const int e = tid + j * 256;
         mine_idx[j] = e < entries ? source_of(e) : FGX_EMPTY32;
-        if (mine_idx[j] != FGX_EMPTY32) insert(mine_idx[j]);
     }
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j)
+        if (mine_idx[j] != FGX_EMPTY32) insert(mine_idx[j]);
     __syncthreads();
     // the other sources: slots from `base` on in table order (exclusive scan of their positions, four per thread)
     const uint32_t base = own_rows ? (uint32_t)kNarrowRows : 0u;
     if (own_rows) {
-        for (int r = tid; r < kNarrowRows; r += 256) {
-            const uint32_t gr = chunk * kNarrowRows + (uint32_t)r;
-            sources[r] = gr < n ? (order ? (uint32_t)order[gr] : gr) : FGX_EMPTY32;
-        }
+        for (int r = tid; r < kNarrowRows; r += 256) sources[r] = grow_of[r];
     }
     uint32_t own = 0;
     for (int j = 0; j < 4; ++j) own += (keys[tid * 4 + j] != FGX_EMPTY32 && slot_of[tid * 4 + j] == kNarrowOverflow) ? 1u : 0u;
@@ -143,18 +148,19 @@ __global__ void __launch_bounds__(256) narrow_plan_kernel(const uint32_t* __rest
         }
         // what the multipliers read: the byte offset of the row's logical piece 0 in the row buffer
         if (out != (uint16_t)kNarrowOverflow) out = (uint16_t)(out * 64u + (((uint32_t)out >> 2) & 3u) * 16u);
-        table[(e / V) * kNarrowTableStride + (e % V)] = out;
+        table_lds[(e / V) * kNarrowTableStride + (e % V)] = out;
         if (out == (uint16_t)kNarrowOverflow) atomicOr(&row_flags[(e / V) >> 5], 1u << ((e / V) & 31));
     }
     __syncthreads();
-    for (int r = tid; r < kNarrowRows; r += 256) {
-        table[r * kNarrowTableStride + kNarrowTableStride - 1] = (uint16_t)((row_flags[r >> 5] >> (r & 31)) & 1u);
-        for (int v = V; v < kNarrowTableStride - 1; ++v) table[r * kNarrowTableStride + v] = (uint16_t)(kNarrowZeroSlot * 64u);
-    }
+    for (int r = tid; r < kNarrowRows; r += 256)
+        table_lds[r * kNarrowTableStride + kNarrowTableStride - 1] = (uint16_t)((row_flags[r >> 5] >> (r & 31)) & 1u);
     if (tid == 0 && (row_flags[0] | row_flags[1] | row_flags[2] | row_flags[3]) != 0u) atomicAdd((uint32_t*)plan, 1u);
-    for (int r = tid; r < kNarrowRows; r += 256) {
-        const uint32_t g = chunk * kNarrowRows + (uint32_t)r;
-        rows[r] = g < n ? (order ? (uint32_t)order[g] : g) : FGX_EMPTY32;
+    for (int r = tid; r < kNarrowRows; r += 256) rows[r] = grow_of[r];
+    __syncthreads();
+    {
+        const uint4* from = (const uint4*)table_lds;
+        uint4* to = (uint4*)mine;                       // (the plan and its chunks are 16-byte aligned)
+        for (int i = tid; i < kNarrowTableBytes / 16; i += 256) to[i] = from[i];
     }
 }
 

@@ -53,8 +53,8 @@ SORT_BUILDER_MIN_PROBES = 27 * 131072
 GEMM_ITEM_ORDER = "auto"
 # Narrow layers (16-bit, 8 ... 32 channels on both sides, submanifold): the gather GEMM that keeps a chunk's source rows
 # resident in LDS (fgx_conv_narrow_gemm; 0.32 -> 0.19 ms per pass at 2.67 M voxels x 32 channels).  "auto": from 32 768
-# rows on, once a neighbor cache has served five such products on the streaming kernel (the plan it needs costs two thirds
-# of building the cache; a cache made for training with half a million voxels and more gets it at its second product,
+# rows on, once a neighbor cache has served three such products on the streaming kernel (sixteen below half a million
+# rows: the plan it needs costs half of building the cache; a cache made for training with half a million voxels and more gets it at its second product,
 # because the weight gradients gain the most); "on": whenever it fits; "off": never.
 NARROW_RESIDENT = "auto"
 # The bias gradient of a submanifold layer comes out of the streaming wgrad kernel (which loads every grad_output row for

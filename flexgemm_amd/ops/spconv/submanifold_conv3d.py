@@ -702,13 +702,17 @@ def _narrow_applies(cache, src: torch.Tensor, k: int, cols: int, v: int, n: int,
         return False                    # no plan is made inside a graph capture (it would be remade on every replay)
     if mode == "on":
         return True
-    # "auto": the plan costs two thirds of a neighbor-cache build (0.66 ms for 2.7 M voxels) and a call gains 0.1 ms on
-    # it, so a cache gets one once it has served NARROW_RESIDENT_AFTER_CALLS narrow products on the streaming kernel (what
-    # the plan costs in passes): whatever happens next, the detour then costs at most what the calls before it did.
+    # "auto": the plan costs half of a neighbor-cache build (0.48 ms for 2.7 M voxels, 0.16 ms for 252 k) and a call
+    # gains 0.2 - 0.3 ms on it at 2.7 M voxels (0.39 - 0.51 ms on the streaming kernel over the public row order, 0.195 ms
+    # here) but 0.01 ms at 252 k, so a cache gets one once it has served what the plan costs in passes on the streaming
+    # kernel -- NARROW_RESIDENT_AFTER_CALLS of them, NARROW_RESIDENT_AFTER_CALLS_SMALL below half a million rows:
+    # whatever happens next, the detour then costs at most what the calls before it did.
     if n < NARROW_RESIDENT_MIN_ROWS:
         return False
     calls = getattr(cache, "_narrow_calls", 0) + 1
     cache["_narrow_calls"] = calls
+    if n < NARROW_RESIDENT_TRAINING_MIN_ROWS:
+        return calls > NARROW_RESIDENT_AFTER_CALLS_SMALL
     # A cache made for training also serves weight gradients, which gain three times what a forward pass does (0.66 ->
     # 0.26 ms at 2.67 M voxels): with half a million voxels and more its plan pays from the second layer on, so it comes
     # at the second product (a single layer never asks for one).
@@ -750,8 +754,10 @@ def _sweep_fits(n: int, n_in: int, ci: int, co: int, elem_bytes: int, n_pairs: i
 
 # Fewest rows from which NARROW_RESIDENT = "auto" takes the resident-row kernel.
 NARROW_RESIDENT_MIN_ROWS = 32768
-# ... and narrow products a neighbor cache serves on the streaming kernel before it gets the plan.
-NARROW_RESIDENT_AFTER_CALLS = 5
+# ... and narrow products a neighbor cache serves on the streaming kernel before it gets the plan (below
+# NARROW_RESIDENT_TRAINING_MIN_ROWS rows: the second number).
+NARROW_RESIDENT_AFTER_CALLS = 3
+NARROW_RESIDENT_AFTER_CALLS_SMALL = 16
 # ... a cache made for training (it will serve weight gradients too) of this many rows and more: after one product.
 NARROW_RESIDENT_TRAINING_MIN_ROWS = 524288
 NARROW_RESIDENT_AFTER_CALLS_TRAINING = 1
