@@ -216,10 +216,11 @@ def main():
             marks = []
 
             def hook(name, stream):
+                # (the stream the library enqueues the phase on: the caller's, or the library's second one)
                 e = torch.cuda.Event(enable_timing=True)
-                cur = torch.cuda.current_stream()
-                e.record(cur)
-                marks.append((name, e, cur.cuda_stream))
+                on = torch.cuda.ExternalStream(stream) if stream else torch.cuda.current_stream()
+                e.record(on)
+                marks.append((name, e, on.cuda_stream))
 
             gap = "between calls (host: allocations, read-backs)"
             runs = []

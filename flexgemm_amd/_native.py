@@ -28,7 +28,7 @@ EXPORTS = [
     "fgx_hash_insert_3d", "fgx_hash_lookup_3d",
     "fgx_subm_neighbor_map", "fgx_subm_neighbor_map_sorted_workspace_bytes", "fgx_subm_neighbor_map_sorted", "fgx_coords_key_order", "fgx_mask_codes",
     "fgx_sort_workspace_bytes", "fgx_sort_by_code", "fgx_locality_workspace_bytes", "fgx_locality_order", "fgx_locality_order_grid",
-    "fgx_pair_workspace_bytes", "fgx_pair_count", "fgx_pair_fill",
+    "fgx_pair_workspace_bytes", "fgx_pair_count", "fgx_pair_fill", "fgx_subm_cache_workspace_bytes", "fgx_subm_cache_build",
     "fgx_tile_workspace_bytes", "fgx_tile_codes", "fgx_tile_fill",
     "fgx_table_lookup", "fgx_weight_panel_bytes", "fgx_pack_weight",
     "fgx_conv_scratch_bytes", "fgx_conv_gather_gemm", "fgx_conv_gather_gemm_act", "fgx_conv_gather_gemm_act_mask",
@@ -104,7 +104,7 @@ def lib() -> C.CDLL:
                      "fgx_colsum_scratch_bytes", "fgx_spconv_out_coords_workspace_bytes",
                      "fgx_subm_neighbor_map_sorted_workspace_bytes", "fgx_wgrad_block_bounds_count", "fgx_wgrad_item_lists_count", "fgx_narrow_plan_bytes", "fgx_narrow_wgrad_scratch_bytes",
                      "fgx_spconv_neighbor_map_sorted_workspace_bytes", "fgx_serialize_reorder_workspace_bytes",
-                     "fgx_gather_item_order_workspace_bytes", "fgx_wgrad_sweep_plan_bytes", "fgx_wgrad_sweep_scratch_bytes", "fgx_wgrad_sweep_giveup_words"):
+                     "fgx_gather_item_order_workspace_bytes", "fgx_subm_cache_workspace_bytes", "fgx_wgrad_sweep_plan_bytes", "fgx_wgrad_sweep_scratch_bytes", "fgx_wgrad_sweep_giveup_words"):
             getattr(L, name).restype = C.c_size_t
         _lib = L
     return _lib

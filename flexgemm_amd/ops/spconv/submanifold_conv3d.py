@@ -444,6 +444,8 @@ def _pair_lists(nmap: torch.Tensor, gray: torch.Tensor, exact: bool = False):
 
 SORT_DECIDED_ON_DEVICE_MAX = 1 << 21     # fgx_subm_neighbor_map_sorted honours presorted = 2 up to this many voxels
 
+# The masked algorithms' cache through one library call (fgx_subm_cache_build) where it applies; False: step by step.
+CACHE_BUILD_ONE_CALL = True
 # from this many voxels on a training cache's pair lists are made on a second stream, beside the mask sort (below, the
 # build waits for the host, and the second stream's events and context cost it 0.07 ms more: 42 608 voxels 0.149 -> 0.222 ms)
 PAIR_LISTS_SIDE_STREAM_MIN_ROWS = 393216
@@ -502,6 +504,61 @@ def _build_neighbor_map(coords: torch.Tensor, shape, kernel_size, dilation, with
             C.c_int(int(dilation[0])), C.c_int(int(dilation[1])), C.c_int(int(dilation[2])),
             nat.ptr(nmap), nat.ptr(gray), nat.ptr(binary), nat.stream()))
     return nmap, gray, binary
+
+
+def _build_cache_one_call(coords: torch.Tensor, shape, kernel_size, dilation, needs_grad: bool):
+    """The masked algorithms' neighbor cache through fgx_subm_cache_build: map, codes, mask sort and (needs_grad) the pair
+    lists enqueued by one library call, with every buffer allocated beforehand -- the GPU does not wait for the host
+    between the steps.  Returns (nmap, gray, binary, order, pairs or None), or None where the call does not apply (the
+    hash builder's range, kernels beyond what the sorted builder takes, pair lists too large to allocate at their bound)
+    and the step-by-step path runs."""
+    n = coords.shape[0]
+    B, _, W, H, D = [int(s) for s in shape]
+    kw, kh, kd = [int(k) for k in kernel_size]
+    v = kw * kh * kd
+    builder = spconv.NEIGHBOR_MAP_BUILDER
+    if builder == "auto":
+        builder = "sort" if n * v >= spconv.SORT_BUILDER_MIN_PROBES else "hash"
+    vol = B * W * H * D
+    bound = n * v
+    if builder != "sort" or n == 0 or v > 32 or kw * kh > 128 or vol > 2 ** 63 or bound >= 0xFFFFFFFF:
+        return None
+    if needs_grad and bound * 8 > PAIR_LISTS_UNSIZED_MAX_BYTES:
+        return None
+    key_bits = 32 if vol <= 2 ** 32 else 64
+    dev = coords.device
+    with torch.cuda.device(dev):
+        L = nat.lib()
+        presorted = 2                       # (as in _build_neighbor_map)
+        if n > SORT_DECIDED_ON_DEVICE_MAX or key_bits != 32:
+            descents = torch.zeros((1,), dtype=torch.int32, device=dev)
+            nat.check(L.fgx_coords_key_order(nat.ptr(coords), nat.sz(n), C.c_int(W), C.c_int(H), C.c_int(D), nat.ptr(descents), nat.stream()))
+            presorted = 1 if int(descents.item()) == 0 else 0
+        nmap = torch.empty((n, v), dtype=torch.uint32, device=dev)
+        gray = torch.empty((n,), dtype=torch.int32, device=dev)
+        binary = torch.empty((n,), dtype=torch.int32, device=dev)
+        order = torch.empty((n,), dtype=torch.int64, device=dev)
+        seg = buf_i = buf_o = None
+        if needs_grad:
+            seg = torch.empty((v + 1,), dtype=torch.uint32, device=dev)
+            buf_i = torch.empty((bound,), dtype=torch.uint32, device=dev)
+            buf_o = torch.empty((bound,), dtype=torch.uint32, device=dev)
+        ws = nat.workspace(L.fgx_subm_cache_workspace_bytes(nat.sz(n), C.c_int(key_bits), C.c_int(kw), C.c_int(kh), C.c_int(kd),
+                                                            C.c_int(1 if needs_grad else 0)), dev)
+        nat.check(L.fgx_subm_cache_build(
+            nat.ptr(coords), nat.sz(n), C.c_int(B), C.c_int(W), C.c_int(H), C.c_int(D), C.c_int(kw), C.c_int(kh), C.c_int(kd),
+            C.c_int(int(dilation[0])), C.c_int(int(dilation[1])), C.c_int(int(dilation[2])), C.c_int(key_bits), C.c_int(presorted),
+            C.c_int(1 if needs_grad else 0), nat.ptr(ws), nat.sz(ws.numel()), nat.ptr(nmap), nat.ptr(gray), nat.ptr(binary),
+            nat.ptr(order), nat.ptr(seg), nat.ptr(buf_i), nat.ptr(buf_o), nat.stream()))
+        pairs = None
+        if needs_grad:
+            # the lists' length travels to pinned host memory behind an event; the cache cuts them to it when first asked
+            seg_pinned = torch.empty((v + 1,), dtype=torch.int32, pin_memory=True)
+            seg_pinned.copy_(seg.view(torch.int32), non_blocking=True)
+            arrived = torch.cuda.Event()
+            arrived.record()
+            pairs = {"seg": seg, "pending": (buf_i, buf_o, seg_pinned, arrived)}
+    return nmap, gray, binary, order, pairs
 
 
 def _pad_cols(t: torch.Tensor, mult: int) -> torch.Tensor:
@@ -901,6 +958,17 @@ class SubMConv3dFunction(Function):
             # pair lists wgrad needs are derived from it on first use
             nmap, _, _ = _build_neighbor_map(coords, shape, kernel_size, dilation, with_codes=False)
             return SubMConv3dNeighborCache(neighbor_map=nmap)
+        built = _build_cache_one_call(coords, shape, kernel_size, dilation, needs_grad) if CACHE_BUILD_ONE_CALL else None
+        if built is not None:
+            nmap, gray, binary, order, pairs = built
+            cache = SubMConv3dNeighborCache(neighbor_map=nmap, gray_code=gray, sorted_idx=order)
+            cache["_coords"] = coords
+            cache["_needs_grad"] = bool(needs_grad)
+            cache["_grid"] = (int(shape[0]), tuple(int(d) for d in shape[2:]))
+            cache["_binary_code"] = binary
+            if needs_grad:
+                cache._attach_pairs(pairs)
+            return cache
         nmap, gray, binary = _build_neighbor_map(coords, shape, kernel_size, dilation, with_codes=True)
         # The pair lists and the mask sort both start from the map and its codes and need nothing of each other: the lists
         # are made on a second stream while the sort runs on the caller's (both are chains of short kernels that leave

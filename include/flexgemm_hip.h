@@ -168,6 +168,20 @@ int fgx_pair_count(const int32_t* gray, size_t n, int V, uint32_t* seg,
 int fgx_pair_fill(const uint32_t* map, const int32_t* gray, size_t n, int V,
                   const void* workspace, uint32_t* sig_i, uint32_t* sig_o, fgx_stream_t stream);
 
+/* The whole neighbor cache of a submanifold convolution in one call: fgx_subm_neighbor_map_sorted (map, gray / binary
+ * codes), fgx_sort_by_code (sorted_idx) and, with_pairs != 0, fgx_pair_count and fgx_pair_fill (seg[V + 1], sig_i / sig_o
+ * with room for one entry per slot of the map, n * V) -- same arguments, same results, nothing between the kernels for
+ * the GPU to wait for.  From 393 216 voxels on the pair lists are enqueued on a second stream of the library's own
+ * (default priority, one per device, made on first use) beside the mask sort, and `stream` waits for it before the call
+ * returns; never during a stream capture.  Kernel volumes up to 32.  workspace: fgx_subm_cache_workspace_bytes bytes,
+ * 256-byte aligned.  Replaces: SubMConv3dFunction._compute_neighbor_cache's sequence of extension calls
+ * (flex_gemm/ops/spconv/submanifold_conv3d.py:46-107: hashmap insert, neighbor map, gray-code sort, kernel_map post-pass). */
+size_t fgx_subm_cache_workspace_bytes(size_t n, int key_bits, int Kw, int Kh, int Kd, int with_pairs);
+int fgx_subm_cache_build(const int32_t* coords, size_t n, int B, int W, int H, int D, int Kw, int Kh, int Kd, int Dw, int Dh, int Dd,
+                         int key_bits, int presorted, int with_pairs, void* workspace, size_t workspace_bytes, uint32_t* out_map,
+                         int32_t* gray, int32_t* binary, int64_t* sorted_idx, uint32_t* seg, uint32_t* sig_i, uint32_t* sig_o,
+                         fgx_stream_t stream);
+
 /* Per row-tile (block consecutive rows of the sorted order) OR of the masks.
  *   codes: tile_code[nb] <- OR mask, seg[nb+1] <- exclusive offsets of popcounts (seg[nb] = total);
  *   fill : valid_kernel[total] <- set-bit positions, ascending per tile.

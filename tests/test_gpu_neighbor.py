@@ -303,6 +303,43 @@ def test_private_tile_order(gpu_device, res, batch, shuffle):
     assert np.array_equal(_np(cache.valid_kernel_seg_callback(128)), seg)
 
 
+def test_cache_built_by_one_call_equals_the_cache_built_step_by_step(gpu_device):
+    """fgx_subm_cache_build (map, codes, mask sort and pair lists enqueued by one call, the lists on the library's second
+    stream from 393 216 voxels on) against the same cache made call by call: every public field equal, for training and
+    inference caches, coordinates in scan order and shuffled, a dilated kernel, sizes on both sides of the second
+    stream's threshold, and twice in a row (the second build reuses the first one's freed buffers)."""
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    rng = np.random.default_rng(3)
+    cases = [("res 96 shuffled, training", reference_test_shell(96), 96, (3, 3, 3), (1, 1, 1), True, True),
+             ("res 96, inference", reference_test_shell(96), 96, (3, 3, 3), (1, 1, 1), False, False),
+             ("res 64 dilated 3 x 1 x 3", reference_test_shell(64), 64, (3, 1, 3), (2, 1, 2), True, True),
+             ("res 448, training (two streams)", reference_test_shell(448), 448, (3, 3, 3), (1, 1, 1), True, False),
+             ("res 448 shuffled, training (two streams)", reference_test_shell(448), 448, (3, 3, 3), (1, 1, 1), True, True)]
+    old = (impl.CACHE_BUILD_ONE_CALL, flex_gemm.ops.spconv.NEIGHBOR_MAP_BUILDER if hasattr(flex_gemm.ops.spconv, "NEIGHBOR_MAP_BUILDER") else None)
+    flex_gemm.ops.spconv.set_neighbor_map_builder("sort")
+    try:
+        for name, cn, res, ks, dil, grad, shuffle in cases:
+            _say(f"cache by one call: {name} (n={len(cn)})")
+            if shuffle:
+                cn = cn[rng.permutation(len(cn))]
+            coords = torch.from_numpy(np.ascontiguousarray(cn)).to(gpu_device)
+            shape = torch.Size([1, 0, res, res, res])
+            for rep in range(2):
+                impl.CACHE_BUILD_ONE_CALL = False
+                ref = SubMConv3dFunction._compute_neighbor_cache(coords, shape, ks, dil, grad)
+                impl.CACHE_BUILD_ONE_CALL = True
+                got = SubMConv3dFunction._compute_neighbor_cache(coords, shape, ks, dil, grad)
+                fields = ["neighbor_map", "gray_code", "sorted_idx"] + (["valid_signal_seg", "valid_signal_i", "valid_signal_o"] if grad else [])
+                for f in fields:
+                    a, b = getattr(ref, f), getattr(got, f)
+                    assert a.shape == b.shape and a.dtype == b.dtype, (name, f)
+                    assert torch.equal(a.view(torch.int32) if a.dtype == torch.uint32 else a, b.view(torch.int32) if b.dtype == torch.uint32 else b), (name, f, rep)
+                del ref, got
+    finally:
+        impl.CACHE_BUILD_ONE_CALL = old[0]
+        flex_gemm.ops.spconv.set_neighbor_map_builder("auto")
+
+
 def test_locality_order_over_the_grid_bits_equals_the_order_over_all_bits(gpu_device):
     """fgx_locality_order_grid sorts over the key bits a grid can differ in (on 32-bit keys when they fit): the same
     permutation as fgx_locality_order, which sorts over 16 bits per axis and 16 batch bits -- for a grid whose keys fit 32
