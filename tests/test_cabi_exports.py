@@ -147,6 +147,40 @@ def test_argument_errors_map_to_exceptions(library):
     assert b"activation" in L.fgx_last_error()
 
 
+def test_entry_points_of_the_resident_row_kernels_and_the_one_call_cache_check_their_arguments(library):
+    L = nat.lib()
+    sz = ctypes.c_size_t
+    # sizes: pure functions of their arguments
+    assert L.fgx_narrow_plan_bytes(sz(0), 27) == 256 and L.fgx_narrow_plan_bytes(sz(129), 27) == 256 + 2 * 10496
+    assert L.fgx_narrow_plan_bytes(sz(128), 32) == 0                      # kernel volumes up to 31
+    assert L.fgx_subm_cache_workspace_bytes(sz(1000), 32, 3, 3, 3, 1) >= L.fgx_subm_cache_workspace_bytes(sz(1000), 32, 3, 3, 3, 0) > 0
+    assert L.fgx_subm_cache_workspace_bytes(sz(1000), 16, 3, 3, 3, 1) == 0 and L.fgx_subm_cache_workspace_bytes(sz(1000), 32, 3, 3, 5, 1) == 0
+    with pytest.raises(ValueError):   # a kernel volume the mask codes cannot hold
+        nat.check(L.fgx_subm_cache_build(None, sz(10), 1, 8, 8, 8, 3, 3, 5, 1, 1, 1, 32, 2, 0, None, sz(0), None, None, None, None,
+                                         None, None, None, None))
+    assert b"kernel volume" in L.fgx_last_error()
+    with pytest.raises(ValueError):   # pair lists without a segment table
+        nat.check(L.fgx_subm_cache_build(None, sz(10), 1, 8, 8, 8, 3, 3, 3, 1, 1, 1, 32, 2, 1, None, sz(0), None, None, None, None,
+                                         None, None, None, None))
+    assert b"segment table" in L.fgx_last_error()
+    with pytest.raises(ValueError):
+        nat.check(L.fgx_subm_cache_build(None, sz(10), 1, 8, 8, 8, 3, 3, 3, 1, 1, 1, 32, 2, 0, None, sz(0), None, None, None, None,
+                                         None, None, None, None))
+    assert b"null buffer" in L.fgx_last_error()
+    with pytest.raises(ValueError):   # channel counts the resident-row GEMM does not take
+        nat.check(L.fgx_conv_narrow_gemm(0, None, None, None, None, None, sz(10), sz(10), 48, 32, 27, 0, None, None, None))
+    assert b"8, 16, 24 or 32" in L.fgx_last_error()
+    with pytest.raises(ValueError):
+        nat.check(L.fgx_conv_narrow_gemm(2, None, None, None, None, None, sz(10), sz(10), 32, 32, 27, 0, None, None, None))
+    assert b"16-bit" in L.fgx_last_error()
+    with pytest.raises(ValueError):
+        nat.check(L.fgx_locality_order_grid(None, None, sz(10), 27, 8192, 17, 0, None, None, sz(0), None))
+    assert b"bits per axis" in L.fgx_last_error()
+    with pytest.raises(ValueError):
+        nat.check(L.fgx_zorder_rows(None, sz(10), 16, 17, None, None, sz(0), None))
+    assert b"64-bit key" in L.fgx_last_error()
+
+
 def test_host_logic_without_gpu():
     import torch
     import flex_gemm
