@@ -194,12 +194,22 @@ __global__ void __launch_bounds__(64 * kXcds) sweep_units_kernel(const uint32_t*
     // what the layout pass below needs of every unit (steps, offset), kept out of global memory
     __shared__ uint32_t sh_steps[kSwMaxGroups * 2];
     __shared__ uint8_t sh_v[kSwMaxGroups * 2];
-    __shared__ uint32_t sh_vcount[kMaxV];
     const bool by_pairs = nsb <= kSwCumMax;
     if (by_pairs) {
+        // (eight offsets' counts fetched together: a loop over a run-time V waits for every load in turn)
         for (unsigned sb = x; sb <= nsb; sb += blockDim.x) {
             uint32_t c = 0;
-            for (int v = 0; v < V; ++v) c += fine[(size_t)v * (nsb + 1) + sb] - fine[(size_t)v * (nsb + 1)];
+            for (int v0 = 0; v0 < V; v0 += 8) {
+                uint32_t at[8], first[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const int v = v0 + k < V ? v0 + k : V - 1;
+                    at[k] = fine[(size_t)v * (nsb + 1) + sb];
+                    first[k] = fine[(size_t)v * (nsb + 1)];
+                }
+#pragma unroll
+                for (int k = 0; k < 8; ++k) c += v0 + k < V ? at[k] - first[k] : 0u;
+            }
             cum[sb] = c;
         }
     }
@@ -305,33 +315,85 @@ __global__ void __launch_bounds__(64 * kXcds) sweep_units_kernel(const uint32_t*
         }
     }
     __syncthreads();
-    // step-list offsets: a running sum over the workgroups (thread 0, from LDS); the rest in parallel
+    // step-list offsets: an exclusive running sum over the workgroups' step counts (wavefront 0: 64 lanes x up to 8
+    // workgroups each, a shuffle scan across the lanes); active workgroups per XCD: a count per wavefront
     __shared__ uint32_t sh_off[kSwMaxGroups + 1];
-    if (x == 0) {
-        uint32_t off = 0;
-        for (unsigned g = 0; g < (unsigned)kXcds * spx; ++g) {
-            sh_off[g] = off;
-            off += sh_steps[g * 2] + sh_steps[g * 2 + 1];
+    __shared__ uint32_t sh_active[kXcds];
+    const unsigned groups = (unsigned)kXcds * spx;
+    {
+        const unsigned lane = x & 63u;
+        if (x < 64u) {
+            constexpr unsigned kPer = kSwMaxGroups / 64;
+            uint32_t mine[kPer], sum = 0;
+#pragma unroll
+            for (unsigned k = 0; k < kPer; ++k) {
+                const unsigned g = lane * kPer + k;
+                mine[k] = g < groups ? sh_steps[g * 2] + sh_steps[g * 2 + 1] : 0u;
+                sum += mine[k];
+            }
+            uint32_t incl = sum;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const uint32_t up = __shfl_up(incl, d, 64);
+                if ((int)lane >= d) incl += up;
+            }
+            uint32_t off = incl - sum;
+#pragma unroll
+            for (unsigned k = 0; k < kPer; ++k) {
+                const unsigned g = lane * kPer + k;
+                if (g < groups) sh_off[g] = off;
+                off += mine[k];
+            }
         }
+        // wavefront xc counts XCD xc's workgroups that have steps (spx <= 64)
+        const unsigned xc = x >> 6;
+        const bool has = lane < spx && (sh_steps[(xc * spx + lane) * 2] + sh_steps[(xc * spx + lane) * 2 + 1]) != 0u;
+        const unsigned long long mask = __ballot(has);
+        if (lane == 0) sh_active[xc] = (uint32_t)__popcll(mask);
     }
-    if (x < (unsigned)kMaxV) sh_vcount[x] = 0;
     __syncthreads();
-    for (unsigned g = x; g < (unsigned)kXcds * spx; g += blockDim.x) {
-        const unsigned xc = g / spx;
-        uint32_t active = 0;
-        for (unsigned s = 0; s < spx; ++s) active += (sh_steps[(xc * spx + s) * 2] + sh_steps[(xc * spx + s) * 2 + 1]) ? 1u : 0u;
+    for (unsigned g = x; g < groups; g += blockDim.x) {
         wg[g].step_off = sh_off[g];
         wg[g].nsteps = sh_steps[g * 2] + sh_steps[g * 2 + 1];
-        wg[g].active = active;
+        wg[g].active = sh_active[g / spx];
     }
-    // the partial products of every offset, in ascending unit order (the reduction adds them in this order): thread v
-    // collects offset v's
-    const unsigned total_units = kXcds * spx * 2;
-    if (x < (unsigned)V) {
+    // the partial products of every offset, in ascending unit order (the reduction adds them in this order): a unit's
+    // place in its offset's list is the number of units of that offset before it -- counted per wavefront with a ballot
+    // per offset, the wavefronts' counts added up in order
+    const unsigned total_units = groups * 2;
+    __shared__ uint16_t sh_cnt[kMaxV][(kSwMaxGroups * 2) / 64];       // [offset][run of 64 units]
+    const unsigned runs = (total_units + 63u) / 64u;
+    for (unsigned r0 = 0; r0 < runs; r0 += blockDim.x / 64) {
+        const unsigned run = r0 + (x >> 6), q = run * 64 + (x & 63u);
+        const bool live = run < runs && q < total_units && sh_steps[q] != 0u;
+        const int mine_v = live ? (int)sh_v[q] : -1;
+        for (int v = 0; v < V; ++v) {
+            const unsigned long long m = __ballot(mine_v == v);
+            if ((x & 63u) == 0 && run < runs) sh_cnt[v][run] = (uint16_t)__popcll(m);
+        }
+    }
+    __syncthreads();
+    if (x < (unsigned)V) {                 // exclusive sums over the runs, in place; the total is the offset's count
         uint32_t c = 0;
-        for (unsigned q = 0; q < total_units; ++q)
-            if (sh_steps[q] && sh_v[q] == x) vlist[(size_t)x * total_units + c++] = (uint16_t)q;
+        for (unsigned run = 0; run < runs; ++run) {
+            const uint32_t here = sh_cnt[x][run];
+            sh_cnt[x][run] = (uint16_t)c;
+            c += here;
+        }
         vcount[x] = c;
+    }
+    __syncthreads();
+    for (unsigned r0 = 0; r0 < runs; r0 += blockDim.x / 64) {
+        const unsigned run = r0 + (x >> 6), q = run * 64 + (x & 63u);
+        const bool live = run < runs && q < total_units && sh_steps[q] != 0u;
+        const int mine_v = live ? (int)sh_v[q] : -1;
+        for (int v = 0; v < V; ++v) {
+            const unsigned long long m = __ballot(mine_v == v);
+            if (mine_v == v) {
+                const unsigned before = (unsigned)__popcll(m & ((1ull << (x & 63u)) - 1ull));
+                vlist[(size_t)v * total_units + sh_cnt[v][run] + before] = (uint16_t)q;
+            }
+        }
     }
 }
 
