@@ -272,10 +272,9 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
         for (int i = 0; i < C::A_PER; ++i) {
             // 32-row band of this load's rows (a constant when the loaders' loads of one round make up one band)
             const int band = C::NL * C::ROWS_PER_INST == 32 ? i : ((i * C::NL + lw) * C::ROWS_PER_INST) >> 5;
-            // a multiplier wavefront skips all TM bands of its tile or none, so the loaders skip on the same groups:
-            // no row of the group has the offset -> nothing to load, and the stage keeps stale data nobody reads
-            constexpr uint32_t kWaveBands = (1u << C::TM) - 1u;
-            if (!((cur_band >> (band / C::TM * C::TM)) & kWaveBands)) continue;
+            // the multipliers skip a band none of whose rows has the offset, so the loaders skip it too: nothing to load,
+            // and the stage keeps stale data nobody reads
+            if (!((cur_band >> band) & 1u)) continue;
             uint32_t vo = a_voff[i];
             if (tail) vo = a_soff + a_choff[i] < row_bytes ? vo : kOobOffset;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(src_rs, FGX_LDS_PTR(stage + (i * C::NL + lw) * 1024), 16, vo, a_soff, 0, 0);
@@ -417,20 +416,27 @@ gather_gemm_stream_kernel(const typename Tag::type* __restrict__ src, const type
                 m_ring = (m_ring + 1) & (kBandSlots - 1);
             }
             if (m_mine != 0) {
+                // band by band: a 32-row band of the wave tile none of whose rows has the offset is neither read nor
+                // multiplied (for a given accumulator the products still come in the order of the K-blocks)
                 u32x4 af[kChunks / 2][C::TM], bf[kChunks / 2][C::TN];
-#pragma unroll
-                for (int kk = 0; kk < kChunks / 2; ++kk) {
-#pragma unroll
-                    for (int i = 0; i < C::TM; ++i) af[kk][i] = *(const u32x4*)(cur + a_frag[kk][i]);
-#pragma unroll
-                    for (int j = 0; j < C::TN; ++j) bf[kk][j] = *(const u32x4*)(cur + b_frag[kk][j]);
-                }
 #pragma unroll
                 for (int kk = 0; kk < kChunks / 2; ++kk)
 #pragma unroll
-                    for (int i = 0; i < C::TM; ++i)
+                    for (int j = 0; j < C::TN; ++j) bf[kk][j] = *(const u32x4*)(cur + b_frag[kk][j]);
+#pragma unroll
+                for (int i = 0; i < C::TM; ++i) {
+                    if (C::TM > 1 && !((m_mine >> i) & 1u)) continue;
+#pragma unroll
+                    for (int kk = 0; kk < kChunks / 2; ++kk) af[kk][i] = *(const u32x4*)(cur + a_frag[kk][i]);
+                }
+#pragma unroll
+                for (int i = 0; i < C::TM; ++i) {
+                    if (C::TM > 1 && !((m_mine >> i) & 1u)) continue;
+#pragma unroll
+                    for (int kk = 0; kk < kChunks / 2; ++kk)
 #pragma unroll
                         for (int j = 0; j < C::TN; ++j) mma<Tag>(acc[i][j], bf[kk][j], af[kk][i]);   // transposed tile
+                }
             }
         }
 
