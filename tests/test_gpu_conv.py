@@ -820,6 +820,7 @@ def _full_size_check(wl, dt, sample, dev, seed):
     scale = float((conv_nobias.abs() * g64.abs()).sum())
     assert abs(lhs - mid) / scale < 1e-3 and abs(lhs - rhs) / scale < 1e-3
     _assert_close(b.grad, g64.sum(0), dt, "dbias")
+    return cache
 
 
 @pytest.mark.parametrize("name,sample", [("cfg3", 4096), ("cfg2", 2048), ("cfg4", 4096), ("cfg5", 512)])
@@ -828,6 +829,22 @@ def test_full_size_properties(gpu_device, name, sample):
     wl = make_workload(name)
     _say(f"conv {name} full size, n={wl.n} C={wl.feats.shape[1]} {wl.dtype}")
     _full_size_check(wl, wl.dtype, sample, gpu_device, seed=1)
+
+
+def test_full_size_cfg4_through_the_resident_row_kernels(gpu_device):
+    """Configuration 4 at full size (2.67 million voxels, C = 32, bf16) with the resident-row kernels forced on: the
+    automatic policy would send a cache's first products to the streaming kernels, which the test above covers."""
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    wl = make_workload("cfg4")
+    _say(f"conv cfg4 full size through the resident-row kernels, n={wl.n}")
+    old = impl.spconv.NARROW_RESIDENT
+    impl.spconv.NARROW_RESIDENT = "on"
+    try:
+        cache = _full_size_check(wl, wl.dtype, 4096, gpu_device, seed=3)
+    finally:
+        impl.spconv.NARROW_RESIDENT = old
+    assert hasattr(cache, "_narrow_plan_buf") and getattr(cache, "_narrow_overflows", None) == 0, \
+        "the resident-row kernels did not run"
 
 
 def test_full_size_cfg5_fp32_variant(gpu_device):
