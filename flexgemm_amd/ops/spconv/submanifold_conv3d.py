@@ -785,6 +785,7 @@ def _narrow_wgrad_applies(cache, f: torch.Tensor, ci: int, co: int, v: int, n: i
     if mode == "off":
         return False
     fits = (f.element_size() == 2 and 8 <= ci <= 32 and ci % 8 == 0 and 8 <= co <= 32 and co % 8 == 0 and v <= 27
+            and n > 0                   # no rows, no plan: its header would be read before anything wrote it
             and getattr(cache, "_coords", None) is not None and cache._coords.shape[0] == n and n_in == n
             and n * 64 < 0xFF000000 and n * 82 + 10752 < 0xFF000000)
     if not fits or not (mode == "on" or hasattr(cache, "_narrow_plan_buf")):

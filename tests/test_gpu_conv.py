@@ -214,6 +214,35 @@ def test_degenerate_sizes(gpu_device, res):
         _run_and_check(coords_np, torch.Size([1, 64, res, res, res]), 64, 64, dtype, gpu_device, seed=res)
 
 
+def test_empty_input_through_the_operator(gpu_device):
+    """No voxel at all: an empty output, and a backward pass that returns an empty input gradient and zero weight and bias
+    gradients -- both schedules, the resident-row kernels on "auto" and forced on, channel counts that need padding."""
+    from flex_gemm.ops.spconv import set_algorithm
+    from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
+    old = impl.spconv.NARROW_RESIDENT
+    try:
+        for algo in (Algorithm.MASKED_IMPLICIT_GEMM_SPLITK, Algorithm.IMPLICIT_GEMM):
+            set_algorithm(algo)
+            for narrow in ("auto", "on"):
+                impl.spconv.NARROW_RESIDENT = narrow
+                for dt, c in ((torch.float16, 32), (torch.float32, 64), (torch.bfloat16, 20)):
+                    _say(f"conv of an empty input {algo} narrow={narrow} {dt} C={c}")
+                    coords = torch.zeros((0, 4), dtype=torch.int32, device=gpu_device)
+                    f = torch.zeros((0, c), dtype=dt, device=gpu_device, requires_grad=True)
+                    w = torch.randn(c, 3, 3, 3, c, device=gpu_device).to(dt).requires_grad_(True)
+                    b = torch.randn(c, device=gpu_device).to(dt).requires_grad_(True)
+                    out, _ = sparse_submanifold_conv3d(f, coords, torch.Size([1, c, 8, 8, 8]), w, b)
+                    assert out.shape == (0, c) and out.dtype == dt
+                    out.backward(torch.zeros_like(out))
+                    torch.cuda.synchronize()
+                    assert f.grad.shape == (0, c)
+                    assert w.grad.shape == w.shape and float(w.grad.abs().max()) == 0.0
+                    assert b.grad.shape == b.shape and float(b.grad.abs().max()) == 0.0
+    finally:
+        impl.spconv.NARROW_RESIDENT = old
+        set_algorithm(Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
+
+
 def test_odd_channel_counts_batches_dilation_no_bias(gpu_device):
     rng = np.random.default_rng(3)
     res = 12
