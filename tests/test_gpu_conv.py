@@ -345,6 +345,44 @@ def test_private_row_order_is_used_and_equivalent(gpu_device):
         impl.LOCALITY_MAX_ROW_BYTES, impl.LOCALITY_MIN_ROWS, impl.LOCALITY_AFTER_CALLS = old
 
 
+@pytest.mark.parametrize("res,chans,iterations", [(128, (16, 32, 64, 32, 16, 8), 5), (512, (32, 16, 32, 64, 24), 3)])
+def test_kernel_choice_over_a_cache_s_life_keeps_the_results(gpu_device, res, chans, iterations):
+    """Layers of different widths share one cache over several training iterations, the policies left on "auto": the
+    cache's first products run on the streaming kernels, later ones on the resident-row kernels once it has earned
+    their plan (64 160 voxels: after sixteen products; 1 026 536 voxels: from the second product on).  Every iteration's
+    output and gradients stay within fp16 rounding of the first iteration's, and iterations after the switch agree bit
+    for bit.  The upstream gradient has stride 0, as out.sum().backward() makes it (scaled by 2^-10: a million ones would
+    overflow an fp16 bias gradient)."""
+    _say(f"kernel choice over a cache's life, res={res} widths={chans}")
+    dev = gpu_device
+    coords = torch.from_numpy(reference_test_shell(res)).to(dev)
+    n = coords.shape[0]
+    g = torch.Generator().manual_seed(res)
+    feats = torch.randn(n, chans[0], generator=g).half().to(dev).requires_grad_(True)
+    params = [((torch.randn(co, 3, 3, 3, ci, generator=g) / (27 * ci) ** 0.5).half().to(dev).requires_grad_(True),
+               torch.randn(co, generator=g).half().to(dev).requires_grad_(True)) for ci, co in zip(chans[:-1], chans[1:])]
+    shape = torch.Size([1, chans[0], res, res, res])
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+    results = []
+    for it in range(iterations):
+        feats.grad = None
+        for w, b in params:
+            w.grad = None
+            b.grad = None
+        h = feats
+        for w, b in params:
+            h = sparse_submanifold_conv3d(h, coords, shape, w, b, cache)[0]
+        (h.sum() * 2.0 ** -10).backward()
+        torch.cuda.synchronize()
+        results.append([h.detach().clone(), feats.grad.clone()] + [w.grad.clone() for w, _ in params] + [b.grad.clone() for _, b in params])
+    assert hasattr(cache, "_narrow_plan_buf"), "the cache never earned the resident-row plan"
+    assert all(bool(torch.isfinite(r).all()) for r in results[0])
+    for got in results[1:]:
+        for a, r in zip(got, results[0]):
+            assert float((a.float() - r.float()).abs().max() / r.float().abs().max().clamp_min(1e-6)) < 2e-3
+    assert all(torch.equal(a, r) for a, r in zip(results[-1], results[-2]))
+
+
 def test_forced_splitk_matches_unsplit(gpu_device):
     """Split-K partial sums add up to the unsplit result (fp32 rounding apart)."""
     import ctypes as C
