@@ -121,7 +121,12 @@ def check(rc: int) -> None:
 
 
 def ptr(t: Optional[torch.Tensor]) -> C.c_void_p:
-    return C.c_void_p(0 if t is None else t.data_ptr())
+    """Device address of a tensor for the C entry points, which take plain pointers and assume dense rows."""
+    if t is None:
+        return C.c_void_p(0)
+    if not t.is_contiguous():
+        raise ValueError(f"a strided view (shape {tuple(t.shape)}, strides {t.stride()}) was about to be passed as a plain pointer")
+    return C.c_void_p(t.data_ptr())
 
 
 def stream() -> C.c_void_p:

@@ -669,6 +669,8 @@ def _gather_gemm(src: torch.Tensor, weight_cvk: torch.Tensor, bias: Optional[tor
     k = ci if mode == 0 else co
     src = src.contiguous()
     weight_cvk = weight_cvk.contiguous()
+    if bias is not None:
+        bias = bias.contiguous()        # the kernels read it with stride 1 (a view such as a column of a matrix has another)
     sched = nat.table_lookup(nat.PASS_FWD if mode == 0 else nat.PASS_DGRAD, dt, n, ci, co, v)
     splitk = sched.splitk if allow_splitk else 1
     if masked:

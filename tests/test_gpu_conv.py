@@ -243,6 +243,54 @@ def test_empty_input_through_the_operator(gpu_device):
         set_algorithm(Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
 
 
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("dtype,ci,co,res", [(torch.float16, 64, 32, 24), (torch.float32, 5, 7, 16), (torch.bfloat16, 128, 128, 32),
+                                             (torch.float16, 24, 16, 48)])
+def test_strided_views_and_partial_gradients(gpu_device, dtype, ci, co, res, relu):
+    """Arguments that are views with strides of their own -- the weight a permuted [Ci, Kw, Kh, Kd, Co] tensor, the bias
+    a column of a matrix, the upstream gradient a transposed tensor -- give the bits of their dense copies; so do calls
+    where only the weight, or only the features, want a gradient, and a call without bias."""
+    from flex_gemm.ops.spconv import sparse_submanifold_conv3d_relu
+    op = sparse_submanifold_conv3d_relu if relu else sparse_submanifold_conv3d
+    _say(f"strided views {dtype} ci={ci} co={co} res={res} relu={relu}")
+    dev = gpu_device
+    coords = torch.from_numpy(reference_test_shell(res)).to(dev)
+    n = coords.shape[0]
+    shape = torch.Size([1, ci, res, res, res])
+    g = torch.Generator().manual_seed(1)
+    f0 = torch.randn(n, ci, generator=g).to(dtype).to(dev)
+    w0 = (torch.randn(co, 3, 3, 3, ci, generator=g) / (27 * ci) ** 0.5).to(dtype).to(dev)
+    b0 = torch.randn(co, generator=g).to(dtype).to(dev)
+    go0 = torch.randn(n, co, generator=g).to(dtype).to(dev)
+
+    def step(f, w, b, go):
+        out = op(f, coords, shape, w, b)[0]
+        out.backward(go)
+        torch.cuda.synchronize()
+        return out.detach()
+
+    f, w, b = f0.clone().requires_grad_(True), w0.clone().requires_grad_(True), b0.clone().requires_grad_(True)
+    ref = (step(f, w, b, go0), f.grad, w.grad, b.grad)
+    ws = w0.permute(4, 1, 2, 3, 0).contiguous().permute(4, 1, 2, 3, 0).requires_grad_(True)
+    bs = torch.stack([b0, b0], 1)[:, 0].requires_grad_(True)
+    gos = go0.t().contiguous().t()
+    assert not ws.is_contiguous() and not bs.is_contiguous() and not gos.is_contiguous()
+    f = f0.clone().requires_grad_(True)
+    out = step(f, ws, bs, gos)
+    for name, a, r in zip(("output", "input gradient", "weight gradient", "bias gradient"), (out, f.grad, ws.grad, bs.grad), ref):
+        assert a.shape == r.shape and torch.equal(a, r), name
+    w = w0.clone().requires_grad_(True)                         # only the weight wants a gradient
+    assert torch.equal(step(f0, w, b0, go0), ref[0]) and torch.equal(w.grad, ref[2])
+    f = f0.clone().requires_grad_(True)                         # only the features do
+    assert torch.equal(step(f, w0, b0, go0), ref[0]) and torch.equal(f.grad, ref[1])
+    if not relu:                                                # no bias: the gradients do not depend on it
+        f, w = f0.clone().requires_grad_(True), w0.clone().requires_grad_(True)
+        out = step(f, w, None, go0)
+        assert torch.equal(f.grad, ref[1]) and torch.equal(w.grad, ref[2])
+        tol = 1e-4 if dtype == torch.float32 else 1e-2
+        assert float((out.float() + b0.float() - ref[0].float()).abs().max() / ref[0].float().abs().max()) < tol
+
+
 def test_odd_channel_counts_batches_dilation_no_bias(gpu_device):
     rng = np.random.default_rng(3)
     res = 12
