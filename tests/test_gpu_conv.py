@@ -304,6 +304,18 @@ def test_odd_channel_counts_batches_dilation_no_bias(gpu_device):
     _run_and_check(coords_np, shape, 32, 32, torch.float16, gpu_device, seed=1, ksize=(1, 3, 3))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("ci,co", [(1, 1), (1, 3), (3, 1), (2, 130), (130, 2), (257, 9), (9, 520), (1032, 17)])
+def test_extreme_channel_counts(gpu_device, dtype, ci, co):
+    """Single channels, rows shorter than one 16-byte chunk, and counts just past a tile (129-130, 257, 520, 1032) on
+    either side, both masked and unmasked schedules."""
+    res = 14
+    coords_np = reference_test_shell(res)
+    for algo in (Algorithm.MASKED_IMPLICIT_GEMM_SPLITK, Algorithm.IMPLICIT_GEMM):
+        _say(f"conv extreme channels ci={ci} co={co} {dtype} {algo}")
+        _run_and_check(coords_np, torch.Size([1, ci, res, res, res]), ci, co, dtype, gpu_device, seed=ci + co, algo=algo)
+
+
 def test_algorithm_values_and_cache_reuse(gpu_device):
     res, c = 16, 64
     coords_np = reference_test_shell(res)
