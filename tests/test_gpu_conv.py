@@ -316,6 +316,23 @@ def test_extreme_channel_counts(gpu_device, dtype, ci, co):
         _run_and_check(coords_np, torch.Size([1, ci, res, res, res]), ci, co, dtype, gpu_device, seed=ci + co, algo=algo)
 
 
+@pytest.mark.parametrize("c,dtype", [(64, torch.float16), (128, torch.bfloat16), (40, torch.float32)])
+@pytest.mark.parametrize("ksize,dilation", [((5, 5, 1), (1, 1, 1)), ((1, 1, 31), (1, 1, 1)), ((1, 1, 1), (1, 1, 1)), ((3, 1, 3), (1, 2, 3)),
+                                            ((1, 3, 9), (2, 1, 1)), ((1, 1, 5), (1, 1, 4))])
+def test_kernel_volumes_from_1_to_32_on_wide_layers(gpu_device, c, dtype, ksize, dilation):
+    """Kernel volumes other than 27 -- one offset, 31 offsets (the largest odd volume a 32-bit mask code holds) -- with and
+    without dilation, on layers the streaming and sweep kernels serve.  Even extents are refused: the reference's map
+    builder mirrors offset v onto V - 1 - v (subm_neighbor_map.cu:53-60), which only an odd kernel allows."""
+    res = 20
+    _say(f"conv ksize={ksize} dilation={dilation} c={c} {dtype}")
+    coords_np = reference_test_shell(res, batch=2)
+    _run_and_check(coords_np, torch.Size([2, c, res, res, res]), c, c, dtype, gpu_device, seed=c + ksize[0], ksize=ksize,
+                   dilation=dilation)
+    with pytest.raises(ValueError, match="odd"):
+        SubMConv3dFunction._compute_neighbor_cache(torch.from_numpy(coords_np).to(gpu_device), torch.Size([2, c, res, res, res]),
+                                                   (2, 3, 3), (1, 1, 1), True)
+
+
 def test_algorithm_values_and_cache_reuse(gpu_device):
     res, c = 16, 64
     coords_np = reference_test_shell(res)
