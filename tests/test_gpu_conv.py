@@ -333,6 +333,51 @@ def test_kernel_volumes_from_1_to_32_on_wide_layers(gpu_device, c, dtype, ksize,
                                                    (2, 3, 3), (1, 1, 1), True)
 
 
+@pytest.mark.parametrize("res,c", [(512, 32), (256, 128)])
+def test_whole_path_on_a_stream_of_the_caller_s_while_the_default_stream_is_busy(gpu_device, res, c):
+    """Cache build (at a million voxels: map, then mask sort and pair lists side by side on two streams), forward and
+    backward enqueued on a stream of the caller's, the default stream kept busy with unrelated products and no device-wide
+    wait in between: the bits of the same calls on the default stream."""
+    _say(f"whole path on a caller's stream, res={res} c={c}")
+    dev = gpu_device
+    coords = torch.from_numpy(reference_test_shell(res)).to(dev)
+    n = coords.shape[0]
+    shape = torch.Size([1, c, res, res, res])
+    g = torch.Generator().manual_seed(res)
+    f0 = torch.randn(n, c, generator=g).half().to(dev)
+    w0 = (torch.randn(c, 3, 3, 3, c, generator=g) / (27 * c) ** 0.5).half().to(dev)
+    b0 = torch.randn(c, generator=g).half().to(dev)
+    go = torch.randn(n, c, generator=g).half().to(dev)
+
+    def steps(count):
+        got = []
+        for _ in range(count):
+            f, w, b = f0.clone().requires_grad_(True), w0.clone().requires_grad_(True), b0.clone().requires_grad_(True)
+            cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+            h = sparse_submanifold_conv3d(f, coords, shape, w, b, cache)[0]
+            h = sparse_submanifold_conv3d(h, coords, shape, w, b, cache)[0]
+            h.backward(go)
+            got.append((h.detach(), f.grad, w.grad, b.grad, cache.neighbor_map, cache.sorted_idx, cache.valid_signal_i))
+        return got
+
+    ref = steps(1)[0]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    busy = torch.randn(4096, 4096, device=dev)
+    side.wait_stream(torch.cuda.current_stream())
+    for _ in range(20):
+        busy = torch.tanh(busy @ busy) * 0.5
+    with torch.cuda.stream(side):
+        got = steps(3)
+    for _ in range(20):
+        busy = torch.tanh(busy @ busy) * 0.5
+    side.synchronize()
+    torch.cuda.synchronize()
+    for one in got:
+        for name, a, r in zip(("output", "input gradient", "weight gradient", "bias gradient", "map", "order", "pairs"), one, ref):
+            assert torch.equal(a, r), name
+
+
 def test_algorithm_values_and_cache_reuse(gpu_device):
     res, c = 16, 64
     coords_np = reference_test_shell(res)
