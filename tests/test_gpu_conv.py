@@ -378,6 +378,45 @@ def test_whole_path_on_a_stream_of_the_caller_s_while_the_default_stream_is_busy
             assert torch.equal(a, r), name
 
 
+@pytest.mark.parametrize("needs_grad", [True, False])
+def test_one_cache_serves_layers_of_any_type_width_and_schedule(gpu_device, needs_grad):
+    """One neighbor cache (built with or without the gradient tables: a backward pass makes them when they are missing)
+    serves fp16, fp32 and bf16 layers of different widths under the masked and the unmasked schedule, one after the
+    other; every product and gradient has the bits a fresh cache gives.  The tables a cache keeps per shape (work lists,
+    sweep plans, tile orders) must not leak from one layer shape or type into the next."""
+    from flex_gemm.ops.spconv import set_algorithm
+    dev = gpu_device
+    res = 128
+    coords = torch.from_numpy(reference_test_shell(res)).to(dev)
+    n = coords.shape[0]
+    shape = torch.Size([1, 1, res, res, res])
+    masked, plain = Algorithm.MASKED_IMPLICIT_GEMM_SPLITK, Algorithm.IMPLICIT_GEMM
+    layers = [(torch.float16, 128, 128, masked), (torch.float32, 128, 128, masked), (torch.bfloat16, 64, 64, masked),
+              (torch.float16, 128, 256, masked), (torch.float16, 256, 128, plain), (torch.float16, 128, 128, plain),
+              (torch.bfloat16, 128, 128, masked), (torch.float32, 40, 72, masked), (torch.float16, 1024, 64, masked),
+              (torch.float16, 64, 1024, masked), (torch.float16, 128, 128, masked)]
+
+    def step(tensors, cache, algo):
+        set_algorithm(algo)
+        f, w, b = (t.clone().requires_grad_(True) for t in tensors[:3])
+        out = sparse_submanifold_conv3d(f, coords, shape, w, b, cache)[0]
+        out.backward(tensors[3])
+        torch.cuda.synchronize()
+        return out.detach(), f.grad, w.grad, b.grad
+
+    try:
+        shared = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), needs_grad)
+        for i, (dt, ci, co, algo) in enumerate(layers):
+            _say(f"shared cache, layer {i}: {dt} {ci}->{co} {algo}")
+            tensors = tuple(t.to(dev) for t in _case(np.empty((n, 4)), ci, co, dt, seed=i))
+            got = step(tensors, shared, algo)
+            ref = step(tensors, SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True), algo)
+            for name, a, r in zip(("output", "input gradient", "weight gradient", "bias gradient"), got, ref):
+                assert torch.equal(a, r), (i, name)
+    finally:
+        set_algorithm(masked)
+
+
 def test_algorithm_values_and_cache_reuse(gpu_device):
     res, c = 16, 64
     coords_np = reference_test_shell(res)
