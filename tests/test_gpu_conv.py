@@ -1075,6 +1075,85 @@ def test_full_size_cfg4_through_the_resident_row_kernels(gpu_device):
         "the resident-row kernels did not run"
 
 
+@pytest.mark.parametrize("c", [16, 128])
+def test_more_than_2_to_the_24_voxels_and_operands_past_4_gib(gpu_device, c):
+    """A dense block of 257 x 256 x 256 = 16 842 752 voxels, past the 24-bit row numbers of the weight-gradient sweep; with
+    C = 128 in fp16 every operand is 4.3 GB, past the 32-bit byte offsets of the streaming kernels, so the products take
+    the kernels with 64-bit addressing.  In a dense block the neighbor of a voxel is a fixed step in its row number (the
+    27 steps are read off the oracle's map of a small block), which gives, without the oracle's loops: the map of sampled
+    rows and of the rows around 2^24, bit for bit; the pair count in closed form; forward and input gradient of the
+    sampled rows, every element of the weight gradient of six offsets (slices of the block against each other) and the
+    bias gradient, all in float64 torch arithmetic, to 1e-2 of the largest value."""
+    dev = gpu_device
+    X, Y, Z = 257, 256, 256
+    n = X * Y * Z
+    _say(f"dense block of {n} voxels, C={c}")
+    sx, sy, sz = 5, 4, 4
+    small = np.stack([np.zeros(sx * sy * sz, np.int32)] + [a.reshape(-1).astype(np.int32) for a in
+                                                         np.meshgrid(np.arange(sx), np.arange(sy), np.arange(sz), indexing="ij")], 1)
+    smap = nb.neighbor_map(small, (1, 1, sx, sy, sz), (3, 3, 3), (1, 1, 1)).view(np.int32)
+    centre = (2 * sy + 1) * sz + 1
+    assert (smap[centre] >= 0).all()
+    delta = small[smap[centre]][:, 1:] - small[centre][1:]              # [27, 3]: the step of every kernel offset
+    delta_t = torch.from_numpy(delta).to(dev).long()
+    coords = torch.stack([torch.zeros(n, dtype=torch.int32, device=dev),
+                          torch.arange(X, device=dev, dtype=torch.int32).repeat_interleave(Y * Z),
+                          torch.arange(Y, device=dev, dtype=torch.int32).repeat_interleave(Z).repeat(X),
+                          torch.arange(Z, device=dev, dtype=torch.int32).repeat(X * Y)], 1).contiguous()
+
+    def neighbors(rows):                # [S] -> [S, 27] row numbers, -1 outside the block
+        x, y, z = rows // (Y * Z), (rows // Z) % Y, rows % Z
+        nx, ny, nz = x[:, None] + delta_t[:, 0], y[:, None] + delta_t[:, 1], z[:, None] + delta_t[:, 2]
+        inside = (nx >= 0) & (nx < X) & (ny >= 0) & (ny < Y) & (nz >= 0) & (nz < Z)
+        return torch.where(inside, (nx * Y + ny) * Z + nz, torch.full_like(nx, -1))
+
+    def rel(got, ref):
+        return float((got.double() - ref).abs().max() / ref.abs().max())
+
+    dt = torch.float16
+    shape = torch.Size([1, c, X, Y, Z])
+    g = torch.Generator(device=dev).manual_seed(c)
+    f = torch.randn(n, c, generator=g, device=dev, dtype=dt).requires_grad_(True)
+    w = (torch.randn(c, 3, 3, 3, c, generator=g, device=dev) / (27 * c) ** 0.5).to(dt).requires_grad_(True)
+    b = torch.randn(c, generator=g, device=dev).to(dt).requires_grad_(True)
+    go = torch.randn(n, c, generator=g, device=dev, dtype=dt)
+    cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (3, 3, 3), (1, 1, 1), True)
+    rows = torch.cat([torch.randint(0, n, (4096,), device=dev, generator=g),
+                      torch.tensor([0, n - 1, (1 << 24) - 1, 1 << 24, (1 << 24) + 1], device=dev)])
+    nbr = neighbors(rows)
+    assert torch.equal(cache.neighbor_map.view(torch.int32)[rows].long(), nbr), "neighbor map"
+    assert int(cache._seg_host()[-1]) == sum((X - abs(int(d[0]))) * (Y - abs(int(d[1]))) * (Z - abs(int(d[2]))) for d in delta)
+    _say("  forward and backward")
+    out = sparse_submanifold_conv3d(f, coords, shape, w, b, cache)[0]
+    out.backward(go)
+    torch.cuda.synchronize()
+    w64 = w.detach().double().reshape(c, 27, c)
+    fg = f.detach()[nbr.clamp(min=0)].double() * (nbr >= 0)[:, :, None]
+    assert rel(out.detach()[rows], torch.einsum("svc,ovc->so", fg, w64) + b.detach().double()) < 1e-2, "forward"
+    back = torch.flip(nbr, [1])         # the voxel that has this one as its neighbor at offset v is the neighbor at V - 1 - v
+    gg = go[back.clamp(min=0)].double() * (back >= 0)[:, :, None]
+    assert rel(f.grad[rows], torch.einsum("svo,ovc->sc", gg, w64)) < 1e-2, "input gradient"
+    gw = w.grad.reshape(c, 27, c)
+    F, G = f.detach().view(X, Y, Z, c), go.view(X, Y, Z, c)
+    for v in WGRAD_OFFSETS:
+        _say(f"  wgrad slice of offset {v}")
+        dx, dy, dz = (int(t) for t in delta[v])
+        ref = torch.zeros(c, c, dtype=torch.float64, device=dev)
+        x_end = min(X, X - dx)
+        for x0 in range(max(0, -dx), x_end, 16):
+            x1 = min(x0 + 16, x_end)
+            gs = G[x0:x1, max(0, -dy):min(Y, Y - dy), max(0, -dz):min(Z, Z - dz)].reshape(-1, c).double()
+            fs = F[x0 + dx:x1 + dx, max(0, dy):min(Y, Y + dy), max(0, dz):min(Z, Z + dz)].reshape(-1, c).double()
+            ref += gs.t() @ fs
+        assert rel(gw[:, v], ref) < 1e-2, f"weight gradient of offset {v}"
+    ref = torch.zeros(c, dtype=torch.float64, device=dev)
+    for x0 in range(0, X, 16):
+        ref += G[x0:x0 + 16].reshape(-1, c).double().sum(0)
+    assert rel(b.grad, ref) < 1e-2, "bias gradient"
+    del f, w, b, go, out, cache, fg, gg, F, G
+    torch.cuda.empty_cache()
+
+
 def test_full_size_cfg5_fp32_variant(gpu_device):
     """Configuration 5's fp32-input variant (fp32 accumulation) at full size: 42 608 voxels, C = 1024, tolerance 1e-4."""
     wl = make_workload("cfg5")
