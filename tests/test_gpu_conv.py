@@ -217,7 +217,7 @@ def test_degenerate_sizes(gpu_device, res):
 def test_empty_input_through_the_operator(gpu_device):
     """No voxel at all: an empty output, and a backward pass that returns an empty input gradient and zero weight and bias
     gradients -- both schedules, the resident-row kernels on "auto" and forced on, channel counts that need padding."""
-    from flex_gemm.ops.spconv import set_algorithm
+    from flex_gemm.ops.spconv import set_algorithm, sparse_submanifold_conv3d_relu
     from flexgemm_amd.ops.spconv import submanifold_conv3d as impl
     old = impl.spconv.NARROW_RESIDENT
     try:
@@ -231,13 +231,15 @@ def test_empty_input_through_the_operator(gpu_device):
                     f = torch.zeros((0, c), dtype=dt, device=gpu_device, requires_grad=True)
                     w = torch.randn(c, 3, 3, 3, c, device=gpu_device).to(dt).requires_grad_(True)
                     b = torch.randn(c, device=gpu_device).to(dt).requires_grad_(True)
-                    out, _ = sparse_submanifold_conv3d(f, coords, torch.Size([1, c, 8, 8, 8]), w, b)
-                    assert out.shape == (0, c) and out.dtype == dt
-                    out.backward(torch.zeros_like(out))
-                    torch.cuda.synchronize()
-                    assert f.grad.shape == (0, c)
-                    assert w.grad.shape == w.shape and float(w.grad.abs().max()) == 0.0
-                    assert b.grad.shape == b.shape and float(b.grad.abs().max()) == 0.0
+                    for op in (sparse_submanifold_conv3d, sparse_submanifold_conv3d_relu):
+                        f.grad = w.grad = b.grad = None
+                        out, _ = op(f, coords, torch.Size([1, c, 8, 8, 8]), w, b)
+                        assert out.shape == (0, c) and out.dtype == dt
+                        out.backward(torch.zeros_like(out))
+                        torch.cuda.synchronize()
+                        assert f.grad.shape == (0, c)
+                        assert w.grad.shape == w.shape and float(w.grad.abs().max()) == 0.0
+                        assert b.grad.shape == b.shape and float(b.grad.abs().max()) == 0.0
     finally:
         impl.spconv.NARROW_RESIDENT = old
         set_algorithm(Algorithm.MASKED_IMPLICIT_GEMM_SPLITK)
