@@ -25,6 +25,20 @@ def library():
     return ctypes.CDLL(nat.lib_path())
 
 
+@pytest.mark.parametrize("compiler,flags", [("gcc", ["-std=c99", "-x", "c"]), ("g++", ["-std=c++17", "-x", "c++"])])
+def test_header_is_plain_c_and_cxx(compiler, flags):
+    """The boundary is a C ABI: the header must compile on its own as pedantic C99 (what cgo / ctypes-style bindings see)
+    and as C++, without HIP or torch headers on the include path."""
+    import shutil
+    import subprocess
+    if shutil.which(compiler) is None:
+        pytest.skip(f"{compiler} is not installed")
+    header = os.path.join(ROOT, "include", "flexgemm_hip.h")
+    done = subprocess.run([compiler, *flags, "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", header],
+                          capture_output=True, text=True)
+    assert done.returncode == 0, done.stderr
+
+
 def test_header_and_binding_agree():
     assert _declared_symbols() == sorted(nat.EXPORTS)
 
