@@ -1,8 +1,9 @@
 """Build recipe of libflexgemm_hip.so: hipcc, gfx950 only, in-tree output.
 
 `python -m flexgemm_amd.build` compiles every file under flexgemm_amd/csrc/ and links
-flexgemm_amd/_lib/libflexgemm_hip.so.  Objects are rebuilt when their source (or a header) is
-newer; pass --force to rebuild everything.
+flexgemm_amd/_lib/libflexgemm_hip.so, then the tests' torch-free caller of the C ABI against it
+(flexgemm_amd/_lib/conv_host).  Objects are rebuilt when their source (or a header) is newer; pass
+--force to rebuild everything.
 """
 from __future__ import annotations
 
@@ -16,6 +17,9 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG, "csrc")
 OUT_DIR = os.path.join(PKG, "_lib")
 LIB = os.path.join(OUT_DIR, "libflexgemm_hip.so")
+# a caller of the C ABI without Python or torch, run by the GPU tests (tests/cabi_host/conv_host.cpp)
+HOST_CHECK_SRC = os.path.join(PKG, "..", "tests", "cabi_host", "conv_host.cpp")
+HOST_CHECK = os.path.join(OUT_DIR, "conv_host")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
 
@@ -73,6 +77,14 @@ def build(force: bool = False, verbose: bool = True, jobs: int = 4) -> str:
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
+    if os.path.exists(HOST_CHECK_SRC) and (force or todo or _stale(HOST_CHECK, [HOST_CHECK_SRC, LIB] + hdrs)):
+        cmd = [HIPCC] + COMMON_FLAGS + ["-I", os.path.join(PKG, "..", "include"), HOST_CHECK_SRC, "-L", OUT_DIR, "-lflexgemm_hip",
+                                        "-Wl,-rpath,$ORIGIN", "-o", HOST_CHECK]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"building the host check failed:\n{r.stdout}\n{r.stderr}")
     return LIB
 
 

@@ -39,6 +39,16 @@ def test_header_is_plain_c_and_cxx(compiler, flags):
     assert done.returncode == 0, done.stderr
 
 
+def test_host_program_is_built_beside_the_library(library):
+    """The torch-free caller of the C ABI that the GPU tests run links against the in-tree library and nothing of Python."""
+    import subprocess
+    from flexgemm_amd import build
+    if not os.path.exists(build.HOST_CHECK):
+        build.build(verbose=False)
+    needed = subprocess.run(["ldd", build.HOST_CHECK], capture_output=True, text=True).stdout
+    assert "libflexgemm_hip.so" in needed and "torch" not in needed and "python" not in needed.lower()
+
+
 def test_header_and_binding_agree():
     assert _declared_symbols() == sorted(nat.EXPORTS)
 
