@@ -130,6 +130,26 @@ def test_cache_shuffled_batched_dilated(gpu_device):
         _check_cache(cache, coords_np, shape, True, blocks=(2, 64, 100), ks=ks, dil=dil)
 
 
+def test_grids_with_unequal_sides_and_steps_that_leave_the_grid(gpu_device, neighbor_map_builder):
+    """Grids whose three sides differ (one of them 1 or 2 cells), every cell of the boundary occupied, and dilations whose
+    steps reach past the far side or below zero from every voxel: a neighbor outside the grid is absent, never the voxel
+    that the flattened key of the step would alias (x + 1 past the last column is not the first cell of the next row)."""
+    rng = np.random.default_rng(11)
+    for (w, h, d), batch in [((40, 6, 17), 2), ((1, 33, 9), 1), ((2, 2, 64), 3), ((7, 1, 1), 4), ((31, 32, 33), 1)]:
+        cells = np.stack(np.meshgrid(np.arange(batch), np.arange(w), np.arange(h), np.arange(d), indexing="ij"), -1).reshape(-1, 4)
+        keep = rng.random(len(cells)) < 0.6
+        face = ((cells[:, 1] == 0) | (cells[:, 1] == w - 1) | (cells[:, 2] == 0) | (cells[:, 2] == h - 1) | (cells[:, 3] == 0)
+                | (cells[:, 3] == d - 1))
+        coords_np = np.ascontiguousarray(cells[keep | face][rng.permutation(int((keep | face).sum()))].astype(np.int32))
+        coords = torch.from_numpy(coords_np).to(gpu_device)
+        shape = torch.Size([batch, 0, w, h, d])
+        for ks, dil in [((3, 3, 3), (1, 1, 1)), ((3, 3, 3), (w, h, d)), ((3, 3, 3), (max(w - 1, 1), max(h - 1, 1), max(d - 1, 1))),
+                        ((5, 3, 1), (3, 5, 1)), ((1, 1, 9), (1, 1, 7)), ((3, 3, 3), (100, 1, 1000))]:
+            _say(f"neighbor cache grid={(w, h, d)} batch={batch} ks={ks} dil={dil} builder={neighbor_map_builder}")
+            cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, ks, dil, True)
+            _check_cache(cache, coords_np, shape, True, blocks=(64,), ks=ks, dil=dil)
+
+
 def test_large_kernel_explicit_and_uint64_keys(gpu_device):
     rng = np.random.default_rng(11)
     res = 12
