@@ -419,6 +419,53 @@ def test_one_cache_serves_layers_of_any_type_width_and_schedule(gpu_device, need
         set_algorithm(masked)
 
 
+def test_four_host_threads_call_the_library_at_once(gpu_device):
+    """ctypes drops the interpreter lock around a foreign call, so threads of one process are inside the library together.
+    Four threads, each on a stream of its own and with a layer shape of its own, build caches and run forward and
+    backward a few times over; every thread gets the bits the same calls give when they run alone."""
+    import threading
+    dev = gpu_device
+    cases = [(48, 128, 128, torch.float16), (40, 32, 32, torch.bfloat16), (32, 64, 256, torch.float16), (24, 40, 72, torch.float32)]
+
+    def work(res, ci, co, dt, rounds):
+        coords = torch.from_numpy(reference_test_shell(res)).to(dev)
+        shape = torch.Size([1, ci, res, res, res])
+        tensors = [t.to(dev) for t in _case(np.empty((coords.shape[0], 4)), ci, co, dt, seed=res)]
+        got = []
+        for _ in range(rounds):
+            f, w, b = (t.clone().requires_grad_(True) for t in tensors[:3])
+            out, cache = sparse_submanifold_conv3d(f, coords, shape, w, b)
+            out.backward(tensors[3])
+            got.append((out.detach(), f.grad, w.grad, b.grad, cache.sorted_idx))
+        torch.cuda.current_stream().synchronize()
+        return got
+
+    alone = [work(*case, 1)[0] for case in cases]
+    torch.cuda.synchronize()
+    results, errors = [None] * len(cases), []
+
+    def thread_main(i):
+        try:
+            with torch.cuda.stream(torch.cuda.Stream()):
+                results[i] = work(*cases[i], 6)
+        except BaseException as e:              # reported by the main thread
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=thread_main, args=(i,)) for i in range(len(cases))]
+    _say("four threads inside the library")
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not any(t.is_alive() for t in threads), "a thread did not finish"
+    assert not errors, errors
+    torch.cuda.synchronize()
+    for i, rounds in enumerate(results):
+        for got in rounds:
+            for name, a, r in zip(("output", "input gradient", "weight gradient", "bias gradient", "order"), got, alone[i]):
+                assert torch.equal(a, r), (cases[i], name)
+
+
 def test_algorithm_values_and_cache_reuse(gpu_device):
     res, c = 16, 64
     coords_np = reference_test_shell(res)
