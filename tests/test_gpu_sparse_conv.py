@@ -306,6 +306,39 @@ def test_empty_input(gpu_device):
     assert out.shape == (0, 8) and oc.shape == (0, 4) and cache.neighbor_map.shape == (0, 27)
 
 
+@pytest.mark.parametrize("geom", [GEOMS[2], GEOMS[3]])
+def test_strided_views_give_the_bits_of_their_dense_copies(gpu_device, geom):
+    """Weight, bias and upstream gradient handed over as views with strides of their own."""
+    ks, st, pd, dl = geom
+    _say(f"sparse conv with strided arguments, geometry {geom}")
+    dev = gpu_device
+    res, ci, co = 24, 64, 40
+    coords = torch.from_numpy(_shell(res)).to(dev)
+    shape = torch.Size([1, ci, res, res, res])
+    g = torch.Generator().manual_seed(5)
+    f0 = torch.randn(coords.shape[0], ci, generator=g).half().to(dev)
+    w0 = (torch.randn(co, *ks, ci, generator=g) / math.sqrt(ks[0] * ks[1] * ks[2] * ci)).half().to(dev)
+    b0 = torch.randn(co, generator=g).half().to(dev)
+
+    def step(w, b, make_grad):
+        f = f0.clone().requires_grad_(True)
+        out, oc, _ = sparse_conv3d(f, coords, shape, w, b, stride=st, padding=pd, dilation=dl)
+        go = make_grad(out)
+        out.backward(go)
+        torch.cuda.synchronize()
+        return out.detach(), f.grad, w.grad, b.grad, oc
+
+    gen = torch.Generator(device=dev)
+    dense = lambda out: torch.randn(out.shape, generator=gen.manual_seed(9), device=dev).to(out.dtype)
+    ref = step(w0.clone().requires_grad_(True), b0.clone().requires_grad_(True), dense)
+    ws = w0.permute(4, 1, 2, 3, 0).contiguous().permute(4, 1, 2, 3, 0).requires_grad_(True)
+    bs = torch.stack([b0, b0], 1)[:, 0].requires_grad_(True)
+    assert not ws.is_contiguous() and not bs.is_contiguous()
+    got = step(ws, bs, lambda out: dense(out).t().contiguous().t())
+    for name, a, r in zip(("output", "input gradient", "weight gradient", "bias gradient", "output coordinates"), got, ref):
+        assert a.shape == r.shape and torch.equal(a, r), name
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("geom", [GEOMS[0], GEOMS[2], GEOMS[3]])
 def test_relu_in_the_epilogue_equals_relu_after_the_operator(gpu_device, dtype, geom):
