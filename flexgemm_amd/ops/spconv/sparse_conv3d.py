@@ -20,7 +20,8 @@ from .. import spconv, utils
 from .. import serialize
 from . import Algorithm, SerializationMode, SparseConv3dOutCoordAlgorithm
 from .submanifold_conv3d import (EMPTY, _IMPLICIT, _MASKED, _NO_SPLITK, SubMConv3dNeighborCache, _codes_and_order, _colsum,
-                                 _gather_gemm, _gathered_rows, _pair_lists, _relu_mask_apply, _require_cuda, _wgrad)
+                                 _gather_gemm, _gathered_rows, _grad_mode_of_the_caller, _gradients_possible, _pair_lists,
+                                 _relu_mask_apply, _require_cuda, _wgrad)
 
 
 def _triple(x) -> Tuple[int, int, int]:
@@ -399,7 +400,7 @@ class SparseConv3dFunction(Function):
     ):
         co, kw, kh, kd, ci = weight.shape
         assert feats.shape[-1] == ci, f"Input channels ({feats.shape[-1]}) should match weight channels ({ci})"
-        need_grad = any(ctx.needs_input_grad)
+        need_grad = _gradients_possible(ctx)
         given = out_coords is not None
         if out_coords is None:
             out_coords = SparseConv3dFunction._get_output_coords(coords, shape, (kw, kh, kd), stride, padding, dilation)
@@ -470,7 +471,9 @@ def sparse_conv3d(
     Returns:
         (out_feats [M, Co], out_coords [M, 4], neighbor_cache)
     """
-    return SparseConv3dFunction.apply(feats, coords, shape, neighbor_cache, weight, bias, out_coords, stride, padding, dilation)
+    with _grad_mode_of_the_caller():
+        return SparseConv3dFunction.apply(feats, coords, shape, neighbor_cache, weight, bias, out_coords, stride, padding,
+                                          dilation)
 
 
 def sparse_conv3d_relu(
@@ -488,5 +491,6 @@ def sparse_conv3d_relu(
     """relu(sparse_conv3d(...)) with the clamp done in the GEMM's epilogue (no counterpart in the reference; same
     arguments and return values as sparse_conv3d).  Differentiable: backward masks the incoming gradient with the sign
     of the saved output and runs the usual passes."""
-    return SparseConv3dFunction.apply(feats, coords, shape, neighbor_cache, weight, bias, out_coords, stride, padding, dilation,
-                                      True)
+    with _grad_mode_of_the_caller():
+        return SparseConv3dFunction.apply(feats, coords, shape, neighbor_cache, weight, bias, out_coords, stride, padding,
+                                          dilation, True)

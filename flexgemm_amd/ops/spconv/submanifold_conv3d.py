@@ -9,6 +9,7 @@ include/flexgemm_hip.h; torch only allocates tensors and owns the stream.
 from __future__ import annotations
 
 import ctypes as C
+import threading
 import weakref
 from typing import Optional, Tuple
 
@@ -594,6 +595,27 @@ def _release_panel_bytes(nbytes: int) -> None:
     _panel_bytes_kept -= nbytes
 
 
+_public_call = threading.local()
+
+
+class _grad_mode_of_the_caller:
+    """autograd runs Function.forward with grad mode off, so forward cannot see whether its caller stands under
+    torch.no_grad() / inference_mode(); the public wrappers note it here (per thread) around apply().  Direct callers of
+    apply() count as wanting gradients, like in the reference."""
+
+    def __enter__(self):
+        _public_call.grad_enabled = torch.is_grad_enabled()
+
+    def __exit__(self, *exc):
+        _public_call.grad_enabled = True
+        return False
+
+
+def _gradients_possible(ctx) -> bool:
+    """Whether a backward pass can follow this forward: an argument wants a gradient and the caller records them."""
+    return any(ctx.needs_input_grad) and getattr(_public_call, "grad_enabled", True)
+
+
 def _weight_panel(owner: Optional[torch.Tensor], weight_cvk: torch.Tensor, code: int, mode: int, sched, dev) -> torch.Tensor:
     """The weight repacked for the gather GEMM of `mode` under schedule `sched`.  With spconv.WEIGHT_PANEL_CACHE and an
     `owner` (the caller's weight tensor, whose version counter and data pointer say whether it changed) the panel is
@@ -1128,7 +1150,7 @@ class SubMConv3dFunction(Function):
     ) -> Tuple[torch.Tensor, SubMConv3dNeighborCache]:
         co, kw, kh, kd, ci = weight.shape
         assert feats.shape[-1] == ci, f"Input channels ({feats.shape[-1]}) should match weight channels ({ci})"
-        need_grad = any(ctx.needs_input_grad)
+        need_grad = _gradients_possible(ctx)
         if neighbor_cache is None:
             neighbor_cache = SubMConv3dFunction._compute_neighbor_cache(coords, shape, (kw, kh, kd), dilation, need_grad)
         masks = [] if (relu and need_grad and spconv.RELU_BIT_MASK) else None
@@ -1191,7 +1213,8 @@ def sparse_submanifold_conv3d(
     Returns:
         (output [N, Co], neighbor_cache)
     """
-    return SubMConv3dFunction.apply(feats, coords, shape, neighbor_cache, weight, bias, dilation)
+    with _grad_mode_of_the_caller():
+        return SubMConv3dFunction.apply(feats, coords, shape, neighbor_cache, weight, bias, dilation)
 
 
 def sparse_submanifold_conv3d_relu(
@@ -1206,4 +1229,5 @@ def sparse_submanifold_conv3d_relu(
     """relu(sparse_submanifold_conv3d(...)) with the clamp done in the GEMM's epilogue: the output is written once,
     already activated (no counterpart in the reference; same arguments and return values as sparse_submanifold_conv3d).
     Differentiable: backward masks the incoming gradient with the sign of the saved output and runs the usual passes."""
-    return SubMConv3dFunction.apply(feats, coords, shape, neighbor_cache, weight, bias, dilation, True)
+    with _grad_mode_of_the_caller():
+        return SubMConv3dFunction.apply(feats, coords, shape, neighbor_cache, weight, bias, dilation, True)

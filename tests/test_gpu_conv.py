@@ -466,6 +466,38 @@ def test_four_host_threads_call_the_library_at_once(gpu_device):
                 assert torch.equal(a, r), (cases[i], name)
 
 
+@pytest.mark.parametrize("mode", ["no_grad", "inference_mode"])
+def test_calls_that_record_no_gradients_build_no_gradient_tables(gpu_device, mode):
+    """Under torch.no_grad() / inference_mode() the weights still say requires_grad, but no backward pass can follow: the
+    cache such a call builds carries no pair lists, the fused ReLU writes no bit mask, and the results are those of a
+    recording call.  A cache made that way still serves a later training step (its tables are made when asked for)."""
+    from flex_gemm.ops.spconv import sparse_conv3d, sparse_submanifold_conv3d_relu
+    dev = gpu_device
+    res, c = 32, 64
+    _say(f"calls under {mode}")
+    coords = torch.from_numpy(reference_test_shell(res)).to(dev)
+    shape = torch.Size([1, c, res, res, res])
+    f, w, b, go = (t.to(dev) for t in _case(np.empty((coords.shape[0], 4)), c, c, torch.float16, seed=4))
+    w, b = torch.nn.Parameter(w), torch.nn.Parameter(b)
+    ref, trained = sparse_submanifold_conv3d(f, coords, shape, w, b)
+    assert hasattr(trained, "valid_signal_i")
+    with getattr(torch, mode)():
+        out, lean = sparse_submanifold_conv3d(f, coords, shape, w, b)
+        assert torch.equal(out, ref) and not out.requires_grad
+        assert not hasattr(lean, "valid_signal_i"), "gradient tables were built for a call that cannot use them"
+        assert torch.equal(sparse_submanifold_conv3d(f, coords, shape, w, b, trained)[0], ref)
+        assert torch.equal(sparse_submanifold_conv3d_relu(f, coords, shape, w, b, lean)[0], torch.relu(ref))
+        _, _, lean_generic = sparse_conv3d(f, coords, shape, w, b, stride=(2, 2, 2), padding=(1, 1, 1))
+        assert not hasattr(lean_generic, "valid_signal_i")
+    grads = []
+    for cache in (trained, lean):
+        f2 = f.clone().requires_grad_(True)
+        w.grad = b.grad = None
+        sparse_submanifold_conv3d(f2, coords, shape, w, b, cache)[0].backward(go)
+        grads.append((f2.grad, w.grad, b.grad))
+    assert all(torch.equal(a, r) for a, r in zip(grads[1], grads[0]))
+
+
 def test_algorithm_values_and_cache_reuse(gpu_device):
     res, c = 16, 64
     coords_np = reference_test_shell(res)
